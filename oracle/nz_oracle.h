@@ -1,0 +1,122 @@
+/*
+ * nz_oracle.h -- CPU restatement of NeuZephyr's tensor-core GEMM path.
+ *
+ * THIS IS TEST INFRASTRUCTURE.  It is the checker for the HIP library and the
+ * timed CPU baseline of the benchmark; nothing in the shipped library links,
+ * loads or calls it.
+ *
+ * Every function cites the reference file:line it restates (paths are relative
+ * to the NeuZephyr source tree).  The reference itself is CUDA-only (nvcc,
+ * <mma.h>, cuRAND) and cannot be compiled here, so each function is pinned by
+ * the reference's own literal test vectors, by hardware F16C conversion, and
+ * by closed forms / brute force (see tests/test_oracle_*.py).
+ *
+ * Parity status:
+ *   - fp32->fp16 rounding ............ pinned (F16C hardware, exhaustive halfs)
+ *   - GEMM / batched broadcast GEMM .. pinned (reference literal vectors,
+ *                                      integer exactness, fp64 truth bound)
+ *   - im2col / col2im ................ pinned (reference loop-nest spec,
+ *                                      direct-convolution identity)
+ *   - bias add / ReLU ................ pinned (closed form, NaN / -0 cases)
+ *   - bit-level accumulation order of nvcuda::wmma::mma_sync: PARITY UNPINNED
+ *     (unspecified by the vendor; the tolerance contract replaces it).
+ */
+#ifndef NZ_ORACLE_H
+#define NZ_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- fp16 rounding: __float2half in Padding, src/OperationKernels.cu:846-860 */
+uint16_t nzo_f32_to_f16_bits(float x);          /* IEEE RNE, subnormals kept, >=65520 -> inf */
+float nzo_f16_bits_to_f32(uint16_t h);
+float nzo_round_f16(float x);                   /* f16_bits_to_f32(f32_to_f16_bits(x)) */
+void nzo_round_f16_array(float* dst, const float* src, size_t n);
+
+/* ---- single GEMM: GeneralMatrixMulTensorKernel, src/OperationKernels.cu:821-844
+ * C[M,N] = f16(A)[M,K] * f16(B)[K,N], fp32 accumulation, k ascending.
+ * trans_b != 0: B is given as N x K row-major (element (k,n) at B[n*ldb+k]).
+ * Zero padding to multiples of 16 (utils.cuh:13) adds exact zeros and is
+ * therefore not materialised. */
+void nzo_gemm_f16in_f32acc(const float* A, const float* B, float* C,
+                           size_t M, size_t N, size_t K,
+                           size_t lda, size_t ldb, size_t ldc, int trans_b);
+
+/* Same rounded inputs, fp64 accumulation: the truth the tolerances refer to. */
+void nzo_gemm_f16in_f64acc(const float* A, const float* B, double* C,
+                           size_t M, size_t N, size_t K,
+                           size_t lda, size_t ldb, size_t ldc, int trans_b);
+
+/* Rows [row0,row0+nrows) only, fp32 and fp64 accumulation (sampling of big cases). */
+void nzo_gemm_rows(const float* A, const float* B, float* C32, double* C64,
+                   size_t row0, size_t nrows, size_t N, size_t K,
+                   size_t lda, size_t ldb, int trans_b);
+
+/* ---- batched driver: TensorCoreGEMMParallel, src/OperationKernels.cu:914-1026
+ * shapes are {n,c,h,w}; M=A.h, N=B.w, K=A.w; loops over C's (n,c); an operand
+ * whose n (or c) is 1 is broadcast along that axis (:981-984). */
+void nzo_tensorcore_gemm(const float* A, const float* B, float* C,
+                         const size_t shapeA[4], const size_t shapeB[4], const size_t shapeC[4]);
+
+/* fp32-exact matmul behind Tensor::operator*: GeneralMatrixMulKernel,
+ * src/OperationKernels.cu:65-101 (comparator only; no fp16 rounding). */
+void nzo_general_matmul(const float* A, const float* B, float* C,
+                        const size_t shapeA[4], const size_t shapeB[4], const size_t shapeC[4]);
+
+/* ---- im2col: img2colKernel, src/OperationKernels.cu:1308-1328 */
+void nzo_im2col(float* out, const float* in, size_t H_out, size_t W_out, size_t C,
+                size_t K_h, size_t K_w, size_t stride, size_t pad,
+                size_t H_in, size_t W_in, size_t batch);
+
+/* ---- col2im: col2imgKernel, src/OperationKernels.cu:1364-1376 */
+void nzo_col2im(float* out, const float* in, size_t H_out, size_t W_out, size_t C_out, size_t batches);
+
+/* ---- broadcast add: tensorMatrixAdd + MatrixAddKernel,
+ * include/NeuZephyr/TensorOperations.cuh:785-808, src/OperationKernels.cu:12-24 */
+void nzo_matrix_add(float* out, const float* a, const float* b,
+                    const size_t shapeOut[4], const size_t shapeA[4], const size_t shapeB[4]);
+
+/* ---- ReLU: RectifiedLinearUnitKernel, src/OperationKernels.cu:230-235 (x>0?x:0) */
+void nzo_relu(float* out, const float* in, size_t n);
+
+/* ---- Model::Conv2d graph, src/Model.cu:244-263 (+ optional trailing ReLU node):
+ * x[N,C,H,W]; w_ref[Wb,1,C*Kh*Kw,O] with Wb in {1,N}; bias_ref[1,1,Ho*Wo,O] or NULL;
+ * y[N,O,Ho,Wo].  Runs im2col -> GEMM -> add -> col2im (-> ReLU) exactly as the
+ * reference graph does, materialising the intermediates. */
+void nzo_conv2d_graph(float* y, const float* x, const float* w_ref, const float* bias_ref,
+                      size_t N, size_t C, size_t H, size_t W, size_t O,
+                      size_t K_h, size_t K_w, size_t stride, size_t pad,
+                      size_t w_batch, int relu);
+
+/* Independent 7-loop direct convolution of the fp16-rounded operands in fp64,
+ * OIHW weights, per-channel bias (NULL ok).  Used to pin nzo_conv2d_graph. */
+void nzo_conv2d_direct_f64(double* y, const float* x, const float* w_oihw, const float* bias_o,
+                           size_t N, size_t C, size_t H, size_t W, size_t O,
+                           size_t K_h, size_t K_w, size_t stride, size_t pad, int relu);
+
+/* ---- Model::Linear graph, src/Model.cu:87-103 (+ optional ReLU):
+ * y[n][o] = relu(sum_i f16(Wt[o][i]) * f16(x[n][i]) + bias[o]); Wt is [OUT,IN]. */
+void nzo_linear_graph(float* y, const float* x, const float* w_out_in, const float* bias,
+                      size_t batch, size_t in_features, size_t out_features, int relu);
+
+/* ---- error metrics used by the tolerance contract */
+/* max over i of |got-truth| / max(|truth|, floor) and Frobenius ||got-truth|| / ||truth|| */
+void nzo_errors_f32_vs_f64(const float* got, const double* truth, size_t n, double floor_abs,
+                           double* max_rel, double* frob_rel);
+
+/* ---- seeded generators (documented PRNG: splitmix64-seeded xoshiro256**, one
+ * independent stream per block of 4096 elements so generation parallelises;
+ * normals by Box-Muller in double). kind: 0 uniform[lo,hi), 1 normal(mean=lo, std=hi) */
+void nzo_fill(float* dst, size_t n, uint64_t seed, int kind, double lo, double hi);
+
+int nzo_num_threads(void);
+void nzo_set_num_threads(int n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
