@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the fp32-in / fp16-MFMA / fp32-accumulate GEMM path on one MI355X.
+
+A "step" is one pass of the hot path over one batch of synthetic input: one 8192^3 GEMM
+(seeded N(0, 1/sqrt(K)) operands, resident in HBM before the timed region).  Prints ONE JSON
+line.  `--workload` selects another configuration for profiling runs (the default is the one
+the headline metric is quoted on)."""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS_FP16 = 2500.0      # MI355X dense fp16 MFMA
+PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="gemm8192",
+                    choices=["gemm8192", "gemm_batched", "linear", "gemv", "ragged", "conv_a", "conv_b"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary (conv / linear) measurements")
+    ap.add_argument("--no-verify", action="store_true")
+    return ap.parse_args()
+
+
+def dev(a):
+    import numpy as np
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+class Workload:
+    """name, algorithmic flops and bytes per step, a run() closure, and a verify() closure."""
+
+    def __init__(self, name, flops, bytes_, run, verify, bound, desc):
+        self.name, self.flops, self.bytes, self.run, self.verify, self.bound, self.desc = name, flops, bytes_, run, verify, bound, desc
+
+
+def tolerance(orc, got, truth, tag):
+    import numpy as np
+    rms = float(np.sqrt(np.mean(truth ** 2))) or 1.0
+    mr, fr = orc.errors(got, truth, rms)
+    if not (mr <= 1e-3 and fr <= 1e-4):
+        raise SystemExit(f"VERIFY FAILED {tag}: max_rel {mr:.3e} frob_rel {fr:.3e}")
+    return {"max_rel": mr, "frob_rel": fr}
+
+
+def make_workload(name, orc, capi):
+    import numpy as np
+    import torch
+    if name == "gemm8192":
+        n = 8192
+        A = orc.fill((n, n), 5, "normal", 0.0, 1.0 / np.sqrt(n))
+        B = orc.fill((n, n), 1005, "normal", 0.0, 1.0 / np.sqrt(n))
+        Ad, Bd = dev(A), dev(B)
+        out = torch.empty((n, n), device="cuda")
+
+        def run():
+            capi.gemm(Ad, Bd, out=out)
+
+        def verify():
+            rows = np.sort(np.random.default_rng(5).choice(n, size=16, replace=False))
+            truth = np.concatenate([orc.gemm_rows(A, B, int(r), 1, want32=False)[1] for r in rows])
+            return tolerance(orc, out[rows.tolist()].cpu().numpy(), truth, name)
+
+        return Workload(name, 2.0 * n ** 3, 3.0 * n * n * 4, run, verify, "mfma",
+                        "C[8192,8192] = f16(A)[8192,8192] * f16(B)[8192,8192], fp32 in/out, N(0,1/sqrt(K))"), (A, B)
+    if name == "gemm_batched":
+        shape = (8, 16, 1024, 1024)
+        A = orc.fill(shape, 6, "normal", 0.0, 1.0 / 32.0)
+        B = orc.fill(shape, 1006, "normal", 0.0, 1.0 / 32.0)
+        Ad, Bd = dev(A), dev(B)
+        out = torch.empty(shape, device="cuda")
+
+        def run():
+            capi.tensorcore_gemm(Ad, Bd, out=out)
+
+        def verify():
+            return tolerance(orc, out[3, 7].cpu().numpy(), orc.gemm_f64(A[3, 7], B[3, 7]), name)
+
+        return Workload(name, 2.0 * 128 * 1024 ** 3, 3.0 * 128 * 1024 * 1024 * 4, run, verify, "mfma",
+                        "[8,16,1024,1024] x [8,16,1024,1024] batched over (N,C)"), None
+    if name == "linear":
+        Nb, IN, OUT = 4096, 1024, 4096
+        X = orc.fill((Nb, IN), 2, "normal", 0.0, 1.0)
+        bound = float(np.sqrt(6.0 / IN))
+        Wt = orc.fill((OUT, IN), 1002, "uniform", -bound, bound)
+        bias = orc.fill((OUT,), 2002, "uniform", -0.03, 0.03)
+        Xd, Wd, bd = dev(X), dev(Wt), dev(bias)
+        out = torch.empty((Nb, OUT), device="cuda")
+
+        def run():
+            capi.gemm(Xd, Wd, b_trans=True, bias=bd, bias_strides=(0, 1), relu=True, out=out)
+
+        def verify():
+            truth = np.maximum(orc.gemm_f64(X[:256], Wt, trans_b=True) + bias[None, :].astype(np.float64), 0)
+            return tolerance(orc, out[:256].cpu().numpy(), truth, name)
+
+        return Workload(name, 2.0 * Nb * IN * OUT, 4.0 * (Nb * IN + IN * OUT + OUT + Nb * OUT), run, verify, "mfma",
+                        "Linear X[4096,1024] W[4096,1024]^T + bias, ReLU"), None
+    if name == "gemv":
+        a = orc.fill((1, 4096), 4, "uniform", -1.0, 1.0)
+        Bm = orc.fill((4096, 4096), 1004, "uniform", -1.0, 1.0)
+        ad, Bd = dev(a), dev(Bm)
+        out = torch.empty((1, 4096), device="cuda")
+
+        def run():
+            capi.gemm(ad, Bd, out=out)
+
+        def verify():
+            return tolerance(orc, out.cpu().numpy(), orc.gemm_f64(a, Bm), name)
+
+        return Workload(name, 2.0 * 4096 * 4096, 4.0 * (4096 + 4096 * 4096 + 4096), run, verify, "hbm",
+                        "A[1,4096] * B[4096,4096]"), None
+    if name == "ragged":
+        A = orc.fill((1000, 777), 3, "uniform", -1.0, 1.0)
+        B = orc.fill((777, 513), 1003, "uniform", -1.0, 1.0)
+        Ad, Bd = dev(A), dev(B)
+        out = torch.empty((1000, 513), device="cuda")
+
+        def run():
+            capi.gemm(Ad, Bd, out=out)
+
+        def verify():
+            return tolerance(orc, out.cpu().numpy(), orc.gemm_f64(A, B), name)
+
+        return Workload(name, 2.0 * 1000 * 777 * 513, 4.0 * (1000 * 777 + 777 * 513 + 1000 * 513), run, verify, "mfma",
+                        "A[1000,777] * B[777,513]"), None
+    if name in ("conv_a", "conv_b"):
+        if name == "conv_a":
+            N, C, H, W, O = 16, 64, 128, 128, 128
+            x = orc.fill((N, C, H, W), 4, "normal", 0.0, 1.0)
+        else:
+            N, C, H, W, O = 10, 3, 1024, 1024, 1
+            x = orc.fill((N, C, H, W), 14, "uniform", 0.0, 1.0)
+        w = orc.fill((O, C, 3, 3), 1004 if name == "conv_a" else 1014, "normal", 0.0, float(np.sqrt(2.0 / (C * 9))))
+        bias = orc.fill((O,), 2004 if name == "conv_a" else 2014, "uniform", -0.03, 0.03)
+        xd, wd, bd = dev(x), dev(orc.weights_oihw_to_ref(w)), dev(bias)
+        out = torch.empty((N, O, H, W), device="cuda")
+
+        def run():
+            capi.conv2d_forward(xd, wd, bd, 3, 3, 1, 1, bias_strides=(0, 1), relu=True, out=out)
+
+        def verify():
+            truth = orc.conv2d_direct_f64(x[:1], w, bias, 1, 1, relu=True)
+            return tolerance(orc, out[:1].cpu().numpy(), truth, name)
+
+        flops = 2.0 * N * H * W * C * 9 * O
+        bytes_ = 4.0 * (N * C * H * W + O * C * 9 + O + N * O * H * W)
+        return Workload(name, flops, bytes_, run, verify, "hbm",
+                        f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},3,3] s1 p1 + bias + ReLU"), None
+    raise ValueError(name)
+
+
+def time_steps(wl, steps, warmup):
+    """Times exactly `steps` runs with HIP events recorded on the stream the kernels are
+    launched on (torch's current stream), bracketed by device synchronisation."""
+    import torch
+    for _ in range(warmup):
+        wl.run()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        wl.run()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) / steps, wall * 1e3 / steps      # ms per step (device events, host wall)
+
+
+def cpu_baseline_gemm(orc, A, B, rows=4096):
+    """The oracle (a scalar-semantics port with OpenMP) on a bounded sample of the same workload:
+    the first `rows` rows of the 8192^3 product, every host core the process may use."""
+    n = A.shape[1]
+    orc.gemm_rows(A, B, 0, 64, want64=False)                      # warm-up (thread pool, page faults)
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        orc.gemm_rows(A, B, 0, rows, want64=False)
+        dt = time.perf_counter() - t0
+        best = dt if best is None or dt < best else best
+    return {"value": 2.0 * rows * n * B.shape[1] / best / 1e12, "unit": "TFLOP/s", "cores": orc.num_threads(),
+            "kind": "port", "sample": f"rows 0..{rows - 1} of the 8192^3 GEMM ({rows}x8192x8192), best of 2, {best:.2f} s"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU only (the path shards with no exchange; "
+              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    from neuzephyr_amd import capi
+    from oracle import oracle as orc     # checker + cpu_baseline only
+    capi.load()
+
+    wl, host_ops = make_workload(args.workload, orc, capi)
+    ms_dev, ms_wall = time_steps(wl, args.steps, args.warmup)
+    verified = None if args.no_verify else wl.verify()
+
+    tflops = wl.flops / (ms_dev * 1e-3) / 1e12
+    gbps = wl.bytes / (ms_dev * 1e-3) / 1e9
+    if wl.bound == "mfma":
+        roofline = {"bound": "mfma", "achieved": tflops, "peak": PEAK_TFLOPS_FP16, "unit": "TFLOP/s",
+                    "frac": tflops / PEAK_TFLOPS_FP16, "traffic": None}
+    else:
+        roofline = {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": gbps / PEAK_HBM_GBPS, "traffic": None}
+
+    extra = {}
+    if args.workload == "gemm8192" and not args.no_extra:
+        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched"):
+            torch.cuda.empty_cache()
+            w2, _ = make_workload(name, orc, capi)
+            ms2, _ = time_steps(w2, max(10, args.steps // 2), max(3, args.warmup // 2))
+            v2 = None if args.no_verify else w2.verify()
+            extra[name] = {"ms": ms2, "TFLOP/s": w2.flops / ms2 / 1e9, "GB/s": w2.bytes / ms2 / 1e6,
+                           "frac_mfma_peak": w2.flops / ms2 / 1e9 / PEAK_TFLOPS_FP16,
+                           "frac_hbm_peak": w2.bytes / ms2 / 1e6 / PEAK_HBM_GBPS, "verified": v2, "workload": w2.desc}
+            del w2
+
+    cpu = None
+    if args.workload == "gemm8192" and not args.no_cpu_baseline:
+        cpu = cpu_baseline_gemm(orc, *host_ops)
+
+    line = {
+        "metric": "fp16-MFMA TFLOP/s (% peak) on 8192^3 GEMM; Conv2d fwd GB/s (% HBM peak)",
+        "value": tflops if wl.bound == "mfma" else gbps,
+        "unit": "TFLOP/s" if wl.bound == "mfma" else "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_dev, "ms_per_step_host_wall": ms_wall,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (fp32 operands rounded RNE; fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": args.workload, "desc": wl.desc, "algorithmic_flops": wl.flops,
+                   "algorithmic_bytes": wl.bytes},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "verified": verified,
+        "conv_and_other_configs": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,149 @@
+/*
+ * nzhip.h -- C-ABI of the MI355X (gfx950) implementation of NeuZephyr's
+ * tensor-core GEMM path: fp32 operands rounded to fp16 (round-to-nearest-even),
+ * fp16 MFMA with fp32 accumulation, and what feeds and drains it (im2col,
+ * col2im, bias add, ReLU, Conv2d lowering, device allocator, stream manager).
+ *
+ * Conventions
+ *   - every pointer named A/B/C/in/out/x/w/y/bias is a DEVICE pointer (or pinned
+ *     host memory mapped into the device) to contiguous fp32 data owned by the
+ *     caller; the library never takes ownership;
+ *   - `stream` is a hipStream_t passed as void*; NULL is HIP's null stream.  All
+ *     compute entry points only enqueue work and return before it completes;
+ *   - return value: 0 = ok, negative = NZHIP_E_* (invalid argument etc., nothing
+ *     was enqueued), positive = a hipError_t raised by the runtime.  Nothing is
+ *     thrown across this boundary.  nzhip_last_error() returns a thread-local,
+ *     human-readable description of the last non-zero status;
+ *   - shapes given as size_t[4] are NeuZephyr Dimensions {n, c, h, w} of
+ *     contiguous NCHW tensors (reference: src/Dimension.cu:5-10).
+ *
+ * Line numbers cite the NeuZephyr sources each entry point replaces.
+ */
+#ifndef NZHIP_H
+#define NZHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NZHIP_OK 0
+#define NZHIP_E_INVALID (-1)      /* bad pointer / size / stride / enum */
+#define NZHIP_E_SHAPE (-2)        /* shapes are not broadcast compatible */
+#define NZHIP_E_UNSUPPORTED (-3)  /* valid request outside implemented limits */
+#define NZHIP_E_NOMEM (-4)        /* device allocation failed */
+
+#define NZHIP_ACT_NONE 0
+#define NZHIP_ACT_RELU 1          /* x > 0 ? x : 0  (NaN -> 0, -0 -> +0) */
+
+#define NZHIP_LAYOUT_ROW 0        /* operand as written: A is MxK, B is KxN, row-major */
+#define NZHIP_LAYOUT_TRANS 1      /* operand given transposed: A as KxM, B as NxK, row-major */
+
+/* ---- library ------------------------------------------------------------ */
+int nzhip_version(void);
+const char* nzhip_last_error(void);
+/* Device properties the library keys its launch shapes on (CU count, LDS per CU);
+ * 0 on success.  Also the cheapest "is a gfx950 GPU usable" probe. */
+int nzhip_device_info(int* cu_count, size_t* lds_bytes_per_cu, char* arch_name, size_t arch_name_len);
+
+/* ---- GEMM --------------------------------------------------------------- */
+/* General form of the path's one contraction.  For every (i, j) of a two-level
+ * batch (batch_n x batch_c):
+ *     C_ij[M,N] = act( f16(A_ij)[M,K] * f16(B_ij)[K,N] + bias_ij )
+ * with fp32 accumulation.  Replaces Padding + GeneralMatrixMulTensorKernel +
+ * Cutting (src/OperationKernels.cu:821-871) and the per-(n,c) launch loops of
+ * TensorCoreGEMMParallel (:914-1026); the fused bias/activation replaces
+ * MatrixAddKernel (:12-24) and RectifiedLinearUnitKernel (:230-235).
+ * Edges are predicated in-kernel: no padded copies exist.
+ * Strides are in elements; a batch stride of 0 broadcasts that operand.
+ * bias may be NULL; its element for output (m,n) of batch (i,j) is
+ *     bias[i*bias_stride_n_batch + j*bias_stride_c_batch + m*bias_stride_row + n*bias_stride_col]
+ * so a per-row vector, a per-column vector and a full [M,N] matrix are all expressible. */
+typedef struct nzhip_gemm_desc {
+    const float* A;
+    const float* B;
+    float* C;
+    int64_t M, N, K;
+    int64_t lda, ldb, ldc;        /* leading dimensions (row strides) of the arrays as stored */
+    int32_t a_layout;             /* NZHIP_LAYOUT_ROW: A[m*lda+k];  _TRANS: A[k*lda+m] */
+    int32_t b_layout;             /* NZHIP_LAYOUT_ROW: B[k*ldb+n];  _TRANS: B[n*ldb+k] */
+    int64_t batch_n, batch_c;     /* >= 1 */
+    int64_t a_stride_n, a_stride_c;
+    int64_t b_stride_n, b_stride_c;
+    int64_t c_stride_n, c_stride_c;
+    const float* bias;            /* optional */
+    int64_t bias_stride_row, bias_stride_col;
+    int64_t bias_stride_n, bias_stride_c;
+    int32_t activation;           /* NZHIP_ACT_* */
+    int32_t reserved;             /* must be 0 */
+} nzhip_gemm_desc;
+
+int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream);
+
+/* Drop-in for nz::data::iTensorCoreGEMM (include/NeuZephyr/TensorOperations.cuh:1021-1022,
+ * src/TensorOperations.cu:112-115 -> krnl::TensorCoreGEMMParallel, src/OperationKernels.cu:914-1026):
+ * M = A.h, N = B.w, K = A.w; loops over C's (n,c); an operand whose n (or c) is 1 is
+ * broadcast.  Like the reference it validates nothing beyond non-null pointers. */
+int nzhip_tensorcore_gemm(const float* A, const float* B, float* C, const size_t shapeA[4],
+                          const size_t shapeB[4], const size_t shapeC[4], void* stream);
+
+/* ---- conv lowering ------------------------------------------------------ */
+/* nz::data::iImg2col (TensorOperations.cuh:1108-1110; img2colKernel, OperationKernels.cu:1308-1328):
+ * out[b][ho*W_out+wo][c*K_h*K_w + r*K_w + s] = in[b][c][ho*stride-pad+r][wo*stride-pad+s] or 0. */
+int nzhip_im2col(float* out, const float* in, size_t H_out, size_t W_out, size_t C, size_t K_h,
+                 size_t K_w, size_t stride, size_t pad, size_t H_in, size_t W_in, size_t batch,
+                 void* stream);
+
+/* nz::data::iCol2img (TensorOperations.cuh:1132-1133; col2imgKernel, OperationKernels.cu:1364-1376):
+ * out[b][c][h][w] = in[b][(h*W_out+w)*C_out + c]. */
+int nzhip_col2im(float* out, const float* in, size_t H_out, size_t W_out, size_t C_out, size_t batches,
+                 void* stream);
+
+/* The whole Model::Conv2d graph (src/Model.cu:244-263: Img2Col -> MatMul -> Bias -> Col2Img,
+ * optionally followed by the ReLU node) as one fused call with no column matrix in HBM.
+ *   x      [N, C, H, W]
+ *   w_ref  [w_batch, 1, C*K_h*K_w, O], w_batch in {1, N}; row q = c*K_h*K_w + r*K_w + s
+ *   bias   optional; element for output (b, o, p = ho*W_out+wo) is
+ *          bias[p*bias_stride_pixel + o*bias_stride_channel]
+ *          (reference parameter [1,1,H_out*W_out,O]: pixel stride O, channel stride 1;
+ *           ordinary per-channel vector: pixel stride 0, channel stride 1)
+ *   y      [N, O, H_out, W_out] */
+int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref, const float* bias,
+                         size_t N, size_t C, size_t H, size_t W, size_t O, size_t K_h, size_t K_w,
+                         size_t stride, size_t pad, size_t w_batch, int64_t bias_stride_pixel,
+                         int64_t bias_stride_channel, int activation, void* stream);
+
+/* ---- unfused element-wise fallbacks -------------------------------------- */
+/* tensorMatrixAdd + MatrixAddKernel (TensorOperations.cuh:785-808, OperationKernels.cu:12-24):
+ * out[n][c][:] = a[n or 0][c or 0][:] + b[n or 0][c or 0][:]; h, w must agree, n and c broadcast. */
+int nzhip_add_broadcast(float* out, const float* a, const float* b, const size_t shapeOut[4],
+                        const size_t shapeA[4], const size_t shapeB[4], void* stream);
+
+/* nz::data::iRELU (TensorOperations.cuh:19; RectifiedLinearUnitKernel, OperationKernels.cu:230-235). */
+int nzhip_relu(float* out, const float* in, size_t n, void* stream);
+
+/* ---- runtime: device allocator + stream manager -------------------------- */
+/* Replace cuStrm::StreamManager<float> (include/NeuZephyr/StreamManager.cuh:131-911) and
+ * EventPool (EventPool.cuh:165-457).  One ordered compute stream carries every kernel and
+ * every stream-ordered allocation, so producer/consumer order needs no per-buffer events;
+ * nzhip_sync_ptr / nzhip_sync_all are the only blocking calls. */
+void* nzhip_default_stream(void);                 /* the manager's compute stream (hipStream_t) */
+int nzhip_malloc(void** ptr, size_t bytes);       /* StreamManager::malloc (:230-240); size in BYTES */
+int nzhip_free_async(void* ptr);                  /* StreamManager::freeAsync (:325-335): stream-ordered, cached */
+int nzhip_free(void* ptr);                        /* StreamManager::free (:263): blocks until users finished */
+int nzhip_memset(void* ptr, int value, size_t bytes);                 /* :360 */
+int nzhip_memcpy_h2d(void* dst, const void* src, size_t bytes);       /* :391, async w.r.t. device */
+int nzhip_memcpy_d2d(void* dst, const void* src, size_t bytes);
+int nzhip_memcpy_d2h(void* dst, const void* src, size_t bytes);       /* blocks until the copy landed */
+int nzhip_sync_ptr(const void* ptr);              /* StreamManager::syncData (:714): wait for work touching ptr */
+int nzhip_sync_all(void);                         /* StreamManager::sync (:671) */
+/* allocator statistics (bytes handed out, bytes cached, hipMalloc calls so far) */
+int nzhip_allocator_stats(size_t* bytes_in_use, size_t* bytes_cached, size_t* device_allocs);
+int nzhip_allocator_trim(void);                   /* return cached blocks to the driver */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NZHIP_H */

@@ -1,0 +1,205 @@
+"""ctypes view of the C-ABI in include/nzhip.h (test and benchmark plumbing).
+
+No fallback of any kind lives here: if libnzhip.so is missing or a call fails, an exception
+is raised.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+ACT_NONE, ACT_RELU = 0, 1
+LAYOUT_ROW, LAYOUT_TRANS = 0, 1
+
+EXPORTS = [
+    "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_tensorcore_gemm",
+    "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
+    "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
+    "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
+    "nzhip_allocator_stats", "nzhip_allocator_trim",
+]
+
+
+class NzHipError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"nzhip status {status}: {message}")
+        self.status = status
+        self.message = message
+
+
+class GemmDesc(C.Structure):
+    _fields_ = [
+        ("A", C.c_void_p), ("B", C.c_void_p), ("C", C.c_void_p),
+        ("M", C.c_int64), ("N", C.c_int64), ("K", C.c_int64),
+        ("lda", C.c_int64), ("ldb", C.c_int64), ("ldc", C.c_int64),
+        ("a_layout", C.c_int32), ("b_layout", C.c_int32),
+        ("batch_n", C.c_int64), ("batch_c", C.c_int64),
+        ("a_stride_n", C.c_int64), ("a_stride_c", C.c_int64),
+        ("b_stride_n", C.c_int64), ("b_stride_c", C.c_int64),
+        ("c_stride_n", C.c_int64), ("c_stride_c", C.c_int64),
+        ("bias", C.c_void_p),
+        ("bias_stride_row", C.c_int64), ("bias_stride_col", C.c_int64),
+        ("bias_stride_n", C.c_int64), ("bias_stride_c", C.c_int64),
+        ("activation", C.c_int32), ("reserved", C.c_int32),
+    ]
+
+
+def lib_path() -> str:
+    return os.path.join(HERE, "libnzhip.so")
+
+
+def load() -> C.CDLL:
+    """Load libnzhip.so (built in-tree by neuzephyr_amd/build.py). Raises if it is absent."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    path = lib_path()
+    if not os.path.exists(path):
+        raise FileNotFoundError(f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'`")
+    lib = C.CDLL(path)
+    sz, vp, i64 = C.c_size_t, C.c_void_p, C.c_int64
+    shape = C.c_size_t * 4
+    lib.nzhip_version.restype = C.c_int
+    lib.nzhip_last_error.restype = C.c_char_p
+    lib.nzhip_device_info.argtypes = [C.POINTER(C.c_int), C.POINTER(sz), C.c_char_p, sz]
+    lib.nzhip_gemm.argtypes = [C.POINTER(GemmDesc), vp]
+    lib.nzhip_gemm_force_tile.argtypes = [C.POINTER(GemmDesc), C.c_int, vp]
+    lib.nzhip_tensorcore_gemm.argtypes = [vp, vp, vp, shape, shape, shape, vp]
+    lib.nzhip_im2col.argtypes = [vp, vp] + [sz] * 10 + [vp]
+    lib.nzhip_col2im.argtypes = [vp, vp, sz, sz, sz, sz, vp]
+    lib.nzhip_conv2d_forward.argtypes = [vp, vp, vp, vp] + [sz] * 10 + [i64, i64, C.c_int, vp]
+    lib.nzhip_add_broadcast.argtypes = [vp, vp, vp, shape, shape, shape, vp]
+    lib.nzhip_relu.argtypes = [vp, vp, sz, vp]
+    lib.nzhip_default_stream.restype = vp
+    lib.nzhip_malloc.argtypes = [C.POINTER(vp), sz]
+    lib.nzhip_free_async.argtypes = [vp]
+    lib.nzhip_free.argtypes = [vp]
+    lib.nzhip_memset.argtypes = [vp, C.c_int, sz]
+    for n in ("nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h"):
+        getattr(lib, n).argtypes = [vp, vp, sz]
+    lib.nzhip_sync_ptr.argtypes = [vp]
+    lib.nzhip_allocator_stats.argtypes = [C.POINTER(sz), C.POINTER(sz), C.POINTER(sz)]
+    _LIB = lib
+    return lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise NzHipError(status, load().nzhip_last_error().decode(errors="replace"))
+
+
+def shape4(s) -> C.Array:
+    return (C.c_size_t * 4)(*[int(v) for v in s])
+
+
+# --------------------------------------------------------------------------------------------
+# Torch-facing helpers. torch is used for device memory and streams only.
+# --------------------------------------------------------------------------------------------
+def _stream_handle(stream=None) -> int:
+    import torch
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return int(s.cuda_stream)
+
+
+def _dev(t):
+    import torch
+    assert t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), "expects contiguous fp32 CUDA tensors"
+    return t.data_ptr()
+
+
+def gemm(A, B, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), relu=False, out=None,
+         force_tile=0, stream=None):
+    """C = act(f16(A) @ f16(B) + bias) for 2-D tensors. a_trans: A holds K x M; b_trans: B holds N x K.
+    bias_strides = (row stride, column stride) in elements."""
+    import torch
+    lib = load()
+    M, K = (A.shape[1], A.shape[0]) if a_trans else A.shape
+    N = B.shape[0] if b_trans else B.shape[1]
+    assert (B.shape[1] if b_trans else B.shape[0]) == K
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=A.device)
+    d = GemmDesc()
+    d.A, d.B, d.C = _dev(A), _dev(B), _dev(out)
+    d.M, d.N, d.K = M, N, K
+    d.lda, d.ldb, d.ldc = A.shape[1], B.shape[1], N
+    d.a_layout = LAYOUT_TRANS if a_trans else LAYOUT_ROW
+    d.b_layout = LAYOUT_TRANS if b_trans else LAYOUT_ROW
+    d.batch_n = d.batch_c = 1
+    if bias is not None:
+        d.bias = _dev(bias)
+        d.bias_stride_row, d.bias_stride_col = bias_strides
+    d.activation = ACT_RELU if relu else ACT_NONE
+    if force_tile:
+        check(lib.nzhip_gemm_force_tile(C.byref(d), force_tile, _stream_handle(stream)))
+    else:
+        check(lib.nzhip_gemm(C.byref(d), _stream_handle(stream)))
+    return out
+
+
+def tensorcore_gemm(A, B, out=None, stream=None):
+    """4-D batched/broadcast product with the semantics of nz::data::iTensorCoreGEMM."""
+    import torch
+    lib = load()
+    sa, sb = tuple(A.shape), tuple(B.shape)
+    sc = (max(sa[0], sb[0]), max(sa[1], sb[1]), sa[2], sb[3])
+    if out is None:
+        out = torch.empty(sc, dtype=torch.float32, device=A.device)
+    check(lib.nzhip_tensorcore_gemm(_dev(A), _dev(B), _dev(out), shape4(sa), shape4(sb), shape4(tuple(out.shape)),
+                                    _stream_handle(stream)))
+    return out
+
+
+def im2col(x, K_h, K_w, stride, pad, stream=None):
+    import torch
+    lib = load()
+    N, Cc, H, W = x.shape
+    Ho, Wo = (H + 2 * pad - K_h) // stride + 1, (W + 2 * pad - K_w) // stride + 1
+    out = torch.empty((N, 1, Ho * Wo, Cc * K_h * K_w), dtype=torch.float32, device=x.device)
+    check(lib.nzhip_im2col(_dev(out), _dev(x), Ho, Wo, Cc, K_h, K_w, stride, pad, H, W, N, _stream_handle(stream)))
+    return out
+
+
+def col2im(col, Ho, Wo, stream=None):
+    import torch
+    lib = load()
+    N, _, HW, O = col.shape
+    out = torch.empty((N, O, Ho, Wo), dtype=torch.float32, device=col.device)
+    check(lib.nzhip_col2im(_dev(out), _dev(col), Ho, Wo, O, N, _stream_handle(stream)))
+    return out
+
+
+def conv2d_forward(x, w_ref, bias, K_h, K_w, stride, pad, *, bias_strides=(0, 1), relu=False, out=None, stream=None):
+    """x [N,C,H,W]; w_ref [Wb,1,C*Kh*Kw,O]; bias_strides = (pixel stride, channel stride)."""
+    import torch
+    lib = load()
+    N, Cc, H, W = x.shape
+    Wb, _, CKK, O = w_ref.shape
+    assert CKK == Cc * K_h * K_w
+    Ho, Wo = (H + 2 * pad - K_h) // stride + 1, (W + 2 * pad - K_w) // stride + 1
+    if out is None:
+        out = torch.empty((N, O, Ho, Wo), dtype=torch.float32, device=x.device)
+    check(lib.nzhip_conv2d_forward(_dev(out), _dev(x), _dev(w_ref), None if bias is None else _dev(bias), N, Cc, H, W,
+                                   O, K_h, K_w, stride, pad, Wb, bias_strides[0], bias_strides[1],
+                                   ACT_RELU if relu else ACT_NONE, _stream_handle(stream)))
+    return out
+
+
+def add_broadcast(a, b, stream=None):
+    import torch
+    lib = load()
+    so = (max(a.shape[0], b.shape[0]), max(a.shape[1], b.shape[1]), a.shape[2], a.shape[3])
+    out = torch.empty(so, dtype=torch.float32, device=a.device)
+    check(lib.nzhip_add_broadcast(_dev(out), _dev(a), _dev(b), shape4(so), shape4(a.shape), shape4(b.shape),
+                                  _stream_handle(stream)))
+    return out
+
+
+def relu(a, stream=None):
+    import torch
+    lib = load()
+    out = torch.empty_like(a)
+    check(lib.nzhip_relu(_dev(out), _dev(a), a.numel(), _stream_handle(stream)))
+    return out

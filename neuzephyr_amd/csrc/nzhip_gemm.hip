@@ -1,0 +1,382 @@
+// fp32-in / fp16-MFMA / fp32-accumulate GEMM for gfx950 (MI355X).
+//
+// One kernel family replaces the reference's Padding -> GeneralMatrixMulTensorKernel
+// -> Cutting pipeline (src/OperationKernels.cu:821-871) and its per-(n,c) launch
+// loops (:914-1026):
+//   * operands are read as fp32 straight from the caller's buffers, rounded to
+//     fp16 (v_cvt_pk_f16_f32, round-to-nearest-even) on the way into LDS;
+//   * v_mfma_f32_32x32x16_f16 with fp32 accumulators;
+//   * two LDS stages (one barrier per k tile), rows padded by 16 B so that the
+//     128-bit fragment reads and the staging writes hit distinct banks;
+//   * edges are predicated (zero fill on load, masked store) -- no padded copies;
+//   * batch (n,c), broadcast strides, bias and ReLU are handled in-kernel.
+#include <hip/hip_runtime.h>
+
+#include "nzhip_internal.h"
+
+namespace nzhip {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+struct GemmKernelArgs {
+    const float* A;
+    const float* B;
+    float* C;
+    const float* bias;
+    int M, N, K;
+    long lda, ldb, ldc;
+    int batch_c;                      // inner batch extent (grid.y = batch_n * batch_c)
+    long a_sn, a_sc, b_sn, b_sc, c_sn, c_sc, bias_sn, bias_sc;
+    long bias_sm, bias_sk;            // bias row / column strides
+    int relu;
+    int tiles_m, tiles_n;
+    int group_m;                      // tile rows per rasterisation group
+};
+
+// Physical LDS row of logical tile row r. A wave owns TR = 32*FR logical rows; its MFMA
+// block f (0..FR-1) takes the rows r with (r % TR) % FR == f, so that (a) the 32 rows one
+// fragment read touches are consecutive in LDS and (b) each lane ends up holding FR
+// consecutive output columns, which makes the C store a vector store.
+template <int TR, int FR>
+__device__ __forceinline__ int phys_row(int r) {
+    const int w = r / TR, l = r % TR;
+    return (w * FR + (l % FR)) * 32 + l / FR;
+}
+
+// ---- operand staging: global fp32 -> registers -> fp16 in LDS ----------------------------
+// KCONTIG: the operand is stored with k contiguous (A row-major MxK, or B given as NxK).
+template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC>
+struct StageKContig {
+    static constexpr int F4_PER_ROW = BK / 4;
+    static constexpr int ROWS_PER_PASS = NT / F4_PER_ROW;
+    static constexpr int PASSES = BR / ROWS_PER_PASS;
+    static_assert(BR % ROWS_PER_PASS == 0 && PASSES >= 1, "tile/thread mismatch");
+    floatx4 regs[PASSES];
+
+    __device__ __forceinline__ void load(const float* __restrict__ X, long ldx, int row_base, int R, int k_base,
+                                         int K, int tid) {
+        const int k4 = tid % F4_PER_ROW, r0 = tid / F4_PER_ROW;
+        const int gk = k_base + k4 * 4;
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            const int gr = row_base + r0 + p * ROWS_PER_PASS;
+            const float* src = X + (long)gr * ldx + gk;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (gr < R) {
+                if (VEC) {
+                    if (gk < K) v = *reinterpret_cast<const floatx4*>(src);
+                } else {
+                    if (gk + 0 < K) v[0] = src[0];
+                    if (gk + 1 < K) v[1] = src[1];
+                    if (gk + 2 < K) v[2] = src[2];
+                    if (gk + 3 < K) v[3] = src[3];
+                }
+            }
+            regs[p] = v;
+        }
+    }
+
+    __device__ __forceinline__ void store(char* lds, int tid) const {
+        const int k4 = tid % F4_PER_ROW, r0 = tid / F4_PER_ROW;
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            const int r = r0 + p * ROWS_PER_PASS;
+            half4_t h;
+            h[0] = (_Float16)regs[p][0];
+            h[1] = (_Float16)regs[p][1];
+            h[2] = (_Float16)regs[p][2];
+            h[3] = (_Float16)regs[p][3];
+            *reinterpret_cast<half4_t*>(lds + phys_row<TR, FR>(r) * ROWB + k4 * 8) = h;
+        }
+    }
+};
+
+// RCONTIG: the operand is stored with the tile dimension contiguous (B row-major KxN, or
+// A given as KxM). Each thread takes 4 neighbouring tile rows over KPT consecutive k and
+// transposes them in registers, so LDS still holds k-contiguous rows.
+template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC>
+struct StageRContig {
+    static constexpr int F4_PER_KROW = BR / 4;
+    static constexpr int KGROUPS = NT / F4_PER_KROW;
+    static constexpr int KPT = BK / KGROUPS;
+    static_assert(NT % F4_PER_KROW == 0 && KGROUPS >= 1 && BK % KGROUPS == 0, "tile/thread mismatch");
+    static_assert(KPT == 2 || KPT == 4 || KPT == 8, "k per thread must be 2, 4 or 8");
+    floatx4 regs[KPT];
+
+    __device__ __forceinline__ void load(const float* __restrict__ X, long ldx, int row_base, int R, int k_base,
+                                         int K, int tid) {
+        const int r4 = tid % F4_PER_KROW, kg = tid / F4_PER_KROW;
+        const int gr = row_base + r4 * 4;
+#pragma unroll
+        for (int q = 0; q < KPT; q++) {
+            const int gk = k_base + kg * KPT + q;
+            const float* src = X + (long)gk * ldx + gr;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (gk < K) {
+                if (VEC) {
+                    if (gr < R) v = *reinterpret_cast<const floatx4*>(src);
+                } else {
+                    if (gr + 0 < R) v[0] = src[0];
+                    if (gr + 1 < R) v[1] = src[1];
+                    if (gr + 2 < R) v[2] = src[2];
+                    if (gr + 3 < R) v[3] = src[3];
+                }
+            }
+            regs[q] = v;
+        }
+    }
+
+    __device__ __forceinline__ void store(char* lds, int tid) const {
+        const int r4 = tid % F4_PER_KROW, kg = tid / F4_PER_KROW;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            char* dst = lds + phys_row<TR, FR>(r4 * 4 + e) * ROWB + kg * KPT * 2;
+            if constexpr (KPT == 8) {
+                half8_t h;
+#pragma unroll
+                for (int q = 0; q < 8; q++) h[q] = (_Float16)regs[q][e];
+                *reinterpret_cast<half8_t*>(dst) = h;
+            } else if constexpr (KPT == 4) {
+                half4_t h;
+#pragma unroll
+                for (int q = 0; q < 4; q++) h[q] = (_Float16)regs[q][e];
+                *reinterpret_cast<half4_t*>(dst) = h;
+            } else {
+                half2_t h;
+                h[0] = (_Float16)regs[0][e];
+                h[1] = (_Float16)regs[1][e];
+                *reinterpret_cast<half2_t*>(dst) = h;
+            }
+        }
+    }
+};
+
+template <bool RCONTIG, int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC>
+struct StageSelect {
+    using type = StageKContig<BR, BK, NT, TR, FR, ROWB, VEC>;
+};
+template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC>
+struct StageSelect<true, BR, BK, NT, TR, FR, ROWB, VEC> {
+    using type = StageRContig<BR, BK, NT, TR, FR, ROWB, VEC>;
+};
+
+// ---- the kernel ----------------------------------------------------------------------------
+// BM x BN x BK workgroup tile, WM x WN waves, each wave a (BM/WM) x (BN/WN) tile of 32x32 MFMA
+// blocks.  A_TRANS: A given as KxM.  B_TRANS: B given as NxK.  VEC: 16-byte global accesses
+// are legal for both operands (alignment and extents checked on the host).
+template <int BM, int BN, int BK, int WM, int WN, bool A_TRANS, bool B_TRANS, bool VEC>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKernelArgs p) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM, TN = BN / WN;
+    constexpr int FM = TM / 32, FN = TN / 32;
+    constexpr int ROWB = BK * 2 + 16;                     // LDS row pitch in bytes
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB;
+    constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+    static_assert(TM % 32 == 0 && TN % 32 == 0 && BK % 16 == 0, "tile shape");
+
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int li = lane & 31, lh = lane >> 5;
+
+    // ---- which tile: spread consecutive ids over the 8 XCDs, then walk column-major inside
+    // groups of group_m tile rows so that the workgroups resident on one XCD share A rows
+    // and B columns in that XCD's L2.
+    const int total = p.tiles_m * p.tiles_n;
+    int lin = blockIdx.x;
+    {
+        const int xcd = lin & 7, q = lin >> 3;
+        const int per = total >> 3, rem = total & 7;
+        lin = xcd * per + (xcd < rem ? xcd : rem) + q;
+    }
+    const int group_sz = p.group_m * p.tiles_n;
+    const int group = lin / group_sz;
+    const int first_m = group * p.group_m;
+    const int rows_in_group = (p.tiles_m - first_m) < p.group_m ? (p.tiles_m - first_m) : p.group_m;
+    const int tile_m = first_m + (lin % group_sz) % rows_in_group;
+    const int tile_n = (lin % group_sz) / rows_in_group;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int bi = blockIdx.y / p.batch_c, bj = blockIdx.y % p.batch_c;
+    const float* __restrict__ A = p.A + bi * p.a_sn + bj * p.a_sc;
+    const float* __restrict__ B = p.B + bi * p.b_sn + bj * p.b_sc;
+    float* __restrict__ C = p.C + bi * p.c_sn + bj * p.c_sc;
+
+    typename StageSelect<A_TRANS, BM, BK, NT, TM, FM, ROWB, VEC>::type sa;
+    typename StageSelect<!B_TRANS, BN, BK, NT, TN, FN, ROWB, VEC>::type sb;
+
+    floatx16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    const int nk = (p.K + BK - 1) / BK;
+
+    sa.load(A, p.lda, m0, p.M, 0, p.K, tid);
+    sb.load(B, p.ldb, n0, p.N, 0, p.K, tid);
+    sa.store(lds, tid);
+    sb.store(lds + A_BYTES, tid);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; kt++) {
+        char* cur = lds + (kt & 1) * STAGE_BYTES;
+        char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+        const bool more = kt + 1 < nk;
+        if (more) {
+            sa.load(A, p.lda, m0, p.M, (kt + 1) * BK, p.K, tid);
+            sb.load(B, p.ldb, n0, p.N, (kt + 1) * BK, p.K, tid);
+        }
+        const char* la = cur + ((wm * FM) * 32 + li) * ROWB + lh * 16;
+        const char* lb = cur + A_BYTES + ((wn * FN) * 32 + li) * ROWB + lh * 16;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) {
+            half8_t af[FM], bf[FN];
+#pragma unroll
+            for (int i = 0; i < FM; i++) af[i] = *reinterpret_cast<const half8_t*>(la + i * 32 * ROWB + ks * 32);
+#pragma unroll
+            for (int j = 0; j < FN; j++) bf[j] = *reinterpret_cast<const half8_t*>(lb + j * 32 * ROWB + ks * 32);
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            sa.store(nxt, tid);
+            sb.store(nxt + A_BYTES, tid);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: bias, activation, predicated (vector when legal) store ------------------
+    const float* bias = p.bias ? p.bias + bi * p.bias_sn + bj * p.bias_sc : nullptr;
+    const int gn = n0 + wn * TN + li * FN;                // first of this lane's FN columns
+    const bool vec_store = VEC && (FN == 2 || FN == 4) && (gn + FN <= p.N);
+#pragma unroll
+    for (int i = 0; i < FM; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int im = (r >> 2) * 8 + lh * 4 + (r & 3);
+            const int gm = m0 + wm * TM + im * FM + i;
+            if (gm >= p.M) continue;
+            float v[FN];
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                float x = acc[i][j][r];
+                if (bias && gn + j < p.N) x += bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk];
+                if (p.relu) x = x > 0.f ? x : 0.f;
+                v[j] = x;
+            }
+            float* dst = C + (long)gm * p.ldc + gn;
+            if (vec_store) {
+                if constexpr (FN == 4) {
+                    floatx4 o = {v[0], v[1], v[2], v[3]};
+                    *reinterpret_cast<floatx4*>(dst) = o;
+                } else if constexpr (FN == 2) {
+                    floatx2 o = {v[0], v[1]};
+                    *reinterpret_cast<floatx2*>(dst) = o;
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+                    if (gn + j < p.N) dst[j] = v[j];
+            }
+        }
+    }
+}
+
+// ---- host-side selection -------------------------------------------------------------------
+template <int BM, int BN, int BK, int WM, int WN>
+static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool vec, int batch, hipStream_t s) {
+    constexpr int ROWB = BK * 2 + 16;
+    constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * ROWB;
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch, 1), block(WM * WN * 64, 1, 1);
+#define NZHIP_LAUNCH(AT, BT, V)                                                                          \
+    do {                                                                                                 \
+        auto kfn = gemm_f16mfma_kernel<BM, BN, BK, WM, WN, AT, BT, V>;                                   \
+        static bool attr_set = false;                                                                    \
+        if (!attr_set) {                                                                                 \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                       \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); \
+            if (e != hipSuccess) return set_hip_error(e, "hipFuncSetAttribute(gemm)");                   \
+            attr_set = true;                                                                             \
+        }                                                                                                \
+        hipLaunchKernelGGL(kfn, grid, block, lds_bytes, s, a);                                           \
+    } while (0)
+    if (vec) {
+        if (!a_trans && !b_trans) NZHIP_LAUNCH(false, false, true);
+        else if (!a_trans && b_trans) NZHIP_LAUNCH(false, true, true);
+        else if (a_trans && !b_trans) NZHIP_LAUNCH(true, false, true);
+        else NZHIP_LAUNCH(true, true, true);
+    } else {
+        if (!a_trans && !b_trans) NZHIP_LAUNCH(false, false, false);
+        else if (!a_trans && b_trans) NZHIP_LAUNCH(false, true, false);
+        else if (a_trans && !b_trans) NZHIP_LAUNCH(true, false, false);
+        else NZHIP_LAUNCH(true, true, false);
+    }
+#undef NZHIP_LAUNCH
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return set_hip_error(e, "gemm kernel launch");
+    return NZHIP_OK;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile) {
+    GemmKernelArgs a;
+    a.A = d.A;
+    a.B = d.B;
+    a.C = d.C;
+    a.bias = d.bias;
+    a.M = (int)d.M;
+    a.N = (int)d.N;
+    a.K = (int)d.K;
+    a.lda = d.lda;
+    a.ldb = d.ldb;
+    a.ldc = d.ldc;
+    a.batch_c = (int)d.batch_c;
+    a.a_sn = d.a_stride_n;
+    a.a_sc = d.a_stride_c;
+    a.b_sn = d.b_stride_n;
+    a.b_sc = d.b_stride_c;
+    a.c_sn = d.c_stride_n;
+    a.c_sc = d.c_stride_c;
+    a.bias_sn = d.bias_stride_n;
+    a.bias_sc = d.bias_stride_c;
+    a.bias_sm = d.bias_stride_row;
+    a.bias_sk = d.bias_stride_col;
+    a.relu = d.activation == NZHIP_ACT_RELU;
+
+    const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
+    // 16-byte accesses are legal when every row start is 16-byte aligned and the contiguous
+    // extent is a multiple of 4, for every batch member.
+    auto ok4 = [](int64_t v) { return (v & 3) == 0; };
+    const int64_t a_contig = a_trans ? d.M : d.K, b_contig = b_trans ? d.K : d.N;
+    const bool vec = aligned16(d.A) && aligned16(d.B) && aligned16(d.C) && ok4(d.lda) && ok4(d.ldb) && ok4(d.ldc) &&
+                     ok4(a_contig) && ok4(b_contig) && ok4(d.N) && ok4(d.a_stride_n) && ok4(d.a_stride_c) &&
+                     ok4(d.b_stride_n) && ok4(d.b_stride_c) && ok4(d.c_stride_n) && ok4(d.c_stride_c);
+    const int64_t batch = d.batch_n * d.batch_c;
+
+    // Tile choice: 256x256 tiles need enough of them to fill the 256 CUs; otherwise 128x128.
+    const int64_t t256 = ((d.M + 255) / 256) * ((d.N + 255) / 256) * batch;
+    int tile = force_tile ? force_tile : (t256 >= 192 ? 256 : 128);
+    const int bm = tile, bn = tile;
+    a.tiles_m = (int)((d.M + bm - 1) / bm);
+    a.tiles_n = (int)((d.N + bn - 1) / bn);
+    // rows per rasterisation group: with 32 workgroups resident per XCD aim at a 4x8 footprint
+    a.group_m = 4;
+    if (tile == 256) return launch_cfg<256, 256, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
+    return launch_cfg<128, 128, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
+}
+
+}  // namespace nzhip

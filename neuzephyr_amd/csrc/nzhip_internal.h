@@ -1,0 +1,27 @@
+// Internal declarations shared by the translation units of libnzhip.so.
+#ifndef NZHIP_INTERNAL_H
+#define NZHIP_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/nzhip.h"
+
+namespace nzhip {
+
+// Record a failure for nzhip_last_error() and return the status to hand to the caller.
+int set_error(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int set_hip_error(hipError_t e, const char* what);
+
+// MFMA tile kernels (nzhip_gemm.hip). force_tile: 0 = choose, 128 / 256 = that square tile.
+int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile);
+// Bandwidth-bound kernels for M <= 8 (nzhip_skinny.hip).
+int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
+bool gemm_skinny_applicable(const nzhip_gemm_desc& d);
+
+// Stream-ordered workspace from the caching allocator (nzhip_runtime.cpp).
+int workspace_alloc(void** ptr, size_t bytes, hipStream_t stream);
+int workspace_free(void* ptr, hipStream_t stream);
+
+}  // namespace nzhip
+
+#endif

@@ -1,0 +1,198 @@
+// Runtime of libnzhip.so: error reporting, the device caching allocator and the stream
+// manager. Replaces cuStrm::StreamManager<float> + EventPool of the reference
+// (include/NeuZephyr/StreamManager.cuh:131-911, EventPool.cuh:165-457).
+//
+// Design: ONE ordered compute stream. The reference hands every op a different one of 16
+// streams and then re-creates the order with per-buffer events plus a host callback per op;
+// since batches, broadcasts and epilogues run inside single kernels here, there is nothing
+// left to overlap, and stream order itself is the dependency tracker. Blocking happens only
+// in nzhip_sync_ptr / nzhip_sync_all / nzhip_memcpy_d2h / nzhip_free.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+#include "nz_pool_allocator.hpp"
+#include "nzhip_internal.h"
+
+namespace nzhip {
+
+static thread_local char g_err[512] = "";
+
+int set_error(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int set_hip_error(hipError_t e, const char* what) {
+    snprintf(g_err, sizeof(g_err), "%s: %s (hipError_t %d)", what, hipGetErrorString(e), (int)e);
+    return (int)e;
+}
+
+struct HipBackend {
+    int raw_alloc(void** p, size_t bytes) {
+        hipError_t e = hipMalloc(p, bytes);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();   // clear the sticky error so the retry path starts clean
+            *p = nullptr;
+        }
+        return (int)e;
+    }
+    int raw_free(void* p) { return (int)hipFree(p); }
+};
+
+class Runtime {
+public:
+    static Runtime& instance() {
+        static Runtime* rt = new Runtime();   // intentionally leaked: no teardown races at exit
+        return *rt;
+    }
+    int ensure_stream() {
+        std::call_once(once_, [this] {
+            hipError_t e = hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking);
+            if (e != hipSuccess) {
+                init_status_ = set_hip_error(e, "hipStreamCreateWithFlags");
+                stream_ = nullptr;
+            }
+        });
+        return init_status_;
+    }
+    hipStream_t stream() {
+        ensure_stream();
+        return stream_;
+    }
+    PoolAllocator<HipBackend>& pool() { return pool_; }
+
+private:
+    Runtime() = default;
+    std::once_flag once_;
+    int init_status_ = 0;
+    hipStream_t stream_ = nullptr;
+    PoolAllocator<HipBackend> pool_;
+};
+
+int workspace_alloc(void** ptr, size_t bytes, hipStream_t s) {
+    int rc = Runtime::instance().pool().allocate(ptr, bytes, reinterpret_cast<uintptr_t>(s));
+    if (rc != 0) return set_error(NZHIP_E_NOMEM, "workspace allocation of %zu bytes failed (hipError_t %d)", bytes, rc);
+    return NZHIP_OK;
+}
+
+int workspace_free(void* ptr, hipStream_t s) {
+    return Runtime::instance().pool().free_async(ptr, reinterpret_cast<uintptr_t>(s)) == 0
+               ? NZHIP_OK
+               : set_error(NZHIP_E_INVALID, "workspace_free: unknown pointer");
+}
+
+}  // namespace nzhip
+
+using namespace nzhip;
+
+extern "C" {
+
+int nzhip_version(void) { return 100; }
+
+const char* nzhip_last_error(void) { return g_err; }
+
+int nzhip_device_info(int* cu_count, size_t* lds_bytes_per_cu, char* arch_name, size_t arch_name_len) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_hip_error(e, "hipGetDevice");
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return set_hip_error(e, "hipGetDeviceProperties");
+    if (cu_count) *cu_count = prop.multiProcessorCount;
+    if (lds_bytes_per_cu) *lds_bytes_per_cu = prop.maxSharedMemoryPerMultiProcessor;
+    if (arch_name && arch_name_len) {
+        strncpy(arch_name, prop.gcnArchName, arch_name_len - 1);
+        arch_name[arch_name_len - 1] = '\0';
+    }
+    return NZHIP_OK;
+}
+
+void* nzhip_default_stream(void) { return Runtime::instance().stream(); }
+
+int nzhip_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return set_error(NZHIP_E_INVALID, "nzhip_malloc: null out-pointer");
+    Runtime& rt = Runtime::instance();
+    if (int rc = rt.ensure_stream()) return rc;
+    int rc = rt.pool().allocate(ptr, bytes, reinterpret_cast<uintptr_t>(rt.stream()));
+    if (rc != 0) return set_error(NZHIP_E_NOMEM, "nzhip_malloc: %zu bytes: hipError_t %d", bytes, rc);
+    return NZHIP_OK;
+}
+
+int nzhip_free_async(void* ptr) {
+    Runtime& rt = Runtime::instance();
+    if (rt.pool().free_async(ptr, reinterpret_cast<uintptr_t>(rt.stream())) != 0)
+        return set_error(NZHIP_E_INVALID, "nzhip_free_async: pointer %p is not a live nzhip allocation", ptr);
+    return NZHIP_OK;
+}
+
+int nzhip_free(void* ptr) {
+    if (!ptr) return NZHIP_OK;
+    Runtime& rt = Runtime::instance();
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return set_hip_error(e, "hipDeviceSynchronize");
+    if (rt.pool().free_now(ptr) != 0)
+        return set_error(NZHIP_E_INVALID, "nzhip_free: pointer %p is not a live nzhip allocation", ptr);
+    return NZHIP_OK;
+}
+
+int nzhip_memset(void* ptr, int value, size_t bytes) {
+    if (!ptr && bytes) return set_error(NZHIP_E_INVALID, "nzhip_memset: null pointer");
+    hipError_t e = hipMemsetAsync(ptr, value, bytes, Runtime::instance().stream());
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipMemsetAsync");
+}
+
+static int copy(void* dst, const void* src, size_t bytes, hipMemcpyKind kind, const char* what) {
+    if ((!dst || !src) && bytes) return set_error(NZHIP_E_INVALID, "%s: null pointer", what);
+    hipError_t e = hipMemcpyAsync(dst, src, bytes, kind, Runtime::instance().stream());
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, what);
+}
+
+int nzhip_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+    // Pageable host memory: the runtime stages the source before returning, so the caller's
+    // buffer may be reused at once; the device-side copy stays ordered on the compute stream.
+    return copy(dst, src, bytes, hipMemcpyHostToDevice, "nzhip_memcpy_h2d");
+}
+
+int nzhip_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+    return copy(dst, src, bytes, hipMemcpyDeviceToDevice, "nzhip_memcpy_d2d");
+}
+
+int nzhip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+    int rc = copy(dst, src, bytes, hipMemcpyDeviceToHost, "nzhip_memcpy_d2h");
+    if (rc) return rc;
+    hipError_t e = hipStreamSynchronize(Runtime::instance().stream());
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipStreamSynchronize");
+}
+
+int nzhip_sync_ptr(const void* ptr) {
+    (void)ptr;   // one ordered stream: everything that touches ptr is ahead of this point in it
+    hipError_t e = hipStreamSynchronize(Runtime::instance().stream());
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipStreamSynchronize");
+}
+
+int nzhip_sync_all(void) {
+    hipError_t e = hipDeviceSynchronize();
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipDeviceSynchronize");
+}
+
+int nzhip_allocator_stats(size_t* bytes_in_use, size_t* bytes_cached, size_t* device_allocs) {
+    const PoolStats s = Runtime::instance().pool().stats();
+    if (bytes_in_use) *bytes_in_use = s.bytes_in_use;
+    if (bytes_cached) *bytes_cached = s.bytes_cached;
+    if (device_allocs) *device_allocs = s.device_allocs;
+    return NZHIP_OK;
+}
+
+int nzhip_allocator_trim(void) {
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return set_hip_error(e, "hipDeviceSynchronize");
+    Runtime::instance().pool().trim();
+    return NZHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,137 @@
+"""Parity of the conv lowering (im2col, col2im, fused Conv2d forward) on the GPU with the CPU
+oracle; called through the C-ABI.  Integer-valued cases must match bit for bit; float cases
+meet max-rel <= 1e-3 / Frobenius-rel <= 1e-4 against the fp64 direct convolution of the same
+fp16-rounded operands (max-rel floored at the RMS of the truth)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL, FROB_REL = 1e-3, 1e-4
+
+
+@pytest.fixture(scope="module")
+def nz():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from neuzephyr_amd import capi
+    capi.load()
+    return capi
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def check_tolerance(oracle, got, truth64, tag=""):
+    rms = float(np.sqrt(np.mean(np.square(truth64)))) or 1.0
+    mr, fr = oracle.errors(got, truth64, rms)
+    assert mr <= MAX_REL and fr <= FROB_REL, f"{tag}: max_rel {mr:.3e} frob_rel {fr:.3e}"
+
+
+IM2COL_CASES = [((2, 3, 4, 5), 3, 3, 1, 1), ((1, 1, 1, 1), 1, 1, 1, 0), ((2, 2, 7, 6), 3, 2, 2, 0),
+                ((1, 3, 8, 9), 2, 4, 2, 2), ((3, 1, 5, 5), 5, 5, 1, 2), ((2, 4, 6, 6), 1, 1, 3, 0),
+                ((2, 5, 33, 47), 3, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("shape,k_h,k_w,stride,pad", IM2COL_CASES)
+def test_im2col_bit_exact(nz, oracle, shape, k_h, k_w, stride, pad):
+    x = np.random.default_rng(sum(shape)).uniform(0.1, 0.9, size=shape).astype(np.float32)
+    assert np.array_equal(host(nz.im2col(dev(x), k_h, k_w, stride, pad)), oracle.im2col(x, k_h, k_w, stride, pad))
+
+
+@pytest.mark.parametrize("n,c,h,w", [(2, 3, 4, 5), (1, 1, 1, 1), (3, 40, 9, 11), (2, 128, 16, 16), (1, 1, 50, 70)])
+def test_col2im_bit_exact(nz, oracle, n, c, h, w):
+    col = np.random.default_rng(n + c + h + w).uniform(-1, 1, size=(n, 1, h * w, c)).astype(np.float32)
+    assert np.array_equal(host(nz.col2im(dev(col), h, w)), oracle.col2im(col, h, w))
+
+
+def test_add_broadcast_bit_exact(nz, oracle):
+    rng = np.random.default_rng(2)
+    for sa, sb in [((2, 3, 4, 4), (1, 1, 4, 4)), ((2, 3, 5, 3), (1, 3, 5, 3)), ((1, 3, 5, 3), (2, 1, 5, 3)),
+                   ((4, 1, 64, 1), (1, 1, 64, 1)), ((3, 1, 30, 7), (1, 1, 30, 7))]:
+        a = rng.normal(size=sa).astype(np.float32)
+        b = rng.normal(size=sb).astype(np.float32)
+        assert np.array_equal(host(nz.add_broadcast(dev(a), dev(b))), oracle.matrix_add(a, b))
+    with pytest.raises(nz.NzHipError) as ei:
+        nz.add_broadcast(dev(np.zeros((2, 1, 3, 3))), dev(np.zeros((3, 1, 3, 3))))
+    assert ei.value.status == -2 and "not broadcast compatible" in ei.value.message
+
+
+CONV_CASES = [
+    # N, C, H, W, O, k_h, k_w, stride, pad, w_batch
+    (2, 3, 6, 7, 4, 3, 3, 1, 1, 1),
+    (2, 3, 6, 7, 4, 3, 3, 1, 1, 2),
+    (1, 2, 9, 8, 3, 2, 3, 2, 0, 1),
+    (3, 1, 5, 5, 1, 3, 3, 1, 2, 1),
+    (2, 16, 20, 24, 40, 3, 3, 1, 1, 1),
+    (1, 3, 40, 64, 1, 3, 3, 1, 1, 1),
+    (2, 8, 17, 19, 5, 5, 5, 2, 2, 1),
+    (1, 70, 9, 9, 130, 1, 1, 1, 0, 1),
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,k_h,k_w,stride,pad,w_batch", CONV_CASES)
+def test_conv2d_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, pad, w_batch):
+    rng = np.random.default_rng(N + C + H + W + O + k_h)
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    w = rng.integers(-3, 4, size=(O, C, k_h, k_w)).astype(np.float32)
+    bias = rng.integers(-2, 3, size=(O,)).astype(np.float32)
+    w_ref = oracle.weights_oihw_to_ref(w)
+    if w_batch > 1:
+        w_ref = np.ascontiguousarray(np.broadcast_to(w_ref, (w_batch,) + w_ref.shape[1:]))
+    truth = oracle.conv2d_direct_f64(x, w, bias, stride, pad, relu=True)
+    got = host(nz.conv2d_forward(dev(x), dev(w_ref), dev(bias), k_h, k_w, stride, pad, bias_strides=(0, 1), relu=True))
+    assert np.array_equal(got.astype(np.float64), truth)
+    # the unfused graph, node by node (src/Model.cu:244-263), gives the same numbers
+    Ho, Wo = oracle.out_hw(H, W, k_h, k_w, stride, pad)
+    col = nz.im2col(dev(x), k_h, k_w, stride, pad)
+    res = nz.tensorcore_gemm(col, dev(w_ref))
+    res = nz.add_broadcast(res, dev(oracle.bias_channel_to_ref(bias, Ho * Wo)))
+    y = nz.relu(nz.col2im(res, Ho, Wo))
+    assert np.array_equal(host(y), got)
+
+
+def test_conv2d_per_pixel_bias_like_the_reference_parameter(nz, oracle):
+    N, C, H, W, O = 2, 5, 10, 9, 6
+    x = oracle.fill((N, C, H, W), 61, "normal", 0.0, 1.0)
+    w = oracle.fill((O, C, 3, 3), 62, "normal", 0.0, 0.2)
+    Ho, Wo = oracle.out_hw(H, W, 3, 3, 1, 1)
+    bias_px = oracle.fill((1, 1, Ho * Wo, O), 63, "uniform", -0.5, 0.5)
+    truth = oracle.conv2d_direct_f64(x, w, None, 1, 1) + bias_px.reshape(Ho, Wo, O).transpose(2, 0, 1)[None].astype(np.float64)
+    got = host(nz.conv2d_forward(dev(x), dev(oracle.weights_oihw_to_ref(w)), dev(bias_px), 3, 3, 1, 1,
+                                 bias_strides=(O, 1), relu=False))
+    check_tolerance(oracle, got, truth, "per-pixel bias")
+    ref = oracle.conv2d_graph(x, oracle.weights_oihw_to_ref(w), bias_px, 3, 3, 1, 1)
+    assert np.max(np.abs(got - ref)) <= 1e-4
+
+
+def test_config4a_conv_64_to_128_channels(nz, oracle):
+    N, C, H, W, O = 16, 64, 128, 128, 128
+    x = oracle.fill((N, C, H, W), 4, "normal", 0.0, 1.0)
+    w = oracle.fill((O, C, 3, 3), 1004, "normal", 0.0, float(np.sqrt(2.0 / (C * 9))))
+    bias = oracle.fill((O,), 2004, "uniform", -0.03, 0.03)
+    got = nz.conv2d_forward(dev(x), dev(oracle.weights_oihw_to_ref(w)), dev(bias), 3, 3, 1, 1, bias_strides=(0, 1), relu=True)
+    # two whole images against the fp64 direct convolution
+    for b in (0, 11):
+        truth = oracle.conv2d_direct_f64(x[b:b + 1], w, bias, 1, 1, relu=True)
+        check_tolerance(oracle, host(got[b:b + 1]), truth, f"CA image {b}")
+    # translation property at full size: shifting the batch order permutes the output
+    perm = np.roll(np.arange(N), 3)
+    got_p = nz.conv2d_forward(dev(x[perm]), dev(oracle.weights_oihw_to_ref(w)), dev(bias), 3, 3, 1, 1, bias_strides=(0, 1), relu=True)
+    assert np.array_equal(host(got_p), host(got)[perm])
+
+
+def test_config4b_conv_memory_bound_single_channel_out(nz, oracle):
+    N, C, H, W, O = 10, 3, 1024, 1024, 1
+    x = oracle.fill((N, C, H, W), 14, "uniform", 0.0, 1.0)
+    w = oracle.fill((O, C, 3, 3), 1014, "normal", 0.0, float(np.sqrt(2.0 / 27)))
+    bias = oracle.fill((O,), 2014, "uniform", -0.03, 0.03)
+    got = host(nz.conv2d_forward(dev(x), dev(oracle.weights_oihw_to_ref(w)), dev(bias), 3, 3, 1, 1, bias_strides=(0, 1), relu=True))
+    truth = oracle.conv2d_direct_f64(x, w, bias, 1, 1, relu=True)
+    check_tolerance(oracle, got, truth, "CB")

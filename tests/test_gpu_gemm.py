@@ -1,0 +1,260 @@
+"""Parity of the HIP GEMM path (called through the C-ABI of include/nzhip.h) with the CPU
+oracle.  Bar: bit-exact wherever arithmetic is exact (integer-valued operands, the
+reference's literal vectors, identity products); otherwise the stated contract
+max-rel <= 1e-3 and Frobenius-rel <= 1e-4 against an fp64 accumulation of the same
+fp16-rounded inputs, where max-rel uses the RMS of the truth as the absolute floor
+(|got-truth| / max(|truth|, rms(truth)))."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL, FROB_REL = 1e-3, 1e-4
+
+
+@pytest.fixture(scope="module")
+def nz():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from neuzephyr_amd import capi
+    capi.load()
+    return capi
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def check_tolerance(oracle, got, truth64, tag=""):
+    rms = float(np.sqrt(np.mean(np.square(truth64)))) or 1.0
+    mr, fr = oracle.errors(got, truth64, rms)
+    assert mr <= MAX_REL and fr <= FROB_REL, f"{tag}: max_rel {mr:.3e} frob_rel {fr:.3e}"
+    return mr, fr
+
+
+def test_device_is_gfx950(nz):
+    import ctypes as C
+    cu, lds, name = C.c_int(0), C.c_size_t(0), C.create_string_buffer(64)
+    nz.check(nz.load().nzhip_device_info(C.byref(cu), C.byref(lds), name, 64))
+    assert name.value.decode().startswith("gfx950"), name.value
+    assert cu.value >= 200 and lds.value >= 160 * 1024
+
+
+def test_reference_literal_vectors(nz):
+    with open(os.path.join(os.path.dirname(__file__), "golden", "matmul_broadcast.json")) as f:
+        g = json.load(f)
+    A = np.array(g["A"], np.float32).reshape(g["shapeA"])
+    B = np.array(g["B"], np.float32).reshape(g["shapeB"])
+    C = np.array(g["C"], np.float32).reshape(g["shapeC"])
+    assert np.array_equal(host(nz.tensorcore_gemm(dev(A), dev(B))), C)
+
+
+SHAPES = [(1, 1, 1), (3, 5, 2), (16, 16, 16), (17, 33, 15), (64, 100, 132), (130, 257, 67), (128, 32, 128),
+          (256, 64, 256), (257, 31, 255), (300, 40, 520), (1000, 777, 513), (1, 4096, 64), (8, 8, 1024)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+@pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("tile", [128, 256])
+def test_integer_operands_are_bit_exact(nz, M, K, N, a_trans, b_trans, tile):
+    rng = np.random.default_rng(M * 7919 + K * 31 + N)
+    A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+    B = rng.integers(-8, 9, size=(K, N)).astype(np.float32)
+    expect = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)
+    Ad = dev(A.T if a_trans else A)
+    Bd = dev(B.T if b_trans else B)
+    got = host(nz.gemm(Ad, Bd, a_trans=a_trans, b_trans=b_trans, force_tile=tile))
+    assert np.array_equal(got, expect)
+
+
+def test_unaligned_base_pointers_take_the_scalar_path(nz):
+    import torch
+    rng = np.random.default_rng(5)
+    M, K, N = 70, 52, 36
+    A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+    B = rng.integers(-8, 9, size=(K, N)).astype(np.float32)
+    bufA = torch.zeros(M * K + 1, device="cuda")
+    bufB = torch.zeros(K * N + 3, device="cuda")
+    Ad = bufA[1:].view(M, K)
+    Bd = bufB[3:].view(K, N)
+    Ad.copy_(torch.from_numpy(A))
+    Bd.copy_(torch.from_numpy(B))
+    assert Ad.data_ptr() % 16 != 0 and Bd.data_ptr() % 16 != 0
+    got = host(nz.gemm(Ad, Bd))
+    assert np.array_equal(got, (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32))
+
+
+def test_identity_gives_fp16_rounding_including_special_values(nz, oracle):
+    n = 96
+    X = oracle.fill((n, n), 11, "uniform", -4.0, 4.0)
+    X[0, :12] = [65504.0, 65519.0, 65520.0, 1e6, -1e6, 2.0 ** -24, 2.0 ** -25, 1.5 * 2.0 ** -25, 6.0e-8, -2.0 ** -14,
+                 3.0e-5, 1.0 + 2.0 ** -11]
+    got = host(nz.gemm(dev(np.eye(n, dtype=np.float32)), dev(X)))
+    expect = oracle.round_f16(X)                       # I * X = f16(X): zeros elsewhere add exactly
+    # 0 * inf = NaN in the columns that hold an infinity after rounding; compare those apart
+    inf_cols = np.isinf(expect).any(axis=0)
+    assert np.array_equal(got[:, ~inf_cols].view(np.uint32) & 0x7FFFFFFF, expect[:, ~inf_cols].view(np.uint32) & 0x7FFFFFFF)
+    assert np.all(np.isnan(got[1:, inf_cols])) and np.all(np.isinf(got[0, inf_cols]))
+    # subnormal halfs survive the MFMA (no flush to zero)
+    assert got[0, 5] == 2.0 ** -24 and got[0, 6] == 0.0 and got[0, 7] == 2.0 ** -24
+    got_r = host(nz.gemm(dev(X), dev(np.eye(n, dtype=np.float32))))
+    assert np.array_equal(got_r[1:], expect[1:])
+
+
+def test_config1_gemm_256_uniform(nz, oracle):
+    A = oracle.fill((256, 256), 0, "uniform", -1.0, 1.0)
+    B = oracle.fill((256, 256), 1000, "uniform", -1.0, 1.0)
+    truth = oracle.gemm_f64(A, B)
+    for tile in (128, 256):
+        got = host(nz.gemm(dev(A), dev(B), force_tile=tile))
+        check_tolerance(oracle, got, truth, f"G1 tile {tile}")
+        # and against the fp32 sequential oracle: same rounding, only the sum order differs
+        ref32 = oracle.gemm(A, B)
+        assert np.max(np.abs(got - ref32)) <= 256 * 2.0 ** -23 * np.max(np.abs(truth))
+
+
+def test_config3_ragged_and_gemv(nz, oracle):
+    A = oracle.fill((1000, 777), 3, "uniform", -1.0, 1.0)
+    B = oracle.fill((777, 513), 1003, "uniform", -1.0, 1.0)
+    check_tolerance(oracle, host(nz.gemm(dev(A), dev(B))), oracle.gemm_f64(A, B), "R1")
+    a = oracle.fill((1, 4096), 4, "uniform", -1.0, 1.0)
+    Bm = oracle.fill((4096, 4096), 1004, "uniform", -1.0, 1.0)
+    check_tolerance(oracle, host(nz.gemm(dev(a), dev(Bm))), oracle.gemm_f64(a, Bm), "R2")
+
+
+def test_config2_linear_bias_relu(nz, oracle):
+    Nb, IN, OUT = 4096, 1024, 4096
+    X = oracle.fill((Nb, IN), 2, "normal", 0.0, 1.0)
+    bound = float(np.sqrt(6.0 / IN))
+    Wt = oracle.fill((OUT, IN), 1002, "uniform", -bound, bound)       # reference storage [1,1,OUT,IN]
+    bias = oracle.fill((OUT,), 2002, "uniform", -0.03, 0.03)
+    expect32 = oracle.linear_graph(X, Wt, bias, relu=True)
+    truth = oracle.gemm_f64(X, Wt, trans_b=True) + bias.astype(np.float64)[None, :]
+    truth = np.maximum(truth, 0.0)
+    # (1) fused form: Y[Nb,OUT] = relu(X * Wt^T + bias)
+    got = host(nz.gemm(dev(X), dev(Wt), b_trans=True, bias=dev(bias), bias_strides=(0, 1), relu=True))
+    check_tolerance(oracle, got, truth, "L fused")
+    assert np.max(np.abs(got - expect32)) <= 1e-3
+    assert np.array_equal(got == 0.0, np.maximum(got, 0) == 0.0) and got.min() >= 0.0
+    # (2) config form W[K,N] row-major
+    W = np.ascontiguousarray(Wt.T)
+    got2 = host(nz.gemm(dev(X), dev(W), bias=dev(bias), bias_strides=(0, 1), relu=True))
+    check_tolerance(oracle, got2, truth, "L config form")
+    # (3) the graph exactly as Model::Linear builds it: W[1,1,OUT,IN] x[N,1,IN,1] -> [N,1,OUT,1]
+    y = nz.tensorcore_gemm(dev(Wt.reshape(1, 1, OUT, IN)), dev(X.reshape(Nb, 1, IN, 1)))
+    y = nz.relu(nz.add_broadcast(y, dev(bias.reshape(1, 1, OUT, 1))))
+    check_tolerance(oracle, host(y).reshape(Nb, OUT), truth, "L graph")
+
+
+@pytest.mark.parametrize("sa,sb", [((2, 1, 2, 3), (1, 3, 3, 2)), ((3, 2, 5, 7), (3, 2, 7, 4)), ((1, 1, 9, 6), (4, 1, 6, 1)),
+                                    ((2, 3, 4, 5), (1, 1, 5, 6)), ((1, 3, 4, 5), (2, 1, 5, 6)), ((5, 1, 1, 40), (1, 1, 40, 24)),
+                                    ((4, 2, 130, 70), (1, 2, 70, 260)), ((1, 1, 33, 20), (3, 4, 20, 1))])
+def test_batched_broadcast_matches_oracle(nz, oracle, sa, sb):
+    rng = np.random.default_rng(sum(sa) * 3 + sum(sb))
+    A = rng.integers(-6, 7, size=sa).astype(np.float32)
+    B = rng.integers(-6, 7, size=sb).astype(np.float32)
+    assert np.array_equal(host(nz.tensorcore_gemm(dev(A), dev(B))), oracle.tensorcore_gemm(A, B))
+
+
+def test_bias_forms_and_relu_special_values(nz, oracle):
+    M, K, N = 40, 24, 52
+    rng = np.random.default_rng(1)
+    A = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    B = rng.integers(-3, 4, size=(K, N)).astype(np.float32)
+    P = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)
+    row = rng.integers(-5, 6, size=(M,)).astype(np.float32)
+    col = rng.integers(-5, 6, size=(N,)).astype(np.float32)
+    full = rng.integers(-5, 6, size=(M, N)).astype(np.float32)
+    assert np.array_equal(host(nz.gemm(dev(A), dev(B), bias=dev(row), bias_strides=(1, 0))), P + row[:, None])
+    assert np.array_equal(host(nz.gemm(dev(A), dev(B), bias=dev(col), bias_strides=(0, 1))), P + col[None, :])
+    assert np.array_equal(host(nz.gemm(dev(A), dev(B), bias=dev(full), bias_strides=(N, 1), relu=True)),
+                          np.maximum(P + full, 0))
+    # ReLU: NaN -> 0, -0 -> +0  (x > 0 ? x : 0, src/OperationKernels.cu:230-235)
+    nanbias = np.zeros((M, N), np.float32)
+    nanbias[0, 0] = np.nan
+    nanbias[0, 1] = -np.inf
+    out = host(nz.gemm(dev(np.zeros_like(A)), dev(B), bias=dev(nanbias), bias_strides=(N, 1), relu=True))
+    assert out[0, 0] == 0.0 and out[0, 1] == 0.0 and not np.signbit(out).any()
+    v = np.array([np.nan, -0.0, 0.0, -1.5, 2.5, np.inf, -np.inf, 1e-45, 3.0], np.float32)
+    assert np.array_equal(host(nz.relu(dev(v))), oracle.relu(v))
+
+
+def test_empty_extents(nz):
+    import torch
+    A = torch.zeros((0, 8), device="cuda")
+    B = torch.zeros((8, 4), device="cuda")
+    assert nz.gemm(A, B).shape == (0, 4)
+    # K == 0: empty sum, C = act(bias)
+    A = torch.zeros((3, 0), device="cuda")
+    B = torch.zeros((0, 4), device="cuda")
+    bias = dev(np.array([-1, 2, -3, 4], np.float32))
+    out = torch.full((3, 4), 7.0, device="cuda")
+    nz.gemm(A, B, bias=bias, bias_strides=(0, 1), relu=True, out=out)
+    assert np.array_equal(host(out), np.tile(np.array([0, 2, 0, 4], np.float32), (3, 1)))
+
+
+def test_invalid_arguments_are_rejected_without_launching(nz):
+    import ctypes as C
+    import torch
+    A = torch.zeros((4, 4), device="cuda")
+    d = nz.GemmDesc()
+    d.A = d.B = d.C = A.data_ptr()
+    d.M = d.N = d.K = 4
+    d.lda = d.ldb = d.ldc = 4
+    d.batch_n = d.batch_c = 1
+    lib = nz.load()
+    assert lib.nzhip_gemm(C.byref(d), None) == 0
+    d.lda = 2
+    assert lib.nzhip_gemm(C.byref(d), None) == -1 and b"leading dimension" in lib.nzhip_last_error()
+    d.lda = 4
+    d.activation = 9
+    assert lib.nzhip_gemm(C.byref(d), None) == -1
+    d.activation = 0
+    d.batch_n = 0
+    assert lib.nzhip_gemm(C.byref(d), None) == -1
+    d.batch_n = 1
+    d.A = None
+    assert lib.nzhip_gemm(C.byref(d), None) == -1
+    assert lib.nzhip_gemm(None, None) == -1
+    torch.cuda.synchronize()
+
+
+def test_config5_large_square_sampled_rows(nz, oracle):
+    n = 8192
+    A = oracle.fill((n, n), 5, "normal", 0.0, 1.0 / np.sqrt(n))
+    B = oracle.fill((n, n), 1005, "normal", 0.0, 1.0 / np.sqrt(n))
+    got = nz.gemm(dev(A), dev(B))
+    rows = np.random.default_rng(5).choice(n, size=64, replace=False)
+    rows.sort()
+    got_rows = host(got[rows.tolist()])
+    truth = np.empty((64, n), np.float64)
+    for i, r in enumerate(rows):
+        _, t = oracle.gemm_rows(A, B, int(r), 1, want32=False)
+        truth[i] = t[0]
+    check_tolerance(oracle, got_rows, truth, "G2 sampled rows")
+    # size-independent property at full size: (A*B) e_j picks column j -- multiply by the identity
+    # on the right reproduces f16(A) exactly
+    I = dev(np.eye(n, dtype=np.float32))
+    Ad = dev(A)
+    assert np.array_equal(host(nz.gemm(Ad, I)), oracle.round_f16(A))
+
+
+def test_config5_batched_1024(nz, oracle):
+    # [8,16,1024,1024] x [8,16,1024,1024] over (N,C); three seeded batch members checked in full
+    import torch
+    shape = (8, 16, 1024, 1024)
+    A = oracle.fill(shape, 6, "normal", 0.0, 1.0 / 32.0)
+    B = oracle.fill(shape, 1006, "normal", 0.0, 1.0 / 32.0)
+    got = nz.tensorcore_gemm(dev(A), dev(B))
+    for (i, j) in [(0, 0), (3, 7), (7, 15)]:
+        check_tolerance(oracle, host(got[i, j]), oracle.gemm_f64(A[i, j], B[i, j]), f"GB[{i},{j}]")
+    del got
+    torch.cuda.empty_cache()
