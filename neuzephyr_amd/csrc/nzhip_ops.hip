@@ -99,8 +99,10 @@ __global__ __launch_bounds__(256) void relu_kernel(float* __restrict__ out, cons
 }
 
 static int validate_gemm(const nzhip_gemm_desc& d) {
-    if (!d.A || !d.B || !d.C) return set_error(NZHIP_E_INVALID, "nzhip_gemm: null operand pointer");
     if (d.M < 0 || d.N < 0 || d.K < 0) return set_error(NZHIP_E_INVALID, "nzhip_gemm: negative extent");
+    // an operand with no elements may be null
+    if ((!d.A && d.M * d.K > 0) || (!d.B && d.K * d.N > 0) || (!d.C && d.M * d.N > 0))
+        return set_error(NZHIP_E_INVALID, "nzhip_gemm: null operand pointer");
     if (d.batch_n < 1 || d.batch_c < 1) return set_error(NZHIP_E_INVALID, "nzhip_gemm: batch extents must be >= 1");
     if (d.a_layout != NZHIP_LAYOUT_ROW && d.a_layout != NZHIP_LAYOUT_TRANS)
         return set_error(NZHIP_E_INVALID, "nzhip_gemm: bad a_layout %d", d.a_layout);

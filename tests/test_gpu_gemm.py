@@ -222,7 +222,7 @@ def test_invalid_arguments_are_rejected_without_launching(nz):
     assert lib.nzhip_gemm(C.byref(d), None) == -1
     d.batch_n = 1
     d.A = None
-    assert lib.nzhip_gemm(C.byref(d), None) == -1
+    assert lib.nzhip_gemm(C.byref(d), None) == -1 and b"null operand" in lib.nzhip_last_error()
     assert lib.nzhip_gemm(None, None) == -1
     torch.cuda.synchronize()
 
