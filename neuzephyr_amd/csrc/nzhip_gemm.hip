@@ -50,7 +50,10 @@ __device__ __forceinline__ int phys_row(int r) {
 
 // ---- operand staging: global fp32 -> registers -> fp16 in LDS ----------------------------
 // KCONTIG: the operand is stored with k contiguous (A row-major MxK, or B given as NxK).
-template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC>
+// FULL: the tile lies wholly inside the operand and K is a multiple of BK, so no predicate is
+// evaluated. Otherwise loads are predicated WITHOUT branches: an out-of-range lane reads the
+// operand's first element (always mapped) and the value is replaced by zero afterwards.
+template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC, bool FULL>
 struct StageKContig {
     static constexpr int F4_PER_ROW = BK / 4;
     static constexpr int ROWS_PER_PASS = NT / F4_PER_ROW;
@@ -66,18 +69,23 @@ struct StageKContig {
         for (int p = 0; p < PASSES; p++) {
             const int gr = row_base + r0 + p * ROWS_PER_PASS;
             const float* src = X + (long)gr * ldx + gk;
-            floatx4 v = {0.f, 0.f, 0.f, 0.f};
-            if (gr < R) {
-                if (VEC) {
-                    if (gk < K) v = *reinterpret_cast<const floatx4*>(src);
-                } else {
-                    if (gk + 0 < K) v[0] = src[0];
-                    if (gk + 1 < K) v[1] = src[1];
-                    if (gk + 2 < K) v[2] = src[2];
-                    if (gk + 3 < K) v[3] = src[3];
+            if constexpr (FULL) {
+                regs[p] = *reinterpret_cast<const floatx4*>(src);
+            } else if constexpr (VEC) {
+                const bool ok = gr < R && gk < K;
+                const floatx4 v = *reinterpret_cast<const floatx4*>(ok ? src : X);
+                const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+                regs[p] = ok ? v : z;
+            } else {
+                floatx4 v;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const bool ok = gr < R && gk + e < K;
+                    const float x = *(ok ? src + e : X);
+                    v[e] = ok ? x : 0.f;
                 }
+                regs[p] = v;
             }
-            regs[p] = v;
         }
     }
 
@@ -99,7 +107,7 @@ struct StageKContig {
 // RCONTIG: the operand is stored with the tile dimension contiguous (B row-major KxN, or
 // A given as KxM). Each thread takes 4 neighbouring tile rows over KPT consecutive k and
 // transposes them in registers, so LDS still holds k-contiguous rows.
-template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC>
+template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC, bool FULL>
 struct StageRContig {
     static constexpr int F4_PER_KROW = BR / 4;
     static constexpr int KGROUPS = NT / F4_PER_KROW;
@@ -116,18 +124,23 @@ struct StageRContig {
         for (int q = 0; q < KPT; q++) {
             const int gk = k_base + kg * KPT + q;
             const float* src = X + (long)gk * ldx + gr;
-            floatx4 v = {0.f, 0.f, 0.f, 0.f};
-            if (gk < K) {
-                if (VEC) {
-                    if (gr < R) v = *reinterpret_cast<const floatx4*>(src);
-                } else {
-                    if (gr + 0 < R) v[0] = src[0];
-                    if (gr + 1 < R) v[1] = src[1];
-                    if (gr + 2 < R) v[2] = src[2];
-                    if (gr + 3 < R) v[3] = src[3];
+            if constexpr (FULL) {
+                regs[q] = *reinterpret_cast<const floatx4*>(src);
+            } else if constexpr (VEC) {
+                const bool ok = gk < K && gr < R;
+                const floatx4 v = *reinterpret_cast<const floatx4*>(ok ? src : X);
+                const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+                regs[q] = ok ? v : z;
+            } else {
+                floatx4 v;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const bool ok = gk < K && gr + e < R;
+                    const float x = *(ok ? src + e : X);
+                    v[e] = ok ? x : 0.f;
                 }
+                regs[q] = v;
             }
-            regs[q] = v;
         }
     }
 
@@ -156,20 +169,21 @@ struct StageRContig {
     }
 };
 
-template <bool RCONTIG, int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC>
+template <bool RCONTIG, int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC, bool FULL>
 struct StageSelect {
-    using type = StageKContig<BR, BK, NT, TR, FR, ROWB, VEC>;
+    using type = StageKContig<BR, BK, NT, TR, FR, ROWB, VEC, FULL>;
 };
-template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC>
-struct StageSelect<true, BR, BK, NT, TR, FR, ROWB, VEC> {
-    using type = StageRContig<BR, BK, NT, TR, FR, ROWB, VEC>;
+template <int BR, int BK, int NT, int TR, int FR, int ROWB, bool VEC, bool FULL>
+struct StageSelect<true, BR, BK, NT, TR, FR, ROWB, VEC, FULL> {
+    using type = StageRContig<BR, BK, NT, TR, FR, ROWB, VEC, FULL>;
 };
 
 // ---- the kernel ----------------------------------------------------------------------------
 // BM x BN x BK workgroup tile, WM x WN waves, each wave a (BM/WM) x (BN/WN) tile of 32x32 MFMA
 // blocks.  A_TRANS: A given as KxM.  B_TRANS: B given as NxK.  VEC: 16-byte global accesses
-// are legal for both operands (alignment and extents checked on the host).
-template <int BM, int BN, int BK, int WM, int WN, bool A_TRANS, bool B_TRANS, bool VEC>
+// are legal for both operands (alignment and extents checked on the host).  FULL: M, N and K
+// are multiples of BM, BN and BK (implies VEC), so loads and stores carry no predicates.
+template <int BM, int BN, int BK, int WM, int WN, bool A_TRANS, bool B_TRANS, bool VEC, bool FULL>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKernelArgs p) {
     constexpr int NT = WM * WN * 64;
     constexpr int TM = BM / WM, TN = BN / WN;
@@ -209,8 +223,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     const float* __restrict__ B = p.B + bi * p.b_sn + bj * p.b_sc;
     float* __restrict__ C = p.C + bi * p.c_sn + bj * p.c_sc;
 
-    typename StageSelect<A_TRANS, BM, BK, NT, TM, FM, ROWB, VEC>::type sa;
-    typename StageSelect<!B_TRANS, BN, BK, NT, TN, FN, ROWB, VEC>::type sb;
+    typename StageSelect<A_TRANS, BM, BK, NT, TM, FM, ROWB, VEC, FULL>::type sa;
+    typename StageSelect<!B_TRANS, BN, BK, NT, TN, FN, ROWB, VEC, FULL>::type sb;
 
     floatx16 acc[FM][FN];
 #pragma unroll
@@ -261,19 +275,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     // ---- epilogue: bias, activation, predicated (vector when legal) store ------------------
     const float* bias = p.bias ? p.bias + bi * p.bias_sn + bj * p.bias_sc : nullptr;
     const int gn = n0 + wn * TN + li * FN;                // first of this lane's FN columns
-    const bool vec_store = VEC && (FN == 2 || FN == 4) && (gn + FN <= p.N);
+    const bool vec_store = FULL || (VEC && (FN == 2 || FN == 4) && (gn + FN <= p.N));
 #pragma unroll
     for (int i = 0; i < FM; i++) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int im = (r >> 2) * 8 + lh * 4 + (r & 3);
             const int gm = m0 + wm * TM + im * FM + i;
-            if (gm >= p.M) continue;
+            if (!FULL && gm >= p.M) continue;
             float v[FN];
 #pragma unroll
             for (int j = 0; j < FN; j++) {
                 float x = acc[i][j][r];
-                if (bias && gn + j < p.N) x += bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk];
+                if (bias && (FULL || gn + j < p.N)) x += bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk];
                 if (p.relu) x = x > 0.f ? x : 0.f;
                 v[j] = x;
             }
@@ -298,12 +312,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
 // ---- host-side selection -------------------------------------------------------------------
 template <int BM, int BN, int BK, int WM, int WN>
 static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool vec, int batch, hipStream_t s) {
+    const bool full = vec && a.M % BM == 0 && a.N % BN == 0 && a.K % BK == 0;
     constexpr int ROWB = BK * 2 + 16;
     constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * ROWB;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch, 1), block(WM * WN * 64, 1, 1);
-#define NZHIP_LAUNCH(AT, BT, V)                                                                          \
+#define NZHIP_LAUNCH(AT, BT, V, F)                                                                       \
     do {                                                                                                 \
-        auto kfn = gemm_f16mfma_kernel<BM, BN, BK, WM, WN, AT, BT, V>;                                   \
+        auto kfn = gemm_f16mfma_kernel<BM, BN, BK, WM, WN, AT, BT, V, F>;                                \
         static bool attr_set = false;                                                                    \
         if (!attr_set) {                                                                                 \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                       \
@@ -313,16 +328,21 @@ static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool 
         }                                                                                                \
         hipLaunchKernelGGL(kfn, grid, block, lds_bytes, s, a);                                           \
     } while (0)
-    if (vec) {
-        if (!a_trans && !b_trans) NZHIP_LAUNCH(false, false, true);
-        else if (!a_trans && b_trans) NZHIP_LAUNCH(false, true, true);
-        else if (a_trans && !b_trans) NZHIP_LAUNCH(true, false, true);
-        else NZHIP_LAUNCH(true, true, true);
+    if (full) {
+        if (!a_trans && !b_trans) NZHIP_LAUNCH(false, false, true, true);
+        else if (!a_trans && b_trans) NZHIP_LAUNCH(false, true, true, true);
+        else if (a_trans && !b_trans) NZHIP_LAUNCH(true, false, true, true);
+        else NZHIP_LAUNCH(true, true, true, true);
+    } else if (vec) {
+        if (!a_trans && !b_trans) NZHIP_LAUNCH(false, false, true, false);
+        else if (!a_trans && b_trans) NZHIP_LAUNCH(false, true, true, false);
+        else if (a_trans && !b_trans) NZHIP_LAUNCH(true, false, true, false);
+        else NZHIP_LAUNCH(true, true, true, false);
     } else {
-        if (!a_trans && !b_trans) NZHIP_LAUNCH(false, false, false);
-        else if (!a_trans && b_trans) NZHIP_LAUNCH(false, true, false);
-        else if (a_trans && !b_trans) NZHIP_LAUNCH(true, false, false);
-        else NZHIP_LAUNCH(true, true, false);
+        if (!a_trans && !b_trans) NZHIP_LAUNCH(false, false, false, false);
+        else if (!a_trans && b_trans) NZHIP_LAUNCH(false, true, false, false);
+        else if (a_trans && !b_trans) NZHIP_LAUNCH(true, false, false, false);
+        else NZHIP_LAUNCH(true, true, false, false);
     }
 #undef NZHIP_LAUNCH
     hipError_t e = hipGetLastError();

@@ -1,0 +1,393 @@
+// Two-pass route for large products: round A and B to fp16 once into a pooled workspace
+// (zero-padded to tile multiples, both with k contiguous), then run a pure-fp16 MFMA GEMM
+// whose tiles travel global -> LDS directly (global_load_lds_dwordx4, no staging registers).
+//
+// Why two passes when the operands are large: with fp32 operands every workgroup has to pull
+// 4 bytes per element through L2 and the vector memory path for every tile it touches
+// (M/256 + N/256 times per element), and the 256x256 accumulator tile leaves a single wave
+// per SIMD, i.e. nothing to hide the load latency behind. Rounding once (the same RNE
+// conversion the reference's Padding kernel performs, src/OperationKernels.cu:846-860) halves
+// the re-read traffic and frees the registers. Results are identical to the fused kernel's up
+// to fp32 summation order.
+#include <hip/hip_runtime.h>
+
+#include "nzhip_internal.h"
+
+namespace nzhip {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+// ---- pass 1: rounding copies ---------------------------------------------------------------
+// The workspace is NOT a row-major matrix. It is a sequence of 16 KiB blocks, one per
+// (256-row block rb, 32-wide k tile kt), stored at block index rb * (Kp/32) + kt, and each
+// block is the exact image the GEMM wants in LDS: physical row pr (see phys_row_of) at byte
+// pr*64, chunk c (8 halfs) of that row at chunk position c ^ ((pr>>2)&3). The GEMM's
+// global->LDS copies are therefore plain contiguous 1 KiB reads, consecutive k tiles are
+// consecutive 16 KiB blocks (no power-of-two row pitch, so all memory channels stay busy),
+// and rows/columns beyond the operand are zero.
+constexpr int CVT_ROWS = 256, CVT_K = 32, CVT_BLOCK_BYTES = CVT_ROWS * CVT_K * 2;
+
+// Physical LDS row of logical tile row r for a 2x2 wave grid over a 256-row tile (wave tile
+// 128 rows = 4 MFMA blocks, interleaved so that one lane ends up with 4 adjacent columns).
+__device__ __forceinline__ int phys_row_of(int r) {
+    const int w = r >> 7, l = r & 127;
+    return (w * 4 + (l & 3)) * 32 + (l >> 2);
+}
+
+// K_CONTIG: source element (r, k) at src[r*ld + k]; otherwise at src[k*ld + r].
+template <bool K_CONTIG>
+__global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ dst, const float* __restrict__ src,
+                                                        int R, int K, int nkt, long ld, long src_batch,
+                                                        long dst_batch, int vec) {
+    __shared__ __attribute__((aligned(16))) char img[CVT_BLOCK_BYTES];
+    const int kt = blockIdx.x, rb = blockIdx.y;
+    const float* s = src + (long)blockIdx.z * src_batch;
+    const int t = threadIdx.x;
+    const int r0 = rb * CVT_ROWS, k0 = kt * CVT_K;
+    if (K_CONTIG) {
+        // 8 threads per row (one float4 each), 32 rows per pass
+        const int k4 = t & 7, rr = t >> 3;
+#pragma unroll
+        for (int pass = 0; pass < 8; pass++) {
+            const int lr = rr + pass * 32, r = r0 + lr, k = k0 + k4 * 4;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            const float* q = s + (long)r * ld + k;
+            if (r < R) {
+                if (vec && k + 4 <= K) {
+                    v = *reinterpret_cast<const floatx4*>(q);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (k + e < K) v[e] = q[e];
+                }
+            }
+            half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+            const int pr = phys_row_of(lr);
+            const int pos = (k4 >> 1) ^ ((pr >> 2) & 3);
+            *reinterpret_cast<half4_t*>(img + pr * 64 + pos * 16 + (k4 & 1) * 8) = h;
+        }
+    } else {
+        // 64 threads per k row (one float4 of 4 rows each), 4 k rows per pass
+        const int r4 = t & 63, kk0 = t >> 6;
+#pragma unroll
+        for (int pass = 0; pass < 8; pass++) {
+            const int kk = kk0 + pass * 4, k = k0 + kk, lr = r4 * 4, r = r0 + lr;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            const float* q = s + (long)k * ld + r;
+            if (k < K) {
+                if (vec && r + 4 <= R) {
+                    v = *reinterpret_cast<const floatx4*>(q);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (r + e < R) v[e] = q[e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int pr = phys_row_of(lr + e);
+                const int pos = (kk >> 3) ^ ((pr >> 2) & 3);
+                *reinterpret_cast<_Float16*>(img + pr * 64 + pos * 16 + (kk & 7) * 2) = (_Float16)v[e];
+            }
+        }
+    }
+    __syncthreads();
+    char* out = reinterpret_cast<char*>(dst + (long)blockIdx.z * dst_batch) + ((long)rb * nkt + kt) * CVT_BLOCK_BYTES;
+#pragma unroll
+    for (int pass = 0; pass < 4; pass++) {
+        const int off = (pass * 256 + t) * 16;
+        *reinterpret_cast<floatx4*>(out + off) = *reinterpret_cast<const floatx4*>(img + off);
+    }
+}
+
+// ---- pass 2: fp16 GEMM -----------------------------------------------------------------------
+struct H16Args {
+    const _Float16* A;      // blocked image of A: [Mp/256][Kp/32] blocks of 16 KiB
+    const _Float16* B;      // blocked image of B (rows = output columns): [Np/256][Kp/32] blocks
+    float* C;
+    const float* bias;
+    int M, N, Kp;
+    long ldc;
+    int batch_c;
+    long a_batch, b_batch;              // workspace strides per batch member (0 = shared operand)
+    int a_bcast_n, a_bcast_c, b_bcast_n, b_bcast_c;   // 1 = operand is shared along that batch axis
+    int a_cn;                           // extent of A's c axis in the workspace (for indexing)
+    int b_cn;
+    long c_sn, c_sc, bias_sn, bias_sc, bias_sm, bias_sk;
+    int relu;
+    int tiles_m, tiles_n, group_m;
+};
+
+// s_waitcnt on the vector-memory counter only (expcnt / lgkmcnt left at "don't wait").
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0070 | 0x0F00);
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }   // lgkmcnt(0) only
+
+// BM x BN x 32 tiles in an NSTAGE-deep LDS ring. One LDS row = 32 halfs = 64 bytes = 4 chunks of
+// 16 bytes. LDS has 64 banks x 4 B, so a 256-byte bank row spans four tile rows; chunk c of row r
+// is stored at chunk position  c ^ ((r>>2)&3), which puts the 16 rows that one pass of a
+// 128-bit fragment read touches on 16 different 16-byte bank groups.
+template <int BM, int BN, int WM, int WN, int NSTAGE>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_h16_kernel(const H16Args p) {
+    static_assert(BM == CVT_ROWS && BN == CVT_ROWS && WM == 2 && WN == 2, "must match the workspace block image");
+    constexpr int BK = CVT_K, ROWB = 64;
+    constexpr int NW = WM * WN;
+    constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int A_LOADS = BM / 16 / NW, B_LOADS = BN / 16 / NW;   // wave-wide 1 KiB loads (16 rows) per wave
+    constexpr int LOADS = A_LOADS + B_LOADS;
+    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile/wave mismatch");
+    static_assert((NSTAGE - 1) * LOADS < 64, "too many loads in flight for vmcnt");
+
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int li = lane & 31, lh = lane >> 5;
+
+    const int total = p.tiles_m * p.tiles_n;
+    int lin = blockIdx.x;
+    {
+        const int xcd = lin & 7, q = lin >> 3;
+        const int per = total >> 3, rem = total & 7;
+        lin = xcd * per + (xcd < rem ? xcd : rem) + q;
+    }
+    const int group_sz = p.group_m * p.tiles_n;
+    const int group = lin / group_sz;
+    const int first_m = group * p.group_m;
+    const int rows_in_group = (p.tiles_m - first_m) < p.group_m ? (p.tiles_m - first_m) : p.group_m;
+    const int tile_m = first_m + (lin % group_sz) % rows_in_group;
+    const int tile_n = (lin % group_sz) / rows_in_group;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int bi = blockIdx.y / p.batch_c, bj = blockIdx.y % p.batch_c;
+    const long a_idx = (long)(p.a_bcast_n ? 0 : bi) * p.a_cn + (p.a_bcast_c ? 0 : bj);
+    const long b_idx = (long)(p.b_bcast_n ? 0 : bi) * p.b_cn + (p.b_bcast_c ? 0 : bj);
+    const _Float16* __restrict__ A = p.A + a_idx * p.a_batch;
+    const _Float16* __restrict__ B = p.B + b_idx * p.b_batch;
+    float* __restrict__ C = p.C + bi * p.c_sn + bj * p.c_sc;
+
+    // The workspace already holds the LDS image of every (row block, k tile): this wave's
+    // share of a stage is A_LOADS + B_LOADS contiguous 1 KiB pieces, lane l taking bytes
+    // [16 l, 16 l + 16) of each.
+    const int nk = p.Kp / BK;
+    const char* a_tile = reinterpret_cast<const char*>(A) + (long)tile_m * nk * A_BYTES + wave * A_LOADS * 1024 + lane * 16;
+    const char* b_tile = reinterpret_cast<const char*>(B) + (long)tile_n * nk * B_BYTES + wave * B_LOADS * 1024 + lane * 16;
+
+    // Request k tile kt into ring slot `stage`. Past the end the last tile is requested again
+    // (into a slot nobody reads any more) so that the number of loads in flight, which the
+    // vmcnt waits below count on, is the same in every iteration.
+    auto issue_loads = [&](int kt, int stage) {
+        const int kc = kt < nk ? kt : nk - 1;
+        char* sa = lds + stage * STAGE + wave * A_LOADS * 1024;
+        char* sb = lds + stage * STAGE + A_BYTES + wave * B_LOADS * 1024;
+        const char* ak = a_tile + (long)kc * A_BYTES;
+        const char* bk = b_tile + (long)kc * B_BYTES;
+#pragma unroll
+        for (int j = 0; j < A_LOADS; j++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ak + j * 1024),
+                                             (__attribute__((address_space(3))) void*)(sa + j * 1024), 16, 0, 0);
+#pragma unroll
+        for (int j = 0; j < B_LOADS; j++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(bk + j * 1024),
+                                             (__attribute__((address_space(3))) void*)(sb + j * 1024), 16, 0, 0);
+    };
+
+    floatx16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    // fragment addressing: physical row = block*32 + li; chunk position (2*ks + lh) ^ ((row>>2)&3)
+    const int a_row_off = ((wm * FM) * 32 + li) * ROWB;
+    const int b_row_off = A_BYTES + ((wn * FN) * 32 + li) * ROWB;
+    const int sw = (li >> 2) & 3;
+
+    half8_t af[2][FM], bf[2][FN];
+    auto read_frags = [&](const char* base, int ks, int buf) {
+        const int ch = (((ks << 1) | lh) ^ sw) << 4;
+#pragma unroll
+        for (int i = 0; i < FM; i++) af[buf][i] = *reinterpret_cast<const half8_t*>(base + a_row_off + i * 32 * ROWB + ch);
+#pragma unroll
+        for (int j = 0; j < FN; j++) bf[buf][j] = *reinterpret_cast<const half8_t*>(base + b_row_off + j * 32 * ROWB + ch);
+    };
+    auto mfma_block = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[buf][i], bf[buf][j], acc[i][j], 0, 0, 0);
+    };
+
+    // prologue: fill the ring, wait for tile 0
+#pragma unroll
+    for (int t = 0; t < NSTAGE; t++) issue_loads(t, t);
+    wait_vmcnt<(NSTAGE - 1) * LOADS>();
+    __syncthreads();
+    read_frags(lds, 0, 0);
+
+    // Steady state, per k tile: the second half's fragments are fetched under the first half's
+    // MFMAs; then ONE barrier (next tile landed + everybody is done reading this slot), the
+    // next tile's first fragments and the refill of this slot are issued under the second
+    // half's MFMAs.
+    for (int kt = 0; kt < nk; kt++) {
+        const int slot = kt % NSTAGE;
+        const char* base = lds + slot * STAGE;
+        read_frags(base, 1, 1);
+        mfma_block(0);
+        __builtin_amdgcn_sched_barrier(0);      // keep the MFMAs above the waits: they hide the read latency
+        wait_vmcnt<(NSTAGE - 2) * LOADS>();    // tile kt+1 has landed (this wave's share)
+        wait_lgkmcnt0();                        // this wave's reads of slot kt are complete
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        const int nslot = (kt + 1) % NSTAGE;
+        if (kt + 1 < nk) read_frags(lds + nslot * STAGE, 0, 0);
+        issue_loads(kt + NSTAGE, slot);
+        mfma_block(1);
+    }
+    wait_vmcnt<0>();                            // drain the dummy tail requests before LDS goes away
+
+    // ---- epilogue -----------------------------------------------------------------------------
+    const float* bias = p.bias ? p.bias + bi * p.bias_sn + bj * p.bias_sc : nullptr;
+    const int gn = n0 + wn * TN + li * FN;
+    const bool vec_ok = ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (gn + FN <= p.N);
+#pragma unroll
+    for (int i = 0; i < FM; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int im = (r >> 2) * 8 + lh * 4 + (r & 3);
+            const int gm = m0 + wm * TM + im * FM + i;
+            if (gm >= p.M) continue;
+            float v[FN];
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                float x = acc[i][j][r];
+                if (bias && gn + j < p.N) x += bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk];
+                if (p.relu) x = x > 0.f ? x : 0.f;
+                v[j] = x;
+            }
+            float* dst = C + (long)gm * p.ldc + gn;
+            if (vec_ok && FN == 4) {
+                floatx4 o = {v[0], v[1], v[2], v[3]};
+                *reinterpret_cast<floatx4*>(dst) = o;
+            } else if (vec_ok && FN == 2) {
+                floatx2 o = {v[0], v[1]};
+                *reinterpret_cast<floatx2*>(dst) = o;
+            } else {
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+                    if (gn + j < p.N) dst[j] = v[j];
+            }
+        }
+    }
+}
+
+// ---- host side -----------------------------------------------------------------------------
+static inline long round_up(long v, long q) { return (v + q - 1) / q * q; }
+
+bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
+    // Worth it when each operand element is re-read by many tiles, i.e. when the GEMM does far
+    // more work per operand byte than the extra rounding pass moves.
+    const double flops = 2.0 * d.M * d.N * d.K;
+    const double cvt_bytes = 6.0 * ((double)d.M * d.K + (double)d.N * d.K);
+    if (d.M < 512 || d.N < 512 || d.K < 256) return false;
+    return flops / cvt_bytes >= 1024.0;        // >= ~1k flop per byte of conversion traffic
+}
+
+int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
+    constexpr int BM = 256, BN = 256, BK = 32, NSTAGE = 4;
+    const long Mp = round_up(d.M, BM), Np = round_up(d.N, BN), Kp = round_up(d.K, BK);
+    const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
+    // workspace holds one rounded copy per DISTINCT batch member of each operand
+    const long a_n = d.a_stride_n ? d.batch_n : 1, a_c = d.a_stride_c ? d.batch_c : 1;
+    const long b_n = d.b_stride_n ? d.batch_n : 1, b_c = d.b_stride_c ? d.batch_c : 1;
+    const size_t a_elems = (size_t)Mp * Kp, b_elems = (size_t)Np * Kp;
+    const size_t a_total = a_elems * a_n * a_c, b_total = b_elems * b_n * b_c;
+    _Float16* ws = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&ws), (a_total + b_total) * sizeof(_Float16), s)) return rc;
+    _Float16* Ah = ws;
+    _Float16* Bh = ws + a_total;
+
+    const int nkt = (int)(Kp / BK);
+    auto convert = [&](_Float16* dst, const float* src, long R, long Rp, bool k_contig, long ld, long nb, long cb,
+                       long sn, long sc, size_t elems) -> int {
+        for (long i = 0; i < nb; i++) {
+            // the c axis of one n is a plain strided batch -> one launch per n
+            const float* sp = src + i * sn;
+            _Float16* dp = dst + (size_t)i * cb * elems;
+            const int vec = ((ld & 3) == 0) && ((reinterpret_cast<uintptr_t>(sp) & 15) == 0) && ((sc & 3) == 0);
+            dim3 grid((unsigned)nkt, (unsigned)(Rp / CVT_ROWS), (unsigned)cb);
+            if (k_contig)
+                hipLaunchKernelGGL(cvt_block_kernel<true>, grid, dim3(256), 0, s, dp, sp, (int)R, (int)d.K, nkt, ld, sc,
+                                   (long)elems, vec);
+            else
+                hipLaunchKernelGGL(cvt_block_kernel<false>, grid, dim3(256), 0, s, dp, sp, (int)R, (int)d.K, nkt, ld, sc,
+                                   (long)elems, vec);
+        }
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "fp16 rounding pass launch");
+    };
+    int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems);
+    if (rc == NZHIP_OK) rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems);
+    if (rc == NZHIP_OK) {
+        H16Args a;
+        a.A = Ah;
+        a.B = Bh;
+        a.C = d.C;
+        a.bias = d.bias;
+        a.M = (int)d.M;
+        a.N = (int)d.N;
+        a.Kp = (int)Kp;
+        a.ldc = d.ldc;
+        a.batch_c = (int)d.batch_c;
+        a.a_batch = (long)a_elems;
+        a.b_batch = (long)b_elems;
+        a.a_bcast_n = d.a_stride_n == 0;
+        a.a_bcast_c = d.a_stride_c == 0;
+        a.b_bcast_n = d.b_stride_n == 0;
+        a.b_bcast_c = d.b_stride_c == 0;
+        a.a_cn = (int)a_c;
+        a.b_cn = (int)b_c;
+        a.c_sn = d.c_stride_n;
+        a.c_sc = d.c_stride_c;
+        a.bias_sn = d.bias_stride_n;
+        a.bias_sc = d.bias_stride_c;
+        a.bias_sm = d.bias_stride_row;
+        a.bias_sk = d.bias_stride_col;
+        a.relu = d.activation == NZHIP_ACT_RELU;
+        a.tiles_m = (int)(Mp / BM);
+        a.tiles_n = (int)(Np / BN);
+        a.group_m = 4;
+        constexpr size_t lds_bytes = (size_t)NSTAGE * (BM + BN) * 64;
+        auto kfn = gemm_h16_kernel<BM, BN, 2, 2, NSTAGE>;
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) rc = set_hip_error(e, "hipFuncSetAttribute(gemm_h16)");
+            attr_set = true;
+        }
+        if (rc == NZHIP_OK) {
+            dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(d.batch_n * d.batch_c));
+            hipLaunchKernelGGL(kfn, grid, dim3(256), lds_bytes, s, a);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) rc = set_hip_error(e, "gemm_h16 kernel launch");
+        }
+    }
+    int rc2 = workspace_free(ws, s);
+    return rc ? rc : rc2;
+}
+
+}  // namespace nzhip

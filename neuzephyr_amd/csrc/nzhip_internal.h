@@ -14,6 +14,10 @@ int set_hip_error(hipError_t e, const char* what);
 
 // MFMA tile kernels (nzhip_gemm.hip). force_tile: 0 = choose, 128 / 256 = that square tile.
 int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile);
+// Two-pass route for large products: fp16 rounding pass + fp16 GEMM fed by direct-to-LDS loads
+// (nzhip_gemm_h16.hip).
+bool gemm_h16_applicable(const nzhip_gemm_desc& d);
+int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
 // Bandwidth-bound kernels for M <= 8 (nzhip_skinny.hip).
 int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
 bool gemm_skinny_applicable(const nzhip_gemm_desc& d);

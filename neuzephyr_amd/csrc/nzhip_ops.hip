@@ -4,6 +4,8 @@
 // working; the fused route is nzhip_conv2d_forward / nzhip_gemm with bias and activation.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "nzhip_internal.h"
 
 namespace nzhip {
@@ -156,15 +158,22 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
         return check_launch("fill_bias_act_kernel");
     }
     if (gemm_skinny_applicable(d)) return gemm_skinny_dispatch(d, s);
+    // NZHIP_GEMM_ROUTE=fused|h16 overrides the route choice (benchmarking only).
+    static const char* route = getenv("NZHIP_GEMM_ROUTE");
+    const bool force_fused = route && route[0] == 'f', force_h16 = route && route[0] == 'h';
+    if (!force_fused && (force_h16 || gemm_h16_applicable(d))) return gemm_h16_dispatch(d, s);
     return gemm_mfma_dispatch(d, s, 0);
 }
 
-/* Test hook: run the MFMA tile kernel with a forced square tile (128 or 256). */
+/* Test hook: pick the kernel instead of letting the shape decide. tile 128 / 256: the fused
+ * convert-on-load kernel with that square tile; tile 16: the two-pass fp16 route. */
 int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream) {
     if (!desc) return set_error(NZHIP_E_INVALID, "nzhip_gemm: null descriptor");
-    if (tile != 128 && tile != 256) return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128 or 256");
+    if (tile != 128 && tile != 256 && tile != 16)
+        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128, 256 or 16");
     if (int rc = validate_gemm(*desc)) return rc;
     if (desc->M == 0 || desc->N == 0 || desc->K == 0) return nzhip_gemm(desc, stream);
+    if (tile == 16) return gemm_h16_dispatch(*desc, as_stream(stream));
     return gemm_mfma_dispatch(*desc, as_stream(stream), tile);
 }
 

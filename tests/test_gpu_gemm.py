@@ -63,7 +63,7 @@ SHAPES = [(1, 1, 1), (3, 5, 2), (16, 16, 16), (17, 33, 15), (64, 100, 132), (130
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
 @pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("tile", [128, 256, 16])      # fused kernels with that tile; 16 = two-pass fp16 route
 def test_integer_operands_are_bit_exact(nz, M, K, N, a_trans, b_trans, tile):
     rng = np.random.default_rng(M * 7919 + K * 31 + N)
     A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
@@ -113,7 +113,7 @@ def test_config1_gemm_256_uniform(nz, oracle):
     A = oracle.fill((256, 256), 0, "uniform", -1.0, 1.0)
     B = oracle.fill((256, 256), 1000, "uniform", -1.0, 1.0)
     truth = oracle.gemm_f64(A, B)
-    for tile in (128, 256):
+    for tile in (128, 256, 16):
         got = host(nz.gemm(dev(A), dev(B), force_tile=tile))
         check_tolerance(oracle, got, truth, f"G1 tile {tile}")
         # and against the fp32 sequential oracle: same rounding, only the sum order differs
