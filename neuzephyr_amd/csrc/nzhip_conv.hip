@@ -6,6 +6,432 @@
 
 namespace nzhip {
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float round_f16(float x) { return (float)(_Float16)x; }
+
+// ---- direct route: 3x3, stride 1, pad 1, few output channels -------------------------------
+// With a handful of output channels the product has K = C*9 and N = O <= 4: far too small for
+// MFMA to matter, the op is a pure stream (each input element needed by 9 outputs). Every lane
+// owns 4 adjacent output pixels of ROWS consecutive rows, walks down the image keeping the
+// partial sums of the three output rows an input row contributes to, and reads each input row
+// once: one 16-byte load plus the two halo pixels (which hit in L1, they are the neighbour
+// lanes' 16 bytes). Operands are rounded to fp16 and accumulated in fp32 by FMA in the
+// reference's k order q = c*9 + r*3 + s, so the result equals the k-ascending fp32 sum of the
+// im2col + GEMM graph bit for bit. Output stores are 16-byte and contiguous along w.
+constexpr int DC_ROWS = 4;         // output rows per wave
+constexpr int DC_MAX_C = 8;        // input channels held in the rolling window
+constexpr int DC_MAX_O = 4;
+
+// O_T: output channels per thread; C_T: compile-time input-channel count (0 = runtime loop);
+// VEC: W % 4 == 0 and 16-byte aligned tensors, so every lane's 4 pixels are inside the row and
+// move as one 16-byte access.
+template <int O_T, int C_T, bool VEC>
+__global__ __launch_bounds__(256) void conv3x3_direct_kernel(float* __restrict__ y, const float* __restrict__ x,
+                                                             const float* __restrict__ w_ref,
+                                                             const float* __restrict__ bias, int C_rt, int H, int W,
+                                                             int O, long w_batch_stride, long bias_sp, long bias_sc,
+                                                             int relu) {
+    __shared__ _Float16 wsm[DC_MAX_C * 9 * DC_MAX_O];
+    const int C = C_T ? C_T : C_rt;
+    const int b = blockIdx.z;
+    const float* wb = w_ref + (long)b * w_batch_stride;
+    for (int i = threadIdx.x; i < C * 9 * O; i += 256) wsm[i] = (_Float16)wb[i];     // [q][o], RNE
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int w0 = (blockIdx.x * 64 + lane) * 4;
+    const int h0 = (blockIdx.y * 4 + wave) * DC_ROWS;
+    if (w0 >= W || h0 >= H) return;
+    const float* xb = x + (long)b * C * H * W;
+    float* yb = y + (long)b * O * H * W;
+
+    float acc[DC_ROWS][O_T][4];
+#pragma unroll
+    for (int j = 0; j < DC_ROWS; j++)
+#pragma unroll
+        for (int o = 0; o < O_T; o++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[j][o][e] = 0.f;
+
+    // halo columns, clamped so the address is always inside the row; the value is zeroed afterwards
+    const int wl = w0 > 0 ? w0 - 1 : 0, wr = w0 + 4 < W ? w0 + 4 : W - 1;
+    const bool has_l = w0 > 0, has_r = w0 + 4 < W;
+
+    // load one input row of channel c (columns w0-1 .. w0+4) as raw fp32
+    auto load_row = [&](int c, int t, float (&m)[6]) {
+        const int hi = h0 - 1 + t;
+        const bool row_ok = hi >= 0 && hi < H;                           // wave-uniform
+        const float* row = xb + (long)c * H * W + (long)(row_ok ? hi : 0) * W;
+        if (VEC) {
+            const floatx4 q = *reinterpret_cast<const floatx4*>(row + w0);
+            m[1] = q[0]; m[2] = q[1]; m[3] = q[2]; m[4] = q[3];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int we = w0 + e < W ? w0 + e : W - 1;
+                const float q = row[we];
+                m[1 + e] = w0 + e < W ? q : 0.f;
+            }
+        }
+        const float ql = row[wl], qr = row[wr];
+        m[0] = has_l ? ql : 0.f;
+        m[5] = has_r ? qr : 0.f;
+    };
+    // Round the row to fp16 (RNE) and add its contribution. Input row t feeds output row
+    // j = t - r (r = 0..2); for a fixed output row, r = t - j ascends with t, so the accumulation
+    // order is the reference's q = c*9 + r*3 + s.
+    auto consume_row = [&](int c, int t, const float (&m)[6]) {
+        const int hi = h0 - 1 + t;
+        const bool row_ok = hi >= 0 && hi < H;
+        _Float16 v[6];
+#pragma unroll
+        for (int e = 0; e < 6; e++) v[e] = row_ok ? (_Float16)m[e] : (_Float16)0.f;
+#pragma unroll
+        for (int r = 0; r < 3; r++) {
+            const int j = t - r;
+            if (j < 0 || j >= DC_ROWS) continue;
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
+#pragma unroll
+                for (int o = 0; o < O_T; o++) {
+                    const _Float16 wv = wsm[(c * 9 + r * 3 + s) * O + o];
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        acc[j][o][e] = __builtin_fmaf((float)v[e + s], (float)wv, acc[j][o][e]);
+                }
+            }
+        }
+    };
+    if constexpr (C_T > 0 && C_T <= 3) {
+        // few channels: request every row of every channel before touching any, so a wave pays
+        // the memory latency once
+        float raw[C_T][DC_ROWS + 2][6];
+#pragma unroll
+        for (int c = 0; c < C_T; c++)
+#pragma unroll
+            for (int t = 0; t < DC_ROWS + 2; t++) load_row(c, t, raw[c][t]);
+#pragma unroll
+        for (int c = 0; c < C_T; c++)
+#pragma unroll
+            for (int t = 0; t < DC_ROWS + 2; t++) consume_row(c, t, raw[c][t]);
+    } else {
+        for (int c = 0; c < C; c++) {
+            float raw[DC_ROWS + 2][6];
+#pragma unroll
+            for (int t = 0; t < DC_ROWS + 2; t++) load_row(c, t, raw[t]);
+#pragma unroll
+            for (int t = 0; t < DC_ROWS + 2; t++) consume_row(c, t, raw[t]);
+        }
+    }
+
+#pragma unroll
+    for (int j = 0; j < DC_ROWS; j++) {
+        const int ho = h0 + j;
+        if (ho >= H) continue;
+#pragma unroll
+        for (int o = 0; o < O_T; o++) {
+            float out[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float a = acc[j][o][e];
+                if (bias && (VEC || w0 + e < W)) a += bias[((long)ho * W + w0 + e) * bias_sp + (long)o * bias_sc];
+                if (relu) a = a > 0.f ? a : 0.f;
+                out[e] = a;
+            }
+            float* dst = yb + ((long)o * H + ho) * W + w0;
+            if (VEC) {
+                floatx4 ov = {out[0], out[1], out[2], out[3]};
+                *reinterpret_cast<floatx4*>(dst) = ov;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (w0 + e < W) dst[e] = out[e];
+            }
+        }
+    }
+}
+
+static bool conv_direct_applicable(size_t C, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad) {
+    return K_h == 3 && K_w == 3 && stride == 1 && pad == 1 && C <= DC_MAX_C && O <= DC_MAX_O && O >= 1;
+}
+
+static int conv_direct(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C, size_t H,
+                       size_t W, size_t O, size_t w_batch, int64_t bias_sp, int64_t bias_sc, int act, hipStream_t s) {
+    if (N > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: batch above 65535");
+    const int vec = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
+    dim3 grid((unsigned)((W + 255) / 256), (unsigned)((H + 4 * DC_ROWS - 1) / (4 * DC_ROWS)), (unsigned)N);
+    const long wbs = w_batch > 1 ? (long)(C * 9 * O) : 0;
+#define NZHIP_DC(OT, CT, V)                                                                                     \
+    hipLaunchKernelGGL((conv3x3_direct_kernel<OT, CT, V>), grid, dim3(256), 0, s, y, x, w_ref, bias, (int)C, (int)H, \
+                       (int)W, (int)O, wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU)
+#define NZHIP_DC_O(CT, V)            \
+    switch (O) {                     \
+        case 1: NZHIP_DC(1, CT, V); break; \
+        case 2: NZHIP_DC(2, CT, V); break; \
+        case 3: NZHIP_DC(3, CT, V); break; \
+        default: NZHIP_DC(4, CT, V); break; \
+    }
+    if (vec) {
+        if (C == 3) { NZHIP_DC_O(3, true) } else if (C == 1) { NZHIP_DC_O(1, true) } else { NZHIP_DC_O(0, true) }
+    } else {
+        NZHIP_DC_O(0, false)
+    }
+#undef NZHIP_DC_O
+#undef NZHIP_DC
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv3x3_direct_kernel launch");
+}
+
+// ---- implicit-GEMM route: stride 1, many channels ------------------------------------------
+// No column matrix exists anywhere. A workgroup owns an 8 x 32 patch of output pixels of one
+// image and 128 output channels, and walks the input channels 16 at a time. Per chunk it
+//   * stages the (8+KH-1) x (32+KW-1) x 16 input halo ONCE: fp32 NCHW -> fp16 (RNE),
+//     channel-last in LDS, so the 8 consecutive k a lane feeds to an MFMA are the 8
+//     consecutive channels of one pixel (one 16-byte LDS read), for every filter tap;
+//   * pulls the matching weight slab (pre-rounded to fp16 and pre-arranged by a small
+//     pre-pass into the exact LDS image, 16-byte row pad included) with direct-to-LDS loads;
+//   * issues KH*KW k-steps of v_mfma_f32_32x32x16_f16: weights are the row operand, pixels the
+//     column operand, so lanes map to adjacent pixels and the NCHW store (the reference's
+//     col2im transpose, src/OperationKernels.cu:1364-1376) is contiguous, with bias and ReLU
+//     applied on the way out.
+// k runs in the order (channel chunk, tap, channel) instead of the reference's
+// q = c*KH*KW + r*KW + s; only the fp32 summation order differs.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int IG_TH = 8, IG_TW = 32, IG_CC = 16, IG_BN = 128;
+
+template <int KH, int KW>
+struct IgemmGeom {
+    static constexpr int HH = IG_TH + KH - 1, WW = IG_TW + KW - 1, TAPS = KH * KW;
+    static constexpr int HALO_BYTES = HH * WW * 32;
+    static constexpr int W_PITCH = TAPS * 32 + 16;             // odd multiple of 16 B: conflict-free rows
+    static constexpr int W_BYTES = IG_BN * W_PITCH;            // one (o tile, channel chunk) slab
+    static constexpr int W_PIECES = W_BYTES / 1024;
+    static_assert(W_BYTES % 1024 == 0, "slab must be whole 1 KiB wave loads");
+    static constexpr int HALO_OFF = (W_BYTES + 1023) / 1024 * 1024;
+    static constexpr int LDS_BYTES = HALO_OFF + HALO_BYTES;
+    static constexpr int UNITS = HH * WW * 2;                  // (pixel, 8-channel half) staging tasks
+    static constexpr int PASSES = (UNITS + 255) / 256;
+};
+
+// Pre-pass: w_ref [wb][C*TAPS][O] fp32  ->  fp16 slabs [wb][o_tile][chunk][128][W_PITCH/2].
+template <int KH, int KW>
+__global__ __launch_bounds__(256) void conv_weight_image_kernel(_Float16* __restrict__ dst,
+                                                                const float* __restrict__ w_ref, int C, int O,
+                                                                int n_chunks, int n_otiles) {
+    using G = IgemmGeom<KH, KW>;
+    const int slab = blockIdx.y;                               // (wb * n_otiles + o_tile) * n_chunks + chunk
+    const int chunk = slab % n_chunks, o_tile = (slab / n_chunks) % n_otiles, wb = slab / (n_chunks * n_otiles);
+    const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, o fastest
+    const int o_l = t % IG_BN, rest = t / IG_BN;
+    if (rest >= G::TAPS * IG_CC) return;
+    const int cc = rest % IG_CC, tap = rest / IG_CC;
+    const int c = chunk * IG_CC + cc, o = o_tile * IG_BN + o_l;
+    float v = 0.f;
+    if (c < C && o < O) v = w_ref[((long)wb * C * G::TAPS + (long)c * G::TAPS + tap) * O + o];
+    dst[(long)slab * (G::W_BYTES / 2) + o_l * (G::W_PITCH / 2) + tap * IG_CC + cc] = (_Float16)v;
+}
+
+struct IgemmArgs {
+    float* y;
+    const float* x;
+    const _Float16* wimg;
+    const float* bias;
+    int C, H, W, O, H_out, W_out, pad;
+    int n_chunks, n_otiles, tiles_w, tiles_h;
+    int w_batched;
+    long bias_sp, bias_sc;
+    int relu;
+};
+
+template <int KH, int KW>
+__global__ __launch_bounds__(256, 2) void conv_igemm_kernel(const IgemmArgs p) {
+    using G = IgemmGeom<KH, KW>;
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    char* lds_w = lds;
+    char* lds_h = lds + G::HALO_OFF;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;                   // pixel-row half, channel half
+    const int li = lane & 31, lh = lane >> 5;
+    const int tile_w = blockIdx.x % p.tiles_w, tile_h = blockIdx.x / p.tiles_w;
+    const int o_tile = blockIdx.y, b = blockIdx.z;
+    const int th0 = tile_h * IG_TH, tw0 = tile_w * IG_TW;
+
+    const float* xb = p.x + (long)b * p.C * p.H * p.W;
+    const char* wsrc = reinterpret_cast<const char*>(p.wimg) +
+                       ((long)(p.w_batched ? b : 0) * p.n_otiles + o_tile) * p.n_chunks * G::W_BYTES + lane * 16;
+
+    // this thread's staging tasks: (pixel of the halo, which 8 of the chunk's 16 channels)
+    int st_off[G::PASSES];          // element offset of the pixel inside one channel plane (clamped)
+    int st_lds[G::PASSES];          // LDS byte offset of the 16-byte slot
+    bool st_ok[G::PASSES];          // pixel inside the image
+    int st_h8[G::PASSES];
+#pragma unroll
+    for (int ps = 0; ps < G::PASSES; ps++) {
+        const int unit = ps * 256 + tid;
+        const int ww = unit % G::WW, hh = (unit / G::WW) % G::HH, h8 = unit / (G::WW * G::HH);
+        const int h_in = th0 + hh - p.pad, w_in = tw0 + ww - p.pad;
+        const bool ok = unit < G::UNITS && h_in >= 0 && h_in < p.H && w_in >= 0 && w_in < p.W;
+        st_ok[ps] = ok;
+        st_off[ps] = ok ? h_in * p.W + w_in : 0;
+        st_h8[ps] = h8 & 1;
+        st_lds[ps] = unit < G::UNITS ? (hh * G::WW + ww) * 32 + (((h8 & 1) ^ ((ww >> 3) & 1)) << 4) : -1;
+    }
+
+    floatx16 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    const long plane = (long)p.H * p.W;
+    for (int chunk = 0; chunk < p.n_chunks; chunk++) {
+        __syncthreads();                                        // previous chunk's fragments are consumed
+        // weights slab: straight copy, 1 KiB per wave-wide request
+        for (int j = wave; j < G::W_PIECES; j += 4)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(wsrc + (long)chunk * G::W_BYTES + j * 1024),
+                (__attribute__((address_space(3))) void*)(lds_w + j * 1024), 16, 0, 0);
+        // input halo: 8 channels of one pixel per task
+        float raw[G::PASSES][8];
+#pragma unroll
+        for (int ps = 0; ps < G::PASSES; ps++) {
+            const int c0 = chunk * IG_CC + st_h8[ps] * 8;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const bool ok = st_ok[ps] && (c0 + e < p.C);
+                const float v = xb[ok ? (long)(c0 + e) * plane + st_off[ps] : 0];
+                raw[ps][e] = ok ? v : 0.f;
+            }
+        }
+#pragma unroll
+        for (int ps = 0; ps < G::PASSES; ps++) {
+            half8_t h;
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = (_Float16)raw[ps][e];
+            if (st_lds[ps] >= 0) *reinterpret_cast<half8_t*>(lds_h + st_lds[ps]) = h;
+        }
+        __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): the slab has landed
+        __syncthreads();
+
+#pragma unroll
+        for (int kh = 0; kh < KH; kh++) {
+#pragma unroll
+            for (int kw = 0; kw < KW; kw++) {
+                const int tap = kh * KW + kw;
+                half8_t wf[2], pf[4];
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    wf[i] = *reinterpret_cast<const half8_t*>(lds_w + (wn * 64 + i * 32 + li) * G::W_PITCH + tap * 32 + lh * 16);
+                const int col = li + kw;
+                const int pos = (lh ^ ((col >> 3) & 1)) << 4;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    pf[j] = *reinterpret_cast<const half8_t*>(lds_h + ((wm * 4 + j + kh) * G::WW + col) * 32 + pos);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[i], pf[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- epilogue: bias + activation + NCHW store (lanes = adjacent pixels) -------------------
+    const int wo = tw0 + li;
+    float* yb = p.y + (long)b * p.O * p.H_out * p.W_out;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int ho = th0 + wm * 4 + j;
+        if (ho >= p.H_out || wo >= p.W_out) continue;
+        const long pix = (long)ho * p.W_out + wo;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int o = o_tile * IG_BN + wn * 64 + i * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (o >= p.O) continue;
+                float v = acc[i][j][r];
+                if (p.bias) v += p.bias[pix * p.bias_sp + (long)o * p.bias_sc];
+                if (p.relu) v = v > 0.f ? v : 0.f;
+                yb[(long)o * p.H_out * p.W_out + pix] = v;
+            }
+        }
+    }
+}
+
+static bool conv_igemm_applicable(size_t C, size_t O, size_t K_h, size_t K_w, size_t stride, size_t N) {
+    (void)O;
+    return stride == 1 && ((K_h == 3 && K_w == 3) || (K_h == 1 && K_w == 1)) && C >= 8 && N <= 65535;
+}
+
+template <int KH, int KW>
+static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
+                             size_t H, size_t W, size_t O, size_t pad, size_t w_batch, int64_t bias_sp,
+                             int64_t bias_sc, int act, size_t H_out, size_t W_out, hipStream_t s) {
+    using G = IgemmGeom<KH, KW>;
+    const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + IG_BN - 1) / IG_BN);
+    if (n_otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many output channels");
+    const size_t slabs = (size_t)w_batch * n_otiles * n_chunks;
+    _Float16* wimg = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&wimg), slabs * G::W_BYTES, s)) return rc;
+    int rc = NZHIP_OK;
+    {
+        // pad bytes of the slabs are never read as data; no need to clear them
+        dim3 grid((unsigned)((IG_BN * G::TAPS * IG_CC + 255) / 256), (unsigned)slabs);
+        if (slabs > 65535) {
+            rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: weight set too large for the fused route");
+        } else {
+            hipLaunchKernelGGL((conv_weight_image_kernel<KH, KW>), grid, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O,
+                               n_chunks, n_otiles);
+        }
+    }
+    if (rc == NZHIP_OK) {
+        IgemmArgs a;
+        a.y = y;
+        a.x = x;
+        a.wimg = wimg;
+        a.bias = bias;
+        a.C = (int)C;
+        a.H = (int)H;
+        a.W = (int)W;
+        a.O = (int)O;
+        a.H_out = (int)H_out;
+        a.W_out = (int)W_out;
+        a.pad = (int)pad;
+        a.n_chunks = n_chunks;
+        a.n_otiles = n_otiles;
+        a.tiles_w = (int)((W_out + IG_TW - 1) / IG_TW);
+        a.tiles_h = (int)((H_out + IG_TH - 1) / IG_TH);
+        a.w_batched = w_batch > 1;
+        a.bias_sp = bias_sp;
+        a.bias_sc = bias_sc;
+        a.relu = act == NZHIP_ACT_RELU;
+        auto kfn = conv_igemm_kernel<KH, KW>;
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
+            if (e != hipSuccess) rc = set_hip_error(e, "hipFuncSetAttribute(conv_igemm)");
+            attr_set = true;
+        }
+        if (rc == NZHIP_OK) {
+            dim3 grid((unsigned)(a.tiles_w * a.tiles_h), (unsigned)n_otiles, (unsigned)N);
+            hipLaunchKernelGGL(kfn, grid, dim3(256), G::LDS_BYTES, s, a);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm kernel launch");
+        }
+    }
+    int rc2 = workspace_free(wimg, s);
+    return rc ? rc : rc2;
+}
+
 // General route: column matrix in a pooled workspace, then ONE batched GEMM that computes the
 // transposed product  y_b[O, HW] = w_b^T[O, CKK] * col_b^T[CKK, HW]  so that bias, activation
 // and the col2im transpose (src/OperationKernels.cu:1364-1376) all happen in its epilogue and
@@ -72,6 +498,16 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
     const size_t H_out = (H + 2 * pad - K_h) / stride + 1, W_out = (W + 2 * pad - K_w) / stride + 1;   // Nodes.cu:605-617
     if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (conv_direct_applicable(C, O, K_h, K_w, stride, pad))
+        return conv_direct(y, x, w_ref, bias, N, C, H, W, O, w_batch, bias_stride_pixel, bias_stride_channel,
+                           activation, s);
+    if (conv_igemm_applicable(C, O, K_h, K_w, stride, N) && (long)H * W < 0x7fffffffL) {
+        if (K_h == 3)
+            return conv_igemm_launch<3, 3>(y, x, w_ref, bias, N, C, H, W, O, pad, w_batch, bias_stride_pixel,
+                                           bias_stride_channel, activation, H_out, W_out, s);
+        return conv_igemm_launch<1, 1>(y, x, w_ref, bias, N, C, H, W, O, pad, w_batch, bias_stride_pixel,
+                                       bias_stride_channel, activation, H_out, W_out, s);
+    }
     return conv2d_via_workspace(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
                                 bias_stride_channel, activation, H_out, W_out, s);
 }
