@@ -2,6 +2,8 @@
 // Img2Col -> MatMul -> Bias -> Col2Img [-> ReLU]) as one call.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "nzhip_internal.h"
 
 namespace nzhip {
@@ -200,14 +202,20 @@ static int conv_direct(float* y, const float* x, const float* w_ref, const float
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int IG_TH = 8, IG_TW = 32, IG_CC = 16, IG_BN = 128;
+constexpr int IG_PIX = 256, IG_CC = 16;
 
-template <int KH, int KW>
+// TW: width of the pixel patch (32 or 64); its height is 256 / TW. Wider patches read and write
+// longer contiguous runs per channel plane (better DRAM page locality) at the price of more
+// halo rows per output row.
+// BN: output channels per workgroup (64 or 128). 64 halves the accumulator registers, so more
+// workgroups share a CU and their load / MFMA / store phases overlap.
+template <int KH, int KW, int TW = 32, int BN = 64>
 struct IgemmGeom {
-    static constexpr int HH = IG_TH + KH - 1, WW = IG_TW + KW - 1, TAPS = KH * KW;
+    static constexpr int TH = IG_PIX / TW;
+    static constexpr int HH = TH + KH - 1, WW = TW + KW - 1, TAPS = KH * KW;
     static constexpr int HALO_BYTES = HH * WW * 32;
     static constexpr int W_PITCH = TAPS * 32 + 16;             // odd multiple of 16 B: conflict-free rows
-    static constexpr int W_BYTES = IG_BN * W_PITCH;            // one (o tile, channel chunk) slab
+    static constexpr int W_BYTES = BN * W_PITCH;               // one (o tile, channel chunk) slab
     static constexpr int W_PIECES = W_BYTES / 1024;
     static_assert(W_BYTES % 1024 == 0, "slab must be whole 1 KiB wave loads");
     static constexpr int HALO_OFF = (W_BYTES + 1023) / 1024 * 1024;
@@ -216,19 +224,19 @@ struct IgemmGeom {
     static constexpr int PASSES = (UNITS + 255) / 256;
 };
 
-// Pre-pass: w_ref [wb][C*TAPS][O] fp32  ->  fp16 slabs [wb][o_tile][chunk][128][W_PITCH/2].
-template <int KH, int KW>
+// Pre-pass: w_ref [wb][C*TAPS][O] fp32  ->  fp16 slabs [wb][o_tile][chunk][BN][W_PITCH/2].
+template <int KH, int KW, int BN>
 __global__ __launch_bounds__(256) void conv_weight_image_kernel(_Float16* __restrict__ dst,
                                                                 const float* __restrict__ w_ref, int C, int O,
                                                                 int n_chunks, int n_otiles) {
-    using G = IgemmGeom<KH, KW>;
+    using G = IgemmGeom<KH, KW, 32, BN>;
     const int slab = blockIdx.y;                               // (wb * n_otiles + o_tile) * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = (slab / n_chunks) % n_otiles, wb = slab / (n_chunks * n_otiles);
     const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, o fastest
-    const int o_l = t % IG_BN, rest = t / IG_BN;
+    const int o_l = t % BN, rest = t / BN;
     if (rest >= G::TAPS * IG_CC) return;
     const int cc = rest % IG_CC, tap = rest / IG_CC;
-    const int c = chunk * IG_CC + cc, o = o_tile * IG_BN + o_l;
+    const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
     float v = 0.f;
     if (c < C && o < O) v = w_ref[((long)wb * C * G::TAPS + (long)c * G::TAPS + tap) * O + o];
     dst[(long)slab * (G::W_BYTES / 2) + o_l * (G::W_PITCH / 2) + tap * IG_CC + cc] = (_Float16)v;
@@ -246,137 +254,193 @@ struct IgemmArgs {
     int relu;
 };
 
-template <int KH, int KW>
-__global__ __launch_bounds__(256, 2) void conv_igemm_kernel(const IgemmArgs p) {
-    using G = IgemmGeom<KH, KW>;
+template <int KH, int KW, int TW, int BN, bool VEC4>
+__global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(const IgemmArgs p) {
+    using G = IgemmGeom<KH, KW, TW, BN>;
+    constexpr int CB = TW / 32;                                 // 32-pixel MFMA column blocks per patch row
+    constexpr int WN = BN / 64, WM = 4 / WN;                    // wave grid: WN over channels, WM over pixel blocks
+    constexpr int FP = 8 / WM;                                  // 32-pixel blocks per wave (8 per patch)
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     char* lds_w = lds;
     char* lds_h = lds + G::HALO_OFF;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;                   // pixel-row half, channel half
+    const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, lh = lane >> 5;
     const int tile_w = blockIdx.x % p.tiles_w, tile_h = blockIdx.x / p.tiles_w;
     const int o_tile = blockIdx.y, b = blockIdx.z;
-    const int th0 = tile_h * IG_TH, tw0 = tile_w * IG_TW;
+    const int th0 = tile_h * G::TH, tw0 = tile_w * TW;
 
     const float* xb = p.x + (long)b * p.C * p.H * p.W;
     const char* wsrc = reinterpret_cast<const char*>(p.wimg) +
                        ((long)(p.w_batched ? b : 0) * p.n_otiles + o_tile) * p.n_chunks * G::W_BYTES + lane * 16;
 
-    // this thread's staging tasks: (pixel of the halo, which 8 of the chunk's 16 channels)
-    int st_off[G::PASSES];          // element offset of the pixel inside one channel plane (clamped)
-    int st_lds[G::PASSES];          // LDS byte offset of the 16-byte slot
-    bool st_ok[G::PASSES];          // pixel inside the image
-    int st_h8[G::PASSES];
-#pragma unroll
-    for (int ps = 0; ps < G::PASSES; ps++) {
-        const int unit = ps * 256 + tid;
-        const int ww = unit % G::WW, hh = (unit / G::WW) % G::HH, h8 = unit / (G::WW * G::HH);
-        const int h_in = th0 + hh - p.pad, w_in = tw0 + ww - p.pad;
-        const bool ok = unit < G::UNITS && h_in >= 0 && h_in < p.H && w_in >= 0 && w_in < p.W;
-        st_ok[ps] = ok;
-        st_off[ps] = ok ? h_in * p.W + w_in : 0;
-        st_h8[ps] = h8 & 1;
-        st_lds[ps] = unit < G::UNITS ? (hh * G::WW + ww) * 32 + (((h8 & 1) ^ ((ww >> 3) & 1)) << 4) : -1;
+    // Staging tasks of one chunk. "Core" tasks move 4 adjacent pixels x 8 channels: eight 16-byte
+    // loads (one per channel plane, whole 128-byte lines per 8 lanes), transposed in registers
+    // into four channel-last 16-byte LDS slots. "Edge" tasks move the KW-1 halo columns left and
+    // right of the 32-pixel core, one pixel x 8 channels each. VEC4 (W % 4 == 0, aligned x)
+    // guarantees a core quad is entirely inside or outside the image.
+    constexpr int W4 = TW / 4;                                   // quads per patch row
+    constexpr int CORE_TASKS = 2 * G::HH * W4, EDGE_TASKS = 2 * G::HH * (KW - 1);
+    static_assert(CORE_TASKS + EDGE_TASKS <= 256, "one task per thread");
+    const bool is_core = tid < CORE_TASKS, is_edge = !is_core && tid < CORE_TASKS + EDGE_TASKS;
+    int t_h8, t_hh, t_ww;                                        // 8-channel half, halo row, first halo column
+    if (is_core) {
+        const int w4 = tid % W4;
+        t_hh = (tid / W4) % G::HH;
+        t_h8 = tid / (W4 * G::HH);
+        t_ww = p.pad + 4 * w4;                                   // halo column of image column tw0 + 4*w4
+    } else {
+        const int e = tid - CORE_TASKS;
+        const int ecol = (KW > 1) ? e % (KW - 1) : 0;
+        t_hh = (KW > 1) ? (e / (KW - 1)) % G::HH : 0;
+        t_h8 = (KW > 1) ? e / ((KW - 1) * G::HH) : 0;
+        t_ww = ecol < p.pad ? ecol : TW + ecol;
     }
+    const int t_hin = th0 + t_hh - p.pad, t_win = tw0 + t_ww - p.pad;
+    const bool row_ok = (is_core || is_edge) && t_hin >= 0 && t_hin < p.H;
+    bool col_ok[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) col_ok[q] = row_ok && t_win + q >= 0 && t_win + q < p.W && (is_core || q == 0);
+    const int t_off = row_ok ? t_hin * p.W + (t_win < 0 ? 0 : (t_win >= p.W ? p.W - 1 : t_win)) : 0;
+    const bool quad_ok = VEC4 && col_ok[0];                      // whole quad in range, 16-byte aligned
 
-    floatx16 acc[2][4];
+    floatx16 acc[2][FP];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < FP; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     const long plane = (long)p.H * p.W;
-    for (int chunk = 0; chunk < p.n_chunks; chunk++) {
-        __syncthreads();                                        // previous chunk's fragments are consumed
-        // weights slab: straight copy, 1 KiB per wave-wide request
+    floatx4 raw[8];                                              // [channel][pixel of the quad]
+
+    auto load_halo = [&](int chunk) {
+        const int c0 = chunk * IG_CC + t_h8 * 8;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const bool c_ok = c0 + e < p.C;
+            const float* src = xb + (c_ok ? (long)(c0 + e) * plane : 0) + t_off;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (VEC4) {
+                if (is_core) {
+                    const floatx4 q = *reinterpret_cast<const floatx4*>(quad_ok ? src : xb);
+                    v = (quad_ok && c_ok) ? q : v;
+                } else {
+                    const float q = *src;
+                    v[0] = (col_ok[0] && c_ok) ? q : 0.f;
+                }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float f = *(col_ok[q] ? src + q : xb);
+                    v[q] = (col_ok[q] && c_ok) ? f : 0.f;
+                }
+            }
+            raw[e] = v;
+        }
+    };
+    auto store_halo = [&]() {
+        if (!(is_core || is_edge)) return;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            if (q > 0 && !is_core) break;
+            half8_t h;
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = (_Float16)raw[e][q];
+            const int ww = t_ww + q;
+            *reinterpret_cast<half8_t*>(lds_h + (t_hh * G::WW + ww) * 32 + ((t_h8 ^ ((ww >> 3) & 1)) << 4)) = h;
+        }
+    };
+    auto load_slab = [&](int chunk) {
         for (int j = wave; j < G::W_PIECES; j += 4)
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void*)(wsrc + (long)chunk * G::W_BYTES + j * 1024),
                 (__attribute__((address_space(3))) void*)(lds_w + j * 1024), 16, 0, 0);
-        // input halo: 8 channels of one pixel per task
-        float raw[G::PASSES][8];
-#pragma unroll
-        for (int ps = 0; ps < G::PASSES; ps++) {
-            const int c0 = chunk * IG_CC + st_h8[ps] * 8;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const bool ok = st_ok[ps] && (c0 + e < p.C);
-                const float v = xb[ok ? (long)(c0 + e) * plane + st_off[ps] : 0];
-                raw[ps][e] = ok ? v : 0.f;
-            }
-        }
-#pragma unroll
-        for (int ps = 0; ps < G::PASSES; ps++) {
-            half8_t h;
-#pragma unroll
-            for (int e = 0; e < 8; e++) h[e] = (_Float16)raw[ps][e];
-            if (st_lds[ps] >= 0) *reinterpret_cast<half8_t*>(lds_h + st_lds[ps]) = h;
-        }
-        __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): the slab has landed
-        __syncthreads();
+    };
 
+    load_halo(0);
+    load_slab(0);
+    for (int chunk = 0; chunk < p.n_chunks; chunk++) {
+        store_halo();                                           // registers (chunk) -> LDS, fp16 channel-last
+        __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): this wave's slab pieces landed
+        __syncthreads();
+        if (chunk + 1 < p.n_chunks) load_halo(chunk + 1);       // lands while the MFMAs below run
 #pragma unroll
         for (int kh = 0; kh < KH; kh++) {
 #pragma unroll
             for (int kw = 0; kw < KW; kw++) {
                 const int tap = kh * KW + kw;
-                half8_t wf[2], pf[4];
+                half8_t wf[2], pf[FP];
 #pragma unroll
                 for (int i = 0; i < 2; i++)
                     wf[i] = *reinterpret_cast<const half8_t*>(lds_w + (wn * 64 + i * 32 + li) * G::W_PITCH + tap * 32 + lh * 16);
-                const int col = li + kw;
-                const int pos = (lh ^ ((col >> 3) & 1)) << 4;
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    pf[j] = *reinterpret_cast<const half8_t*>(lds_h + ((wm * 4 + j + kh) * G::WW + col) * 32 + pos);
+                for (int j = 0; j < FP; j++) {
+                    const int blk = wm * FP + j;                  // pixel block: patch row blk / CB, column block blk % CB
+                    const int col = (blk % CB) * 32 + li + kw;
+                    pf[j] = *reinterpret_cast<const half8_t*>(lds_h + ((blk / CB + kh) * G::WW + col) * 32 +
+                                                               ((lh ^ ((col >> 3) & 1)) << 4));
+                }
 #pragma unroll
                 for (int i = 0; i < 2; i++)
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
+                    for (int j = 0; j < FP; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[i], pf[j], acc[i][j], 0, 0, 0);
             }
         }
+        __syncthreads();                                        // everyone is done reading this chunk's LDS
+        if (chunk + 1 < p.n_chunks) load_slab(chunk + 1);
     }
 
     // ---- epilogue: bias + activation + NCHW store (lanes = adjacent pixels) -------------------
-    const int wo = tw0 + li;
+    // The bias values of one pixel row are requested together, so the wave waits for memory
+    // once per row instead of once per element.
     float* yb = p.y + (long)b * p.O * p.H_out * p.W_out;
+    const long hw_out = (long)p.H_out * p.W_out;
+    const int o_base = o_tile * BN + wn * 64 + lh * 4;
+    const bool o_full = o_tile * BN + BN <= p.O;
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int ho = th0 + wm * 4 + j;
+    for (int j = 0; j < FP; j++) {
+        const int blk = wm * FP + j;
+        const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
         if (ho >= p.H_out || wo >= p.W_out) continue;
         const long pix = (long)ho * p.W_out + wo;
+        float bv[2][16];
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+        for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const int o = o_tile * IG_BN + wn * 64 + i * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (o >= p.O) continue;
-                float v = acc[i][j][r];
-                if (p.bias) v += p.bias[pix * p.bias_sp + (long)o * p.bias_sc];
-                if (p.relu) v = v > 0.f ? v : 0.f;
-                yb[(long)o * p.H_out * p.W_out + pix] = v;
+                const int o = o_base + i * 32 + (r >> 2) * 8 + (r & 3);
+                bv[i][r] = (p.bias && (o_full || o < p.O)) ? p.bias[pix * p.bias_sp + (long)o * p.bias_sc] : 0.f;
             }
-        }
+        float* dst = yb + pix;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int o = o_base + i * 32 + (r >> 2) * 8 + (r & 3);
+                float v = acc[i][j][r] + bv[i][r];
+                if (p.relu) v = v > 0.f ? v : 0.f;
+                if (o_full || o < p.O) dst[(long)o * hw_out] = v;
+            }
     }
 }
 
-static bool conv_igemm_applicable(size_t C, size_t O, size_t K_h, size_t K_w, size_t stride, size_t N) {
+static bool conv_igemm_applicable(size_t C, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t N) {
     (void)O;
-    return stride == 1 && ((K_h == 3 && K_w == 3) || (K_h == 1 && K_w == 1)) && C >= 8 && N <= 65535;
+    // pad <= K_w - 1 keeps the 32 aligned core columns of a tile inside its halo
+    return stride == 1 && ((K_h == 3 && K_w == 3) || (K_h == 1 && K_w == 1)) && pad <= K_w - 1 && C >= 8 && N <= 65535;
 }
 
-template <int KH, int KW>
+template <int KH, int KW, int TW, int BN>
 static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
                              size_t H, size_t W, size_t O, size_t pad, size_t w_batch, int64_t bias_sp,
                              int64_t bias_sc, int act, size_t H_out, size_t W_out, hipStream_t s) {
-    using G = IgemmGeom<KH, KW>;
-    const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + IG_BN - 1) / IG_BN);
+    using G = IgemmGeom<KH, KW, TW, BN>;
+    const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
     if (n_otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many output channels");
     const size_t slabs = (size_t)w_batch * n_otiles * n_chunks;
     _Float16* wimg = nullptr;
@@ -384,11 +448,11 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     int rc = NZHIP_OK;
     {
         // pad bytes of the slabs are never read as data; no need to clear them
-        dim3 grid((unsigned)((IG_BN * G::TAPS * IG_CC + 255) / 256), (unsigned)slabs);
+        dim3 grid((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)slabs);
         if (slabs > 65535) {
             rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: weight set too large for the fused route");
         } else {
-            hipLaunchKernelGGL((conv_weight_image_kernel<KH, KW>), grid, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O,
+            hipLaunchKernelGGL((conv_weight_image_kernel<KH, KW, BN>), grid, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O,
                                n_chunks, n_otiles);
         }
     }
@@ -407,17 +471,21 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         a.pad = (int)pad;
         a.n_chunks = n_chunks;
         a.n_otiles = n_otiles;
-        a.tiles_w = (int)((W_out + IG_TW - 1) / IG_TW);
-        a.tiles_h = (int)((H_out + IG_TH - 1) / IG_TH);
+        a.tiles_w = (int)((W_out + TW - 1) / TW);
+        a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
         a.w_batched = w_batch > 1;
         a.bias_sp = bias_sp;
         a.bias_sc = bias_sc;
         a.relu = act == NZHIP_ACT_RELU;
-        auto kfn = conv_igemm_kernel<KH, KW>;
+        const bool vec4 = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+        auto kfn = vec4 ? conv_igemm_kernel<KH, KW, TW, BN, true> : conv_igemm_kernel<KH, KW, TW, BN, false>;
         static bool attr_set = false;
         if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(conv_igemm_kernel<KH, KW, TW, BN, true>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
+            if (e == hipSuccess)
+                e = hipFuncSetAttribute(reinterpret_cast<const void*>(conv_igemm_kernel<KH, KW, TW, BN, false>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
             if (e != hipSuccess) rc = set_hip_error(e, "hipFuncSetAttribute(conv_igemm)");
             attr_set = true;
         }
@@ -501,12 +569,24 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
     if (conv_direct_applicable(C, O, K_h, K_w, stride, pad))
         return conv_direct(y, x, w_ref, bias, N, C, H, W, O, w_batch, bias_stride_pixel, bias_stride_channel,
                            activation, s);
-    if (conv_igemm_applicable(C, O, K_h, K_w, stride, N) && (long)H * W < 0x7fffffffL) {
-        if (K_h == 3)
-            return conv_igemm_launch<3, 3>(y, x, w_ref, bias, N, C, H, W, O, pad, w_batch, bias_stride_pixel,
-                                           bias_stride_channel, activation, H_out, W_out, s);
-        return conv_igemm_launch<1, 1>(y, x, w_ref, bias, N, C, H, W, O, pad, w_batch, bias_stride_pixel,
-                                       bias_stride_channel, activation, H_out, W_out, s);
+    if (conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL) {
+        // NZHIP_CONV_TW=32|64 and NZHIP_CONV_BN=64|128 override the tile choice (benchmarking only)
+        static const char* tw_env = getenv("NZHIP_CONV_TW");
+        static const char* bn_env = getenv("NZHIP_CONV_BN");
+        const bool wide = tw_env ? atoi(tw_env) == 64 : W_out >= 64;
+        const bool bn128 = bn_env ? atoi(bn_env) == 128 : O > 64;
+#define NZHIP_IG(KH_, TW_, BN_)                                                                                      \
+    return conv_igemm_launch<KH_, KH_, TW_, BN_>(y, x, w_ref, bias, N, C, H, W, O, pad, w_batch, bias_stride_pixel, \
+                                                 bias_stride_channel, activation, H_out, W_out, s)
+        if (K_h == 3) {
+            if (wide && bn128) NZHIP_IG(3, 64, 128);
+            if (wide) NZHIP_IG(3, 64, 64);
+            if (bn128) NZHIP_IG(3, 32, 128);
+            NZHIP_IG(3, 32, 64);
+        }
+        if (wide) NZHIP_IG(1, 64, 64);
+        NZHIP_IG(1, 32, 64);
+#undef NZHIP_IG
     }
     return conv2d_via_workspace(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
                                 bias_stride_channel, activation, H_out, W_out, s);

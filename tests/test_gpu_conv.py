@@ -73,6 +73,10 @@ CONV_CASES = [
     (1, 3, 40, 64, 1, 3, 3, 1, 1, 1),
     (2, 8, 17, 19, 5, 5, 5, 2, 2, 1),
     (1, 70, 9, 9, 130, 1, 1, 1, 0, 1),
+    (2, 24, 40, 70, 9, 3, 3, 1, 0, 1),      # no padding, ragged width (scalar staging path)
+    (1, 9, 33, 36, 140, 3, 3, 1, 2, 1),     # padding 2: both halo columns on the left
+    (2, 20, 16, 64, 64, 3, 3, 1, 1, 2),     # per-sample weights
+    (1, 16, 12, 40, 8, 3, 3, 1, 3, 1),      # padding larger than the kernel reach: workspace route
 ]
 
 
