@@ -66,8 +66,7 @@ def make_workload(name, orc, capi):
         Ad, Bd = dev(A), dev(B)
         out = torch.empty((n, n), device="cuda")
 
-        def run():
-            capi.gemm(Ad, Bd, out=out)
+        run = capi.prepare_gemm(Ad, Bd, out)
 
         def verify():
             rows = np.sort(np.random.default_rng(5).choice(n, size=16, replace=False))
@@ -100,8 +99,7 @@ def make_workload(name, orc, capi):
         Xd, Wd, bd = dev(X), dev(Wt), dev(bias)
         out = torch.empty((Nb, OUT), device="cuda")
 
-        def run():
-            capi.gemm(Xd, Wd, b_trans=True, bias=bd, bias_strides=(0, 1), relu=True, out=out)
+        run = capi.prepare_gemm(Xd, Wd, out, b_trans=True, bias=bd, bias_strides=(0, 1), relu=True)
 
         def verify():
             truth = np.maximum(orc.gemm_f64(X[:256], Wt, trans_b=True) + bias[None, :].astype(np.float64), 0)
@@ -115,8 +113,7 @@ def make_workload(name, orc, capi):
         ad, Bd = dev(a), dev(Bm)
         out = torch.empty((1, 4096), device="cuda")
 
-        def run():
-            capi.gemm(ad, Bd, out=out)
+        run = capi.prepare_gemm(ad, Bd, out)
 
         def verify():
             return tolerance(orc, out.cpu().numpy(), orc.gemm_f64(a, Bm), name)
@@ -129,8 +126,7 @@ def make_workload(name, orc, capi):
         Ad, Bd = dev(A), dev(B)
         out = torch.empty((1000, 513), device="cuda")
 
-        def run():
-            capi.gemm(Ad, Bd, out=out)
+        run = capi.prepare_gemm(Ad, Bd, out)
 
         def verify():
             return tolerance(orc, out.cpu().numpy(), orc.gemm_f64(A, B), name)

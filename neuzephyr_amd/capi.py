@@ -139,6 +139,32 @@ def gemm(A, B, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), 
     return out
 
 
+def prepare_gemm(A, B, out, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), relu=False, stream=None):
+    """Build the descriptor once and return a zero-argument callable that only enqueues the
+    product (for timing loops, where per-call Python work would otherwise dominate small shapes)."""
+    lib = load()
+    M, K = (A.shape[1], A.shape[0]) if a_trans else A.shape
+    N = B.shape[0] if b_trans else B.shape[1]
+    d = GemmDesc()
+    d.A, d.B, d.C = _dev(A), _dev(B), _dev(out)
+    d.M, d.N, d.K = M, N, K
+    d.lda, d.ldb, d.ldc = A.shape[1], B.shape[1], N
+    d.a_layout = LAYOUT_TRANS if a_trans else LAYOUT_ROW
+    d.b_layout = LAYOUT_TRANS if b_trans else LAYOUT_ROW
+    d.batch_n = d.batch_c = 1
+    if bias is not None:
+        d.bias = _dev(bias)
+        d.bias_stride_row, d.bias_stride_col = bias_strides
+    d.activation = ACT_RELU if relu else ACT_NONE
+    ref, h, fn = C.byref(d), C.c_void_p(_stream_handle(stream)), lib.nzhip_gemm
+
+    def call(_keep=(d, A, B, out, bias)):
+        st = fn(ref, h)
+        if st:
+            check(st)
+    return call
+
+
 def tensorcore_gemm(A, B, out=None, stream=None):
     """4-D batched/broadcast product with the semantics of nz::data::iTensorCoreGEMM."""
     import torch

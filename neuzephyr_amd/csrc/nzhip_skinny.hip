@@ -1,16 +1,314 @@
-// Bandwidth-bound GEMM kernels for very few output rows (M <= 8): GEMV-shaped products such
-// as a single sample through Model::Linear or the M = 1 case of TensorCoreGEMMParallel
-// (src/OperationKernels.cu:914-1026), where an MFMA tile would be 97 % padding.
+// Bandwidth-bound GEMM kernels for products with very few rows or columns (min(M, N) <= 8):
+// GEMV-shaped work such as one sample through Model::Linear or the M = 1 case of
+// TensorCoreGEMMParallel (src/OperationKernels.cu:914-1026), where an MFMA tile would be >= 75 %
+// padding and the reference pads 1 row up to 16 (:921-923). The big operand is streamed from
+// HBM exactly once with 16-byte loads; both operands are rounded to fp16 (RNE) on the fly and
+// products are accumulated in fp32, as the tensor-core path does.
+//
+// Formulation: out(s, l) = sum_k S(s, k) * L(k, l), s < SR <= 8 ("skinny" side), l the long side.
+//   KL kernel: L is stored with l contiguous  (L(k,l) at L[k*ld + l]); lanes own 4 adjacent l,
+//              waves and grid.y split k; partial sums meet in LDS, then (if k is split over
+//              blocks) in a workspace that a small second kernel reduces deterministically.
+//   LK kernel: L is stored with k contiguous  (L(k,l) at L[l*ld + k]); a wave owns 4 rows l,
+//              lanes stride k, and the 64 partial sums are folded with cross-lane shuffles.
 #include <hip/hip_runtime.h>
 
 #include "nzhip_internal.h"
 
 namespace nzhip {
 
-bool gemm_skinny_applicable(const nzhip_gemm_desc&) { return false; }
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-int gemm_skinny_dispatch(const nzhip_gemm_desc&, hipStream_t) {
-    return set_error(NZHIP_E_UNSUPPORTED, "skinny GEMM path not built");
+__device__ __forceinline__ float rnd16(float x) { return (float)(_Float16)x; }
+
+struct SkinnyArgs {
+    const float* S;
+    const float* L;
+    float* out;
+    const float* bias;
+    int SR, LN, K;                  // skinny rows, long extent, reduction extent
+    long s_ss, s_sk;                // S(s,k) at S[s*s_ss + k*s_sk]
+    long ldl;                       // leading dimension of L
+    long o_ss, o_sl;                // out(s,l) at out[s*o_ss + l*o_sl]
+    long b_ss, b_sl;                // bias strides
+    int batch_c;
+    long S_sn, S_sc, L_sn, L_sc, o_sn, o_sc, b_sn, b_sc;
+    int relu;
+    int ksplit, kslice;             // KL: blocks along k and k per block
+    float* partial;                 // KL with ksplit > 1: [batch][ksplit][SR][LN]
+    int vec;
+};
+
+// ---- KL: stream rows of L -------------------------------------------------------------------
+template <int SR>
+__global__ __launch_bounds__(256) void skinny_kl_kernel(const SkinnyArgs p) {
+    __shared__ float red[4][SR][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int bz = blockIdx.z, bi = bz / p.batch_c, bj = bz % p.batch_c;
+    const float* __restrict__ S = p.S + bi * p.S_sn + bj * p.S_sc;
+    const float* __restrict__ L = p.L + bi * p.L_sn + bj * p.L_sc;
+    const int l0 = (blockIdx.x * 64 + lane) * 4;
+    const int kb = blockIdx.y * p.kslice;
+    const int ke = (kb + p.kslice < p.K) ? kb + p.kslice : p.K;
+
+    float acc[SR][4];
+#pragma unroll
+    for (int s = 0; s < SR; s++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[s][e] = 0.f;
+
+    const bool in_l = l0 < p.LN;
+    const bool full = p.vec && (l0 + 4 <= p.LN);
+    // waves interleave k so that the four of them read four adjacent rows at a time
+    for (int k = kb + wave; k < ke; k += 4) {
+        floatx4 v = {0.f, 0.f, 0.f, 0.f};
+        const float* row = L + (long)k * p.ldl;
+        if (full) {
+            v = *reinterpret_cast<const floatx4*>(row + l0);
+        } else if (in_l) {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (l0 + e < p.LN) v[e] = row[l0 + e];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = rnd16(v[e]);
+#pragma unroll
+        for (int s = 0; s < SR; s++) {
+            const float a = (s < p.SR) ? rnd16(S[s * p.s_ss + k * p.s_sk]) : 0.f;   // wave-uniform address
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[s][e] = __builtin_fmaf(a, v[e], acc[s][e]);
+        }
+    }
+    // fold the four waves
+#pragma unroll
+    for (int s = 0; s < SR; s++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) red[wave][s][lane * 4 + e] = acc[s][e];
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < SR * 256; idx += 256) {
+        const int s = idx / 256, c = idx % 256;
+        const int l = blockIdx.x * 256 + c;
+        if (s >= p.SR || l >= p.LN) continue;
+        const float v = (red[0][s][c] + red[1][s][c]) + (red[2][s][c] + red[3][s][c]);
+        if (p.ksplit > 1) {
+            p.partial[(((long)bz * p.ksplit + blockIdx.y) * p.SR + s) * p.LN + l] = v;
+        } else {
+            float x = v;
+            if (p.bias) x += p.bias[bi * p.b_sn + bj * p.b_sc + s * p.b_ss + l * p.b_sl];
+            if (p.relu) x = x > 0.f ? x : 0.f;
+            p.out[bi * p.o_sn + bj * p.o_sc + s * p.o_ss + l * p.o_sl] = x;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(const SkinnyArgs p) {
+    // 64 outputs per block; the 4 waves take interleaved partials (fixed order => deterministic),
+    // loads are independent so they pipeline, and LDS folds the 4 wave sums.
+    __shared__ float red[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const long t = (long)blockIdx.x * 64 + lane;
+    const long total = (long)p.SR * p.LN;
+    const int bz = blockIdx.z, bi = bz / p.batch_c, bj = bz % p.batch_c;
+    float x = 0.f;
+    if (t < total) {
+        const float* src = p.partial + (long)bz * p.ksplit * total + t;
+#pragma unroll 8
+        for (int q = wave; q < p.ksplit; q += 4) x += src[(long)q * total];
+    }
+    red[wave][lane] = x;
+    __syncthreads();
+    if (wave == 0 && t < total) {
+        const int s = (int)(t / p.LN), l = (int)(t % p.LN);
+        x = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
+        if (p.bias) x += p.bias[bi * p.b_sn + bj * p.b_sc + s * p.b_ss + l * p.b_sl];
+        if (p.relu) x = x > 0.f ? x : 0.f;
+        p.out[bi * p.o_sn + bj * p.o_sc + s * p.o_ss + l * p.o_sl] = x;
+    }
+}
+
+// ---- LK: rows of L are dot products ------------------------------------------------------------
+template <int SR>
+__global__ __launch_bounds__(256) void skinny_lk_kernel(const SkinnyArgs p) {
+    constexpr int LR = 4;                                          // rows of L per wave
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int bz = blockIdx.z, bi = bz / p.batch_c, bj = bz % p.batch_c;
+    const float* __restrict__ S = p.S + bi * p.S_sn + bj * p.S_sc;
+    const float* __restrict__ L = p.L + bi * p.L_sn + bj * p.L_sc;
+    const int l0 = (blockIdx.x * 4 + wave) * LR;
+    if (l0 >= p.LN) return;
+
+    float acc[SR][LR];
+#pragma unroll
+    for (int s = 0; s < SR; s++)
+#pragma unroll
+        for (int r = 0; r < LR; r++) acc[s][r] = 0.f;
+
+    const bool s_contig = p.s_sk == 1;
+    for (int k0 = lane * 4; k0 < p.K; k0 += 256) {
+        const bool fullk = p.vec && (k0 + 4 <= p.K);
+        floatx4 sv[SR];
+#pragma unroll
+        for (int s = 0; s < SR; s++) {
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (s < p.SR) {
+                const float* q = S + s * p.s_ss + (long)k0 * p.s_sk;
+                if (fullk && s_contig && ((p.s_ss & 3) == 0)) {
+                    v = *reinterpret_cast<const floatx4*>(q);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (k0 + e < p.K) v[e] = q[e * p.s_sk];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = rnd16(v[e]);
+            sv[s] = v;
+        }
+#pragma unroll
+        for (int r = 0; r < LR; r++) {
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (l0 + r < p.LN) {
+                const float* q = L + (long)(l0 + r) * p.ldl + k0;
+                if (fullk) {
+                    v = *reinterpret_cast<const floatx4*>(q);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (k0 + e < p.K) v[e] = q[e];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = rnd16(v[e]);
+#pragma unroll
+            for (int s = 0; s < SR; s++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[s][r] = __builtin_fmaf(sv[s][e], v[e], acc[s][r]);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < SR; s++)
+#pragma unroll
+        for (int r = 0; r < LR; r++) {
+            float v = acc[s][r];
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+            acc[s][r] = v;
+        }
+    if (lane == 0) {
+#pragma unroll
+        for (int s = 0; s < SR; s++)
+#pragma unroll
+            for (int r = 0; r < LR; r++) {
+                const int l = l0 + r;
+                if (s >= p.SR || l >= p.LN) continue;
+                float x = acc[s][r];
+                if (p.bias) x += p.bias[bi * p.b_sn + bj * p.b_sc + s * p.b_ss + l * p.b_sl];
+                if (p.relu) x = x > 0.f ? x : 0.f;
+                p.out[bi * p.o_sn + bj * p.o_sc + s * p.o_ss + l * p.o_sl] = x;
+            }
+    }
+}
+
+// ---- host side -------------------------------------------------------------------------------
+bool gemm_skinny_applicable(const nzhip_gemm_desc& d) {
+    const int64_t small = d.M < d.N ? d.M : d.N, big = d.M < d.N ? d.N : d.M;
+    return small >= 1 && small <= 8 && big >= 1 && d.batch_n * d.batch_c <= 65535;
+}
+
+int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream) {
+    const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
+    SkinnyArgs p = {};
+    bool l_is_kl;                    // long operand stored with l contiguous
+    if (d.M <= d.N) {
+        // skinny side = rows of A, long side = columns of B
+        p.S = d.A;
+        p.L = d.B;
+        p.SR = (int)d.M;
+        p.LN = (int)d.N;
+        p.s_ss = a_trans ? 1 : d.lda;
+        p.s_sk = a_trans ? d.lda : 1;
+        p.ldl = d.ldb;
+        l_is_kl = !b_trans;
+        p.o_ss = d.ldc;
+        p.o_sl = 1;
+        p.b_ss = d.bias_stride_row;
+        p.b_sl = d.bias_stride_col;
+        p.S_sn = d.a_stride_n; p.S_sc = d.a_stride_c;
+        p.L_sn = d.b_stride_n; p.L_sc = d.b_stride_c;
+    } else {
+        // skinny side = columns of B, long side = rows of A:  out(s=n, l=m) = sum_k B(k,n) A(m,k)
+        p.S = d.B;
+        p.L = d.A;
+        p.SR = (int)d.N;
+        p.LN = (int)d.M;
+        p.s_ss = b_trans ? d.ldb : 1;
+        p.s_sk = b_trans ? 1 : d.ldb;
+        p.ldl = d.lda;
+        l_is_kl = a_trans;
+        p.o_ss = 1;
+        p.o_sl = d.ldc;
+        p.b_ss = d.bias_stride_col;
+        p.b_sl = d.bias_stride_row;
+        p.S_sn = d.b_stride_n; p.S_sc = d.b_stride_c;
+        p.L_sn = d.a_stride_n; p.L_sc = d.a_stride_c;
+    }
+    p.out = d.C;
+    p.bias = d.bias;
+    p.K = (int)d.K;
+    p.batch_c = (int)d.batch_c;
+    p.o_sn = d.c_stride_n; p.o_sc = d.c_stride_c;
+    p.b_sn = d.bias_stride_n; p.b_sc = d.bias_stride_c;
+    p.relu = d.activation == NZHIP_ACT_RELU;
+    p.vec = ((p.ldl & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.L) & 15) == 0) && ((p.L_sn & 3) == 0) &&
+            ((p.L_sc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.S) & 15) == 0) && ((p.S_sn & 3) == 0) &&
+            ((p.S_sc & 3) == 0);
+    const unsigned batch = (unsigned)(d.batch_n * d.batch_c);
+    const int sr_t = p.SR <= 1 ? 1 : (p.SR <= 2 ? 2 : (p.SR <= 4 ? 4 : 8));
+    int rc = NZHIP_OK;
+    float* partial = nullptr;
+    if (l_is_kl) {
+        const unsigned lblocks = (unsigned)((p.LN + 255) / 256);
+        // split k until ~4 blocks per CU are in flight, keeping at least 64 k per block
+        int ksplit = (int)(1024 / ((long)lblocks * batch));
+        const int kmax = (p.K + 63) / 64;
+        if (ksplit > kmax) ksplit = kmax;
+        if (ksplit < 1) ksplit = 1;
+        if (ksplit > 65535) ksplit = 65535;
+        p.kslice = ((p.K + ksplit - 1) / ksplit + 3) / 4 * 4;
+        p.ksplit = (p.K + p.kslice - 1) / p.kslice;
+        if (p.ksplit > 1) {
+            rc = workspace_alloc(reinterpret_cast<void**>(&partial), sizeof(float) * batch * p.ksplit * p.SR * p.LN, stream);
+            if (rc) return rc;
+            p.partial = partial;
+        }
+        dim3 grid(lblocks, (unsigned)p.ksplit, batch);
+        switch (sr_t) {
+            case 1: hipLaunchKernelGGL(skinny_kl_kernel<1>, grid, dim3(256), 0, stream, p); break;
+            case 2: hipLaunchKernelGGL(skinny_kl_kernel<2>, grid, dim3(256), 0, stream, p); break;
+            case 4: hipLaunchKernelGGL(skinny_kl_kernel<4>, grid, dim3(256), 0, stream, p); break;
+            default: hipLaunchKernelGGL(skinny_kl_kernel<8>, grid, dim3(256), 0, stream, p); break;
+        }
+        if (p.ksplit > 1) {
+            dim3 g2((unsigned)(((long)p.SR * p.LN + 63) / 64), 1, batch);
+            hipLaunchKernelGGL(skinny_reduce_kernel, g2, dim3(256), 0, stream, p);
+        }
+    } else {
+        dim3 grid((unsigned)((p.LN + 15) / 16), 1, batch);
+        if (grid.x > 0x7fffffffu / 2) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_gemm: long extent too large");
+        switch (sr_t) {
+            case 1: hipLaunchKernelGGL(skinny_lk_kernel<1>, grid, dim3(256), 0, stream, p); break;
+            case 2: hipLaunchKernelGGL(skinny_lk_kernel<2>, grid, dim3(256), 0, stream, p); break;
+            case 4: hipLaunchKernelGGL(skinny_lk_kernel<4>, grid, dim3(256), 0, stream, p); break;
+            default: hipLaunchKernelGGL(skinny_lk_kernel<8>, grid, dim3(256), 0, stream, p); break;
+        }
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) rc = set_hip_error(e, "skinny GEMM kernel launch");
+    if (partial) {
+        int rc2 = workspace_free(partial, stream);
+        if (!rc) rc = rc2;
+    }
+    return rc;
 }
 
 }  // namespace nzhip

@@ -75,6 +75,40 @@ def test_integer_operands_are_bit_exact(nz, M, K, N, a_trans, b_trans, tile):
     assert np.array_equal(got, expect)
 
 
+SKINNY = [(1, 1, 1), (1, 4096, 64), (1, 777, 513), (3, 300, 1000), (8, 64, 260), (5, 1000, 7), (1000, 77, 3),
+          (300, 40, 1), (2049, 130, 8), (7, 9, 4100), (1, 5, 3)]
+
+
+@pytest.mark.parametrize("M,K,N", SKINNY)
+@pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
+def test_skinny_products_are_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans):
+    # min(M, N) <= 8 takes the bandwidth-bound kernels; bias and ReLU ride along
+    rng = np.random.default_rng(M * 31 + K * 7 + N)
+    A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+    B = rng.integers(-8, 9, size=(K, N)).astype(np.float32)
+    bias = rng.integers(-50, 51, size=(M, N)).astype(np.float32)
+    expect = np.maximum((A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32) + bias, 0)
+    got = host(nz.gemm(dev(A.T if a_trans else A), dev(B.T if b_trans else B), a_trans=a_trans, b_trans=b_trans,
+                       bias=dev(bias), bias_strides=(N, 1), relu=True))
+    assert np.array_equal(got, expect)
+
+
+def test_skinny_batched_linear_single_sample(nz, oracle):
+    # one sample through Model::Linear: W[1,1,OUT,IN] x[1,1,IN,1]
+    OUT, IN = 1000, 515
+    W = oracle.fill((1, 1, OUT, IN), 71, "uniform", -0.1, 0.1)
+    x = oracle.fill((1, 1, IN, 1), 72, "normal", 0.0, 1.0)
+    got = host(nz.tensorcore_gemm(dev(W), dev(x))).reshape(OUT)
+    truth = oracle.gemm_f64(W.reshape(OUT, IN), x.reshape(IN, 1)).reshape(OUT)
+    check_tolerance(oracle, got, truth, "single-sample linear")
+    # batched GEMVs that cannot be collapsed (both operands batched): [3,2,1,64] x [3,2,64,300]
+    A = oracle.fill((3, 2, 1, 64), 73, "uniform", -1.0, 1.0)
+    Bm = oracle.fill((3, 2, 64, 300), 74, "uniform", -1.0, 1.0)
+    got = host(nz.tensorcore_gemm(dev(A), dev(Bm)))
+    ref = oracle.tensorcore_gemm(A, Bm)
+    assert np.max(np.abs(got - ref)) <= 1e-4
+
+
 def test_unaligned_base_pointers_take_the_scalar_path(nz):
     import torch
     rng = np.random.default_rng(5)
