@@ -45,8 +45,38 @@ def build_library(verbose: bool = False) -> str:
     return LIB
 
 
+NZ = os.path.join(HERE, "nz")
+NZ_LIB = os.path.join(HERE, "libnz_amd.so")
+CXX = os.environ.get("CXX", "g++")
+
+
+def build_host_layer(verbose: bool = False) -> str:
+    """libnz_amd.so: the C++ nz:: API (plain host C++; talks to libnzhip.so through the C-ABI),
+    plus its two test executables."""
+    inc = ["-I" + os.path.join(NZ, "include"), "-I" + os.path.join(os.path.dirname(HERE), "include")]
+    srcs = sorted(os.path.join(NZ, "src", f) for f in os.listdir(os.path.join(NZ, "src")) if f.endswith(".cpp"))
+    link = ["-L" + HERE, "-lnzhip"]
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd)
+
+    run([CXX, "-std=c++17", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "-fvisibility=hidden", *inc, *srcs,
+         "-o", NZ_LIB, *link, "-Wl,-rpath,$ORIGIN"])
+    tests = os.path.join(NZ, "tests")
+    common = ["-std=c++17", "-Wall", "-Wno-unused-result", *inc, "-L" + HERE, "-lnz_amd", "-lnzhip",
+              "-Wl,-rpath,$ORIGIN/../..", "-pthread"]
+    # host-only tests run under AddressSanitizer + UBSan (host code only; no GPU code is involved)
+    run([CXX, "-O1", "-g", "-fsanitize=address,undefined", os.path.join(tests, "test_host.cpp"),
+         "-o", os.path.join(tests, "test_host"), *common])
+    run([CXX, "-O2", "-mf16c", os.path.join(tests, "test_gpu.cpp"), "-o", os.path.join(tests, "test_gpu"), *common])
+    return NZ_LIB
+
+
 def build_all(verbose: bool = False) -> None:
     build_library(verbose=verbose)
+    build_host_layer(verbose=verbose)
 
 
 if __name__ == "__main__":

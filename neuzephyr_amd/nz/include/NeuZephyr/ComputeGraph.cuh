@@ -1,0 +1,51 @@
+// Topological executor for the forward pass (reference: include/NeuZephyr/ComputeGraph.cuh,
+// src/ComputeGraph.cu:258-296 Kahn sort, :405-412 forward). On top of the reference's
+// node-by-node execution, chains of Model-internal nodes that form a Conv2d
+// (Img2Col -> MatMul [-> Add] -> Col2Img [-> ReLU]) or a Linear (MatMul(W, x) [-> Add] [-> ReLU])
+// are issued as ONE fused kernel; setFusion(false) restores plain node-by-node execution,
+// which yields the same values up to fp32 summation order.
+#ifndef NZ_COMPUTE_GRAPH_CUH
+#define NZ_COMPUTE_GRAPH_CUH
+#include <functional>
+#include <iosfwd>
+#include <string>
+#include <vector>
+
+#include "Nodes.cuh"
+#include "dl_export.cuh"
+
+namespace nz::graph {
+    using namespace nodes;
+    using namespace data;
+
+    class DL_API ComputeGraph {
+    public:
+        ComputeGraph() = default;
+        friend DL_API std::ostream& operator<<(std::ostream& os, ComputeGraph& graph);
+
+        Node* addNode(Node* node);
+        io::InputNode* addInput(io::InputNode* input);
+        io::OutputNode* addOutput(io::OutputNode* node);
+        [[nodiscard]] bool inGraph(Node* node) const;
+        void topologicalSort();                          // throws std::runtime_error("Graph has cycle")
+        [[nodiscard]] bool isSorted() const;
+        void forward();
+        void backward();                                 // not part of this path: throws std::logic_error
+        [[nodiscard]] io::OutputNode* getOutputNode() const;   // throws std::runtime_error without exactly one output
+        void setFusion(bool enabled);
+        [[nodiscard]] size_t fusedGroupCount() const { return fusedGroups; }
+        [[nodiscard]] const std::vector<Node*>& getNodes() const { return nodes; }
+
+    private:
+        void buildPlan();
+        std::vector<Node*> nodes;
+        std::vector<io::InputNode*> inputNodes;
+        std::vector<io::OutputNode*> outputNodes;
+        std::vector<Node*> sortedNodes;
+        std::vector<std::function<void()>> plan;         // what forward() runs, in order
+        bool fusion = true;
+        bool planned = false;
+        size_t fusedGroups = 0;
+    };
+}
+#endif

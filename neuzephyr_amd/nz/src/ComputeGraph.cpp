@@ -1,0 +1,212 @@
+#include "NeuZephyr/ComputeGraph.cuh"
+
+#include <algorithm>
+#include <iostream>
+#include <queue>
+#include <stdexcept>
+#include <unordered_map>
+#include <unordered_set>
+
+#include "NeuZephyr/TensorOperations.cuh"
+
+namespace nz::graph {
+    Node* ComputeGraph::addNode(Node* node) {
+        if (!inGraph(node)) {
+            nodes.push_back(node);
+            planned = false;
+            sortedNodes.clear();
+        }
+        return node;
+    }
+
+    io::InputNode* ComputeGraph::addInput(io::InputNode* input) {
+        addNode(input);
+        inputNodes.push_back(input);
+        return input;
+    }
+
+    io::OutputNode* ComputeGraph::addOutput(io::OutputNode* node) {
+        addNode(node);
+        outputNodes.push_back(node);
+        return node;
+    }
+
+    bool ComputeGraph::inGraph(Node* node) const { return std::find(nodes.begin(), nodes.end(), node) != nodes.end(); }
+
+    bool ComputeGraph::isSorted() const { return !nodes.empty() && sortedNodes.size() == nodes.size(); }
+
+    void ComputeGraph::setFusion(const bool enabled) {
+        fusion = enabled;
+        planned = false;
+    }
+
+    // Kahn's algorithm, breadth first in insertion order (src/ComputeGraph.cu:258-296).
+    void ComputeGraph::topologicalSort() {
+        sortedNodes.clear();
+        std::unordered_map<Node*, int> inDegree;
+        std::unordered_map<Node*, std::vector<Node*>> consumers;
+        for (Node* node : nodes) {
+            inDegree.emplace(node, 0);
+            for (Node* input : node->inputs) {
+                consumers[input].push_back(node);
+                inDegree[node]++;
+            }
+        }
+        std::queue<Node*> ready;
+        for (Node* node : nodes)
+            if (inDegree[node] == 0) ready.push(node);
+        while (!ready.empty()) {
+            Node* node = ready.front();
+            ready.pop();
+            sortedNodes.push_back(node);
+            for (Node* next : consumers[node])
+                if (--inDegree[next] == 0) ready.push(next);
+        }
+        if (sortedNodes.size() != nodes.size()) throw std::runtime_error("Graph has cycle");
+        planned = false;
+    }
+
+    namespace {
+        template <typename T>
+        T* as(Node* n, const char* type) {
+            return (n && n->type == type) ? dynamic_cast<T*>(n) : nullptr;
+        }
+    }
+
+    // Turns the sorted node list into the list of calls forward() makes. A chain is fused only if
+    // every node whose output is skipped is Model-internal and has exactly one consumer.
+    void ComputeGraph::buildPlan() {
+        plan.clear();
+        fusedGroups = 0;
+        std::unordered_map<Node*, std::vector<Node*>> consumers;
+        for (Node* node : nodes)
+            for (Node* input : node->inputs) consumers[input].push_back(node);
+        const auto soleConsumer = [&](Node* n) -> Node* {
+            const auto it = consumers.find(n);
+            return (it != consumers.end() && it->second.size() == 1) ? it->second[0] : nullptr;
+        };
+        const auto skippable = [&](Node* n) { return n->internal && soleConsumer(n) != nullptr; };
+        struct Group {
+            std::vector<Node*> members;          // nodes whose forward() the fused call replaces
+            std::function<void()> call;
+        };
+        std::vector<Group> groups;
+        std::unordered_map<Node*, size_t> groupOf;
+        const auto covered = [&](Node* n) { return groupOf.count(n) != 0; };
+        const auto addGroup = [&](std::vector<Node*> members, std::function<void()> call) {
+            for (Node* n : members) groupOf[n] = groups.size();
+            groups.push_back({std::move(members), std::move(call)});
+        };
+
+        if (fusion) {
+            for (Node* node : sortedNodes) {
+                auto* mm = as<calc::MatMulNode>(node, "MatMul");
+                if (!mm || covered(mm) || !skippable(mm)) continue;
+                Node* lhs = mm->inputs[0];
+                Node* rhs = mm->inputs[1];
+
+                // ---- Conv2d: Img2Col -> MatMul [-> Add(bias [1,1,HW,O])] -> Col2Img [-> ReLU]
+                if (auto* i2c = as<calc::Img2ColNode>(lhs, "Img2Col"); i2c && skippable(i2c) && !covered(i2c)) {
+                    Node* cur = soleConsumer(mm);
+                    calc::AddNode* add = as<calc::AddNode>(cur, "Add");
+                    Node* biasNode = nullptr;
+                    if (add) {
+                        biasNode = add->inputs[0] == mm ? add->inputs[1] : add->inputs[0];
+                        const auto bs = biasNode->output->shape(), ms = mm->output->shape();
+                        if (!(skippable(add) && bs[0] == 1 && bs[1] == 1 && bs[2] == ms[2] && bs[3] == ms[3])) continue;
+                        cur = soleConsumer(add);
+                    }
+                    auto* c2i = as<calc::Col2ImgNode>(cur, "Col2Img");
+                    const auto xs = i2c->inputs[0]->output->shape(), ws = rhs->output->shape();
+                    if (!c2i || c2i->outputHeight != i2c->outputHeight || c2i->outputWidth != i2c->outputWidth) continue;
+                    if (ws[1] != 1 || (ws[0] != 1 && ws[0] != xs[0]) ||
+                        ws[2] != xs[1] * i2c->kernelHeight * i2c->kernelWidth)
+                        continue;
+                    Node* last = c2i;
+                    bool relu = false;
+                    if (auto* r = as<calc::ReLUNode>(soleConsumer(c2i), "ReLU"); r && skippable(c2i)) {
+                        last = r;
+                        relu = true;
+                    }
+                    Node* x = i2c->inputs[0];
+                    const size_t O = ws[3];
+                    std::vector<Node*> members = {i2c, mm, c2i};
+                    if (add) members.push_back(add);
+                    if (relu) members.push_back(last);
+                    addGroup(std::move(members), [=] {
+                        iConv2dForward(last->output->data(), x->output->data(), rhs->output->data(),
+                                       biasNode ? biasNode->output->data() : nullptr, xs[0], xs[1], xs[2], xs[3], O,
+                                       i2c->kernelHeight, i2c->kernelWidth, i2c->stride, i2c->padding, ws[0],
+                                       static_cast<long long>(O), 1, relu);
+                    });
+                    continue;
+                }
+
+                // ---- Linear: MatMul(W[1,1,OUT,IN], x[N,1,IN,1]) -> Add(bias [1,1,OUT,1]) [-> ReLU]
+                const auto ls = lhs->output->shape(), rs = rhs->output->shape();
+                if (ls[0] == 1 && ls[1] == 1 && rs[1] == 1 && rs[3] == 1 && rs[2] == ls[3]) {
+                    auto* add = as<calc::AddNode>(soleConsumer(mm), "Add");
+                    if (!add) continue;                      // a bare MatMul already is a single kernel
+                    Node* biasNode = add->inputs[0] == mm ? add->inputs[1] : add->inputs[0];
+                    const auto bs = biasNode->output->shape();
+                    if (bs[0] != 1 || bs[1] != 1 || bs[2] != ls[2] || bs[3] != 1) continue;
+                    Node* last = add;
+                    bool relu = false;
+                    if (auto* r = as<calc::ReLUNode>(soleConsumer(add), "ReLU"); r && skippable(add)) {
+                        last = r;
+                        relu = true;
+                    }
+                    const size_t batch = rs[0], in = ls[3], out = ls[2];
+                    std::vector<Node*> members = {mm, add};
+                    if (relu) members.push_back(last);
+                    addGroup(std::move(members), [=] {
+                        iLinearForward(last->output->data(), rhs->output->data(), lhs->output->data(),
+                                       biasNode->output->data(), batch, in, out, relu);
+                    });
+                }
+            }
+        }
+
+        // Emit in topological order. A fused call runs at the position of the LAST of its members,
+        // where every external input of the chain (weights, bias) is guaranteed to be ready.
+        std::unordered_map<Node*, size_t> position;
+        for (size_t i = 0; i < sortedNodes.size(); ++i) position[sortedNodes[i]] = i;
+        std::vector<size_t> emitAt(groups.size(), 0);
+        for (size_t g = 0; g < groups.size(); ++g)
+            for (Node* n : groups[g].members) emitAt[g] = std::max(emitAt[g], position[n]);
+        for (size_t i = 0; i < sortedNodes.size(); ++i) {
+            Node* node = sortedNodes[i];
+            const auto it = groupOf.find(node);
+            if (it == groupOf.end()) {
+                plan.emplace_back([node] { node->forward(); });
+            } else if (emitAt[it->second] == i) {
+                plan.push_back(groups[it->second].call);
+            }
+        }
+        fusedGroups = groups.size();
+        planned = true;
+    }
+
+    void ComputeGraph::forward() {
+        if (!isSorted()) topologicalSort();
+        if (!planned) buildPlan();
+        for (auto& step : plan) step();
+    }
+
+    void ComputeGraph::backward() {
+        throw std::logic_error("ComputeGraph::backward: the backward pass is outside this build's path");
+    }
+
+    io::OutputNode* ComputeGraph::getOutputNode() const {
+        if (outputNodes.empty()) throw std::runtime_error("No output node");
+        if (outputNodes.size() > 1) throw std::runtime_error("Multiple output nodes");
+        return outputNodes[0];
+    }
+
+    std::ostream& operator<<(std::ostream& os, ComputeGraph& graph) {
+        if (!graph.isSorted()) graph.topologicalSort();
+        os << "ComputeGraph: " << graph.nodes.size() << " nodes" << std::endl;
+        for (Node* node : graph.sortedNodes) node->print(os);
+        return os;
+    }
+}

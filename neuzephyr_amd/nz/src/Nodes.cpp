@@ -1,0 +1,155 @@
+#include "NeuZephyr/Nodes.cuh"
+
+#include <algorithm>
+#include <iostream>
+#include <stdexcept>
+
+#include "NeuZephyr/NeuZephyrCudaErrorHandling.cuh"
+#include "NeuZephyr/TensorOperations.cuh"
+#include "nzhip.h"
+
+namespace nz::nodes {
+    namespace {
+        [[noreturn]] void noBackward(const char* node) {
+            throw std::logic_error(std::string(node) + "::backward: the backward pass is outside this build's path");
+        }
+    }
+
+    void Node::print(std::ostream& os) const {
+        os << "Node(" << type << ")";
+        if (output) os << " shape " << output->shape();
+        os << std::endl;
+    }
+
+    void Node::dataInject(Tensor::value_type* data, const bool grad) const { output->dataInject(data, grad); }
+
+    void Node::dataInject(const std::initializer_list<Tensor::value_type>& data, const bool grad) const {
+        output->dataInject(data, grad);
+    }
+
+    namespace io {
+        InputNode::InputNode(const Tensor::shape_type& shape, const bool requires_grad) {
+            output = std::make_shared<Tensor>(shape, requires_grad);
+            type = "Input";
+        }
+
+        InputNode::InputNode(const Tensor& tensor) {
+            output = std::make_shared<Tensor>(tensor);
+            type = "Input";
+        }
+
+        InputNode::InputNode(const Tensor::shape_type& shape, Tensor::value_type* data, const bool requires_grad,
+                             const bool host) {
+            output = std::make_shared<Tensor>(shape, data, requires_grad, host);
+            type = "Input";
+        }
+
+        InputNode::InputNode(const Tensor::shape_type& shape, const std::initializer_list<Tensor::value_type>& data,
+                             const bool requires_grad) {
+            output = std::make_shared<Tensor>(shape, data, requires_grad);
+            type = "Input";
+        }
+
+        OutputNode::OutputNode(Node* input) : loss(0) {
+            inputs.push_back(input);
+            type = "Output";
+        }
+
+        void OutputNode::forward() { output = inputs[0]->output; }
+
+        void OutputNode::backward() { noBackward("OutputNode"); }
+    }
+
+    namespace calc {
+        AddNode::AddNode(Node* input_left, Node* input_right) {
+            const auto l = input_left->output->shape(), r = input_right->output->shape();
+            if (!l.isBroadcastCompatible(r) || l.H() != r.H() || l.W() != r.W()) {
+                throw std::invalid_argument("Shapes are not broadcast compatible.");
+            }
+            inputs.push_back(input_left);
+            inputs.push_back(input_right);
+            const bool requires_grad = input_left->output->requiresGrad() || input_right->output->requiresGrad();
+            output = std::make_shared<Tensor>(l.Broadcast(r), requires_grad);
+            type = "Add";
+        }
+
+        void AddNode::forward() { tensorMatrixAdd(*output, *inputs[0]->output, *inputs[1]->output); }
+        void AddNode::backward() { noBackward("AddNode"); }
+
+        MatMulNode::MatMulNode(Node* input_left, Node* input_right) {
+            const auto l = input_left->output->shape(), r = input_right->output->shape();
+            if (!l.isBroadcastCompatible(r) || l.W() != r.H()) {
+                throw std::invalid_argument("Shapes are not broadcast compatible.");
+            }
+            inputs.push_back(input_left);
+            inputs.push_back(input_right);
+            const bool requires_grad = input_left->output->requiresGrad() || input_right->output->requiresGrad();
+            const Tensor::shape_type shape = {std::max(l[0], r[0]), std::max(l[1], r[1]), l[2], r[3]};
+            output = std::make_shared<Tensor>(shape, requires_grad);
+            type = "MatMul";
+        }
+
+        void MatMulNode::forward() { GEMMTensorCore(*output, *inputs[0]->output, *inputs[1]->output); }
+        void MatMulNode::backward() { noBackward("MatMulNode"); }
+
+        ReLUNode::ReLUNode(Node* input) {
+            inputs.push_back(input);
+            output = std::make_shared<Tensor>(input->output->shape(), input->output->requiresGrad());
+            type = "ReLU";
+        }
+
+        void ReLUNode::forward() { iRELU(output->data(), inputs[0]->output->data(), output->size()); }
+        void ReLUNode::backward() { noBackward("ReLUNode"); }
+
+        ReshapeNode::ReshapeNode(Node* input, const Tensor::shape_type& newShape) : newShape(newShape) {
+            if (input->output->shape().size() != newShape.size()) {
+                throw std::invalid_argument("ReshapeNode: input and new shape must have the same number of dimensions");
+            }
+            inputs.push_back(input);
+            output = std::make_shared<Tensor>(newShape, input->output->requiresGrad());
+            type = "Reshape";
+        }
+
+        void ReshapeNode::forward() {
+            NZ_CHECK(nzhip_memcpy_d2d(output->data(), inputs[0]->output->data(), output->size() * sizeof(Tensor::value_type)));
+        }
+        void ReshapeNode::backward() { noBackward("ReshapeNode"); }
+
+        Img2ColNode::Img2ColNode(Node* input, const Tensor::size_type kernelHeight, const Tensor::size_type kernelWidth,
+                                 const Tensor::size_type stride, const Tensor::size_type padding)
+            : kernelHeight(kernelHeight), kernelWidth(kernelWidth), stride(stride), padding(padding),
+              outputHeight((input->output->shape().H() + 2 * padding - kernelHeight) / stride + 1),
+              outputWidth((input->output->shape().W() + 2 * padding - kernelWidth) / stride + 1) {
+            inputs.push_back(input);
+            const auto s = input->output->shape();
+            output = std::make_shared<Tensor>(
+                Tensor::shape_type{s[0], 1, static_cast<size_t>(outputHeight * outputWidth),
+                                   static_cast<size_t>(kernelHeight * kernelWidth * s[1])},
+                input->output->requiresGrad());
+            type = "Img2Col";
+        }
+
+        void Img2ColNode::forward() {
+            const auto s = inputs[0]->output->shape();
+            iImg2col(output->data(), inputs[0]->output->data(), outputHeight, outputWidth, s[1], kernelHeight, kernelWidth,
+                     stride, padding, s[2], s[3], s[0]);
+        }
+        void Img2ColNode::backward() { noBackward("Img2ColNode"); }
+
+        Col2ImgNode::Col2ImgNode(Node* input, const Tensor::size_type outputHeight, const Tensor::size_type outputWidth)
+            : outputHeight(outputHeight), outputWidth(outputWidth), outputChannels(input->output->shape()[3]) {
+            inputs.push_back(input);
+            output = std::make_shared<Tensor>(
+                Tensor::shape_type(input->output->shape()[0], static_cast<size_t>(outputChannels),
+                                   static_cast<size_t>(outputHeight), static_cast<size_t>(outputWidth)),
+                input->output->requiresGrad());
+            type = "Col2Img";
+        }
+
+        void Col2ImgNode::forward() {
+            iCol2img(output->data(), inputs[0]->output->data(), outputHeight, outputWidth, outputChannels,
+                     inputs[0]->output->shape()[0]);
+        }
+        void Col2ImgNode::backward() { noBackward("Col2ImgNode"); }
+    }
+}

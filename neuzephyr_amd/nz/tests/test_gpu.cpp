@@ -1,0 +1,307 @@
+// GPU tests of the nz:: C++ API on the GEMM path. They restate, against this build, the
+// reference's own tests for the path (test/Test.cpp:708-818 literal MatMul vectors,
+// :2880-3009 im2col loop nest, :3074-3142 col2im) and add Model::Linear / Model::Conv2d, which
+// the reference never tests, against a host computation with the same semantics
+// (fp16-rounded operands via the CPU's F16C converter, wide accumulation).
+#include <immintrin.h>
+
+#include <cmath>
+#include <random>
+#include <sstream>
+
+#include "NeuZephyr/ComputeGraph.cuh"
+#include "NeuZephyr/Model.cuh"
+#include "NeuZephyr/Nodes.cuh"
+#include "NeuZephyr/TensorOperations.cuh"
+#include "mini_test.hpp"
+#include "nzhip.h"
+
+using namespace nz::data;
+using namespace nz::nodes;
+using namespace nz::nodes::io;
+using namespace nz::nodes::calc;
+
+static float f16(float x) { return _cvtsh_ss(_cvtss_sh(x, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC)); }
+
+static std::vector<float> randomVec(size_t n, unsigned seed, float lo, float hi) {
+    std::mt19937 gen(seed);
+    std::uniform_real_distribution<float> dist(lo, hi);
+    std::vector<float> v(n);
+    for (auto& x : v) x = dist(gen);
+    return v;
+}
+
+static bool closeTo(const std::vector<float>& got, const std::vector<double>& want, double rel) {
+    double rms = 0;
+    for (double w : want) rms += w * w;
+    rms = std::sqrt(rms / (want.empty() ? 1 : want.size()));
+    for (size_t i = 0; i < want.size(); ++i) {
+        const double d = std::fabs(got[i] - want[i]);
+        if (!(d <= rel * std::max(std::fabs(want[i]), rms))) {
+            std::printf("  mismatch at %zu: got %g want %g\n", i, got[i], want[i]);
+            return false;
+        }
+    }
+    return got.size() == want.size();
+}
+
+static const std::vector<float> kData1 = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12};
+static const std::vector<float> kData2 = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18};
+static const std::vector<float> kExpected = {22, 28, 49, 64, 58, 64, 139, 154, 94, 100, 229, 244,
+                                             76, 100, 103, 136, 220, 244, 301, 334, 364, 388, 499, 532};
+
+TEST(TensorCore, TensorCoreGEMMTest) {
+    Tensor tensor1({2, 1, 2, 3}), tensor2({1, 3, 3, 2});
+    tensor1.dataInject(kData1.begin(), kData1.end());
+    tensor2.dataInject(kData2.begin(), kData2.end());
+    Tensor result({2, 3, 2, 2});
+    GEMMTensorCore(result, tensor1, tensor2);
+    Tensor expected({2, 3, 2, 2});
+    expected.dataInject(kExpected.begin(), kExpected.end());
+    EXPECT_EQ(result, expected);
+    EXPECT_TRUE(result.hostData() == kExpected);             // exact, not merely within 1e-5
+}
+
+TEST(NodeBasic, MatMulForward) {
+    InputNode input1({2, 1, 2, 3}), input2({1, 3, 3, 2});
+    input1.dataInject(kData1.begin(), kData1.end());
+    input2.dataInject(kData2.begin(), kData2.end());
+    MatMulNode mul(&input1, &input2);
+    mul.forward();
+    Tensor expected({2, 3, 2, 2});
+    expected.dataInject(kExpected.begin(), kExpected.end());
+    EXPECT_EQ(*mul.output, expected);
+}
+
+TEST(TensorBasic, InjectCompareCopyMove) {
+    Tensor t({1, 2, 2, 2});
+    std::vector<float> shortData(7, 1.f), data = {1, 2, 3, 4, 5, 6, 7, 8};
+    EXPECT_THROW(t.dataInject(shortData.begin(), shortData.end()), std::runtime_error);
+    t.dataInject(data.begin(), data.end());
+    EXPECT_TRUE(t.hostData() == data);
+    Tensor copy(t);
+    EXPECT_EQ(copy, t);
+    Tensor moved(std::move(copy));
+    EXPECT_EQ(moved, t);
+    EXPECT_EQ(copy.size(), 0u);
+    Tensor other({1, 2, 2, 2}, {1, 2, 3, 4, 5, 6, 7, 8.001f});
+    EXPECT_TRUE(other != t);
+    Tensor withGrad({1, 2, 2, 2}, true);
+    EXPECT_TRUE(withGrad != t);                               // requiresGrad flags differ
+    EXPECT_THROW(Tensor({1, 1, 2, 2}, {1.f, 2.f}), std::invalid_argument);
+    t.fill(3.5f);
+    EXPECT_TRUE(t.hostData() == std::vector<float>(8, 3.5f));
+    t.randomize(3);
+    for (float v : t.hostData()) EXPECT_TRUE(v > 0.f && v <= 1.f);
+}
+
+TEST(NodeBasic, img2colForward) {
+    const size_t n = 2, c = 3, h = 4, w = 5, k_h = 3, k_w = 3, stride = 1, pad = 1;
+    const size_t H_out = (h + 2 * pad - k_h) / stride + 1, W_out = (w + 2 * pad - k_w) / stride + 1;
+    std::vector<float> inputData = randomVec(n * c * h * w, 11, 0.1f, 0.9f);
+    std::vector<float> expectedData(n * H_out * W_out * k_h * k_w * c);
+    for (size_t b = 0; b < n; ++b)
+        for (size_t i = 0; i < H_out; ++i)
+            for (size_t j = 0; j < W_out; ++j)
+                for (size_t r = 0; r < k_h; ++r)
+                    for (size_t s = 0; s < k_w; ++s)
+                        for (size_t c_in = 0; c_in < c; ++c_in) {
+                            const int h_in = static_cast<int>(i * stride + r) - static_cast<int>(pad);
+                            const int w_in = static_cast<int>(j * stride + s) - static_cast<int>(pad);
+                            float val = 0.0f;
+                            if (h_in >= 0 && h_in < static_cast<int>(h) && w_in >= 0 && w_in < static_cast<int>(w))
+                                val = inputData[b * (c * h * w) + c_in * (h * w) + h_in * w + w_in];
+                            expectedData[b * (H_out * W_out * k_h * k_w * c) + (i * W_out + j) * (k_h * k_w * c) +
+                                         c_in * (k_h * k_w) + r * k_w + s] = val;
+                        }
+    InputNode input({n, c, h, w});
+    input.dataInject(inputData.begin(), inputData.end());
+    Img2ColNode result(&input, k_h, k_w, stride, pad);
+    result.forward();
+    Tensor expected({n, 1, H_out * W_out, k_h * k_w * c});
+    expected.dataInject(expectedData.begin(), expectedData.end());
+    EXPECT_EQ(expected, *result.output);
+    EXPECT_EQ(expected, tensorImg2col(*input.output, k_h, k_w, stride, pad));
+}
+
+TEST(NodeBasic, col2imgForward) {
+    const size_t n = 2, c = 3, h = 4, w = 5;
+    std::vector<float> inputData = randomVec(n * c * h * w, 12, 0.1f, 0.9f), expectedData(n * c * h * w);
+    for (size_t b = 0; b < n; ++b)
+        for (size_t j = 0; j < c; ++j)
+            for (size_t k = 0; k < h; ++k)
+                for (size_t l = 0; l < w; ++l)
+                    expectedData[b * (c * h * w) + j * (h * w) + k * w + l] = inputData[b * (c * h * w) + (k * w + l) * c + j];
+    InputNode input({n, 1, h * w, c});
+    input.dataInject(inputData.begin(), inputData.end());
+    Col2ImgNode result(&input, h, w);
+    result.forward();
+    Tensor expected({n, c, h, w});
+    expected.dataInject(expectedData.begin(), expectedData.end());
+    EXPECT_EQ(expected, *result.output);
+    EXPECT_EQ(expected, tensorCol2img(*input.output, h, w));
+}
+
+TEST(NodeBasic, AddBroadcastAndReLU) {
+    InputNode a({2, 2, 1, 3}, {1, -2, 3, -4, 5, -6, 7, -8, 9, -10, 11, -12});
+    InputNode b({1, 1, 1, 3}, {0.5f, 0.5f, -20.f});
+    AddNode add(&a, &b);
+    add.forward();
+    ReLUNode relu(&add);
+    relu.forward();
+    const std::vector<float> want = {1.5f, 0, 0, 0, 5.5f, 0, 7.5f, 0, 0, 0, 11.5f, 0};
+    EXPECT_TRUE(relu.output->hostData() == want);
+    Tensor out({2, 2, 1, 3});
+    Tensor bad({1, 1, 2, 3});
+    EXPECT_THROW(tensorMatrixAdd(out, *a.output, bad), std::invalid_argument);
+}
+
+// ---- Model::Linear ----------------------------------------------------------------------------
+struct LinearModel : nz::Model {
+    InputNode input;
+    LinearModel(size_t batch, size_t features, size_t out, bool relu) : input({batch, 1, features, 1}) {
+        Node* x = Linear(&input, out);
+        if (relu) x = ReLU(x);
+        defaultOutput(x);
+    }
+};
+
+TEST(Model, LinearFusedEqualsUnfusedEqualsHost) {
+    const size_t batch = 37, in = 200, out = 130;
+    LinearModel m(batch, in, out, true);
+    EXPECT_EQ(m.parameters().size(), 2u);
+    EXPECT_TRUE(m.parameters()[0]->output->shape() == Dimension(1, 1, out, in));      // weight [1,1,OUT,IN]
+    EXPECT_TRUE(m.parameters()[1]->output->shape() == Dimension(1, 1, out, 1));       // bias   [1,1,OUT,1]
+    auto x = randomVec(batch * in, 1, -1.f, 1.f), W = randomVec(out * in, 2, -0.2f, 0.2f), b = randomVec(out, 3, -0.3f, 0.3f);
+    m.input.dataInject(x.begin(), x.end());
+    m.parameters()[0]->dataInject(W.begin(), W.end());
+    m.parameters()[1]->dataInject(b.begin(), b.end());
+    std::vector<double> want(batch * out);
+    for (size_t n = 0; n < batch; ++n)
+        for (size_t o = 0; o < out; ++o) {
+            double acc = 0;
+            for (size_t k = 0; k < in; ++k) acc += static_cast<double>(f16(W[o * in + k])) * f16(x[n * in + k]);
+            acc += b[o];
+            want[n * out + o] = acc > 0 ? acc : 0;
+        }
+    const auto fused = m.forward().hostData();
+    EXPECT_EQ(m.graph().fusedGroupCount(), 1u);
+    EXPECT_TRUE(m.forward().shape() == Dimension(batch, 1, out, 1));
+    EXPECT_TRUE(closeTo(fused, want, 1e-5));
+    m.graph().setFusion(false);
+    const auto unfused = m.forward().hostData();
+    EXPECT_EQ(m.graph().fusedGroupCount(), 0u);
+    EXPECT_TRUE(closeTo(unfused, want, 1e-5));
+}
+
+// ---- Model::Conv2d ----------------------------------------------------------------------------
+struct ConvModel : nz::Model {
+    InputNode input;
+    ConvModel(size_t n, size_t c, size_t h, size_t w, size_t o, size_t k, size_t stride, size_t pad, bool relu)
+        : input({n, c, h, w}) {
+        Node* x = Conv2d(&input, o, k, k, stride, pad);
+        if (relu) x = ReLU(x);
+        defaultOutput(x);
+    }
+};
+
+static void convCase(size_t n, size_t c, size_t h, size_t w, size_t o, size_t k, size_t stride, size_t pad) {
+    ConvModel m(n, c, h, w, o, k, stride, pad, true);
+    const size_t Ho = (h + 2 * pad - k) / stride + 1, Wo = (w + 2 * pad - k) / stride + 1, ckk = c * k * k;
+    EXPECT_TRUE(m.parameters()[0]->output->shape() == Dimension(n, 1, ckk, o));        // one weight copy per sample
+    EXPECT_TRUE(m.parameters()[1]->output->shape() == Dimension(1, 1, Ho * Wo, o));    // per-pixel-per-channel bias
+    auto x = randomVec(n * c * h * w, 5, -1.f, 1.f), W1 = randomVec(ckk * o, 6, -0.3f, 0.3f);
+    auto b = randomVec(Ho * Wo * o, 7, -0.5f, 0.5f);
+    std::vector<float> W(n * ckk * o);
+    for (size_t i = 0; i < n; ++i) std::copy(W1.begin(), W1.end(), W.begin() + i * ckk * o);
+    m.input.dataInject(x.begin(), x.end());
+    m.parameters()[0]->dataInject(W.begin(), W.end());
+    m.parameters()[1]->dataInject(b.begin(), b.end());
+    std::vector<double> want(n * o * Ho * Wo);
+    for (size_t bi = 0; bi < n; ++bi)
+        for (size_t oc = 0; oc < o; ++oc)
+            for (size_t ho = 0; ho < Ho; ++ho)
+                for (size_t wo = 0; wo < Wo; ++wo) {
+                    double acc = 0;
+                    for (size_t ci = 0; ci < c; ++ci)
+                        for (size_t r = 0; r < k; ++r)
+                            for (size_t s = 0; s < k; ++s) {
+                                const long hi = static_cast<long>(ho * stride + r) - static_cast<long>(pad);
+                                const long wi = static_cast<long>(wo * stride + s) - static_cast<long>(pad);
+                                if (hi < 0 || hi >= static_cast<long>(h) || wi < 0 || wi >= static_cast<long>(w)) continue;
+                                acc += static_cast<double>(f16(x[((bi * c + ci) * h + hi) * w + wi])) *
+                                       f16(W1[(ci * k * k + r * k + s) * o + oc]);
+                            }
+                    acc += b[(ho * Wo + wo) * o + oc];
+                    want[((bi * o + oc) * Ho + ho) * Wo + wo] = acc > 0 ? acc : 0;
+                }
+    size_t inUseBefore = 0, inUseFused = 0, cached = 0, allocs = 0;
+    nzhip_allocator_stats(&inUseBefore, &cached, &allocs);
+    const auto fused = m.forward().hostData();
+    nzhip_allocator_stats(&inUseFused, &cached, &allocs);
+    EXPECT_EQ(m.graph().fusedGroupCount(), 1u);
+    EXPECT_TRUE(m.forward().shape() == Dimension(n, o, Ho, Wo));
+    EXPECT_TRUE(closeTo(fused, want, 1e-5));
+    // fused: the column matrix [n,1,Ho*Wo,ckk] was never allocated
+    EXPECT_TRUE(inUseFused - inUseBefore < n * Ho * Wo * ckk * sizeof(float) + n * o * Ho * Wo * sizeof(float) * 2);
+    m.graph().setFusion(false);
+    const auto unfused = m.forward().hostData();
+    EXPECT_TRUE(closeTo(unfused, want, 1e-5));
+}
+
+TEST(Model, Conv2dFusedEqualsUnfusedEqualsHost) {
+    convCase(2, 3, 9, 11, 4, 3, 1, 1);        // few channels: direct stencil route
+    convCase(2, 16, 12, 40, 24, 3, 1, 1);     // implicit-GEMM route
+    convCase(1, 5, 10, 9, 6, 3, 2, 0);        // stride 2: workspace route
+}
+
+struct TwoLayer : nz::Model {
+    InputNode input{{4, 3, 16, 16}};
+    TwoLayer() {
+        Node* x = Conv2d(&input, 8, 3, 3, 1, 1);
+        x = ReLU(x);
+        x = Conv2d(x, 2, 3, 3, 1, 1);
+        x = Linear(x, 10);
+        defaultOutput(x);
+    }
+};
+
+TEST(Model, ConvReluConvLinearRunsFusedAndUnfusedAlike) {
+    TwoLayer m;
+    auto x = randomVec(4 * 3 * 16 * 16, 9, 0.f, 1.f);
+    m.input.dataInject(x.begin(), x.end());
+    for (size_t i = 0; i < m.parameters().size(); ++i) {
+        auto p = randomVec(m.parameters()[i]->output->size(), 20 + i, -0.1f, 0.1f);
+        m.parameters()[i]->dataInject(p.begin(), p.end());
+    }
+    const auto fused = m.forward().hostData();
+    EXPECT_EQ(m.graph().fusedGroupCount(), 3u);
+    EXPECT_TRUE(m.forward().shape() == Dimension(4, 1, 10, 1));
+    m.graph().setFusion(false);
+    const auto unfused = m.forward().hostData();
+    std::vector<double> want(unfused.begin(), unfused.end());
+    EXPECT_TRUE(closeTo(fused, want, 1e-4));
+    std::ostringstream os;
+    os << m.graph();
+    EXPECT_TRUE(os.str().find("Img2Col") != std::string::npos);
+}
+
+TEST(Runtime, AllocatorCachesAndErrorsSurfaceAsExceptions) {
+    size_t inUse0 = 0, cached0 = 0, allocs0 = 0, inUse1 = 0, cached1 = 0, allocs1 = 0;
+    {
+        Tensor t({1, 1, 256, 256});
+        t.clear();
+    }
+    nzhip_allocator_stats(&inUse0, &cached0, &allocs0);
+    {
+        Tensor t({1, 1, 256, 256});
+        t.clear();                                            // served from the cache: no new device allocation
+    }
+    nzhip_allocator_stats(&inUse1, &cached1, &allocs1);
+    EXPECT_EQ(allocs0, allocs1);
+    EXPECT_EQ(inUse0, inUse1);
+    float* out = nullptr;
+    EXPECT_THROW(iRELU(out, out, 16), std::invalid_argument);  // C-ABI status -> exception, nothing launched
+}
+
+int main(int argc, char** argv) { return mini::run_all(argc > 1 ? argv[1] : nullptr); }
