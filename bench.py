@@ -27,7 +27,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
-                    choices=["gemm8192", "gemm_batched", "linear", "gemv", "ragged", "conv_a", "conv_b"])
+                    choices=["gemm8192", "gemm_batched", "linear", "gemv", "ragged", "conv_a", "conv_b", "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary (conv / linear) measurements")
     ap.add_argument("--no-verify", action="store_true")
@@ -156,6 +156,21 @@ def make_workload(name, orc, capi):
         bytes_ = 4.0 * (N * C * H * W + O * C * 9 + O + N * O * H * W)
         return Workload(name, flops, bytes_, run, verify, "hbm",
                         f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},3,3] s1 p1 + bias + ReLU"), None
+    if name == "copy":
+        # Calibration only: a plain device copy of known size (1 GiB read + 1 GiB written), so that
+        # rocprofv3's FETCH_SIZE / WRITE_SIZE readings can be scaled to bytes.
+        n = 1 << 28
+        src = torch.rand(n, device="cuda")
+        dst = torch.empty(n, device="cuda")
+
+        def run():
+            dst.copy_(src)
+
+        def verify():
+            assert torch.equal(dst, src)
+            return {"max_rel": 0.0, "frob_rel": 0.0}
+
+        return Workload(name, 0.0, 8.0 * n, run, verify, "hbm", "torch elementwise copy of 2^28 fp32 (calibration)"), None
     raise ValueError(name)
 
 
