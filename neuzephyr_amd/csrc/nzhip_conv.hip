@@ -12,6 +12,13 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float round_f16(float x) { return (float)(_Float16)x; }
 
+// v when keep, +0 otherwise, as a bit mask: keeps the producing load unconditional (a select on
+// the value invites the compiler to sink the load into a branch, which then has to wait for it
+// immediately and serialises the prefetch).
+__device__ __forceinline__ float keep_or_zero(float v, bool keep) {
+    return __builtin_bit_cast(float, __builtin_bit_cast(unsigned, v) & (keep ? 0xffffffffu : 0u));
+}
+
 // ---- direct route: 3x3, stride 1, pad 1, few output channels -------------------------------
 // With a handful of output channels the product has K = C*9 and N = O <= 4: far too small for
 // MFMA to matter, the op is a pure stream (each input element needed by 9 outputs). Every lane
@@ -77,8 +84,8 @@ __global__ __launch_bounds__(256) void conv3x3_direct_kernel(float* __restrict__
             }
         }
         const float ql = row[wl], qr = row[wr];
-        m[0] = has_l ? ql : 0.f;
-        m[5] = has_r ? qr : 0.f;
+        m[0] = keep_or_zero(ql, has_l);
+        m[5] = keep_or_zero(qr, has_r);
     };
     // Round the row to fp16 (RNE) and add its contribution. Input row t feeds output row
     // j = t - r (r = 0..2); for a fixed output row, r = t - j ascends with t, so the accumulation
@@ -154,6 +161,133 @@ __global__ __launch_bounds__(256) void conv3x3_direct_kernel(float* __restrict__
     }
 }
 
+// ---- streaming variant of the direct route (C <= 4, O <= 2, 16-byte aligned rows) ----------
+// A wave owns a strip of 256 columns x ST_ROWS output rows and walks DOWN it: every input row
+// is requested once, ST_AHEAD rows ahead of its use, rounded to fp16 once, and kept in a
+// rolling window of three rows per channel; as soon as a row arrives, the output row above it
+// is complete and is computed in the reference's k order (c, r, s) and stored. Loads of later
+// rows are in flight while the FMAs of the current row run, so memory and VALU time overlap
+// inside every wave instead of relying on other waves being out of phase.
+constexpr int ST_ROWS = 16, ST_AHEAD = 3;
+
+template <int O_T, int C_T>
+__global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__ y, const float* __restrict__ x,
+                                                             const float* __restrict__ w_ref,
+                                                             const float* __restrict__ bias, int H, int W,
+                                                             long w_batch_stride, long bias_sp, long bias_sc,
+                                                             int relu) {
+    __shared__ float wsm[C_T * 9 * O_T];
+    const int b = blockIdx.z;
+    const float* wb = w_ref + (long)b * w_batch_stride;
+    for (int i = threadIdx.x; i < C_T * 9 * O_T; i += 256) wsm[i] = round_f16(wb[i]);   // [q][o]
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int w0 = (blockIdx.x * 64 + lane) * 4;
+    const int h0 = (blockIdx.y * 4 + wave) * ST_ROWS;
+    if (w0 >= W || h0 >= H) return;
+    const float* xb = x + (long)b * C_T * H * W;
+    float* yb = y + (long)b * O_T * H * W;
+    const long plane = (long)H * W;
+    const int wl = w0 > 0 ? w0 - 1 : 0, wr = w0 + 4 < W ? w0 + 4 : W - 1;
+    const bool has_l = w0 > 0, has_r = w0 + 4 < W;
+    const int rows = (H - h0) < ST_ROWS ? (H - h0) : ST_ROWS;   // output rows of this strip
+    const int T = rows + 2;                                      // input rows h0-1 .. h0+rows
+
+    float raw[3][C_T][6];                                        // rows in flight (t % 3)
+    float braw[3][O_T][4];                                       // bias of the output row each of them completes
+    float win[3][C_T][6];                                        // rounded rows t-2, t-1, t (t % 3)
+
+    // Requests are unconditional (rows beyond the image read row 0, halo columns are clamped);
+    // what must be zero is masked when the row is consumed, so nothing waits at request time.
+    auto row_in_image = [&](int t) { const int hi = h0 - 1 + t; return t < T && hi >= 0 && hi < H; };
+    auto request = [&](int t, float (&dst)[C_T][6], float (&bdst)[O_T][4]) {
+        const float* row = xb + (long)(row_in_image(t) ? h0 - 1 + t : 0) * W;
+        // the bias of output row h0 + t - 2 travels with the input row that completes it, so its
+        // wait never drains the rows requested after it
+        const int hb = (t >= 2 && t < T) ? h0 + t - 2 : h0;
+#pragma unroll
+        for (int o = 0; o < O_T; o++)
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                bdst[o][e] = bias ? bias[((long)hb * W + w0 + e) * bias_sp + (long)o * bias_sc] : 0.f;
+#pragma unroll
+        for (int c = 0; c < C_T; c++) {
+            const floatx4 q = *reinterpret_cast<const floatx4*>(row + c * plane + w0);
+            dst[c][0] = row[c * plane + wl];
+            dst[c][1] = q[0];
+            dst[c][2] = q[1];
+            dst[c][3] = q[2];
+            dst[c][4] = q[3];
+            dst[c][5] = row[c * plane + wr];
+        }
+    };
+
+#pragma unroll
+    for (int t = 0; t < ST_AHEAD; t++) request(t, raw[t], braw[t]);
+
+    for (int t0 = 0; t0 < T; t0 += 3) {
+#pragma unroll
+        for (int u = 0; u < 3; u++) {
+            const int t = t0 + u;                                // t % 3 == u because t0 % 3 == 0
+            if (t >= T) break;
+#pragma unroll
+            for (int c = 0; c < C_T; c++)
+#pragma unroll
+                for (int e = 0; e < 6; e++) {
+                    // Opaque use: pins the rounding (and therefore the wait for the load) HERE, three
+                    // rows after the request; otherwise the compiler moves the conversion up to the
+                    // load and the wave waits for every row as soon as it has asked for it.
+                    float v = raw[u][c][e];
+                    asm volatile("" : "+v"(v));
+                    const bool keep = row_in_image(t) && (e != 0 || has_l) && (e != 5 || has_r);
+                    win[u][c][e] = keep ? round_f16(v) : 0.f;
+                }
+            float bnow[O_T][4];
+#pragma unroll
+            for (int o = 0; o < O_T; o++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    bnow[o][e] = braw[u][o][e];
+                    asm volatile("" : "+v"(bnow[o][e]));
+                }
+            request(t + ST_AHEAD, raw[u], braw[u]);              // slot u is free again
+            if (t < 2) continue;
+            const int ho = h0 + t - 2;                           // output row fed by input rows t-2, t-1, t
+            float acc[O_T][4];
+#pragma unroll
+            for (int o = 0; o < O_T; o++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[o][e] = 0.f;
+#pragma unroll
+            for (int c = 0; c < C_T; c++)
+#pragma unroll
+                for (int r = 0; r < 3; r++) {
+                    const int slot = (u + 1 + r) % 3;            // row t-2+r lives in slot (t-2+r) % 3
+#pragma unroll
+                    for (int s2 = 0; s2 < 3; s2++)
+#pragma unroll
+                        for (int o = 0; o < O_T; o++) {
+                            const float wv = wsm[(c * 9 + r * 3 + s2) * O_T + o];
+#pragma unroll
+                            for (int e = 0; e < 4; e++) acc[o][e] = __builtin_fmaf(win[slot][c][e + s2], wv, acc[o][e]);
+                        }
+                }
+#pragma unroll
+            for (int o = 0; o < O_T; o++) {
+                floatx4 ov;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float a = acc[o][e] + bnow[o][e];
+                    if (relu) a = a > 0.f ? a : 0.f;
+                    ov[e] = a;
+                }
+                *reinterpret_cast<floatx4*>(yb + ((long)o * H + ho) * W + w0) = ov;
+            }
+        }
+    }
+}
+
 static bool conv_direct_applicable(size_t C, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad) {
     return K_h == 3 && K_w == 3 && stride == 1 && pad == 1 && C <= DC_MAX_C && O <= DC_MAX_O && O >= 1;
 }
@@ -164,6 +298,25 @@ static int conv_direct(float* y, const float* x, const float* w_ref, const float
     const int vec = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(y) & 15) == 0);
     dim3 grid((unsigned)((W + 255) / 256), (unsigned)((H + 4 * DC_ROWS - 1) / (4 * DC_ROWS)), (unsigned)N);
     const long wbs = w_batch > 1 ? (long)(C * 9 * O) : 0;
+    if (vec && C <= 4 && O <= 2 && H >= 8) {
+        dim3 sgrid((unsigned)((W + 255) / 256), (unsigned)((H + 4 * ST_ROWS - 1) / (4 * ST_ROWS)), (unsigned)N);
+#define NZHIP_ST(OT, CT)                                                                                         \
+    hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H, (int)W, \
+                       wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU)
+        switch ((int)(O * 10 + C)) {
+            case 11: NZHIP_ST(1, 1); break;
+            case 12: NZHIP_ST(1, 2); break;
+            case 13: NZHIP_ST(1, 3); break;
+            case 14: NZHIP_ST(1, 4); break;
+            case 21: NZHIP_ST(2, 1); break;
+            case 22: NZHIP_ST(2, 2); break;
+            case 23: NZHIP_ST(2, 3); break;
+            default: NZHIP_ST(2, 4); break;
+        }
+#undef NZHIP_ST
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv3x3_stream_kernel launch");
+    }
 #define NZHIP_DC(OT, CT, V)                                                                                     \
     hipLaunchKernelGGL((conv3x3_direct_kernel<OT, CT, V>), grid, dim3(256), 0, s, y, x, w_ref, bias, (int)C, (int)H, \
                        (int)W, (int)O, wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU)
