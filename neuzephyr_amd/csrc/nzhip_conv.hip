@@ -582,6 +582,250 @@ __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(con
     }
 }
 
+// ---- implicit GEMM with the whole weight set resident in LDS -------------------------------
+// When O <= 128 per tile and C*KH*KW*128 fp16 weights (plus one halo) fit in the 160 KiB of LDS,
+// a persistent workgroup loads the weights ONCE and then walks over pixel patches. This removes
+// the per-patch weight re-fetch (half of the L1 fill traffic of the streaming-slab kernel) and
+// lets the epilogue stores of one patch drain while the next patch is staged and computed.
+// Weight rows are unpadded (TAPS*32 bytes); rows o and o+8 would share LDS banks, so the two
+// 16-byte halves of every (row, tap) are swapped when bit 3 of the row is set.
+template <int KH, int KW>
+__global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float16* __restrict__ dst,
+                                                                         const float* __restrict__ w_ref, int C,
+                                                                         int O, int n_chunks, int n_otiles) {
+    constexpr int TAPS = KH * KW, BN = 128;
+    const int slab = blockIdx.y;                               // o_tile * n_chunks + chunk
+    const int chunk = slab % n_chunks, o_tile = slab / n_chunks;
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    const int o_l = t % BN, rest = t / BN;
+    if (rest >= TAPS * IG_CC) return;
+    const int cc = rest % IG_CC, tap = rest / IG_CC;
+    const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
+    float v = 0.f;
+    if (c < C && o < O) v = w_ref[((long)c * TAPS + tap) * O + o];
+    const int half = (cc >> 3) ^ ((o_l >> 3) & 1);
+    dst[(long)slab * (BN * TAPS * IG_CC) + o_l * (TAPS * IG_CC) + tap * IG_CC + half * 8 + (cc & 7)] = (_Float16)v;
+}
+
+template <int KH, int KW, int TW, bool VEC4>
+__global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArgs p, const int n_patches) {
+    using G = IgemmGeom<KH, KW, TW, 128>;
+    constexpr int BN = 128, CB = TW / 32, FP = 4;
+    constexpr int W_PITCH = G::TAPS * 32, W_CHUNK = BN * W_PITCH;           // unpadded rows
+    static_assert(W_CHUNK % 1024 == 0, "chunk must be whole 1 KiB wave loads");
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    char* lds_w = lds;
+    char* lds_h = lds + p.n_chunks * W_CHUNK;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+    const int o_tile = blockIdx.y;
+    const int patches_per_image = p.tiles_w * p.tiles_h;
+    const long plane = (long)p.H * p.W;
+
+    // resident weights: n_chunks * W_CHUNK bytes, 1 KiB per wave-wide request
+    {
+        const char* wsrc = reinterpret_cast<const char*>(p.wimg) + (long)o_tile * p.n_chunks * W_CHUNK + lane * 16;
+        const int pieces = p.n_chunks * (W_CHUNK / 1024);
+        for (int j = wave; j < pieces; j += 4)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc + (long)j * 1024),
+                                             (__attribute__((address_space(3))) void*)(lds_w + j * 1024), 16, 0, 0);
+    }
+
+    // staging task of this thread (same decomposition as the slab kernel)
+    constexpr int W4 = TW / 4;
+    constexpr int CORE_TASKS = 2 * G::HH * W4, EDGE_TASKS = 2 * G::HH * (KW - 1);
+    static_assert(CORE_TASKS + EDGE_TASKS <= 256, "one task per thread");
+    const bool is_core = tid < CORE_TASKS, is_edge = !is_core && tid < CORE_TASKS + EDGE_TASKS;
+    int t_h8, t_hh, t_ww;
+    if (is_core) {
+        t_hh = (tid / W4) % G::HH;
+        t_h8 = tid / (W4 * G::HH);
+        t_ww = p.pad + 4 * (tid % W4);
+    } else {
+        const int e = tid - CORE_TASKS;
+        const int ecol = (KW > 1) ? e % (KW > 1 ? KW - 1 : 1) : 0;
+        t_hh = (KW > 1) ? (e / (KW > 1 ? KW - 1 : 1)) % G::HH : 0;
+        t_h8 = (KW > 1) ? e / ((KW > 1 ? KW - 1 : 1) * G::HH) : 0;
+        t_ww = ecol < p.pad ? ecol : TW + ecol;
+    }
+    t_h8 &= 1;
+
+    // work items of this workgroup: (patch, chunk) pairs, patches strided by the grid
+    const int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int total = my_patches * p.n_chunks;
+
+    floatx4 raw[2][8];
+    auto load_item = [&](int it, floatx4 (&dst)[8]) {
+        if (it >= total) return;
+        const int patch = blockIdx.x + (it / p.n_chunks) * gridDim.x, chunk = it % p.n_chunks;
+        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
+        const int hin = th0 + t_hh - p.pad, win = tw0 + t_ww - p.pad;
+        const bool row_ok = (is_core || is_edge) && hin >= 0 && hin < p.H;
+        const float* xb = p.x + (long)b * p.C * plane;
+        const int c0 = chunk * IG_CC + t_h8 * 8;
+        if (VEC4 && is_core) {
+            const bool ok = row_ok && win >= 0 && win < p.W;       // W % 4 == 0: the quad is all in or all out
+            const long off = ok ? (long)hin * p.W + win : 0;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const bool c_ok = ok && (c0 + e < p.C);
+                const floatx4 q = *reinterpret_cast<const floatx4*>(xb + (c_ok ? (long)(c0 + e) * plane + off : 0));
+                const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+                dst[e] = c_ok ? q : z;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                floatx4 v = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const bool ok = row_ok && (c0 + e < p.C) && win + q >= 0 && win + q < p.W && (is_core || q == 0);
+                    const float f = xb[ok ? (long)(c0 + e) * plane + (long)hin * p.W + win + q : 0];
+                    v[q] = ok ? f : 0.f;
+                }
+                dst[e] = v;
+            }
+        }
+    };
+    auto store_halo = [&](const floatx4 (&src)[8]) {
+        if (!(is_core || is_edge)) return;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            if (q > 0 && !is_core) break;
+            half8_t h;
+#pragma unroll
+            for (int e = 0; e < 8; e++) h[e] = (_Float16)src[e][q];
+            const int ww = t_ww + q;
+            *reinterpret_cast<half8_t*>(lds_h + (t_hh * G::WW + ww) * 32 + ((t_h8 ^ ((ww >> 3) & 1)) << 4)) = h;
+        }
+    };
+
+    floatx16 acc[2][FP];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < FP; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    };
+    zero_acc();
+
+    auto compute = [&](int chunk) {
+        const char* wbase = lds_w + chunk * W_CHUNK;
+#pragma unroll 1
+        for (int kh = 0; kh < KH; kh++) {
+#pragma unroll
+            for (int kw = 0; kw < KW; kw++) {
+                const int tap = kh * KW + kw;
+                half8_t wf[2], pf[FP];
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+                    wf[i] = *reinterpret_cast<const half8_t*>(wbase + (wn * 64 + i * 32 + li) * W_PITCH + tap * 32 +
+                                                               ((lh ^ ((li >> 3) & 1)) << 4));
+#pragma unroll
+                for (int j = 0; j < FP; j++) {
+                    const int blk = wm * FP + j;
+                    const int col = (blk % CB) * 32 + li + kw;
+                    pf[j] = *reinterpret_cast<const half8_t*>(lds_h + ((blk / CB + kh) * G::WW + col) * 32 +
+                                                               ((lh ^ ((col >> 3) & 1)) << 4));
+                }
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < FP; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[i], pf[j], acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+
+    // Per-channel bias (pixel stride 0) is the same for every patch: fetch it once.
+    const int o_base = o_tile * BN + wn * 64 + lh * 4;
+    const bool bias_per_channel = p.bias && p.bias_sp == 0;
+    float bch[2][16];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int rr = 0; rr < 16; rr++) {
+            const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
+            bch[i][rr] = (bias_per_channel && o < p.O) ? p.bias[(long)o * p.bias_sc] : 0.f;
+        }
+
+    auto epilogue = [&](int patch) {
+        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
+        float* yb = p.y + (long)b * p.O * p.H_out * p.W_out;
+        const long hw_out = (long)p.H_out * p.W_out;
+        // whole patch and whole channel tile inside the output: no per-element predicates (uniform test)
+        const bool inside = th0 + G::TH <= p.H_out && tw0 + TW <= p.W_out && o_tile * BN + BN <= p.O;
+#pragma unroll
+        for (int j = 0; j < FP; j++) {
+            const int blk = wm * FP + j;
+            const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
+            const bool pix_ok = inside || (ho < p.H_out && wo < p.W_out);
+            const long pix = pix_ok ? (long)ho * p.W_out + wo : 0;
+            float bv[2][16];
+            if (p.bias && !bias_per_channel) {                   // per-pixel bias: one batch of requests per row
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int rr = 0; rr < 16; rr++) {
+                        const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
+                        bv[i][rr] = p.bias[pix * p.bias_sp + (long)((inside || o < p.O) ? o : 0) * p.bias_sc];
+                    }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int rr = 0; rr < 16; rr++) bv[i][rr] = bch[i][rr];
+            }
+            float* dst = yb + pix;
+            if (inside) {
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int rr = 0; rr < 16; rr++) {
+                        const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
+                        float v = acc[i][j][rr] + bv[i][rr];
+                        if (p.relu) v = v > 0.f ? v : 0.f;
+                        dst[(long)o * hw_out] = v;
+                    }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int rr = 0; rr < 16; rr++) {
+                        const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
+                        float v = acc[i][j][rr] + bv[i][rr];
+                        if (p.relu) v = v > 0.f ? v : 0.f;
+                        if (pix_ok && o < p.O) dst[(long)o * hw_out] = v;
+                    }
+            }
+        }
+    };
+
+    load_item(0, raw[0]);
+    load_item(1, raw[1]);
+    int it = 0;
+    for (int pi = 0; pi < my_patches; pi++) {
+        zero_acc();
+        for (int chunk = 0; chunk < p.n_chunks; chunk++, it++) {
+            const bool odd = it & 1;                             // uniform: which register set holds item it
+            if (odd) store_halo(raw[1]); else store_halo(raw[0]);   // registers (item it) -> LDS
+            if (it == 0) __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);   // vmcnt(0): resident weights landed
+            __syncthreads();
+            if (odd) load_item(it + 2, raw[1]); else load_item(it + 2, raw[0]);   // two items ahead
+            compute(chunk);
+            __syncthreads();                                     // halo may be overwritten
+        }
+        epilogue(blockIdx.x + pi * gridDim.x);
+    }
+}
+
 static bool conv_igemm_applicable(size_t C, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t N) {
     (void)O;
     // pad <= K_w - 1 keeps the 32 aligned core columns of a tile inside its halo
@@ -595,6 +839,53 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     using G = IgemmGeom<KH, KW, TW, BN>;
     const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
     if (n_otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many output channels");
+    // Resident-weight route: shared weights whose fp16 image (unpadded) plus one halo fit in LDS.
+    if constexpr (BN == 128) {
+        constexpr size_t W_CHUNK_R = 128 * (size_t)G::TAPS * 32;
+        const size_t lds_need = (size_t)n_chunks * W_CHUNK_R + G::HALO_BYTES;
+        static const char* res_env = getenv("NZHIP_CONV_RESIDENT");
+        const bool allow = res_env ? atoi(res_env) != 0 : true;
+        if (allow && w_batch == 1 && lds_need <= 160 * 1024 - 512) {
+            _Float16* wres = nullptr;
+            const size_t bytes = (size_t)n_otiles * n_chunks * W_CHUNK_R;
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&wres), bytes, s)) return rc;
+            dim3 pg((unsigned)((128 * G::TAPS * IG_CC + 255) / 256), (unsigned)(n_otiles * n_chunks));
+            hipLaunchKernelGGL((conv_weight_image_resident_kernel<KH, KW>), pg, dim3(256), 0, s, wres, w_ref, (int)C,
+                               (int)O, n_chunks, n_otiles);
+            IgemmArgs a;
+            a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
+            a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.H_out = (int)H_out; a.W_out = (int)W_out;
+            a.pad = (int)pad; a.n_chunks = n_chunks; a.n_otiles = n_otiles;
+            a.tiles_w = (int)((W_out + TW - 1) / TW);
+            a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
+            a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.relu = act == NZHIP_ACT_RELU;
+            const long n_patches = (long)N * a.tiles_w * a.tiles_h;
+            int rc = NZHIP_OK;
+            if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
+            const bool vec4r = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+            auto kres = vec4r ? conv_igemm_resident_kernel<KH, KW, TW, true> : conv_igemm_resident_kernel<KH, KW, TW, false>;
+            if (rc == NZHIP_OK) {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kres),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_need);
+                if (e != hipSuccess) rc = set_hip_error(e, "hipFuncSetAttribute(conv_igemm_resident)");
+            }
+            if (rc == NZHIP_OK) {
+                int cus = 256;
+                hipDeviceProp_t prop;
+                int dev = 0;
+                if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+                    cus = prop.multiProcessorCount;
+                int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
+                if ((long)per_tile > n_patches) per_tile = (int)n_patches;
+                dim3 grid((unsigned)per_tile, (unsigned)n_otiles, 1);
+                hipLaunchKernelGGL(kres, grid, dim3(256), lds_need, s, a, (int)n_patches);
+                hipError_t e = hipGetLastError();
+                if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm_resident kernel launch");
+            }
+            int rc2 = workspace_free(wres, s);
+            return rc ? rc : rc2;
+        }
+    }
     const size_t slabs = (size_t)w_batch * n_otiles * n_chunks;
     _Float16* wimg = nullptr;
     if (int rc = workspace_alloc(reinterpret_cast<void**>(&wimg), slabs * G::W_BYTES, s)) return rc;
