@@ -607,7 +607,9 @@ __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float1
     dst[(long)slab * (BN * TAPS * IG_CC) + o_l * (TAPS * IG_CC) + tap * IG_CC + half * 8 + (cc & 7)] = (_Float16)v;
 }
 
-template <int KH, int KW, int TW, bool VEC4>
+// PIX_BIAS: the bias varies per pixel (the reference's Bias node after the matmul); otherwise it is
+// absent or per channel and is fetched once per workgroup.
+template <int KH, int KW, int TW, bool VEC4, bool PIX_BIAS>
 __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArgs p, const int n_patches) {
     using G = IgemmGeom<KH, KW, TW, 128>;
     constexpr int BN = 128, CB = TW / 32, FP = 4;
@@ -657,27 +659,39 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
     const int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
     const int total = my_patches * p.n_chunks;
 
+    // Staging is split in "request" (load_item, two items ahead) and "consume" (store_halo).
+    // Requests are unconditional loads from clamped, always valid addresses; padding pixels and
+    // channels past C are zeroed at consumption through nv[] (number of valid channels of the
+    // thread's 8, 0 for a pixel outside the image). With VEC4 an edge pixel is fetched as the
+    // aligned quad that holds it (component t_comp), so every lane issues the same instruction.
     floatx4 raw[2][8];
-    auto load_item = [&](int it, floatx4 (&dst)[8]) {
-        if (it >= total) return;
-        const int patch = blockIdx.x + (it / p.n_chunks) * gridDim.x, chunk = it % p.n_chunks;
-        const int b = patch / patches_per_image, r = patch % patches_per_image;
+    int nv[2] = {0, 0};
+    const int t_comp = (t_ww - p.pad) & 3;
+    int ld_patch = blockIdx.x, ld_chunk = 0, ld_it = 0;
+    auto load_item = [&](floatx4 (&dst)[8], int& nvalid) {
+        if (ld_it >= total) return;                              // uniform
+        const int b = ld_patch / patches_per_image, r = ld_patch % patches_per_image;
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
         const int hin = th0 + t_hh - p.pad, win = tw0 + t_ww - p.pad;
         const bool row_ok = (is_core || is_edge) && hin >= 0 && hin < p.H;
         const float* xb = p.x + (long)b * p.C * plane;
-        const int c0 = chunk * IG_CC + t_h8 * 8;
-        if (VEC4 && is_core) {
+        const int c0 = ld_chunk * IG_CC + t_h8 * 8;
+        if (VEC4) {
             const bool ok = row_ok && win >= 0 && win < p.W;       // W % 4 == 0: the quad is all in or all out
-            const long off = ok ? (long)hin * p.W + win : 0;
+            int n = p.C - c0;
+            n = n < 0 ? 0 : (n > 8 ? 8 : n);
+            n = ok ? n : 0;
+            nvalid = n;
+            // lanes without work read the first quad of the image; channels past n repeat the last valid one
+            const long first = ((long)c0 * plane + (long)hin * p.W + (win & ~3)) & -(long)(n > 0);
+            const float* src = xb + first;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const bool c_ok = ok && (c0 + e < p.C);
-                const floatx4 q = *reinterpret_cast<const floatx4*>(xb + (c_ok ? (long)(c0 + e) * plane + off : 0));
-                const floatx4 z = {0.f, 0.f, 0.f, 0.f};
-                dst[e] = c_ok ? q : z;
+                dst[e] = *reinterpret_cast<const floatx4*>(src);
+                src += plane & -(long)(e + 1 < n);
             }
         } else {
+            nvalid = 8;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
@@ -690,17 +704,33 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
                 dst[e] = v;
             }
         }
+        ld_it++;
+        if (++ld_chunk == p.n_chunks) { ld_chunk = 0; ld_patch += gridDim.x; }
     };
-    auto store_halo = [&](const floatx4 (&src)[8]) {
+    auto store_halo = [&](const floatx4 (&src)[8], const int nvalid) {
         if (!(is_core || is_edge)) return;
+        if (is_core) {
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            if (q > 0 && !is_core) break;
+            for (int q = 0; q < 4; q++) {
+                half8_t h;
+#pragma unroll
+                for (int e = 0; e < 8; e++) h[e] = e < nvalid ? (_Float16)src[e][q] : (_Float16)0.f;
+                const int ww = t_ww + q;
+                *reinterpret_cast<half8_t*>(lds_h + (t_hh * G::WW + ww) * 32 + ((t_h8 ^ ((ww >> 3) & 1)) << 4)) = h;
+            }
+        } else {
             half8_t h;
 #pragma unroll
-            for (int e = 0; e < 8; e++) h[e] = (_Float16)src[e][q];
-            const int ww = t_ww + q;
-            *reinterpret_cast<half8_t*>(lds_h + (t_hh * G::WW + ww) * 32 + ((t_h8 ^ ((ww >> 3) & 1)) << 4)) = h;
+            for (int e = 0; e < 8; e++) {
+                float f = src[e][0];
+                if (VEC4) {
+                    f = t_comp == 1 ? src[e][1] : f;
+                    f = t_comp == 2 ? src[e][2] : f;
+                    f = t_comp == 3 ? src[e][3] : f;
+                }
+                h[e] = e < nvalid ? (_Float16)f : (_Float16)0.f;
+            }
+            *reinterpret_cast<half8_t*>(lds_h + (t_hh * G::WW + t_ww) * 32 + ((t_h8 ^ ((t_ww >> 3) & 1)) << 4)) = h;
         }
     };
 
@@ -716,7 +746,7 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
     zero_acc();
 
     auto compute = [&](int chunk) {
-        const char* wbase = lds_w + chunk * W_CHUNK;
+        const char* wbase = lds_w + chunk * W_CHUNK + (wn * 64 + li) * W_PITCH + ((lh ^ ((li >> 3) & 1)) << 4);
 #pragma unroll 1
         for (int kh = 0; kh < KH; kh++) {
 #pragma unroll
@@ -725,8 +755,7 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
                 half8_t wf[2], pf[FP];
 #pragma unroll
                 for (int i = 0; i < 2; i++)
-                    wf[i] = *reinterpret_cast<const half8_t*>(wbase + (wn * 64 + i * 32 + li) * W_PITCH + tap * 32 +
-                                                               ((lh ^ ((li >> 3) & 1)) << 4));
+                    wf[i] = *reinterpret_cast<const half8_t*>(wbase + i * 32 * W_PITCH + tap * 32);
 #pragma unroll
                 for (int j = 0; j < FP; j++) {
                     const int blk = wm * FP + j;
@@ -745,14 +774,15 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
 
     // Per-channel bias (pixel stride 0) is the same for every patch: fetch it once.
     const int o_base = o_tile * BN + wn * 64 + lh * 4;
-    const bool bias_per_channel = p.bias && p.bias_sp == 0;
+    const bool bias_per_channel = !PIX_BIAS && p.bias;
     float bch[2][16];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int rr = 0; rr < 16; rr++) {
             const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
-            bch[i][rr] = (bias_per_channel && o < p.O) ? p.bias[(long)o * p.bias_sc] : 0.f;
+            bch[i][rr] = 0.f;
+            if (bias_per_channel) bch[i][rr] = p.bias[(long)(o < p.O ? o : p.O - 1) * p.bias_sc];   // uniform branch
         }
 
     auto epilogue = [&](int patch) {
@@ -769,7 +799,7 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
             const bool pix_ok = inside || (ho < p.H_out && wo < p.W_out);
             const long pix = pix_ok ? (long)ho * p.W_out + wo : 0;
             float bv[2][16];
-            if (p.bias && !bias_per_channel) {                   // per-pixel bias: one batch of requests per row
+            if (PIX_BIAS) {                                      // per-pixel bias: one batch of requests per row
 #pragma unroll
                 for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -808,17 +838,17 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
         }
     };
 
-    load_item(0, raw[0]);
-    load_item(1, raw[1]);
+    load_item(raw[0], nv[0]);
+    load_item(raw[1], nv[1]);
     int it = 0;
     for (int pi = 0; pi < my_patches; pi++) {
         zero_acc();
         for (int chunk = 0; chunk < p.n_chunks; chunk++, it++) {
             const bool odd = it & 1;                             // uniform: which register set holds item it
-            if (odd) store_halo(raw[1]); else store_halo(raw[0]);   // registers (item it) -> LDS
+            if (odd) store_halo(raw[1], nv[1]); else store_halo(raw[0], nv[0]);   // registers (item it) -> LDS
             if (it == 0) __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);   // vmcnt(0): resident weights landed
             __syncthreads();
-            if (odd) load_item(it + 2, raw[1]); else load_item(it + 2, raw[0]);   // two items ahead
+            if (odd) load_item(raw[1], nv[1]); else load_item(raw[0], nv[0]);   // request item it + 2
             compute(chunk);
             __syncthreads();                                     // halo may be overwritten
         }
@@ -863,7 +893,11 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             int rc = NZHIP_OK;
             if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
             const bool vec4r = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
-            auto kres = vec4r ? conv_igemm_resident_kernel<KH, KW, TW, true> : conv_igemm_resident_kernel<KH, KW, TW, false>;
+            const bool pixb = bias && bias_sp != 0;
+            auto kres = vec4r ? (pixb ? conv_igemm_resident_kernel<KH, KW, TW, true, true>
+                                      : conv_igemm_resident_kernel<KH, KW, TW, true, false>)
+                              : (pixb ? conv_igemm_resident_kernel<KH, KW, TW, false, true>
+                                      : conv_igemm_resident_kernel<KH, KW, TW, false, false>);
             if (rc == NZHIP_OK) {
                 hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kres),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_need);
