@@ -669,11 +669,14 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
     const int t_comp = (t_ww - p.pad) & 3;
     int ld_patch = blockIdx.x, ld_chunk = 0, ld_it = 0;
     auto load_item = [&](floatx4 (&dst)[8], int& nvalid) {
-        if (ld_it >= total) return;                              // uniform
-        const int b = ld_patch / patches_per_image, r = ld_patch % patches_per_image;
+        // Past the last item the requests are still issued (to the first quad of x, results unused):
+        // a fixed number of requests per item lets every wait name exactly the set it needs.
+        const bool live = ld_it < total;                         // uniform
+        const int patch = live ? ld_patch : (int)blockIdx.x;
+        const int b = patch / patches_per_image, r = patch % patches_per_image;
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
         const int hin = th0 + t_hh - p.pad, win = tw0 + t_ww - p.pad;
-        const bool row_ok = (is_core || is_edge) && hin >= 0 && hin < p.H;
+        const bool row_ok = live && (is_core || is_edge) && hin >= 0 && hin < p.H;
         const float* xb = p.x + (long)b * p.C * plane;
         const int c0 = ld_chunk * IG_CC + t_h8 * 8;
         if (VEC4) {
@@ -745,29 +748,39 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
     };
     zero_acc();
 
+    // One fragment set per kw. The LDS reads of a tap are issued before the MFMAs of the tap before
+    // it (the first tap of a filter row is requested during the last tap of the row above), so the
+    // matrix pipe does not wait for LDS latency at every tap.
     auto compute = [&](int chunk) {
         const char* wbase = lds_w + chunk * W_CHUNK + (wn * 64 + li) * W_PITCH + ((lh ^ ((li >> 3) & 1)) << 4);
+        half8_t wf[KW][2], pf[KW][FP];
+        auto read_frags = [&](int kh, int kw, half8_t (&w)[2], half8_t (&x)[FP]) {
+            const int tap = kh * KW + kw;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                w[i] = *reinterpret_cast<const half8_t*>(wbase + i * 32 * W_PITCH + tap * 32);
+#pragma unroll
+            for (int j = 0; j < FP; j++) {
+                const int blk = wm * FP + j;
+                const int col = (blk % CB) * 32 + li + kw;
+                x[j] = *reinterpret_cast<const half8_t*>(lds_h + ((blk / CB + kh) * G::WW + col) * 32 +
+                                                          ((lh ^ ((col >> 3) & 1)) << 4));
+            }
+        };
+        read_frags(0, 0, wf[0], pf[0]);
 #pragma unroll 1
         for (int kh = 0; kh < KH; kh++) {
 #pragma unroll
             for (int kw = 0; kw < KW; kw++) {
-                const int tap = kh * KW + kw;
-                half8_t wf[2], pf[FP];
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-                    wf[i] = *reinterpret_cast<const half8_t*>(wbase + i * 32 * W_PITCH + tap * 32);
-#pragma unroll
-                for (int j = 0; j < FP; j++) {
-                    const int blk = wm * FP + j;
-                    const int col = (blk % CB) * 32 + li + kw;
-                    pf[j] = *reinterpret_cast<const half8_t*>(lds_h + ((blk / CB + kh) * G::WW + col) * 32 +
-                                                               ((lh ^ ((col >> 3) & 1)) << 4));
-                }
+                if (kw + 1 < KW) read_frags(kh, kw + 1, wf[kw + 1], pf[kw + 1]);
+                else if (kh + 1 < KH) read_frags(kh + 1, 0, wf[0], pf[0]);
+                __builtin_amdgcn_sched_barrier(0);               // requests stay ahead of the MFMAs below
 #pragma unroll
                 for (int i = 0; i < 2; i++)
 #pragma unroll
                     for (int j = 0; j < FP; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[i], pf[j], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kw][i], pf[kw][j], acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
@@ -838,19 +851,39 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
         }
     };
 
+    // LDS-only barrier: waits for this wave's LDS traffic, not for the global requests in flight.
+    auto lds_barrier = []() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    // One work item. The register set is a compile-time choice (items alternate between the two
+    // sets), so a set is never copied and its requests stay in flight across a whole item.
+    auto item = [&](floatx4 (&r)[8], int& n, int chunk) {
+        store_halo(r, n);                                        // registers -> LDS (waits for this set only)
+        lds_barrier();
+        load_item(r, n);                                         // request the item two ahead into the same set
+        compute(chunk);
+        lds_barrier();                                           // halo may be overwritten
+    };
+
     load_item(raw[0], nv[0]);
     load_item(raw[1], nv[1]);
-    int it = 0;
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);                 // vmcnt(0): resident weights landed
     for (int pi = 0; pi < my_patches; pi++) {
         zero_acc();
-        for (int chunk = 0; chunk < p.n_chunks; chunk++, it++) {
-            const bool odd = it & 1;                             // uniform: which register set holds item it
-            if (odd) store_halo(raw[1], nv[1]); else store_halo(raw[0], nv[0]);   // registers (item it) -> LDS
-            if (it == 0) __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);   // vmcnt(0): resident weights landed
-            __syncthreads();
-            if (odd) load_item(raw[1], nv[1]); else load_item(raw[0], nv[0]);   // request item it + 2
-            compute(chunk);
-            __syncthreads();                                     // halo may be overwritten
+        int chunk = 0;
+        for (; chunk + 1 < p.n_chunks; chunk += 2) {
+            item(raw[0], nv[0], chunk);
+            item(raw[1], nv[1], chunk + 1);
+        }
+        if (chunk < p.n_chunks) {                                // odd chunk count: the sets trade places
+            item(raw[0], nv[0], chunk);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const floatx4 t = raw[0][e];
+                raw[0][e] = raw[1][e];
+                raw[1][e] = t;
+            }
+            const int t = nv[0];
+            nv[0] = nv[1];
+            nv[1] = t;
         }
         epilogue(blockIdx.x + pi * gridDim.x);
     }
