@@ -609,19 +609,31 @@ __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float1
 
 // PIX_BIAS: the bias varies per pixel (the reference's Bias node after the matmul); otherwise it is
 // absent or per channel and is fetched once per workgroup.
+//
+// Eight waves, two per SIMD. Wave (wm, wn) owns 64 pixels (two 32-pixel blocks) x 64 channels of
+// the 256 x 128 patch tile. A work item is one 16-channel chunk of one patch:
+//     store_halo (registers -> fp16 LDS)  | barrier |  MFMAs  +  "other"  | barrier
+// where "other" = request the halo two items ahead. The two waves of a SIMD run MFMAs and "other"
+// in opposite order, so the matrix pipe of the SIMD is fed by one wave while its partner issues
+// memory and address instructions. After the last chunk of a patch every wave writes its 64 x 64
+// results (bias already in the accumulator, activation on the way out).
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+
 template <int KH, int KW, int TW, bool VEC4, bool PIX_BIAS>
-__global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArgs p, const int n_patches) {
+__global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArgs p, const int n_patches) {
     using G = IgemmGeom<KH, KW, TW, 128>;
-    constexpr int BN = 128, CB = TW / 32, FP = 4;
+    constexpr int BN = 128, CB = TW / 32, FP = 2, NW = 8;
     constexpr int W_PITCH = G::TAPS * 32, W_CHUNK = BN * W_PITCH;           // unpadded rows
     static_assert(W_CHUNK % 1024 == 0, "chunk must be whole 1 KiB wave loads");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     char* lds_w = lds;
     char* lds_h = lds + p.n_chunks * W_CHUNK;
+    float* lds_bias = reinterpret_cast<float*>(lds_h + G::HALO_BYTES);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
+    const bool early = wave < NW / 2;                           // waves w and w + 4 share a SIMD
     const int li = lane & 31, lh = lane >> 5;
     const int o_tile = blockIdx.y;
     const int patches_per_image = p.tiles_w * p.tiles_h;
@@ -631,44 +643,54 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
     {
         const char* wsrc = reinterpret_cast<const char*>(p.wimg) + (long)o_tile * p.n_chunks * W_CHUNK + lane * 16;
         const int pieces = p.n_chunks * (W_CHUNK / 1024);
-        for (int j = wave; j < pieces; j += 4)
+        for (int j = wave; j < pieces; j += NW)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc + (long)j * 1024),
                                              (__attribute__((address_space(3))) void*)(lds_w + j * 1024), 16, 0, 0);
     }
+    float my_bias = 0.f;                                         // requested now, parked in LDS before the first patch
+    if (!PIX_BIAS && p.bias && tid < BN && o_tile * BN + tid < p.O) my_bias = p.bias[(long)(o_tile * BN + tid) * p.bias_sc];
 
-    // staging task of this thread (same decomposition as the slab kernel)
+    // Staging task of this thread: 4 adjacent pixels x 4 channels ("core": four 16-byte loads, one
+    // per channel plane, transposed in registers into four channel-last 8-byte LDS slots) or one
+    // halo-column pixel x 4 channels ("edge").
     constexpr int W4 = TW / 4;
-    constexpr int CORE_TASKS = 2 * G::HH * W4, EDGE_TASKS = 2 * G::HH * (KW - 1);
-    static_assert(CORE_TASKS + EDGE_TASKS <= 256, "one task per thread");
+    constexpr int CORE_TASKS = 4 * G::HH * W4, EDGE_TASKS = 4 * G::HH * (KW - 1);
+    static_assert(CORE_TASKS + EDGE_TASKS <= 512, "one task per thread");
     const bool is_core = tid < CORE_TASKS, is_edge = !is_core && tid < CORE_TASKS + EDGE_TASKS;
-    int t_h8, t_hh, t_ww;
+    int t_q4, t_hh, t_ww;                                        // channel quarter, halo row, first halo column
     if (is_core) {
         t_hh = (tid / W4) % G::HH;
-        t_h8 = tid / (W4 * G::HH);
+        t_q4 = tid / (W4 * G::HH);
         t_ww = p.pad + 4 * (tid % W4);
     } else {
         const int e = tid - CORE_TASKS;
         const int ecol = (KW > 1) ? e % (KW > 1 ? KW - 1 : 1) : 0;
         t_hh = (KW > 1) ? (e / (KW > 1 ? KW - 1 : 1)) % G::HH : 0;
-        t_h8 = (KW > 1) ? e / ((KW > 1 ? KW - 1 : 1) * G::HH) : 0;
+        t_q4 = (KW > 1) ? e / ((KW > 1 ? KW - 1 : 1) * G::HH) : 0;
         t_ww = ecol < p.pad ? ecol : TW + ecol;
     }
-    t_h8 &= 1;
+    t_q4 &= 3;
+    auto halo_slot = [&](int hh, int ww) {                       // 8-byte slot of this thread's channel quarter
+        return lds_h + (hh * G::WW + ww) * 32 + (((t_q4 >> 1) ^ ((ww >> 3) & 1)) << 4) + (t_q4 & 1) * 8;
+    };
 
     // work items of this workgroup: (patch, chunk) pairs, patches strided by the grid
     const int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-    const int total = my_patches * p.n_chunks;
+    // Items per patch are rounded up to an even count: an odd chunk count gets one empty item
+    // (zero halo, no MFMAs) so that every patch starts on the same register set.
+    const int n_items = (p.n_chunks + 1) & ~1;
+    const int total = my_patches * n_items;
 
     // Staging is split in "request" (load_item, two items ahead) and "consume" (store_halo).
     // Requests are unconditional loads from clamped, always valid addresses; padding pixels and
     // channels past C are zeroed at consumption through nv[] (number of valid channels of the
-    // thread's 8, 0 for a pixel outside the image). With VEC4 an edge pixel is fetched as the
+    // thread's 4, 0 for a pixel outside the image). With VEC4 an edge pixel is fetched as the
     // aligned quad that holds it (component t_comp), so every lane issues the same instruction.
-    floatx4 raw[2][8];
+    floatx4 raw[2][4];
     int nv[2] = {0, 0};
     const int t_comp = (t_ww - p.pad) & 3;
     int ld_patch = blockIdx.x, ld_chunk = 0, ld_it = 0;
-    auto load_item = [&](floatx4 (&dst)[8], int& nvalid) {
+    auto load_item = [&](floatx4 (&dst)[4], int& nvalid) {
         // Past the last item the requests are still issued (to the first quad of x, results unused):
         // a fixed number of requests per item lets every wait name exactly the set it needs.
         const bool live = ld_it < total;                         // uniform
@@ -678,25 +700,25 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
         const int hin = th0 + t_hh - p.pad, win = tw0 + t_ww - p.pad;
         const bool row_ok = live && (is_core || is_edge) && hin >= 0 && hin < p.H;
         const float* xb = p.x + (long)b * p.C * plane;
-        const int c0 = ld_chunk * IG_CC + t_h8 * 8;
+        const int c0 = ld_chunk * IG_CC + t_q4 * 4;
         if (VEC4) {
             const bool ok = row_ok && win >= 0 && win < p.W;       // W % 4 == 0: the quad is all in or all out
             int n = p.C - c0;
-            n = n < 0 ? 0 : (n > 8 ? 8 : n);
+            n = n < 0 ? 0 : (n > 4 ? 4 : n);
             n = ok ? n : 0;
             nvalid = n;
             // lanes without work read the first quad of the image; channels past n repeat the last valid one
             const long first = ((long)c0 * plane + (long)hin * p.W + (win & ~3)) & -(long)(n > 0);
             const float* src = xb + first;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
+            for (int e = 0; e < 4; e++) {
                 dst[e] = *reinterpret_cast<const floatx4*>(src);
                 src += plane & -(long)(e + 1 < n);
             }
         } else {
-            nvalid = 8;
+            nvalid = 4;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
+            for (int e = 0; e < 4; e++) {
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
@@ -708,23 +730,26 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
             }
         }
         ld_it++;
-        if (++ld_chunk == p.n_chunks) { ld_chunk = 0; ld_patch += gridDim.x; }
+        if (++ld_chunk == n_items) { ld_chunk = 0; ld_patch += gridDim.x; }
     };
-    auto store_halo = [&](const floatx4 (&src)[8], const int nvalid) {
+    auto store_halo = [&](const floatx4 (&src)[4], const int nvalid) {
+        // Every lane takes delivery of the set here, also lanes without a task: a request left
+        // pending on some path would force a full drain before the registers are reused.
+#pragma unroll
+        for (int e = 0; e < 4; e++) asm volatile("" ::"v"(src[e]));
         if (!(is_core || is_edge)) return;
         if (is_core) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                half8_t h;
+                half4_t h;
 #pragma unroll
-                for (int e = 0; e < 8; e++) h[e] = e < nvalid ? (_Float16)src[e][q] : (_Float16)0.f;
-                const int ww = t_ww + q;
-                *reinterpret_cast<half8_t*>(lds_h + (t_hh * G::WW + ww) * 32 + ((t_h8 ^ ((ww >> 3) & 1)) << 4)) = h;
+                for (int e = 0; e < 4; e++) h[e] = e < nvalid ? (_Float16)src[e][q] : (_Float16)0.f;
+                *reinterpret_cast<half4_t*>(halo_slot(t_hh, t_ww + q)) = h;
             }
         } else {
-            half8_t h;
+            half4_t h;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
+            for (int e = 0; e < 4; e++) {
                 float f = src[e][0];
                 if (VEC4) {
                     f = t_comp == 1 ? src[e][1] : f;
@@ -733,29 +758,33 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
                 }
                 h[e] = e < nvalid ? (_Float16)f : (_Float16)0.f;
             }
-            *reinterpret_cast<half8_t*>(lds_h + (t_hh * G::WW + t_ww) * 32 + ((t_h8 ^ ((t_ww >> 3) & 1)) << 4)) = h;
+            *reinterpret_cast<half4_t*>(halo_slot(t_hh, t_ww)) = h;
         }
     };
 
+    // A per-channel bias (or zero) is the starting value of every accumulator; the 128 values of the
+    // channel tile sit in LDS behind the halo and are read back at the start of each patch.
     floatx16 acc[2][FP];
-    auto zero_acc = [&]() {
+    auto init_acc = [&]() {
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int j = 0; j < FP; j++)
+            for (int g = 0; g < 4; g++) {
+                const floatx4 bq = *reinterpret_cast<const floatx4*>(lds_bias + wn * 64 + i * 32 + g * 8 + lh * 4);
 #pragma unroll
-                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+                for (int j = 0; j < FP; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) acc[i][j][g * 4 + q] = bq[q];
+            }
     };
-    zero_acc();
 
-    // One fragment set per kw. The LDS reads of a tap are issued before the MFMAs of the tap before
-    // it (the first tap of a filter row is requested during the last tap of the row above), so the
+    // Two fragment sets: the LDS reads of tap t + 1 are issued before the MFMAs of tap t, so the
     // matrix pipe does not wait for LDS latency at every tap.
     auto compute = [&](int chunk) {
         const char* wbase = lds_w + chunk * W_CHUNK + (wn * 64 + li) * W_PITCH + ((lh ^ ((li >> 3) & 1)) << 4);
-        half8_t wf[KW][2], pf[KW][FP];
-        auto read_frags = [&](int kh, int kw, half8_t (&w)[2], half8_t (&x)[FP]) {
-            const int tap = kh * KW + kw;
+        half8_t wf[2][2], pf[2][FP];
+        auto read_frags = [&](const int tap, half8_t (&w)[2], half8_t (&x)[FP]) {
+            const int kh = tap / KW, kw = tap % KW;
 #pragma unroll
             for (int i = 0; i < 2; i++)
                 w[i] = *reinterpret_cast<const half8_t*>(wbase + i * 32 * W_PITCH + tap * 32);
@@ -767,125 +796,109 @@ __global__ __launch_bounds__(256) void conv_igemm_resident_kernel(const IgemmArg
                                                           ((lh ^ ((col >> 3) & 1)) << 4));
             }
         };
-        read_frags(0, 0, wf[0], pf[0]);
-#pragma unroll 1
-        for (int kh = 0; kh < KH; kh++) {
+        read_frags(0, wf[0], pf[0]);
 #pragma unroll
-            for (int kw = 0; kw < KW; kw++) {
-                if (kw + 1 < KW) read_frags(kh, kw + 1, wf[kw + 1], pf[kw + 1]);
-                else if (kh + 1 < KH) read_frags(kh + 1, 0, wf[0], pf[0]);
-                __builtin_amdgcn_sched_barrier(0);               // requests stay ahead of the MFMAs below
+        for (int tap = 0; tap < G::TAPS; tap++) {
+            if (tap + 1 < G::TAPS) read_frags(tap + 1, wf[(tap + 1) & 1], pf[(tap + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);                   // requests stay ahead of the MFMAs below
 #pragma unroll
-                for (int i = 0; i < 2; i++)
+            for (int i = 0; i < 2; i++)
 #pragma unroll
-                    for (int j = 0; j < FP; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[kw][i], pf[kw][j], acc[i][j], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+                for (int j = 0; j < FP; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[tap & 1][i], pf[tap & 1][j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    // Per-channel bias (pixel stride 0) is the same for every patch: fetch it once.
-    const int o_base = o_tile * BN + wn * 64 + lh * 4;
-    const bool bias_per_channel = !PIX_BIAS && p.bias;
-    float bch[2][16];
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int rr = 0; rr < 16; rr++) {
-            const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
-            bch[i][rr] = 0.f;
-            if (bias_per_channel) bch[i][rr] = p.bias[(long)(o < p.O ? o : p.O - 1) * p.bias_sc];   // uniform branch
-        }
+    const int o_wave = o_tile * BN + wn * 64;                    // uniform; lane channel = o_wave + lh*4 + i*32 + ...
+    const bool o_full = o_tile * BN + BN <= p.O;                 // uniform: whole channel tile exists
+    const long hw_out = (long)p.H_out * p.W_out;
 
-    auto epilogue = [&](int patch) {
+    // Write unit (j, i) of the finished patch: pixel block j x 32 channels, 16 stores per lane.
+    // bias (if per pixel) + activation + NCHW store, lanes = adjacent pixels. The address of a store
+    // is a wave-uniform channel plane (scalar registers, stepped with scalar adds) plus one per-lane
+    // byte offset shared by the 16 stores: pixel, and 4 planes up for the upper half-wave.
+    // A patch that lies wholly inside the output takes the unpredicated path.
+    auto flush_unit = [&](const int j, const int i, const int patch) {
         const int b = patch / patches_per_image, r = patch % patches_per_image;
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
-        float* yb = p.y + (long)b * p.O * p.H_out * p.W_out;
-        const long hw_out = (long)p.H_out * p.W_out;
-        // whole patch and whole channel tile inside the output: no per-element predicates (uniform test)
-        const bool inside = th0 + G::TH <= p.H_out && tw0 + TW <= p.W_out && o_tile * BN + BN <= p.O;
+        const int blk = wm * FP + j;
+        const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
+        const bool inside = o_full && th0 + G::TH <= p.H_out && tw0 + TW <= p.W_out;   // uniform
+        const bool pix_ok = inside || (ho < p.H_out && wo < p.W_out);
+        const long pix = pix_ok ? (long)ho * p.W_out + wo : 0;
+        const unsigned lane_bytes = (unsigned)((pix + (long)lh * 4 * hw_out) * 4);
+        char* pl = reinterpret_cast<char*>(p.y + ((long)b * p.O + o_wave + i * 32) * hw_out);
+        const int o_lane = o_wave + i * 32 + lh * 4;
+        float bv[16];
+        if (PIX_BIAS) {                                          // one batch of requests per unit
 #pragma unroll
-        for (int j = 0; j < FP; j++) {
-            const int blk = wm * FP + j;
-            const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
-            const bool pix_ok = inside || (ho < p.H_out && wo < p.W_out);
-            const long pix = pix_ok ? (long)ho * p.W_out + wo : 0;
-            float bv[2][16];
-            if (PIX_BIAS) {                                      // per-pixel bias: one batch of requests per row
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-#pragma unroll
-                    for (int rr = 0; rr < 16; rr++) {
-                        const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
-                        bv[i][rr] = p.bias[pix * p.bias_sp + (long)((inside || o < p.O) ? o : 0) * p.bias_sc];
-                    }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-#pragma unroll
-                    for (int rr = 0; rr < 16; rr++) bv[i][rr] = bch[i][rr];
+            for (int rr = 0; rr < 16; rr++) {
+                const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
+                bv[rr] = p.bias[pix * p.bias_sp + (long)((o_full || o < p.O) ? o : 0) * p.bias_sc];
             }
-            float* dst = yb + pix;
-            if (inside) {
+        }
+        auto finished = [&](const int rr) {
+            float v = acc[i][j][rr];
+            if (PIX_BIAS) v += bv[rr];                           // a per-channel bias is already in the accumulator
+            return fmaxf(v, p.relu ? 0.f : v);                  // NaN -> 0 under ReLU, like x > 0 ? x : 0
+        };
+        // The step between channel planes is opaque so that the plane addresses are not precomputed
+        // and kept in registers across the whole kernel.
+        int step_lo = __builtin_amdgcn_readfirstlane((int)(hw_out * 4)),
+            step_hi = __builtin_amdgcn_readfirstlane((int)((hw_out * 4) >> 32));
+        asm volatile("" : "+s"(step_lo), "+s"(step_hi));
+        const long step1 = ((long)step_hi << 32) | (unsigned)step_lo, step5 = step1 * 5;
+        if (inside) {
 #pragma unroll
-                for (int i = 0; i < 2; i++)
+            for (int rr = 0; rr < 16; rr++) {
+                *reinterpret_cast<float*>(pl + lane_bytes) = finished(rr);
+                pl += (rr & 3) == 3 ? step5 : step1;             // channels +1 +1 +1 +5: 0..3, 8..11, 16..19, 24..27
+            }
+        } else {
 #pragma unroll
-                    for (int rr = 0; rr < 16; rr++) {
-                        const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
-                        float v = acc[i][j][rr] + bv[i][rr];
-                        if (p.relu) v = v > 0.f ? v : 0.f;
-                        dst[(long)o * hw_out] = v;
-                    }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-#pragma unroll
-                    for (int rr = 0; rr < 16; rr++) {
-                        const int o = o_base + i * 32 + (rr >> 2) * 8 + (rr & 3);
-                        float v = acc[i][j][rr] + bv[i][rr];
-                        if (p.relu) v = v > 0.f ? v : 0.f;
-                        if (pix_ok && o < p.O) dst[(long)o * hw_out] = v;
-                    }
+            for (int rr = 0; rr < 16; rr++) {
+                const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
+                const float v = finished(rr);
+                if (pix_ok && o < p.O) *reinterpret_cast<float*>(pl + lane_bytes) = v;
+                pl += (rr & 3) == 3 ? step5 : step1;
             }
         }
     };
 
     // LDS-only barrier: waits for this wave's LDS traffic, not for the global requests in flight.
     auto lds_barrier = []() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-    // One work item. The register set is a compile-time choice (items alternate between the two
-    // sets), so a set is never copied and its requests stay in flight across a whole item.
-    auto item = [&](floatx4 (&r)[8], int& n, int chunk) {
+    // One work item. The register set r (parity of the item index) is a compile-time choice, so
+    // nothing is copied and a set's requests stay in flight across a whole item.
+    auto item = [&](floatx4 (&r)[4], int& n, const int c) {
         store_halo(r, n);                                        // registers -> LDS (waits for this set only)
         lds_barrier();
-        load_item(r, n);                                         // request the item two ahead into the same set
-        compute(chunk);
+        if (early) {
+            load_item(r, n);                                     // request the item two ahead into the same set
+            if (c < p.n_chunks) compute(c);
+        } else {
+            if (c < p.n_chunks) compute(c);
+            load_item(r, n);
+        }
         lds_barrier();                                           // halo may be overwritten
     };
 
     load_item(raw[0], nv[0]);
     load_item(raw[1], nv[1]);
+    if (tid < BN) lds_bias[tid] = my_bias;
     __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);                 // vmcnt(0): resident weights landed
+    lds_barrier();
     for (int pi = 0; pi < my_patches; pi++) {
-        zero_acc();
-        int chunk = 0;
-        for (; chunk + 1 < p.n_chunks; chunk += 2) {
-            item(raw[0], nv[0], chunk);
-            item(raw[1], nv[1], chunk + 1);
+        init_acc();
+        for (int c = 0; c < n_items; c += 2) {
+            item(raw[0], nv[0], c);
+            item(raw[1], nv[1], c + 1);
         }
-        if (chunk < p.n_chunks) {                                // odd chunk count: the sets trade places
-            item(raw[0], nv[0], chunk);
+        const int patch = blockIdx.x + pi * gridDim.x;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const floatx4 t = raw[0][e];
-                raw[0][e] = raw[1][e];
-                raw[1][e] = t;
-            }
-            const int t = nv[0];
-            nv[0] = nv[1];
-            nv[1] = t;
-        }
-        epilogue(blockIdx.x + pi * gridDim.x);
+        for (int j = 0; j < FP; j++)
+#pragma unroll
+            for (int i = 0; i < 2; i++) flush_unit(j, i, patch);
     }
 }
 
@@ -905,7 +918,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     // Resident-weight route: shared weights whose fp16 image (unpadded) plus one halo fit in LDS.
     if constexpr (BN == 128) {
         constexpr size_t W_CHUNK_R = 128 * (size_t)G::TAPS * 32;
-        const size_t lds_need = (size_t)n_chunks * W_CHUNK_R + G::HALO_BYTES;
+        const size_t lds_need = (size_t)n_chunks * W_CHUNK_R + G::HALO_BYTES + 128 * sizeof(float);   // + bias
         static const char* res_env = getenv("NZHIP_CONV_RESIDENT");
         const bool allow = res_env ? atoi(res_env) != 0 : true;
         if (allow && w_batch == 1 && lds_need <= 160 * 1024 - 512) {
@@ -945,7 +958,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                 int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
                 if ((long)per_tile > n_patches) per_tile = (int)n_patches;
                 dim3 grid((unsigned)per_tile, (unsigned)n_otiles, 1);
-                hipLaunchKernelGGL(kres, grid, dim3(256), lds_need, s, a, (int)n_patches);
+                hipLaunchKernelGGL(kres, grid, dim3(512), lds_need, s, a, (int)n_patches);
                 hipError_t e = hipGetLastError();
                 if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm_resident kernel launch");
             }
