@@ -690,26 +690,32 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     int nv[2] = {0, 0};
     const int t_comp = (t_ww - p.pad) & 3;
     int ld_patch = blockIdx.x, ld_chunk = 0, ld_it = 0;
+    const float* ld_src = p.x;                                   // this thread's pixel, channel t_q4*4, current patch
+    bool ld_ok = false;                                          // the pixel (VEC4: its quad) is inside the image
+    int ld_hin = 0, ld_win = 0;
     auto load_item = [&](floatx4 (&dst)[4], int& nvalid) {
         // Past the last item the requests are still issued (to the first quad of x, results unused):
         // a fixed number of requests per item lets every wait name exactly the set it needs.
-        const bool live = ld_it < total;                         // uniform
-        const int patch = live ? ld_patch : (int)blockIdx.x;
-        const int b = patch / patches_per_image, r = patch % patches_per_image;
-        const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
-        const int hin = th0 + t_hh - p.pad, win = tw0 + t_ww - p.pad;
-        const bool row_ok = live && (is_core || is_edge) && hin >= 0 && hin < p.H;
-        const float* xb = p.x + (long)b * p.C * plane;
+        if (ld_chunk == 0) {                                     // new patch: redo the geometry (uniform branch)
+            const bool live = ld_it < total;
+            const int patch = live ? ld_patch : (int)blockIdx.x;
+            const int b = patch / patches_per_image, r = patch % patches_per_image;
+            const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
+            ld_hin = th0 + t_hh - p.pad;
+            ld_win = tw0 + t_ww - p.pad;
+            const bool row_ok = live && (is_core || is_edge) && ld_hin >= 0 && ld_hin < p.H;
+            ld_ok = row_ok && (!VEC4 || (ld_win >= 0 && ld_win < p.W));   // W % 4 == 0: a quad is all in or all out
+            ld_src = p.x + ((long)b * p.C + t_q4 * 4) * plane +
+                     (ld_ok ? (long)ld_hin * p.W + (VEC4 ? (ld_win & ~3) : ld_win) : 0);
+        }
         const int c0 = ld_chunk * IG_CC + t_q4 * 4;
         if (VEC4) {
-            const bool ok = row_ok && win >= 0 && win < p.W;       // W % 4 == 0: the quad is all in or all out
             int n = p.C - c0;
             n = n < 0 ? 0 : (n > 4 ? 4 : n);
-            n = ok ? n : 0;
+            n = ld_ok ? n : 0;
             nvalid = n;
-            // lanes without work read the first quad of the image; channels past n repeat the last valid one
-            const long first = ((long)c0 * plane + (long)hin * p.W + (win & ~3)) & -(long)(n > 0);
-            const float* src = xb + first;
+            // lanes without work read the first quad of x; channels past n repeat the last valid one
+            const float* src = n > 0 ? ld_src + (long)ld_chunk * IG_CC * plane : p.x;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 dst[e] = *reinterpret_cast<const floatx4*>(src);
@@ -722,8 +728,8 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const bool ok = row_ok && (c0 + e < p.C) && win + q >= 0 && win + q < p.W && (is_core || q == 0);
-                    const float f = xb[ok ? (long)(c0 + e) * plane + (long)hin * p.W + win + q : 0];
+                    const bool ok = ld_ok && (c0 + e < p.C) && ld_win + q >= 0 && ld_win + q < p.W && (is_core || q == 0);
+                    const float f = *(ok ? ld_src + ((long)ld_chunk * IG_CC + e) * plane + q : p.x);
                     v[q] = ok ? f : 0.f;
                 }
                 dst[e] = v;
@@ -873,13 +879,10 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     auto item = [&](floatx4 (&r)[4], int& n, const int c) {
         store_halo(r, n);                                        // registers -> LDS (waits for this set only)
         lds_barrier();
-        if (early) {
-            load_item(r, n);                                     // request the item two ahead into the same set
-            if (c < p.n_chunks) compute(c);
-        } else {
-            if (c < p.n_chunks) compute(c);
-            load_item(r, n);
-        }
+        // the requests sit outside the branches: every path issues the same number of them
+        if (!early && c < p.n_chunks) compute(c);
+        load_item(r, n);                                         // request the item two ahead into the same set
+        if (early && c < p.n_chunks) compute(c);
         lds_barrier();                                           // halo may be overwritten
     };
 
@@ -944,17 +947,10 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                                       : conv_igemm_resident_kernel<KH, KW, TW, true, false>)
                               : (pixb ? conv_igemm_resident_kernel<KH, KW, TW, false, true>
                                       : conv_igemm_resident_kernel<KH, KW, TW, false, false>);
+            if (rc == NZHIP_OK)
+                rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kres), (int)lds_need, "hipFuncSetAttribute(conv_igemm_resident)");
             if (rc == NZHIP_OK) {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kres),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_need);
-                if (e != hipSuccess) rc = set_hip_error(e, "hipFuncSetAttribute(conv_igemm_resident)");
-            }
-            if (rc == NZHIP_OK) {
-                int cus = 256;
-                hipDeviceProp_t prop;
-                int dev = 0;
-                if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
-                    cus = prop.multiProcessorCount;
+                const int cus = device_cu_count();
                 int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
                 if ((long)per_tile > n_patches) per_tile = (int)n_patches;
                 dim3 grid((unsigned)per_tile, (unsigned)n_otiles, 1);
@@ -1003,16 +999,8 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         a.relu = act == NZHIP_ACT_RELU;
         const bool vec4 = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
         auto kfn = vec4 ? conv_igemm_kernel<KH, KW, TW, BN, true> : conv_igemm_kernel<KH, KW, TW, BN, false>;
-        static bool attr_set = false;
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(conv_igemm_kernel<KH, KW, TW, BN, true>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
-            if (e == hipSuccess)
-                e = hipFuncSetAttribute(reinterpret_cast<const void*>(conv_igemm_kernel<KH, KW, TW, BN, false>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
-            if (e != hipSuccess) rc = set_hip_error(e, "hipFuncSetAttribute(conv_igemm)");
-            attr_set = true;
-        }
+        if (rc == NZHIP_OK)
+            rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), G::LDS_BYTES, "hipFuncSetAttribute(conv_igemm)");
         if (rc == NZHIP_OK) {
             dim3 grid((unsigned)(a.tiles_w * a.tiles_h), (unsigned)n_otiles, (unsigned)N);
             hipLaunchKernelGGL(kfn, grid, dim3(256), G::LDS_BYTES, s, a);

@@ -336,13 +336,9 @@ static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool 
 #define NZHIP_LAUNCH(AT, BT, V, F)                                                                       \
     do {                                                                                                 \
         auto kfn = gemm_f16mfma_kernel<BM, BN, BK, WM, WN, AT, BT, V, F>;                                \
-        static bool attr_set = false;                                                                    \
-        if (!attr_set) {                                                                                 \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),                       \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes); \
-            if (e != hipSuccess) return set_hip_error(e, "hipFuncSetAttribute(gemm)");                   \
-            attr_set = true;                                                                             \
-        }                                                                                                \
+        if (int lrc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes,             \
+                                         "hipFuncSetAttribute(gemm)"))                                   \
+            return lrc;                                                                                  \
         hipLaunchKernelGGL(kfn, grid, block, lds_bytes, s, a);                                           \
     } while (0)
     if (full) {

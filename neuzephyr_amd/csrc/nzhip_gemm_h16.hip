@@ -394,13 +394,8 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
         a.group_m = 4;
         constexpr size_t lds_bytes = (size_t)NSTAGE * (BM + BN) * 64;
         auto kfn = gemm_h16_kernel<BM, BN, 2, 2, NSTAGE>;
-        static bool attr_set = false;
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kfn),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            if (e != hipSuccess) rc = set_hip_error(e, "hipFuncSetAttribute(gemm_h16)");
-            attr_set = true;
-        }
+        if (rc == NZHIP_OK)
+            rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(gemm_h16)");
         if (rc == NZHIP_OK) {
             dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(d.batch_n * d.batch_c));
             hipLaunchKernelGGL(kfn, grid, dim3(256), lds_bytes, s, a);

@@ -26,6 +26,13 @@ bool gemm_skinny_applicable(const nzhip_gemm_desc& d);
 int workspace_alloc(void** ptr, size_t bytes, hipStream_t stream);
 int workspace_free(void* ptr, hipStream_t stream);
 
+// Compute units of the current device (queried once per device, then cached).
+int device_cu_count();
+
+// Raise a kernel's dynamic LDS limit to at least `bytes` on the current device. The limit reached is
+// remembered per (device, kernel), so repeated launches cost a table lookup, not a driver call.
+int ensure_dynamic_lds(const void* kernel, int bytes, const char* what);
+
 }  // namespace nzhip
 
 #endif

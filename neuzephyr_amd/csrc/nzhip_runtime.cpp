@@ -9,8 +9,11 @@
 // in nzhip_sync_ptr / nzhip_sync_all / nzhip_memcpy_d2h / nzhip_free.
 #include <cstdarg>
 #include <cstdio>
+#include <atomic>
 #include <cstring>
+#include <map>
 #include <mutex>
+#include <utility>
 
 #include "nz_pool_allocator.hpp"
 #include "nzhip_internal.h"
@@ -84,6 +87,34 @@ int workspace_free(void* ptr, hipStream_t s) {
     return Runtime::instance().pool().free_async(ptr, reinterpret_cast<uintptr_t>(s)) == 0
                ? NZHIP_OK
                : set_error(NZHIP_E_INVALID, "workspace_free: unknown pointer");
+}
+
+int device_cu_count() {
+    static std::atomic<int> cached[64];                          // 0 = not queried yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int cus = cached[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        hipDeviceProp_t prop;
+        cus = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        cached[dev].store(cus, std::memory_order_relaxed);
+    }
+    return cus;
+}
+
+int ensure_dynamic_lds(const void* kernel, int bytes, const char* what) {
+    static std::mutex mu;
+    static std::map<std::pair<int, const void*>, int> reached;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_hip_error(e, "hipGetDevice");
+    std::lock_guard<std::mutex> lock(mu);
+    int& cur = reached[{dev, kernel}];
+    if (cur >= bytes) return NZHIP_OK;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return set_hip_error(e, what);
+    cur = bytes;
+    return NZHIP_OK;
 }
 
 }  // namespace nzhip
