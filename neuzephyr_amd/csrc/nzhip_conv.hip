@@ -612,11 +612,11 @@ __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float1
 //
 // Eight waves, two per SIMD. Wave (wm, wn) owns 64 pixels (two 32-pixel blocks) x 64 channels of
 // the 256 x 128 patch tile. A work item is one 16-channel chunk of one patch:
-//     store_halo (registers -> fp16 LDS)  | barrier |  MFMAs  +  "other"  | barrier
-// where "other" = request the halo two items ahead. The two waves of a SIMD run MFMAs and "other"
-// in opposite order, so the matrix pipe of the SIMD is fed by one wave while its partner issues
-// memory and address instructions. After the last chunk of a patch every wave writes its 64 x 64
-// results (bias already in the accumulator, activation on the way out).
+//     store_halo (registers -> fp16 LDS)  | barrier |  MFMAs, with the loads of the halo two items
+//     ahead issued one behind every other filter tap  | barrier
+// A wave held up at the memory pipe leaves the matrix pipe to its partner on the SIMD. After the
+// last chunk of a patch every wave writes its 64 x 64 results (bias already in the accumulator,
+// activation on the way out).
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
 template <int KH, int KW, int TW, bool VEC4, bool PIX_BIAS>
@@ -633,7 +633,6 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
-    const bool early = wave < NW / 2;                           // waves w and w + 4 share a SIMD
     const int li = lane & 31, lh = lane >> 5;
     const int o_tile = blockIdx.y;
     const int patches_per_image = p.tiles_w * p.tiles_h;
@@ -693,9 +692,13 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     const float* ld_src = p.x;                                   // this thread's pixel, channel t_q4*4, current patch
     bool ld_ok = false;                                          // the pixel (VEC4: its quad) is inside the image
     int ld_hin = 0, ld_win = 0;
-    auto load_item = [&](floatx4 (&dst)[4], int& nvalid) {
-        // Past the last item the requests are still issued (to the first quad of x, results unused):
-        // a fixed number of requests per item lets every wait name exactly the set it needs.
+    // A request is issued in three steps so that its four loads can be spread between the MFMAs of
+    // the item in progress: load_begin (addresses), load_one x 4, load_end (advance to the next item).
+    // Past the last item the requests are still issued (to the first quad of x, results unused):
+    // a fixed number of requests per item lets every wait name exactly the set it needs.
+    const float* ld_cur = p.x;
+    int ld_n = 0, ld_c0 = 0;
+    auto load_begin = [&](int& nvalid) {
         if (ld_chunk == 0) {                                     // new patch: redo the geometry (uniform branch)
             const bool live = ld_it < total;
             const int patch = live ? ld_patch : (int)blockIdx.x;
@@ -708,35 +711,38 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
             ld_src = p.x + ((long)b * p.C + t_q4 * 4) * plane +
                      (ld_ok ? (long)ld_hin * p.W + (VEC4 ? (ld_win & ~3) : ld_win) : 0);
         }
-        const int c0 = ld_chunk * IG_CC + t_q4 * 4;
+        ld_c0 = ld_chunk * IG_CC + t_q4 * 4;
+        int n = p.C - ld_c0;
+        n = n < 0 ? 0 : (n > 4 ? 4 : n);
+        ld_n = ld_ok ? n : 0;
+        nvalid = VEC4 ? ld_n : 4;
+        // lanes without work read the first quad of x; channels past n repeat the last valid one
+        ld_cur = ld_n > 0 ? ld_src + (long)ld_chunk * IG_CC * plane : p.x;
+    };
+    auto load_one = [&](floatx4 (&dst)[4], const int e) {
         if (VEC4) {
-            int n = p.C - c0;
-            n = n < 0 ? 0 : (n > 4 ? 4 : n);
-            n = ld_ok ? n : 0;
-            nvalid = n;
-            // lanes without work read the first quad of x; channels past n repeat the last valid one
-            const float* src = n > 0 ? ld_src + (long)ld_chunk * IG_CC * plane : p.x;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                dst[e] = *reinterpret_cast<const floatx4*>(src);
-                src += plane & -(long)(e + 1 < n);
-            }
+            dst[e] = *reinterpret_cast<const floatx4*>(ld_cur);
+            ld_cur += plane & -(long)(e + 1 < ld_n);
         } else {
-            nvalid = 4;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                floatx4 v = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const bool ok = ld_ok && (c0 + e < p.C) && ld_win + q >= 0 && ld_win + q < p.W && (is_core || q == 0);
-                    const float f = *(ok ? ld_src + ((long)ld_chunk * IG_CC + e) * plane + q : p.x);
-                    v[q] = ok ? f : 0.f;
-                }
-                dst[e] = v;
+            for (int q = 0; q < 4; q++) {
+                const bool ok = e < ld_n && ld_win + q >= 0 && ld_win + q < p.W && (is_core || q == 0);
+                const float f = *(ok ? ld_cur + (long)e * plane + q : p.x);
+                v[q] = ok ? f : 0.f;
             }
+            dst[e] = v;
         }
+    };
+    auto load_end = [&]() {
         ld_it++;
         if (++ld_chunk == n_items) { ld_chunk = 0; ld_patch += gridDim.x; }
+    };
+    auto load_item = [&](floatx4 (&dst)[4], int& nvalid) {
+        load_begin(nvalid);
+#pragma unroll
+        for (int e = 0; e < 4; e++) load_one(dst, e);
+        load_end();
     };
     auto store_halo = [&](const floatx4 (&src)[4], const int nvalid) {
         // Every lane takes delivery of the set here, also lanes without a task: a request left
@@ -786,7 +792,10 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
 
     // Two fragment sets: the LDS reads of tap t + 1 are issued before the MFMAs of tap t, so the
     // matrix pipe does not wait for LDS latency at every tap.
-    auto compute = [&](int chunk) {
+    // after_tap(tap) runs behind the MFMAs of each tap (used to spread the next halo request). It
+    // sits outside the branch on `live`, so an empty item (odd chunk count) issues the same requests
+    // as a full one without touching LDS or the matrix pipe.
+    auto compute = [&](int chunk, const bool live, auto after_tap) {
         const char* wbase = lds_w + chunk * W_CHUNK + (wn * 64 + li) * W_PITCH + ((lh ^ ((li >> 3) & 1)) << 4);
         half8_t wf[2][2], pf[2][FP];
         auto read_frags = [&](const int tap, half8_t (&w)[2], half8_t (&x)[FP]) {
@@ -802,16 +811,19 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
                                                           ((lh ^ ((col >> 3) & 1)) << 4));
             }
         };
-        read_frags(0, wf[0], pf[0]);
+        if (live) read_frags(0, wf[0], pf[0]);
 #pragma unroll
         for (int tap = 0; tap < G::TAPS; tap++) {
-            if (tap + 1 < G::TAPS) read_frags(tap + 1, wf[(tap + 1) & 1], pf[(tap + 1) & 1]);
-            __builtin_amdgcn_sched_barrier(0);                   // requests stay ahead of the MFMAs below
+            if (live) {
+                if (tap + 1 < G::TAPS) read_frags(tap + 1, wf[(tap + 1) & 1], pf[(tap + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);               // requests stay ahead of the MFMAs below
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+                for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < FP; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[tap & 1][i], pf[tap & 1][j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < FP; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[tap & 1][i], pf[tap & 1][j], acc[i][j], 0, 0, 0);
+            }
+            after_tap(tap);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -879,10 +891,15 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     auto item = [&](floatx4 (&r)[4], int& n, const int c) {
         store_halo(r, n);                                        // registers -> LDS (waits for this set only)
         lds_barrier();
-        // the requests sit outside the branches: every path issues the same number of them
-        if (!early && c < p.n_chunks) compute(c);
-        load_item(r, n);                                         // request the item two ahead into the same set
-        if (early && c < p.n_chunks) compute(c);
+        // Request the item two ahead into the same set: one load behind every other tap, so a wave
+        // held up at the memory pipe leaves the matrix pipe to its partner on the SIMD.
+        load_begin(n);
+        compute(c, c < p.n_chunks, [&](const int tap) {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (tap == (2 * e + 1 < G::TAPS ? 2 * e + 1 : G::TAPS - 1)) load_one(r, e);
+        });
+        load_end();
         lds_barrier();                                           // halo may be overwritten
     };
 
