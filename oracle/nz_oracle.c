@@ -301,6 +301,101 @@ void nzo_relu(float* out, const float* in, size_t n) {
 }
 
 /* ------------------------------------------------------------------------- */
+/* Backward of the path.                                                      */
+/* ------------------------------------------------------------------------- */
+/* src/OperationKernels.cu:1028-1144: same M/N/K and offsets as the forward driver, the batch
+ * runs over max(A,B) and a C dimension of 1 collects every member (CuttingAndCompress). */
+void nzo_gemm_backward(const float* A, const float* B, float* C, const size_t shapeA[4],
+                       const size_t shapeB[4], const size_t shapeC[4]) {
+    const size_t M = shapeA[2], N = shapeB[3], K = shapeA[3];
+    const size_t bn = shapeA[0] > shapeB[0] ? shapeA[0] : shapeB[0];
+    const size_t bc = shapeA[1] > shapeB[1] ? shapeA[1] : shapeB[1];
+    float* tmp = (float*)malloc((M * N > 0 ? M * N : 1) * sizeof(float));
+    for (size_t i = 0; i < bn; i++) {
+        for (size_t j = 0; j < bc; j++) {
+            const size_t oa = i * (shapeA[0] > 1 ? stride0(shapeA) : 0) + j * (shapeA[1] > 1 ? stride1(shapeA) : 0);
+            const size_t ob = i * (shapeB[0] > 1 ? stride0(shapeB) : 0) + j * (shapeB[1] > 1 ? stride1(shapeB) : 0);
+            const size_t oc = i * (shapeC[0] > 1 ? stride0(shapeC) : 0) + j * (shapeC[1] > 1 ? stride1(shapeC) : 0);
+            nzo_gemm_f16in_f32acc(A + oa, B + ob, tmp, M, N, K, K, N, N, 0);
+            for (size_t e = 0; e < M * N; e++) C[oc + e] += tmp[e];      /* :873-883 */
+        }
+    }
+    free(tmp);
+}
+
+static void transpose_batched(float* dst, const float* src, const size_t shape[4]) {   /* :125-145 */
+    const size_t R = shape[2], Cn = shape[3], nb = shape[0] * shape[1];
+    for (size_t b = 0; b < nb; b++)
+        for (size_t r = 0; r < R; r++)
+            for (size_t c = 0; c < Cn; c++) dst[b * R * Cn + c * R + r] = src[b * R * Cn + r * Cn + c];
+}
+
+void nzo_matmul_backward(float* dA, float* dB, const float* A, const float* B, const float* dC,
+                         const size_t shapeA[4], const size_t shapeB[4], const size_t shapeC[4]) {
+    if (dA) {                                                          /* Nodes.cu:171-175 */
+        const size_t nB = shapeB[0] * shapeB[1] * shapeB[2] * shapeB[3];
+        float* bt = (float*)malloc((nB ? nB : 1) * sizeof(float));
+        const size_t shapeBT[4] = {shapeB[0], shapeB[1], shapeB[3], shapeB[2]};
+        transpose_batched(bt, B, shapeB);
+        nzo_gemm_backward(dC, bt, dA, shapeC, shapeBT, shapeA);
+        free(bt);
+    }
+    if (dB) {                                                          /* Nodes.cu:177-181 */
+        const size_t nA = shapeA[0] * shapeA[1] * shapeA[2] * shapeA[3];
+        float* at = (float*)malloc((nA ? nA : 1) * sizeof(float));
+        const size_t shapeAT[4] = {shapeA[0], shapeA[1], shapeA[3], shapeA[2]};
+        transpose_batched(at, A, shapeA);
+        nzo_gemm_backward(at, dC, dB, shapeAT, shapeC, shapeB);
+        free(at);
+    }
+}
+
+void nzo_relu_backward(float* dx, const float* x, const float* dy, size_t n) {
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; i++) dx[i] = x[i] > 0 ? dy[i] : 0;
+}
+
+void nzo_add_backward(float* din, const float* dout, const size_t shapeIn[4], const size_t shapeOut[4]) {
+    const size_t n = shapeOut[2] * shapeOut[3];
+    if (shapeIn[0] == shapeOut[0] && shapeIn[1] == shapeOut[1] && shapeIn[2] == shapeOut[2] &&
+        shapeIn[3] == shapeOut[3]) {                                   /* Nodes.cu:101-105: memcpy */
+        memcpy(din, dout, shapeOut[0] * shapeOut[1] * n * sizeof(float));
+        return;
+    }
+    for (size_t i = 0; i < shapeOut[0]; i++)                           /* Nodes.cu:107-121 */
+        for (size_t j = 0; j < shapeOut[1]; j++) {
+            const float* src = dout + i * stride0(shapeOut) + j * stride1(shapeOut);
+            float* dst = din + i * (shapeIn[0] > 1 ? stride0(shapeIn) : 0) + j * (shapeIn[1] > 1 ? stride1(shapeIn) : 0);
+            for (size_t idx = 0; idx < n; idx++) dst[idx] += src[idx];
+        }
+}
+
+void nzo_im2col_backward(float* dx, const float* dcol, size_t H_out, size_t W_out, size_t C, size_t K_h,
+                         size_t K_w, size_t stride, size_t pad, size_t H_in, size_t W_in, size_t batch) {
+    const size_t per = H_out * W_out * C * K_h * K_w;
+    for (size_t idx = 0; idx < per * batch; idx++) {                   /* :1341-1354, index by index */
+        const size_t fixedIdx = idx % per, currentBatch = idx / per;
+        const size_t k = fixedIdx / (C * K_h * K_w), m = fixedIdx % (C * K_h * K_w);
+        const size_t c = m / (K_h * K_w);
+        const long long h = (long long)((k / W_out) * stride) - (long long)pad + (long long)((m % (K_h * K_w)) / K_w);
+        const long long w = (long long)((k % W_out) * stride) - (long long)pad + (long long)(m % K_w);
+        if (h >= 0 && h < (long long)H_in && w >= 0 && w < (long long)W_in)
+            dx[currentBatch * (C * H_in * W_in) + c * (H_in * W_in) + (size_t)h * W_in + (size_t)w] += dcol[idx];
+    }
+}
+
+void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_out, size_t C_out, size_t batches) {
+    const size_t per = C_out * H_out * W_out;
+#pragma omp parallel for schedule(static)
+    for (size_t idx = 0; idx < per * batches; idx++) {                 /* :1386-1395 */
+        const size_t batch = idx / per, fixedIdx = idx % per;
+        const size_t c = fixedIdx / (H_out * W_out);
+        const size_t h = (fixedIdx % (H_out * W_out)) / W_out, w = (fixedIdx % (H_out * W_out)) % W_out;
+        dcol[batch * per + (h * W_out + w) * C_out + c] = dy[idx];
+    }
+}
+
+/* ------------------------------------------------------------------------- */
 /* Model::Conv2d graph (src/Model.cu:244-263): Img2Col -> MatMul -> Bias(Add)  */
 /* -> Col2Img, then an optional ReLU node; intermediates materialised.         */
 /* ------------------------------------------------------------------------- */

@@ -18,6 +18,9 @@
  *   - im2col / col2im ................ pinned (reference loop-nest spec,
  *                                      direct-convolution identity)
  *   - bias add / ReLU ................ pinned (closed form, NaN / -0 cases)
+ *   - backward (GEMM, add, ReLU, im2col, col2im) pinned (reference literal vectors
+ *                                      Test.cpp:820-903, loop nests :3011-3072 and
+ *                                      :3144-3177, adjoint identities <Jv,u> = <v,J^T u>)
  *   - bit-level accumulation order of nvcuda::wmma::mma_sync: PARITY UNPINNED
  *     (unspecified by the vendor; the tolerance contract replaces it).
  */
@@ -104,6 +107,29 @@ void nzo_linear_graph(float* y, const float* x, const float* w_out_in, const flo
                       size_t batch, size_t in_features, size_t out_features, int relu);
 
 /* ---- error metrics used by the tolerance contract */
+/* ---- backward of the same path -------------------------------------------
+ * GEMMBackwardParallel, src/OperationKernels.cu:1028-1144 (+ CuttingAndCompress :873-883):
+ * for every (i,j) of the batch max(A,B):  C[i or 0][j or 0] += f16(A_ij)[M,K] * f16(B_ij)[K,N]
+ * (fp32 accumulation per product, k ascending; products ADDED to what C holds, members of a
+ * reduced batch dimension in ascending order -- the reference's atomicAdd leaves that order open). */
+void nzo_gemm_backward(const float* A, const float* B, float* C, const size_t shapeA[4],
+                       const size_t shapeB[4], const size_t shapeC[4]);
+/* MatMulNode::backward, src/Nodes.cu:169-182: dA += dC * B^T, dB += A^T * dC through explicit
+ * transposes (TransposeKernel, OperationKernels.cu:125-145) and nzo_gemm_backward.  dA / dB may be NULL. */
+void nzo_matmul_backward(float* dA, float* dB, const float* A, const float* B, const float* dC,
+                         const size_t shapeA[4], const size_t shapeB[4], const size_t shapeC[4]);
+/* ReLUBackwardKernel, src/OperationKernels.cu:242-248: dx = x > 0 ? dy : 0 (overwrites). */
+void nzo_relu_backward(float* dx, const float* x, const float* dy, size_t n);
+/* AddNode::backward for one input, src/Nodes.cu:99-146: equal shapes -> copy (overwrite);
+ * otherwise din[n or 0][c or 0][:] += dout[n][c][:] for every (n,c) (gradCopyKernel :1230-1236). */
+void nzo_add_backward(float* din, const float* dout, const size_t shapeIn[4], const size_t shapeOut[4]);
+/* img2colBackwardKernel, src/OperationKernels.cu:1337-1355: every column-matrix gradient element is
+ * ADDED to the image gradient element it was copied from (padding positions dropped). */
+void nzo_im2col_backward(float* dx, const float* dcol, size_t H_out, size_t W_out, size_t C, size_t K_h,
+                         size_t K_w, size_t stride, size_t pad, size_t H_in, size_t W_in, size_t batch);
+/* col2imgBackwardKernel, src/OperationKernels.cu:1384-1396: dcol[b][(h*W+w)*C+c] = dy[b][c][h][w]. */
+void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_out, size_t C_out, size_t batches);
+
 /* max over i of |got-truth| / max(|truth|, floor) and Frobenius ||got-truth|| / ||truth|| */
 void nzo_errors_f32_vs_f64(const float* got, const double* truth, size_t n, double floor_abs,
                            double* max_rel, double* frob_rel);

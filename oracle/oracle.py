@@ -75,6 +75,12 @@ _im2col = _sig("nzo_im2col", None, _f32p, _f32p, *([_sz] * 10))
 _col2im = _sig("nzo_col2im", None, _f32p, _f32p, _sz, _sz, _sz, _sz)
 _madd = _sig("nzo_matrix_add", None, _f32p, _f32p, _f32p, _Shape, _Shape, _Shape)
 _relu = _sig("nzo_relu", None, _f32p, _f32p, _sz)
+_gemm_bwd = _sig("nzo_gemm_backward", None, _f32p, _f32p, _f32p, _Shape, _Shape, _Shape)
+_matmul_bwd = _sig("nzo_matmul_backward", None, C.c_void_p, C.c_void_p, _f32p, _f32p, _f32p, _Shape, _Shape, _Shape)
+_relu_bwd = _sig("nzo_relu_backward", None, _f32p, _f32p, _f32p, _sz)
+_add_bwd = _sig("nzo_add_backward", None, _f32p, _f32p, _Shape, _Shape)
+_im2col_bwd = _sig("nzo_im2col_backward", None, _f32p, _f32p, *([_sz] * 10))
+_col2im_bwd = _sig("nzo_col2im_backward", None, _f32p, _f32p, _sz, _sz, _sz, _sz)
 _conv_graph = _sig("nzo_conv2d_graph", None, _f32p, _f32p, _f32p, C.c_void_p, *([_sz] * 10), C.c_int)
 _conv_direct = _sig("nzo_conv2d_direct_f64", None, _f64p, _f32p, _f32p, C.c_void_p, *([_sz] * 9), C.c_int)
 _linear = _sig("nzo_linear_graph", None, _f32p, _f32p, _f32p, C.c_void_p, _sz, _sz, _sz, C.c_int)
@@ -210,6 +216,56 @@ def relu(a: np.ndarray) -> np.ndarray:
     a = _c(a)
     out = np.empty_like(a)
     _relu(out.reshape(-1), a.reshape(-1), a.size)
+    return out
+
+
+# ---- backward of the path ---------------------------------------------------
+def gemm_backward(A: np.ndarray, B: np.ndarray, C_acc: np.ndarray) -> np.ndarray:
+    """iGEMMBackward: returns C_acc + sum over the broadcast batch of f16(A)·f16(B) (C_acc is not modified)."""
+    A, B = _c(A), _c(B)
+    out = _c(C_acc).copy()
+    _gemm_bwd(A.reshape(-1), B.reshape(-1), out.reshape(-1), _Shape(*A.shape), _Shape(*B.shape), _Shape(*out.shape))
+    return out
+
+
+def matmul_backward(A, B, dC, dA0=None, dB0=None):
+    """MatMulNode::backward: (dA0 + dC·Bᵀ, dB0 + Aᵀ·dC); a gradient whose start value is None is skipped."""
+    A, B, dC = _c(A), _c(B), _c(dC)
+    dA = None if dA0 is None else _c(dA0).copy()
+    dB = None if dB0 is None else _c(dB0).copy()
+    _matmul_bwd(_ptr(dA), _ptr(dB), A.reshape(-1), B.reshape(-1), dC.reshape(-1), _Shape(*A.shape), _Shape(*B.shape),
+                _Shape(*dC.shape))
+    return dA, dB
+
+
+def relu_backward(x: np.ndarray, dy: np.ndarray) -> np.ndarray:
+    x, dy = _c(x), _c(dy)
+    out = np.empty_like(x)
+    _relu_bwd(out.reshape(-1), x.reshape(-1), dy.reshape(-1), x.size)
+    return out
+
+
+def add_backward(din0: np.ndarray, dout: np.ndarray) -> np.ndarray:
+    """AddNode::backward for one input whose gradient currently holds din0."""
+    out, dout = _c(din0).copy(), _c(dout)
+    _add_bwd(out.reshape(-1), dout.reshape(-1), _Shape(*out.shape), _Shape(*dout.shape))
+    return out
+
+
+def im2col_backward(dx0: np.ndarray, dcol: np.ndarray, K_h: int, K_w: int, stride: int, pad: int) -> np.ndarray:
+    out, dcol = _c(dx0).copy(), _c(dcol)
+    N, Cc, H, W = out.shape
+    Ho, Wo = out_hw(H, W, K_h, K_w, stride, pad)
+    assert dcol.size == N * Ho * Wo * Cc * K_h * K_w
+    _im2col_bwd(out.reshape(-1), dcol.reshape(-1), Ho, Wo, Cc, K_h, K_w, stride, pad, H, W, N)
+    return out
+
+
+def col2im_backward(dy: np.ndarray) -> np.ndarray:
+    dy = _c(dy)
+    N, O, Ho, Wo = dy.shape
+    out = np.empty((N, 1, Ho * Wo, O), np.float32)
+    _col2im_bwd(out.reshape(-1), dy.reshape(-1), Ho, Wo, O, N)
     return out
 
 
