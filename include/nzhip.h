@@ -124,6 +124,41 @@ int nzhip_add_broadcast(float* out, const float* a, const float* b, const size_t
 /* nz::data::iRELU (TensorOperations.cuh:19; RectifiedLinearUnitKernel, OperationKernels.cu:230-235). */
 int nzhip_relu(float* out, const float* in, size_t n, void* stream);
 
+/* ---- backward of the same path -------------------------------------------- */
+/* nz::data::iGEMMBackward (include/NeuZephyr/TensorOperations.cuh:1030-1031, src/TensorOperations.cu:117-120
+ * -> krnl::GEMMBackwardParallel, src/OperationKernels.cu:1028-1144): over the batch max(A, B),
+ *     C[n or 0][c or 0] += f16(A_nc)[M,K] * f16(B_nc)[K,N]          (M = A.h, K = A.w, N = B.w)
+ * i.e. the products are ADDED to what C holds, and a batch dimension in which C has extent 1
+ * collects every member (CuttingAndCompress, :873-883). Members are added in a fixed order
+ * (the reference's atomicAdd leaves it open). */
+int nzhip_gemm_backward(const float* A, const float* B, float* C, const size_t shapeA[4],
+                        const size_t shapeB[4], const size_t shapeC[4], void* stream);
+
+/* MatMulNode::backward (src/Nodes.cu:169-182) without the materialised transposes:
+ *     dA += dC * B^T        dB += A^T * dC
+ * for C = A * B with the forward's shapes and broadcast rules; dA or dB may be NULL to skip it. */
+int nzhip_matmul_backward(float* dA, float* dB, const float* A, const float* B, const float* dC,
+                          const size_t shapeA[4], const size_t shapeB[4], const size_t shapeC[4], void* stream);
+
+/* ReLUBackwardKernel (src/OperationKernels.cu:242-253): dx = x > 0 ? dy : 0 (overwrites dx). */
+int nzhip_relu_backward(float* dx, const float* x, const float* dy, size_t n, void* stream);
+
+/* AddNode::backward for one input (src/Nodes.cu:99-146): equal shapes -> din = dout (copy);
+ * otherwise din[n or 0][c or 0][:] += dout[n][c][:] over every (n, c) (gradCopyKernel, :1230-1236). */
+int nzhip_add_backward(float* din, const float* dout, const size_t shapeIn[4], const size_t shapeOut[4],
+                       void* stream);
+
+/* nz::data::iImg2colBackward (img2colBackwardKernel, src/OperationKernels.cu:1337-1362): every element of the
+ * column-matrix gradient is ADDED to the image-gradient element it was copied from. */
+int nzhip_im2col_backward(float* dx, const float* dcol, size_t H_out, size_t W_out, size_t C, size_t K_h,
+                          size_t K_w, size_t stride, size_t pad, size_t H_in, size_t W_in, size_t batch,
+                          void* stream);
+
+/* nz::data::iCol2imgBackward (col2imgBackwardKernel, src/OperationKernels.cu:1384-1402):
+ * dcol[b][(h*W_out+w)*C_out + c] = dy[b][c][h][w]. */
+int nzhip_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_out, size_t C_out,
+                          size_t batches, void* stream);
+
 /* ---- runtime: device allocator + stream manager -------------------------- */
 /* Replace cuStrm::StreamManager<float> (include/NeuZephyr/StreamManager.cuh:131-911) and
  * EventPool (EventPool.cuh:165-457).  One ordered compute stream carries every kernel and

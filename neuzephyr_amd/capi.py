@@ -17,6 +17,8 @@ LAYOUT_ROW, LAYOUT_TRANS = 0, 1
 EXPORTS = [
     "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_tensorcore_gemm",
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
+    "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
+    "nzhip_im2col_backward", "nzhip_col2im_backward",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
@@ -73,6 +75,12 @@ def load() -> C.CDLL:
     lib.nzhip_conv2d_forward.argtypes = [vp, vp, vp, vp] + [sz] * 10 + [i64, i64, C.c_int, vp]
     lib.nzhip_add_broadcast.argtypes = [vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_relu.argtypes = [vp, vp, sz, vp]
+    lib.nzhip_gemm_backward.argtypes = [vp, vp, vp, shape, shape, shape, vp]
+    lib.nzhip_matmul_backward.argtypes = [vp, vp, vp, vp, vp, shape, shape, shape, vp]
+    lib.nzhip_relu_backward.argtypes = [vp, vp, vp, sz, vp]
+    lib.nzhip_add_backward.argtypes = [vp, vp, shape, shape, vp]
+    lib.nzhip_im2col_backward.argtypes = [vp, vp] + [sz] * 10 + [vp]
+    lib.nzhip_col2im_backward.argtypes = [vp, vp, sz, sz, sz, sz, vp]
     lib.nzhip_default_stream.restype = vp
     lib.nzhip_malloc.argtypes = [C.POINTER(vp), sz]
     lib.nzhip_free_async.argtypes = [vp]
@@ -228,4 +236,52 @@ def relu(a, stream=None):
     lib = load()
     out = torch.empty_like(a)
     check(lib.nzhip_relu(_dev(out), _dev(a), a.numel(), _stream_handle(stream)))
+    return out
+
+
+# ---- backward of the path (gradient buffers are updated in place, as in the reference) ----------
+def gemm_backward(A, B, C, stream=None):
+    """C[n or 0][c or 0] += f16(A)·f16(B) over the batch max(A, B); C is modified in place."""
+    lib = load()
+    check(lib.nzhip_gemm_backward(_dev(A), _dev(B), _dev(C), shape4(A.shape), shape4(B.shape), shape4(C.shape),
+                                  _stream_handle(stream)))
+    return C
+
+
+def matmul_backward(dA, dB, A, B, dC, stream=None):
+    """dA += dC·Bᵀ, dB += Aᵀ·dC in place; pass None for a gradient that is not wanted."""
+    lib = load()
+    check(lib.nzhip_matmul_backward(None if dA is None else _dev(dA), None if dB is None else _dev(dB), _dev(A), _dev(B),
+                                    _dev(dC), shape4(A.shape), shape4(B.shape), shape4(dC.shape), _stream_handle(stream)))
+    return dA, dB
+
+
+def relu_backward(x, dy, stream=None):
+    import torch
+    lib = load()
+    dx = torch.empty_like(x)
+    check(lib.nzhip_relu_backward(_dev(dx), _dev(x), _dev(dy), x.numel(), _stream_handle(stream)))
+    return dx
+
+
+def add_backward(din, dout, stream=None):
+    lib = load()
+    check(lib.nzhip_add_backward(_dev(din), _dev(dout), shape4(din.shape), shape4(dout.shape), _stream_handle(stream)))
+    return din
+
+
+def im2col_backward(dx, dcol, K_h, K_w, stride, pad, stream=None):
+    lib = load()
+    N, Cc, H, W = dx.shape
+    Ho, Wo = (H + 2 * pad - K_h) // stride + 1, (W + 2 * pad - K_w) // stride + 1
+    check(lib.nzhip_im2col_backward(_dev(dx), _dev(dcol), Ho, Wo, Cc, K_h, K_w, stride, pad, H, W, N, _stream_handle(stream)))
+    return dx
+
+
+def col2im_backward(dy, stream=None):
+    import torch
+    lib = load()
+    N, O, Ho, Wo = dy.shape
+    out = torch.empty((N, 1, Ho * Wo, O), dtype=torch.float32, device=dy.device)
+    check(lib.nzhip_col2im_backward(_dev(out), _dev(dy), Ho, Wo, O, N, _stream_handle(stream)))
     return out

@@ -100,6 +100,73 @@ __global__ __launch_bounds__(256) void relu_kernel(float* __restrict__ out, cons
     }
 }
 
+// ---- backward element-wise kernels -----------------------------------------------------------
+// ReLUBackwardKernel (src/OperationKernels.cu:242-248): dx = x > 0 ? dy : 0 (overwrites dx).
+__global__ __launch_bounds__(256) void relu_backward_kernel(float* __restrict__ dx, const float* __restrict__ x,
+                                                            const float* __restrict__ dy, long n, int vec) {
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec) {
+        if (t * 4 + 3 < n) {
+            const floatx4 a = reinterpret_cast<const floatx4*>(x)[t], g = reinterpret_cast<const floatx4*>(dy)[t];
+            floatx4 o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = a[e] > 0.f ? g[e] : 0.f;
+            reinterpret_cast<floatx4*>(dx)[t] = o;
+        } else {
+            for (long k = t * 4; k < n; k++) dx[k] = x[k] > 0.f ? dy[k] : 0.f;
+        }
+    } else if (t < n) {
+        dx[t] = x[t] > 0.f ? dy[t] : 0.f;
+    }
+}
+
+// gradCopyKernel over every (n,c) of the output (src/Nodes.cu:107-121, OperationKernels.cu:1230-1236):
+// din[n or 0][c or 0][:] += dout[n][c][:]. One thread owns one element of din and adds the members
+// that map onto it in ascending (n,c) order, so the sum does not depend on scheduling.
+__global__ __launch_bounds__(256) void grad_reduce_kernel(float* __restrict__ din, const float* __restrict__ dout,
+                                                          long hw, int in_n, int in_c, int out_n, int out_c) {
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= hw) return;
+    const int i0 = blockIdx.y / in_c, j0 = blockIdx.y % in_c;
+    float* dst = din + ((long)i0 * in_c + j0) * hw + t;
+    float acc = *dst;
+    const int i_lo = in_n > 1 ? i0 : 0, i_hi = in_n > 1 ? i0 + 1 : out_n;
+    const int j_lo = in_c > 1 ? j0 : 0, j_hi = in_c > 1 ? j0 + 1 : out_c;
+    for (int i = i_lo; i < i_hi; i++)
+        for (int j = j_lo; j < j_hi; j++) acc += dout[((long)i * out_c + j) * hw + t];
+    *dst = acc;
+}
+
+// img2colBackwardKernel (src/OperationKernels.cu:1337-1355) as a gather: one thread owns one image
+// gradient element and adds the column-matrix gradient entries that were copied from it, in
+// ascending pixel order (the order in which the reference's element index visits them); no atomics.
+__global__ __launch_bounds__(256) void im2col_backward_kernel(float* __restrict__ dx, const float* __restrict__ dcol,
+                                                              int H_out, int W_out, int C, int K_h, int K_w,
+                                                              int stride, int pad, int H_in, int W_in) {
+    const long per_img = (long)C * H_in * W_in;
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= per_img) return;
+    const int b = blockIdx.y;
+    const int c = (int)(t / ((long)H_in * W_in));
+    const int h = (int)((t / W_in) % H_in), w = (int)(t % W_in);
+    const int CKK = C * K_h * K_w;
+    const float* col = dcol + (long)b * H_out * W_out * CKK + (long)c * K_h * K_w;
+    float acc = dx[(long)b * per_img + t];
+    // ho*stride - pad + r == h with 0 <= r < K_h  <=>  ho in [ceil((h+pad-K_h+1)/stride), (h+pad)/stride]
+    const int ho_lo = h + pad - K_h + 1 > 0 ? (h + pad - K_h + 1 + stride - 1) / stride : 0;
+    const int ho_hi = (h + pad) / stride < H_out - 1 ? (h + pad) / stride : H_out - 1;
+    const int wo_lo = w + pad - K_w + 1 > 0 ? (w + pad - K_w + 1 + stride - 1) / stride : 0;
+    const int wo_hi = (w + pad) / stride < W_out - 1 ? (w + pad) / stride : W_out - 1;
+    for (int ho = ho_lo; ho <= ho_hi; ho++) {
+        const int r = h + pad - ho * stride;
+        for (int wo = wo_lo; wo <= wo_hi; wo++) {
+            const int sx = w + pad - wo * stride;
+            acc += col[((long)ho * W_out + wo) * CKK + r * K_w + sx];
+        }
+    }
+    dx[(long)b * per_img + t] = acc;
+}
+
 static int validate_gemm(const nzhip_gemm_desc& d) {
     if (d.M < 0 || d.N < 0 || d.K < 0) return set_error(NZHIP_E_INVALID, "nzhip_gemm: negative extent");
     // an operand with no elements may be null
@@ -298,6 +365,216 @@ int nzhip_relu(float* out, const float* in, size_t n, void* stream) {
     hipLaunchKernelGGL(relu_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, as_stream(stream), out, in,
                        (long)n, vec);
     return check_launch("relu_kernel");
+}
+
+// ---- backward of the path ---------------------------------------------------------------------
+namespace {
+
+struct BwdOperand {
+    const float* p;
+    int layout;
+    int64_t ld;
+    int64_t sn, sc;                                        // batch strides, 0 = broadcast
+};
+
+// For every (i, j) of a bn x bc batch:  C[i*c_sn + j*c_sc] += f16(A_ij)[M,K] * f16(B_ij)[K,N].
+// A batch stride of 0 on C makes that batch dimension a reduction (CuttingAndCompress,
+// src/OperationKernels.cu:873-883, adds every member onto the same matrix). "+=" is the GEMM's bias
+// operand pointed at C itself: every element is read and then written by the same lane.
+// Reductions are folded into the contraction (K' = members x K, one launch) when both operands are
+// laid out so that the member index continues the k index; otherwise the members are added one
+// launch after the other, which fixes the summation order.
+int accumulate_products(float* C, int64_t ldc, int64_t c_sn, int64_t c_sc, BwdOperand A, BwdOperand B, int64_t M,
+                        int64_t N, int64_t K, int64_t bn, int64_t bc, void* stream) {
+    if (bn == 0 || bc == 0 || M == 0 || N == 0) return NZHIP_OK;
+    auto launch = [&](const float* a, const float* b, float* c, int64_t k, int la, int64_t lda, int lb, int64_t ldb,
+                      int64_t nb_n, int64_t nb_c, int64_t csn, int64_t csc) {
+        nzhip_gemm_desc g = {};
+        g.A = a; g.B = b; g.C = c;
+        g.M = M; g.N = N; g.K = k;
+        g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+        g.a_layout = la; g.b_layout = lb;
+        g.batch_n = nb_n; g.batch_c = nb_c;
+        g.a_stride_n = A.sn; g.a_stride_c = A.sc;
+        g.b_stride_n = B.sn; g.b_stride_c = B.sc;
+        g.c_stride_n = csn; g.c_stride_c = csc;
+        g.bias = c;
+        g.bias_stride_row = ldc; g.bias_stride_col = 1;
+        g.bias_stride_n = csn; g.bias_stride_c = csc;
+        return nzhip_gemm(&g, stream);
+    };
+    const bool red_n = c_sn == 0 && bn > 1, red_c = c_sc == 0 && bc > 1;
+    // distance between consecutive batch members of an operand, if it is the same for all of them
+    auto spacing = [&](int64_t sn, int64_t sc, int64_t& s) {
+        if (bc == 1) { s = sn; return true; }
+        if (bn == 1) { s = sc; return true; }
+        s = sc;
+        return sn == bc * sc;
+    };
+    if (!red_n && !red_c && bn * bc > 1 && K > 0) {
+        // One shared matrix against a batch of vectors is a single GEMM whose rows are the members
+        // (the shared operand is then read once instead of once per member).
+        const int64_t T = bn * bc;
+        int64_t sc_ = 0, sa = 0, sb = 0;
+        const bool uc = spacing(c_sn, c_sc, sc_), ua = spacing(A.sn, A.sc, sa), ub = spacing(B.sn, B.sc, sb);
+        const bool a_shared = A.sn == 0 && A.sc == 0, b_shared = B.sn == 0 && B.sc == 0;
+        if (N == 1 && a_shared && uc && ub && ldc == 1 && sc_ >= M && sb >= K && (B.layout == NZHIP_LAYOUT_TRANS || B.ld == 1)) {
+            // C_t[M,1] = A[M,K] * B_t[K,1]   ->   Cmat[T,M] = Bmat[T,K] * A^T
+            nzhip_gemm_desc g = {};
+            g.A = B.p; g.B = A.p; g.C = C;
+            g.M = T; g.N = M; g.K = K;
+            g.lda = sb; g.ldb = A.ld; g.ldc = sc_;
+            g.a_layout = NZHIP_LAYOUT_ROW;
+            g.b_layout = A.layout == NZHIP_LAYOUT_ROW ? NZHIP_LAYOUT_TRANS : NZHIP_LAYOUT_ROW;
+            g.batch_n = g.batch_c = 1;
+            g.bias = C; g.bias_stride_row = sc_; g.bias_stride_col = 1;
+            return nzhip_gemm(&g, stream);
+        }
+        if (M == 1 && b_shared && uc && ua && sc_ >= N && sa >= K && (A.layout == NZHIP_LAYOUT_ROW || A.ld == 1)) {
+            // C_t[1,N] = A_t[1,K] * B[K,N]   ->   Cmat[T,N] = Amat[T,K] * B
+            nzhip_gemm_desc g = {};
+            g.A = A.p; g.B = B.p; g.C = C;
+            g.M = T; g.N = N; g.K = K;
+            g.lda = sa; g.ldb = B.ld; g.ldc = sc_;
+            g.a_layout = NZHIP_LAYOUT_ROW; g.b_layout = B.layout;
+            g.batch_n = g.batch_c = 1;
+            g.bias = C; g.bias_stride_row = sc_; g.bias_stride_col = 1;
+            return nzhip_gemm(&g, stream);
+        }
+    }
+    if (!red_n && !red_c) {
+        if (bn * bc <= 65535) return launch(A.p, B.p, C, K, A.layout, A.ld, B.layout, B.ld, bn, bc, c_sn, c_sc);
+        for (int64_t i = 0; i < bn; i++)
+            for (int64_t j0 = 0; j0 < bc; j0 += 65535) {
+                const int64_t cnt = bc - j0 < 65535 ? bc - j0 : 65535;
+                if (int rc = launch(A.p + i * A.sn + j0 * A.sc, B.p + i * B.sn + j0 * B.sc, C + i * c_sn + j0 * c_sc, K,
+                                    A.layout, A.ld, B.layout, B.ld, 1, cnt, 0, c_sc))
+                    return rc;
+            }
+        return NZHIP_OK;
+    }
+    // every member reduces into one matrix and the members are evenly spaced: fold them into K
+    const bool all = (red_n || bn == 1) && (red_c || bc == 1);
+    if (all && K > 0) {
+        const int64_t T = bn * bc;
+        int64_t sa = 0, sb = 0;
+        const bool ua = spacing(A.sn, A.sc, sa), ub = spacing(B.sn, B.sc, sb);
+        int la = -1, lb = -1;
+        int64_t lda = 0, ldb = 0;
+        if (ua && A.layout == NZHIP_LAYOUT_TRANS && sa == K * A.ld) { la = NZHIP_LAYOUT_TRANS; lda = A.ld; }
+        else if (ua && K == 1 && sa >= M && (A.layout == NZHIP_LAYOUT_TRANS || A.ld == 1)) { la = NZHIP_LAYOUT_TRANS; lda = sa; }
+        if (ub && B.layout == NZHIP_LAYOUT_ROW && sb == K * B.ld) { lb = NZHIP_LAYOUT_ROW; ldb = B.ld; }
+        else if (ub && K == 1 && sb >= N && (B.layout == NZHIP_LAYOUT_ROW || B.ld == 1)) { lb = NZHIP_LAYOUT_ROW; ldb = sb; }
+        if (la >= 0 && lb >= 0 && T * K <= 0x3fffffff) {
+            BwdOperand a1 = A, b1 = B;
+            A.sn = A.sc = B.sn = B.sc = 0;                       // one member left
+            const int rc = launch(a1.p, b1.p, C, T * K, la, lda, lb, ldb, 1, 1, 0, 0);
+            A = a1; B = b1;
+            return rc;
+        }
+    }
+    // members one after the other; a dimension that does not reduce stays a batch of the launch
+    for (int64_t i = 0; i < (red_n ? bn : 1); i++)
+        for (int64_t j = 0; j < (red_c ? bc : 1); j++) {
+            const int64_t nb_n = red_n ? 1 : bn, nb_c = red_c ? 1 : bc;
+            if (nb_n * nb_c > 65535) return set_error(NZHIP_E_UNSUPPORTED, "gemm backward: more than 65535 batch members");
+            if (int rc = launch(A.p + i * A.sn + j * A.sc, B.p + i * B.sn + j * B.sc, C, K, A.layout, A.ld, B.layout,
+                                B.ld, nb_n, nb_c, c_sn, c_sc))
+                return rc;
+        }
+    return NZHIP_OK;
+}
+
+inline int64_t bstride_n(const size_t s[4]) { return s[0] > 1 ? (int64_t)(s[1] * s[2] * s[3]) : 0; }
+inline int64_t bstride_c(const size_t s[4]) { return s[1] > 1 ? (int64_t)(s[2] * s[3]) : 0; }
+
+}  // namespace
+
+int nzhip_gemm_backward(const float* A, const float* B, float* C, const size_t sA[4], const size_t sB[4],
+                        const size_t sC[4], void* stream) {
+    if (!A || !B || !C || !sA || !sB || !sC) return set_error(NZHIP_E_INVALID, "nzhip_gemm_backward: null argument");
+    const int64_t M = (int64_t)sA[2], N = (int64_t)sB[3], K = (int64_t)sA[3];      // src/OperationKernels.cu:1032-1034
+    const int64_t bn = (int64_t)(sA[0] > sB[0] ? sA[0] : sB[0]), bc = (int64_t)(sA[1] > sB[1] ? sA[1] : sB[1]);
+    BwdOperand a = {A, NZHIP_LAYOUT_ROW, K, bstride_n(sA), bstride_c(sA)};
+    BwdOperand b = {B, NZHIP_LAYOUT_ROW, N, bstride_n(sB), bstride_c(sB)};
+    return accumulate_products(C, N, bstride_n(sC), bstride_c(sC), a, b, M, N, K, bn, bc, stream);   // :1116-1124
+}
+
+int nzhip_matmul_backward(float* dA, float* dB, const float* A, const float* B, const float* dC, const size_t sA[4],
+                          const size_t sB[4], const size_t sC[4], void* stream) {
+    if (!dC || !sA || !sB || !sC || (dA && !B) || (dB && !A))
+        return set_error(NZHIP_E_INVALID, "nzhip_matmul_backward: null argument");
+    const int64_t M = (int64_t)sA[2], K = (int64_t)sA[3], N = (int64_t)sB[3];
+    if ((int64_t)sB[2] != K || (int64_t)sC[2] != M || (int64_t)sC[3] != N)
+        return set_error(NZHIP_E_SHAPE, "nzhip_matmul_backward: shapes do not describe C = A * B");
+    const int64_t bn = (int64_t)sC[0], bc = (int64_t)sC[1];
+    const BwdOperand g = {dC, NZHIP_LAYOUT_ROW, N, (int64_t)(sC[1] * sC[2] * sC[3]), (int64_t)(sC[2] * sC[3])};
+    if (dA) {                                              // dA += dC * B^T   (src/Nodes.cu:171-175)
+        const BwdOperand bt = {B, NZHIP_LAYOUT_TRANS, N, bstride_n(sB), bstride_c(sB)};
+        if (int rc = accumulate_products(dA, K, bstride_n(sA), bstride_c(sA), g, bt, M, K, N, bn, bc, stream)) return rc;
+    }
+    if (dB) {                                              // dB += A^T * dC   (src/Nodes.cu:177-181)
+        const BwdOperand at = {A, NZHIP_LAYOUT_TRANS, K, bstride_n(sA), bstride_c(sA)};
+        if (int rc = accumulate_products(dB, N, bstride_n(sB), bstride_c(sB), at, g, K, N, M, bn, bc, stream)) return rc;
+    }
+    return NZHIP_OK;
+}
+
+int nzhip_relu_backward(float* dx, const float* x, const float* dy, size_t n, void* stream) {
+    if ((!dx || !x || !dy) && n) return set_error(NZHIP_E_INVALID, "nzhip_relu_backward: null pointer");
+    if (n == 0) return NZHIP_OK;
+    const int vec = aligned16(dx) && aligned16(x) && aligned16(dy);
+    const size_t threads = vec ? (n + 3) / 4 : n;
+    hipLaunchKernelGGL(relu_backward_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, as_stream(stream),
+                       dx, x, dy, (long)n, vec);
+    return check_launch("relu_backward_kernel");
+}
+
+int nzhip_add_backward(float* din, const float* dout, const size_t sIn[4], const size_t sOut[4], void* stream) {
+    if (!din || !dout || !sIn || !sOut) return set_error(NZHIP_E_INVALID, "nzhip_add_backward: null argument");
+    if (sIn[2] != sOut[2] || sIn[3] != sOut[3] || (sIn[0] != sOut[0] && sIn[0] != 1) || (sIn[1] != sOut[1] && sIn[1] != 1))
+        return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
+    const size_t hw = sOut[2] * sOut[3], total = sOut[0] * sOut[1] * hw;
+    if (total == 0) return NZHIP_OK;
+    if (sIn[0] == sOut[0] && sIn[1] == sOut[1]) {          // src/Nodes.cu:101-105: plain copy
+        hipError_t e = hipMemcpyAsync(din, dout, total * sizeof(float), hipMemcpyDeviceToDevice, as_stream(stream));
+        return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipMemcpyAsync(add backward)");
+    }
+    if (sIn[0] * sIn[1] > 65535 || sOut[0] > 0x7fffffff || sOut[1] > 0x7fffffff)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_add_backward: more than 65535 (n,c) planes");
+    dim3 grid((unsigned)((hw + 255) / 256), (unsigned)(sIn[0] * sIn[1]));
+    hipLaunchKernelGGL(grad_reduce_kernel, grid, dim3(256), 0, as_stream(stream), din, dout, (long)hw, (int)sIn[0],
+                       (int)sIn[1], (int)sOut[0], (int)sOut[1]);
+    return check_launch("grad_reduce_kernel");
+}
+
+int nzhip_im2col_backward(float* dx, const float* dcol, size_t H_out, size_t W_out, size_t C, size_t K_h, size_t K_w,
+                          size_t stride, size_t pad, size_t H_in, size_t W_in, size_t batch, void* stream) {
+    if (!dx || !dcol) return set_error(NZHIP_E_INVALID, "nzhip_im2col_backward: null pointer");
+    if (stride == 0 || K_h == 0 || K_w == 0)
+        return set_error(NZHIP_E_INVALID, "nzhip_im2col_backward: zero stride or kernel extent");
+    const size_t per = C * H_in * W_in;
+    if (per == 0 || batch == 0 || H_out == 0 || W_out == 0) return NZHIP_OK;
+    if (per > 0x7fffffffull * 256 || batch > 65535 || H_in > 0x3fffffff || W_in > 0x3fffffff || pad > 0x3fffffff ||
+        H_out * W_out * C * K_h * K_w > 0x7fffffffffffull)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_im2col_backward: extent too large");
+    dim3 grid((unsigned)((per + 255) / 256), (unsigned)batch);
+    hipLaunchKernelGGL(im2col_backward_kernel, grid, dim3(256), 0, as_stream(stream), dx, dcol, (int)H_out, (int)W_out,
+                       (int)C, (int)K_h, (int)K_w, (int)stride, (int)pad, (int)H_in, (int)W_in);
+    return check_launch("im2col_backward_kernel");
+}
+
+int nzhip_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_out, size_t C_out, size_t batches,
+                          void* stream) {
+    if (!dcol || !dy) return set_error(NZHIP_E_INVALID, "nzhip_col2im_backward: null pointer");
+    const size_t HW = H_out * W_out;
+    if (HW == 0 || C_out == 0 || batches == 0) return NZHIP_OK;
+    if (C_out > 0x7fffffff || (HW + 31) / 32 > 65535 || batches > 65535)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_col2im_backward: extent too large");
+    // the inverse transpose of col2im: [C_out, HW] -> [HW, C_out] per image
+    dim3 grid((unsigned)((C_out + 31) / 32), (unsigned)((HW + 31) / 32), (unsigned)batches);
+    hipLaunchKernelGGL(col2im_kernel, grid, dim3(256), 0, as_stream(stream), dcol, dy, (int)C_out, (int)HW);
+    return check_launch("col2im_kernel (backward)");
 }
 
 }  // extern "C"

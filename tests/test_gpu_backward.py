@@ -1,0 +1,184 @@
+"""Parity of the backward entry points (GEMM backward with batch reduction, MatMul / Add / ReLU /
+im2col / col2im backward) on the GPU with the CPU oracle, through the C-ABI.  Integer-valued cases
+must match bit for bit (sums are exact in any order); float cases meet max-rel <= 1e-3 /
+Frobenius-rel <= 1e-4 against fp64 accumulation of the same fp16-rounded operands (max-rel floored
+at the RMS of the truth)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+MAX_REL, FROB_REL = 1e-3, 1e-4
+
+
+@pytest.fixture(scope="module")
+def nz():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from neuzephyr_amd import capi
+    capi.load()
+    return capi
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def check_tolerance(oracle, got, truth64, tag=""):
+    rms = float(np.sqrt(np.mean(np.square(truth64)))) or 1.0
+    mr, fr = oracle.errors(got, truth64, rms)
+    assert mr <= MAX_REL and fr <= FROB_REL, f"{tag}: max_rel {mr:.3e} frob_rel {fr:.3e}"
+
+
+def ints(rng, shape, lo=-4, hi=5):
+    return rng.integers(lo, hi, shape).astype(np.float32)
+
+
+def test_matmul_backward_reference_vectors(nz):
+    # test/Test.cpp:820-903
+    n, c, m, k, p = 2, 3, 2, 3, 2
+    A = np.ones((n, 1, m, k), np.float32); B = np.ones((1, c, k, p), np.float32); dC = np.ones((n, c, m, p), np.float32)
+    dA, dB = dev(np.zeros_like(A)), dev(np.zeros_like(B))
+    nz.matmul_backward(dA, dB, dev(A), dev(B), dev(dC))
+    assert np.array_equal(host(dA), np.full_like(A, 2 * c)) and np.array_equal(host(dB), np.full_like(B, 2 * n))
+    A = np.array([1, 2, 3, 4, 5, 6, 2, 3, 4, 5, 6, 7, 3, 4, 5, 6, 7, 8] * 2, np.float32).reshape(n, c, m, k)
+    B = np.array([1, 4, 2, 5, 3, 6, 2, 5, 3, 6, 4, 7, 3, 6, 4, 7, 5, 8], np.float32).reshape(1, c, k, p)
+    Agrad = np.array([5, 7, 9, 5, 7, 9, 7, 9, 11, 7, 9, 11, 9, 11, 13, 9, 11, 13] * 2, np.float32).reshape(n, c, m, k)
+    Bgrad = np.array([10, 10, 14, 14, 18, 18, 14, 14, 18, 18, 22, 22, 18, 18, 22, 22, 26, 26], np.float32).reshape(1, c, k, p)
+    dA, dB = dev(np.zeros_like(A)), dev(np.zeros_like(B))
+    nz.matmul_backward(dA, dB, dev(A), dev(B), dev(dC))
+    assert np.array_equal(host(dA), Agrad) and np.array_equal(host(dB), Bgrad)
+
+
+# (shapeA, shapeB): every broadcast pattern, ragged extents, the vector collapses and the K-folded reductions
+MATMUL_BWD_CASES = [
+    ((2, 3, 5, 7), (2, 3, 7, 6)),        # no broadcast
+    ((2, 1, 5, 7), (1, 3, 7, 6)),        # both broadcast in different dims
+    ((1, 1, 9, 4), (3, 2, 4, 5)),        # A shared: dA reduces over n and c (sequential members)
+    ((3, 2, 9, 4), (1, 1, 4, 5)),        # B shared: dB reduces over both, folded into K
+    ((4, 1, 33, 20), (1, 1, 20, 17)),    # conv-like: column matrix per image, shared weights
+    ((1, 1, 24, 16), (5, 1, 16, 1)),     # Model::Linear: W[OUT,IN] * x_n[IN,1]
+    ((6, 1, 1, 12), (1, 1, 12, 10)),     # row vectors against a shared matrix
+    ((1, 3, 8, 8), (4, 3, 8, 8)),        # reduce over n only, c stays a batch
+    ((2, 2, 1, 1), (2, 2, 1, 1)),
+    ((1, 1, 130, 70), (1, 1, 70, 140)),  # one matrix, larger than a tile
+]
+
+
+@pytest.mark.parametrize("sa,sb", MATMUL_BWD_CASES)
+def test_matmul_backward_integers_bit_exact(nz, oracle, sa, sb):
+    rng = np.random.default_rng(hash((sa, sb)) % (1 << 31))
+    A, B = ints(rng, sa, -3, 4), ints(rng, sb, -3, 4)
+    sc = (max(sa[0], sb[0]), max(sa[1], sb[1]), sa[2], sb[3])
+    dC = ints(rng, sc, -3, 4)
+    dA0, dB0 = ints(rng, sa, -9, 10), ints(rng, sb, -9, 10)       # gradients already hold something: "+="
+    want_dA, want_dB = oracle.matmul_backward(A, B, dC, dA0, dB0)
+    dA, dB = dev(dA0), dev(dB0)
+    nz.matmul_backward(dA, dB, dev(A), dev(B), dev(dC))
+    assert np.array_equal(host(dA), want_dA), "dA"
+    assert np.array_equal(host(dB), want_dB), "dB"
+    # one gradient at a time
+    dA = dev(dA0); nz.matmul_backward(dA, None, dev(A), dev(B), dev(dC)); assert np.array_equal(host(dA), want_dA)
+    dB = dev(dB0); nz.matmul_backward(None, dB, dev(A), dev(B), dev(dC)); assert np.array_equal(host(dB), want_dB)
+
+
+@pytest.mark.parametrize("sa,sb,sc", [((2, 3, 5, 7), (2, 3, 7, 6), (2, 3, 5, 6)), ((3, 1, 5, 7), (1, 2, 7, 6), (1, 1, 5, 6)),
+                                     ((3, 2, 5, 7), (3, 2, 7, 6), (1, 2, 5, 6)), ((3, 2, 5, 7), (3, 2, 7, 6), (3, 1, 5, 6)),
+                                     ((1, 1, 40, 33), (1, 1, 33, 50), (1, 1, 40, 50))])
+def test_gemm_backward_entry_integers_bit_exact(nz, oracle, sa, sb, sc):
+    rng = np.random.default_rng(17)
+    A, B, C0 = ints(rng, sa), ints(rng, sb), ints(rng, sc, -9, 10)
+    want = oracle.gemm_backward(A, B, C0)
+    C = dev(C0)
+    nz.gemm_backward(dev(A), dev(B), C)
+    assert np.array_equal(host(C), want)
+
+
+def test_linear_layer_backward_float_tolerance(nz, oracle):
+    # Model::Linear shapes (W[1,1,OUT,IN] * x[n,1,IN,1]) at a size the oracle finishes quickly
+    n, IN, OUT = 192, 256, 320
+    W = oracle.fill((1, 1, OUT, IN), 2101, "uniform", -0.0765, 0.0765)
+    x = oracle.fill((n, 1, IN, 1), 2102, "normal", 0.0, 1.0)
+    dy = oracle.fill((n, 1, OUT, 1), 2103, "normal", 0.0, 1.0)
+    dW, dx = dev(np.zeros_like(W)), dev(np.zeros_like(x))
+    nz.matmul_backward(dW, dx, dev(W), dev(x), dev(dy))
+    dyr, xr, Wr = (oracle.round_f16(t).astype(np.float64) for t in (dy, x, W))
+    truth_dW = dyr.reshape(n, OUT).T @ xr.reshape(n, IN)
+    truth_dx = dyr.reshape(n, OUT) @ Wr.reshape(OUT, IN)
+    check_tolerance(oracle, host(dW).reshape(OUT, IN), truth_dW, "dW")
+    check_tolerance(oracle, host(dx).reshape(n, IN), truth_dx, "dx")
+
+
+def test_conv_weight_gradient_float_tolerance(nz, oracle):
+    # dW = sum over images of col_n^T * dZ_n : the reduction folded into one contraction of length n * pixels
+    n, P, CKK, O = 6, 400, 72, 40
+    col = oracle.fill((n, 1, P, CKK), 2201, "normal", 0.0, 1.0)
+    Wt = oracle.fill((1, 1, CKK, O), 2202, "normal", 0.0, 0.1)
+    dZ = oracle.fill((n, 1, P, O), 2203, "normal", 0.0, 1.0)
+    dcol, dW = dev(np.zeros_like(col)), dev(np.zeros_like(Wt))
+    nz.matmul_backward(dcol, dW, dev(col), dev(Wt), dev(dZ))
+    cr, wr, zr = (oracle.round_f16(t).astype(np.float64) for t in (col, Wt, dZ))
+    truth_dW = cr.reshape(n * P, CKK).T @ zr.reshape(n * P, O)
+    truth_dcol = zr.reshape(n * P, O) @ wr.reshape(CKK, O).T
+    check_tolerance(oracle, host(dW).reshape(CKK, O), truth_dW, "dW")
+    check_tolerance(oracle, host(dcol).reshape(n * P, CKK), truth_dcol, "dcol")
+
+
+def test_relu_backward_bit_exact(nz, oracle):
+    rng = np.random.default_rng(23)
+    for n in (1, 3, 4, 255, 4099):
+        x = rng.standard_normal(n).astype(np.float32)
+        x[:: 7] = 0.0
+        if n > 8:
+            x[1], x[2], x[3], x[5] = np.nan, -0.0, np.inf, -np.inf
+        dy = rng.standard_normal(n).astype(np.float32)
+        assert np.array_equal(host(nz.relu_backward(dev(x), dev(dy))), oracle.relu_backward(x, dy))
+
+
+def test_add_backward_bit_exact(nz, oracle):
+    rng = np.random.default_rng(29)
+    for s_in, s_out in [((3, 2, 4, 5), (3, 2, 4, 5)), ((1, 2, 4, 5), (3, 2, 4, 5)), ((3, 1, 4, 5), (3, 2, 4, 5)),
+                        ((1, 1, 30, 7), (4, 3, 30, 7)), ((1, 1, 64, 1), (5, 1, 64, 1))]:
+        din0, dout = ints(rng, s_in, -9, 10), ints(rng, s_out, -9, 10)
+        got = nz.add_backward(dev(din0), dev(dout))
+        assert np.array_equal(host(got), oracle.add_backward(din0, dout)), (s_in, s_out)
+    # float data: same summation order as the oracle -> identical bits
+    din0 = rng.standard_normal((1, 2, 9, 5)).astype(np.float32)
+    dout = rng.standard_normal((7, 2, 9, 5)).astype(np.float32)
+    assert np.array_equal(host(nz.add_backward(dev(din0), dev(dout))), oracle.add_backward(din0, dout))
+    with pytest.raises(nz.NzHipError):
+        nz.add_backward(dev(np.zeros((2, 1, 3, 3))), dev(np.zeros((3, 1, 3, 3))))
+
+
+IM2COL_CASES = [((2, 3, 4, 5), 3, 3, 1, 1), ((1, 1, 1, 1), 1, 1, 1, 0), ((2, 2, 7, 6), 3, 2, 2, 0),
+                ((1, 3, 8, 9), 2, 4, 2, 2), ((3, 1, 5, 5), 5, 5, 1, 2), ((2, 4, 6, 6), 1, 1, 3, 0),
+                ((2, 5, 33, 47), 3, 3, 1, 1), ((1, 2, 9, 9), 3, 3, 3, 1)]
+
+
+@pytest.mark.parametrize("shape,k_h,k_w,stride,pad", IM2COL_CASES)
+def test_im2col_backward_bit_exact(nz, oracle, shape, k_h, k_w, stride, pad):
+    rng = np.random.default_rng(31)
+    n, c, h, w = shape
+    Ho, Wo = (h + 2 * pad - k_h) // stride + 1, (w + 2 * pad - k_w) // stride + 1
+    dcol = ints(rng, (n, 1, Ho * Wo, c * k_h * k_w), -5, 6)
+    dx0 = ints(rng, shape, -9, 10)
+    got = nz.im2col_backward(dev(dx0), dev(dcol), k_h, k_w, stride, pad)
+    assert np.array_equal(host(got), oracle.im2col_backward(dx0, dcol, k_h, k_w, stride, pad))
+    # float data: the gather adds in the oracle's element order -> identical bits
+    dcol_f = rng.standard_normal(dcol.shape).astype(np.float32)
+    got = nz.im2col_backward(dev(np.zeros(shape, np.float32)), dev(dcol_f), k_h, k_w, stride, pad)
+    assert np.array_equal(host(got), oracle.im2col_backward(np.zeros(shape, np.float32), dcol_f, k_h, k_w, stride, pad))
+
+
+@pytest.mark.parametrize("n,c,h,w", [(2, 3, 4, 5), (1, 1, 1, 1), (3, 40, 9, 11), (2, 128, 16, 16), (1, 1, 50, 70)])
+def test_col2im_backward_bit_exact(nz, oracle, n, c, h, w):
+    rng = np.random.default_rng(37)
+    dy = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    got = host(nz.col2im_backward(dev(dy)))
+    assert np.array_equal(got, oracle.col2im_backward(dy))
+    assert np.array_equal(host(nz.col2im(dev(got), h, w)), dy)       # round trip with the forward transpose
