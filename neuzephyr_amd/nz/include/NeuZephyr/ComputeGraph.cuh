@@ -30,7 +30,11 @@ namespace nz::graph {
         void topologicalSort();                          // throws std::runtime_error("Graph has cycle")
         [[nodiscard]] bool isSorted() const;
         void forward();
-        void backward();                                 // not part of this path: throws std::logic_error
+        // Reverse pass over the sorted nodes (reference: src/ComputeGraph.cu:414-432); throws
+        // std::runtime_error if the graph is not sorted or does not have exactly one output node. If the
+        // last forward() fused node chains, the skipped intermediates are recomputed first.
+        void backward();
+        void zeroGrad() const;                           // src/ComputeGraph.cu:434-438
         [[nodiscard]] io::OutputNode* getOutputNode() const;   // throws std::runtime_error without exactly one output
         void setFusion(bool enabled);
         [[nodiscard]] size_t fusedGroupCount() const { return fusedGroups; }
@@ -43,6 +47,8 @@ namespace nz::graph {
         std::vector<io::OutputNode*> outputNodes;
         std::vector<Node*> sortedNodes;
         std::vector<std::function<void()>> plan;         // what forward() runs, in order
+        std::vector<Node*> fusedMembers;                 // nodes inside fused chains, in sorted order
+        bool intermediatesStale = false;                 // a fused forward() skipped their outputs
         bool fusion = true;
         bool planned = false;
         size_t fusedGroups = 0;

@@ -23,7 +23,7 @@ namespace nz {
         Model& operator=(const Model&) = delete;
 
         data::Tensor& forward();
-        void backward();                                 // not part of this path: throws std::logic_error
+        void backward();                                 // reverse pass of the graph (src/Model.cu:17-19)
         graph::ComputeGraph& graph() { return computeGraph; }
         // Parameters (weights, biases) in creation order, so that callers can inject values.
         [[nodiscard]] const std::vector<io::InputNode*>& parameters() const { return params; }

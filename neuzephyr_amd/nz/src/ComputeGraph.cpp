@@ -184,6 +184,9 @@ namespace nz::graph {
             }
         }
         fusedGroups = groups.size();
+        fusedMembers.clear();
+        for (Node* node : sortedNodes)
+            if (groupOf.count(node)) fusedMembers.push_back(node);
         planned = true;
     }
 
@@ -191,10 +194,24 @@ namespace nz::graph {
         if (!isSorted()) topologicalSort();
         if (!planned) buildPlan();
         for (auto& step : plan) step();
+        intermediatesStale = !fusedMembers.empty();
     }
 
     void ComputeGraph::backward() {
-        throw std::logic_error("ComputeGraph::backward: the backward pass is outside this build's path");
+        if (!isSorted()) throw std::runtime_error("Graph is not sorted");
+        if (outputNodes.empty()) throw std::runtime_error("No output node");
+        if (outputNodes.size() > 1) throw std::runtime_error("Multiple output nodes");
+        if (intermediatesStale) {
+            // node-level gradients read the outputs a fused chain never wrote: produce them now
+            for (Node* node : fusedMembers) node->forward();
+            intermediatesStale = false;
+        }
+        for (auto it = sortedNodes.rbegin(); it != sortedNodes.rend(); ++it) (*it)->backward();
+    }
+
+    void ComputeGraph::zeroGrad() const {
+        for (Node* node : nodes)
+            if (node->output && node->output->requiresGrad()) node->output->zeroGrad();
     }
 
     io::OutputNode* ComputeGraph::getOutputNode() const {

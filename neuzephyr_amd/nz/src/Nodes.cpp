@@ -9,12 +9,6 @@
 #include "nzhip.h"
 
 namespace nz::nodes {
-    namespace {
-        [[noreturn]] void noBackward(const char* node) {
-            throw std::logic_error(std::string(node) + "::backward: the backward pass is outside this build's path");
-        }
-    }
-
     void Node::print(std::ostream& os) const {
         os << "Node(" << type << ")";
         if (output) os << " shape " << output->shape();
@@ -57,7 +51,9 @@ namespace nz::nodes {
 
         void OutputNode::forward() { output = inputs[0]->output; }
 
-        void OutputNode::backward() { noBackward("OutputNode"); }
+        void OutputNode::backward() {                                  // src/Nodes.cu:62-66
+            if (inputs[0]->output->requiresGrad()) inputs[0]->output->fill(1, true);
+        }
     }
 
     namespace calc {
@@ -74,7 +70,10 @@ namespace nz::nodes {
         }
 
         void AddNode::forward() { tensorMatrixAdd(*output, *inputs[0]->output, *inputs[1]->output); }
-        void AddNode::backward() { noBackward("AddNode"); }
+        void AddNode::backward() {                                     // src/Nodes.cu:99-146
+            for (Node* in : inputs)
+                if (in->output->requiresGrad()) iAddBackward(in->output->grad(), output->grad(), in->output->shape(), output->shape());
+        }
 
         MatMulNode::MatMulNode(Node* input_left, Node* input_right) {
             const auto l = input_left->output->shape(), r = input_right->output->shape();
@@ -90,7 +89,13 @@ namespace nz::nodes {
         }
 
         void MatMulNode::forward() { GEMMTensorCore(*output, *inputs[0]->output, *inputs[1]->output); }
-        void MatMulNode::backward() { noBackward("MatMulNode"); }
+        void MatMulNode::backward() {                                  // src/Nodes.cu:169-182: dA += dC*B^T, dB += A^T*dC
+            Tensor& a = *inputs[0]->output;
+            Tensor& b = *inputs[1]->output;
+            if (!a.requiresGrad() && !b.requiresGrad()) return;
+            iMatMulBackward(a.requiresGrad() ? a.grad() : nullptr, b.requiresGrad() ? b.grad() : nullptr, a.data(), b.data(),
+                            output->grad(), a.shape(), b.shape(), output->shape());
+        }
 
         ReLUNode::ReLUNode(Node* input) {
             inputs.push_back(input);
@@ -99,7 +104,10 @@ namespace nz::nodes {
         }
 
         void ReLUNode::forward() { iRELU(output->data(), inputs[0]->output->data(), output->size()); }
-        void ReLUNode::backward() { noBackward("ReLUNode"); }
+        void ReLUNode::backward() {                                    // src/Nodes.cu:357-364
+            if (inputs[0]->output->requiresGrad())
+                iReLUBackward(inputs[0]->output->grad(), inputs[0]->output->data(), output->grad(), output->size());
+        }
 
         ReshapeNode::ReshapeNode(Node* input, const Tensor::shape_type& newShape) : newShape(newShape) {
             if (input->output->shape().size() != newShape.size()) {
@@ -113,7 +121,10 @@ namespace nz::nodes {
         void ReshapeNode::forward() {
             NZ_CHECK(nzhip_memcpy_d2d(output->data(), inputs[0]->output->data(), output->size() * sizeof(Tensor::value_type)));
         }
-        void ReshapeNode::backward() { noBackward("ReshapeNode"); }
+        void ReshapeNode::backward() {                                 // src/Nodes.cu:565-571
+            if (inputs[0]->output->requiresGrad())
+                NZ_CHECK(nzhip_memcpy_d2d(inputs[0]->output->grad(), output->grad(), output->size() * sizeof(Tensor::value_type)));
+        }
 
         Img2ColNode::Img2ColNode(Node* input, const Tensor::size_type kernelHeight, const Tensor::size_type kernelWidth,
                                  const Tensor::size_type stride, const Tensor::size_type padding)
@@ -134,7 +145,12 @@ namespace nz::nodes {
             iImg2col(output->data(), inputs[0]->output->data(), outputHeight, outputWidth, s[1], kernelHeight, kernelWidth,
                      stride, padding, s[2], s[3], s[0]);
         }
-        void Img2ColNode::backward() { noBackward("Img2ColNode"); }
+        void Img2ColNode::backward() {                                 // src/Nodes.cu:632-640
+            if (!inputs[0]->output->requiresGrad()) return;
+            const auto s = inputs[0]->output->shape();
+            iImg2colBackward(inputs[0]->output->grad(), output->grad(), outputHeight, outputWidth, s[1], kernelHeight,
+                             kernelWidth, stride, padding, s[2], s[3], s[0]);
+        }
 
         Col2ImgNode::Col2ImgNode(Node* input, const Tensor::size_type outputHeight, const Tensor::size_type outputWidth)
             : outputHeight(outputHeight), outputWidth(outputWidth), outputChannels(input->output->shape()[3]) {
@@ -150,6 +166,10 @@ namespace nz::nodes {
             iCol2img(output->data(), inputs[0]->output->data(), outputHeight, outputWidth, outputChannels,
                      inputs[0]->output->shape()[0]);
         }
-        void Col2ImgNode::backward() { noBackward("Col2ImgNode"); }
+        void Col2ImgNode::backward() {                                 // src/Nodes.cu:660-665
+            if (inputs[0]->output->requiresGrad())
+                iCol2imgBackward(inputs[0]->output->grad(), output->grad(), outputHeight, outputWidth, outputChannels,
+                                 inputs[0]->output->shape()[0]);
+        }
     }
 }

@@ -53,6 +53,47 @@ namespace nz::data {
         NZ_CHECK(nzhip_col2im(out, in, H_out, W_out, C_out, batches, nzhip_default_stream()));
     }
 
+    void iGEMMBackward(float* A, float* B, float* C, const Dimension& shapeA, const Dimension& shapeB,
+                       const Dimension& shapeC) {
+        size_t sa[4], sb[4], sc[4];
+        dims4(shapeA, sa);
+        dims4(shapeB, sb);
+        dims4(shapeC, sc);
+        NZ_CHECK(nzhip_gemm_backward(A, B, C, sa, sb, sc, nzhip_default_stream()));
+    }
+
+    void iImg2colBackward(float* out, float* in, const size_t H_out, const size_t W_out, const size_t C,
+                          const size_t K_h, const size_t K_w, const size_t stride, const size_t pad, const size_t H_in,
+                          const size_t W_in, const size_t batch) {
+        NZ_CHECK(nzhip_im2col_backward(out, in, H_out, W_out, C, K_h, K_w, stride, pad, H_in, W_in, batch,
+                                       nzhip_default_stream()));
+    }
+
+    void iCol2imgBackward(float* out, float* in, const size_t H_out, const size_t W_out, const size_t C_out,
+                          const size_t batches) {
+        NZ_CHECK(nzhip_col2im_backward(out, in, H_out, W_out, C_out, batches, nzhip_default_stream()));
+    }
+
+    void iMatMulBackward(float* dA, float* dB, float* A, float* B, float* dC, const Dimension& shapeA,
+                         const Dimension& shapeB, const Dimension& shapeC) {
+        size_t sa[4], sb[4], sc[4];
+        dims4(shapeA, sa);
+        dims4(shapeB, sb);
+        dims4(shapeC, sc);
+        NZ_CHECK(nzhip_matmul_backward(dA, dB, A, B, dC, sa, sb, sc, nzhip_default_stream()));
+    }
+
+    void iReLUBackward(float* dx, float* x, float* dy, const unsigned long long size) {
+        NZ_CHECK(nzhip_relu_backward(dx, x, dy, static_cast<size_t>(size), nzhip_default_stream()));
+    }
+
+    void iAddBackward(float* din, float* dout, const Dimension& shapeIn, const Dimension& shapeOut) {
+        size_t si[4], so[4];
+        dims4(shapeIn, si);
+        dims4(shapeOut, so);
+        NZ_CHECK(nzhip_add_backward(din, dout, si, so, nzhip_default_stream()));
+    }
+
     void iConv2dForward(float* y, float* x, float* w, float* bias, const size_t N, const size_t C, const size_t H,
                         const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
                         const size_t pad, const size_t weightBatch, const long long biasPixelStride,
