@@ -27,7 +27,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
-                    choices=["gemm8192", "gemm_batched", "linear", "gemv", "ragged", "conv_a", "conv_b", "copy"])
+                    choices=["gemm8192", "gemm_batched", "linear", "linear_bwd", "conv_dw", "gemv", "ragged", "conv_a", "conv_b",
+                             "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary (conv / linear) measurements")
     ap.add_argument("--no-verify", action="store_true")
@@ -107,6 +108,57 @@ def make_workload(name, orc, capi):
 
         return Workload(name, 2.0 * Nb * IN * OUT, 4.0 * (Nb * IN + IN * OUT + OUT + Nb * OUT), run, verify, "mfma",
                         "Linear X[4096,1024] W[4096,1024]^T + bias, ReLU"), None
+    if name == "linear_bwd":
+        # backward of Model::Linear at the L config: W[1,1,OUT,IN] * x[n,1,IN,1] -> dW += dY^T X, dx += dY W
+        Nb, IN, OUT = 4096, 1024, 4096
+        X = orc.fill((Nb, 1, IN, 1), 2, "normal", 0.0, 1.0)
+        bound = float(np.sqrt(6.0 / IN))
+        Wt = orc.fill((1, 1, OUT, IN), 1002, "uniform", -bound, bound)
+        dY = orc.fill((Nb, 1, OUT, 1), 3002, "normal", 0.0, 1.0)
+        Xd, Wd, dYd = dev(X), dev(Wt), dev(dY)
+        dW, dX = torch.zeros((1, 1, OUT, IN), device="cuda"), torch.zeros((Nb, 1, IN, 1), device="cuda")
+
+        def run():
+            capi.matmul_backward(dW, dX, Wd, Xd, dYd)
+
+        def verify():
+            # gradients accumulate over the timed calls: measure one call from zero
+            dW.zero_(); dX.zero_()
+            run()
+            dyr, xr, wr = (orc.round_f16(t).astype(np.float64) for t in (dY, X, Wt))
+            t_dW = dyr.reshape(Nb, OUT)[:, :128].T @ xr.reshape(Nb, IN)
+            t_dX = dyr.reshape(Nb, OUT)[:128] @ wr.reshape(OUT, IN)
+            a = tolerance(orc, dW.reshape(OUT, IN)[:128].cpu().numpy(), t_dW, name + " dW")
+            b = tolerance(orc, dX.reshape(Nb, IN)[:128].cpu().numpy(), t_dX, name + " dx")
+            return {k: max(a[k], b[k]) for k in a}
+
+        # operands once, gradients read and written ("+=")
+        return Workload(name, 2 * 2.0 * Nb * IN * OUT, 4.0 * (Nb * OUT + Nb * IN + OUT * IN + 2 * OUT * IN + 2 * Nb * IN),
+                        run, verify, "mfma", "Linear backward: dW[4096,1024] += dY^T X, dx[4096,1024] += dY W (n=4096)"), None
+    if name == "conv_dw":
+        # weight gradient of the CA convolution from its column matrix: dW[576,128] += sum_n col_n^T dZ_n,
+        # the batch reduction folded into one contraction of length 16 * 16384
+        N, P, CKK, O = 16, 128 * 128, 64 * 9, 128
+        col = orc.fill((N, 1, P, CKK), 4004, "normal", 0.0, 1.0)
+        dZ = orc.fill((N, 1, P, O), 4005, "normal", 0.0, 1.0)
+        Wr = torch.zeros((1, 1, CKK, O), device="cuda")
+        cold, dZd = dev(col), dev(dZ)
+        dWd = torch.zeros((1, 1, CKK, O), device="cuda")
+
+        def run():
+            capi.matmul_backward(None, dWd, cold, Wr, dZd)
+
+        def verify():
+            dWd.zero_()
+            run()
+            # every output needs the whole contraction: fp64 truth for the first 48 rows of dW
+            cr = orc.round_f16(col).reshape(N * P, CKK)[:, :48].astype(np.float64)
+            zr = orc.round_f16(dZ).reshape(N * P, O).astype(np.float64)
+            truth = cr.T @ zr
+            return tolerance(orc, dWd.reshape(CKK, O)[:48].cpu().numpy(), truth, name)
+
+        return Workload(name, 2.0 * N * P * CKK * O, 4.0 * (N * P * CKK + N * P * O + 2 * CKK * O), run, verify, "hbm",
+                        "Conv weight gradient: dW[576,128] += col[16x16384,576]^T dZ[16x16384,128]"), None
     if name == "gemv":
         a = orc.fill((1, 4096), 4, "uniform", -1.0, 1.0)
         Bm = orc.fill((4096, 4096), 1004, "uniform", -1.0, 1.0)
@@ -247,7 +299,7 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched"):
+        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched", "linear_bwd", "conv_dw"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)
             ms2, _ = time_steps(w2, max(10, args.steps // 2), max(3, args.warmup // 2))

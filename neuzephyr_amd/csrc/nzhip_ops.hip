@@ -207,6 +207,21 @@ __global__ __launch_bounds__(256) void fill_bias_act_kernel(nzhip_gemm_desc d) {
     d.C[i * d.c_stride_n + j * d.c_stride_c + m * d.ldc + n] = x;
 }
 
+// ---- split-k for few-tile, long-contraction GEMMs ---------------------------------------------
+// C = act(bias + sum over chunks s of P[s]), chunks added in ascending order by one thread per
+// element, so the result does not depend on scheduling.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(nzhip_gemm_desc d, const float* __restrict__ P, int S) {
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long mn = d.M * d.N;
+    if (t >= mn) return;
+    const long m = t / d.N, n = t % d.N;
+    float x = P[t];
+    for (int s = 1; s < S; s++) x += P[(long)s * mn + t];
+    if (d.bias) x += d.bias[m * d.bias_stride_row + n * d.bias_stride_col];
+    if (d.activation == NZHIP_ACT_RELU) x = x > 0.f ? x : 0.f;
+    d.C[m * d.ldc + n] = x;
+}
+
 }  // namespace nzhip
 
 using namespace nzhip;
@@ -225,6 +240,44 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
         return check_launch("fill_bias_act_kernel");
     }
     if (gemm_skinny_applicable(d)) return gemm_skinny_dispatch(d, s);
+    // One matrix with few output tiles and a long contraction (weight gradients: K = batch x pixels):
+    // cut K into chunks that run as a batch into a workspace, then add the chunks in order.
+    if (d.batch_n * d.batch_c == 1 && d.K >= 4096) {
+        const int cus = device_cu_count();
+        const int64_t tiles = ((d.M + 127) / 128) * ((d.N + 127) / 128);
+        if (tiles * 2 <= cus) {
+            int64_t S = (2 * cus + tiles - 1) / tiles;
+            if (S > d.K / 1024) S = d.K / 1024;
+            if (S > 1024) S = 1024;
+            const int64_t Kc = ((d.K + S - 1) / S + 31) / 32 * 32;          // chunk length, whole 32-wide k tiles
+            const int64_t full = d.K / Kc, rem = d.K - full * Kc;
+            const int parts = (int)(full + (rem ? 1 : 0));
+            if (full >= 2) {
+                float* P = nullptr;
+                if (int rc = workspace_alloc(reinterpret_cast<void**>(&P), (size_t)parts * d.M * d.N * sizeof(float), s)) return rc;
+                const int64_t a_step = d.a_layout == NZHIP_LAYOUT_ROW ? Kc : Kc * d.lda;   // next chunk of A / B
+                const int64_t b_step = d.b_layout == NZHIP_LAYOUT_ROW ? Kc * d.ldb : Kc;
+                nzhip_gemm_desc g = d;
+                g.C = P; g.ldc = d.N; g.K = Kc;
+                g.batch_n = 1; g.batch_c = full;
+                g.a_stride_c = a_step; g.b_stride_c = b_step; g.c_stride_c = d.M * d.N;
+                g.bias = nullptr; g.activation = NZHIP_ACT_NONE;
+                int rc = nzhip_gemm(&g, stream);
+                if (rc == NZHIP_OK && rem) {
+                    g.A = d.A + full * a_step; g.B = d.B + full * b_step; g.C = P + full * d.M * d.N;
+                    g.K = rem; g.batch_c = 1;
+                    g.a_stride_c = g.b_stride_c = g.c_stride_c = 0;
+                    rc = nzhip_gemm(&g, stream);
+                }
+                if (rc == NZHIP_OK) {
+                    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((d.M * d.N + 255) / 256)), dim3(256), 0, s, d, P, parts);
+                    rc = check_launch("splitk_reduce_kernel");
+                }
+                const int rc2 = workspace_free(P, s);
+                return rc ? rc : rc2;
+            }
+        }
+    }
     // NZHIP_GEMM_ROUTE=fused|h16 overrides the route choice (benchmarking only).
     static const char* route = getenv("NZHIP_GEMM_ROUTE");
     const bool force_fused = route && route[0] == 'f', force_h16 = route && route[0] == 'h';

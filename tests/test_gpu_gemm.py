@@ -93,6 +93,24 @@ def test_skinny_products_are_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans
     assert np.array_equal(got, expect)
 
 
+SPLITK = [(130, 9000, 70), (576, 16384, 128), (64, 4096, 64), (33, 20001, 300), (128, 8192, 129)]
+
+
+@pytest.mark.parametrize("M,K,N", SPLITK)
+@pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
+def test_long_contractions_with_few_tiles_are_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans):
+    # few output tiles and K >= 4096: the contraction is cut into chunks that are added in order;
+    # a full [M,N] bias and ReLU are applied once, after the last chunk
+    rng = np.random.default_rng(M * 13 + K + N * 5)
+    A = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, size=(K, N)).astype(np.float32)
+    bias = rng.integers(-50, 51, size=(M, N)).astype(np.float32)
+    expect = np.maximum((A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32) + bias, 0)
+    got = host(nz.gemm(dev(A.T if a_trans else A), dev(B.T if b_trans else B), a_trans=a_trans, b_trans=b_trans,
+                       bias=dev(bias), bias_strides=(N, 1), relu=True))
+    assert np.array_equal(got, expect)
+
+
 def test_skinny_batched_linear_single_sample(nz, oracle):
     # one sample through Model::Linear: W[1,1,OUT,IN] x[1,1,IN,1]
     OUT, IN = 1000, 515
