@@ -11,6 +11,8 @@
 // to fp32 summation order.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "nzhip_internal.h"
 
 namespace nzhip {
@@ -31,18 +33,19 @@ typedef float floatx2 __attribute__((ext_vector_type(2)));
 // and rows/columns beyond the operand are zero.
 constexpr int CVT_ROWS = 256, CVT_K = 32, CVT_BLOCK_BYTES = CVT_ROWS * CVT_K * 2;
 
-// Physical LDS row of logical tile row r for a 2x2 wave grid over a 256-row tile (wave tile
-// 128 rows = 4 MFMA blocks, interleaved so that one lane ends up with 4 adjacent columns).
-__device__ __forceinline__ int phys_row_of(int r) {
-    const int w = r >> 7, l = r & 127;
-    return (w * 4 + (l & 3)) * 32 + (l >> 2);
+// Physical LDS row of logical tile row r when a wave owns FR consecutive 32-row MFMA blocks of the
+// 256-row tile (FR = 4: two waves along that dimension, FR = 2: four). The rows of a wave are
+// interleaved over its blocks so that one lane ends up with FR adjacent rows / columns.
+__device__ __forceinline__ int phys_row_of(int r, int fr) {
+    const int tr = 32 * fr, w = r / tr, l = r % tr;
+    return (w * fr + (l % fr)) * 32 + (l / fr);
 }
 
 // K_CONTIG: source element (r, k) at src[r*ld + k]; otherwise at src[k*ld + r].
 template <bool K_CONTIG>
 __global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ dst, const float* __restrict__ src,
                                                         int R, int K, int nkt, long ld, long src_batch,
-                                                        long dst_batch, int vec) {
+                                                        long dst_batch, int vec, int fr) {
     __shared__ __attribute__((aligned(16))) char img[CVT_BLOCK_BYTES];
     const int kt = blockIdx.x, rb = blockIdx.y;
     const float* s = src + (long)blockIdx.z * src_batch;
@@ -66,7 +69,7 @@ __global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ d
                 }
             }
             half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-            const int pr = phys_row_of(lr);
+            const int pr = phys_row_of(lr, fr);
             const int pos = (k4 >> 1) ^ ((pr >> 2) & 3);
             *reinterpret_cast<half4_t*>(img + pr * 64 + pos * 16 + (k4 & 1) * 8) = h;
         }
@@ -89,7 +92,7 @@ __global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ d
             }
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int pr = phys_row_of(lr + e);
+                const int pr = phys_row_of(lr + e, fr);
                 const int pos = (kk >> 3) ^ ((pr >> 2) & 3);
                 *reinterpret_cast<_Float16*>(img + pr * 64 + pos * 16 + (kk & 7) * 2) = (_Float16)v[e];
             }
@@ -136,7 +139,7 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC
 // 128-bit fragment read touches on 16 different 16-byte bank groups.
 template <int BM, int BN, int WM, int WN, int NSTAGE>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_h16_kernel(const H16Args p) {
-    static_assert(BM == CVT_ROWS && BN == CVT_ROWS && WM == 2 && WN == 2, "must match the workspace block image");
+    static_assert(BM == CVT_ROWS && BN == CVT_ROWS, "must match the workspace block image");
     constexpr int BK = CVT_K, ROWB = 64;
     constexpr int NW = WM * WN;
     constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
@@ -344,7 +347,7 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
 
     const int nkt = (int)(Kp / BK);
     auto convert = [&](_Float16* dst, const float* src, long R, long Rp, bool k_contig, long ld, long nb, long cb,
-                       long sn, long sc, size_t elems) -> int {
+                       long sn, long sc, size_t elems, int fr) -> int {
         for (long i = 0; i < nb; i++) {
             // the c axis of one n is a plain strided batch -> one launch per n
             const float* sp = src + i * sn;
@@ -353,16 +356,21 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
             dim3 grid((unsigned)nkt, (unsigned)(Rp / CVT_ROWS), (unsigned)cb);
             if (k_contig)
                 hipLaunchKernelGGL(cvt_block_kernel<true>, grid, dim3(256), 0, s, dp, sp, (int)R, (int)d.K, nkt, ld, sc,
-                                   (long)elems, vec);
+                                   (long)elems, vec, fr);
             else
                 hipLaunchKernelGGL(cvt_block_kernel<false>, grid, dim3(256), 0, s, dp, sp, (int)R, (int)d.K, nkt, ld, sc,
-                                   (long)elems, vec);
+                                   (long)elems, vec, fr);
         }
         hipError_t e = hipGetLastError();
         return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "fp16 rounding pass launch");
     };
-    int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems);
-    if (rc == NZHIP_OK) rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems);
+    // Wave grid of the GEMM kernel: WM x 2 waves, each owning 256/WM rows and 128 columns of the tile.
+    // 2 x 2 (one wave per SIMD, 256 accumulators) measures 1-2 % faster than 4 x 2 on 8192^3;
+    // NZHIP_H16_WAVES=8 selects the latter (benchmarking only).
+    static const char* waves_env = getenv("NZHIP_H16_WAVES");
+    const int wm_waves = (waves_env && atoi(waves_env) == 8) ? 4 : 2;
+    int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, 8 / wm_waves);
+    if (rc == NZHIP_OK) rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems, 4);
     if (rc == NZHIP_OK) {
         H16Args a;
         a.A = Ah;
@@ -393,12 +401,12 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
         a.tiles_n = (int)(Np / BN);
         a.group_m = 4;
         constexpr size_t lds_bytes = (size_t)NSTAGE * (BM + BN) * 64;
-        auto kfn = gemm_h16_kernel<BM, BN, 2, 2, NSTAGE>;
+        void (*kfn)(const H16Args) = wm_waves == 4 ? gemm_h16_kernel<BM, BN, 4, 2, NSTAGE> : gemm_h16_kernel<BM, BN, 2, 2, NSTAGE>;
         if (rc == NZHIP_OK)
             rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(gemm_h16)");
         if (rc == NZHIP_OK) {
             dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(d.batch_n * d.batch_c));
-            hipLaunchKernelGGL(kfn, grid, dim3(256), lds_bytes, s, a);
+            hipLaunchKernelGGL(kfn, grid, dim3(wm_waves * 2 * 64), lds_bytes, s, a);
             hipError_t e = hipGetLastError();
             if (e != hipSuccess) rc = set_hip_error(e, "gemm_h16 kernel launch");
         }
