@@ -159,6 +159,26 @@ int nzhip_im2col_backward(float* dx, const float* dcol, size_t H_out, size_t W_o
 int nzhip_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_out, size_t C_out,
                           size_t batches, void* stream);
 
+/* ---- fp32-exact matmul and optimizer steps ---------------------------------- */
+/* nz::data::tensorGeneralMatrixMul / iGeneralMatrixMul behind Tensor::operator*
+ * (include/NeuZephyr/TensorOperations.cuh:998-1019, src/TensorOperations.cu:104-110; GeneralMatrixMulKernel,
+ * src/OperationKernels.cu:65-101): C[n][c] = A[n or 0][c or 0] * B[n or 0][c or 0] with NO rounding of
+ * the operands, fp32 FMA accumulation in ascending k. M = A.h, N = B.w, K = A.w = B.h. */
+int nzhip_matmul_f32(const float* A, const float* B, float* C, const size_t shapeA[4],
+                     const size_t shapeB[4], const size_t shapeC[4], void* stream);
+
+/* opt::SGD::step (src/Optimizer.cu:14-19; StochasticGradientDescentKernel, src/OperationKernels.cu:634-640):
+ * data -= lr * grad. */
+int nzhip_sgd_step(float* data, const float* grad, float lr, size_t n, void* stream);
+
+/* opt::Adam::step (src/Optimizer.cu:86-102; AdamKernel, src/OperationKernels.cu:753-766), t = 1, 2, ...:
+ *   m = beta1*m + (1-beta1)*g;  v = beta2*v + (1-beta2)*g*g;
+ *   data -= lr * (m / (1-beta1^t)) / (sqrt(v / (1-beta2^t)) + eps)
+ * beta^t is evaluated with powf; the reference kernel uses CUDA's approximate __powf, so the last
+ * bits of the bias corrections are not pinned by it (its own test compares against std::pow). */
+int nzhip_adam_step(float* data, float* m, float* v, const float* grad, float lr, float beta1,
+                    float beta2, float eps, int t, size_t n, void* stream);
+
 /* ---- runtime: device allocator + stream manager -------------------------- */
 /* Replace cuStrm::StreamManager<float> (include/NeuZephyr/StreamManager.cuh:131-911) and
  * EventPool (EventPool.cuh:165-457).  One ordered compute stream carries every kernel and

@@ -10,7 +10,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libnzhip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SOURCES = ["nzhip_gemm.hip", "nzhip_gemm_h16.hip", "nzhip_skinny.hip", "nzhip_conv.hip", "nzhip_ops.hip", "nzhip_runtime.cpp"]
+SOURCES = ["nzhip_gemm.hip", "nzhip_gemm_h16.hip", "nzhip_skinny.hip", "nzhip_conv.hip", "nzhip_ops.hip", "nzhip_fp32.hip",
+           "nzhip_runtime.cpp"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=default",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

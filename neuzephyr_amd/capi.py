@@ -18,7 +18,7 @@ EXPORTS = [
     "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_tensorcore_gemm",
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
-    "nzhip_im2col_backward", "nzhip_col2im_backward",
+    "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
@@ -81,6 +81,9 @@ def load() -> C.CDLL:
     lib.nzhip_add_backward.argtypes = [vp, vp, shape, shape, vp]
     lib.nzhip_im2col_backward.argtypes = [vp, vp] + [sz] * 10 + [vp]
     lib.nzhip_col2im_backward.argtypes = [vp, vp, sz, sz, sz, sz, vp]
+    lib.nzhip_matmul_f32.argtypes = [vp, vp, vp, shape, shape, shape, vp]
+    lib.nzhip_sgd_step.argtypes = [vp, vp, C.c_float, sz, vp]
+    lib.nzhip_adam_step.argtypes = [vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, sz, vp]
     lib.nzhip_default_stream.restype = vp
     lib.nzhip_malloc.argtypes = [C.POINTER(vp), sz]
     lib.nzhip_free_async.argtypes = [vp]
@@ -285,3 +288,27 @@ def col2im_backward(dy, stream=None):
     out = torch.empty((N, 1, Ho * Wo, O), dtype=torch.float32, device=dy.device)
     check(lib.nzhip_col2im_backward(_dev(out), _dev(dy), Ho, Wo, O, N, _stream_handle(stream)))
     return out
+
+
+# ---- fp32-exact matmul and optimizer steps ---------------------------------------------------------
+def matmul_f32(A, B, out=None, stream=None):
+    import torch
+    lib = load()
+    so = (max(A.shape[0], B.shape[0]), max(A.shape[1], B.shape[1]), A.shape[2], B.shape[3])
+    if out is None:
+        out = torch.empty(so, dtype=torch.float32, device=A.device)
+    check(lib.nzhip_matmul_f32(_dev(A), _dev(B), _dev(out), shape4(A.shape), shape4(B.shape), shape4(so), _stream_handle(stream)))
+    return out
+
+
+def sgd_step(data, grad, lr, stream=None):
+    lib = load()
+    check(lib.nzhip_sgd_step(_dev(data), _dev(grad), lr, data.numel(), _stream_handle(stream)))
+    return data
+
+
+def adam_step(data, m, v, grad, lr, beta1, beta2, eps, t, stream=None):
+    lib = load()
+    check(lib.nzhip_adam_step(_dev(data), _dev(m), _dev(v), _dev(grad), lr, beta1, beta2, eps, t, data.numel(),
+                              _stream_handle(stream)))
+    return data, m, v

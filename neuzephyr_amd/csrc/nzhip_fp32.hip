@@ -1,0 +1,210 @@
+// fp32-exact pieces next to the fp16 path: the matmul behind Tensor::operator* (no rounding of the
+// operands, fp32 FMA accumulation in ascending k, reference: GeneralMatrixMulKernel,
+// src/OperationKernels.cu:65-101) and the optimizer steps that close a training iteration
+// (StochasticGradientDescentKernel :634-640, AdamKernel :753-766).
+#include <hip/hip_runtime.h>
+
+#include "nzhip_internal.h"
+
+namespace nzhip {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, what);
+}
+
+// ---- fp32 matmul --------------------------------------------------------------------------------
+// 128 x 128 output tile per workgroup, 16 x 16 threads with an 8 x 8 register block each, k in
+// steps of 16 through LDS (A stored k-major so that both fragment reads are contiguous). Every
+// output is one chain of FMAs in ascending k, the same arithmetic as a scalar loop
+// `sum = fma(a[k], b[k], sum)`, so integer data and the CPU restatement match bit for bit.
+struct F32Args {
+    const float* A;
+    const float* B;
+    float* C;
+    int M, N, K;
+    long a_sn, a_sc, b_sn, b_sc, c_sn, c_sc;
+    int batch_c;
+    int vec_a, vec_b;
+};
+
+constexpr int F32_BM = 128, F32_BN = 128, F32_BK = 16;
+
+__global__ __launch_bounds__(256) void matmul_f32_kernel(const F32Args p) {
+    __shared__ __attribute__((aligned(16))) float As[2][F32_BK][F32_BM + 4];   // [k][m]
+    __shared__ __attribute__((aligned(16))) float Bs[2][F32_BK][F32_BN + 4];   // [k][n]
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int m0 = blockIdx.y * F32_BM, n0 = blockIdx.x * F32_BN;
+    const int bi = blockIdx.z / p.batch_c, bj = blockIdx.z % p.batch_c;
+    const float* __restrict__ A = p.A + bi * p.a_sn + bj * p.a_sc;
+    const float* __restrict__ B = p.B + bi * p.b_sn + bj * p.b_sc;
+    float* __restrict__ C = p.C + bi * p.c_sn + bj * p.c_sc;
+
+    // staging: A tile 128 x 16 = 512 float4 along k (2 per thread); B tile 16 x 128 = 512 float4 along n
+    floatx4 ra[2], rb[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int q = tid + h * 256;
+            {   // A: row m = q / 4, k quad = q % 4
+                const int m = m0 + (q >> 2), k = k0 + (q & 3) * 4;
+                floatx4 v = {0.f, 0.f, 0.f, 0.f};
+                if (m < p.M) {
+                    const float* s = A + (long)m * p.K + k;
+                    if (p.vec_a && k + 4 <= p.K) v = *reinterpret_cast<const floatx4*>(s);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) if (k + e < p.K) v[e] = s[e];
+                    }
+                }
+                ra[h] = v;
+            }
+            {   // B: row k = q / 32, n quad = q % 32
+                const int k = k0 + (q >> 5), n = n0 + (q & 31) * 4;
+                floatx4 v = {0.f, 0.f, 0.f, 0.f};
+                if (k < p.K) {
+                    const float* s = B + (long)k * p.N + n;
+                    if (p.vec_b && n + 4 <= p.N) v = *reinterpret_cast<const floatx4*>(s);
+                    else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) if (n + e < p.N) v[e] = s[e];
+                    }
+                }
+                rb[h] = v;
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int q = tid + h * 256;
+#pragma unroll
+            for (int e = 0; e < 4; e++) As[buf][(q & 3) * 4 + e][q >> 2] = ra[h][e];
+            *reinterpret_cast<floatx4*>(&Bs[buf][q >> 5][(q & 31) * 4]) = rb[h];
+        }
+    };
+
+    float acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc[i][j] = 0.f;
+
+    const int nk = (p.K + F32_BK - 1) / F32_BK;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt++) {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) fetch((kt + 1) * F32_BK);
+#pragma unroll
+        for (int k = 0; k < F32_BK; k++) {
+            // rows ty*4..+3 and 64+ty*4..+3, columns tx*4..+3 and 64+tx*4..+3
+            const floatx4 a0 = *reinterpret_cast<const floatx4*>(&As[buf][k][ty * 4]);
+            const floatx4 a1 = *reinterpret_cast<const floatx4*>(&As[buf][k][64 + ty * 4]);
+            const floatx4 b0 = *reinterpret_cast<const floatx4*>(&Bs[buf][k][tx * 4]);
+            const floatx4 b1 = *reinterpret_cast<const floatx4*>(&Bs[buf][k][64 + tx * 4]);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float a = i < 4 ? a0[i] : a1[i - 4];
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc[i][j] = __builtin_fmaf(a, j < 4 ? b0[j] : b1[j - 4], acc[i][j]);
+            }
+        }
+        if (kt + 1 < nk) stash(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int m = m0 + (i < 4 ? ty * 4 + i : 64 + ty * 4 + i - 4);
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int n = n0 + (j < 4 ? tx * 4 + j : 64 + tx * 4 + j - 4);
+            if (n < p.N) C[(long)m * p.N + n] = acc[i][j];
+        }
+    }
+}
+
+// ---- optimizer steps ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void sgd_kernel(float* __restrict__ data, const float* __restrict__ grad, float lr,
+                                                  long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) data[i] -= lr * grad[i];
+}
+
+// bias corrections 1 - beta^t are computed once on the host (in fp32, like the kernel of the reference)
+__global__ __launch_bounds__(256) void adam_kernel(float* __restrict__ data, float* __restrict__ m,
+                                                   float* __restrict__ v, const float* __restrict__ grad, float lr,
+                                                   float beta1, float beta2, float eps, float corr1, float corr2,
+                                                   long n) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float g = grad[i];
+    const float m_temp = m[i] * beta1 + g * (1 - beta1);
+    const float v_temp = v[i] * beta2 + g * g * (1 - beta2);
+    const float m_modified = m_temp / corr1;
+    const float v_modified = v_temp / corr2;
+    data[i] -= lr * m_modified / (sqrtf(v_modified) + eps);
+    m[i] = m_temp;
+    v[i] = v_temp;
+}
+
+}  // namespace nzhip
+
+using namespace nzhip;
+
+extern "C" {
+
+int nzhip_matmul_f32(const float* A, const float* B, float* C, const size_t sA[4], const size_t sB[4],
+                     const size_t sC[4], void* stream) {
+    if (!A || !B || !C || !sA || !sB || !sC) return set_error(NZHIP_E_INVALID, "nzhip_matmul_f32: null argument");
+    for (int i = 0; i < 2; i++)
+        if (sA[i] != sB[i] && sA[i] != 1 && sB[i] != 1) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
+    if (sA[3] != sB[2]) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
+    const size_t M = sA[2], N = sB[3], K = sA[3];
+    const size_t bn = sC[0], bc = sC[1];
+    if (M == 0 || N == 0 || bn == 0 || bc == 0) return NZHIP_OK;
+    if (M > 0x3fffffff || N > 0x3fffffff || K > 0x3fffffff || bn * bc > 65535 || (M + F32_BM - 1) / F32_BM > 65535)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_matmul_f32: extent too large");
+    F32Args a;
+    a.A = A; a.B = B; a.C = C;
+    a.M = (int)M; a.N = (int)N; a.K = (int)K;
+    a.a_sn = sA[0] > 1 ? (long)(sA[1] * sA[2] * sA[3]) : 0;      // TensorOperations.cuh:1006-1014
+    a.a_sc = sA[1] > 1 ? (long)(sA[2] * sA[3]) : 0;
+    a.b_sn = sB[0] > 1 ? (long)(sB[1] * sB[2] * sB[3]) : 0;
+    a.b_sc = sB[1] > 1 ? (long)(sB[2] * sB[3]) : 0;
+    a.c_sn = (long)(sC[1] * sC[2] * sC[3]);
+    a.c_sc = (long)(sC[2] * sC[3]);
+    a.batch_c = (int)bc;
+    a.vec_a = aligned16(A) && (K % 4 == 0);
+    a.vec_b = aligned16(B) && (N % 4 == 0);
+    dim3 grid((unsigned)((N + F32_BN - 1) / F32_BN), (unsigned)((M + F32_BM - 1) / F32_BM), (unsigned)(bn * bc));
+    hipLaunchKernelGGL(matmul_f32_kernel, grid, dim3(256), 0, as_stream(stream), a);
+    return check_launch("matmul_f32_kernel");
+}
+
+int nzhip_sgd_step(float* data, const float* grad, float lr, size_t n, void* stream) {
+    if ((!data || !grad) && n) return set_error(NZHIP_E_INVALID, "nzhip_sgd_step: null pointer");
+    if (n == 0) return NZHIP_OK;
+    hipLaunchKernelGGL(sgd_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), data, grad, lr, (long)n);
+    return check_launch("sgd_kernel");
+}
+
+int nzhip_adam_step(float* data, float* m, float* v, const float* grad, float lr, float beta1, float beta2, float eps,
+                    int t, size_t n, void* stream) {
+    if ((!data || !m || !v || !grad) && n) return set_error(NZHIP_E_INVALID, "nzhip_adam_step: null pointer");
+    if (t < 1) return set_error(NZHIP_E_INVALID, "nzhip_adam_step: the step count starts at 1");
+    if (n == 0) return NZHIP_OK;
+    const float corr1 = 1.0f - powf(beta1, (float)t), corr2 = 1.0f - powf(beta2, (float)t);
+    hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), data, m, v, grad, lr,
+                       beta1, beta2, eps, corr1, corr2, (long)n);
+    return check_launch("adam_kernel");
+}
+
+}  // extern "C"

@@ -331,7 +331,7 @@ bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
     return flops / cvt_bytes >= 512.0;
 }
 
-int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
+int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
     constexpr int BM = 256, BN = 256, BK = 32, NSTAGE = 4;
     const long Mp = round_up(d.M, BM), Np = round_up(d.N, BN), Kp = round_up(d.K, BK);
     const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
@@ -368,7 +368,7 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
     // 2 x 2 (one wave per SIMD, 256 accumulators) measures 1-2 % faster than 4 x 2 on 8192^3;
     // NZHIP_H16_WAVES=8 selects the latter (benchmarking only).
     static const char* waves_env = getenv("NZHIP_H16_WAVES");
-    const int wm_waves = (waves_env && atoi(waves_env) == 8) ? 4 : 2;
+    const int wm_waves = (waves == 8 || (waves == 0 && waves_env && atoi(waves_env) == 8)) ? 4 : 2;
     int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, 8 / wm_waves);
     if (rc == NZHIP_OK) rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems, 4);
     if (rc == NZHIP_OK) {

@@ -234,7 +234,8 @@ void nzo_general_matmul(const float* A, const float* B, float* C, const size_t s
             for (size_t r = 0; r < M; r++)
                 for (size_t q = 0; q < N; q++) {
                     float sum = 0.0f;
-                    for (size_t k = 0; k < K; k++) sum += a[r * K + k] * b[k * N + q];
+                    /* nvcc contracts `sum += As*Bs` (:92-93) into one FMA per k (its default -fmad=true) */
+                    for (size_t k = 0; k < K; k++) sum = fmaf(a[r * K + k], b[k * N + q], sum);
                     c[r * N + q] = sum;
                 }
         }
@@ -392,6 +393,27 @@ void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_ou
         const size_t c = fixedIdx / (H_out * W_out);
         const size_t h = (fixedIdx % (H_out * W_out)) / W_out, w = (fixedIdx % (H_out * W_out)) % W_out;
         dcol[batch * per + (h * W_out + w) * C_out + c] = dy[idx];
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Optimizer steps: src/OperationKernels.cu:634-640 and :753-766.             */
+/* ------------------------------------------------------------------------- */
+void nzo_sgd_step(float* data, const float* grad, float lr, size_t n) {
+    for (size_t i = 0; i < n; i++) data[i] -= lr * grad[i];
+}
+
+void nzo_adam_step(float* data, float* m, float* v, const float* grad, float lr, float beta1, float beta2,
+                   float eps, int t, size_t n) {
+    const float corr1 = 1.0f - powf(beta1, (float)t), corr2 = 1.0f - powf(beta2, (float)t);
+    for (size_t i = 0; i < n; i++) {
+        const float m_temp = m[i] * beta1 + grad[i] * (1 - beta1);
+        const float v_temp = v[i] * beta2 + grad[i] * grad[i] * (1 - beta2);
+        const float m_modified = m_temp / corr1;
+        const float v_modified = v_temp / corr2;
+        data[i] -= lr * m_modified / (sqrtf(v_modified) + eps);
+        m[i] = m_temp;
+        v[i] = v_temp;
     }
 }
 

@@ -21,6 +21,12 @@
  *   - backward (GEMM, add, ReLU, im2col, col2im) pinned (reference literal vectors
  *                                      Test.cpp:820-903, loop nests :3011-3072 and
  *                                      :3144-3177, adjoint identities <Jv,u> = <v,J^T u>)
+ *   - fp32 matmul, SGD ............... pinned (reference literal vector Test.cpp:119-184, closed form);
+ *                                      whether each k step is one FMA or a rounded multiply and add is
+ *                                      the CUDA compiler's choice (default: FMA, restated here): the last
+ *                                      bit of non-integer results is PARITY UNPINNED
+ *   - Adam ........................... pinned against the host formula of the reference's own test
+ *                                      (Test.cpp:2398-2452); the kernel's __powf bits: PARITY UNPINNED
  *   - bit-level accumulation order of nvcuda::wmma::mma_sync: PARITY UNPINNED
  *     (unspecified by the vendor; the tolerance contract replaces it).
  */
@@ -129,6 +135,14 @@ void nzo_im2col_backward(float* dx, const float* dcol, size_t H_out, size_t W_ou
                          size_t K_w, size_t stride, size_t pad, size_t H_in, size_t W_in, size_t batch);
 /* col2imgBackwardKernel, src/OperationKernels.cu:1384-1396: dcol[b][(h*W+w)*C+c] = dy[b][c][h][w]. */
 void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_out, size_t C_out, size_t batches);
+
+/* ---- optimizer steps ------------------------------------------------------
+ * StochasticGradientDescentKernel, src/OperationKernels.cu:634-640: data -= lr * grad. */
+void nzo_sgd_step(float* data, const float* grad, float lr, size_t n);
+/* AdamKernel, src/OperationKernels.cu:753-766 (fp32 throughout). beta^t through powf: the reference
+ * uses CUDA's approximate __powf there, whose last bits are PARITY UNPINNED. */
+void nzo_adam_step(float* data, float* m, float* v, const float* grad, float lr, float beta1, float beta2,
+                   float eps, int t, size_t n);
 
 /* max over i of |got-truth| / max(|truth|, floor) and Frobenius ||got-truth|| / ||truth|| */
 void nzo_errors_f32_vs_f64(const float* got, const double* truth, size_t n, double floor_abs,

@@ -81,6 +81,8 @@ _relu_bwd = _sig("nzo_relu_backward", None, _f32p, _f32p, _f32p, _sz)
 _add_bwd = _sig("nzo_add_backward", None, _f32p, _f32p, _Shape, _Shape)
 _im2col_bwd = _sig("nzo_im2col_backward", None, _f32p, _f32p, *([_sz] * 10))
 _col2im_bwd = _sig("nzo_col2im_backward", None, _f32p, _f32p, _sz, _sz, _sz, _sz)
+_sgd = _sig("nzo_sgd_step", None, _f32p, _f32p, C.c_float, _sz)
+_adam = _sig("nzo_adam_step", None, _f32p, _f32p, _f32p, _f32p, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, _sz)
 _conv_graph = _sig("nzo_conv2d_graph", None, _f32p, _f32p, _f32p, C.c_void_p, *([_sz] * 10), C.c_int)
 _conv_direct = _sig("nzo_conv2d_direct_f64", None, _f64p, _f32p, _f32p, C.c_void_p, *([_sz] * 9), C.c_int)
 _linear = _sig("nzo_linear_graph", None, _f32p, _f32p, _f32p, C.c_void_p, _sz, _sz, _sz, C.c_int)
@@ -267,6 +269,19 @@ def col2im_backward(dy: np.ndarray) -> np.ndarray:
     out = np.empty((N, 1, Ho * Wo, O), np.float32)
     _col2im_bwd(out.reshape(-1), dy.reshape(-1), Ho, Wo, O, N)
     return out
+
+
+def sgd_step(data, grad, lr):
+    out = _c(data).copy()
+    _sgd(out.reshape(-1), _c(grad).reshape(-1), lr, out.size)
+    return out
+
+
+def adam_step(data, m, v, grad, lr, beta1, beta2, eps, t):
+    """One Adam step; returns the new (data, m, v)."""
+    d, m2, v2 = _c(data).copy(), _c(m).copy(), _c(v).copy()
+    _adam(d.reshape(-1), m2.reshape(-1), v2.reshape(-1), _c(grad).reshape(-1), lr, beta1, beta2, eps, t, d.size)
+    return d, m2, v2
 
 
 def conv2d_graph(x, w_ref, bias_ref, K_h, K_w, stride, pad, relu=False) -> np.ndarray:

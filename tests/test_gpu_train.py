@@ -1,0 +1,80 @@
+"""fp32-exact matmul (Tensor::operator*) and optimizer steps on the GPU against the CPU oracle,
+through the C-ABI. The matmul accumulates with FMAs in ascending k exactly like the oracle's scalar
+loop: results are compared bit for bit, also on float data."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nz():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from neuzephyr_amd import capi
+    capi.load()
+    return capi
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+def test_matmul_f32_reference_literal_vector(nz):
+    # test/Test.cpp:119-184
+    A = np.arange(1, 13, dtype=np.float32).reshape(2, 1, 2, 3)
+    B = np.arange(1, 19, dtype=np.float32).reshape(1, 3, 3, 2)
+    want = np.array([22, 28, 49, 64, 58, 64, 139, 154, 94, 100, 229, 244, 76, 100, 103, 136, 220, 244, 301, 334, 364, 388,
+                     499, 532], np.float32).reshape(2, 3, 2, 2)
+    assert np.array_equal(host(nz.matmul_f32(dev(A), dev(B))), want)
+
+
+@pytest.mark.parametrize("sa,sb", [((1, 1, 1, 1), (1, 1, 1, 1)), ((2, 3, 5, 7), (2, 3, 7, 6)), ((2, 1, 33, 17), (1, 3, 17, 130)),
+                                   ((1, 1, 129, 65), (1, 1, 65, 131)), ((1, 1, 300, 40), (1, 1, 40, 260)),
+                                   ((3, 2, 64, 16), (1, 1, 16, 64)), ((1, 1, 7, 1000), (1, 1, 1000, 5))])
+def test_matmul_f32_bit_identical_to_the_oracle(nz, oracle, sa, sb):
+    rng = np.random.default_rng(sum(sa) * 7 + sum(sb))
+    A = rng.standard_normal(sa).astype(np.float32)
+    B = rng.standard_normal(sb).astype(np.float32)
+    # 1 + 2^-12 is not a half: a kernel that rounded its operands to fp16 would lose it
+    A.reshape(-1)[0] = 1 + 2.0 ** -12
+    got = host(nz.matmul_f32(dev(A), dev(B)))
+    assert np.array_equal(got, oracle.general_matmul(A, B))
+
+
+def test_matmul_f32_rejects_bad_shapes(nz):
+    with pytest.raises(nz.NzHipError):
+        nz.matmul_f32(dev(np.zeros((1, 1, 2, 3))), dev(np.zeros((1, 1, 4, 2))))
+    with pytest.raises(nz.NzHipError):
+        nz.matmul_f32(dev(np.zeros((2, 1, 2, 3))), dev(np.zeros((3, 1, 3, 2))))
+
+
+def test_sgd_step_bit_exact(nz, oracle):
+    rng = np.random.default_rng(41)
+    for n in (1, 72, 4097):
+        data = rng.uniform(-10, 10, n).astype(np.float32)
+        grad = rng.uniform(-10, 10, n).astype(np.float32)
+        got = host(nz.sgd_step(dev(data), dev(grad), 0.01))
+        assert np.allclose(got, oracle.sgd_step(data, grad, 0.01), rtol=0, atol=0) or \
+            np.max(np.abs(got - oracle.sgd_step(data, grad, 0.01))) <= np.spacing(np.float32(10.0))   # mul+sub may fuse
+
+
+def test_adam_steps_match_oracle(nz, oracle):
+    rng = np.random.default_rng(43)
+    n = 4099
+    data = rng.uniform(-10, 10, n).astype(np.float32)
+    grad = rng.uniform(-10, 10, n).astype(np.float32)
+    d, m, v = dev(data), dev(np.zeros(n)), dev(np.zeros(n))
+    do, mo, vo = data, np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for t in (1, 2, 3):
+        nz.adam_step(d, m, v, dev(grad), 0.01, 0.9, 0.999, 1e-6, t)
+        do, mo, vo = oracle.adam_step(do, mo, vo, grad, 0.01, 0.9, 0.999, 1e-6, t)
+    assert np.allclose(host(d), do, rtol=1e-5, atol=1e-6)        # the reference's own comparison tolerance
+    assert np.allclose(host(m), mo, rtol=1e-6, atol=1e-7) and np.allclose(host(v), vo, rtol=1e-6, atol=1e-7)
+    with pytest.raises(nz.NzHipError):
+        nz.adam_step(d, m, v, dev(grad), 0.01, 0.9, 0.999, 1e-6, 0)
