@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "Nodes.cuh"
+#include "Optimizer.cuh"
 #include "dl_export.cuh"
 
 namespace nz::graph {
@@ -35,6 +36,7 @@ namespace nz::graph {
         // last forward() fused node chains, the skipped intermediates are recomputed first.
         void backward();
         void zeroGrad() const;                           // src/ComputeGraph.cu:434-438
+        void update(opt::Optimizer* optimizer) const;    // one step() per node that requires gradients (:541-547)
         [[nodiscard]] io::OutputNode* getOutputNode() const;   // throws std::runtime_error without exactly one output
         void setFusion(bool enabled);
         [[nodiscard]] size_t fusedGroupCount() const { return fusedGroups; }

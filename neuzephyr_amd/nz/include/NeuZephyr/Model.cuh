@@ -24,6 +24,7 @@ namespace nz {
 
         data::Tensor& forward();
         void backward();                                 // reverse pass of the graph (src/Model.cu:17-19)
+        void update(opt::Optimizer* optimizer) const;    // graph update, then zeroGrad (src/Model.cu:20-23)
         graph::ComputeGraph& graph() { return computeGraph; }
         // Parameters (weights, biases) in creation order, so that callers can inject values.
         [[nodiscard]] const std::vector<io::InputNode*>& parameters() const { return params; }

@@ -70,6 +70,8 @@ namespace nz::data {
         void randomize(unsigned long long seed = 0) const;
         void reshape(const shape_type& shape);
 
+        // fp32-exact batched matrix product with (n, c) broadcast (reference: src/Tensor.cu:343-350)
+        Tensor operator*(const Tensor& other) const;
         bool operator==(const Tensor& other) const;               // rel 1e-5 / abs 1e-6, also compares gradients
         bool operator!=(const Tensor& other) const { return !(*this == other); }
 

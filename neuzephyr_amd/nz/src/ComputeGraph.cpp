@@ -209,6 +209,11 @@ namespace nz::graph {
         for (auto it = sortedNodes.rbegin(); it != sortedNodes.rend(); ++it) (*it)->backward();
     }
 
+    void ComputeGraph::update(opt::Optimizer* optimizer) const {
+        for (Node* node : nodes)
+            if (node->output && node->output->requiresGrad()) optimizer->step(node);
+    }
+
     void ComputeGraph::zeroGrad() const {
         for (Node* node : nodes)
             if (node->output && node->output->requiresGrad()) node->output->zeroGrad();

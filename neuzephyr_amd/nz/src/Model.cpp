@@ -14,6 +14,11 @@ namespace nz {
 
     void Model::backward() { computeGraph.backward(); }
 
+    void Model::update(opt::Optimizer* optimizer) const {
+        computeGraph.update(optimizer);
+        computeGraph.zeroGrad();
+    }
+
     Node* Model::track(Node* node) {
         node->internal = true;
         hiddenNodes.push_back(node);

@@ -175,6 +175,23 @@ namespace nz::data {
         _shape = shape;
     }
 
+    Tensor Tensor::operator*(const Tensor& other) const {
+        if (!_shape.isBroadcastCompatible(other._shape) || _shape.W() != other._shape.H()) {
+            throw std::invalid_argument("Shapes are not broadcast compatible.");
+        }
+        Tensor result({std::max(_shape.N(), other._shape.N()), std::max(_shape.C(), other._shape.C()), _shape.H(),
+                       other._shape.W()},
+                      _requires_grad || other._requires_grad);
+        size_t sa[4], sb[4], sc[4];
+        for (size_t i = 0; i < 4; ++i) {
+            sa[i] = _shape[i];
+            sb[i] = other._shape[i];
+            sc[i] = result._shape[i];
+        }
+        NZ_CHECK(nzhip_matmul_f32(data(), other.data(), result.data(), sa, sb, sc, nzhip_default_stream()));
+        return result;
+    }
+
     bool Tensor::operator==(const Tensor& other) const {
         if (_requires_grad != other._requires_grad || _shape != other._shape) return false;
         constexpr value_type abs_epsilon = 1e-6f, rel_epsilon = 1e-5f;   // src/Tensor.cu:513-514

@@ -33,6 +33,23 @@ namespace nz::data {
         NZ_CHECK(nzhip_add_broadcast(out, in1, in2, so, s1, s2, nzhip_default_stream()));
     }
 
+    void iGeneralMatrixMul(float* A, float* B, float* C, const size_t M, const size_t N, const size_t K,
+                           const std::vector<size_t>& offsetC, const std::vector<size_t>& offsetA,
+                           const std::vector<size_t>& offsetB) {
+        const size_t sa[4] = {1, 1, M, K}, sb[4] = {1, 1, K, N}, sc[4] = {1, 1, M, N};
+        for (size_t i = 0; i < offsetC.size(); ++i)
+            NZ_CHECK(nzhip_matmul_f32(A + offsetA[i], B + offsetB[i], C + offsetC[i], sa, sb, sc, nzhip_default_stream()));
+    }
+
+    void iGeneralMatrixMulBroadcast(float* A, float* B, float* C, const Dimension& shapeA, const Dimension& shapeB,
+                                    const Dimension& shapeC) {
+        size_t sa[4], sb[4], sc[4];
+        dims4(shapeA, sa);
+        dims4(shapeB, sb);
+        dims4(shapeC, sc);
+        NZ_CHECK(nzhip_matmul_f32(A, B, C, sa, sb, sc, nzhip_default_stream()));
+    }
+
     void iTensorCoreGEMM(float* A, float* B, float* C, const Dimension& shapeA, const Dimension& shapeB,
                          const Dimension& shapeC) {
         size_t sa[4], sb[4], sc[4];

@@ -13,6 +13,7 @@
 #include "NeuZephyr/ComputeGraph.cuh"
 #include "NeuZephyr/Model.cuh"
 #include "NeuZephyr/Nodes.cuh"
+#include "NeuZephyr/Optimizer.cuh"
 #include "NeuZephyr/TensorOperations.cuh"
 #include "mini_test.hpp"
 #include "nzhip.h"
@@ -463,6 +464,114 @@ TEST(Model, Conv2dBackwardMatchesFiniteStructure) {
                         }
     EXPECT_TRUE(closeTo(m.parameters()[0]->output->hostGrad(), dW, 1e-5));        // weights are per sample
     for (float v : m.parameters()[1]->output->hostGrad()) EXPECT_TRUE(v == static_cast<float>(n));
+}
+
+// ---- fp32 matmul and optimizers (test/Test.cpp:119-184, 2230-2265, 2398-2452, 2816-2878) ------------
+TEST(TensorBasic, TensorMultiplicationTest) {
+    Tensor tensor1({2, 1, 2, 3});
+    Tensor tensor2({1, 3, 3, 2});
+    tensor1.dataInject(kData1.begin(), kData1.end());
+    tensor2.dataInject(kData2.begin(), kData2.end());
+    Tensor result = tensor1 * tensor2;
+    Tensor expected({2, 3, 2, 2});
+    expected.dataInject(kExpected.begin(), kExpected.end());
+    EXPECT_TRUE(result == expected);
+    // the tensor-core path agrees with it on integers (test/Test.cpp:708-751)
+    Tensor tc({2, 3, 2, 2});
+    GEMMTensorCore(tc, tensor1, tensor2);
+    EXPECT_EQ(tc, result);
+    // no fp16 rounding on this path: 1 + 2^-12 survives
+    Tensor a({1, 1, 1, 1}), b({1, 1, 1, 1});
+    a.fill(1.f + 1.f / 4096.f);
+    b.fill(1.f);
+    EXPECT_TRUE((a * b).hostData()[0] == 1.f + 1.f / 4096.f);
+    Tensor bad({1, 1, 4, 2});
+    EXPECT_THROW(tensor1 * bad, std::invalid_argument);
+}
+
+TEST(OptimizerBasic, SGDTest) {
+    const size_t n = 2, c = 3, h = 3, w = 4;
+    const float learningRate = 0.01f;
+    auto data = randomVec(n * c * h * w, 51, -10.f, 10.f), grad = randomVec(n * c * h * w, 52, -10.f, 10.f);
+    std::vector<float> expectedData(data.size());
+    for (size_t i = 0; i < data.size(); i++) expectedData[i] = data[i] - learningRate * grad[i];
+    InputNode input({n, c, h, w}, true);
+    input.dataInject(data.begin(), data.end());
+    input.dataInject(grad.begin(), grad.end(), true);
+    nz::opt::SGD optimizer(learningRate);
+    optimizer.step(&input);
+    Tensor expected({n, c, h, w}, true);
+    expected.dataInject(expectedData.begin(), expectedData.end());
+    expected.dataInject(grad.begin(), grad.end(), true);
+    EXPECT_EQ(*input.output, expected);
+}
+
+TEST(OptimizerBasic, AdamTest) {
+    const size_t n = 2, c = 3, h = 3, w = 4;
+    const float learningRate = 0.01f, beta1 = 0.9f, beta2 = 0.999f, epsilon = 1e-6f;
+    auto data = randomVec(n * c * h * w, 53, -10.f, 10.f), grad = randomVec(n * c * h * w, 54, -10.f, 10.f);
+    std::vector<float> expectedData(data), m(data.size(), 0.f), v(data.size(), 0.f);
+    for (int it = 1; it <= 2; it++)
+        for (size_t i = 0; i < data.size(); i++) {
+            m[i] = beta1 * m[i] + (1 - beta1) * grad[i];
+            v[i] = beta2 * v[i] + (1 - beta2) * grad[i] * grad[i];
+            const float modified_m = m[i] / (1 - std::pow(beta1, it));
+            const float modified_v = v[i] / (1 - std::pow(beta2, it));
+            expectedData[i] = expectedData[i] - (learningRate / (std::sqrt(modified_v) + epsilon)) * modified_m;
+        }
+    InputNode input({n, c, h, w}, true);
+    input.dataInject(data.begin(), data.end());
+    input.dataInject(grad.begin(), grad.end(), true);
+    nz::opt::Adam optimizer(learningRate, beta1, beta2);
+    optimizer.step(&input);
+    optimizer.step(&input);
+    Tensor expected({n, c, h, w}, true);
+    expected.dataInject(expectedData.begin(), expectedData.end());
+    expected.dataInject(grad.begin(), grad.end(), true);
+    EXPECT_EQ(*input.output, expected);
+}
+
+struct SGDTestModel : nz::Model {                               // test/Test.cpp:2816-2835
+    InputNode input1{{5, 3, 12, 1}, true};
+    InputNode input2{{5, 3, 12, 1}, false};
+    SGDTestModel() {
+        auto x = Add(&input1, &input2);
+        defaultOutput(x);
+    }
+};
+
+TEST(Model, SGDOptimize) {
+    const size_t count = 5 * 3 * 12;
+    const float lr = 0.01f;
+    auto d1 = randomVec(count, 61, 0.1f, 0.9f), d2 = randomVec(count, 62, 0.1f, 0.9f), g1 = randomVec(count, 63, 0.1f, 0.9f);
+    std::vector<float> expectedData(count);
+    for (size_t i = 0; i < count; i++) expectedData[i] = d1[i] - lr * g1[i];
+    SGDTestModel model{};
+    model.input1.dataInject(d1.begin(), d1.end());
+    model.input2.dataInject(d2.begin(), d2.end());
+    model.input1.dataInject(g1.begin(), g1.end(), true);
+    nz::opt::SGD optimizer(lr);
+    model.update(&optimizer);
+    Tensor expected({5, 3, 12, 1}, true);
+    expected.dataInject(expectedData.begin(), expectedData.end());
+    EXPECT_EQ(expected, *model.input1.output);                   // gradient was reset by update()
+}
+
+TEST(Model, LinearTrainingStepLowersTheOutputSum) {
+    // forward -> backward (d(sum of outputs)) -> SGD: the sum of the outputs must go down
+    LinearModel m(16, 40, 24, false);
+    auto x = randomVec(16 * 40, 71, -1.f, 1.f);
+    m.input.dataInject(x.begin(), x.end());
+    auto total = [&] {
+        double s = 0;
+        for (float v : m.forward().hostData()) s += v;
+        return s;
+    };
+    const double before = total();
+    m.backward();
+    nz::opt::SGD optimizer(0.01f);
+    m.update(&optimizer);
+    EXPECT_TRUE(total() < before);
 }
 
 TEST(Runtime, AllocatorCachesAndErrorsSurfaceAsExceptions) {
