@@ -262,8 +262,8 @@ def cpu_baseline_gemm(orc, A, B, rows=8192):
 def main():
     args = parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures ONE GPU only (the path shards with no exchange; "
-              "see DESIGN.md); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build measures ONE GPU only (the path shards by rows or batch members with no "
+              "exchange between GPUs); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():
