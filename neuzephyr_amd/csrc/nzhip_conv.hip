@@ -168,9 +168,25 @@ __global__ __launch_bounds__(256) void conv3x3_direct_kernel(float* __restrict__
 // is complete and is computed in the reference's k order (c, r, s) and stored. Loads of later
 // rows are in flight while the FMAs of the current row run, so memory and VALU time overlap
 // inside every wave instead of relying on other waves being out of phase.
-constexpr int ST_ROWS = 16, ST_AHEAD = 3;
+// A lane's two halo columns are its neighbours' pixels: they come over the wave (DPP shift by one
+// lane) after rounding; only the first and the last lane of a wave read theirs from memory, with
+// one extra 4-byte request per row and channel that every lane issues (the others re-read a word
+// of their own quad). PIX_BIAS: the bias varies per pixel and travels with the row ring; otherwise
+// it is absent or per channel and is fetched once.
+constexpr int ST_ROWS = 16, ST_AHEAD = 3;         // ST_AHEAD: a multiple of 3 (the window depth)
 
-template <int O_T, int C_T>
+// value of `v` in lane - 1 (lane 0 keeps its own)
+__device__ __forceinline__ float from_lane_below(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                 0x138 /* wave_shr:1 */, 0xf, 0xf, false));
+}
+// value of `v` in lane + 1 (lane 63 keeps its own)
+__device__ __forceinline__ float from_lane_above(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                 0x130 /* wave_shl:1 */, 0xf, 0xf, false));
+}
+
+template <int O_T, int C_T, bool PIX_BIAS>
 __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__ y, const float* __restrict__ x,
                                                              const float* __restrict__ w_ref,
                                                              const float* __restrict__ bias, int H, int W,
@@ -189,67 +205,80 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
     const float* xb = x + (long)b * C_T * H * W;
     float* yb = y + (long)b * O_T * H * W;
     const long plane = (long)H * W;
-    const int wl = w0 > 0 ? w0 - 1 : 0, wr = w0 + 4 < W ? w0 + 4 : W - 1;
     const bool has_l = w0 > 0, has_r = w0 + 4 < W;
+    // column of the extra request: left halo for the first lane, right halo for the last, else own quad
+    const int wx = lane == 0 ? (has_l ? w0 - 1 : w0) : (lane == 63 && has_r ? w0 + 4 : w0);
     const int rows = (H - h0) < ST_ROWS ? (H - h0) : ST_ROWS;   // output rows of this strip
     const int T = rows + 2;                                      // input rows h0-1 .. h0+rows
 
-    float raw[3][C_T][6];                                        // rows in flight (t % 3)
-    float braw[3][O_T][4];                                       // bias of the output row each of them completes
+    float raw[ST_AHEAD][C_T][5];                                 // rows in flight (t % ST_AHEAD): own quad + extra word
+    float braw[ST_AHEAD][O_T][4];                                // per-pixel bias of the output row each completes
     float win[3][C_T][6];                                        // rounded rows t-2, t-1, t (t % 3)
+    float bch[O_T];                                              // per-channel bias
+#pragma unroll
+    for (int o = 0; o < O_T; o++) bch[o] = (!PIX_BIAS && bias) ? bias[(long)o * bias_sc] : 0.f;
 
-    // Requests are unconditional (rows beyond the image read row 0, halo columns are clamped);
-    // what must be zero is masked when the row is consumed, so nothing waits at request time.
+    // Requests are unconditional (rows beyond the image read row 0); what must be zero is masked
+    // when the row is consumed, so nothing waits at request time.
     auto row_in_image = [&](int t) { const int hi = h0 - 1 + t; return t < T && hi >= 0 && hi < H; };
-    auto request = [&](int t, float (&dst)[C_T][6], float (&bdst)[O_T][4]) {
+    auto request = [&](int t, float (&dst)[C_T][5], float (&bdst)[O_T][4]) {
         const float* row = xb + (long)(row_in_image(t) ? h0 - 1 + t : 0) * W;
-        // the bias of output row h0 + t - 2 travels with the input row that completes it, so its
-        // wait never drains the rows requested after it
-        const int hb = (t >= 2 && t < T) ? h0 + t - 2 : h0;
+        if (PIX_BIAS) {
+            // the bias of output row h0 + t - 2 travels with the input row that completes it, so its
+            // wait never drains the rows requested after it
+            const int hb = (t >= 2 && t < T) ? h0 + t - 2 : h0;
 #pragma unroll
-        for (int o = 0; o < O_T; o++)
+            for (int o = 0; o < O_T; o++)
 #pragma unroll
-            for (int e = 0; e < 4; e++)
-                bdst[o][e] = bias ? bias[((long)hb * W + w0 + e) * bias_sp + (long)o * bias_sc] : 0.f;
+                for (int e = 0; e < 4; e++) bdst[o][e] = bias[((long)hb * W + w0 + e) * bias_sp + (long)o * bias_sc];
+        }
 #pragma unroll
         for (int c = 0; c < C_T; c++) {
             const floatx4 q = *reinterpret_cast<const floatx4*>(row + c * plane + w0);
-            dst[c][0] = row[c * plane + wl];
-            dst[c][1] = q[0];
-            dst[c][2] = q[1];
-            dst[c][3] = q[2];
-            dst[c][4] = q[3];
-            dst[c][5] = row[c * plane + wr];
+            dst[c][0] = q[0];
+            dst[c][1] = q[1];
+            dst[c][2] = q[2];
+            dst[c][3] = q[3];
+            dst[c][4] = row[c * plane + wx];
         }
     };
 
 #pragma unroll
     for (int t = 0; t < ST_AHEAD; t++) request(t, raw[t], braw[t]);
 
-    for (int t0 = 0; t0 < T; t0 += 3) {
+    static_assert(ST_AHEAD % 3 == 0, "the request ring must be a whole number of windows");
+    for (int t0 = 0; t0 < T; t0 += ST_AHEAD) {
 #pragma unroll
-        for (int u = 0; u < 3; u++) {
-            const int t = t0 + u;                                // t % 3 == u because t0 % 3 == 0
+        for (int u = 0; u < ST_AHEAD; u++) {
+            const int t = t0 + u;                                // t % ST_AHEAD == u, and t % 3 == u % 3
+            const int wu = u % 3;
             if (t >= T) break;
+            const bool in_img = row_in_image(t);
 #pragma unroll
-            for (int c = 0; c < C_T; c++)
+            for (int c = 0; c < C_T; c++) {
+                float r5[5];
 #pragma unroll
-                for (int e = 0; e < 6; e++) {
+                for (int e = 0; e < 5; e++) {
                     // Opaque use: pins the rounding (and therefore the wait for the load) HERE, three
                     // rows after the request; otherwise the compiler moves the conversion up to the
                     // load and the wave waits for every row as soon as it has asked for it.
                     float v = raw[u][c][e];
                     asm volatile("" : "+v"(v));
-                    const bool keep = row_in_image(t) && (e != 0 || has_l) && (e != 5 || has_r);
-                    win[u][c][e] = keep ? round_f16(v) : 0.f;
+                    r5[e] = in_img ? round_f16(v) : 0.f;
                 }
+                const float below = from_lane_below(r5[3]), above = from_lane_above(r5[0]);
+                win[wu][c][0] = has_l ? (lane == 0 ? r5[4] : below) : 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; e++) win[wu][c][1 + e] = r5[e];
+                win[wu][c][5] = has_r ? (lane == 63 ? r5[4] : above) : 0.f;
+            }
             float bnow[O_T][4];
 #pragma unroll
             for (int o = 0; o < O_T; o++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    bnow[o][e] = braw[u][o][e];
-                    asm volatile("" : "+v"(bnow[o][e]));
+                    bnow[o][e] = PIX_BIAS ? braw[u][o][e] : bch[o];
+                    if (PIX_BIAS) asm volatile("" : "+v"(bnow[o][e]));
                 }
             request(t + ST_AHEAD, raw[u], braw[u]);              // slot u is free again
             if (t < 2) continue;
@@ -263,7 +292,7 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
             for (int c = 0; c < C_T; c++)
 #pragma unroll
                 for (int r = 0; r < 3; r++) {
-                    const int slot = (u + 1 + r) % 3;            // row t-2+r lives in slot (t-2+r) % 3
+                    const int slot = (wu + 1 + r) % 3;           // row t-2+r lives in slot (t-2+r) % 3
 #pragma unroll
                     for (int s2 = 0; s2 < 3; s2++)
 #pragma unroll
@@ -300,9 +329,16 @@ static int conv_direct(float* y, const float* x, const float* w_ref, const float
     const long wbs = w_batch > 1 ? (long)(C * 9 * O) : 0;
     if (vec && C <= 4 && O <= 2 && H >= 8) {
         dim3 sgrid((unsigned)((W + 255) / 256), (unsigned)((H + 4 * ST_ROWS - 1) / (4 * ST_ROWS)), (unsigned)N);
-#define NZHIP_ST(OT, CT)                                                                                         \
-    hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H, (int)W, \
-                       wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU)
+        const bool pixb = bias && bias_sp != 0;
+#define NZHIP_ST(OT, CT)                                                                                             \
+    do {                                                                                                             \
+        if (pixb)                                                                                                    \
+            hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT, true>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H, \
+                               (int)W, wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU);                   \
+        else                                                                                                         \
+            hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT, false>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H, \
+                               (int)W, wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU);                   \
+    } while (0)
         switch ((int)(O * 10 + C)) {
             case 11: NZHIP_ST(1, 1); break;
             case 12: NZHIP_ST(1, 2); break;
