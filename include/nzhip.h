@@ -179,6 +179,19 @@ int nzhip_sgd_step(float* data, const float* grad, float lr, size_t n, void* str
 int nzhip_adam_step(float* data, float* m, float* v, const float* grad, float lr, float beta1,
                     float beta2, float eps, int t, size_t n, void* stream);
 
+/* ---- softmax (third caller of the GEMM entry: its backward is Jacobian x gradient) --------- */
+/* nz::data::Softmax over `batch` contiguous vectors of `len` elements (TensorOperations.cuh:379-392;
+ * SummationExpKernel + SoftmaxKernel, src/OperationKernels.cu:477-523): out = exp(in) / sum(exp(in)),
+ * no maximum subtracted. exp is the fast hardware form (the reference uses __expf) and the sum is a
+ * tree: last bits are not pinned by the reference. */
+int nzhip_softmax(float* out, const float* in, size_t len, size_t batch, void* stream);
+
+/* nz::data::softmaxJacobian / iSoftmaxJacobian (TensorOperations.cuh:1091-1106; SoftmaxJacobianKernel,
+ * src/OperationKernels.cu:550-565): out[b][x][y] = s_x (1 - s_x) if x == y else -s_x s_y, s = in[b].
+ * SoftmaxNode::backward (src/Nodes.cu:538-548) is this followed by nzhip_tensorcore_gemm
+ * (J x dY for column vectors, dY x J for row vectors). */
+int nzhip_softmax_jacobian(float* out, const float* in, size_t n, size_t batch, void* stream);
+
 /* ---- runtime: device allocator + stream manager -------------------------- */
 /* Replace cuStrm::StreamManager<float> (include/NeuZephyr/StreamManager.cuh:131-911) and
  * EventPool (EventPool.cuh:165-457).  One ordered compute stream carries every kernel and

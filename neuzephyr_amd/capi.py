@@ -19,6 +19,7 @@ EXPORTS = [
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
+    "nzhip_softmax", "nzhip_softmax_jacobian",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
@@ -83,6 +84,8 @@ def load() -> C.CDLL:
     lib.nzhip_col2im_backward.argtypes = [vp, vp, sz, sz, sz, sz, vp]
     lib.nzhip_matmul_f32.argtypes = [vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_sgd_step.argtypes = [vp, vp, C.c_float, sz, vp]
+    lib.nzhip_softmax.argtypes = [vp, vp, sz, sz, vp]
+    lib.nzhip_softmax_jacobian.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_adam_step.argtypes = [vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, sz, vp]
     lib.nzhip_default_stream.restype = vp
     lib.nzhip_malloc.argtypes = [C.POINTER(vp), sz]
@@ -312,3 +315,26 @@ def adam_step(data, m, v, grad, lr, beta1, beta2, eps, t, stream=None):
     check(lib.nzhip_adam_step(_dev(data), _dev(m), _dev(v), _dev(grad), lr, beta1, beta2, eps, t, data.numel(),
                               _stream_handle(stream)))
     return data, m, v
+
+
+def softmax(x, stream=None):
+    import torch
+    lib = load()
+    out = torch.empty_like(x)
+    check(lib.nzhip_softmax(_dev(out), _dev(x), x.shape[2] * x.shape[3], x.shape[0] * x.shape[1], _stream_handle(stream)))
+    return out
+
+
+def softmax_jacobian(s, stream=None):
+    import torch
+    lib = load()
+    n = max(s.shape[2], s.shape[3])
+    out = torch.empty((s.shape[0], s.shape[1], n, n), dtype=torch.float32, device=s.device)
+    check(lib.nzhip_softmax_jacobian(_dev(out), _dev(s), n, s.shape[0] * s.shape[1], _stream_handle(stream)))
+    return out
+
+
+def softmax_backward(s, dy, stream=None):
+    """SoftmaxNode::backward: Jacobian times gradient through the fp16 GEMM entry."""
+    jac = softmax_jacobian(s, stream)
+    return tensorcore_gemm(jac, dy, stream=stream) if s.shape[2] > s.shape[3] else tensorcore_gemm(dy, jac, stream=stream)

@@ -1,7 +1,9 @@
 // fp32-exact pieces next to the fp16 path: the matmul behind Tensor::operator* (no rounding of the
 // operands, fp32 FMA accumulation in ascending k, reference: GeneralMatrixMulKernel,
 // src/OperationKernels.cu:65-101) and the optimizer steps that close a training iteration
-// (StochasticGradientDescentKernel :634-640, AdamKernel :753-766).
+// (StochasticGradientDescentKernel :634-640, AdamKernel :753-766), plus the softmax forward and its
+// Jacobian, whose product with the incoming gradient is one more call of the fp16 GEMM entry
+// (SoftmaxNode::backward, src/Nodes.cu:538-548).
 #include <hip/hip_runtime.h>
 
 #include "nzhip_internal.h"
@@ -155,6 +157,34 @@ __global__ __launch_bounds__(256) void adam_kernel(float* __restrict__ data, flo
     v[i] = v_temp;
 }
 
+// ---- softmax over one vector per (n, c) and its Jacobian ---------------------------------------
+// One workgroup per vector: exp(x) summed in a fixed tree order (lane stride, wave shuffle, four
+// waves), then every element divided by the sum. No maximum is subtracted, like the reference
+// (SummationExpKernel / SoftmaxKernel, src/OperationKernels.cu:477-523).
+__global__ __launch_bounds__(256) void softmax_kernel(float* __restrict__ out, const float* __restrict__ in, long len) {
+    __shared__ float part[4];
+    const float* x = in + (long)blockIdx.x * len;
+    float* y = out + (long)blockIdx.x * len;
+    float s = 0.f;
+    for (long i = threadIdx.x; i < len; i += 256) s += __expf(x[i]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    const float total = (part[0] + part[1]) + (part[2] + part[3]);
+    for (long i = threadIdx.x; i < len; i += 256) y[i] = __expf(x[i]) / total;
+}
+
+// SoftmaxJacobianKernel (:550-565): J[x][y] = s_x (1 - s_x) on the diagonal, -s_x s_y elsewhere.
+__global__ __launch_bounds__(256) void softmax_jacobian_kernel(float* __restrict__ out, const float* __restrict__ in,
+                                                               int n) {
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (long)n * n) return;
+    const int r = (int)(t / n), c = (int)(t % n);
+    const float* s = in + (long)blockIdx.y * n;
+    out[(long)blockIdx.y * n * n + t] = r == c ? s[r] * (1 - s[r]) : -s[r] * s[c];
+}
+
 }  // namespace nzhip
 
 using namespace nzhip;
@@ -205,6 +235,23 @@ int nzhip_adam_step(float* data, float* m, float* v, const float* grad, float lr
     hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), data, m, v, grad, lr,
                        beta1, beta2, eps, corr1, corr2, (long)n);
     return check_launch("adam_kernel");
+}
+
+int nzhip_softmax(float* out, const float* in, size_t len, size_t batch, void* stream) {
+    if ((!out || !in) && len * batch) return set_error(NZHIP_E_INVALID, "nzhip_softmax: null pointer");
+    if (len == 0 || batch == 0) return NZHIP_OK;
+    if (batch > 0x7fffffff) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_softmax: too many vectors");
+    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)batch), dim3(256), 0, as_stream(stream), out, in, (long)len);
+    return check_launch("softmax_kernel");
+}
+
+int nzhip_softmax_jacobian(float* out, const float* in, size_t n, size_t batch, void* stream) {
+    if ((!out || !in) && n * batch) return set_error(NZHIP_E_INVALID, "nzhip_softmax_jacobian: null pointer");
+    if (n == 0 || batch == 0) return NZHIP_OK;
+    if (n > 46340 || batch > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_softmax_jacobian: extent too large");
+    dim3 grid((unsigned)((n * n + 255) / 256), (unsigned)batch);
+    hipLaunchKernelGGL(softmax_jacobian_kernel, grid, dim3(256), 0, as_stream(stream), out, in, (int)n);
+    return check_launch("softmax_jacobian_kernel");
 }
 
 }  // extern "C"

@@ -109,6 +109,29 @@ namespace nz::nodes {
                 iReLUBackward(inputs[0]->output->grad(), inputs[0]->output->data(), output->grad(), output->size());
         }
 
+        SoftmaxNode::SoftmaxNode(Node* input) {
+            if (std::min(input->output->shape().H(), input->output->shape().W()) != 1) {
+                throw std::invalid_argument("SoftmaxNode: input must be 1D");
+            }
+            inputs.push_back(input);
+            output = std::make_shared<Tensor>(input->output->shape(), input->output->requiresGrad());
+            type = "Softmax";
+        }
+
+        void SoftmaxNode::forward() { Softmax(*output, *inputs[0]->output); }
+
+        void SoftmaxNode::backward() {                                 // src/Nodes.cu:538-548
+            if (!inputs[0]->output->requiresGrad()) return;
+            auto jacobian = softmaxJacobian(*output);
+            if (output->shape()[2] > output->shape()[3]) {
+                iTensorCoreGEMM(jacobian.data(), output->grad(), inputs[0]->output->grad(), jacobian.shape(),
+                                output->shape(), inputs[0]->output->shape());
+            } else {
+                iTensorCoreGEMM(output->grad(), jacobian.data(), inputs[0]->output->grad(), output->shape(),
+                                jacobian.shape(), inputs[0]->output->shape());
+            }
+        }
+
         ReshapeNode::ReshapeNode(Node* input, const Tensor::shape_type& newShape) : newShape(newShape) {
             if (input->output->shape().size() != newShape.size()) {
                 throw std::invalid_argument("ReshapeNode: input and new shape must have the same number of dimensions");

@@ -574,6 +574,45 @@ TEST(Model, LinearTrainingStepLowersTheOutputSum) {
     EXPECT_TRUE(total() < before);
 }
 
+// ---- softmax (test/Test.cpp:1733-1870) -------------------------------------------------------------
+TEST(NodeBasic, SoftmaxForwardJacobianBackward) {
+    const size_t n = 2, c = 3, h = 12, w = 1;
+    auto inputData = randomVec(n * c * h * w, 81, -10.f, 10.f), grad = randomVec(n * c * h * w, 82, -10.f, 10.f);
+    std::vector<float> outputData(inputData.size()), jacobianData(n * c * h * h);
+    for (size_t i = 0; i < n * c; i++) {
+        float sum = 0.0f;
+        for (size_t k = 0; k < h; k++) sum += std::exp(inputData[i * h + k]);
+        for (size_t k = 0; k < h; k++) outputData[i * h + k] = std::exp(inputData[i * h + k]) / sum;
+        for (size_t x = 0; x < h; x++)
+            for (size_t y = 0; y < h; y++)
+                jacobianData[i * h * h + x * h + y] = x == y ? outputData[i * h + x] * (1 - outputData[i * h + x])
+                                                             : -outputData[i * h + x] * outputData[i * h + y];
+    }
+    InputNode input({n, c, h, w}, true);
+    input.dataInject(inputData.begin(), inputData.end());
+    SoftmaxNode softmax(&input);
+    softmax.forward();
+    Tensor expectedOut({n, c, h, w}, true);
+    expectedOut.dataInject(outputData.begin(), outputData.end());
+    EXPECT_EQ(expectedOut, *softmax.output);
+    Tensor probs({n, c, h, w});
+    probs.dataInject(outputData.begin(), outputData.end());
+    Tensor expectedJ({n, c, h, h});
+    expectedJ.dataInject(jacobianData.begin(), jacobianData.end());
+    EXPECT_EQ(softmaxJacobian(probs), expectedJ);
+    // backward: Jacobian x gradient through the fp16 GEMM, exactly what the reference's test builds
+    Tensor outputGrad({n, c, h, w}), inputGrad({n, c, h, w});
+    outputGrad.dataInject(grad.begin(), grad.end());
+    GEMMTensorCore(inputGrad, expectedJ, outputGrad);
+    const auto want = inputGrad.hostData();
+    softmax.output->dataInject(grad.begin(), grad.end(), true);
+    softmax.backward();
+    std::vector<double> wantD(want.begin(), want.end());
+    EXPECT_TRUE(closeTo(input.output->hostGrad(), wantD, 1e-4));
+    InputNode notVector({1, 1, 2, 2});
+    EXPECT_THROW(SoftmaxNode bad(&notVector), std::invalid_argument);
+}
+
 TEST(Runtime, AllocatorCachesAndErrorsSurfaceAsExceptions) {
     size_t inUse0 = 0, cached0 = 0, allocs0 = 0, inUse1 = 0, cached1 = 0, allocs1 = 0;
     {

@@ -397,6 +397,24 @@ void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_ou
 }
 
 /* ------------------------------------------------------------------------- */
+/* Softmax and its Jacobian: test/Test.cpp:1823-1832 and :1782-1795.          */
+/* ------------------------------------------------------------------------- */
+void nzo_softmax(float* out, const float* in, size_t len, size_t batch) {
+    for (size_t b = 0; b < batch; b++) {
+        float sum = 0.0f;
+        for (size_t k = 0; k < len; k++) sum += expf(in[b * len + k]);
+        for (size_t k = 0; k < len; k++) out[b * len + k] = expf(in[b * len + k]) / sum;
+    }
+}
+
+void nzo_softmax_jacobian(float* out, const float* in, size_t n, size_t batch) {
+    for (size_t b = 0; b < batch; b++)
+        for (size_t x = 0; x < n; x++)
+            for (size_t y = 0; y < n; y++)
+                out[b * n * n + x * n + y] = x == y ? in[b * n + x] * (1 - in[b * n + x]) : -in[b * n + x] * in[b * n + y];
+}
+
+/* ------------------------------------------------------------------------- */
 /* Optimizer steps: src/OperationKernels.cu:634-640 and :753-766.             */
 /* ------------------------------------------------------------------------- */
 void nzo_sgd_step(float* data, const float* grad, float lr, size_t n) {

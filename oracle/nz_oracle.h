@@ -136,6 +136,13 @@ void nzo_im2col_backward(float* dx, const float* dcol, size_t H_out, size_t W_ou
 /* col2imgBackwardKernel, src/OperationKernels.cu:1384-1396: dcol[b][(h*W+w)*C+c] = dy[b][c][h][w]. */
 void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_out, size_t C_out, size_t batches);
 
+/* ---- softmax -------------------------------------------------------------
+ * Host statement of the reference's own tests (test/Test.cpp:1823-1832, 1782-1795): exp / sum(exp)
+ * per contiguous vector with the sum taken in ascending order, and the Jacobian loop nest. The kernels
+ * use __expf and a tree sum: their last bits are PARITY UNPINNED (the tests compare at 1e-5). */
+void nzo_softmax(float* out, const float* in, size_t len, size_t batch);
+void nzo_softmax_jacobian(float* out, const float* in, size_t n, size_t batch);
+
 /* ---- optimizer steps ------------------------------------------------------
  * StochasticGradientDescentKernel, src/OperationKernels.cu:634-640: data -= lr * grad. */
 void nzo_sgd_step(float* data, const float* grad, float lr, size_t n);

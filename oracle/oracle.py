@@ -81,6 +81,8 @@ _relu_bwd = _sig("nzo_relu_backward", None, _f32p, _f32p, _f32p, _sz)
 _add_bwd = _sig("nzo_add_backward", None, _f32p, _f32p, _Shape, _Shape)
 _im2col_bwd = _sig("nzo_im2col_backward", None, _f32p, _f32p, *([_sz] * 10))
 _col2im_bwd = _sig("nzo_col2im_backward", None, _f32p, _f32p, _sz, _sz, _sz, _sz)
+_softmax = _sig("nzo_softmax", None, _f32p, _f32p, _sz, _sz)
+_softmax_jac = _sig("nzo_softmax_jacobian", None, _f32p, _f32p, _sz, _sz)
 _sgd = _sig("nzo_sgd_step", None, _f32p, _f32p, C.c_float, _sz)
 _adam = _sig("nzo_adam_step", None, _f32p, _f32p, _f32p, _f32p, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, _sz)
 _conv_graph = _sig("nzo_conv2d_graph", None, _f32p, _f32p, _f32p, C.c_void_p, *([_sz] * 10), C.c_int)
@@ -269,6 +271,28 @@ def col2im_backward(dy: np.ndarray) -> np.ndarray:
     out = np.empty((N, 1, Ho * Wo, O), np.float32)
     _col2im_bwd(out.reshape(-1), dy.reshape(-1), Ho, Wo, O, N)
     return out
+
+
+def softmax(x: np.ndarray) -> np.ndarray:
+    """Softmax over the (h, w) vector of every (n, c); min(h, w) must be 1."""
+    x = _c(x)
+    out = np.empty_like(x)
+    _softmax(out.reshape(-1), x.reshape(-1), x.shape[2] * x.shape[3], x.shape[0] * x.shape[1])
+    return out
+
+
+def softmax_jacobian(s: np.ndarray) -> np.ndarray:
+    s = _c(s)
+    n = max(s.shape[2], s.shape[3])
+    out = np.empty((s.shape[0], s.shape[1], n, n), np.float32)
+    _softmax_jac(out.reshape(-1), s.reshape(-1), n, s.shape[0] * s.shape[1])
+    return out
+
+
+def softmax_backward(s: np.ndarray, dy: np.ndarray) -> np.ndarray:
+    """SoftmaxNode::backward (src/Nodes.cu:538-548): Jacobian times gradient through the fp16 GEMM."""
+    jac = softmax_jacobian(s)
+    return tensorcore_gemm(jac, dy) if s.shape[2] > s.shape[3] else tensorcore_gemm(dy, jac)
 
 
 def sgd_step(data, grad, lr):

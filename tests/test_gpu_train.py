@@ -78,3 +78,18 @@ def test_adam_steps_match_oracle(nz, oracle):
     assert np.allclose(host(m), mo, rtol=1e-6, atol=1e-7) and np.allclose(host(v), vo, rtol=1e-6, atol=1e-7)
     with pytest.raises(nz.NzHipError):
         nz.adam_step(d, m, v, dev(grad), 0.01, 0.9, 0.999, 1e-6, 0)
+
+
+def test_softmax_forward_jacobian_backward(nz, oracle):
+    rng = np.random.default_rng(47)
+    for shape in [(2, 3, 12, 1), (1, 2, 1, 300), (3, 1, 1000, 1), (1, 1, 1, 1)]:
+        x = rng.uniform(-10, 10, shape).astype(np.float32)
+        s = host(nz.softmax(dev(x)))
+        so = oracle.softmax(x)
+        assert np.allclose(s, so, rtol=2e-6, atol=1e-9), shape          # fast exp + tree sum vs expf + serial sum
+        J = host(nz.softmax_jacobian(dev(so)))
+        assert np.array_equal(J, oracle.softmax_jacobian(so)), shape
+        dy = rng.uniform(-10, 10, shape).astype(np.float32)
+        got = host(nz.softmax_backward(dev(so), dev(dy)))
+        want = oracle.softmax_backward(so, dy)
+        assert got.shape == want.shape and np.allclose(got, want, rtol=1e-5, atol=1e-6), shape

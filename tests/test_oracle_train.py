@@ -44,3 +44,33 @@ def test_adam_first_step_moves_by_lr_against_the_gradient_sign(oracle):
     d0, _, _ = oracle.adam_step(np.ones(3, np.float32), np.zeros(3, np.float32), np.zeros(3, np.float32),
                                 np.zeros(3, np.float32), 0.1, 0.9, 0.999, 1e-6, 1)
     assert np.array_equal(d0, np.ones(3, np.float32))
+
+
+def test_softmax_and_jacobian_loop_nests(oracle):
+    # test/Test.cpp:1823-1832 (softmax) and :1782-1795 (Jacobian), plus what the mathematics fixes
+    rng = np.random.default_rng(4)
+    x = rng.uniform(-10, 10, (2, 3, 12, 1)).astype(np.float32)
+    want = np.empty_like(x)
+    for i in range(2):
+        for j in range(3):
+            e = np.exp(x[i, j, :, 0].astype(np.float64))
+            want[i, j, :, 0] = (e / e.sum()).astype(np.float32)
+    s = oracle.softmax(x)
+    assert np.allclose(s, want, rtol=1e-6, atol=1e-9)
+    assert np.allclose(s.sum(axis=2), 1.0, atol=1e-6)
+    assert np.allclose(oracle.softmax(x + 3.0), s, rtol=1e-5)          # shift invariance
+    J = oracle.softmax_jacobian(s)
+    for i in range(2):
+        for j in range(3):
+            v = s[i, j, :, 0]
+            assert np.array_equal(J[i, j], (np.diag(v * (1 - v)) - np.outer(v, v) * (1 - np.eye(12, dtype=np.float32))).astype(np.float32))
+    assert np.allclose(J.sum(axis=3), 0.0, atol=1e-6)                   # rows of a softmax Jacobian sum to zero
+    assert np.array_equal(J, J.transpose(0, 1, 3, 2))                   # and it is symmetric
+    # row-vector input: same Jacobian, gradient multiplied from the left
+    dy = rng.uniform(-1, 1, (2, 3, 12, 1)).astype(np.float32)
+    col = oracle.softmax_backward(s, dy)
+    row = oracle.softmax_backward(s.reshape(2, 3, 1, 12), dy.reshape(2, 3, 1, 12))
+    assert np.allclose(col.reshape(-1), row.reshape(-1), rtol=1e-6, atol=1e-7)
+    # closed form s * (dy - <s, dy>) within the fp16 rounding of the GEMM operands
+    ref = s * (dy - (s * dy).sum(axis=2, keepdims=True))
+    assert np.allclose(col, ref, atol=2e-3)
