@@ -138,8 +138,8 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC
 // is stored at chunk position  c ^ ((r>>2)&3), which puts the 16 rows that one pass of a
 // 128-bit fragment read touches on 16 different 16-byte bank groups.
 template <int BM, int BN, int WM, int WN, int NSTAGE>
-__global__ __launch_bounds__(WM* WN * 64) void gemm_h16_kernel(const H16Args p) {
-    static_assert(BM == CVT_ROWS && BN == CVT_ROWS, "must match the workspace block image");
+__global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16_kernel(const H16Args p) {
+    static_assert((BM == CVT_ROWS || BM * 2 == CVT_ROWS) && BN == CVT_ROWS, "must match the workspace block image");
     constexpr int BK = CVT_K, ROWB = 64;
     constexpr int NW = WM * WN;
     constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
@@ -183,7 +183,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_h16_kernel(const H16Args p) 
     // share of a stage is A_LOADS + B_LOADS contiguous 1 KiB pieces, lane l taking bytes
     // [16 l, 16 l + 16) of each.
     const int nk = p.Kp / BK;
-    const char* a_tile = reinterpret_cast<const char*>(A) + (long)tile_m * nk * A_BYTES + wave * A_LOADS * 1024 + lane * 16;
+    // a BM = 128 tile is one half of a 256-row block of the image (its 128 physical rows are contiguous)
+    constexpr int A_BLOCK = CVT_ROWS * ROWB, A_PER_BLOCK = CVT_ROWS / BM;
+    const char* a_tile = reinterpret_cast<const char*>(A) + (long)(tile_m / A_PER_BLOCK) * nk * A_BLOCK +
+                         (tile_m % A_PER_BLOCK) * A_BYTES + wave * A_LOADS * 1024 + lane * 16;
     const char* b_tile = reinterpret_cast<const char*>(B) + (long)tile_n * nk * B_BYTES + wave * B_LOADS * 1024 + lane * 16;
 
     // Request k tile kt into ring slot `stage`. Past the end the last tile is requested again
@@ -193,7 +196,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_h16_kernel(const H16Args p) 
         const int kc = kt < nk ? kt : nk - 1;
         char* sa = lds + stage * STAGE + wave * A_LOADS * 1024;
         char* sb = lds + stage * STAGE + A_BYTES + wave * B_LOADS * 1024;
-        const char* ak = a_tile + (long)kc * A_BYTES;
+        const char* ak = a_tile + (long)kc * A_BLOCK;
         const char* bk = b_tile + (long)kc * B_BYTES;
 #pragma unroll
         for (int j = 0; j < A_LOADS; j++)
@@ -364,12 +367,21 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
         hipError_t e = hipGetLastError();
         return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "fp16 rounding pass launch");
     };
-    // Wave grid of the GEMM kernel: WM x 2 waves, each owning 256/WM rows and 128 columns of the tile.
-    // 2 x 2 (one wave per SIMD, 256 accumulators) measures 1-2 % faster than 4 x 2 on 8192^3;
-    // NZHIP_H16_WAVES=8 selects the latter (benchmarking only).
+    // Kernel variants (waves: 0 = choose, 4 / 8 / 2 = force):
+    //   4: 256 x 256 tile, 2 x 2 waves (one wave per SIMD, 256 accumulators), 4-stage ring, 1 workgroup per CU
+    //   8: 256 x 256 tile, 4 x 2 waves (1-2 % slower on 8192^3)
+    //   2: 128 x 256 tile, 2 x 2 waves, 3-stage ring of 72 KiB: two workgroups share a CU, so the output
+    //      stores and ring fill of one overlap the MFMAs of the other -- for products with few tiles
     static const char* waves_env = getenv("NZHIP_H16_WAVES");
-    const int wm_waves = (waves == 8 || (waves == 0 && waves_env && atoi(waves_env) == 8)) ? 4 : 2;
-    int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, 8 / wm_waves);
+    if (waves == 0 && waves_env) waves = atoi(waves_env);
+    if (waves != 2 && waves != 4 && waves != 8) {
+        const long t256 = (Mp / 256) * (Np / 256) * d.batch_n * d.batch_c;
+        waves = t256 < 2 * device_cu_count() ? 2 : 4;
+    }
+    const bool half_m = waves == 2;
+    const int wm_waves = waves == 8 ? 4 : 2;
+    const int fr_a = half_m ? 2 : 8 / wm_waves;
+    int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, fr_a);
     if (rc == NZHIP_OK) rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems, 4);
     if (rc == NZHIP_OK) {
         H16Args a;
@@ -397,11 +409,13 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
         a.bias_sm = d.bias_stride_row;
         a.bias_sk = d.bias_stride_col;
         a.relu = d.activation == NZHIP_ACT_RELU;
-        a.tiles_m = (int)(Mp / BM);
+        a.tiles_m = (int)(Mp / (half_m ? 128 : BM));
         a.tiles_n = (int)(Np / BN);
-        a.group_m = 4;
-        constexpr size_t lds_bytes = (size_t)NSTAGE * (BM + BN) * 64;
-        void (*kfn)(const H16Args) = wm_waves == 4 ? gemm_h16_kernel<BM, BN, 4, 2, NSTAGE> : gemm_h16_kernel<BM, BN, 2, 2, NSTAGE>;
+        a.group_m = half_m ? 8 : 4;
+        const size_t lds_bytes = half_m ? (size_t)3 * (128 + BN) * 64 : (size_t)NSTAGE * (BM + BN) * 64;
+        void (*kfn)(const H16Args) = half_m          ? gemm_h16_kernel<128, BN, 2, 2, 3>
+                                     : wm_waves == 4 ? gemm_h16_kernel<BM, BN, 4, 2, NSTAGE>
+                                                     : gemm_h16_kernel<BM, BN, 2, 2, NSTAGE>;
         if (rc == NZHIP_OK)
             rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(gemm_h16)");
         if (rc == NZHIP_OK) {

@@ -287,15 +287,16 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
 
 /* Test hook: pick the kernel instead of letting the shape decide. tile 128 / 256: the fused
  * convert-on-load kernel with that square tile; tile 16: the two-pass fp16 route (2x2 waves);
- * tile 18: the two-pass route with the 4x2 wave grid. */
+ * tile 18: the two-pass route with the 4x2 wave grid; tile 12: the two-pass route with 128x256 tiles. */
 int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream) {
     if (!desc) return set_error(NZHIP_E_INVALID, "nzhip_gemm: null descriptor");
-    if (tile != 128 && tile != 256 && tile != 16 && tile != 18)
-        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128, 256, 16 or 18");
+    if (tile != 128 && tile != 256 && tile != 16 && tile != 18 && tile != 12)
+        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128, 256, 16, 18 or 12");
     if (int rc = validate_gemm(*desc)) return rc;
     if (desc->M == 0 || desc->N == 0 || desc->K == 0) return nzhip_gemm(desc, stream);
     if (tile == 16) return gemm_h16_dispatch(*desc, as_stream(stream), 4);
     if (tile == 18) return gemm_h16_dispatch(*desc, as_stream(stream), 8);
+    if (tile == 12) return gemm_h16_dispatch(*desc, as_stream(stream), 2);
     return gemm_mfma_dispatch(*desc, as_stream(stream), tile);
 }
 
