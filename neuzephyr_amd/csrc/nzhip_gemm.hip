@@ -36,6 +36,7 @@ struct GemmKernelArgs {
     int relu;
     int tiles_m, tiles_n;
     int group_m;                      // tile rows per rasterisation group
+    int k_total;                      // > 0: member j of the inner batch contracts min(K, k_total - j*K) (split-k chunks)
 };
 
 // Physical LDS row of logical tile row r. A wave owns TR = 32*FR logical rows; its MFMA
@@ -234,10 +235,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    const int nk = (p.K + BK - 1) / BK;
+    // the last chunk of a split contraction may be shorter than the others
+    const int K = (p.k_total > 0 && p.k_total - bj * p.K < p.K) ? p.k_total - bj * p.K : p.K;
+    const int nk = (K + BK - 1) / BK;
 
-    sa.load(A, p.lda, m0, p.M, 0, p.K, tid);
-    sb.load(B, p.ldb, n0, p.N, 0, p.K, tid);
+    sa.load(A, p.lda, m0, p.M, 0, K, tid);
+    sb.load(B, p.ldb, n0, p.N, 0, K, tid);
     sa.store(lds, tid);
     sb.store(lds + A_BYTES, tid);
     __syncthreads();
@@ -247,8 +250,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
         char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
         const bool more = kt + 1 < nk;
         if (more) {
-            sa.load(A, p.lda, m0, p.M, (kt + 1) * BK, p.K, tid);
-            sb.load(B, p.ldb, n0, p.N, (kt + 1) * BK, p.K, tid);
+            sa.load(A, p.lda, m0, p.M, (kt + 1) * BK, K, tid);
+            sb.load(B, p.ldb, n0, p.N, (kt + 1) * BK, K, tid);
         }
         const char* la = cur + ((wm * FM) * 32 + li) * ROWB + lh * 16;
         const char* lb = cur + A_BYTES + ((wn * FN) * 32 + li) * ROWB + lh * 16;
@@ -329,7 +332,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
 // ---- host-side selection -------------------------------------------------------------------
 template <int BM, int BN, int BK, int WM, int WN>
 static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool vec, int batch, hipStream_t s) {
-    const bool full = vec && a.M % BM == 0 && a.N % BN == 0 && a.K % BK == 0;
+    const bool full = vec && a.M % BM == 0 && a.N % BN == 0 && a.K % BK == 0 && (a.k_total <= 0 || a.k_total % a.K == 0);
     constexpr int ROWB = BK * 2 + 16;
     constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * ROWB;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch, 1), block(WM * WN * 64, 1, 1);
@@ -365,7 +368,7 @@ static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool 
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile) {
+int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile, int64_t k_total) {
     GemmKernelArgs a;
     a.A = d.A;
     a.B = d.B;
@@ -389,6 +392,7 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
     a.bias_sm = d.bias_stride_row;
     a.bias_sk = d.bias_stride_col;
     a.relu = d.activation == NZHIP_ACT_RELU;
+    a.k_total = (int)k_total;
 
     const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
     // 16-byte accesses are legal when every row start is 16-byte aligned and the contiguous

@@ -13,7 +13,9 @@ int set_error(int status, const char* fmt, ...) __attribute__((format(printf, 2,
 int set_hip_error(hipError_t e, const char* what);
 
 // MFMA tile kernels (nzhip_gemm.hip). force_tile: 0 = choose, 128 / 256 = that square tile.
-int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile);
+// k_total > 0: the inner batch members are consecutive chunks of one contraction of that length
+// (d.K is the chunk length; the last member contracts what is left)
+int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile, int64_t k_total = 0);
 // Two-pass route for large products: fp16 rounding pass + fp16 GEMM fed by direct-to-LDS loads
 // (nzhip_gemm_h16.hip).
 bool gemm_h16_applicable(const nzhip_gemm_desc& d);

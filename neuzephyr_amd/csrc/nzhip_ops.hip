@@ -208,15 +208,24 @@ __global__ __launch_bounds__(256) void fill_bias_act_kernel(nzhip_gemm_desc d) {
 }
 
 // ---- split-k for few-tile, long-contraction GEMMs ---------------------------------------------
-// C = act(bias + sum over chunks s of P[s]), chunks added in ascending order by one thread per
-// element, so the result does not depend on scheduling.
+// C = act(bias + sum over chunks s of P[s]). Eight threads share an output: thread q adds the
+// chunks of its contiguous eighth in ascending order, then the eight partial sums are added in
+// ascending q, so the result depends on the number of chunks only, never on scheduling.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(nzhip_gemm_desc d, const float* __restrict__ P, int S) {
-    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    __shared__ float part[8][32];
     const long mn = d.M * d.N;
-    if (t >= mn) return;
+    const int q = threadIdx.x >> 5, tl = threadIdx.x & 31;          // a wave reads two chunk rows of 32 outputs
+    const long t = (long)blockIdx.x * 32 + tl;
+    const int per = (S + 7) / 8, s0 = q * per, s1 = s0 + per < S ? s0 + per : S;
+    float x = 0.f;
+    if (t < mn)
+        for (int s = s0; s < s1; s++) x += P[(long)s * mn + t];
+    part[q][tl] = x;
+    __syncthreads();
+    if (q != 0 || t >= mn) return;
+#pragma unroll
+    for (int k = 1; k < 8; k++) x += part[k][tl];
     const long m = t / d.N, n = t % d.N;
-    float x = P[t];
-    for (int s = 1; s < S; s++) x += P[(long)s * mn + t];
     if (d.bias) x += d.bias[m * d.bias_stride_row + n * d.bias_stride_col];
     if (d.activation == NZHIP_ACT_RELU) x = x > 0.f ? x : 0.f;
     d.C[m * d.ldc + n] = x;
@@ -250,27 +259,21 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
             if (S > d.K / 1024) S = d.K / 1024;
             if (S > 1024) S = 1024;
             const int64_t Kc = ((d.K + S - 1) / S + 31) / 32 * 32;          // chunk length, whole 32-wide k tiles
-            const int64_t full = d.K / Kc, rem = d.K - full * Kc;
-            const int parts = (int)(full + (rem ? 1 : 0));
-            if (full >= 2) {
+            const int parts = (int)((d.K + Kc - 1) / Kc);                    // the last one may be shorter
+            if (parts >= 2) {
                 float* P = nullptr;
                 if (int rc = workspace_alloc(reinterpret_cast<void**>(&P), (size_t)parts * d.M * d.N * sizeof(float), s)) return rc;
-                const int64_t a_step = d.a_layout == NZHIP_LAYOUT_ROW ? Kc : Kc * d.lda;   // next chunk of A / B
-                const int64_t b_step = d.b_layout == NZHIP_LAYOUT_ROW ? Kc * d.ldb : Kc;
                 nzhip_gemm_desc g = d;
                 g.C = P; g.ldc = d.N; g.K = Kc;
-                g.batch_n = 1; g.batch_c = full;
-                g.a_stride_c = a_step; g.b_stride_c = b_step; g.c_stride_c = d.M * d.N;
+                g.batch_n = 1; g.batch_c = parts;
+                g.a_stride_c = d.a_layout == NZHIP_LAYOUT_ROW ? Kc : Kc * d.lda;   // next chunk of A / B
+                g.b_stride_c = d.b_layout == NZHIP_LAYOUT_ROW ? Kc * d.ldb : Kc;
+                g.c_stride_c = d.M * d.N;
                 g.bias = nullptr; g.activation = NZHIP_ACT_NONE;
-                int rc = nzhip_gemm(&g, stream);
-                if (rc == NZHIP_OK && rem) {
-                    g.A = d.A + full * a_step; g.B = d.B + full * b_step; g.C = P + full * d.M * d.N;
-                    g.K = rem; g.batch_c = 1;
-                    g.a_stride_c = g.b_stride_c = g.c_stride_c = 0;
-                    rc = nzhip_gemm(&g, stream);
-                }
+                int rc = gemm_mfma_dispatch(g, s, 0, d.K);
                 if (rc == NZHIP_OK) {
-                    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((d.M * d.N + 255) / 256)), dim3(256), 0, s, d, P, parts);
+                    const long groups = (d.M * d.N + 31) / 32;                   // 32 outputs x 8 chunk lanes per workgroup
+                    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)groups), dim3(256), 0, s, d, P, parts);
                     rc = check_launch("splitk_reduce_kernel");
                 }
                 const int rc2 = workspace_free(P, s);
