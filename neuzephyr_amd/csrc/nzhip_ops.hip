@@ -249,14 +249,15 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
         return check_launch("fill_bias_act_kernel");
     }
     if (gemm_skinny_applicable(d)) return gemm_skinny_dispatch(d, s);
-    // One matrix with few output tiles and a long contraction (weight gradients: K = batch x pixels):
-    // cut K into chunks that run as a batch into a workspace, then add the chunks in order.
-    if (d.batch_n * d.batch_c == 1 && d.K >= 4096) {
+    // One matrix with few output tiles (weight gradients with K = batch x pixels, mid-size products):
+    // a workgroup's k loop is latency-bound, so cut K into chunks that run as a batch into a workspace,
+    // then add the chunks in order.
+    if (d.batch_n * d.batch_c == 1 && d.K >= 512) {
         const int cus = device_cu_count();
         const int64_t tiles = ((d.M + 127) / 128) * ((d.N + 127) / 128);
         if (tiles * 2 <= cus) {
             int64_t S = (2 * cus + tiles - 1) / tiles;
-            if (S > d.K / 1024) S = d.K / 1024;
+            if (S > d.K / 128) S = d.K / 128;                                 // at least four k tiles per chunk
             if (S > 1024) S = 1024;
             const int64_t Kc = ((d.K + S - 1) / S + 31) / 32 * 32;          // chunk length, whole 32-wide k tiles
             const int parts = (int)((d.K + Kc - 1) / Kc);                    // the last one may be shorter
