@@ -12,6 +12,8 @@
 //   * batch (n,c), broadcast strides, bias and ReLU are handled in-kernel.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "nzhip_internal.h"
 
 namespace nzhip {
@@ -224,8 +226,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     const float* __restrict__ B = p.B + bi * p.b_sn + bj * p.b_sc;
     float* __restrict__ C = p.C + bi * p.c_sn + bj * p.c_sc;
 
-    typename StageSelect<A_TRANS, BM, BK, NT, TM, FM, ROWB, VEC, FULL>::type sa;
-    typename StageSelect<!B_TRANS, BN, BK, NT, TN, FN, ROWB, VEC, FULL>::type sb;
+    using StageA = typename StageSelect<A_TRANS, BM, BK, NT, TM, FM, ROWB, VEC, FULL>::type;
+    using StageB = typename StageSelect<!B_TRANS, BN, BK, NT, TN, FN, ROWB, VEC, FULL>::type;
+    // The 128x128 tile has registers to spare for a second staging set per operand: the tile two k
+    // steps ahead is requested while the current one is multiplied, so a request has two MFMA
+    // phases to land before it is converted into LDS. The 256x256 tile (256 accumulator registers
+    // per lane) stages one tile ahead.
+    constexpr bool TWO_AHEAD = BM * BN <= 128 * 128;
+    StageA sa0, sa1;
+    StageB sb0, sb1;
 
     floatx16 acc[FM][FN];
 #pragma unroll
@@ -239,20 +248,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     const int K = (p.k_total > 0 && p.k_total - bj * p.K < p.K) ? p.k_total - bj * p.K : p.K;
     const int nk = (K + BK - 1) / BK;
 
-    sa.load(A, p.lda, m0, p.M, 0, K, tid);
-    sb.load(B, p.ldb, n0, p.N, 0, K, tid);
-    sa.store(lds, tid);
-    sb.store(lds + A_BYTES, tid);
-    __syncthreads();
-
-    for (int kt = 0; kt < nk; kt++) {
-        char* cur = lds + (kt & 1) * STAGE_BYTES;
-        char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
-        const bool more = kt + 1 < nk;
-        if (more) {
-            sa.load(A, p.lda, m0, p.M, (kt + 1) * BK, K, tid);
-            sb.load(B, p.ldb, n0, p.N, (kt + 1) * BK, K, tid);
-        }
+    // LDS-only barrier: waits for this wave's LDS traffic, not for the global requests in flight
+    auto lds_barrier = []() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    // Requests past the last tile repeat the last tile (results unused): the number of requests
+    // per step is the same on every path, so each wait names exactly the set it needs.
+    auto request = [&](StageA& ra, StageB& rb, int kt) {
+        const int kc = kt < nk ? kt : nk - 1;
+        ra.load(A, p.lda, m0, p.M, kc * BK, K, tid);
+        rb.load(B, p.ldb, n0, p.N, kc * BK, K, tid);
+    };
+    auto multiply = [&](const char* cur) {
         const char* la = cur + ((wm * FM) * 32 + li) * ROWB + lh * 16;
         const char* lb = cur + A_BYTES + ((wn * FN) * 32 + li) * ROWB + lh * 16;
 #pragma unroll
@@ -268,11 +273,53 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
                 for (int j = 0; j < FN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
-        if (more) {
-            sa.store(nxt, tid);
-            sb.store(nxt + A_BYTES, tid);
+    };
+    if constexpr (TWO_AHEAD) {
+        // one k step: tile kt is in LDS stage `cur`; `ra/rb` held it and are free again; `qa/qb`
+        // hold tile kt + 1. Steps come in pairs; with an odd tile count the last step only moves
+        // data (requests and stores are issued on every path, the MFMAs are skipped).
+        auto step = [&](int kt, char* cur, char* nxt, StageA& ra, StageB& rb, StageA& qa, StageB& qb) {
+            request(ra, rb, kt + 2);
+            if (kt < nk) multiply(cur);
+            qa.store(nxt, tid);                               // tile kt + 1 (a repeat of the last tile past the end)
+            qb.store(nxt + A_BYTES, tid);
+            lds_barrier();
+        };
+        request(sa0, sb0, 0);
+        request(sa1, sb1, 1);
+        sa0.store(lds, tid);
+        sb0.store(lds + A_BYTES, tid);
+        lds_barrier();
+        char* st0 = lds;
+        char* st1 = lds + STAGE_BYTES;
+        for (int kt = 0; kt < nk; kt += 2) {
+            step(kt, st0, st1, sa0, sb0, sa1, sb1);
+            step(kt + 1, st1, st0, sa1, sb1, sa0, sb0);
         }
+        // the requests issued for tiles past the end are still in flight: take delivery before
+        // the registers are reused by the epilogue
+        __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);
+    } else {
+        sa0.load(A, p.lda, m0, p.M, 0, K, tid);
+        sb0.load(B, p.ldb, n0, p.N, 0, K, tid);
+        sa0.store(lds, tid);
+        sb0.store(lds + A_BYTES, tid);
         __syncthreads();
+        for (int kt = 0; kt < nk; kt++) {
+            char* cur = lds + (kt & 1) * STAGE_BYTES;
+            char* nxt = lds + ((kt + 1) & 1) * STAGE_BYTES;
+            const bool more = kt + 1 < nk;
+            if (more) {
+                sa0.load(A, p.lda, m0, p.M, (kt + 1) * BK, K, tid);
+                sb0.load(B, p.ldb, n0, p.N, (kt + 1) * BK, K, tid);
+            }
+            multiply(cur);
+            if (more) {
+                sa0.store(nxt, tid);
+                sb0.store(nxt + A_BYTES, tid);
+            }
+            __syncthreads();
+        }
     }
 
     // ---- epilogue: bias, activation, predicated (vector when legal) store ------------------
@@ -409,6 +456,8 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
     const int64_t t256 = ((d.M + 255) / 256) * ((d.N + 255) / 256) * batch;
     const int64_t t128 = ((d.M + 127) / 128) * ((d.N + 127) / 128) * batch;
     const bool pads_little = t256 * 4 * 4 <= t128 * 5;               // at most 25 % more padded area
+    static const char* tile_env = getenv("NZHIP_GEMM_TILE");         // 128 | 256: benchmarking only
+    if (!force_tile && tile_env && (atoi(tile_env) == 128 || atoi(tile_env) == 256)) force_tile = atoi(tile_env);
     int tile = force_tile ? force_tile : (t256 >= 192 && pads_little ? 256 : 128);
     const int bm = tile, bn = tile;
     a.tiles_m = (int)((d.M + bm - 1) / bm);

@@ -248,20 +248,36 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
     // MFMAs; then ONE barrier (next tile landed + everybody is done reading this slot), the
     // next tile's first fragments and the refill of this slot are issued under the second
     // half's MFMAs.
+    // Instruction order inside each half is pinned: one LDS read (and, in the second half, one
+    // global request) behind each MFMA, so that their issue slots fall into the 32 cycles the
+    // matrix pipe spends on the MFMA before and the pipe never waits for the wave to get through a
+    // burst of memory instructions.
+    constexpr int NMF = FM * FN, NRD = FM + FN;
     for (int kt = 0; kt < nk; kt++) {
         const int slot = kt % NSTAGE;
         const char* base = lds + slot * STAGE;
         read_frags(base, 1, 1);
         mfma_block(0);
+#pragma unroll
+        for (int i = 0; i < NMF; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 // MFMA
+            if (i < NRD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // LDS read
+        }
         __builtin_amdgcn_sched_barrier(0);      // keep the MFMAs above the waits: they hide the read latency
         wait_vmcnt<(NSTAGE - 2) * LOADS>();    // tile kt+1 has landed (this wave's share)
         wait_lgkmcnt0();                        // this wave's reads of slot kt are complete
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
         const int nslot = (kt + 1) % NSTAGE;
-        if (kt + 1 < nk) read_frags(lds + nslot * STAGE, 0, 0);
+        read_frags(lds + nslot * STAGE, 0, 0);  // after the last tile: a dummy tile, never multiplied
         issue_loads(kt + NSTAGE, slot);
         mfma_block(1);
+#pragma unroll
+        for (int i = 0; i < NMF; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < NRD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            else if (i - NRD < LOADS) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);   // global -> LDS request
+        }
     }
     wait_vmcnt<0>();                            // drain the dummy tail requests before LDS goes away
 
