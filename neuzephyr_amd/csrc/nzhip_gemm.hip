@@ -32,7 +32,8 @@ struct GemmKernelArgs {
     const float* bias;
     int M, N, K;
     long lda, ldb, ldc;
-    int batch_c;                      // inner batch extent (grid.y = batch_n * batch_c)
+    int batch_c;                      // inner batch extent
+    int batch;                        // batch_n * batch_c (the grid holds tiles_m * tiles_n * batch workgroups)
     long a_sn, a_sc, b_sn, b_sc, c_sn, c_sc, bias_sn, bias_sc;
     long bias_sm, bias_sk;            // bias row / column strides
     int relu;
@@ -206,13 +207,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     // ---- which tile: spread consecutive ids over the 8 XCDs, then walk column-major inside
     // groups of group_m tile rows so that the workgroups resident on one XCD share A rows
     // and B columns in that XCD's L2.
+    // The grid is one-dimensional over (batch member, tile), member-major: each XCD gets one
+    // contiguous eighth of that list, so all tiles of a member with few tiles run on the same XCD
+    // and its operands come from HBM once.
     const int total = p.tiles_m * p.tiles_n;
     int lin = blockIdx.x;
     {
+        const int units = total * p.batch;
         const int xcd = lin & 7, q = lin >> 3;
-        const int per = total >> 3, rem = total & 7;
+        const int per = units >> 3, rem = units & 7;
         lin = xcd * per + (xcd < rem ? xcd : rem) + q;
     }
+    const int member = lin / total;
+    lin -= member * total;
     const int group_sz = p.group_m * p.tiles_n;
     const int group = lin / group_sz;
     const int first_m = group * p.group_m;
@@ -221,7 +228,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     const int tile_n = (lin % group_sz) / rows_in_group;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    const int bi = blockIdx.y / p.batch_c, bj = blockIdx.y % p.batch_c;
+    const int bi = member / p.batch_c, bj = member % p.batch_c;
     const float* __restrict__ A = p.A + bi * p.a_sn + bj * p.a_sc;
     const float* __restrict__ B = p.B + bi * p.b_sn + bj * p.b_sc;
     float* __restrict__ C = p.C + bi * p.c_sn + bj * p.c_sc;
@@ -382,7 +389,7 @@ static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool 
     const bool full = vec && a.M % BM == 0 && a.N % BN == 0 && a.K % BK == 0 && (a.k_total <= 0 || a.k_total % a.K == 0);
     constexpr int ROWB = BK * 2 + 16;
     constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * ROWB;
-    dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)batch, 1), block(WM * WN * 64, 1, 1);
+    dim3 grid((unsigned)((int64_t)a.tiles_m * a.tiles_n * batch), 1, 1), block(WM * WN * 64, 1, 1);
 #define NZHIP_LAUNCH(AT, BT, V, F)                                                                       \
     do {                                                                                                 \
         auto kfn = gemm_f16mfma_kernel<BM, BN, BK, WM, WN, AT, BT, V, F>;                                \
@@ -428,6 +435,7 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
     a.ldb = d.ldb;
     a.ldc = d.ldc;
     a.batch_c = (int)d.batch_c;
+    a.batch = (int)(d.batch_n * d.batch_c);
     a.a_sn = d.a_stride_n;
     a.a_sc = d.a_stride_c;
     a.b_sn = d.b_stride_n;
@@ -462,6 +470,8 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
     const int bm = tile, bn = tile;
     a.tiles_m = (int)((d.M + bm - 1) / bm);
     a.tiles_n = (int)((d.N + bn - 1) / bn);
+    if ((int64_t)a.tiles_m * a.tiles_n * batch > 0x7fffffff)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_gemm: more than 2^31 output tiles in one call");
     // rows per rasterisation group: with 32 workgroups resident per XCD aim at a 4x8 footprint
     a.group_m = 4;
     if (tile == 256) return launch_cfg<256, 256, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);

@@ -116,6 +116,7 @@ struct H16Args {
     int M, N, Kp;
     long ldc;
     int batch_c;
+    int batch;                        // batch_n * batch_c
     long a_batch, b_batch;              // workspace strides per batch member (0 = shared operand)
     int a_bcast_n, a_bcast_c, b_bcast_n, b_bcast_c;   // 1 = operand is shared along that batch axis
     int a_cn;                           // extent of A's c axis in the workspace (for indexing)
@@ -157,13 +158,17 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
     const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, lh = lane >> 5;
 
+    // one-dimensional grid over (batch member, tile), member-major, one contiguous eighth per XCD
     const int total = p.tiles_m * p.tiles_n;
     int lin = blockIdx.x;
     {
+        const int units = total * p.batch;
         const int xcd = lin & 7, q = lin >> 3;
-        const int per = total >> 3, rem = total & 7;
+        const int per = units >> 3, rem = units & 7;
         lin = xcd * per + (xcd < rem ? xcd : rem) + q;
     }
+    const int member = lin / total;
+    lin -= member * total;
     const int group_sz = p.group_m * p.tiles_n;
     const int group = lin / group_sz;
     const int first_m = group * p.group_m;
@@ -172,7 +177,7 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
     const int tile_n = (lin % group_sz) / rows_in_group;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-    const int bi = blockIdx.y / p.batch_c, bj = blockIdx.y % p.batch_c;
+    const int bi = member / p.batch_c, bj = member % p.batch_c;
     const long a_idx = (long)(p.a_bcast_n ? 0 : bi) * p.a_cn + (p.a_bcast_c ? 0 : bj);
     const long b_idx = (long)(p.b_bcast_n ? 0 : bi) * p.b_cn + (p.b_bcast_c ? 0 : bj);
     const _Float16* __restrict__ A = p.A + a_idx * p.a_batch;
@@ -410,6 +415,7 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
         a.Kp = (int)Kp;
         a.ldc = d.ldc;
         a.batch_c = (int)d.batch_c;
+        a.batch = (int)(d.batch_n * d.batch_c);
         a.a_batch = (long)a_elems;
         a.b_batch = (long)b_elems;
         a.a_bcast_n = d.a_stride_n == 0;
@@ -435,7 +441,7 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
         if (rc == NZHIP_OK)
             rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(gemm_h16)");
         if (rc == NZHIP_OK) {
-            dim3 grid((unsigned)(a.tiles_m * a.tiles_n), (unsigned)(d.batch_n * d.batch_c));
+            dim3 grid((unsigned)((int64_t)a.tiles_m * a.tiles_n * a.batch));
             hipLaunchKernelGGL(kfn, grid, dim3(wm_waves * 2 * 64), lds_bytes, s, a);
             hipError_t e = hipGetLastError();
             if (e != hipSuccess) rc = set_hip_error(e, "gemm_h16 kernel launch");
