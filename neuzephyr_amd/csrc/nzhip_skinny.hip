@@ -13,6 +13,8 @@
 //              lanes stride k, and the 64 partial sums are folded with cross-lane shuffles.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "nzhip_internal.h"
 
 namespace nzhip {
@@ -212,7 +214,14 @@ __global__ __launch_bounds__(256) void skinny_lk_kernel(const SkinnyArgs p) {
 // ---- host side -------------------------------------------------------------------------------
 bool gemm_skinny_applicable(const nzhip_gemm_desc& d) {
     const int64_t small = d.M < d.N ? d.M : d.N, big = d.M < d.N ? d.N : d.M;
-    return small >= 1 && small <= 8 && big >= 1 && d.batch_n * d.batch_c <= 65535;
+    // A single product with 3 or more skinny rows is faster through the MFMA kernel with the
+    // contraction split over workgroups (4096^2: 20 us for any M <= 8, against 22..35 us here);
+    // with N = 3 that kernel would fall back to scalar loads, so 3 columns stay here. Batched
+    // and short (K < 512) products have no split contraction and keep the streaming kernel up to 8.
+    int64_t lim = (d.batch_n * d.batch_c > 1 || d.K < 512) ? 8 : (d.N < d.M ? 3 : 2);
+    static const char* lim_env = getenv("NZHIP_SKINNY_MAX");            // benchmarking only
+    if (lim_env) lim = atoi(lim_env);
+    return small >= 1 && small <= lim && big >= 1 && d.batch_n * d.batch_c <= 65535;
 }
 
 int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream) {
