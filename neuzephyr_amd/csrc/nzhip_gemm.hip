@@ -459,14 +459,14 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
                      ok4(d.b_stride_n) && ok4(d.b_stride_c) && ok4(d.c_stride_n) && ok4(d.c_stride_c);
     const int64_t batch = d.batch_n * d.batch_c;
 
-    // Tile choice: 256x256 tiles need enough of them to fill the 256 CUs and must not pad the
-    // matrix much more than 128x128 tiles would (the padding is computed and thrown away).
+    // Tile choice: 256x256 tiles need enough of them to fill the 256 CUs and pay only in their
+    // unpredicated instance (5000x1000x5000: 379 us with predicated 256x256 tiles, 156 us with
+    // 128x128 tiles).
     const int64_t t256 = ((d.M + 255) / 256) * ((d.N + 255) / 256) * batch;
-    const int64_t t128 = ((d.M + 127) / 128) * ((d.N + 127) / 128) * batch;
-    const bool pads_little = t256 * 4 * 4 <= t128 * 5;               // at most 25 % more padded area
+    const bool whole256 = vec && d.M % 256 == 0 && d.N % 256 == 0 && d.K % 32 == 0 && (k_total <= 0 || k_total % d.K == 0);
     static const char* tile_env = getenv("NZHIP_GEMM_TILE");         // 128 | 256: benchmarking only
     if (!force_tile && tile_env && (atoi(tile_env) == 128 || atoi(tile_env) == 256)) force_tile = atoi(tile_env);
-    int tile = force_tile ? force_tile : (t256 >= 192 && pads_little ? 256 : 128);
+    int tile = force_tile ? force_tile : (t256 >= 192 && whole256 ? 256 : 128);
     const int bm = tile, bn = tile;
     a.tiles_m = (int)((d.M + bm - 1) / bm);
     a.tiles_n = (int)((d.N + bn - 1) / bn);

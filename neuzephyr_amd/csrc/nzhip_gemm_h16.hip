@@ -345,14 +345,18 @@ static inline long round_up(long v, long q) { return (v + q - 1) / q * q; }
 
 bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
     // Worth it when each operand element is re-read by many tiles, i.e. when the GEMM does far
-    // more work per operand byte than the extra rounding pass moves.
+    // more work per operand byte than the extra rounding pass moves. Measured on MI355X
+    // (microseconds, fused / two-pass): 4096x1024x4096 66 / 60, 3072^3 136 / 102, 4096^3 197 / 163,
+    // but 2048^3 44 / 53, 4096x256x4096 30 / 36, 8192x512x8192 160 / 168 (short contractions leave
+    // the rounding pass and the C stores nothing to hide behind). Shapes that are not whole
+    // 256x256x32 tiles take the fused kernel's predicated instance, which is much slower, so the
+    // threshold is lower for them: 2500^3 101 / 68, 5000x1000x5000 156 / 94, 2000^3 56 / 55.
+    if (d.M < 512 || d.N < 512 || d.K < 768) return false;
     const double flops = 2.0 * d.M * d.N * d.K;
     const double cvt_bytes = 6.0 * ((double)d.M * d.K + (double)d.N * d.K);
-    if (d.M < 512 || d.N < 512 || d.K < 256) return false;
-    // Measured on MI355X: the fused convert-on-load kernel saturates the vector memory path at
-    // about 0.65 PFLOP/s (fp32 tiles are twice the bytes), the fp16 kernel runs at about
-    // 1.1 PFLOP/s; the rounding pass pays for itself above roughly 500 flop per byte it moves.
-    return flops / cvt_bytes >= 512.0;
+    const bool whole_tiles = d.M % 256 == 0 && d.N % 256 == 0 && d.K % 32 == 0 && d.lda % 4 == 0 && d.ldb % 4 == 0 &&
+                             d.ldc % 4 == 0;
+    return flops / cvt_bytes >= (whole_tiles ? 512.0 : 300.0);
 }
 
 int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
