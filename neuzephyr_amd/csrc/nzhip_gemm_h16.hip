@@ -36,16 +36,16 @@ constexpr int CVT_ROWS = 256, CVT_K = 32, CVT_BLOCK_BYTES = CVT_ROWS * CVT_K * 2
 // Physical LDS row of logical tile row r when a wave owns FR consecutive 32-row MFMA blocks of the
 // 256-row tile (FR = 4: two waves along that dimension, FR = 2: four). The rows of a wave are
 // interleaved over its blocks so that one lane ends up with FR adjacent rows / columns.
-__device__ __forceinline__ int phys_row_of(int r, int fr) {
-    const int tr = 32 * fr, w = r / tr, l = r % tr;
-    return (w * fr + (l % fr)) * 32 + (l / fr);
+__device__ __forceinline__ int phys_row_of(int r, int fr, int blk) {
+    const int tr = blk * fr, w = r / tr, l = r % tr;
+    return (w * fr + (l % fr)) * blk + (l / fr);
 }
 
 // K_CONTIG: source element (r, k) at src[r*ld + k]; otherwise at src[k*ld + r].
 template <bool K_CONTIG>
 __global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ dst, const float* __restrict__ src,
                                                         int R, int K, int nkt, long ld, long src_batch,
-                                                        long dst_batch, int vec, int fr) {
+                                                        long dst_batch, int vec, int fr, int blk) {
     __shared__ __attribute__((aligned(16))) char img[CVT_BLOCK_BYTES];
     const int kt = blockIdx.x, rb = blockIdx.y;
     const float* s = src + (long)blockIdx.z * src_batch;
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ d
                 }
             }
             half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-            const int pr = phys_row_of(lr, fr);
+            const int pr = phys_row_of(lr, fr, blk);
             const int pos = (k4 >> 1) ^ ((pr >> 2) & 3);
             *reinterpret_cast<half4_t*>(img + pr * 64 + pos * 16 + (k4 & 1) * 8) = h;
         }
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ d
             }
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int pr = phys_row_of(lr + e, fr);
+                const int pr = phys_row_of(lr + e, fr, blk);
                 const int pos = (kk >> 3) ^ ((pr >> 2) & 3);
                 *reinterpret_cast<_Float16*>(img + pr * 64 + pos * 16 + (kk & 7) * 2) = (_Float16)v[e];
             }
@@ -340,6 +340,217 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
     }
 }
 
+// Same tiles, ring and rasterisation with v_mfma_f32_16x16x32_f16: one MFMA covers the whole 32-wide
+// k tile of a 16-row block, a wave's tile is (TM/16) x (TN/16) blocks. A register-only loop of this
+// instruction sustains 1.9 PFLOP/s on random fp16 data on an MI355X against 1.62 PFLOP/s for
+// 32x32x16 (the chip is power-limited on real data).
+// Image rows are interleaved in 16-row blocks (phys_row_of(r, TM/16 or TN/16, 16)): a lane ends
+// up with TN/16 = 8 adjacent output columns of 4 rows per A block.
+template <int BM, int BN, int WM, int WN, int NSTAGE>
+__global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16x_kernel(const H16Args p) {
+    static_assert((BM == CVT_ROWS || BM * 2 == CVT_ROWS) && BN == CVT_ROWS, "must match the workspace block image");
+    constexpr int BK = CVT_K, ROWB = 64;
+    constexpr int NW = WM * WN;
+    constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 16, FN = TN / 16;
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int A_LOADS = BM / 16 / NW, B_LOADS = BN / 16 / NW;   // wave-wide 1 KiB loads (16 rows) per wave
+    constexpr int LOADS = A_LOADS + B_LOADS;
+    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "tile/wave mismatch");
+    static_assert((NSTAGE - 1) * LOADS < 64, "too many loads in flight for vmcnt");
+    static_assert(FN == 8 && FM % 2 == 0, "the epilogue stores 8 adjacent columns per lane");
+
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int l16 = lane & 15, lq = lane >> 4;
+
+    // one-dimensional grid over (batch member, tile), member-major, one contiguous eighth per XCD
+    const int total = p.tiles_m * p.tiles_n;
+    int lin = blockIdx.x;
+    {
+        const int units = total * p.batch;
+        const int xcd = lin & 7, q = lin >> 3;
+        const int per = units >> 3, rem = units & 7;
+        lin = xcd * per + (xcd < rem ? xcd : rem) + q;
+    }
+    const int member = lin / total;
+    lin -= member * total;
+    const int group_sz = p.group_m * p.tiles_n;
+    const int group = lin / group_sz;
+    const int first_m = group * p.group_m;
+    const int rows_in_group = (p.tiles_m - first_m) < p.group_m ? (p.tiles_m - first_m) : p.group_m;
+    const int tile_m = first_m + (lin % group_sz) % rows_in_group;
+    const int tile_n = (lin % group_sz) / rows_in_group;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const int bi = member / p.batch_c, bj = member % p.batch_c;
+    const long a_idx = (long)(p.a_bcast_n ? 0 : bi) * p.a_cn + (p.a_bcast_c ? 0 : bj);
+    const long b_idx = (long)(p.b_bcast_n ? 0 : bi) * p.b_cn + (p.b_bcast_c ? 0 : bj);
+    const _Float16* __restrict__ A = p.A + a_idx * p.a_batch;
+    const _Float16* __restrict__ B = p.B + b_idx * p.b_batch;
+    float* __restrict__ C = p.C + bi * p.c_sn + bj * p.c_sc;
+
+    const int nk = p.Kp / BK;
+    constexpr int A_BLOCK = CVT_ROWS * ROWB, A_PER_BLOCK = CVT_ROWS / BM;
+    const char* a_tile = reinterpret_cast<const char*>(A) + (long)(tile_m / A_PER_BLOCK) * nk * A_BLOCK +
+                         (tile_m % A_PER_BLOCK) * A_BYTES + wave * A_LOADS * 1024 + lane * 16;
+    const char* b_tile = reinterpret_cast<const char*>(B) + (long)tile_n * nk * B_BYTES + wave * B_LOADS * 1024 + lane * 16;
+
+    // Past the end the last tile is requested again (into a slot nobody reads any more) so that
+    // the number of loads in flight, which the vmcnt waits count on, is the same in every step.
+    auto issue_loads = [&](int kt, int stage) {
+        const int kc = kt < nk ? kt : nk - 1;
+        char* sa = lds + stage * STAGE + wave * A_LOADS * 1024;
+        char* sb = lds + stage * STAGE + A_BYTES + wave * B_LOADS * 1024;
+        const char* ak = a_tile + (long)kc * A_BLOCK;
+        const char* bk = b_tile + (long)kc * B_BYTES;
+#pragma unroll
+        for (int j = 0; j < A_LOADS; j++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(ak + j * 1024),
+                                             (__attribute__((address_space(3))) void*)(sa + j * 1024), 16, 0, 0);
+#pragma unroll
+        for (int j = 0; j < B_LOADS; j++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(bk + j * 1024),
+                                             (__attribute__((address_space(3))) void*)(sb + j * 1024), 16, 0, 0);
+    };
+
+    // Accumulators are named by issue position: on this chip back-to-back MFMAs run fastest when
+    // they walk the accumulator registers in ascending order (register-only loop, random fp16 data:
+    // 1.92 PFLOP/s in that order, 1.73 with a stride of 8 accumulators, 1.41 with a permuted order;
+    // which A / B fragments they take makes no difference). Position t = h*HALF + i*4 + jj is the
+    // product of A block i and B block j = 4h + jj: two passes over the A blocks, each against one
+    // half of the B blocks, so that every fragment is free again at least 29 MFMAs before its next use
+    // and one fragment set is enough.
+    constexpr int HALF = FM * 4, NPOS = 2 * HALF;
+    // request number q (A pieces first, then B pieces) of k tile kt into ring slot `stage`
+    auto issue_load = [&](int kt, int stage, int q) {
+        const int kc = kt < nk ? kt : nk - 1;
+        const bool is_a = q < A_LOADS;
+        const int j = is_a ? q : q - A_LOADS;
+        char* dst = lds + stage * STAGE + (is_a ? 0 : A_BYTES) + (wave * (is_a ? A_LOADS : B_LOADS) + j) * 1024;
+        const char* src = is_a ? a_tile + (long)kc * A_BLOCK + j * 1024 : b_tile + (long)kc * B_BYTES + j * 1024;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    };
+    floatx4 acc[NPOS];
+#pragma unroll
+    for (int t = 0; t < NPOS; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[t][r] = 0.f;
+
+    // fragment addressing: physical row = block*16 + l16, the lane's 8 k values are chunk lq,
+    // stored at chunk position lq ^ ((row>>2)&3)
+    const int frag_off = l16 * ROWB + ((lq ^ ((l16 >> 2) & 3)) << 4);
+    const int a_off = (wm * FM) * 16 * ROWB + frag_off;
+    const int b_off = A_BYTES + (wn * FN) * 16 * ROWB + frag_off;
+
+    half8_t af[FM], bf[FN];
+    auto read_a = [&](const char* base, int i) { af[i] = *reinterpret_cast<const half8_t*>(base + a_off + i * 16 * ROWB); };
+    auto read_b = [&](const char* base, int j) { bf[j] = *reinterpret_cast<const half8_t*>(base + b_off + j * 16 * ROWB); };
+    auto mfma_at = [&](int t) {
+        const int h = t / HALF, i = (t % HALF) / 4, j = 4 * h + (t & 3);
+        // Written as assembly so that the accumulator is updated in place in the accumulation
+        // registers: given the builtin, the register allocator moves a dozen of the 64 accumulators
+        // through a temporary every k tile (four copy instructions per MFMA).
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[t]) : "v"(af[i]), "v"(bf[j]));
+    };
+
+    // prologue: fill the ring, wait for tile 0, read its fragments
+#pragma unroll
+    for (int t = 0; t < NSTAGE; t++) issue_loads(t, t);
+    wait_vmcnt<(NSTAGE - 1) * LOADS>();
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < FN; j++) read_b(lds, j);
+#pragma unroll
+    for (int i = 0; i < FM; i++) read_a(lds, i);
+
+    // One k tile: PRE MFMAs, then ONE barrier (tile kt+1 has landed for every wave, and every
+    // wave has finished reading slot kt: its last reads were issued at the end of the previous
+    // tile), then the refill of slot kt and, as each fragment is used for the last time, the read
+    // of its successor from tile kt+1 — one memory instruction behind one MFMA.
+    constexpr int PRE = 16 < HALF - 4 ? 16 : HALF - 4 - LOADS;
+    static_assert(PRE >= 1 && PRE + LOADS <= HALF - 4, "the refill must be issued before the first fragment is re-read");
+    for (int kt = 0; kt < nk; kt++) {
+        const char* nxt = lds + ((kt + 1) % NSTAGE) * STAGE;   // after the last tile: a dummy tile, never multiplied
+        // a scheduling fence behind every position keeps the instruction order exactly as written
+#pragma unroll
+        for (int t = 0; t < PRE; t++) {
+            mfma_at(t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        wait_vmcnt<(NSTAGE - 2) * LOADS>();    // tile kt+1 has landed (this wave's share)
+        wait_lgkmcnt0();                        // this wave's reads of slot kt are complete
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = PRE; t < NPOS; t++) {
+            mfma_at(t);
+            if (t - PRE < LOADS) issue_load(kt + NSTAGE, kt % NSTAGE, t - PRE);
+            // last use of B block jj of the first half: position HALF - 4 + jj
+            if (t >= HALF - 4 && t < HALF) read_b(nxt, t - (HALF - 4));
+            // last use of A block i: position HALF + 4 i + 3
+            if (t >= HALF && (t & 3) == 3) read_a(nxt, (t - HALF) / 4);
+            // last use of B block 4 + jj: position NPOS - 4 + jj
+            if (t >= NPOS - 4) read_b(nxt, 4 + t - (NPOS - 4));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    wait_vmcnt<0>();                            // drain the dummy tail requests before LDS goes away
+    // the last MFMAs must have left the pipeline before ordinary instructions read their results
+    // (the compiler does not know that the assembly statements above are MFMAs)
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: bias, activation, predicated (vector when legal) store ------------------
+    // Accumulator of (A block i, B block j), register r: row (lq*4 + r) of the block, column l16; with the interleaved
+    // images that is output row wm*TM + (lq*4 + r)*FM + i and output column wn*TN + l16*FN + j.
+    const float* bias = p.bias ? p.bias + bi * p.bias_sn + bj * p.bias_sc : nullptr;
+    const int gn = n0 + wn * TN + l16 * FN;               // first of this lane's FN columns
+    const bool vec_ok = ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 15) == 0) && (gn + FN <= p.N);
+    float bcol[FN];
+    const bool bias_rowless = bias && p.bias_sm == 0;
+#pragma unroll
+    for (int j = 0; j < FN; j++) bcol[j] = (bias_rowless && gn + j < p.N) ? bias[(long)(gn + j) * p.bias_sk] : 0.f;
+#pragma unroll
+    for (int i = 0; i < FM; i++) {
+        float bv[4][FN];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int gm = m0 + wm * TM + (lq * 4 + r) * FM + i;
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                bv[r][j] = (bias && !bias_rowless && gm < p.M && gn + j < p.N)
+                               ? bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk]
+                               : bcol[j];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int gm = m0 + wm * TM + (lq * 4 + r) * FM + i;
+            if (gm >= p.M) continue;
+            float v[FN];
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                float x = acc[(j >> 2) * HALF + i * 4 + (j & 3)][r] + bv[r][j];
+                if (p.relu) x = x > 0.f ? x : 0.f;
+                v[j] = x;
+            }
+            float* dst = C + (long)gm * p.ldc + gn;
+            if (vec_ok) {
+                floatx4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
+                *reinterpret_cast<floatx4*>(dst) = o0;
+                *reinterpret_cast<floatx4*>(dst + 4) = o1;
+            } else {
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+                    if (gn + j < p.N) dst[j] = v[j];
+            }
+        }
+    }
+}
+
 // ---- host side -----------------------------------------------------------------------------
 static inline long round_up(long v, long q) { return (v + q - 1) / q * q; }
 
@@ -359,7 +570,7 @@ bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
     return flops / cvt_bytes >= (whole_tiles ? 512.0 : 300.0);
 }
 
-int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
+int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mfma) {
     constexpr int BM = 256, BN = 256, BK = 32, NSTAGE = 4;
     const long Mp = round_up(d.M, BM), Np = round_up(d.N, BN), Kp = round_up(d.K, BK);
     const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
@@ -375,7 +586,7 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
 
     const int nkt = (int)(Kp / BK);
     auto convert = [&](_Float16* dst, const float* src, long R, long Rp, bool k_contig, long ld, long nb, long cb,
-                       long sn, long sc, size_t elems, int fr) -> int {
+                       long sn, long sc, size_t elems, int fr, int blk) -> int {
         for (long i = 0; i < nb; i++) {
             // the c axis of one n is a plain strided batch -> one launch per n
             const float* sp = src + i * sn;
@@ -384,30 +595,38 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
             dim3 grid((unsigned)nkt, (unsigned)(Rp / CVT_ROWS), (unsigned)cb);
             if (k_contig)
                 hipLaunchKernelGGL(cvt_block_kernel<true>, grid, dim3(256), 0, s, dp, sp, (int)R, (int)d.K, nkt, ld, sc,
-                                   (long)elems, vec, fr);
+                                   (long)elems, vec, fr, blk);
             else
                 hipLaunchKernelGGL(cvt_block_kernel<false>, grid, dim3(256), 0, s, dp, sp, (int)R, (int)d.K, nkt, ld, sc,
-                                   (long)elems, vec, fr);
+                                   (long)elems, vec, fr, blk);
         }
         hipError_t e = hipGetLastError();
         return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "fp16 rounding pass launch");
     };
     // Kernel variants (waves: 0 = choose, 4 / 8 / 2 = force):
+    //   8: 256 x 256 tile, 4 x 2 waves (two per SIMD, 128 accumulators each): the memory instructions of one
+    //      wave issue under the MFMAs of the other (8192^3 with 16x16x32: 1.08 ms against 1.10 ms with 4 waves)
     //   4: 256 x 256 tile, 2 x 2 waves (one wave per SIMD, 256 accumulators), 4-stage ring, 1 workgroup per CU
-    //   8: 256 x 256 tile, 4 x 2 waves (1-2 % slower on 8192^3)
     //   2: 128 x 256 tile, 2 x 2 waves, 3-stage ring of 72 KiB: two workgroups share a CU, so the output
     //      stores and ring fill of one overlap the MFMAs of the other -- for products with few tiles
+    // mfma: 0 = choose (16), 16 = v_mfma_f32_16x16x32_f16, 32 = v_mfma_f32_32x32x16_f16 (8192^3: 1.10 / 1.13 ms
+    // with 4 waves; the 32x32x16 loop is kept for comparison).
     static const char* waves_env = getenv("NZHIP_H16_WAVES");
     if (waves == 0 && waves_env) waves = atoi(waves_env);
+    static const char* mfma_env = getenv("NZHIP_H16_MFMA");             // 16 | 32: benchmarking only
+    if (mfma == 0 && mfma_env) mfma = atoi(mfma_env);
+    const bool mf16 = mfma != 32;
     if (waves != 2 && waves != 4 && waves != 8) {
         const long t256 = (Mp / 256) * (Np / 256) * d.batch_n * d.batch_c;
-        waves = t256 < 2 * device_cu_count() ? 2 : 4;
+        waves = t256 < 2 * device_cu_count() ? 2 : (mf16 ? 8 : 4);
     }
     const bool half_m = waves == 2;
     const int wm_waves = waves == 8 ? 4 : 2;
-    const int fr_a = half_m ? 2 : 8 / wm_waves;
-    int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, fr_a);
-    if (rc == NZHIP_OK) rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems, 4);
+    const int blk = mf16 ? 16 : 32;                                     // rows per MFMA block
+    const int fr_a = (half_m ? 64 : 256 / wm_waves) / blk, fr_b = 128 / blk;   // blocks per wave tile
+    int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, fr_a, blk);
+    if (rc == NZHIP_OK)
+        rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems, fr_b, blk);
     if (rc == NZHIP_OK) {
         H16Args a;
         a.A = Ah;
@@ -442,6 +661,10 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves) {
         void (*kfn)(const H16Args) = half_m          ? gemm_h16_kernel<128, BN, 2, 2, 3>
                                      : wm_waves == 4 ? gemm_h16_kernel<BM, BN, 4, 2, NSTAGE>
                                                      : gemm_h16_kernel<BM, BN, 2, 2, NSTAGE>;
+        if (mf16)
+            kfn = half_m          ? gemm_h16x_kernel<128, BN, 2, 2, 3>
+                  : wm_waves == 4 ? gemm_h16x_kernel<BM, BN, 4, 2, NSTAGE>
+                                  : gemm_h16x_kernel<BM, BN, 2, 2, NSTAGE>;
         if (rc == NZHIP_OK)
             rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(gemm_h16)");
         if (rc == NZHIP_OK) {

@@ -290,17 +290,20 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
 }
 
 /* Test hook: pick the kernel instead of letting the shape decide. tile 128 / 256: the fused
- * convert-on-load kernel with that square tile; tile 16: the two-pass fp16 route (2x2 waves);
- * tile 18: the two-pass route with the 4x2 wave grid; tile 12: the two-pass route with 128x256 tiles. */
+ * convert-on-load kernel with that square tile; tile 16 / 18 / 12: the two-pass fp16 route with
+ * 256x256 tiles and 4 waves / 256x256 tiles and 8 waves / 128x256 tiles, 16x16x32 MFMAs;
+ * tile 316 / 318 / 312: the same three with 32x32x16 MFMAs. */
 int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream) {
     if (!desc) return set_error(NZHIP_E_INVALID, "nzhip_gemm: null descriptor");
-    if (tile != 128 && tile != 256 && tile != 16 && tile != 18 && tile != 12)
-        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128, 256, 16, 18 or 12");
+    const int base = tile > 300 ? tile - 300 : tile;
+    if (tile != 128 && tile != 256 && base != 16 && base != 18 && base != 12)
+        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128, 256, 16, 18, 12, 316, 318 or 312");
     if (int rc = validate_gemm(*desc)) return rc;
     if (desc->M == 0 || desc->N == 0 || desc->K == 0) return nzhip_gemm(desc, stream);
-    if (tile == 16) return gemm_h16_dispatch(*desc, as_stream(stream), 4);
-    if (tile == 18) return gemm_h16_dispatch(*desc, as_stream(stream), 8);
-    if (tile == 12) return gemm_h16_dispatch(*desc, as_stream(stream), 2);
+    const int mfma = tile > 300 ? 32 : 16;
+    if (base == 16) return gemm_h16_dispatch(*desc, as_stream(stream), 4, mfma);
+    if (base == 18) return gemm_h16_dispatch(*desc, as_stream(stream), 8, mfma);
+    if (base == 12) return gemm_h16_dispatch(*desc, as_stream(stream), 2, mfma);
     return gemm_mfma_dispatch(*desc, as_stream(stream), tile);
 }
 

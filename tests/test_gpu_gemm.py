@@ -63,7 +63,7 @@ SHAPES = [(1, 1, 1), (3, 5, 2), (16, 16, 16), (17, 33, 15), (64, 100, 132), (130
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
 @pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("tile", [128, 256, 16, 18, 12])  # fused kernels with that tile; 16 / 18 / 12 = two-pass fp16 route variants
+@pytest.mark.parametrize("tile", [128, 256, 16, 18, 12, 316, 318, 312])  # fused kernels with that tile; 16 / 18 / 12 = two-pass fp16 route variants (16x16x32 MFMAs), 3xx = the same with 32x32x16
 def test_integer_operands_are_bit_exact(nz, M, K, N, a_trans, b_trans, tile):
     rng = np.random.default_rng(M * 7919 + K * 31 + N)
     A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
