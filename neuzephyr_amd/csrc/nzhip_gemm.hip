@@ -235,11 +235,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
 
     using StageA = typename StageSelect<A_TRANS, BM, BK, NT, TM, FM, ROWB, VEC, FULL>::type;
     using StageB = typename StageSelect<!B_TRANS, BN, BK, NT, TN, FN, ROWB, VEC, FULL>::type;
-    // The 128x128 tile has registers to spare for a second staging set per operand: the tile two k
-    // steps ahead is requested while the current one is multiplied, so a request has two MFMA
-    // phases to land before it is converted into LDS. The 256x256 tile (256 accumulator registers
-    // per lane) stages one tile ahead.
-    constexpr bool TWO_AHEAD = BM * BN <= 128 * 128;
+    // With 128 or fewer accumulator registers per lane (128x128 tiles, or 256x256 tiles on eight waves)
+    // there is room for a second staging set per operand: the tile two k steps ahead is requested
+    // while the current one is multiplied, so a request has two MFMA phases to land before it is
+    // converted into LDS. The 256x256 tile on four waves (256 accumulator registers per lane) stages
+    // one tile ahead.
+    constexpr bool TWO_AHEAD = BM * BN <= 128 * 128 || WM * WN >= 8;
     StageA sa0, sa1;
     StageB sb0, sb1;
 
@@ -474,7 +475,13 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
         return set_error(NZHIP_E_UNSUPPORTED, "nzhip_gemm: more than 2^31 output tiles in one call");
     // rows per rasterisation group: with 32 workgroups resident per XCD aim at a 4x8 footprint
     a.group_m = 4;
-    if (tile == 256) return launch_cfg<256, 256, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
+    // 256x256 tiles run with 4 x 2 waves (two per SIMD, 128 accumulators each): that leaves registers for
+    // the second staging set, and one wave converts while the other multiplies (batched 128 x 1024^3:
+    // 0.63 ms with 2 x 2 waves, 0.55 ms with 4 x 2). NZHIP_GEMM_WAVES=4 selects 2 x 2 (benchmarking only).
+    static const char* waves_env = getenv("NZHIP_GEMM_WAVES");
+    if (tile == 256 && waves_env && atoi(waves_env) == 4)
+        return launch_cfg<256, 256, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
+    if (tile == 256) return launch_cfg<256, 256, 32, 4, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
     return launch_cfg<128, 128, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
 }
 
