@@ -423,6 +423,17 @@ static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool 
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// 16-byte accesses are legal when every row start is 16-byte aligned and the contiguous extent is
+// a multiple of 4, for every batch member.
+bool gemm_vec_legal(const nzhip_gemm_desc& d) {
+    const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
+    auto ok4 = [](int64_t v) { return (v & 3) == 0; };
+    const int64_t a_contig = a_trans ? d.M : d.K, b_contig = b_trans ? d.K : d.N;
+    return aligned16(d.A) && aligned16(d.B) && aligned16(d.C) && ok4(d.lda) && ok4(d.ldb) && ok4(d.ldc) &&
+           ok4(a_contig) && ok4(b_contig) && ok4(d.N) && ok4(d.a_stride_n) && ok4(d.a_stride_c) &&
+           ok4(d.b_stride_n) && ok4(d.b_stride_c) && ok4(d.c_stride_n) && ok4(d.c_stride_c);
+}
+
 int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile, int64_t k_total) {
     GemmKernelArgs a;
     a.A = d.A;
@@ -451,13 +462,7 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
     a.k_total = (int)k_total;
 
     const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
-    // 16-byte accesses are legal when every row start is 16-byte aligned and the contiguous
-    // extent is a multiple of 4, for every batch member.
-    auto ok4 = [](int64_t v) { return (v & 3) == 0; };
-    const int64_t a_contig = a_trans ? d.M : d.K, b_contig = b_trans ? d.K : d.N;
-    const bool vec = aligned16(d.A) && aligned16(d.B) && aligned16(d.C) && ok4(d.lda) && ok4(d.ldb) && ok4(d.ldc) &&
-                     ok4(a_contig) && ok4(b_contig) && ok4(d.N) && ok4(d.a_stride_n) && ok4(d.a_stride_c) &&
-                     ok4(d.b_stride_n) && ok4(d.b_stride_c) && ok4(d.c_stride_n) && ok4(d.c_stride_c);
+    const bool vec = gemm_vec_legal(d);
     const int64_t batch = d.batch_n * d.batch_c;
 
     // Tile choice: 256x256 tiles need enough of them to fill the 256 CUs and pay only in their

@@ -19,6 +19,7 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
 // Two-pass route for large products: fp16 rounding pass + fp16 GEMM fed by direct-to-LDS loads
 // (nzhip_gemm_h16.hip).
 bool gemm_h16_applicable(const nzhip_gemm_desc& d);
+bool gemm_vec_legal(const nzhip_gemm_desc& d);   // 16-byte global accesses are legal for A, B and C
 // waves: 0 = choose, else 2 / 4 / 8; mfma: 0 = choose, else 16 (16x16x32) / 32 (32x32x16)
 int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int waves = 0, int mfma = 0);
 // Bandwidth-bound kernels for M <= 8 (nzhip_skinny.hip).

@@ -231,6 +231,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(nzhip_gemm_desc d, c
     d.C[m * d.ldc + n] = x;
 }
 
+// The same sum for few chunks and many outputs: one thread per output adds its chunks in ascending
+// order (coalesced along the outputs).
+__global__ __launch_bounds__(256) void splitk_reduce_wide_kernel(nzhip_gemm_desc d, const float* __restrict__ P, int S) {
+    const long mn = d.M * d.N;
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= mn) return;
+    float x = 0.f;
+    for (int s = 0; s < S; s++) x += P[(long)s * mn + t];
+    const long m = t / d.N, n = t % d.N;
+    if (d.bias) x += d.bias[m * d.bias_stride_row + n * d.bias_stride_col];
+    if (d.activation == NZHIP_ACT_RELU) x = x > 0.f ? x : 0.f;
+    d.C[m * d.ldc + n] = x;
+}
+
 }  // namespace nzhip
 
 using namespace nzhip;
@@ -250,15 +264,23 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
     }
     if (gemm_skinny_applicable(d)) return gemm_skinny_dispatch(d, s);
     // One matrix with few output tiles (weight gradients with K = batch x pixels, mid-size products):
-    // a workgroup's k loop is latency-bound, so cut K into chunks that run as a batch into a workspace,
-    // then add the chunks in order.
+    // a workgroup's k loop is latency-bound (about 0.55 us per 32-wide k tile with 16-byte loads, 2 us
+    // without), so cut K into chunks that run as a batch into a workspace, then add the chunks in
+    // order. The extra pass over the partial sums costs 5..15 us, so a chunk keeps at least 512 of
+    // the contraction when loads are vectorised (1024^3: 23 us unsplit, 31 us in two chunks;
+    // 1024x4096x1024: 71 us unsplit, 39 us in eight chunks) and 128 otherwise.
     if (d.batch_n * d.batch_c == 1 && d.K >= 512) {
         const int cus = device_cu_count();
         const int64_t tiles = ((d.M + 127) / 128) * ((d.N + 127) / 128);
         if (tiles * 2 <= cus) {
+            const bool narrow = d.M <= 64 || d.N <= 64;            // padded tiles: the k loop is shorter per byte
+            const int64_t min_chunk = gemm_vec_legal(d) && !narrow ? 512 : 128;
             int64_t S = (2 * cus + tiles - 1) / tiles;
-            if (S > d.K / 128) S = d.K / 128;                                 // at least four k tiles per chunk
+            if (S > d.K / min_chunk) S = d.K / min_chunk;
             if (S > 1024) S = 1024;
+            static const char* sk_env = getenv("NZHIP_SPLITK");                  // benchmarking only
+            if (sk_env && atoi(sk_env) >= 1) S = atoi(sk_env);
+            if (S < 1) S = 1;
             const int64_t Kc = ((d.K + S - 1) / S + 31) / 32 * 32;          // chunk length, whole 32-wide k tiles
             const int parts = (int)((d.K + Kc - 1) / Kc);                    // the last one may be shorter
             if (parts >= 2) {
@@ -273,8 +295,13 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
                 g.bias = nullptr; g.activation = NZHIP_ACT_NONE;
                 int rc = gemm_mfma_dispatch(g, s, 0, d.K);
                 if (rc == NZHIP_OK) {
-                    const long groups = (d.M * d.N + 31) / 32;                   // 32 outputs x 8 chunk lanes per workgroup
-                    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)groups), dim3(256), 0, s, d, P, parts);
+                    if (parts > 16 || d.M * d.N < (1 << 18)) {                  // few outputs: spread each over eight lanes
+                        const long groups = (d.M * d.N + 31) / 32;               // 32 outputs x 8 chunk lanes per workgroup
+                        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)groups), dim3(256), 0, s, d, P, parts);
+                    } else {
+                        const long groups = (d.M * d.N + 255) / 256;
+                        hipLaunchKernelGGL(splitk_reduce_wide_kernel, dim3((unsigned)groups), dim3(256), 0, s, d, P, parts);
+                    }
                     rc = check_launch("splitk_reduce_kernel");
                 }
                 const int rc2 = workspace_free(P, s);
