@@ -111,6 +111,40 @@ def test_long_contractions_with_few_tiles_are_bit_exact_on_integers(nz, M, K, N,
     assert np.array_equal(got, expect)
 
 
+def _route_sweep_cases():
+    # seeded shapes aimed at the boundaries of the route choice: skinny extents 1..9 on either side,
+    # long contractions with few tiles (split or not, vectorisable or not), mid-size and ragged shapes,
+    # and two shapes big enough for the two-pass route under the default rule
+    rng = np.random.default_rng(20240607)
+    cases = []
+    for _ in range(10):
+        cases.append((int(rng.integers(1, 10)), int(rng.integers(400, 3000)), int(rng.integers(100, 1500))))
+        cases.append((int(rng.integers(100, 1500)), int(rng.integers(400, 3000)), int(rng.integers(1, 10))))
+    for _ in range(10):
+        cases.append((int(rng.integers(10, 400)), int(rng.integers(500, 6000)), int(rng.integers(10, 400))))
+        cases.append((4 * int(rng.integers(3, 100)), 4 * int(rng.integers(128, 1500)), 4 * int(rng.integers(3, 100))))
+    for _ in range(6):
+        cases.append((int(rng.integers(200, 900)), int(rng.integers(30, 700)), int(rng.integers(200, 900))))
+    cases += [(1800, 800, 1804), (1024, 1024, 1024), (512, 768, 2048), (1792, 1024, 1792)]
+    return cases
+
+
+@pytest.mark.parametrize("M,K,N", _route_sweep_cases())
+def test_default_route_is_bit_exact_on_integers(nz, M, K, N):
+    # no forced kernel: whatever nzhip_gemm picks for the shape must give the exact integer product
+    rng = np.random.default_rng(M * 1009 + K * 17 + N)
+    a_trans, b_trans = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    A = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, size=(K, N)).astype(np.float32)
+    bias = rng.integers(-50, 51, size=(N,)).astype(np.float32)
+    # float64 BLAS is exact here: |sum| <= 16 K < 2^53
+    expect = np.maximum((A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32) + bias[None, :], 0)
+    got = host(nz.gemm(dev(np.ascontiguousarray(A.T) if a_trans else A), dev(np.ascontiguousarray(B.T) if b_trans else B),
+                       a_trans=a_trans, b_trans=b_trans, bias=dev(bias), bias_strides=(0, 1), relu=True))
+    assert np.array_equal(got, expect)
+
+
+
 def test_skinny_batched_linear_single_sample(nz, oracle):
     # one sample through Model::Linear: W[1,1,OUT,IN] x[1,1,IN,1]
     OUT, IN = 1000, 515
