@@ -42,13 +42,20 @@ __device__ __forceinline__ int phys_row_of(int r, int fr, int blk) {
 }
 
 // K_CONTIG: source element (r, k) at src[r*ld + k]; otherwise at src[k*ld + r].
+struct CvtOperand {
+    _Float16* dst;
+    const float* src;
+    int R;                      // rows of the operand (output rows for A, output columns for B)
+    long ld, src_batch, dst_batch;
+    int vec, fr;
+};
+
 template <bool K_CONTIG>
-__global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ dst, const float* __restrict__ src,
-                                                        int R, int K, int nkt, long ld, long src_batch,
-                                                        long dst_batch, int vec, int fr, int blk) {
-    __shared__ __attribute__((aligned(16))) char img[CVT_BLOCK_BYTES];
-    const int kt = blockIdx.x, rb = blockIdx.y;
-    const float* s = src + (long)blockIdx.z * src_batch;
+__device__ __forceinline__ void cvt_block(char* img, const CvtOperand& o, int K, int nkt, int blk, int kt, int rb, int member) {
+    _Float16* dst = o.dst;
+    const int R = o.R, vec = o.vec, fr = o.fr;
+    const long ld = o.ld, dst_batch = o.dst_batch;
+    const float* s = o.src + (long)member * o.src_batch;
     const int t = threadIdx.x;
     const int r0 = rb * CVT_ROWS, k0 = kt * CVT_K;
     if (K_CONTIG) {
@@ -99,12 +106,30 @@ __global__ __launch_bounds__(256) void cvt_block_kernel(_Float16* __restrict__ d
         }
     }
     __syncthreads();
-    char* out = reinterpret_cast<char*>(dst + (long)blockIdx.z * dst_batch) + ((long)rb * nkt + kt) * CVT_BLOCK_BYTES;
+    char* out = reinterpret_cast<char*>(dst + (long)member * dst_batch) + ((long)rb * nkt + kt) * CVT_BLOCK_BYTES;
 #pragma unroll
     for (int pass = 0; pass < 4; pass++) {
         const int off = (pass * 256 + t) * 16;
         *reinterpret_cast<floatx4*>(out + off) = *reinterpret_cast<const floatx4*>(img + off);
     }
+}
+
+template <bool K_CONTIG>
+__global__ __launch_bounds__(256) void cvt_block_kernel(CvtOperand o, int K, int nkt, int blk) {
+    __shared__ __attribute__((aligned(16))) char img[CVT_BLOCK_BYTES];
+    cvt_block<K_CONTIG>(img, o, K, nkt, blk, blockIdx.x, blockIdx.y, blockIdx.z);
+}
+
+// Both operands in one launch (the usual case: neither is batched differently from the other): row
+// blocks [0, a_blocks) of the grid's y axis belong to A, the rest to B.
+template <bool A_K_CONTIG, bool B_K_CONTIG>
+__global__ __launch_bounds__(256) void cvt_pair_kernel(CvtOperand a, CvtOperand b, int a_blocks, int K, int nkt, int blk) {
+    __shared__ __attribute__((aligned(16))) char img[CVT_BLOCK_BYTES];
+    const int rb = blockIdx.y;
+    if (rb < a_blocks)
+        cvt_block<A_K_CONTIG>(img, a, K, nkt, blk, blockIdx.x, rb, blockIdx.z);
+    else
+        cvt_block<B_K_CONTIG>(img, b, K, nkt, blk, blockIdx.x, rb - a_blocks, blockIdx.z);
 }
 
 // ---- pass 2: fp16 GEMM -----------------------------------------------------------------------
@@ -585,21 +610,43 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mf
     _Float16* Bh = ws + a_total;
 
     const int nkt = (int)(Kp / BK);
+    auto operand = [&](_Float16* dst, const float* src, long R, long ld, long sc, size_t elems, int fr) {
+        CvtOperand o;
+        o.dst = dst;
+        o.src = src;
+        o.R = (int)R;
+        o.ld = ld;
+        o.src_batch = sc;
+        o.dst_batch = (long)elems;
+        o.vec = ((ld & 3) == 0) && ((reinterpret_cast<uintptr_t>(src) & 15) == 0) && ((sc & 3) == 0);
+        o.fr = fr;
+        return o;
+    };
     auto convert = [&](_Float16* dst, const float* src, long R, long Rp, bool k_contig, long ld, long nb, long cb,
                        long sn, long sc, size_t elems, int fr, int blk) -> int {
         for (long i = 0; i < nb; i++) {
             // the c axis of one n is a plain strided batch -> one launch per n
-            const float* sp = src + i * sn;
-            _Float16* dp = dst + (size_t)i * cb * elems;
-            const int vec = ((ld & 3) == 0) && ((reinterpret_cast<uintptr_t>(sp) & 15) == 0) && ((sc & 3) == 0);
+            const CvtOperand o = operand(dst + (size_t)i * cb * elems, src + i * sn, R, ld, sc, elems, fr);
             dim3 grid((unsigned)nkt, (unsigned)(Rp / CVT_ROWS), (unsigned)cb);
             if (k_contig)
-                hipLaunchKernelGGL(cvt_block_kernel<true>, grid, dim3(256), 0, s, dp, sp, (int)R, (int)d.K, nkt, ld, sc,
-                                   (long)elems, vec, fr, blk);
+                hipLaunchKernelGGL(cvt_block_kernel<true>, grid, dim3(256), 0, s, o, (int)d.K, nkt, blk);
             else
-                hipLaunchKernelGGL(cvt_block_kernel<false>, grid, dim3(256), 0, s, dp, sp, (int)R, (int)d.K, nkt, ld, sc,
-                                   (long)elems, vec, fr, blk);
+                hipLaunchKernelGGL(cvt_block_kernel<false>, grid, dim3(256), 0, s, o, (int)d.K, nkt, blk);
         }
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "fp16 rounding pass launch");
+    };
+    // both operands in one launch when they have the same batch structure (one n, equal c extents)
+    auto convert_pair = [&](int fr_a, int fr_b, int blk) -> int {
+        const CvtOperand oa = operand(Ah, d.A, d.M, d.lda, d.a_stride_c, a_elems, fr_a);
+        const CvtOperand ob = operand(Bh, d.B, d.N, d.ldb, d.b_stride_c, b_elems, fr_b);
+        const int a_blocks = (int)(Mp / CVT_ROWS), b_blocks = (int)(Np / CVT_ROWS);
+        dim3 grid((unsigned)nkt, (unsigned)(a_blocks + b_blocks), (unsigned)a_c);
+        const bool ka = !a_trans, kb = b_trans;
+        if (ka && kb) hipLaunchKernelGGL((cvt_pair_kernel<true, true>), grid, dim3(256), 0, s, oa, ob, a_blocks, (int)d.K, nkt, blk);
+        else if (ka) hipLaunchKernelGGL((cvt_pair_kernel<true, false>), grid, dim3(256), 0, s, oa, ob, a_blocks, (int)d.K, nkt, blk);
+        else if (kb) hipLaunchKernelGGL((cvt_pair_kernel<false, true>), grid, dim3(256), 0, s, oa, ob, a_blocks, (int)d.K, nkt, blk);
+        else hipLaunchKernelGGL((cvt_pair_kernel<false, false>), grid, dim3(256), 0, s, oa, ob, a_blocks, (int)d.K, nkt, blk);
         hipError_t e = hipGetLastError();
         return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "fp16 rounding pass launch");
     };
@@ -624,9 +671,14 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mf
     const int wm_waves = waves == 8 ? 4 : 2;
     const int blk = mf16 ? 16 : 32;                                     // rows per MFMA block
     const int fr_a = (half_m ? 64 : 256 / wm_waves) / blk, fr_b = 128 / blk;   // blocks per wave tile
-    int rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, fr_a, blk);
-    if (rc == NZHIP_OK)
-        rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems, fr_b, blk);
+    int rc;
+    if (a_n == 1 && b_n == 1 && a_c == b_c && (Mp + Np) / CVT_ROWS <= 65535) {
+        rc = convert_pair(fr_a, fr_b, blk);
+    } else {
+        rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, fr_a, blk);
+        if (rc == NZHIP_OK)
+            rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems, fr_b, blk);
+    }
     if (rc == NZHIP_OK) {
         H16Args a;
         a.A = Ah;
