@@ -1,4 +1,5 @@
-// Bandwidth-bound GEMM kernels for products with very few rows or columns (min(M, N) <= 8):
+// Bandwidth-bound GEMM kernels for products with very few rows or columns (min(M, N) <= 8; which of
+// those shapes come here is decided in gemm_skinny_applicable):
 // GEMV-shaped work such as one sample through Model::Linear or the M = 1 case of
 // TensorCoreGEMMParallel (src/OperationKernels.cu:914-1026), where an MFMA tile would be >= 75 %
 // padding and the reference pads 1 row up to 16 (:921-923). The big operand is streamed from

@@ -82,7 +82,8 @@ SKINNY = [(1, 1, 1), (1, 4096, 64), (1, 777, 513), (3, 300, 1000), (8, 64, 260),
 @pytest.mark.parametrize("M,K,N", SKINNY)
 @pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
 def test_skinny_products_are_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans):
-    # min(M, N) <= 8 takes the bandwidth-bound kernels; bias and ReLU ride along
+    # min(M, N) <= 8: the bandwidth-bound streaming kernels (up to 2 rows / 3 columns, or K < 512) or the MFMA
+    # kernel with a split contraction; bias and ReLU ride along
     rng = np.random.default_rng(M * 31 + K * 7 + N)
     A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
     B = rng.integers(-8, 9, size=(K, N)).astype(np.float32)
@@ -99,7 +100,7 @@ SPLITK = [(130, 9000, 70), (576, 16384, 128), (64, 4096, 64), (33, 20001, 300), 
 @pytest.mark.parametrize("M,K,N", SPLITK)
 @pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
 def test_long_contractions_with_few_tiles_are_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans):
-    # few output tiles and K >= 4096: the contraction is cut into chunks that are added in order;
+    # few output tiles and a long contraction: it is cut into chunks that are added in order;
     # a full [M,N] bias and ReLU are applied once, after the last chunk
     rng = np.random.default_rng(M * 13 + K + N * 5)
     A = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
