@@ -251,6 +251,17 @@ def test_batched_broadcast_matches_oracle(nz, oracle, sa, sb):
     assert np.array_equal(host(nz.tensorcore_gemm(dev(A), dev(B))), oracle.tensorcore_gemm(A, B))
 
 
+@pytest.mark.parametrize("sa,sb", [((255, 257, 3, 5), (255, 257, 5, 2)),       # 65 535 members, skinny kernels
+                                   ((255, 257, 9, 16), (1, 257, 16, 9)),       # 65 535 members, MFMA kernel, A-side n broadcast
+                                   ((300, 300, 2, 3), (300, 1, 3, 2))])        # 90 000 members: split into several launches
+def test_largest_batches(nz, sa, sb):
+    rng = np.random.default_rng(sa[0] + sa[2])
+    A = rng.integers(-6, 7, size=sa).astype(np.float32)
+    B = rng.integers(-6, 7, size=sb).astype(np.float32)
+    expect = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(np.float32)   # broadcasts n and c like the reference
+    assert np.array_equal(host(nz.tensorcore_gemm(dev(A), dev(B))), expect)
+
+
 def test_bias_forms_and_relu_special_values(nz, oracle):
     M, K, N = 40, 24, 52
     rng = np.random.default_rng(1)
