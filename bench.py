@@ -27,7 +27,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
-                    choices=["gemm8192", "gemm_batched", "linear", "linear_bwd", "conv_dw", "gemv", "ragged", "conv_a", "conv_b",
+                    choices=["gemm8192", "gemm_batched", "linear", "linear_bwd", "conv_dw", "conv_dx", "gemv", "ragged", "conv_a", "conv_b",
                              "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary (conv / linear) measurements")
@@ -135,6 +135,35 @@ def make_workload(name, orc, capi):
         # operands once, gradients read and written ("+=")
         return Workload(name, 2 * 2.0 * Nb * IN * OUT, 4.0 * (Nb * OUT + Nb * IN + OUT * IN + 2 * OUT * IN + 2 * Nb * IN),
                         run, verify, "mfma", "Linear backward: dW[4096,1024] += dY^T X, dx[4096,1024] += dY W (n=4096)"), None
+    if name == "conv_dx":
+        # data gradient of the CA convolution as one call: dx[16,64,128,128] += conv^T(dy[16,128,128,128], w)
+        N, C, H, W, O = 16, 64, 128, 128, 128
+        dy = orc.fill((N, O, H, W), 4104, "normal", 0.0, 1.0)
+        w = orc.fill((O, C, 3, 3), 1004, "normal", 0.0, float(np.sqrt(2.0 / (C * 9))))
+        w_ref = orc.weights_oihw_to_ref(w)
+        dyd, wd = dev(dy), dev(w_ref)
+        dxd = torch.zeros((N, C, H, W), device="cuda")
+
+        def run():
+            capi.conv2d_backward_data(dxd, dyd, wd, 3, 3, 1, 1, accumulate=True)
+
+        def verify():
+            dxd.zero_()
+            run()
+            # fp64 truth for the first image: mirrored convolution of the fp16-rounded operands
+            dyr = orc.round_f16(dy[:1]).astype(np.float64)
+            wt = orc.round_f16(w_ref).astype(np.float64)[0, 0].reshape(C, 3, 3, O)
+            truth = np.zeros((1, C, H, W))
+            for r in range(3):
+                for sx in range(3):
+                    g = np.einsum("nohw,co->nchw", dyr, wt[:, r, sx, :])
+                    h0, w0 = r - 1, sx - 1
+                    hs, ws = slice(max(0, -h0), min(H, H - h0)), slice(max(0, -w0), min(W, W - w0))
+                    truth[:, :, hs.start + h0:hs.stop + h0, ws.start + w0:ws.stop + w0] += g[:, :, hs, ws]
+            return tolerance(orc, dxd[:1].cpu().numpy(), truth, name)
+
+        return Workload(name, 2.0 * N * H * W * C * 9 * O, 4.0 * (N * O * H * W + O * C * 9 + 2 * N * C * H * W), run, verify,
+                        "hbm", "Conv2d data gradient: dx[16,64,128,128] += dy[16,128,128,128] (*) mirrored w[128,64,3,3]"), None
     if name == "conv_dw":
         # weight gradient of the CA convolution from its column matrix: dW[576,128] += sum_n col_n^T dZ_n,
         # the batch reduction folded into one contraction of length 16 * 16384
@@ -322,7 +351,7 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched", "linear_bwd", "conv_dw"):
+        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)
             ms2, _ = time_steps(w2, max(10, args.steps // 2), max(3, args.warmup // 2))

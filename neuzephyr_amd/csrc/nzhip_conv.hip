@@ -1113,6 +1113,33 @@ static int conv2d_via_workspace(float* y, const float* x, const float* w_ref, co
     return rc ? rc : rc2;
 }
 
+// Weights of the data-gradient convolution: the gradient with respect to x of a stride-1 convolution is
+// itself a stride-1 convolution of dy (O channels in, C channels out) with the taps mirrored:
+//   w'[wb][(o, r', s')][c] = w[wb][(c, K_h-1-r', K_w-1-s')][o]
+__global__ __launch_bounds__(256) void conv_weight_flip_kernel(float* __restrict__ dst, const float* __restrict__ src,
+                                                               int C, int O, int K_h, int K_w, long total) {
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;      // index into dst, c fastest
+    if (t >= total) return;
+    const int taps = K_h * K_w;
+    const int c = (int)(t % C);
+    const long q = t / C;                                       // (wb, o, r', s')
+    const int tap = (int)(q % taps), o = (int)((q / taps) % O);
+    const long wb = q / ((long)taps * O);
+    const int r = K_h - 1 - tap / K_w, sx = K_w - 1 - tap % K_w;
+    dst[t] = src[((wb * C + c) * taps + (long)r * K_w + sx) * O + o];
+}
+
+__global__ __launch_bounds__(256) void accumulate_kernel(float* __restrict__ dst, const float* __restrict__ src, long n) {
+    const long t = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (t + 4 <= n && ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15) == 0) {
+        floatx4 a = *reinterpret_cast<const floatx4*>(dst + t), b = *reinterpret_cast<const floatx4*>(src + t);
+        a[0] += b[0]; a[1] += b[1]; a[2] += b[2]; a[3] += b[3];
+        *reinterpret_cast<floatx4*>(dst + t) = a;
+    } else {
+        for (long i = t; i < n && i < t + 4; i++) dst[i] += src[i];
+    }
+}
+
 }  // namespace nzhip
 
 using namespace nzhip;
@@ -1155,4 +1182,49 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
     }
     return conv2d_via_workspace(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
                                 bias_stride_channel, activation, H_out, W_out, s);
+}
+
+/* Gradient of nzhip_conv2d_forward with respect to x for stride 1: one convolution of dy with the
+ * mirrored weights instead of the reference's chain Col2ImgNode::backward -> MatMulNode::backward
+ * (dA += dC * B^T) -> Img2ColNode::backward (src/Nodes.cu:660-665, 169-182, 632-640), which writes and
+ * re-reads a column-matrix gradient of K_h*K_w times the size of x. */
+extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
+                                          size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                                          size_t w_batch, int accumulate, void* stream) {
+    if (!dx || !dy || !w_ref) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_data: null pointer");
+    if (stride == 0 || K_h == 0 || K_w == 0)
+        return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_data: zero stride or kernel extent");
+    if (w_batch != 1 && w_batch != N) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
+    if (H + 2 * pad < K_h || W + 2 * pad < K_w)
+        return set_error(NZHIP_E_SHAPE, "nzhip_conv2d_backward_data: kernel larger than the padded input");
+    if (stride != 1 || K_h != K_w || pad > K_h - 1)
+        return set_error(NZHIP_E_UNSUPPORTED,
+                         "nzhip_conv2d_backward_data: only stride 1, square kernels and pad <= K-1 (use the column-matrix chain)");
+    if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const size_t H_out = H + 2 * pad - K_h + 1, W_out = W + 2 * pad - K_w + 1;
+    const size_t w_elems = w_batch * C * K_h * K_w * O, x_elems = N * C * H * W;
+    float* wflip = nullptr;
+    float* tmp = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&wflip), w_elems * sizeof(float), s)) return rc;
+    int rc = NZHIP_OK;
+    if (accumulate) rc = workspace_alloc(reinterpret_cast<void**>(&tmp), x_elems * sizeof(float), s);
+    if (rc == NZHIP_OK) {
+        hipLaunchKernelGGL(conv_weight_flip_kernel, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, s, wflip, w_ref,
+                           (int)C, (int)O, (int)K_h, (int)K_w, (long)w_elems);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "conv_weight_flip kernel launch");
+    }
+    if (rc == NZHIP_OK)
+        rc = nzhip_conv2d_forward(accumulate ? tmp : dx, dy, wflip, nullptr, N, O, H_out, W_out, C, K_h, K_w, 1,
+                                  K_h - 1 - pad, w_batch, 0, 0, NZHIP_ACT_NONE, stream);
+    if (rc == NZHIP_OK && accumulate) {
+        hipLaunchKernelGGL(accumulate_kernel, dim3((unsigned)((x_elems / 4 + 256) / 256)), dim3(256), 0, s, dx, tmp,
+                           (long)x_elems);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "accumulate kernel launch");
+    }
+    int rc2 = tmp ? workspace_free(tmp, s) : NZHIP_OK;
+    int rc3 = workspace_free(wflip, s);
+    return rc ? rc : (rc2 ? rc2 : rc3);
 }

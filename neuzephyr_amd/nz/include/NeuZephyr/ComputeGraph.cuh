@@ -49,7 +49,8 @@ namespace nz::graph {
         std::vector<io::OutputNode*> outputNodes;
         std::vector<Node*> sortedNodes;
         std::vector<std::function<void()>> plan;         // what forward() runs, in order
-        std::vector<Node*> fusedMembers;                 // nodes inside fused chains, in sorted order
+        std::vector<std::function<void()>> backPlan;     // what backward() runs, in order
+        std::vector<Node*> fusedMembers;                 // nodes of fused chains whose outputs backward() needs, in sorted order
         bool intermediatesStale = false;                 // a fused forward() skipped their outputs
         bool fusion = true;
         bool planned = false;

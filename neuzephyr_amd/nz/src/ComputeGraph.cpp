@@ -89,13 +89,15 @@ namespace nz::graph {
         struct Group {
             std::vector<Node*> members;          // nodes whose forward() the fused call replaces
             std::function<void()> call;
+            std::function<void()> back;          // fused backward of the whole chain (empty: node by node)
         };
         std::vector<Group> groups;
         std::unordered_map<Node*, size_t> groupOf;
         const auto covered = [&](Node* n) { return groupOf.count(n) != 0; };
-        const auto addGroup = [&](std::vector<Node*> members, std::function<void()> call) {
+        const auto addGroup = [&](std::vector<Node*> members, std::function<void()> call,
+                                  std::function<void()> back = {}) {
             for (Node* n : members) groupOf[n] = groups.size();
-            groups.push_back({std::move(members), std::move(call)});
+            groups.push_back({std::move(members), std::move(call), std::move(back)});
         };
 
         if (fusion) {
@@ -133,12 +135,43 @@ namespace nz::graph {
                     std::vector<Node*> members = {i2c, mm, c2i};
                     if (add) members.push_back(add);
                     if (relu) members.push_back(last);
+                    // Backward of the whole chain without the column-matrix gradient: dZ = dY masked by the
+                    // activation; bias and weight gradients from dZ in pixel-major form (Col2Img.backward,
+                    // Add.backward, MatMul.backward for B with the column matrix recomputed); the data gradient
+                    // as one convolution of dZ. Same accumulate / overwrite behaviour as the node chain.
+                    std::function<void()> back;
+                    if (i2c->stride == 1 && i2c->kernelHeight == i2c->kernelWidth && i2c->padding <= i2c->kernelHeight - 1) {
+                        Node* pre = add ? static_cast<Node*>(add) : static_cast<Node*>(mm);   // holds [N,1,HW,O] gradients
+                        back = [=] {
+                            float* dZ = last->output->grad();
+                            if (relu) {
+                                iReLUBackward(c2i->output->grad(), last->output->data(), dZ, last->output->size());
+                                dZ = c2i->output->grad();
+                            }
+                            const bool needW = rhs->output->requiresGrad();
+                            const bool needB = biasNode && biasNode->output->requiresGrad();
+                            if (needW || needB)
+                                iCol2imgBackward(pre->output->grad(), dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
+                            if (needB)
+                                iAddBackward(biasNode->output->grad(), pre->output->grad(), biasNode->output->shape(),
+                                             pre->output->shape());
+                            if (needW) {
+                                i2c->forward();                      // the column matrix the fused forward never wrote
+                                iMatMulBackward(nullptr, rhs->output->grad(), i2c->output->data(), rhs->output->data(),
+                                                pre->output->grad(), i2c->output->shape(), rhs->output->shape(),
+                                                mm->output->shape());
+                            }
+                            if (x->output->requiresGrad())
+                                iConv2dBackwardData(x->output->grad(), dZ, rhs->output->data(), xs[0], xs[1], xs[2], xs[3], O,
+                                                    i2c->kernelHeight, i2c->kernelWidth, i2c->stride, i2c->padding, ws[0]);
+                        };
+                    }
                     addGroup(std::move(members), [=] {
                         iConv2dForward(last->output->data(), x->output->data(), rhs->output->data(),
                                        biasNode ? biasNode->output->data() : nullptr, xs[0], xs[1], xs[2], xs[3], O,
                                        i2c->kernelHeight, i2c->kernelWidth, i2c->stride, i2c->padding, ws[0],
                                        static_cast<long long>(O), 1, relu);
-                    });
+                    }, std::move(back));
                     continue;
                 }
 
@@ -183,10 +216,23 @@ namespace nz::graph {
                 plan.push_back(groups[it->second].call);
             }
         }
+        // backward: reverse topological order; a chain with a fused backward runs it at the position of its
+        // last member (by then every consumer has added its share to that member's gradient)
+        backPlan.clear();
+        for (size_t i = sortedNodes.size(); i-- > 0;) {
+            Node* node = sortedNodes[i];
+            const auto it = groupOf.find(node);
+            if (it == groupOf.end() || !groups[it->second].back) {
+                backPlan.emplace_back([node] { node->backward(); });
+            } else if (emitAt[it->second] == i) {
+                backPlan.push_back(groups[it->second].back);
+            }
+        }
         fusedGroups = groups.size();
         fusedMembers.clear();
         for (Node* node : sortedNodes)
-            if (groupOf.count(node)) fusedMembers.push_back(node);
+            if (const auto it = groupOf.find(node); it != groupOf.end() && !groups[it->second].back)
+                fusedMembers.push_back(node);
         planned = true;
     }
 
@@ -201,12 +247,13 @@ namespace nz::graph {
         if (!isSorted()) throw std::runtime_error("Graph is not sorted");
         if (outputNodes.empty()) throw std::runtime_error("No output node");
         if (outputNodes.size() > 1) throw std::runtime_error("Multiple output nodes");
+        if (!planned) buildPlan();
         if (intermediatesStale) {
             // node-level gradients read the outputs a fused chain never wrote: produce them now
             for (Node* node : fusedMembers) node->forward();
             intermediatesStale = false;
         }
-        for (auto it = sortedNodes.rbegin(); it != sortedNodes.rend(); ++it) (*it)->backward();
+        for (auto& step : backPlan) step();
     }
 
     void ComputeGraph::update(opt::Optimizer* optimizer) const {

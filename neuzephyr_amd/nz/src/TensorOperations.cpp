@@ -127,6 +127,15 @@ namespace nz::data {
                                       biasChannelStride, relu ? NZHIP_ACT_RELU : NZHIP_ACT_NONE, nzhip_default_stream()));
     }
 
+    bool iConv2dBackwardData(float* dx, float* dy, float* w, const size_t N, const size_t C, const size_t H,
+                             const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
+                             const size_t pad, const size_t weightBatch) {
+        if (stride != 1 || K_h != K_w || pad > K_h - 1) return false;
+        NZ_CHECK(nzhip_conv2d_backward_data(dx, dy, w, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch, 1,
+                                            nzhip_default_stream()));
+        return true;
+    }
+
     void iLinearForward(float* y, float* x, float* wOutIn, float* bias, const size_t batch, const size_t in,
                         const size_t out, const bool relu) {
         nzhip_gemm_desc d = {};

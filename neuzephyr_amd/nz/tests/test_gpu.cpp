@@ -466,6 +466,56 @@ TEST(Model, Conv2dBackwardMatchesFiniteStructure) {
     for (float v : m.parameters()[1]->output->hostGrad()) EXPECT_TRUE(v == static_cast<float>(n));
 }
 
+struct ConvGradModel : nz::Model {
+    InputNode input;
+    ConvGradModel(size_t n, size_t c, size_t h, size_t w, size_t o, size_t k, size_t stride, size_t pad, bool relu)
+        : input({n, c, h, w}, true) {                               // the input wants its gradient too
+        Node* x = Conv2d(&input, o, k, k, stride, pad);
+        if (relu) x = ReLU(x);
+        defaultOutput(x);
+    }
+};
+
+static void convBackwardFusedEqualsChain(size_t n, size_t c, size_t h, size_t w, size_t o, size_t k, size_t stride,
+                                         size_t pad, bool relu) {
+    // integer-valued data: every gradient is exact, so the fused chain backward (one convolution for dx,
+    // no column-matrix gradient) must equal the node-by-node backward bit for bit
+    ConvGradModel m(n, c, h, w, o, k, stride, pad, relu);
+    auto ints = [](size_t count, unsigned seed, int lo, int hi) {
+        auto v = randomVec(count, seed, static_cast<float>(lo), static_cast<float>(hi) + 0.999f);
+        for (auto& e : v) e = std::floor(e);
+        return v;
+    };
+    const size_t Ho = (h + 2 * pad - k) / stride + 1, Wo = (w + 2 * pad - k) / stride + 1, ckk = c * k * k;
+    auto x = ints(n * c * h * w, 61, -3, 3), W = ints(n * ckk * o, 62, -2, 2), b = ints(Ho * Wo * o, 63, -4, 4);
+    m.input.dataInject(x.begin(), x.end());
+    m.parameters()[0]->dataInject(W.begin(), W.end());
+    m.parameters()[1]->dataInject(b.begin(), b.end());
+    m.graph().zeroGrad();
+    m.forward();
+    EXPECT_EQ(m.graph().fusedGroupCount(), 1u);
+    m.backward();
+    const auto dx = m.input.output->hostGrad(), dW = m.parameters()[0]->output->hostGrad(),
+               db = m.parameters()[1]->output->hostGrad();
+    m.graph().setFusion(false);
+    m.graph().zeroGrad();
+    m.forward();
+    m.backward();
+    EXPECT_TRUE(m.input.output->hostGrad() == dx);
+    EXPECT_TRUE(m.parameters()[0]->output->hostGrad() == dW);
+    EXPECT_TRUE(m.parameters()[1]->output->hostGrad() == db);
+    bool anyX = false;
+    for (float v : dx) anyX = anyX || v != 0.f;
+    EXPECT_TRUE(anyX);
+}
+
+TEST(Model, Conv2dFusedBackwardEqualsNodeChain) {
+    convBackwardFusedEqualsChain(2, 3, 7, 9, 5, 3, 1, 1, true);
+    convBackwardFusedEqualsChain(1, 16, 12, 40, 24, 3, 1, 1, true);   // implicit-GEMM kernels
+    convBackwardFusedEqualsChain(2, 4, 6, 6, 3, 1, 1, 0, false);      // 1x1, no activation
+    convBackwardFusedEqualsChain(2, 3, 9, 8, 4, 3, 2, 1, true);       // stride 2: the chain falls back to the nodes
+}
+
 // ---- fp32 matmul and optimizers (test/Test.cpp:119-184, 2230-2265, 2398-2452, 2816-2878) ------------
 TEST(TensorBasic, TensorMultiplicationTest) {
     Tensor tensor1({2, 1, 2, 3});

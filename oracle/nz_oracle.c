@@ -396,6 +396,45 @@ void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_ou
     }
 }
 
+/* Data gradient of the Model::Conv2d graph in one statement (stride 1). The reference computes it
+ * as the chain Col2ImgNode::backward (src/Nodes.cu:660-665) -> MatMulNode::backward, dA += dC * B^T
+ * with fp16-rounded operands and fp32 accumulation (:169-182) -> Img2ColNode::backward (:632-640,
+ * img2colBackwardKernel, src/OperationKernels.cu:1337-1362). Composed:
+ *   dx[b][c][h][w] += sum over r, s, o of f16(dy[b][o][h+pad-r][w+pad-s]) * f16(W[wb][(c,r,s)][o])
+ * for the (r, s) whose output position exists. Here o runs innermost in ascending order inside each
+ * (r, s), then the taps in ascending (r, s): the grouping of the chain (a dot product over o per
+ * column-matrix entry, then one addition per tap). */
+void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
+                              size_t W, size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch) {
+    const size_t H_out = H + 2 * pad - K_h + 1, W_out = W + 2 * pad - K_w + 1, CKK = C * K_h * K_w;
+    float* dyr = (float*)malloc(sizeof(float) * N * O * H_out * W_out);
+    float* wr = (float*)malloc(sizeof(float) * w_batch * CKK * O);
+    nzo_round_f16_array(dyr, dy, N * O * H_out * W_out);
+    nzo_round_f16_array(wr, w_ref, w_batch * CKK * O);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (size_t b = 0; b < N; b++)
+        for (size_t c = 0; c < C; c++) {
+            const float* wb = wr + (w_batch > 1 ? b : 0) * CKK * O;
+            for (size_t h = 0; h < H; h++)
+                for (size_t w = 0; w < W; w++) {
+                    float g = dx[((b * C + c) * H + h) * W + w];
+                    for (size_t r = 0; r < K_h; r++)
+                        for (size_t s = 0; s < K_w; s++) {
+                            const long long ho = (long long)(h + pad) - (long long)r, wo = (long long)(w + pad) - (long long)s;
+                            if (ho < 0 || ho >= (long long)H_out || wo < 0 || wo >= (long long)W_out) continue;
+                            const float* wrow = wb + ((c * K_h + r) * K_w + s) * O;
+                            float dot = 0.0f;
+                            for (size_t o = 0; o < O; o++)
+                                dot += dyr[((b * O + o) * H_out + (size_t)ho) * W_out + (size_t)wo] * wrow[o];
+                            g += dot;
+                        }
+                    dx[((b * C + c) * H + h) * W + w] = g;
+                }
+        }
+    free(dyr);
+    free(wr);
+}
+
 /* ------------------------------------------------------------------------- */
 /* Softmax and its Jacobian: test/Test.cpp:1823-1832 and :1782-1795.          */
 /* ------------------------------------------------------------------------- */

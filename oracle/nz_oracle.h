@@ -135,6 +135,10 @@ void nzo_im2col_backward(float* dx, const float* dcol, size_t H_out, size_t W_ou
                          size_t K_w, size_t stride, size_t pad, size_t H_in, size_t W_in, size_t batch);
 /* col2imgBackwardKernel, src/OperationKernels.cu:1384-1396: dcol[b][(h*W+w)*C+c] = dy[b][c][h][w]. */
 void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_out, size_t C_out, size_t batches);
+/* dx += data gradient of the stride-1 Conv2d graph (the chain Nodes.cu:660-665 -> :169-182 -> :632-640 in one
+ * statement); dy [N,O,H_out,W_out], w_ref [w_batch,1,C*K_h*K_w,O], dx [N,C,H,W]. */
+void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
+                              size_t W, size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch);
 
 /* ---- softmax -------------------------------------------------------------
  * Host statement of the reference's own tests (test/Test.cpp:1823-1832, 1782-1795): exp / sum(exp)

@@ -81,6 +81,7 @@ _relu_bwd = _sig("nzo_relu_backward", None, _f32p, _f32p, _f32p, _sz)
 _add_bwd = _sig("nzo_add_backward", None, _f32p, _f32p, _Shape, _Shape)
 _im2col_bwd = _sig("nzo_im2col_backward", None, _f32p, _f32p, *([_sz] * 10))
 _col2im_bwd = _sig("nzo_col2im_backward", None, _f32p, _f32p, _sz, _sz, _sz, _sz)
+_conv_bwd_data = _sig("nzo_conv2d_backward_data", None, _f32p, _f32p, _f32p, *([_sz] * 9))
 _softmax = _sig("nzo_softmax", None, _f32p, _f32p, _sz, _sz)
 _softmax_jac = _sig("nzo_softmax_jacobian", None, _f32p, _f32p, _sz, _sz)
 _sgd = _sig("nzo_sgd_step", None, _f32p, _f32p, C.c_float, _sz)
@@ -271,6 +272,17 @@ def col2im_backward(dy: np.ndarray) -> np.ndarray:
     out = np.empty((N, 1, Ho * Wo, O), np.float32)
     _col2im_bwd(out.reshape(-1), dy.reshape(-1), Ho, Wo, O, N)
     return out
+
+
+def conv2d_backward_data(dx: np.ndarray, dy: np.ndarray, w_ref: np.ndarray, K_h: int, K_w: int, pad: int) -> np.ndarray:
+    """dx += gradient of the stride-1 Conv2d graph with respect to its input (in place, returns dx)."""
+    dy, w_ref = _c(dy), _c(w_ref)
+    assert dx.dtype == np.float32 and dx.flags.c_contiguous
+    N, Cc, H, W = dx.shape
+    O = dy.shape[1]
+    assert dy.shape == (N, O, H + 2 * pad - K_h + 1, W + 2 * pad - K_w + 1) and w_ref.shape[2:] == (Cc * K_h * K_w, O)
+    _conv_bwd_data(dx.reshape(-1), dy.reshape(-1), w_ref.reshape(-1), N, Cc, H, W, O, K_h, K_w, pad, w_ref.shape[0])
+    return dx
 
 
 def softmax(x: np.ndarray) -> np.ndarray:

@@ -182,3 +182,59 @@ def test_col2im_backward_bit_exact(nz, oracle, n, c, h, w):
     got = host(nz.col2im_backward(dev(dy)))
     assert np.array_equal(got, oracle.col2im_backward(dy))
     assert np.array_equal(host(nz.col2im(dev(got), h, w)), dy)       # round trip with the forward transpose
+
+
+CONV_BWD_DATA = [  # N, C, H, W, O, K, pad, w_batch
+    (2, 3, 5, 6, 4, 3, 1, 1), (1, 2, 4, 4, 3, 3, 0, 1), (2, 2, 6, 5, 2, 3, 2, 2), (1, 3, 5, 5, 2, 1, 0, 1),
+    (2, 16, 20, 36, 24, 3, 1, 1), (1, 64, 32, 64, 128, 3, 1, 1), (3, 8, 17, 33, 70, 3, 1, 3), (2, 40, 9, 70, 12, 1, 0, 1),
+    (1, 3, 40, 40, 1, 3, 1, 1), (2, 1, 12, 16, 2, 3, 1, 1)]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,K,pad,wb", CONV_BWD_DATA)
+@pytest.mark.parametrize("accumulate", [True, False])
+def test_conv2d_backward_data_matches_the_chain_on_integers(nz, oracle, N, C, H, W, O, K, pad, wb, accumulate):
+    # one fused call == Col2Img.backward -> MatMul.backward (dA) -> Img2Col.backward, exact on integers
+    rng = np.random.default_rng(N * 131 + C * 17 + H * 7 + W + O * 3 + K)
+    Ho, Wo = H + 2 * pad - K + 1, W + 2 * pad - K + 1
+    dy = rng.integers(-4, 5, size=(N, O, Ho, Wo)).astype(np.float32)
+    w = rng.integers(-4, 5, size=(wb, 1, C * K * K, O)).astype(np.float32)
+    dx0 = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    expect = oracle.conv2d_backward_data(dx0.copy() if accumulate else np.zeros_like(dx0), dy, w, K, K, pad)
+    got = host(nz.conv2d_backward_data(dev(dx0), dev(dy), dev(w), K, K, 1, pad, accumulate=accumulate))
+    assert np.array_equal(got, expect)
+
+
+def test_conv2d_backward_data_float_tolerance_and_adjoint(nz, oracle):
+    N, C, H, W, O, K, pad = 2, 32, 24, 40, 48, 3, 1
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, O, H, W)).astype(np.float32)
+    w = (rng.standard_normal((1, 1, C * K * K, O)) * 0.1).astype(np.float32)
+    got = host(nz.conv2d_backward_data(dev(np.zeros_like(x)), dev(dy), dev(w), K, K, 1, pad, accumulate=True))
+    # truth: fp64 accumulation over the fp16-rounded operands, tap by tap
+    dyr, wr = oracle.round_f16(dy).astype(np.float64), oracle.round_f16(w).astype(np.float64)
+    wt = wr[0, 0].reshape(C, K, K, O)
+    truth = np.zeros((N, C, H, W))
+    for r in range(K):
+        for sx in range(K):
+            g = np.einsum("nohw,co->nchw", dyr, wt[:, r, sx, :])      # contribution of dy[ho, wo] to x[ho - pad + r, wo - pad + sx]
+            h0, w0 = r - pad, sx - pad
+            hs, ws = slice(max(0, -h0), min(H, H - h0)), slice(max(0, -w0), min(W, W - w0))
+            hd, wd = slice(hs.start + h0, hs.stop + h0), slice(ws.start + w0, ws.stop + w0)
+            truth[:, :, hd, wd] += g[:, :, hs, ws]
+    rms = float(np.sqrt(np.mean(truth ** 2)))
+    mr, fr = oracle.errors(got, truth, rms)
+    assert mr <= 1e-3 and fr <= 1e-4, (mr, fr)
+    # adjoint identity with the forward kernel: <conv(x), dy> == <x, conv^T(dy)> for rounded x
+    xr = oracle.round_f16(x)
+    y = host(nz.conv2d_forward(dev(xr), dev(w), None, K, K, 1, pad))
+    lhs = float(np.sum(y.astype(np.float64) * dyr))
+    rhs = float(np.sum(xr.astype(np.float64) * got.astype(np.float64)))
+    assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), abs(rhs), 1.0)
+
+
+def test_conv2d_backward_data_rejects_what_it_does_not_cover(nz):
+    from neuzephyr_amd.capi import NzHipError
+    dx, dy, w = dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 4, 4))), dev(np.zeros((1, 1, 18, 3)))
+    with pytest.raises(NzHipError):
+        nz.conv2d_backward_data(dx, dy, w, 3, 3, 2, 1)
