@@ -40,6 +40,77 @@ __global__ __launch_bounds__(256) void im2col_kernel(float* __restrict__ out, co
     out[(long)b * per + idx] = v;
 }
 
+// The same with four consecutive column indices per thread and one 16-byte store (C*K_h*K_w a
+// multiple of 4, 16-byte aligned output): a quarter of the store instructions and index divisions.
+__global__ __launch_bounds__(256) void im2col_vec4_kernel(float* __restrict__ out, const float* __restrict__ in,
+                                                          int H_out, int W_out, int C, int K_h, int K_w, int stride,
+                                                          int pad, int H_in, int W_in) {
+    const int CKK = C * K_h * K_w, KK = K_h * K_w;
+    const long per = (long)H_out * W_out * CKK;
+    const long idx = ((long)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (idx >= per) return;
+    const int b = blockIdx.y;
+    const int pix = (int)(idx / CKK), q = (int)(idx % CKK);    // q % 4 == 0 and CKK % 4 == 0: all four in this row
+    int c = q / KK, rs = q % KK;
+    const int h0 = (pix / W_out) * stride - pad, w0 = (pix % W_out) * stride - pad;
+    const float* img = in + (long)b * C * H_in * W_in;
+    floatx4 v;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int h = h0 + rs / K_w, w = w0 + rs % K_w;
+        v[e] = (h >= 0 && h < H_in && w >= 0 && w < W_in) ? img[((long)c * H_in + h) * W_in + w] : 0.f;
+        if (++rs == KK) {
+            rs = 0;
+            c++;
+        }
+    }
+    *reinterpret_cast<floatx4*>(out + (long)b * per + idx) = v;
+}
+
+// Stride 1: a workgroup takes 64 adjacent output pixels of one row and 32 channels, reads the K_h
+// input rows they touch once (coalesced along w) into LDS and writes, per pixel, its contiguous run of
+// 32*K_h*K_w column entries with 16-byte stores (for 3x3 that is 1152 bytes: whole 128-byte lines). The scattered 4-byte global reads of the kernels
+// above (a wave touches 64 channel planes per instruction) are what bounds them.
+constexpr int I2C_PX = 64, I2C_CH = 32, I2C_MAXK = 5, I2C_ROW = I2C_PX + I2C_MAXK;   // floats per staged row
+// KH, KW > 0: kernel extents known at compile time (the index divisions become multiplications).
+template <int KH, int KW>
+__global__ __launch_bounds__(256) void im2col_rows_kernel(float* __restrict__ out, const float* __restrict__ in,
+                                                          int H_out, int W_out, int C, int K_h_rt, int K_w_rt, int pad,
+                                                          int H_in, int W_in, int segs) {
+    __shared__ float rows[I2C_CH * I2C_MAXK * I2C_ROW];
+    const int K_h = KH > 0 ? KH : K_h_rt, K_w = KW > 0 ? KW : K_w_rt;
+    const int KK = K_h * K_w, CKK = C * KK;
+    const int seg = blockIdx.x % segs, ho = blockIdx.x / segs;
+    const int c0 = blockIdx.y * I2C_CH, b = blockIdx.z;
+    const int nch = (C - c0) < I2C_CH ? (C - c0) : I2C_CH;
+    const int wo0 = seg * I2C_PX;
+    const int span = I2C_PX + K_w - 1;                           // input columns wo0 - pad .. wo0 - pad + span - 1
+    const float* img = in + ((long)b * C + c0) * H_in * W_in;
+    for (int e = threadIdx.x; e < nch * K_h * span; e += 256) {
+        const int col = e % span, r = (e / span) % K_h, c = e / (span * K_h);
+        const int h = ho - pad + r, w = wo0 - pad + col;
+        rows[(c * K_h + r) * I2C_ROW + col] = (h >= 0 && h < H_in && w >= 0 && w < W_in) ? img[((long)c * H_in + h) * W_in + w] : 0.f;
+    }
+    __syncthreads();
+    const int run4 = nch * KK / 4;                               // 16-byte pieces per pixel (nch*KK is a multiple of 4)
+    const int npx = (W_out - wo0) < I2C_PX ? (W_out - wo0) : I2C_PX;
+    float* dst = out + ((long)b * H_out * W_out + (long)ho * W_out + wo0) * CKK + (long)c0 * KK;
+    for (int e = threadIdx.x; e < npx * run4; e += 256) {
+        const int px = e / run4, q4 = e % run4;
+        int c = (q4 * 4) / KK, rs = (q4 * 4) % KK;
+        floatx4 v;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[j] = rows[(c * K_h + rs / K_w) * I2C_ROW + px + rs % K_w];
+            if (++rs == KK) {
+                rs = 0;
+                c++;
+            }
+        }
+        *reinterpret_cast<floatx4*>(dst + (long)px * CKK + q4 * 4) = v;
+    }
+}
+
 // ---- col2im (col2imgKernel, :1364-1376): per-image transpose [HW, O] -> [O, HW] through LDS --
 __global__ __launch_bounds__(256) void col2im_kernel(float* __restrict__ out, const float* __restrict__ in, int HW,
                                                      int O) {
@@ -406,6 +477,26 @@ int nzhip_im2col(float* out, const float* in, size_t H_out, size_t W_out, size_t
     if (per == 0 || batch == 0) return NZHIP_OK;
     if (per > 0x7fffffffull * 256 || batch > 65535 || H_in > 0x3fffffff || W_in > 0x3fffffff)
         return set_error(NZHIP_E_UNSUPPORTED, "nzhip_im2col: extent too large");
+    if (stride == 1 && K_h <= (size_t)I2C_MAXK && K_w <= (size_t)I2C_MAXK && (C * K_h * K_w) % 4 == 0 &&
+        (I2C_CH * K_h * K_w) % 4 == 0 && aligned16(out)) {
+        const size_t segs = (W_out + I2C_PX - 1) / I2C_PX, chunks = (C + I2C_CH - 1) / I2C_CH;
+        if (segs * H_out <= 0x7fffffffull && chunks <= 65535) {
+            dim3 grid((unsigned)(segs * H_out), (unsigned)chunks, (unsigned)batch);
+            auto kfn = (K_h == 3 && K_w == 3)   ? im2col_rows_kernel<3, 3>
+                       : (K_h == 1 && K_w == 1) ? im2col_rows_kernel<1, 1>
+                       : (K_h == 5 && K_w == 5) ? im2col_rows_kernel<5, 5>
+                                                : im2col_rows_kernel<0, 0>;
+            hipLaunchKernelGGL(kfn, grid, dim3(256), 0, as_stream(stream), out, in, (int)H_out, (int)W_out, (int)C, (int)K_h,
+                               (int)K_w, (int)pad, (int)H_in, (int)W_in, (int)segs);
+            return check_launch("im2col_rows_kernel");
+        }
+    }
+    if ((C * K_h * K_w) % 4 == 0 && aligned16(out)) {
+        dim3 grid((unsigned)((per / 4 + 255) / 256), (unsigned)batch);
+        hipLaunchKernelGGL(im2col_vec4_kernel, grid, dim3(256), 0, as_stream(stream), out, in, (int)H_out, (int)W_out,
+                           (int)C, (int)K_h, (int)K_w, (int)stride, (int)pad, (int)H_in, (int)W_in);
+        return check_launch("im2col_vec4_kernel");
+    }
     dim3 grid((unsigned)((per + 255) / 256), (unsigned)batch);
     hipLaunchKernelGGL(im2col_kernel, grid, dim3(256), 0, as_stream(stream), out, in, (int)H_out, (int)W_out, (int)C,
                        (int)K_h, (int)K_w, (int)stride, (int)pad, (int)H_in, (int)W_in);
