@@ -27,7 +27,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
-                    choices=["gemm8192", "gemm_batched", "linear", "linear_bwd", "conv_dw", "conv_dx", "gemv", "ragged", "conv_a", "conv_b",
+                    choices=["gemm8192", "gemm_batched", "linear", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "gemv", "ragged", "conv_a", "conv_b",
                              "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary (conv / linear) measurements")
@@ -164,6 +164,31 @@ def make_workload(name, orc, capi):
 
         return Workload(name, 2.0 * N * H * W * C * 9 * O, 4.0 * (N * O * H * W + O * C * 9 + 2 * N * C * H * W), run, verify,
                         "hbm", "Conv2d data gradient: dx[16,64,128,128] += dy[16,128,128,128] (*) mirrored w[128,64,3,3]"), None
+    if name == "conv_dwx":
+        # weight gradient of the CA convolution straight from x and dy (no column matrix)
+        N, C, H, W, O = 16, 64, 128, 128, 128
+        x = orc.fill((N, C, H, W), 4, "normal", 0.0, 1.0)
+        dy = orc.fill((N, O, H, W), 4104, "normal", 0.0, 1.0)
+        xd, dyd = dev(x), dev(dy)
+        dwd = torch.zeros((1, 1, C * 9, O), device="cuda")
+
+        def run():
+            capi.conv2d_backward_weights(dwd, xd, dyd, 3, 3, 1, 1)
+
+        def verify():
+            dwd.zero_()
+            run()
+            # fp64 truth for the first 4 input channels (all taps, all output channels)
+            xr = np.pad(orc.round_f16(x[:, :4]).astype(np.float64), ((0, 0), (0, 0), (1, 1), (1, 1)))
+            dyr = orc.round_f16(dy).astype(np.float64)
+            truth = np.zeros((4, 3, 3, O))
+            for r in range(3):
+                for sx in range(3):
+                    truth[:, r, sx, :] = np.einsum("nchw,nohw->co", xr[:, :, r:r + H, sx:sx + W], dyr)
+            return tolerance(orc, dwd.reshape(C, 9, O)[:4].cpu().numpy().reshape(-1), truth.reshape(-1), name)
+
+        return Workload(name, 2.0 * N * H * W * C * 9 * O, 4.0 * (N * C * H * W + N * O * H * W + 2 * C * 9 * O), run, verify,
+                        "hbm", "Conv2d weight gradient: dW[576,128] += x[16,64,128,128] (*) dy[16,128,128,128], no column matrix"), None
     if name == "conv_dw":
         # weight gradient of the CA convolution from its column matrix: dW[576,128] += sum_n col_n^T dZ_n,
         # the batch reduction folded into one contraction of length 16 * 16384
@@ -351,7 +376,7 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx"):
+        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)
             ms2, _ = time_steps(w2, max(10, args.steps // 2), max(3, args.warmup // 2))

@@ -18,7 +18,7 @@ EXPORTS = [
     "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_tensorcore_gemm",
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
-    "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
+    "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
     "nzhip_softmax", "nzhip_softmax_jacobian",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
@@ -75,6 +75,7 @@ def load() -> C.CDLL:
     lib.nzhip_col2im.argtypes = [vp, vp, sz, sz, sz, sz, vp]
     lib.nzhip_conv2d_forward.argtypes = [vp, vp, vp, vp] + [sz] * 10 + [i64, i64, C.c_int, vp]
     lib.nzhip_conv2d_backward_data.argtypes = [vp, vp, vp] + [sz] * 10 + [C.c_int, vp]
+    lib.nzhip_conv2d_backward_weights.argtypes = [vp, vp, vp] + [sz] * 10 + [vp]
     lib.nzhip_add_broadcast.argtypes = [vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_relu.argtypes = [vp, vp, sz, vp]
     lib.nzhip_gemm_backward.argtypes = [vp, vp, vp, shape, shape, shape, vp]
@@ -292,6 +293,15 @@ def conv2d_backward_data(dx, dy, w_ref, K_h, K_w, stride, pad, *, accumulate=Tru
     check(lib.nzhip_conv2d_backward_data(_dev(dx), _dev(dy), _dev(w_ref), N, Cc, H, W, dy.shape[1], K_h, K_w, stride, pad,
                                          w_ref.shape[0], 1 if accumulate else 0, _stream_handle(stream)))
     return dx
+
+
+def conv2d_backward_weights(dw, x, dy, K_h, K_w, stride, pad, stream=None):
+    """dw += gradient of conv2d_forward with respect to w_ref; dw [w_batch,1,C*K_h*K_w,O] is modified in place."""
+    lib = load()
+    N, Cc, H, W = x.shape
+    check(lib.nzhip_conv2d_backward_weights(_dev(dw), _dev(x), _dev(dy), N, Cc, H, W, dy.shape[1], K_h, K_w, stride, pad,
+                                            dw.shape[0], _stream_handle(stream)))
+    return dw
 
 
 def col2im_backward(dy, stream=None):

@@ -1113,6 +1113,204 @@ static int conv2d_via_workspace(float* y, const float* x, const float* w_ref, co
     return rc ? rc : rc2;
 }
 
+// ---- weight gradient of the 3x3, stride 1, pad 1 convolution without a column matrix ----------------
+//   dW[(c, r, s)][o] += sum over n, h, w of f16(x[n][c][h+r-1][w+s-1]) * f16(dy[n][o][h][w])
+// As a GEMM the contraction runs over pixels, and both operands already are pixel-contiguous in NCHW.
+// A workgroup owns 32 input channels x 128 output channels (9 x 4 blocks of 32x32, one column of blocks
+// per wave) and a band of rows of one image. Per row and 128-pixel segment it keeps in LDS
+//   * the dy row, fp16, [o][pixel];
+//   * the x rows h-1, h, h+1 (a rolling window of three), each as THREE copies shifted by s-1 pixels, so
+//     that every tap reads 16-byte aligned runs of 8 pixels. The copies are made in registers: a lane holds
+//     8 adjacent pixels, takes the pixel to its left / right from the neighbouring lane (DPP row shift; the
+//     first and last lane of a row of 16 load it) and funnel-shifts.
+// Next row's operands are requested into registers before the MFMA phase. Partial sums of the row bands go to
+// a workspace and are added in a fixed order by conv_dw_reduce_kernel.
+constexpr int DW_CC = 32, DW_OT = 128, DW_PX = 128, DW_PITCH = DW_PX * 2 + 16;      // LDS row pitch in bytes
+constexpr int DW_XS_BYTES = 3 * 3 * DW_CC * DW_PITCH, DW_ZS_BYTES = DW_OT * DW_PITCH;
+
+struct ConvDwArgs {
+    const float* x;        // [N, C, H, W]
+    const float* dy;       // [N, O, H, W]
+    float* partial;        // [chunk][o_tile][image][band][rows = nch*9][ncols]
+    int C, H, W, O;
+    int bands, band_rows;  // row bands per image and rows per band
+    int n_images;
+};
+
+__global__ __launch_bounds__(256) void conv_dw_kernel(const ConvDwArgs p) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    char* xs = lds;                       // [slot 3][shift 3][channel 32] rows of DW_PITCH bytes
+    char* zs = lds + DW_XS_BYTES;         // [o 128] rows of DW_PITCH bytes
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const int band = blockIdx.x % p.bands, img = blockIdx.x / p.bands;
+    const int c0 = blockIdx.y * DW_CC, o0 = blockIdx.z * DW_OT;
+    const int nch = (p.C - c0) < DW_CC ? (p.C - c0) : DW_CC;
+    const int ncols = (p.O - o0) < DW_OT ? (p.O - o0) : DW_OT;
+    const int h_begin = band * p.band_rows;
+    const int h_end = (h_begin + p.band_rows) < p.H ? (h_begin + p.band_rows) : p.H;
+    const long plane = (long)p.H * p.W;
+    const float* ximg = p.x + ((long)img * p.C + c0) * plane;
+    const float* zimg = p.dy + ((long)img * p.O + o0) * plane;
+
+    floatx16 acc[9];
+#pragma unroll
+    for (int t = 0; t < 9; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+
+    // staging tasks: x row = 32 channels x 16 groups of 8 pixels (two per thread: channels tid/16 and 16 + tid/16);
+    // dy row = 128 output channels x 16 groups (eight per thread)
+    const int g = tid & 15;
+    float xr[2][8], xl[2], xrt[2];        // a task's 8 pixels, the pixel left of them, the pixel right of them
+    float zr[8][8];
+
+    auto load_x = [&](int h, int w0) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int c = u * 16 + (tid >> 4);
+            const int w = w0 + g * 8;
+            const bool ok = c < nch && h >= 0 && h < p.H && w < p.W;       // W is a multiple of 8: a group is inside or outside
+            const float* src = ximg + (long)c * plane + (long)h * p.W + w;
+#pragma unroll
+            for (int e = 0; e < 8; e++) xr[u][e] = 0.f;
+            xl[u] = 0.f;
+            xrt[u] = 0.f;
+            if (ok) {
+                const floatx4 a = *reinterpret_cast<const floatx4*>(src), b = *reinterpret_cast<const floatx4*>(src + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    xr[u][e] = a[e];
+                    xr[u][4 + e] = b[e];
+                }
+                if (g == 0 && w > 0) xl[u] = src[-1];
+                if (g == 15 && w + 8 < p.W) xrt[u] = src[8];
+            }
+        }
+    };
+    auto load_z = [&](int h, int w0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int o = i * 16 + (tid >> 4);
+            const int w = w0 + g * 8;
+            const bool ok = o < ncols && h < p.H && w < p.W;
+            const float* src = zimg + (long)o * plane + (long)h * p.W + w;
+#pragma unroll
+            for (int e = 0; e < 8; e++) zr[i][e] = 0.f;
+            if (ok) {
+                const floatx4 a = *reinterpret_cast<const floatx4*>(src), b = *reinterpret_cast<const floatx4*>(src + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    zr[i][e] = a[e];
+                    zr[i][4 + e] = b[e];
+                }
+            }
+        }
+    };
+    auto pack2 = [](float lo, float hi) -> unsigned {
+        const _Float16 a = (_Float16)lo, b = (_Float16)hi;
+        return (unsigned)__builtin_bit_cast(unsigned short, a) | ((unsigned)__builtin_bit_cast(unsigned short, b) << 16);
+    };
+    typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+    auto store_x = [&](int slot) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int c = u * 16 + (tid >> 4);
+            const unsigned p0 = pack2(xr[u][0], xr[u][1]), p1 = pack2(xr[u][2], xr[u][3]), p2 = pack2(xr[u][4], xr[u][5]),
+                           p3 = pack2(xr[u][6], xr[u][7]);
+            // neighbour pixels: from the lane one group to the left / right inside the row of 16 lanes;
+            // the outermost lanes keep the pixel they loaded themselves
+            const unsigned left = (unsigned)__builtin_amdgcn_update_dpp((int)pack2(0.f, xl[u]), (int)p3, 0x111, 0xf, 0xf, false);
+            const unsigned right = (unsigned)__builtin_amdgcn_update_dpp((int)pack2(xrt[u], 0.f), (int)p0, 0x101, 0xf, 0xf, false);
+            const uintx4 sm = {__builtin_amdgcn_alignbit(p0, left, 16), __builtin_amdgcn_alignbit(p1, p0, 16),
+                               __builtin_amdgcn_alignbit(p2, p1, 16), __builtin_amdgcn_alignbit(p3, p2, 16)};   // x[w-1]
+            const uintx4 s0 = {p0, p1, p2, p3};                                                                  // x[w]
+            const uintx4 sp = {__builtin_amdgcn_alignbit(p1, p0, 16), __builtin_amdgcn_alignbit(p2, p1, 16),
+                               __builtin_amdgcn_alignbit(p3, p2, 16), __builtin_amdgcn_alignbit(right, p3, 16)}; // x[w+1]
+            char* base = xs + ((slot * 3) * DW_CC + c) * DW_PITCH + g * 16;
+            *reinterpret_cast<uintx4*>(base) = sm;
+            *reinterpret_cast<uintx4*>(base + DW_CC * DW_PITCH) = s0;
+            *reinterpret_cast<uintx4*>(base + 2 * DW_CC * DW_PITCH) = sp;
+        }
+    };
+    auto store_z = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int o = i * 16 + (tid >> 4);
+            const uintx4 v = {pack2(zr[i][0], zr[i][1]), pack2(zr[i][2], zr[i][3]), pack2(zr[i][4], zr[i][5]),
+                              pack2(zr[i][6], zr[i][7])};
+            *reinterpret_cast<uintx4*>(zs + o * DW_PITCH + g * 16) = v;
+        }
+    };
+
+    for (int w0 = 0; w0 < p.W; w0 += DW_PX) {
+        // rows h_begin - 1 and h_begin of this segment go into their slots, then row h_begin + 1 and the
+        // first dy row wait in registers like in every later iteration
+        __syncthreads();                                       // the previous segment's readers are done
+        load_x(h_begin - 1, w0);
+        store_x((h_begin + 2) % 3);                            // slot of row h: (h + 3) % 3, here h = h_begin - 1
+        load_x(h_begin, w0);
+        store_x(h_begin % 3);
+        load_x(h_begin + 1, w0);
+        load_z(h_begin, w0);
+        for (int h = h_begin; h < h_end; h++) {
+            store_x((h + 1) % 3);
+            store_z();
+            __syncthreads();
+            load_x(h + 2, w0);                                 // past the image: zeros; past the band's last use: never read
+            load_z(h + 1 < h_end ? h + 1 : p.H, w0);
+            const char* zrow = zs + (wave * 32 + li) * DW_PITCH + lh * 16;
+#pragma unroll 2
+            for (int j = 0; j < DW_PX / 16; j++) {
+                const half8_t bfrag = *reinterpret_cast<const half8_t*>(zrow + j * 32);
+#pragma unroll
+                for (int r = 0; r < 3; r++) {
+                    const int slot = (h + r + 2) % 3;          // row h + r - 1
+                    const char* arow = xs + ((slot * 3) * DW_CC + li) * DW_PITCH + lh * 16 + j * 32;
+#pragma unroll
+                    for (int sx = 0; sx < 3; sx++) {
+                        const half8_t afrag = *reinterpret_cast<const half8_t*>(arow + sx * DW_CC * DW_PITCH);
+                        acc[r * 3 + sx] = __builtin_amdgcn_mfma_f32_32x32x16_f16(afrag, bfrag, acc[r * 3 + sx], 0, 0, 0);
+                    }
+                }
+            }
+            __syncthreads();                                   // before zs and the oldest x slot are overwritten
+        }
+    }
+
+    // partial sums of this band: rows (c, tap) in the order of dW, columns o
+    const long region = (long)DW_CC * 9 * DW_OT;
+    float* P = p.partial + ((((long)blockIdx.y * gridDim.z + blockIdx.z) * p.n_images + img) * p.bands + band) * region;
+    const int o = wave * 32 + li;
+#pragma unroll
+    for (int t = 0; t < 9; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int c = (r >> 2) * 8 + lh * 4 + (r & 3);
+            if (c < nch && o < ncols) P[(long)(c * 9 + t) * ncols + o] = acc[t][r];
+        }
+}
+
+// dW[b][(c0 + c)*9 + t][o0 + o] += sum over the S partial regions of image group b, in ascending order.
+// b: one index per weight copy (per-sample weights: S = bands of that image; shared weights: S = images x bands).
+__global__ __launch_bounds__(256) void conv_dw_reduce_kernel(float* __restrict__ dW, const float* __restrict__ P, int S,
+                                                             int C, int O, int n_otiles, long group_stride_P,
+                                                             long group_stride_dW) {
+    const int chunk = blockIdx.y / n_otiles, ot = blockIdx.y % n_otiles, b = blockIdx.z;
+    const int c0 = chunk * DW_CC, o0 = ot * DW_OT;
+    const int nch = (C - c0) < DW_CC ? (C - c0) : DW_CC;
+    const int ncols = (O - o0) < DW_OT ? (O - o0) : DW_OT;
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t >= nch * 9 * ncols) return;
+    const long region = (long)DW_CC * 9 * DW_OT;
+    const float* src = P + (long)blockIdx.y * gridDim.z * group_stride_P + (long)b * group_stride_P + t;
+    float sum = 0.f;
+    for (int s = 0; s < S; s++) sum += src[(long)s * region];
+    const int row = t / ncols, col = t % ncols;
+    dW[(long)b * group_stride_dW + ((long)c0 * 9 + row) * O + o0 + col] += sum;
+}
+
 // Weights of the data-gradient convolution: the gradient with respect to x of a stride-1 convolution is
 // itself a stride-1 convolution of dy (O channels in, C channels out) with the taps mirrored:
 //   w'[wb][(o, r', s')][c] = w[wb][(c, K_h-1-r', K_w-1-s')][o]
@@ -1227,4 +1425,60 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     int rc2 = tmp ? workspace_free(tmp, s) : NZHIP_OK;
     int rc3 = workspace_free(wflip, s);
     return rc ? rc : (rc2 ? rc2 : rc3);
+}
+
+/* Gradient of nzhip_conv2d_forward with respect to the weights, without the column matrix the reference's
+ * chain needs (Img2ColNode::forward output as A in MatMulNode::backward, dB += A^T * dC, src/Nodes.cu:169-182):
+ *   dW[wb][(c, r, s)][o] += sum over h, w (and over n when the weights are shared) of
+ *                           f16(x[n][c][h+r-pad][w+s-pad]) * f16(dy[n][o][h][w]) */
+extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H,
+                                             size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                                             size_t w_batch, void* stream) {
+    if (!dw || !x || !dy) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_weights: null pointer");
+    if (w_batch != 1 && w_batch != N) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
+    if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1 || W % 8 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(dy) & 15) != 0 || H == 0 ||
+        H > 0x3fffffff || W > 0x3fffffff || C > 0x3fffffff || O > 0x3fffffff || N > 65535)
+        return set_error(NZHIP_E_UNSUPPORTED,
+                         "nzhip_conv2d_backward_weights: only 3x3, stride 1, pad 1, W a multiple of 8, 16-byte aligned "
+                         "tensors (use the column-matrix chain)");
+    if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const int chunks = (int)((C + DW_CC - 1) / DW_CC), otiles = (int)((O + DW_OT - 1) / DW_OT);
+    if (chunks > 65535 || otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_weights: too many channels");
+    // about two workgroups per CU in total; a band is a whole number of rows of one image
+    const int cus = device_cu_count();
+    long want = (2L * cus + (long)chunks * otiles * (long)N - 1) / ((long)chunks * otiles * (long)N);
+    if (want < 1) want = 1;
+    if (want > (long)H) want = (long)H;
+    const int band_rows = (int)((H + want - 1) / want);
+    const int bands = (int)((H + band_rows - 1) / band_rows);
+    const size_t region = (size_t)DW_CC * 9 * DW_OT;
+    const size_t regions = (size_t)chunks * otiles * N * bands;
+    if (N * (size_t)bands > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_weights: too many row bands");
+    float* partial = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), regions * region * sizeof(float), s)) return rc;
+    ConvDwArgs a;
+    a.x = x; a.dy = dy; a.partial = partial;
+    a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O;
+    a.bands = bands; a.band_rows = band_rows; a.n_images = (int)N;
+    const int lds_bytes = DW_XS_BYTES + DW_ZS_BYTES;
+    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(conv_dw_kernel), lds_bytes, "hipFuncSetAttribute(conv_dw)");
+    if (rc == NZHIP_OK) {
+        dim3 grid((unsigned)(N * bands), (unsigned)chunks, (unsigned)otiles);
+        hipLaunchKernelGGL(conv_dw_kernel, grid, dim3(256), lds_bytes, s, a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "conv_dw kernel launch");
+    }
+    if (rc == NZHIP_OK) {
+        const bool shared = w_batch == 1;
+        const int S = shared ? (int)(N * bands) : bands;
+        const int groups = shared ? 1 : (int)N;
+        dim3 grid((unsigned)((region + 255) / 256), (unsigned)(chunks * otiles), (unsigned)groups);
+        hipLaunchKernelGGL(conv_dw_reduce_kernel, grid, dim3(256), 0, s, dw, partial, S, (int)C, (int)O, otiles,
+                           (long)((size_t)S * region), (long)(C * 9 * O));
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "conv_dw_reduce kernel launch");
+    }
+    int rc2 = workspace_free(partial, s);
+    return rc ? rc : rc2;
 }

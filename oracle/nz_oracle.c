@@ -435,6 +435,38 @@ void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, si
     free(wr);
 }
 
+/* Weight gradient of the Model::Conv2d graph in one statement (stride 1): MatMulNode::backward's
+ * dB += A^T * dC (src/Nodes.cu:169-182) with A the column matrix of Img2ColNode::forward (:605-630,
+ * img2colKernel src/OperationKernels.cu:1308-1328) and dC the pixel-major gradient of
+ * Col2ImgNode::backward (:660-665); fp16-rounded operands, fp32 accumulation over the pixels in
+ * ascending order (and over the images, for shared weights). */
+void nzo_conv2d_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W,
+                                 size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch) {
+    const size_t H_out = H + 2 * pad - K_h + 1, W_out = W + 2 * pad - K_w + 1, CKK = C * K_h * K_w;
+    float* xr = (float*)malloc(sizeof(float) * N * C * H * W);
+    float* dyr = (float*)malloc(sizeof(float) * N * O * H_out * W_out);
+    nzo_round_f16_array(xr, x, N * C * H * W);
+    nzo_round_f16_array(dyr, dy, N * O * H_out * W_out);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (size_t q = 0; q < CKK; q++)
+        for (size_t o = 0; o < O; o++) {
+            const size_t c = q / (K_h * K_w), r = (q % (K_h * K_w)) / K_w, s = q % K_w;
+            for (size_t wb = 0; wb < w_batch; wb++) {
+                float acc = 0.0f;
+                for (size_t b = (w_batch > 1 ? wb : 0); b < (w_batch > 1 ? wb + 1 : N); b++)
+                    for (size_t ho = 0; ho < H_out; ho++)
+                        for (size_t wo = 0; wo < W_out; wo++) {
+                            const long long h = (long long)(ho + r) - (long long)pad, w = (long long)(wo + s) - (long long)pad;
+                            if (h < 0 || h >= (long long)H || w < 0 || w >= (long long)W) continue;
+                            acc += xr[((b * C + c) * H + (size_t)h) * W + (size_t)w] * dyr[((b * O + o) * H_out + ho) * W_out + wo];
+                        }
+                dw[(wb * CKK + q) * O + o] += acc;
+            }
+        }
+    free(xr);
+    free(dyr);
+}
+
 /* ------------------------------------------------------------------------- */
 /* Softmax and its Jacobian: test/Test.cpp:1823-1832 and :1782-1795.          */
 /* ------------------------------------------------------------------------- */

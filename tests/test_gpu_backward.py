@@ -238,3 +238,45 @@ def test_conv2d_backward_data_rejects_what_it_does_not_cover(nz):
     dx, dy, w = dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 4, 4))), dev(np.zeros((1, 1, 18, 3)))
     with pytest.raises(NzHipError):
         nz.conv2d_backward_data(dx, dy, w, 3, 3, 2, 1)
+
+
+CONV_BWD_W = [  # N, C, H, W, O, w_batch   (3x3, stride 1, pad 1, W a multiple of 8)
+    (1, 3, 4, 8, 2, 1), (2, 5, 7, 16, 9, 1), (2, 32, 9, 24, 40, 2), (3, 40, 6, 136, 130, 1), (1, 64, 16, 128, 128, 1),
+    (2, 33, 5, 264, 129, 2), (4, 8, 33, 40, 16, 1), (1, 1, 1, 8, 1, 1)]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,wb", CONV_BWD_W)
+def test_conv2d_backward_weights_is_bit_exact_on_integers(nz, oracle, N, C, H, W, O, wb):
+    # one fused call == Img2Col.forward -> MatMul.backward (dB); every partial sum is an exact integer
+    rng = np.random.default_rng(N * 131 + C * 17 + H * 7 + W + O * 3 + wb)
+    x = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    dy = rng.integers(-3, 4, size=(N, O, H, W)).astype(np.float32)
+    dw0 = rng.integers(-5, 6, size=(wb, 1, C * 9, O)).astype(np.float32)
+    expect = oracle.conv2d_backward_weights(dw0.copy(), x, dy, 3, 3, 1)
+    got = host(nz.conv2d_backward_weights(dev(dw0), dev(x), dev(dy), 3, 3, 1, 1))
+    assert np.array_equal(got, expect)
+
+
+def test_conv2d_backward_weights_float_tolerance(nz, oracle):
+    N, C, H, W, O = 2, 48, 20, 72, 80
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, O, H, W)).astype(np.float32)
+    got = host(nz.conv2d_backward_weights(dev(np.zeros((1, 1, C * 9, O))), dev(x), dev(dy), 3, 3, 1, 1))
+    xr, dyr = oracle.round_f16(x).astype(np.float64), oracle.round_f16(dy).astype(np.float64)
+    xp = np.pad(xr, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    truth = np.zeros((C, 3, 3, O))
+    for r in range(3):
+        for sx in range(3):
+            truth[:, r, sx, :] = np.einsum("nchw,nohw->co", xp[:, :, r:r + H, sx:sx + W], dyr)
+    truth = truth.reshape(1, 1, C * 9, O)
+    mr, fr = oracle.errors(got, truth, float(np.sqrt(np.mean(truth ** 2))))
+    assert mr <= 1e-3 and fr <= 1e-4, (mr, fr)
+
+
+def test_conv2d_backward_weights_rejects_what_it_does_not_cover(nz):
+    from neuzephyr_amd.capi import NzHipError
+    with pytest.raises(NzHipError):      # W not a multiple of 8
+        nz.conv2d_backward_weights(dev(np.zeros((1, 1, 18, 3))), dev(np.zeros((1, 2, 6, 6))), dev(np.zeros((1, 3, 6, 6))), 3, 3, 1, 1)
+    with pytest.raises(NzHipError):      # 5x5
+        nz.conv2d_backward_weights(dev(np.zeros((1, 1, 50, 3))), dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 8, 8))), 5, 5, 1, 2)

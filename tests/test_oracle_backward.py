@@ -146,3 +146,18 @@ def test_conv2d_backward_data_equals_the_pinned_chain(oracle, N, C, H, W, O, K, 
     x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
     y = oracle.col2im(oracle.tensorcore_gemm(oracle.im2col(x, K, K, 1, pad), w), Ho, Wo)
     assert float((y.astype(np.float64) * dy).sum()) == float((x.astype(np.float64) * (got - dx0)).sum())
+
+
+@pytest.mark.parametrize("N,C,H,W,O,K,pad,wb", [(2, 3, 5, 6, 4, 3, 1, 1), (1, 2, 4, 4, 3, 3, 0, 1), (2, 2, 6, 5, 2, 3, 2, 2),
+                                                 (1, 3, 5, 5, 2, 1, 0, 1), (3, 4, 7, 9, 5, 3, 1, 3)])
+def test_conv2d_backward_weights_equals_the_pinned_chain(oracle, N, C, H, W, O, K, pad, wb):
+    # the one-statement weight gradient == Img2Col.forward -> MatMul.backward (dB) fed by Col2Img.backward;
+    # exact on integers
+    rng = np.random.default_rng(N + 10 * C + 100 * H + O + 7)
+    Ho, Wo = H + 2 * pad - K + 1, W + 2 * pad - K + 1
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    dy = rng.integers(-4, 5, size=(N, O, Ho, Wo)).astype(np.float32)
+    dw0 = rng.integers(-3, 4, size=(wb, 1, C * K * K, O)).astype(np.float32)
+    got = oracle.conv2d_backward_weights(dw0.copy(), x, dy, K, K, pad)
+    _, want = oracle.matmul_backward(oracle.im2col(x, K, K, 1, pad), dw0, oracle.col2im_backward(dy), dB0=dw0)
+    assert np.array_equal(got, want)
