@@ -150,12 +150,16 @@ namespace nz::graph {
                             }
                             const bool needW = rhs->output->requiresGrad();
                             const bool needB = biasNode && biasNode->output->requiresGrad();
-                            if (needW || needB)
+                            // weights straight from x and dZ where the geometry allows, else through the column matrix
+                            const bool directW = needW && iConv2dBackwardWeights(rhs->output->grad(), x->output->data(), dZ, xs[0],
+                                                                                 xs[1], xs[2], xs[3], O, i2c->kernelHeight,
+                                                                                 i2c->kernelWidth, i2c->stride, i2c->padding, ws[0]);
+                            if ((needW && !directW) || needB)
                                 iCol2imgBackward(pre->output->grad(), dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
                             if (needB)
                                 iAddBackward(biasNode->output->grad(), pre->output->grad(), biasNode->output->shape(),
                                              pre->output->shape());
-                            if (needW) {
+                            if (needW && !directW) {
                                 i2c->forward();                      // the column matrix the fused forward never wrote
                                 iMatMulBackward(nullptr, rhs->output->grad(), i2c->output->data(), rhs->output->data(),
                                                 pre->output->grad(), i2c->output->shape(), rhs->output->shape(),
