@@ -439,7 +439,7 @@ struct IgemmArgs {
     int C, H, W, O, H_out, W_out, pad;
     int n_chunks, n_otiles, tiles_w, tiles_h;
     int w_batched;
-    long bias_sp, bias_sc;
+    long bias_sp, bias_sc, bias_sn;   // bias element of (image b, pixel, channel o): bias[b*bias_sn + pixel*bias_sp + o*bias_sc]
     int relu;
 };
 
@@ -603,7 +603,7 @@ __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(con
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int o = o_base + i * 32 + (r >> 2) * 8 + (r & 3);
-                bv[i][r] = (p.bias && (o_full || o < p.O)) ? p.bias[pix * p.bias_sp + (long)o * p.bias_sc] : 0.f;
+                bv[i][r] = (p.bias && (o_full || o < p.O)) ? p.bias[(long)b * p.bias_sn + pix * p.bias_sp + (long)o * p.bias_sc] : 0.f;
             }
         float* dst = yb + pix;
 #pragma unroll
@@ -889,7 +889,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
 #pragma unroll
             for (int rr = 0; rr < 16; rr++) {
                 const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
-                bv[rr] = p.bias[pix * p.bias_sp + (long)((o_full || o < p.O) ? o : 0) * p.bias_sc];
+                bv[rr] = p.bias[(long)b * p.bias_sn + pix * p.bias_sp + (long)((o_full || o < p.O) ? o : 0) * p.bias_sc];
             }
         }
         auto finished = [&](const int rr) {
@@ -967,7 +967,7 @@ static bool conv_igemm_applicable(size_t C, size_t O, size_t K_h, size_t K_w, si
 template <int KH, int KW, int TW, int BN>
 static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
                              size_t H, size_t W, size_t O, size_t pad, size_t w_batch, int64_t bias_sp,
-                             int64_t bias_sc, int act, size_t H_out, size_t W_out, hipStream_t s) {
+                             int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out, hipStream_t s) {
     using G = IgemmGeom<KH, KW, TW, BN>;
     const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
     if (n_otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many output channels");
@@ -990,7 +990,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             a.pad = (int)pad; a.n_chunks = n_chunks; a.n_otiles = n_otiles;
             a.tiles_w = (int)((W_out + TW - 1) / TW);
             a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
-            a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.relu = act == NZHIP_ACT_RELU;
+            a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
             const long n_patches = (long)N * a.tiles_w * a.tiles_h;
             int rc = NZHIP_OK;
             if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
@@ -1049,6 +1049,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         a.w_batched = w_batch > 1;
         a.bias_sp = bias_sp;
         a.bias_sc = bias_sc;
+        a.bias_sn = bias_sn;
         a.relu = act == NZHIP_ACT_RELU;
         const bool vec4 = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
         auto kfn = vec4 ? conv_igemm_kernel<KH, KW, TW, BN, true> : conv_igemm_kernel<KH, KW, TW, BN, false>;
@@ -1297,16 +1298,27 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(const ConvDwArgs p) {
 __global__ __launch_bounds__(256) void conv_dw_reduce_kernel(float* __restrict__ dW, const float* __restrict__ P, int S,
                                                              int C, int O, int n_otiles, long group_stride_P,
                                                              long group_stride_dW) {
+    // 32 outputs per workgroup, eight threads per output: thread q adds the regions of its contiguous
+    // eighth in ascending order, then the eight sums are added in ascending q
+    __shared__ float part[8][32];
     const int chunk = blockIdx.y / n_otiles, ot = blockIdx.y % n_otiles, b = blockIdx.z;
     const int c0 = chunk * DW_CC, o0 = ot * DW_OT;
     const int nch = (C - c0) < DW_CC ? (C - c0) : DW_CC;
     const int ncols = (O - o0) < DW_OT ? (O - o0) : DW_OT;
-    const int t = blockIdx.x * 256 + threadIdx.x;
-    if (t >= nch * 9 * ncols) return;
+    const int q = threadIdx.x >> 5, tl = threadIdx.x & 31;
+    const int t = blockIdx.x * 32 + tl;
+    const bool live = t < nch * 9 * ncols;
     const long region = (long)DW_CC * 9 * DW_OT;
-    const float* src = P + (long)blockIdx.y * gridDim.z * group_stride_P + (long)b * group_stride_P + t;
+    const float* src = P + ((long)blockIdx.y * gridDim.z + b) * group_stride_P + t;
+    const int per = (S + 7) / 8, s0 = q * per, s1 = (s0 + per) < S ? (s0 + per) : S;
     float sum = 0.f;
-    for (int s = 0; s < S; s++) sum += src[(long)s * region];
+    if (live)
+        for (int s = s0; s < s1; s++) sum += src[(long)s * region];
+    part[q][tl] = sum;
+    __syncthreads();
+    if (q != 0 || !live) return;
+#pragma unroll
+    for (int k = 1; k < 8; k++) sum += part[k][tl];
     const int row = t / ncols, col = t % ncols;
     dW[(long)b * group_stride_dW + ((long)c0 * 9 + row) * O + o0 + col] += sum;
 }
@@ -1342,10 +1354,12 @@ __global__ __launch_bounds__(256) void accumulate_kernel(float* __restrict__ dst
 
 using namespace nzhip;
 
-extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref, const float* bias, size_t N,
-                                    size_t C, size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride,
-                                    size_t pad, size_t w_batch, int64_t bias_stride_pixel,
-                                    int64_t bias_stride_channel, int activation, void* stream) {
+// bias_stride_image != 0: the bias varies per image too (used to add into an existing tensor: bias = y with
+// strides (1, H_out*W_out, O*H_out*W_out)); only the implicit-GEMM kernels take it.
+static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
+                               size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                               size_t w_batch, int64_t bias_stride_pixel, int64_t bias_stride_channel,
+                               int64_t bias_stride_image, int activation, void* stream) {
     if (!y || !x || !w_ref) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_forward: null pointer");
     if (stride == 0 || K_h == 0 || K_w == 0) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_forward: zero stride or kernel extent");
     if (w_batch != 1 && w_batch != N) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
@@ -1356,6 +1370,10 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
     const size_t H_out = (H + 2 * pad - K_h) / stride + 1, W_out = (W + 2 * pad - K_w) / stride + 1;   // Nodes.cu:605-617
     if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const bool igemm_ok = !conv_direct_applicable(C, O, K_h, K_w, stride, pad) &&
+                          conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL;
+    if (bias_stride_image != 0 && !igemm_ok)
+        return set_error(NZHIP_E_UNSUPPORTED, "conv2d: a per-image bias needs the implicit-GEMM route");
     if (conv_direct_applicable(C, O, K_h, K_w, stride, pad))
         return conv_direct(y, x, w_ref, bias, N, C, H, W, O, w_batch, bias_stride_pixel, bias_stride_channel,
                            activation, s);
@@ -1367,7 +1385,7 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
         const bool bn128 = bn_env ? atoi(bn_env) == 128 : O > 64;
 #define NZHIP_IG(KH_, TW_, BN_)                                                                                      \
     return conv_igemm_launch<KH_, KH_, TW_, BN_>(y, x, w_ref, bias, N, C, H, W, O, pad, w_batch, bias_stride_pixel, \
-                                                 bias_stride_channel, activation, H_out, W_out, s)
+                                                 bias_stride_channel, bias_stride_image, activation, H_out, W_out, s)
         if (K_h == 3) {
             if (wide && bn128) NZHIP_IG(3, 64, 128);
             if (wide) NZHIP_IG(3, 64, 64);
@@ -1380,6 +1398,14 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
     }
     return conv2d_via_workspace(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
                                 bias_stride_channel, activation, H_out, W_out, s);
+}
+
+extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref, const float* bias, size_t N,
+                                    size_t C, size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride,
+                                    size_t pad, size_t w_batch, int64_t bias_stride_pixel,
+                                    int64_t bias_stride_channel, int activation, void* stream) {
+    return conv2d_forward_impl(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
+                               bias_stride_channel, 0, activation, stream);
 }
 
 /* Gradient of nzhip_conv2d_forward with respect to x for stride 1: one convolution of dy with the
@@ -1406,17 +1432,25 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     float* tmp = nullptr;
     if (int rc = workspace_alloc(reinterpret_cast<void**>(&wflip), w_elems * sizeof(float), s)) return rc;
     int rc = NZHIP_OK;
-    if (accumulate) rc = workspace_alloc(reinterpret_cast<void**>(&tmp), x_elems * sizeof(float), s);
+    // "+=": the implicit-GEMM kernels read dx as their bias (same lane reads, then writes each element); the other
+    // routes go through a temporary and one add pass
+    const size_t pad_t = K_h - 1 - pad;
+    const bool in_place = accumulate && !conv_direct_applicable(O, C, K_h, K_w, 1, pad_t) &&
+                          conv_igemm_applicable(O, C, K_h, K_w, 1, pad_t, N) && (long)H_out * W_out < 0x7fffffffL;
+    if (accumulate && !in_place) rc = workspace_alloc(reinterpret_cast<void**>(&tmp), x_elems * sizeof(float), s);
     if (rc == NZHIP_OK) {
         hipLaunchKernelGGL(conv_weight_flip_kernel, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, s, wflip, w_ref,
                            (int)C, (int)O, (int)K_h, (int)K_w, (long)w_elems);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_weight_flip kernel launch");
     }
-    if (rc == NZHIP_OK)
-        rc = nzhip_conv2d_forward(accumulate ? tmp : dx, dy, wflip, nullptr, N, O, H_out, W_out, C, K_h, K_w, 1,
-                                  K_h - 1 - pad, w_batch, 0, 0, NZHIP_ACT_NONE, stream);
-    if (rc == NZHIP_OK && accumulate) {
+    if (rc == NZHIP_OK && in_place)
+        rc = conv2d_forward_impl(dx, dy, wflip, dx, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t, w_batch, 1, (int64_t)(H * W),
+                                 (int64_t)(C * H * W), NZHIP_ACT_NONE, stream);
+    else if (rc == NZHIP_OK)
+        rc = conv2d_forward_impl(accumulate ? tmp : dx, dy, wflip, nullptr, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t,
+                                 w_batch, 0, 0, 0, NZHIP_ACT_NONE, stream);
+    if (rc == NZHIP_OK && accumulate && !in_place) {
         hipLaunchKernelGGL(accumulate_kernel, dim3((unsigned)((x_elems / 4 + 256) / 256)), dim3(256), 0, s, dx, tmp,
                            (long)x_elems);
         hipError_t e = hipGetLastError();
@@ -1445,9 +1479,10 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const int chunks = (int)((C + DW_CC - 1) / DW_CC), otiles = (int)((O + DW_OT - 1) / DW_OT);
     if (chunks > 65535 || otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_weights: too many channels");
-    // about two workgroups per CU in total; a band is a whole number of rows of one image
+    // one workgroup per CU in total (its LDS footprint leaves room for no second one); a band is a whole
+    // number of rows of one image
     const int cus = device_cu_count();
-    long want = (2L * cus + (long)chunks * otiles * (long)N - 1) / ((long)chunks * otiles * (long)N);
+    long want = ((long)cus + (long)chunks * otiles * (long)N - 1) / ((long)chunks * otiles * (long)N);
     if (want < 1) want = 1;
     if (want > (long)H) want = (long)H;
     const int band_rows = (int)((H + want - 1) / want);
@@ -1473,7 +1508,7 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
         const bool shared = w_batch == 1;
         const int S = shared ? (int)(N * bands) : bands;
         const int groups = shared ? 1 : (int)N;
-        dim3 grid((unsigned)((region + 255) / 256), (unsigned)(chunks * otiles), (unsigned)groups);
+        dim3 grid((unsigned)((region + 31) / 32), (unsigned)(chunks * otiles), (unsigned)groups);
         hipLaunchKernelGGL(conv_dw_reduce_kernel, grid, dim3(256), 0, s, dw, partial, S, (int)C, (int)O, otiles,
                            (long)((size_t)S * region), (long)(C * 9 * O));
         hipError_t e = hipGetLastError();
