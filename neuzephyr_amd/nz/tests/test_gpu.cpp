@@ -625,6 +625,32 @@ TEST(Model, LinearTrainingStepLowersTheOutputSum) {
     EXPECT_TRUE(total() < before);
 }
 
+TEST(Model, ConvTrainingStepsLowerTheOutputSum) {
+    // Conv2d + ReLU: forward -> fused backward (weights straight from x and dy, data gradient as one convolution)
+    // -> Adam, three times; the sum of the outputs goes down every step
+    ConvModel m(2, 16, 12, 24, 20, 3, 1, 1, true);
+    auto x = randomVec(2 * 16 * 12 * 24, 91, -1.f, 1.f);
+    m.input.dataInject(x.begin(), x.end());
+    auto W = randomVec(2 * 16 * 9 * 20, 92, 0.0f, 0.2f), b = randomVec(12 * 24 * 20, 93, 0.1f, 0.3f);
+    m.parameters()[0]->dataInject(W.begin(), W.end());
+    m.parameters()[1]->dataInject(b.begin(), b.end());
+    auto total = [&] {
+        double s = 0;
+        for (float v : m.forward().hostData()) s += v;
+        return s;
+    };
+    nz::opt::Adam optimizer(0.01f, 0.9f, 0.999f);
+    double before = total();
+    EXPECT_EQ(m.graph().fusedGroupCount(), 1u);
+    for (int step = 0; step < 3; ++step) {
+        m.backward();
+        m.update(&optimizer);
+        const double after = total();
+        EXPECT_TRUE(after < before);
+        before = after;
+    }
+}
+
 // ---- softmax (test/Test.cpp:1733-1870) -------------------------------------------------------------
 TEST(NodeBasic, SoftmaxForwardJacobianBackward) {
     const size_t n = 2, c = 3, h = 12, w = 1;
