@@ -36,7 +36,13 @@ def check_tolerance(oracle, got, truth64, tag=""):
 
 IM2COL_CASES = [((2, 3, 4, 5), 3, 3, 1, 1), ((1, 1, 1, 1), 1, 1, 1, 0), ((2, 2, 7, 6), 3, 2, 2, 0),
                 ((1, 3, 8, 9), 2, 4, 2, 2), ((3, 1, 5, 5), 5, 5, 1, 2), ((2, 4, 6, 6), 1, 1, 3, 0),
-                ((2, 5, 33, 47), 3, 3, 1, 1)]
+                ((2, 5, 33, 47), 3, 3, 1, 1),
+                # stride 1 with C*K_h*K_w a multiple of 4: the kernel that stages input rows in LDS (64-pixel segments,
+                # 32-channel chunks with a tail, compile-time and run-time kernel extents)
+                ((2, 4, 6, 7), 3, 3, 1, 1), ((1, 64, 5, 130), 3, 3, 1, 1), ((2, 40, 9, 70), 3, 3, 1, 0),
+                ((2, 8, 7, 66), 1, 1, 1, 0), ((1, 4, 9, 75), 5, 5, 1, 2), ((2, 2, 8, 9), 2, 2, 1, 1), ((1, 36, 4, 64), 3, 3, 1, 2),
+                # other strides with a multiple of 4: the 16-byte store variant of the per-element kernel
+                ((2, 4, 9, 9), 3, 3, 2, 1), ((1, 8, 10, 12), 2, 3, 3, 0)]
 
 
 @pytest.mark.parametrize("shape,k_h,k_w,stride,pad", IM2COL_CASES)
