@@ -1138,6 +1138,9 @@ struct ConvDwArgs {
     int n_images;
 };
 
+// VEC: W is a multiple of 8 and x, dy are 16-byte aligned (two 16-byte loads per group of 8 pixels); otherwise
+// every pixel is loaded and bounds-checked on its own.
+template <bool VEC>
 __global__ __launch_bounds__(256) void conv_dw_kernel(const ConvDwArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     char* xs = lds;                       // [slot 3][shift 3][channel 32] rows of DW_PITCH bytes
@@ -1172,18 +1175,24 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(const ConvDwArgs p) {
         for (int u = 0; u < 2; u++) {
             const int c = u * 16 + (tid >> 4);
             const int w = w0 + g * 8;
-            const bool ok = c < nch && h >= 0 && h < p.H && w < p.W;       // W is a multiple of 8: a group is inside or outside
+            const bool ok = c < nch && h >= 0 && h < p.H && w < p.W;       // VEC: a group is wholly inside or outside
             const float* src = ximg + (long)c * plane + (long)h * p.W + w;
 #pragma unroll
             for (int e = 0; e < 8; e++) xr[u][e] = 0.f;
             xl[u] = 0.f;
             xrt[u] = 0.f;
             if (ok) {
-                const floatx4 a = *reinterpret_cast<const floatx4*>(src), b = *reinterpret_cast<const floatx4*>(src + 4);
+                if (VEC) {
+                    const floatx4 a = *reinterpret_cast<const floatx4*>(src), b = *reinterpret_cast<const floatx4*>(src + 4);
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    xr[u][e] = a[e];
-                    xr[u][4 + e] = b[e];
+                    for (int e = 0; e < 4; e++) {
+                        xr[u][e] = a[e];
+                        xr[u][4 + e] = b[e];
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        if (w + e < p.W) xr[u][e] = src[e];
                 }
                 if (g == 0 && w > 0) xl[u] = src[-1];
                 if (g == 15 && w + 8 < p.W) xrt[u] = src[8];
@@ -1200,11 +1209,17 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(const ConvDwArgs p) {
 #pragma unroll
             for (int e = 0; e < 8; e++) zr[i][e] = 0.f;
             if (ok) {
-                const floatx4 a = *reinterpret_cast<const floatx4*>(src), b = *reinterpret_cast<const floatx4*>(src + 4);
+                if (VEC) {
+                    const floatx4 a = *reinterpret_cast<const floatx4*>(src), b = *reinterpret_cast<const floatx4*>(src + 4);
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    zr[i][e] = a[e];
-                    zr[i][4 + e] = b[e];
+                    for (int e = 0; e < 4; e++) {
+                        zr[i][e] = a[e];
+                        zr[i][4 + e] = b[e];
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        if (w + e < p.W) zr[i][e] = src[e];
                 }
             }
         }
@@ -1470,11 +1485,11 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
                                              size_t w_batch, void* stream) {
     if (!dw || !x || !dy) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_weights: null pointer");
     if (w_batch != 1 && w_batch != N) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
-    if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1 || W % 8 != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(dy) & 15) != 0 || H == 0 ||
-        H > 0x3fffffff || W > 0x3fffffff || C > 0x3fffffff || O > 0x3fffffff || N > 65535)
+    if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1 || H == 0 || W == 0 || H > 0x3fffffff || W > 0x3fffffff ||
+        C > 0x3fffffff || O > 0x3fffffff || N > 65535)
         return set_error(NZHIP_E_UNSUPPORTED,
-                         "nzhip_conv2d_backward_weights: only 3x3, stride 1, pad 1, W a multiple of 8, 16-byte aligned "
-                         "tensors (use the column-matrix chain)");
+                         "nzhip_conv2d_backward_weights: only 3x3, stride 1, pad 1 (use the column-matrix chain)");
+    const bool vec = W % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
     if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const int chunks = (int)((C + DW_CC - 1) / DW_CC), otiles = (int)((O + DW_OT - 1) / DW_OT);
@@ -1497,10 +1512,11 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
     a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O;
     a.bands = bands; a.band_rows = band_rows; a.n_images = (int)N;
     const int lds_bytes = DW_XS_BYTES + DW_ZS_BYTES;
-    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(conv_dw_kernel), lds_bytes, "hipFuncSetAttribute(conv_dw)");
+    auto kfn = vec ? conv_dw_kernel<true> : conv_dw_kernel<false>;
+    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), lds_bytes, "hipFuncSetAttribute(conv_dw)");
     if (rc == NZHIP_OK) {
         dim3 grid((unsigned)(N * bands), (unsigned)chunks, (unsigned)otiles);
-        hipLaunchKernelGGL(conv_dw_kernel, grid, dim3(256), lds_bytes, s, a);
+        hipLaunchKernelGGL(kfn, grid, dim3(256), lds_bytes, s, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_dw kernel launch");
     }

@@ -141,8 +141,7 @@ namespace nz::data {
     bool iConv2dBackwardWeights(float* dw, float* x, float* dy, const size_t N, const size_t C, const size_t H,
                                 const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
                                 const size_t pad, const size_t weightBatch) {
-        if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1 || W % 8 != 0) return false;
-        if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(dy) & 15) != 0) return false;
+        if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1) return false;
         NZ_CHECK(nzhip_conv2d_backward_weights(dw, x, dy, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch,
                                                nzhip_default_stream()));
         return true;

@@ -240,9 +240,10 @@ def test_conv2d_backward_data_rejects_what_it_does_not_cover(nz):
         nz.conv2d_backward_data(dx, dy, w, 3, 3, 2, 1)
 
 
-CONV_BWD_W = [  # N, C, H, W, O, w_batch   (3x3, stride 1, pad 1, W a multiple of 8)
+CONV_BWD_W = [  # N, C, H, W, O, w_batch   (3x3, stride 1, pad 1; W a multiple of 8 takes 16-byte loads)
     (1, 3, 4, 8, 2, 1), (2, 5, 7, 16, 9, 1), (2, 32, 9, 24, 40, 2), (3, 40, 6, 136, 130, 1), (1, 64, 16, 128, 128, 1),
-    (2, 33, 5, 264, 129, 2), (4, 8, 33, 40, 16, 1), (1, 1, 1, 8, 1, 1)]
+    (2, 33, 5, 264, 129, 2), (4, 8, 33, 40, 16, 1), (1, 1, 1, 8, 1, 1),
+    (2, 3, 28, 28, 6, 1), (1, 5, 7, 9, 4, 1), (2, 20, 6, 131, 33, 2), (1, 2, 3, 1, 2, 1), (1, 4, 5, 127, 3, 1)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,wb", CONV_BWD_W)
@@ -276,7 +277,7 @@ def test_conv2d_backward_weights_float_tolerance(nz, oracle):
 
 def test_conv2d_backward_weights_rejects_what_it_does_not_cover(nz):
     from neuzephyr_amd.capi import NzHipError
-    with pytest.raises(NzHipError):      # W not a multiple of 8
-        nz.conv2d_backward_weights(dev(np.zeros((1, 1, 18, 3))), dev(np.zeros((1, 2, 6, 6))), dev(np.zeros((1, 3, 6, 6))), 3, 3, 1, 1)
+    with pytest.raises(NzHipError):      # stride 2
+        nz.conv2d_backward_weights(dev(np.zeros((1, 1, 18, 3))), dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 4, 4))), 3, 3, 2, 1)
     with pytest.raises(NzHipError):      # 5x5
         nz.conv2d_backward_weights(dev(np.zeros((1, 1, 50, 3))), dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 8, 8))), 5, 5, 1, 2)
