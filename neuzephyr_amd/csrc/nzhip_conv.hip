@@ -625,11 +625,11 @@ __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(con
 // lets the epilogue stores of one patch drain while the next patch is staged and computed.
 // Weight rows are unpadded (TAPS*32 bytes); rows o and o+8 would share LDS banks, so the two
 // 16-byte halves of every (row, tap) are swapped when bit 3 of the row is set.
-template <int KH, int KW>
+template <int KH, int KW, int BN>
 __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float16* __restrict__ dst,
                                                                          const float* __restrict__ w_ref, int C,
                                                                          int O, int n_chunks, int n_otiles) {
-    constexpr int TAPS = KH * KW, BN = 128;
+    constexpr int TAPS = KH * KW;
     const int slab = blockIdx.y;                               // o_tile * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = slab / n_chunks;
     const int t = blockIdx.x * 256 + threadIdx.x;
@@ -655,10 +655,11 @@ __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float1
 // activation on the way out).
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 
-template <int KH, int KW, int TW, bool VEC4, bool PIX_BIAS>
+// NI: 32-channel blocks per wave; the channel tile of a workgroup is BN = 64 * NI (128 or 64) output channels.
+template <int KH, int KW, int TW, bool VEC4, bool PIX_BIAS, int NI>
 __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArgs p, const int n_patches) {
     using G = IgemmGeom<KH, KW, TW, 128>;
-    constexpr int BN = 128, CB = TW / 32, FP = 2, NW = 8;
+    constexpr int BN = 64 * NI, WCH = 32 * NI, CB = TW / 32, FP = 2, NW = 8;   // WCH: channels per wave
     constexpr int W_PITCH = G::TAPS * 32, W_CHUNK = BN * W_PITCH;           // unpadded rows
     static_assert(W_CHUNK % 1024 == 0, "chunk must be whole 1 KiB wave loads");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -812,13 +813,13 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
 
     // A per-channel bias (or zero) is the starting value of every accumulator; the 128 values of the
     // channel tile sit in LDS behind the halo and are read back at the start of each patch.
-    floatx16 acc[2][FP];
+    floatx16 acc[NI][FP];
     auto init_acc = [&]() {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int i = 0; i < NI; i++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const floatx4 bq = *reinterpret_cast<const floatx4*>(lds_bias + wn * 64 + i * 32 + g * 8 + lh * 4);
+                const floatx4 bq = *reinterpret_cast<const floatx4*>(lds_bias + wn * WCH + i * 32 + g * 8 + lh * 4);
 #pragma unroll
                 for (int j = 0; j < FP; j++)
 #pragma unroll
@@ -832,12 +833,12 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     // sits outside the branch on `live`, so an empty item (odd chunk count) issues the same requests
     // as a full one without touching LDS or the matrix pipe.
     auto compute = [&](int chunk, const bool live, auto after_tap) {
-        const char* wbase = lds_w + chunk * W_CHUNK + (wn * 64 + li) * W_PITCH + ((lh ^ ((li >> 3) & 1)) << 4);
-        half8_t wf[2][2], pf[2][FP];
-        auto read_frags = [&](const int tap, half8_t (&w)[2], half8_t (&x)[FP]) {
+        const char* wbase = lds_w + chunk * W_CHUNK + (wn * WCH + li) * W_PITCH + ((lh ^ ((li >> 3) & 1)) << 4);
+        half8_t wf[2][NI], pf[2][FP];
+        auto read_frags = [&](const int tap, half8_t (&w)[NI], half8_t (&x)[FP]) {
             const int kh = tap / KW, kw = tap % KW;
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < NI; i++)
                 w[i] = *reinterpret_cast<const half8_t*>(wbase + i * 32 * W_PITCH + tap * 32);
 #pragma unroll
             for (int j = 0; j < FP; j++) {
@@ -854,7 +855,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
                 if (tap + 1 < G::TAPS) read_frags(tap + 1, wf[(tap + 1) & 1], pf[(tap + 1) & 1]);
                 __builtin_amdgcn_sched_barrier(0);               // requests stay ahead of the MFMAs below
 #pragma unroll
-                for (int i = 0; i < 2; i++)
+                for (int i = 0; i < NI; i++)
 #pragma unroll
                     for (int j = 0; j < FP; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[tap & 1][i], pf[tap & 1][j], acc[i][j], 0, 0, 0);
@@ -864,7 +865,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
         }
     };
 
-    const int o_wave = o_tile * BN + wn * 64;                    // uniform; lane channel = o_wave + lh*4 + i*32 + ...
+    const int o_wave = o_tile * BN + wn * WCH;                   // uniform; lane channel = o_wave + lh*4 + i*32 + ...
     const bool o_full = o_tile * BN + BN <= p.O;                 // uniform: whole channel tile exists
     const long hw_out = (long)p.H_out * p.W_out;
 
@@ -954,7 +955,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
 #pragma unroll
         for (int j = 0; j < FP; j++)
 #pragma unroll
-            for (int i = 0; i < 2; i++) flush_unit(j, i, patch);
+            for (int i = 0; i < NI; i++) flush_unit(j, i, patch);
     }
 }
 
@@ -972,8 +973,9 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
     if (n_otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many output channels");
     // Resident-weight route: shared weights whose fp16 image (unpadded) plus one halo fit in LDS.
-    if constexpr (BN == 128) {
-        constexpr size_t W_CHUNK_R = 128 * (size_t)G::TAPS * 32;
+    {
+        constexpr size_t W_CHUNK_R = BN * (size_t)G::TAPS * 32;
+        constexpr int NI = BN / 64;
         const size_t lds_need = (size_t)n_chunks * W_CHUNK_R + G::HALO_BYTES + 128 * sizeof(float);   // + bias
         static const char* res_env = getenv("NZHIP_CONV_RESIDENT");
         const bool allow = res_env ? atoi(res_env) != 0 : true;
@@ -981,8 +983,8 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             _Float16* wres = nullptr;
             const size_t bytes = (size_t)n_otiles * n_chunks * W_CHUNK_R;
             if (int rc = workspace_alloc(reinterpret_cast<void**>(&wres), bytes, s)) return rc;
-            dim3 pg((unsigned)((128 * G::TAPS * IG_CC + 255) / 256), (unsigned)(n_otiles * n_chunks));
-            hipLaunchKernelGGL((conv_weight_image_resident_kernel<KH, KW>), pg, dim3(256), 0, s, wres, w_ref, (int)C,
+            dim3 pg((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)(n_otiles * n_chunks));
+            hipLaunchKernelGGL((conv_weight_image_resident_kernel<KH, KW, BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C,
                                (int)O, n_chunks, n_otiles);
             IgemmArgs a;
             a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
@@ -996,10 +998,10 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
             const bool vec4r = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
             const bool pixb = bias && bias_sp != 0;
-            auto kres = vec4r ? (pixb ? conv_igemm_resident_kernel<KH, KW, TW, true, true>
-                                      : conv_igemm_resident_kernel<KH, KW, TW, true, false>)
-                              : (pixb ? conv_igemm_resident_kernel<KH, KW, TW, false, true>
-                                      : conv_igemm_resident_kernel<KH, KW, TW, false, false>);
+            auto kres = vec4r ? (pixb ? conv_igemm_resident_kernel<KH, KW, TW, true, true, NI>
+                                      : conv_igemm_resident_kernel<KH, KW, TW, true, false, NI>)
+                              : (pixb ? conv_igemm_resident_kernel<KH, KW, TW, false, true, NI>
+                                      : conv_igemm_resident_kernel<KH, KW, TW, false, false, NI>);
             if (rc == NZHIP_OK)
                 rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kres), (int)lds_need, "hipFuncSetAttribute(conv_igemm_resident)");
             if (rc == NZHIP_OK) {
