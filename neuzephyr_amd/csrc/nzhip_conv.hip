@@ -1394,7 +1394,9 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
     if (conv_direct_applicable(C, O, K_h, K_w, stride, pad))
         return conv_direct(y, x, w_ref, bias, N, C, H, W, O, w_batch, bias_stride_pixel, bias_stride_channel,
                            activation, s);
-    if (conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL) {
+    static const char* route_env = getenv("NZHIP_CONV_ROUTE");      // "workspace": column matrix + GEMM (benchmarking only)
+    const bool force_ws = route_env && route_env[0] == 'w' && bias_stride_image == 0;
+    if (!force_ws && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL) {
         // NZHIP_CONV_TW=32|64 and NZHIP_CONV_BN=64|128 override the tile choice (benchmarking only)
         static const char* tw_env = getenv("NZHIP_CONV_TW");
         static const char* bn_env = getenv("NZHIP_CONV_BN");
