@@ -28,6 +28,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
                     choices=["gemm8192", "gemm_batched", "linear", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "gemv", "ragged", "conv_a", "conv_b",
+                             "adam", "softmax_bwd", "matmul_f32",
                              "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary (conv / linear) measurements")
@@ -262,6 +263,75 @@ def make_workload(name, orc, capi):
         bytes_ = 4.0 * (N * C * H * W + O * C * 9 + O + N * O * H * W)
         return Workload(name, flops, bytes_, run, verify, "hbm",
                         f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},3,3] s1 p1 + bias + ReLU"), None
+    if name == "adam":
+        # opt::Adam::step over 2^26 parameters: data, m, v read and written, the gradient read
+        n = 1 << 26
+        gen = torch.Generator(device="cuda").manual_seed(5)
+        d = torch.randn(n, device="cuda", generator=gen)
+        g = torch.randn(n, device="cuda", generator=gen)
+        m = torch.zeros(n, device="cuda")
+        v = torch.zeros(n, device="cuda")
+        step = [0]
+
+        def run():
+            step[0] += 1
+            capi.adam_step(d, m, v, g, 1e-3, 0.9, 0.999, 1e-8, step[0])
+
+        def verify():
+            # one more step on a slice of the live state against the CPU restatement
+            k = 1 << 16
+            hs = [t[:k].cpu().numpy().copy() for t in (d, m, v, g)]
+            ds, ms_, vs = d[:k].clone(), m[:k].clone(), v[:k].clone()
+            capi.adam_step(ds, ms_, vs, g[:k], 1e-3, 0.9, 0.999, 1e-8, step[0] + 1)
+            do, mo, vo = orc.adam_step(hs[0], hs[1], hs[2], hs[3], 1e-3, 0.9, 0.999, 1e-8, step[0] + 1)
+            ok = (np.allclose(ds.cpu().numpy(), do, rtol=1e-5, atol=1e-6) and np.allclose(ms_.cpu().numpy(), mo, rtol=1e-6, atol=1e-7)
+                  and np.allclose(vs.cpu().numpy(), vo, rtol=1e-6, atol=1e-7))
+            if not ok:
+                raise SystemExit("VERIFY FAILED adam")
+            return {"allclose_1e-5": True}
+
+        return Workload(name, 12.0 * n, 28.0 * n, run, verify, "hbm", "Adam step over 2^26 fp32 parameters"), None
+    if name == "softmax_bwd":
+        # SoftmaxNode::backward for 64 vectors of 4096 classes: Jacobian x gradient, fp16-rounded operands,
+        # the Jacobian never in memory (the two-call spelling would write and read 64 x 64 MiB)
+        n, batch = 4096, 64
+        x = orc.fill((batch, 1, n, 1), 6, "uniform", -4.0, 4.0)
+        so = orc.softmax(x)
+        dy = orc.fill((batch, 1, n, 1), 1006, "uniform", -1.0, 1.0)
+        sd, dyd = dev(so), dev(dy)
+        out = [None]
+
+        def run():
+            out[0] = capi.softmax_backward(sd, dyd)
+
+        def verify():
+            want = orc.softmax_backward(so[:2], dy[:2])
+            if not np.array_equal(out[0][:2].cpu().numpy(), want):
+                raise SystemExit("VERIFY FAILED softmax_bwd")
+            return {"bit_exact": True}
+
+        return Workload(name, 2.0 * n * n * batch, 12.0 * n * batch, run, verify, "mfma",
+                        "softmax backward, 64 vectors x 4096 (fp32 VALU kernel, fp16-rounded operands)"), None
+    if name == "matmul_f32":
+        # Tensor::operator*: fp32-exact product, one FMA chain per output in ascending k (VALU kernel)
+        M = 2048
+        A = orc.fill((M, M), 7, "uniform", -1.0, 1.0)
+        B = orc.fill((M, M), 1007, "uniform", -1.0, 1.0)
+        Ad, Bd = dev(A).reshape(1, 1, M, M), dev(B).reshape(1, 1, M, M)
+        out = torch.empty((1, 1, M, M), device="cuda")
+
+        def run():
+            capi.matmul_f32(Ad, Bd, out=out)
+
+        def verify():
+            rows = 16
+            want = orc.general_matmul(A[:rows].reshape(1, 1, rows, M), B.reshape(1, 1, M, M))
+            if not np.array_equal(out[0, 0, :rows].cpu().numpy(), want.reshape(rows, M)):
+                raise SystemExit("VERIFY FAILED matmul_f32")
+            return {"bit_exact": True}
+
+        return Workload(name, 2.0 * M ** 3, 12.0 * M * M, run, verify, "mfma",
+                        "fp32-exact A[2048,2048] * B[2048,2048] (fp32 VALU kernel; fp32 vector peak 157.3 TFLOP/s)"), None
     if name == "copy":
         # Calibration only: a plain device copy of known size (1 GiB read + 1 GiB written), so that
         # rocprofv3's FETCH_SIZE / WRITE_SIZE readings can be scaled to bytes.
@@ -376,7 +446,8 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx"):
+        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "adam",
+                     "softmax_bwd", "matmul_f32"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)
             ms2, _ = time_steps(w2, max(10, args.steps // 2), max(3, args.warmup // 2))

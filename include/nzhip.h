@@ -212,6 +212,12 @@ int nzhip_softmax(float* out, const float* in, size_t len, size_t batch, void* s
  * (J x dY for column vectors, dY x J for row vectors). */
 int nzhip_softmax_jacobian(float* out, const float* in, size_t n, size_t batch, void* stream);
 
+/* SoftmaxNode::backward (src/Nodes.cu:538-548) in one kernel, without the n x n Jacobian in memory:
+ * dx[b][i] = sum_j fp16(J[b][i][j]) * fp16(dy[b][j]) with J as above, fp32 accumulation in ascending j,
+ * i.e. the values nzhip_softmax_jacobian + nzhip_tensorcore_gemm give up to the order of the fp32
+ * additions (the Jacobian is symmetric, so column and row vectors are the same sums). dx is overwritten. */
+int nzhip_softmax_backward(float* dx, const float* s, const float* dy, size_t n, size_t batch, void* stream);
+
 /* ---- runtime: device allocator + stream manager -------------------------- */
 /* Replace cuStrm::StreamManager<float> (include/NeuZephyr/StreamManager.cuh:131-911) and
  * EventPool (EventPool.cuh:165-457).  One ordered compute stream carries every kernel and

@@ -19,7 +19,7 @@ EXPORTS = [
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
-    "nzhip_softmax", "nzhip_softmax_jacobian",
+    "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
@@ -88,6 +88,7 @@ def load() -> C.CDLL:
     lib.nzhip_sgd_step.argtypes = [vp, vp, C.c_float, sz, vp]
     lib.nzhip_softmax.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_softmax_jacobian.argtypes = [vp, vp, sz, sz, vp]
+    lib.nzhip_softmax_backward.argtypes = [vp, vp, vp, sz, sz, vp]
     lib.nzhip_adam_step.argtypes = [vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, sz, vp]
     lib.nzhip_default_stream.restype = vp
     lib.nzhip_malloc.argtypes = [C.POINTER(vp), sz]
@@ -355,6 +356,16 @@ def softmax_jacobian(s, stream=None):
 
 
 def softmax_backward(s, dy, stream=None):
-    """SoftmaxNode::backward: Jacobian times gradient through the fp16 GEMM entry."""
+    """SoftmaxNode::backward in one kernel (no Jacobian in memory)."""
+    import torch
+    lib = load()
+    dx = torch.empty_like(s)
+    check(lib.nzhip_softmax_backward(_dev(dx), _dev(s), _dev(dy), s.shape[2] * s.shape[3], s.shape[0] * s.shape[1],
+                                     _stream_handle(stream)))
+    return dx
+
+
+def softmax_backward_gemm(s, dy, stream=None):
+    """SoftmaxNode::backward as the reference spells it: Jacobian times gradient through the fp16 GEMM entry."""
     jac = softmax_jacobian(s, stream)
     return tensorcore_gemm(jac, dy, stream=stream) if s.shape[2] > s.shape[3] else tensorcore_gemm(dy, jac, stream=stream)

@@ -11,6 +11,7 @@
 namespace nzhip {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 
 static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -134,27 +135,75 @@ __global__ __launch_bounds__(256) void matmul_f32_kernel(const F32Args p) {
 }
 
 // ---- optimizer steps ----------------------------------------------------------------------------
+// One thread updates four adjacent elements (16-byte loads and stores) when the arrays are 16-byte
+// aligned, one element otherwise; the last n % 4 elements go to the first threads of the last
+// workgroup. The arithmetic per element is the same expression in every variant.
+// The multiply-adds are spelled as FMAs (what a contracting compiler makes of `d -= lr * g` and of
+// `m * beta1 + g * (1 - beta1)`), so that every variant of a kernel rounds the same way.
+__device__ __forceinline__ float sgd_one(float d, float g, float lr) { return __builtin_fmaf(-lr, g, d); }
+
+template <int VEC>
 __global__ __launch_bounds__(256) void sgd_kernel(float* __restrict__ data, const float* __restrict__ grad, float lr,
                                                   long n) {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) data[i] -= lr * grad[i];
+    if constexpr (VEC == 4) {
+        const long n4 = n >> 2;
+        if (i < n4) {
+            floatx4 d = reinterpret_cast<const floatx4*>(data)[i];
+            const floatx4 g = reinterpret_cast<const floatx4*>(grad)[i];
+#pragma unroll
+            for (int e = 0; e < 4; e++) d[e] = sgd_one(d[e], g[e], lr);
+            reinterpret_cast<floatx4*>(data)[i] = d;
+        }
+        const long t = n4 * 4 + threadIdx.x;
+        if (blockIdx.x == gridDim.x - 1 && t < n) data[t] = sgd_one(data[t], grad[t], lr);
+    } else {
+        if (i < n) data[i] = sgd_one(data[i], grad[i], lr);
+    }
 }
 
 // bias corrections 1 - beta^t are computed once on the host (in fp32, like the kernel of the reference)
+struct AdamArgs {
+    float lr, beta1, beta2, eps, corr1, corr2;
+};
+
+__device__ __forceinline__ void adam_one(float& d, float& m, float& v, float g, const AdamArgs& a) {
+    const float m_temp = __builtin_fmaf(m, a.beta1, g * (1 - a.beta1));
+    const float v_temp = __builtin_fmaf(v, a.beta2, (g * g) * (1 - a.beta2));
+    const float m_modified = m_temp / a.corr1;
+    const float v_modified = v_temp / a.corr2;
+    d -= a.lr * m_modified / (sqrtf(v_modified) + a.eps);
+    m = m_temp;
+    v = v_temp;
+}
+
+template <int VEC>
 __global__ __launch_bounds__(256) void adam_kernel(float* __restrict__ data, float* __restrict__ m,
-                                                   float* __restrict__ v, const float* __restrict__ grad, float lr,
-                                                   float beta1, float beta2, float eps, float corr1, float corr2,
-                                                   long n) {
+                                                   float* __restrict__ v, const float* __restrict__ grad,
+                                                   const AdamArgs a, long n) {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const float g = grad[i];
-    const float m_temp = m[i] * beta1 + g * (1 - beta1);
-    const float v_temp = v[i] * beta2 + g * g * (1 - beta2);
-    const float m_modified = m_temp / corr1;
-    const float v_modified = v_temp / corr2;
-    data[i] -= lr * m_modified / (sqrtf(v_modified) + eps);
-    m[i] = m_temp;
-    v[i] = v_temp;
+    if constexpr (VEC == 4) {
+        const long n4 = n >> 2;
+        if (i < n4) {
+            floatx4 d = reinterpret_cast<const floatx4*>(data)[i];
+            floatx4 mm = reinterpret_cast<const floatx4*>(m)[i];
+            floatx4 vv = reinterpret_cast<const floatx4*>(v)[i];
+            const floatx4 g = reinterpret_cast<const floatx4*>(grad)[i];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float de = d[e], me = mm[e], ve = vv[e];
+                adam_one(de, me, ve, g[e], a);
+                d[e] = de; mm[e] = me; vv[e] = ve;
+            }
+            reinterpret_cast<floatx4*>(data)[i] = d;
+            reinterpret_cast<floatx4*>(m)[i] = mm;
+            reinterpret_cast<floatx4*>(v)[i] = vv;
+        }
+        const long t = n4 * 4 + threadIdx.x;
+        if (blockIdx.x == gridDim.x - 1 && t < n) adam_one(data[t], m[t], v[t], grad[t], a);
+    } else {
+        if (i < n) adam_one(data[i], m[i], v[i], grad[i], a);
+    }
 }
 
 // ---- softmax over one vector per (n, c) and its Jacobian ---------------------------------------
@@ -183,6 +232,66 @@ __global__ __launch_bounds__(256) void softmax_jacobian_kernel(float* __restrict
     const int r = (int)(t / n), c = (int)(t % n);
     const float* s = in + (long)blockIdx.y * n;
     out[(long)blockIdx.y * n * n + t] = r == c ? s[r] * (1 - s[r]) : -s[r] * s[c];
+}
+
+// SoftmaxNode::backward (src/Nodes.cu:538-548) without the n x n Jacobian in memory: output i is
+//   sum_j fp16(J[i][j]) * fp16(dy[j]),  J[i][j] = s_i (1 - s_i) if i == j else -s_i s_j,
+// the Jacobian entry computed in fp32 exactly as softmax_jacobian_kernel does, rounded to fp16 like an
+// operand of the GEMM, multiplied with the rounded gradient (exact in fp32) and added in ascending j.
+// The Jacobian is symmetric, so J x dy (column vectors) and dy x J (row vectors) are the same sums.
+// One thread per output i; s and the rounded gradient pass through LDS in chunks of SB_CHUNK entries.
+constexpr int SB_CHUNK = 1024;
+
+// fp16(fp32(s_i * t)): two roundings, like a Jacobian stored in fp32 and then rounded as a GEMM operand.
+// The empty asm keeps the compiler from folding the product and the conversion into one mixed-precision
+// FMA, which rounds the exact product once and differs in the last fp16 bit now and then.
+__device__ __forceinline__ float jacobian_entry_f16(float si, float t) {
+    float p = si * t;
+    asm volatile("" : "+v"(p));
+    return (float)(_Float16)p;
+}
+
+__global__ __launch_bounds__(256) void softmax_backward_kernel(float* __restrict__ dx, const float* __restrict__ s,
+                                                               const float* __restrict__ dy, int n) {
+    __shared__ __attribute__((aligned(16))) float tj[SB_CHUNK];        // -s_j
+    __shared__ __attribute__((aligned(16))) _Float16 gj[SB_CHUNK];     // fp16(dy_j)
+    const float* sv = s + (long)blockIdx.y * n;
+    const float* gv = dy + (long)blockIdx.y * n;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const float si = i < n ? sv[i] : 0.f;
+    const float diag = 1 - si;
+    float acc = 0.f;
+    for (int j0 = 0; j0 < n; j0 += SB_CHUNK) {
+        const int cnt = min(SB_CHUNK, n - j0);
+        __syncthreads();
+        for (int q = threadIdx.x; q < cnt; q += 256) {
+            tj[q] = -sv[j0 + q];
+            gj[q] = (_Float16)gv[j0 + q];
+        }
+        __syncthreads();
+        // the chunk holding this workgroup's own outputs (256 | SB_CHUNK) needs the diagonal term
+        const bool own = (blockIdx.x * 256) / SB_CHUNK == j0 / SB_CHUNK;
+        const int jd = own ? i - j0 : -1;
+        int q = 0;
+        for (; q + 8 <= cnt; q += 8) {
+            const floatx4 ta = *reinterpret_cast<const floatx4*>(&tj[q]);
+            const floatx4 tb = *reinterpret_cast<const floatx4*>(&tj[q + 4]);
+            const halfx8 g8 = *reinterpret_cast<const halfx8*>(&gj[q]);
+            if (own) {      // uniform over the workgroup
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float t = q + e == jd ? diag : (e < 4 ? ta[e] : tb[e - 4]);
+                    acc = __builtin_fmaf(jacobian_entry_f16(si, t), (float)g8[e], acc);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    acc = __builtin_fmaf(jacobian_entry_f16(si, e < 4 ? ta[e] : tb[e - 4]), (float)g8[e], acc);
+            }
+        }
+        for (; q < cnt; q++) acc = __builtin_fmaf(jacobian_entry_f16(si, q == jd ? diag : tj[q]), (float)gj[q], acc);
+    }
+    if (i < n) dx[(long)blockIdx.y * n + i] = acc;
 }
 
 }  // namespace nzhip
@@ -222,7 +331,12 @@ int nzhip_matmul_f32(const float* A, const float* B, float* C, const size_t sA[4
 int nzhip_sgd_step(float* data, const float* grad, float lr, size_t n, void* stream) {
     if ((!data || !grad) && n) return set_error(NZHIP_E_INVALID, "nzhip_sgd_step: null pointer");
     if (n == 0) return NZHIP_OK;
-    hipLaunchKernelGGL(sgd_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), data, grad, lr, (long)n);
+    if (aligned16(data) && aligned16(grad) && n >= 4)
+        hipLaunchKernelGGL(sgd_kernel<4>, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, as_stream(stream), data, grad,
+                           lr, (long)n);
+    else
+        hipLaunchKernelGGL(sgd_kernel<1>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), data, grad, lr,
+                           (long)n);
     return check_launch("sgd_kernel");
 }
 
@@ -231,9 +345,16 @@ int nzhip_adam_step(float* data, float* m, float* v, const float* grad, float lr
     if ((!data || !m || !v || !grad) && n) return set_error(NZHIP_E_INVALID, "nzhip_adam_step: null pointer");
     if (t < 1) return set_error(NZHIP_E_INVALID, "nzhip_adam_step: the step count starts at 1");
     if (n == 0) return NZHIP_OK;
-    const float corr1 = 1.0f - powf(beta1, (float)t), corr2 = 1.0f - powf(beta2, (float)t);
-    hipLaunchKernelGGL(adam_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), data, m, v, grad, lr,
-                       beta1, beta2, eps, corr1, corr2, (long)n);
+    AdamArgs a;
+    a.lr = lr; a.beta1 = beta1; a.beta2 = beta2; a.eps = eps;
+    a.corr1 = 1.0f - powf(beta1, (float)t);
+    a.corr2 = 1.0f - powf(beta2, (float)t);
+    if (aligned16(data) && aligned16(m) && aligned16(v) && aligned16(grad) && n >= 4)
+        hipLaunchKernelGGL(adam_kernel<4>, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, as_stream(stream), data, m, v,
+                           grad, a, (long)n);
+    else
+        hipLaunchKernelGGL(adam_kernel<1>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), data, m, v,
+                           grad, a, (long)n);
     return check_launch("adam_kernel");
 }
 
@@ -252,6 +373,15 @@ int nzhip_softmax_jacobian(float* out, const float* in, size_t n, size_t batch, 
     dim3 grid((unsigned)((n * n + 255) / 256), (unsigned)batch);
     hipLaunchKernelGGL(softmax_jacobian_kernel, grid, dim3(256), 0, as_stream(stream), out, in, (int)n);
     return check_launch("softmax_jacobian_kernel");
+}
+
+int nzhip_softmax_backward(float* dx, const float* s, const float* dy, size_t n, size_t batch, void* stream) {
+    if ((!dx || !s || !dy) && n * batch) return set_error(NZHIP_E_INVALID, "nzhip_softmax_backward: null pointer");
+    if (n == 0 || batch == 0) return NZHIP_OK;
+    if (n > 0x3fffffff || batch > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_softmax_backward: extent too large");
+    dim3 grid((unsigned)((n + 255) / 256), (unsigned)batch);
+    hipLaunchKernelGGL(softmax_backward_kernel, grid, dim3(256), 0, as_stream(stream), dx, s, dy, (int)n);
+    return check_launch("softmax_backward_kernel");
 }
 
 }  // extern "C"

@@ -122,14 +122,11 @@ namespace nz::nodes {
 
         void SoftmaxNode::backward() {                                 // src/Nodes.cu:538-548
             if (!inputs[0]->output->requiresGrad()) return;
-            auto jacobian = softmaxJacobian(*output);
-            if (output->shape()[2] > output->shape()[3]) {
-                iTensorCoreGEMM(jacobian.data(), output->grad(), inputs[0]->output->grad(), jacobian.shape(),
-                                output->shape(), inputs[0]->output->shape());
-            } else {
-                iTensorCoreGEMM(output->grad(), jacobian.data(), inputs[0]->output->grad(), output->shape(),
-                                jacobian.shape(), inputs[0]->output->shape());
-            }
+            // Jacobian x gradient (J x dY for column vectors, dY x J for rows: the Jacobian is symmetric, so
+            // both are the same sums) with fp16-rounded operands like the GEMM the reference calls, fused so
+            // that the n x n Jacobian never reaches memory
+            const auto& s = output->shape();
+            iSoftmaxBackward(inputs[0]->output->grad(), output->data(), output->grad(), s[2] * s[3], s[0] * s[1]);
         }
 
         ReshapeNode::ReshapeNode(Node* input, const Tensor::shape_type& newShape) : newShape(newShape) {

@@ -121,6 +121,10 @@ namespace nz::data {
         NZ_CHECK(nzhip_softmax_jacobian(out, in, n, batch, nzhip_default_stream()));
     }
 
+    void iSoftmaxBackward(float* dx, float* s, float* dy, const size_t n, const size_t batch) {
+        NZ_CHECK(nzhip_softmax_backward(dx, s, dy, n, batch, nzhip_default_stream()));
+    }
+
     void iConv2dForward(float* y, float* x, float* w, float* bias, const size_t N, const size_t C, const size_t H,
                         const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
                         const size_t pad, const size_t weightBatch, const long long biasPixelStride,

@@ -90,6 +90,59 @@ def test_softmax_forward_jacobian_backward(nz, oracle):
         J = host(nz.softmax_jacobian(dev(so)))
         assert np.array_equal(J, oracle.softmax_jacobian(so)), shape
         dy = rng.uniform(-10, 10, shape).astype(np.float32)
-        got = host(nz.softmax_backward(dev(so), dev(dy)))
         want = oracle.softmax_backward(so, dy)
+        got = host(nz.softmax_backward_gemm(dev(so), dev(dy)))      # Jacobian in memory, then the GEMM entry
         assert got.shape == want.shape and np.allclose(got, want, rtol=1e-5, atol=1e-6), shape
+        # the fused kernel adds in ascending j like the oracle's GEMM: the same bits
+        fused = host(nz.softmax_backward(dev(so), dev(dy)))
+        assert fused.shape == want.shape and np.array_equal(fused, want), shape
+
+
+def test_softmax_backward_fused_sizes(nz, oracle):
+    """Chunk boundaries of the fused kernel (1024 entries per LDS chunk, 256 outputs per workgroup), fp16
+    subnormal Jacobian entries (s_i s_j far below 6e-5) and the closed form dx = s * (dy - <s, dy>)."""
+    rng = np.random.default_rng(48)
+    for shape in [(1, 1, 255, 1), (2, 1, 1, 256), (1, 2, 1024, 1), (1, 1, 1, 1025), (2, 2, 2303, 1), (1, 1, 4097, 1)]:
+        x = rng.uniform(-4, 4, shape).astype(np.float32)
+        so = oracle.softmax(x)
+        dy = rng.uniform(-3, 3, shape).astype(np.float32)
+        want = oracle.softmax_backward(so, dy)
+        got = host(nz.softmax_backward(dev(so), dev(dy)))
+        assert np.array_equal(got, want), shape
+        s64, g64 = so.astype(np.float64), dy.astype(np.float64)
+        axis = 2 if shape[2] > 1 else 3
+        closed = s64 * (g64 - (s64 * g64).sum(axis=axis, keepdims=True))
+        assert np.abs(got - closed).max() <= 2e-3 * np.abs(closed).max(), shape   # fp16 operands
+    # a gradient beyond fp16 range rounds to infinity in the GEMM operands, and so it does here
+    so = oracle.softmax(np.zeros((1, 1, 8, 1), np.float32))
+    dy = np.full((1, 1, 8, 1), 1e5, np.float32)
+    got = host(nz.softmax_backward(dev(so), dev(dy)))
+    want = oracle.softmax_backward(so, dy)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+
+
+def test_optimizer_steps_vector_and_tail_paths(nz, oracle):
+    """Four elements per thread on 16-byte aligned arrays plus the n % 4 tail, and one element per thread on a
+    view that is only 4-byte aligned: the same bits per element, and the oracle's values at the tolerance of
+    the tests above."""
+    rng = np.random.default_rng(49)
+    for n in (1, 3, 4, 1023, 1024, 1027, 262147):
+        base = [rng.standard_normal(n + 1).astype(np.float32) for _ in range(2)]
+        base.append((0.1 * rng.standard_normal(n + 1)).astype(np.float32))
+        base.append(np.abs(0.1 * rng.standard_normal(n + 1)).astype(np.float32))
+        vals = [np.ascontiguousarray(a[1:]) for a in base]            # data, grad, m, v
+        results = []
+        for unaligned in (False, True):
+            d, g, m, v = (dev(a)[1:] for a in base) if unaligned else (dev(a) for a in vals)
+            assert (d.data_ptr() % 16 != 0) == unaligned
+            d_sgd = d.clone() if not unaligned else dev(base[0])[1:]
+            nz.sgd_step(d_sgd, g, 0.05)
+            nz.adam_step(d, m, v, g, 0.01, 0.9, 0.999, 1e-6, 3)
+            results.append([host(t) for t in (d_sgd, d, m, v)])
+        for a, b in zip(*results):
+            assert np.array_equal(a, b), n
+        sgd, d, m, v = results[0]
+        assert np.max(np.abs(sgd - oracle.sgd_step(vals[0], vals[1], 0.05))) <= np.spacing(np.float32(8.0)), n
+        do, mo, vo = oracle.adam_step(vals[0], vals[2], vals[3], vals[1], 0.01, 0.9, 0.999, 1e-6, 3)
+        assert np.allclose(d, do, rtol=1e-5, atol=1e-6), n
+        assert np.allclose(m, mo, rtol=1e-6, atol=1e-7) and np.allclose(v, vo, rtol=1e-6, atol=1e-7), n
