@@ -441,6 +441,7 @@ struct IgemmArgs {
     int w_batched;
     long bias_sp, bias_sc, bias_sn;   // bias element of (image b, pixel, channel o): bias[b*bias_sn + pixel*bias_sp + o*bias_sc]
     int relu;
+    int patch_map;                    // resident kernel: 0 strided by the grid, 1 XCD-contiguous, 2 XCD-contiguous runs
 };
 
 template <int KH, int KW, int TW, int BN, bool VEC4>
@@ -710,8 +711,28 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
         return lds_h + (hh * G::WW + ww) * 32 + (((t_q4 >> 1) ^ ((ww >> 3) & 1)) << 4) + (t_q4 & 1) * 8;
     };
 
-    // work items of this workgroup: (patch, chunk) pairs, patches strided by the grid
-    const int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    // Patches of this workgroup: first_patch + pi * patch_stride, pi < my_patches. Workgroups go to the
+    // eight XCDs round-robin by their linear index and every XCD has an L2 of its own, so (when the grid
+    // is a multiple of 8 wide) the workgroups of one XCD share a contiguous eighth of the patches: halo
+    // rows and columns that neighbouring patches have in common are then found in that L2 instead of
+    // being fetched again from memory.
+    int first_patch = blockIdx.x, patch_stride = gridDim.x;
+    int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    if (p.patch_map != 0 && gridDim.x % 8 == 0) {
+        const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3, nq = gridDim.x >> 3;
+        const int lo = (int)((long)n_patches * xcd / 8), hi = (int)((long)n_patches * (xcd + 1) / 8);
+        if (p.patch_map == 1) {                                  // the XCD's workgroups sweep its range side by side
+            first_patch = lo + q;
+            patch_stride = nq;
+            my_patches = q < hi - lo ? (hi - lo - q + nq - 1) / nq : 0;
+        } else {                                                 // every workgroup walks a run of its own
+            const int a = lo + (int)((long)(hi - lo) * q / nq), b = lo + (int)((long)(hi - lo) * (q + 1) / nq);
+            first_patch = a;
+            patch_stride = 1;
+            my_patches = b - a;
+        }
+    }
+    // work items of this workgroup: (patch, chunk) pairs
     // Items per patch are rounded up to an even count: an odd chunk count gets one empty item
     // (zero halo, no MFMAs) so that every patch starts on the same register set.
     const int n_items = (p.n_chunks + 1) & ~1;
@@ -725,7 +746,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     floatx4 raw[2][4];
     int nv[2] = {0, 0};
     const int t_comp = (t_ww - p.pad) & 3;
-    int ld_patch = blockIdx.x, ld_chunk = 0, ld_it = 0;
+    int ld_patch = first_patch, ld_chunk = 0, ld_it = 0;
     const float* ld_src = p.x;                                   // this thread's pixel, channel t_q4*4, current patch
     bool ld_ok = false;                                          // the pixel (VEC4: its quad) is inside the image
     int ld_hin = 0, ld_win = 0;
@@ -738,7 +759,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     auto load_begin = [&](int& nvalid) {
         if (ld_chunk == 0) {                                     // new patch: redo the geometry (uniform branch)
             const bool live = ld_it < total;
-            const int patch = live ? ld_patch : (int)blockIdx.x;
+            const int patch = live ? ld_patch : 0;
             const int b = patch / patches_per_image, r = patch % patches_per_image;
             const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
             ld_hin = th0 + t_hh - p.pad;
@@ -773,7 +794,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     };
     auto load_end = [&]() {
         ld_it++;
-        if (++ld_chunk == n_items) { ld_chunk = 0; ld_patch += gridDim.x; }
+        if (++ld_chunk == n_items) { ld_chunk = 0; ld_patch += patch_stride; }
     };
     auto load_item = [&](floatx4 (&dst)[4], int& nvalid) {
         load_begin(nvalid);
@@ -951,7 +972,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
             item(raw[0], nv[0], c);
             item(raw[1], nv[1], c + 1);
         }
-        const int patch = blockIdx.x + pi * gridDim.x;
+        const int patch = first_patch + pi * patch_stride;
 #pragma unroll
         for (int j = 0; j < FP; j++)
 #pragma unroll
@@ -993,6 +1014,8 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             a.tiles_w = (int)((W_out + TW - 1) / TW);
             a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
             a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
+            static const char* map_env = getenv("NZHIP_CONV_PATCH_MAP");
+            a.patch_map = map_env ? atoi(map_env) : 1;
             const long n_patches = (long)N * a.tiles_w * a.tiles_h;
             int rc = NZHIP_OK;
             if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
@@ -1053,6 +1076,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         a.bias_sc = bias_sc;
         a.bias_sn = bias_sn;
         a.relu = act == NZHIP_ACT_RELU;
+        a.patch_map = 0;
         const bool vec4 = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
         auto kfn = vec4 ? conv_igemm_kernel<KH, KW, TW, BN, true> : conv_igemm_kernel<KH, KW, TW, BN, false>;
         if (rc == NZHIP_OK)
