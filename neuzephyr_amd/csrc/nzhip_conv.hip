@@ -2,6 +2,8 @@
 // Img2Col -> MatMul -> Bias -> Col2Img [-> ReLU]) as one call.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <cstdlib>
 
 #include "nzhip_internal.h"
@@ -32,6 +34,22 @@ constexpr int DC_ROWS = 4;         // output rows per wave
 constexpr int DC_MAX_C = 8;        // input channels held in the rolling window
 constexpr int DC_MAX_O = 4;
 
+// Workgroups are dealt to the eight XCDs round-robin by their linear index, and every XCD has an L2 of
+// its own. This renumbers them so that each XCD works on one contiguous run of the (x, y, z) grid in
+// x-fastest order: neighbouring tiles, which share halo rows and the memory lines of their edge
+// columns, then meet in one L2 instead of fetching those lines twice.
+__device__ __forceinline__ void xcd_contiguous_block(int& bx, int& by, int& bz) {
+    const long gx = gridDim.x, gy = gridDim.y;
+    const long total = gx * gy * gridDim.z;
+    const long lin = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+    const long xcd = lin & 7, q = lin >> 3;
+    const long rem = total & 7;
+    const long unit = xcd * (total >> 3) + (xcd < rem ? xcd : rem) + q;
+    bx = (int)(unit % gx);
+    by = (int)((unit / gx) % gy);
+    bz = (int)(unit / (gx * gy));
+}
+
 // O_T: output channels per thread; C_T: compile-time input-channel count (0 = runtime loop);
 // VEC: W % 4 == 0 and 16-byte aligned tensors, so every lane's 4 pixels are inside the row and
 // move as one 16-byte access.
@@ -43,14 +61,15 @@ __global__ __launch_bounds__(256) void conv3x3_direct_kernel(float* __restrict__
                                                              int relu) {
     __shared__ _Float16 wsm[DC_MAX_C * 9 * DC_MAX_O];
     const int C = C_T ? C_T : C_rt;
-    const int b = blockIdx.z;
+    int bx, by, b;
+    xcd_contiguous_block(bx, by, b);
     const float* wb = w_ref + (long)b * w_batch_stride;
     for (int i = threadIdx.x; i < C * 9 * O; i += 256) wsm[i] = (_Float16)wb[i];     // [q][o], RNE
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int w0 = (blockIdx.x * 64 + lane) * 4;
-    const int h0 = (blockIdx.y * 4 + wave) * DC_ROWS;
+    const int w0 = (bx * 64 + lane) * 4;
+    const int h0 = (by * 4 + wave) * DC_ROWS;
     if (w0 >= W || h0 >= H) return;
     const float* xb = x + (long)b * C * H * W;
     float* yb = y + (long)b * O * H * W;
@@ -193,14 +212,15 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
                                                              long w_batch_stride, long bias_sp, long bias_sc,
                                                              int relu) {
     __shared__ float wsm[C_T * 9 * O_T];
-    const int b = blockIdx.z;
+    int bx, by, b;
+    xcd_contiguous_block(bx, by, b);
     const float* wb = w_ref + (long)b * w_batch_stride;
     for (int i = threadIdx.x; i < C_T * 9 * O_T; i += 256) wsm[i] = round_f16(wb[i]);   // [q][o]
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int w0 = (blockIdx.x * 64 + lane) * 4;
-    const int h0 = (blockIdx.y * 4 + wave) * ST_ROWS;
+    const int w0 = (bx * 64 + lane) * 4;
+    const int h0 = (by * 4 + wave) * ST_ROWS;
     if (w0 >= W || h0 >= H) return;
     const float* xb = x + (long)b * C_T * H * W;
     float* yb = y + (long)b * O_T * H * W;
@@ -210,7 +230,16 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
     const int wx = lane == 0 ? (has_l ? w0 - 1 : w0) : (lane == 63 && has_r ? w0 + 4 : w0);
     const int rows = (H - h0) < ST_ROWS ? (H - h0) : ST_ROWS;   // output rows of this strip
     const int T = rows + 2;                                      // input rows h0-1 .. h0+rows
-
+    // Odd strips walk upwards. A strip shares its first and its last input rows with its neighbours;
+    // with alternating directions both neighbours touch a shared row at the same moment (both at the
+    // start, or both at the end of their walk), so the second request finds it in L2. Walking all
+    // strips downwards puts a whole strip's duration between the two uses and the row comes from
+    // memory twice. The walk is instantiated once per direction and a wave runs one of the two.
+    const bool rev = ((by * 4 + wave) & 1) != 0;
+    auto walk = [&](auto upwards) {
+    constexpr bool UP = decltype(upwards)::value;
+    const int row_first = UP ? h0 + rows : h0 - 1, row_step = UP ? -1 : 1;
+    auto out_row = [&](int t) { return UP ? h0 + rows + 1 - t : h0 + t - 2; };   // completed by step t >= 2
     float raw[ST_AHEAD][C_T][5];                                 // rows in flight (t % ST_AHEAD): own quad + extra word
     float braw[ST_AHEAD][O_T][4];                                // per-pixel bias of the output row each completes
     float win[3][C_T][6];                                        // rounded rows t-2, t-1, t (t % 3)
@@ -220,13 +249,13 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
 
     // Requests are unconditional (rows beyond the image read row 0); what must be zero is masked
     // when the row is consumed, so nothing waits at request time.
-    auto row_in_image = [&](int t) { const int hi = h0 - 1 + t; return t < T && hi >= 0 && hi < H; };
+    auto row_in_image = [&](int t) { const int hi = row_first + t * row_step; return t < T && hi >= 0 && hi < H; };
     auto request = [&](int t, float (&dst)[C_T][5], float (&bdst)[O_T][4]) {
-        const float* row = xb + (long)(row_in_image(t) ? h0 - 1 + t : 0) * W;
+        const float* row = xb + (long)(row_in_image(t) ? row_first + t * row_step : 0) * W;
         if (PIX_BIAS) {
-            // the bias of output row h0 + t - 2 travels with the input row that completes it, so its
+            // the bias of the output row a step completes travels with that step's input row, so its
             // wait never drains the rows requested after it
-            const int hb = (t >= 2 && t < T) ? h0 + t - 2 : h0;
+            const int hb = (t >= 2 && t < T) ? out_row(t) : h0;
 #pragma unroll
             for (int o = 0; o < O_T; o++)
 #pragma unroll
@@ -282,17 +311,19 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
                 }
             request(t + ST_AHEAD, raw[u], braw[u]);              // slot u is free again
             if (t < 2) continue;
-            const int ho = h0 + t - 2;                           // output row fed by input rows t-2, t-1, t
+            const int ho = out_row(t);                           // output row fed by the rows of steps t-2, t-1, t
             float acc[O_T][4];
 #pragma unroll
             for (int o = 0; o < O_T; o++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) acc[o][e] = 0.f;
+            // Filter row r meets the input row of step t-2+r (walking down) or t-r (walking up), which
+            // lives in slot (step % 3); the sum runs over c, r, s in ascending order either way.
 #pragma unroll
             for (int c = 0; c < C_T; c++)
 #pragma unroll
                 for (int r = 0; r < 3; r++) {
-                    const int slot = (wu + 1 + r) % 3;           // row t-2+r lives in slot (t-2+r) % 3
+                    const int slot = UP ? (wu + 3 - r) % 3 : (wu + 1 + r) % 3;
 #pragma unroll
                     for (int s2 = 0; s2 < 3; s2++)
 #pragma unroll
@@ -315,6 +346,9 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
             }
         }
     }
+    };
+    if (rev) walk(std::true_type{});
+    else walk(std::false_type{});
 }
 
 static bool conv_direct_applicable(size_t C, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad) {
@@ -458,8 +492,9 @@ __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(con
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int li = lane & 31, lh = lane >> 5;
-    const int tile_w = blockIdx.x % p.tiles_w, tile_h = blockIdx.x / p.tiles_w;
-    const int o_tile = blockIdx.y, b = blockIdx.z;
+    int tile, o_tile, b;
+    xcd_contiguous_block(tile, o_tile, b);
+    const int tile_w = tile % p.tiles_w, tile_h = tile / p.tiles_w;
     const int th0 = tile_h * G::TH, tw0 = tile_w * TW;
 
     const float* xb = p.x + (long)b * p.C * p.H * p.W;
