@@ -1455,12 +1455,24 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
                            activation, s);
     static const char* route_env = getenv("NZHIP_CONV_ROUTE");      // "workspace": column matrix + GEMM (benchmarking only)
     const bool force_ws = route_env && route_env[0] == 'w' && bias_stride_image == 0;
-    if (!force_ws && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL) {
-        // NZHIP_CONV_TW=32|64 and NZHIP_CONV_BN=64|128 override the tile choice (benchmarking only)
-        static const char* tw_env = getenv("NZHIP_CONV_TW");
-        static const char* bn_env = getenv("NZHIP_CONV_BN");
-        const bool wide = tw_env ? atoi(tw_env) == 64 : W_out >= 64;
-        const bool bn128 = bn_env ? atoi(bn_env) == 128 : O > 64;
+    // NZHIP_CONV_TW=32|64 and NZHIP_CONV_BN=64|128 override the tile choice (benchmarking only)
+    static const char* tw_env = getenv("NZHIP_CONV_TW");
+    static const char* bn_env = getenv("NZHIP_CONV_BN");
+    const bool wide = tw_env ? atoi(tw_env) == 64 : W_out >= 64;
+    const bool bn128 = bn_env ? atoi(bn_env) == 128 : O > 64;
+    // Small images with many channels: the weights do not fit LDS, so the implicit-GEMM kernel runs one
+    // patch per workgroup with the whole C x taps contraction inside, and there are too few patches to
+    // fill the CUs (8 x 512 x 16 x 16 -> 512: 64 workgroups, 190 us). The column matrix of such a layer is
+    // small; its batched GEMM splits the contraction over the idle CUs instead (83 us).
+    bool few_patches = false;
+    if (bias_stride_image == 0) {
+        const size_t tw = wide ? 64 : 32, th = 256 / tw, bn = bn128 ? 128 : 64;
+        const size_t units = N * ((W_out + tw - 1) / tw) * ((H_out + th - 1) / th) * ((O + bn - 1) / bn);
+        const size_t w_lds = ((C + IG_CC - 1) / IG_CC) * bn * K_h * K_w * 32;       // fp16 weight image of one channel tile
+        const bool resident = w_batch == 1 && w_lds <= 148 * 1024;
+        few_patches = !resident && units * 4 <= (size_t)device_cu_count();
+    }
+    if (!force_ws && !few_patches && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL) {
 #define NZHIP_IG(KH_, TW_, BN_)                                                                                      \
     return conv_igemm_launch<KH_, KH_, TW_, BN_>(y, x, w_ref, bias, N, C, H, W, O, pad, w_batch, bias_stride_pixel, \
                                                  bias_stride_channel, bias_stride_image, activation, H_out, W_out, s)

@@ -67,41 +67,49 @@ __global__ __launch_bounds__(256) void im2col_vec4_kernel(float* __restrict__ ou
     *reinterpret_cast<floatx4*>(out + (long)b * per + idx) = v;
 }
 
-// Stride 1: a workgroup takes 64 adjacent output pixels of one row and 32 channels, reads the K_h
-// input rows they touch once (coalesced along w) into LDS and writes, per pixel, its contiguous run of
-// 32*K_h*K_w column entries with 16-byte stores (for 3x3 that is 1152 bytes: whole 128-byte lines). The scattered 4-byte global reads of the kernels
-// above (a wave touches 64 channel planes per instruction) are what bounds them.
+// Stride 1: a workgroup takes 64 adjacent output pixels of one row (or, for images narrower than 64
+// pixels, the whole rows that make up at most 64 pixels) and 32 channels, reads the input rows they
+// touch once (coalesced along w) into LDS and writes, per pixel, its contiguous run of 32*K_h*K_w column
+// entries with 16-byte stores (for 3x3 that is 1152 bytes: whole 128-byte lines). The scattered 4-byte
+// global reads of the kernels above (a wave touches 64 channel planes per instruction) are what bounds
+// them.
 constexpr int I2C_PX = 64, I2C_CH = 32, I2C_MAXK = 5, I2C_ROW = I2C_PX + I2C_MAXK;   // floats per staged row
+constexpr int I2C_LDS = I2C_CH * I2C_MAXK * I2C_ROW;                                  // floats of staging space
 // KH, KW > 0: kernel extents known at compile time (the index divisions become multiplications).
+// rpw: output rows per workgroup (1 when a row has several 64-pixel segments).
 template <int KH, int KW>
 __global__ __launch_bounds__(256) void im2col_rows_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                           int H_out, int W_out, int C, int K_h_rt, int K_w_rt, int pad,
-                                                          int H_in, int W_in, int segs) {
-    __shared__ float rows[I2C_CH * I2C_MAXK * I2C_ROW];
+                                                          int H_in, int W_in, int segs, int rpw) {
+    __shared__ float rows[I2C_LDS];
     const int K_h = KH > 0 ? KH : K_h_rt, K_w = KW > 0 ? KW : K_w_rt;
     const int KK = K_h * K_w, CKK = C * KK;
-    const int seg = blockIdx.x % segs, ho = blockIdx.x / segs;
+    const int seg = blockIdx.x % segs, ho0 = (blockIdx.x / segs) * rpw;
     const int c0 = blockIdx.y * I2C_CH, b = blockIdx.z;
     const int nch = (C - c0) < I2C_CH ? (C - c0) : I2C_CH;
     const int wo0 = seg * I2C_PX;
-    const int span = I2C_PX + K_w - 1;                           // input columns wo0 - pad .. wo0 - pad + span - 1
+    const int wpx = (W_out - wo0) < I2C_PX ? (W_out - wo0) : I2C_PX;      // output pixels per row of this workgroup
+    const int nrow = (H_out - ho0) < rpw ? (H_out - ho0) : rpw;           // output rows of this workgroup
+    const int span = wpx + K_w - 1;                              // input columns wo0 - pad .. wo0 - pad + span - 1
+    const int rt = nrow + K_h - 1;                               // input rows ho0 - pad .. ho0 - pad + rt - 1
     const float* img = in + ((long)b * C + c0) * H_in * W_in;
-    for (int e = threadIdx.x; e < nch * K_h * span; e += 256) {
-        const int col = e % span, r = (e / span) % K_h, c = e / (span * K_h);
-        const int h = ho - pad + r, w = wo0 - pad + col;
-        rows[(c * K_h + r) * I2C_ROW + col] = (h >= 0 && h < H_in && w >= 0 && w < W_in) ? img[((long)c * H_in + h) * W_in + w] : 0.f;
+    for (int e = threadIdx.x; e < nch * rt * span; e += 256) {
+        const int col = e % span, r = (e / span) % rt, c = e / (span * rt);
+        const int h = ho0 - pad + r, w = wo0 - pad + col;
+        rows[(c * rt + r) * span + col] = (h >= 0 && h < H_in && w >= 0 && w < W_in) ? img[((long)c * H_in + h) * W_in + w] : 0.f;
     }
     __syncthreads();
     const int run4 = nch * KK / 4;                               // 16-byte pieces per pixel (nch*KK is a multiple of 4)
-    const int npx = (W_out - wo0) < I2C_PX ? (W_out - wo0) : I2C_PX;
-    float* dst = out + ((long)b * H_out * W_out + (long)ho * W_out + wo0) * CKK + (long)c0 * KK;
+    const int npx = nrow * wpx;                                  // rpw > 1 only with whole rows: pixels stay contiguous
+    float* dst = out + ((long)b * H_out * W_out + (long)ho0 * W_out + wo0) * CKK + (long)c0 * KK;
     for (int e = threadIdx.x; e < npx * run4; e += 256) {
         const int px = e / run4, q4 = e % run4;
+        const int pr = px / wpx, pw = px % wpx;
         int c = (q4 * 4) / KK, rs = (q4 * 4) % KK;
         floatx4 v;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            v[j] = rows[(c * K_h + rs / K_w) * I2C_ROW + px + rs % K_w];
+            v[j] = rows[(c * rt + pr + rs / K_w) * span + pw + rs % K_w];
             if (++rs == KK) {
                 rs = 0;
                 c++;
@@ -282,9 +290,12 @@ __global__ __launch_bounds__(256) void fill_bias_act_kernel(nzhip_gemm_desc d) {
 // C = act(bias + sum over chunks s of P[s]). Eight threads share an output: thread q adds the
 // chunks of its contiguous eighth in ascending order, then the eight partial sums are added in
 // ascending q, so the result depends on the number of chunks only, never on scheduling.
+// blockIdx.y is the batch member (n); its chunks are P[n][s][M][N].
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(nzhip_gemm_desc d, const float* __restrict__ P, int S) {
     __shared__ float part[8][32];
     const long mn = d.M * d.N;
+    const long bn = blockIdx.y;
+    P += bn * S * mn;
     const int q = threadIdx.x >> 5, tl = threadIdx.x & 31;          // a wave reads two chunk rows of 32 outputs
     const long t = (long)blockIdx.x * 32 + tl;
     const int per = (S + 7) / 8, s0 = q * per, s1 = s0 + per < S ? s0 + per : S;
@@ -297,9 +308,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(nzhip_gemm_desc d, c
 #pragma unroll
     for (int k = 1; k < 8; k++) x += part[k][tl];
     const long m = t / d.N, n = t % d.N;
-    if (d.bias) x += d.bias[m * d.bias_stride_row + n * d.bias_stride_col];
+    if (d.bias) x += d.bias[bn * d.bias_stride_n + m * d.bias_stride_row + n * d.bias_stride_col];
     if (d.activation == NZHIP_ACT_RELU) x = x > 0.f ? x : 0.f;
-    d.C[m * d.ldc + n] = x;
+    d.C[bn * d.c_stride_n + m * d.ldc + n] = x;
 }
 
 // The same sum for few chunks and many outputs: one thread per output adds its chunks in ascending
@@ -308,12 +319,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_wide_kernel(nzhip_gemm_desc
     const long mn = d.M * d.N;
     const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= mn) return;
+    const long bn = blockIdx.y;
+    P += bn * S * mn;
     float x = 0.f;
     for (int s = 0; s < S; s++) x += P[(long)s * mn + t];
     const long m = t / d.N, n = t % d.N;
-    if (d.bias) x += d.bias[m * d.bias_stride_row + n * d.bias_stride_col];
+    if (d.bias) x += d.bias[bn * d.bias_stride_n + m * d.bias_stride_row + n * d.bias_stride_col];
     if (d.activation == NZHIP_ACT_RELU) x = x > 0.f ? x : 0.f;
-    d.C[m * d.ldc + n] = x;
+    d.C[bn * d.c_stride_n + m * d.ldc + n] = x;
 }
 
 }  // namespace nzhip
@@ -340,9 +353,11 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
     // order. The extra pass over the partial sums costs 5..15 us, so a chunk keeps at least 512 of
     // the contraction when loads are vectorised (1024^3: 23 us unsplit, 31 us in two chunks;
     // 1024x4096x1024: 71 us unsplit, 39 us in eight chunks) and 128 otherwise.
-    if (d.batch_n * d.batch_c == 1 && d.K >= 512) {
+    // A batch over n alone (batch_c == 1: shared-weight layers, the conv column-matrix route) splits the
+    // same way; its chunks take the c dimension of the launch.
+    if (d.batch_c == 1 && d.batch_n <= 65535 && d.K >= 512) {
         const int cus = device_cu_count();
-        const int64_t tiles = ((d.M + 127) / 128) * ((d.N + 127) / 128);
+        const int64_t tiles = ((d.M + 127) / 128) * ((d.N + 127) / 128) * d.batch_n;
         if (tiles * 2 <= cus) {
             const bool narrow = d.M <= 64 || d.N <= 64;            // padded tiles: the k loop is shorter per byte
             const int64_t min_chunk = gemm_vec_legal(d) && !narrow ? 512 : 128;
@@ -356,10 +371,12 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
             const int parts = (int)((d.K + Kc - 1) / Kc);                    // the last one may be shorter
             if (parts >= 2) {
                 float* P = nullptr;
-                if (int rc = workspace_alloc(reinterpret_cast<void**>(&P), (size_t)parts * d.M * d.N * sizeof(float), s)) return rc;
+                if (int rc = workspace_alloc(reinterpret_cast<void**>(&P), (size_t)d.batch_n * parts * d.M * d.N * sizeof(float), s))
+                    return rc;
                 nzhip_gemm_desc g = d;
                 g.C = P; g.ldc = d.N; g.K = Kc;
-                g.batch_n = 1; g.batch_c = parts;
+                g.batch_c = parts;
+                g.c_stride_n = (int64_t)parts * d.M * d.N;
                 g.a_stride_c = d.a_layout == NZHIP_LAYOUT_ROW ? Kc : Kc * d.lda;   // next chunk of A / B
                 g.b_stride_c = d.b_layout == NZHIP_LAYOUT_ROW ? Kc * d.ldb : Kc;
                 g.c_stride_c = d.M * d.N;
@@ -368,10 +385,10 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
                 if (rc == NZHIP_OK) {
                     if (parts > 16 || d.M * d.N < (1 << 18)) {                  // few outputs: spread each over eight lanes
                         const long groups = (d.M * d.N + 31) / 32;               // 32 outputs x 8 chunk lanes per workgroup
-                        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)groups), dim3(256), 0, s, d, P, parts);
+                        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
                     } else {
                         const long groups = (d.M * d.N + 255) / 256;
-                        hipLaunchKernelGGL(splitk_reduce_wide_kernel, dim3((unsigned)groups), dim3(256), 0, s, d, P, parts);
+                        hipLaunchKernelGGL(splitk_reduce_wide_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
                     }
                     rc = check_launch("splitk_reduce_kernel");
                 }
@@ -480,14 +497,23 @@ int nzhip_im2col(float* out, const float* in, size_t H_out, size_t W_out, size_t
     if (stride == 1 && K_h <= (size_t)I2C_MAXK && K_w <= (size_t)I2C_MAXK && (C * K_h * K_w) % 4 == 0 &&
         (I2C_CH * K_h * K_w) % 4 == 0 && aligned16(out)) {
         const size_t segs = (W_out + I2C_PX - 1) / I2C_PX, chunks = (C + I2C_CH - 1) / I2C_CH;
-        if (segs * H_out <= 0x7fffffffull && chunks <= 65535) {
-            dim3 grid((unsigned)(segs * H_out), (unsigned)chunks, (unsigned)batch);
+        // narrow images: as many whole rows per workgroup as make up 64 pixels and fit the staging space
+        size_t rpw = 1;
+        if (segs == 1) {
+            rpw = I2C_PX / W_out;
+            if (rpw > H_out) rpw = H_out;
+            while (rpw > 1 && I2C_CH * (rpw + K_h - 1) * (W_out + K_w - 1) > (size_t)I2C_LDS) rpw--;
+            if (rpw < 1) rpw = 1;
+        }
+        const size_t hblocks = (H_out + rpw - 1) / rpw;
+        if (segs * hblocks <= 0x7fffffffull && chunks <= 65535) {
+            dim3 grid((unsigned)(segs * hblocks), (unsigned)chunks, (unsigned)batch);
             auto kfn = (K_h == 3 && K_w == 3)   ? im2col_rows_kernel<3, 3>
                        : (K_h == 1 && K_w == 1) ? im2col_rows_kernel<1, 1>
                        : (K_h == 5 && K_w == 5) ? im2col_rows_kernel<5, 5>
                                                 : im2col_rows_kernel<0, 0>;
             hipLaunchKernelGGL(kfn, grid, dim3(256), 0, as_stream(stream), out, in, (int)H_out, (int)W_out, (int)C, (int)K_h,
-                               (int)K_w, (int)pad, (int)H_in, (int)W_in, (int)segs);
+                               (int)K_w, (int)pad, (int)H_in, (int)W_in, (int)segs, (int)rpw);
             return check_launch("im2col_rows_kernel");
         }
     }

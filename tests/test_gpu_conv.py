@@ -41,6 +41,10 @@ IM2COL_CASES = [((2, 3, 4, 5), 3, 3, 1, 1), ((1, 1, 1, 1), 1, 1, 1, 0), ((2, 2, 
                 # 32-channel chunks with a tail, compile-time and run-time kernel extents)
                 ((2, 4, 6, 7), 3, 3, 1, 1), ((1, 64, 5, 130), 3, 3, 1, 1), ((2, 40, 9, 70), 3, 3, 1, 0),
                 ((2, 8, 7, 66), 1, 1, 1, 0), ((1, 4, 9, 75), 5, 5, 1, 2), ((2, 2, 8, 9), 2, 2, 1, 1), ((1, 36, 4, 64), 3, 3, 1, 2),
+                # narrow images: several whole output rows per workgroup (4 rows of 16, 9 of 7 with a 7-row tail image,
+                # 2 of 30 with an odd row count, one pixel per row, pad 0 so that the output is narrower than the input)
+                ((2, 40, 16, 16), 3, 3, 1, 1), ((3, 12, 7, 7), 3, 3, 1, 1), ((1, 8, 5, 30), 3, 3, 1, 1),
+                ((2, 4, 9, 1), 3, 3, 1, 1), ((2, 16, 12, 12), 5, 5, 1, 0), ((1, 68, 14, 14), 1, 1, 1, 0),
                 # other strides with a multiple of 4: the 16-byte store variant of the per-element kernel
                 ((2, 4, 9, 9), 3, 3, 2, 1), ((1, 8, 10, 12), 2, 3, 3, 0)]
 

@@ -262,6 +262,19 @@ def test_largest_batches(nz, sa, sb):
     assert np.array_equal(host(nz.tensorcore_gemm(dev(A), dev(B))), expect)
 
 
+@pytest.mark.parametrize("sa,sb", [((4, 1, 100, 1500), (1, 1, 1500, 130)),       # 4 members x 2 tiles, B shared
+                                   ((3, 1, 130, 1100), (3, 1, 1100, 70)),        # both batched over n
+                                   ((2, 1, 257, 4608), (1, 1, 4608, 250))])      # the column-matrix conv shape, small images
+def test_batched_products_with_few_tiles_split_the_contraction(nz, sa, sb):
+    """Products batched over n whose tiles leave most CUs idle run their contraction in chunks (a
+    workspace of partial sums per member, added in a fixed order): exact on integers."""
+    rng = np.random.default_rng(sa[2] + sb[3])
+    A = rng.integers(-4, 5, size=sa).astype(np.float32)
+    B = rng.integers(-4, 5, size=sb).astype(np.float32)
+    expect = np.matmul(A.astype(np.float64), B.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(host(nz.tensorcore_gemm(dev(A), dev(B))), expect)
+
+
 def test_bias_forms_and_relu_special_values(nz, oracle):
     M, K, N = 40, 24, 52
     rng = np.random.default_rng(1)
