@@ -218,6 +218,36 @@ int nzhip_softmax_jacobian(float* out, const float* in, size_t n, size_t batch, 
  * additions (the Jacobian is symmetric, so column and row vectors are the same sums). dx is overwritten. */
 int nzhip_softmax_backward(float* dx, const float* s, const float* dy, size_t n, size_t batch, void* stream);
 
+/* ---- the rest of the reference's example network (README.md:62-90): pooling, loss, target expansion ---- */
+/* nz::data::iAveragePooling (AveragePoolingKernel, src/OperationKernels.cu:1404-1429; AveragePoolingNode::forward,
+ * src/Nodes.cu:678-682): square window, out = mean over the window cells inside the image (cells in the
+ * padding do not count), summed row by row, left to right. H_out = (H_in + 2 pad - pool) / stride + 1. */
+int nzhip_avgpool2d(float* out, const float* in, size_t pool, size_t stride, size_t pad, size_t batches,
+                    size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out, void* stream);
+
+/* nz::data::iAveragePoolingBackward (AveragePoolingBackwardKernel, :1439-1486; AveragePoolingNode::backward,
+ * src/Nodes.cu:684-690): din += dout / divisor over every window that covers the element, divisor = pool^2
+ * without padding, the number of window cells inside the image with padding. The reference scatters with
+ * atomicAdd; here every input element gathers its windows in ascending (row, column) order, the order of a
+ * serial run of that scatter. */
+int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches,
+                             size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out, void* stream);
+
+/* BinaryCrossEntropyNode::forward (src/Nodes.cu:822-840; BinaryCrossEntropyKernel, src/OperationKernels.cu:648-685):
+ * *loss (device memory) = sum_i (-t_i log p_i - (1 - t_i) log(1 - p_i)) / n with the fast hardware logarithm
+ * (the reference uses __logf) and a fixed two-level summation order; the reference adds per-block partial sums
+ * on the host. Last bits are not pinned by the reference (its test compares at 1e-2). */
+int nzhip_bce_loss(float* loss, const float* predict, const float* real, size_t n, void* stream);
+
+/* BinaryCrossEntropyNode::backward (src/Nodes.cu:842-849; BCEBackwardKernel, :692-699):
+ * grad_i = ((p_i - t_i) / (p_i (1 - p_i))) / n, overwriting grad. */
+int nzhip_bce_backward(float* grad, const float* predict, const float* real, size_t n, void* stream);
+
+/* ExpandNode::forward / backward (src/Nodes.cu:585-603; ExpandKernel, CompressKernel, :1282-1301):
+ * out[b*n + j] = in[j] for b < batches; and out[j] += sum_b in[b*n + j] in ascending b. */
+int nzhip_expand(float* out, const float* in, size_t n, size_t batches, void* stream);
+int nzhip_compress(float* out, const float* in, size_t n, size_t batches, void* stream);
+
 /* ---- runtime: device allocator + stream manager -------------------------- */
 /* Replace cuStrm::StreamManager<float> (include/NeuZephyr/StreamManager.cuh:131-911) and
  * EventPool (EventPool.cuh:165-457).  One ordered compute stream carries every kernel and

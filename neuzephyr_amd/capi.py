@@ -20,6 +20,7 @@ EXPORTS = [
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
     "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
+    "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_expand", "nzhip_compress",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
@@ -89,6 +90,12 @@ def load() -> C.CDLL:
     lib.nzhip_softmax.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_softmax_jacobian.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_softmax_backward.argtypes = [vp, vp, vp, sz, sz, vp]
+    lib.nzhip_avgpool2d.argtypes = [vp, vp] + [sz] * 9 + [vp]
+    lib.nzhip_avgpool2d_backward.argtypes = [vp, vp] + [sz] * 9 + [vp]
+    lib.nzhip_bce_loss.argtypes = [vp, vp, vp, sz, vp]
+    lib.nzhip_bce_backward.argtypes = [vp, vp, vp, sz, vp]
+    lib.nzhip_expand.argtypes = [vp, vp, sz, sz, vp]
+    lib.nzhip_compress.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_adam_step.argtypes = [vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, sz, vp]
     lib.nzhip_default_stream.restype = vp
     lib.nzhip_malloc.argtypes = [C.POINTER(vp), sz]
@@ -369,3 +376,55 @@ def softmax_backward_gemm(s, dy, stream=None):
     """SoftmaxNode::backward as the reference spells it: Jacobian times gradient through the fp16 GEMM entry."""
     jac = softmax_jacobian(s, stream)
     return tensorcore_gemm(jac, dy, stream=stream) if s.shape[2] > s.shape[3] else tensorcore_gemm(dy, jac, stream=stream)
+
+
+def avgpool2d(x, pool, stride, pad, stream=None):
+    import torch
+    lib = load()
+    N, Cc, H, W = x.shape
+    ok = stride > 0 and H + 2 * pad >= pool and W + 2 * pad >= pool       # otherwise the library rejects the call
+    Ho, Wo = ((H + 2 * pad - pool) // stride + 1, (W + 2 * pad - pool) // stride + 1) if ok else (1, 1)
+    out = torch.empty((N, Cc, Ho, Wo), dtype=torch.float32, device=x.device)
+    check(lib.nzhip_avgpool2d(_dev(out), _dev(x), pool, stride, pad, N, Cc, H, W, Ho, Wo, _stream_handle(stream)))
+    return out
+
+
+def avgpool2d_backward(dx, dy, pool, stride, pad, stream=None):
+    """dx += gradient of avgpool2d; dx has the input's shape, dy the output's."""
+    lib = load()
+    N, Cc, H, W = dx.shape
+    check(lib.nzhip_avgpool2d_backward(_dev(dx), _dev(dy), pool, stride, pad, N, Cc, H, W, dy.shape[2], dy.shape[3],
+                                       _stream_handle(stream)))
+    return dx
+
+
+def bce_loss(predict, real, stream=None):
+    """Device scalar (a 1-element tensor) holding the mean binary cross-entropy."""
+    import torch
+    lib = load()
+    loss = torch.empty(1, dtype=torch.float32, device=predict.device)
+    check(lib.nzhip_bce_loss(_dev(loss), _dev(predict), _dev(real), predict.numel(), _stream_handle(stream)))
+    return loss
+
+
+def bce_backward(predict, real, stream=None):
+    import torch
+    lib = load()
+    grad = torch.empty_like(predict)
+    check(lib.nzhip_bce_backward(_dev(grad), _dev(predict), _dev(real), predict.numel(), _stream_handle(stream)))
+    return grad
+
+
+def expand(x, batches, stream=None):
+    import torch
+    lib = load()
+    out = torch.empty((batches,) + tuple(x.shape[1:]), dtype=torch.float32, device=x.device)
+    check(lib.nzhip_expand(_dev(out), _dev(x), x.numel(), batches, _stream_handle(stream)))
+    return out
+
+
+def compress(out, x, stream=None):
+    """out[0] += sum over the batch of x."""
+    lib = load()
+    check(lib.nzhip_compress(_dev(out), _dev(x), out.numel(), x.shape[0], _stream_handle(stream)))
+    return out

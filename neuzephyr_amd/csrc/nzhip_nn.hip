@@ -1,0 +1,237 @@
+// What stands between the convolution / linear layers and a loss in the reference's own example
+// network (README.md:62-90: Conv2d, ReLU, Conv2d, AvgPool2d, Linear, Softmax, BCELoss): average
+// pooling and its gradient (AveragePoolingKernel / AveragePoolingBackwardKernel,
+// src/OperationKernels.cu:1404-1486), the binary cross-entropy loss and its gradient
+// (BinaryCrossEntropyKernel / BCEBackwardKernel, :648-700) and the batch expansion of a target
+// (ExpandKernel / CompressKernel, :1282-1301). All of them are streams over memory.
+#include <hip/hip_runtime.h>
+
+#include "nzhip_internal.h"
+
+namespace nzhip {
+
+static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+static int check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, what);
+}
+
+struct PoolArgs {
+    int pool, stride, pad;
+    int H_in, W_in, H_out, W_out;
+    long planes;            // batches * channels
+};
+
+// One thread per output element: the window is summed row by row, left to right (the reference's
+// loop order), and divided by the number of window cells inside the image.
+__global__ __launch_bounds__(256) void avgpool_kernel(float* __restrict__ out, const float* __restrict__ in,
+                                                      const PoolArgs p) {
+    const long per = (long)p.H_out * p.W_out;
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= p.planes * per) return;
+    const long plane = idx / per;
+    const int h = (int)((idx % per) / p.W_out), w = (int)((idx % per) % p.W_out);
+    const int h0 = h * p.stride - p.pad, w0 = w * p.stride - p.pad;
+    const float* src = in + plane * p.H_in * p.W_in;
+    float sum = 0.f;
+    int count = 0;
+    for (int i = 0; i < p.pool; i++) {
+        const int hi = h0 + i;
+        if (hi < 0 || hi >= p.H_in) continue;
+        for (int j = 0; j < p.pool; j++) {
+            const int wi = w0 + j;
+            if (wi >= 0 && wi < p.W_in) {
+                sum += src[(long)hi * p.W_in + wi];
+                count++;
+            }
+        }
+    }
+    out[idx] = count > 0 ? sum / (float)count : 0.f;
+}
+
+// Gradient as a gather: one thread per INPUT element adds, in ascending (row, column) order of the
+// output windows that cover it, dout / divisor onto the value already there. That is the order in
+// which a serial run of the reference's scatter loop reaches this element, so the result does not
+// depend on scheduling (the reference's atomicAdd order does). The divisor is pool^2 without padding
+// and the number of window cells inside the image with padding (:1451-1480).
+__global__ __launch_bounds__(256) void avgpool_backward_kernel(float* __restrict__ din, const float* __restrict__ dout,
+                                                               const PoolArgs p) {
+    const long per = (long)p.H_in * p.W_in;
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= p.planes * per) return;
+    const long plane = idx / per;
+    const int h = (int)((idx % per) / p.W_in), w = (int)((idx % per) % p.W_in);
+    // windows with oh*stride - pad <= h <= oh*stride - pad + pool - 1
+    const int hp = h + p.pad, wp = w + p.pad;
+    int oh_lo = hp - p.pool + 1 <= 0 ? 0 : (hp - p.pool + p.stride) / p.stride;
+    int ow_lo = wp - p.pool + 1 <= 0 ? 0 : (wp - p.pool + p.stride) / p.stride;
+    int oh_hi = hp / p.stride, ow_hi = wp / p.stride;
+    if (oh_hi > p.H_out - 1) oh_hi = p.H_out - 1;
+    if (ow_hi > p.W_out - 1) ow_hi = p.W_out - 1;
+    const float* g = dout + plane * p.H_out * p.W_out;
+    float acc = din[idx];
+    for (int oh = oh_lo; oh <= oh_hi; oh++) {
+        const int h0 = oh * p.stride - p.pad;
+        const int rows = min(h0 + p.pool, p.H_in) - max(h0, 0);
+        for (int ow = ow_lo; ow <= ow_hi; ow++) {
+            const int w0 = ow * p.stride - p.pad;
+            const int cols = min(w0 + p.pool, p.W_in) - max(w0, 0);
+            const float div = p.pad == 0 ? (float)(p.pool * p.pool) : (float)(rows * cols);
+            acc += g[(long)oh * p.W_out + ow] / div;
+        }
+    }
+    din[idx] = acc;
+}
+
+// ---- binary cross-entropy ------------------------------------------------------------------------
+// loss = sum_i (-t_i log p_i - (1 - t_i) log(1 - p_i)) / n. Two steps with a fixed shape: up to 1024
+// workgroups add their grid-strided terms (lane, wave shuffle, four waves), then one workgroup adds the
+// partial sums the same way, so the value depends on n only. __logf is the fast hardware logarithm,
+// as in the reference's kernel.
+constexpr int BCE_MAX_BLOCKS = 1024;
+
+__device__ __forceinline__ float block_sum_256(float v, float* part) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+__global__ __launch_bounds__(256) void bce_partial_kernel(float* __restrict__ partial, const float* __restrict__ predict,
+                                                          const float* __restrict__ real, long n) {
+    __shared__ float part[4];
+    float s = 0.f;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        const float p = predict[i], t = real[i];
+        s += (-t * __logf(p) - (1 - t) * __logf(1 - p)) / (float)n;
+    }
+    const float total = block_sum_256(s, part);
+    if (threadIdx.x == 0) partial[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(256) void bce_final_kernel(float* __restrict__ loss, const float* __restrict__ partial, int m) {
+    __shared__ float part[4];
+    float s = 0.f;
+    for (int i = threadIdx.x; i < m; i += 256) s += partial[i];
+    const float total = block_sum_256(s, part);
+    if (threadIdx.x == 0) *loss = total;
+}
+
+__global__ __launch_bounds__(256) void bce_backward_kernel(float* __restrict__ grad, const float* __restrict__ predict,
+                                                           const float* __restrict__ real, long n) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float p = predict[i];
+    grad[i] = ((p - real[i]) / (p * (1 - p))) / (float)n;
+}
+
+// ---- expand / compress --------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void expand_kernel(float* __restrict__ out, const float* __restrict__ in, long n, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < total) out[i] = in[i % n];
+}
+
+// out[j] += in[j] + in[n + j] + ... in ascending batch order (a serial run of the reference's atomicAdd loop)
+__global__ __launch_bounds__(256) void compress_kernel(float* __restrict__ out, const float* __restrict__ in, long n, long batches) {
+    const long j = (long)blockIdx.x * 256 + threadIdx.x;
+    if (j >= n) return;
+    float acc = out[j];
+    for (long b = 0; b < batches; b++) acc += in[b * n + j];
+    out[j] = acc;
+}
+
+static int pool_args(PoolArgs& p, size_t pool, size_t stride, size_t pad, size_t batches, size_t channels, size_t H_in,
+                     size_t W_in, size_t H_out, size_t W_out, const char* who) {
+    if (pool == 0 || stride == 0) return set_error(NZHIP_E_INVALID, "%s: zero pool size or stride", who);
+    if (H_in + 2 * pad < pool || W_in + 2 * pad < pool) return set_error(NZHIP_E_SHAPE, "%s: window larger than the padded input", who);
+    if (H_out != (H_in + 2 * pad - pool) / stride + 1 || W_out != (W_in + 2 * pad - pool) / stride + 1)
+        return set_error(NZHIP_E_SHAPE, "%s: output extent does not match (in + 2 pad - pool) / stride + 1", who);
+    if (pool > 0x7fff || stride > 0x3fffffff || pad > 0x3fffffff || H_in > 0x3fffffff || W_in > 0x3fffffff ||
+        batches * channels > 0x7fffffffffffull / ((H_in * W_in) | 1))
+        return set_error(NZHIP_E_UNSUPPORTED, "%s: extent too large", who);
+    p.pool = (int)pool; p.stride = (int)stride; p.pad = (int)pad;
+    p.H_in = (int)H_in; p.W_in = (int)W_in; p.H_out = (int)H_out; p.W_out = (int)W_out;
+    p.planes = (long)(batches * channels);
+    return NZHIP_OK;
+}
+
+}  // namespace nzhip
+
+using namespace nzhip;
+
+extern "C" {
+
+int nzhip_avgpool2d(float* out, const float* in, size_t pool, size_t stride, size_t pad, size_t batches, size_t channels,
+                    size_t H_in, size_t W_in, size_t H_out, size_t W_out, void* stream) {
+    if (!out || !in) return set_error(NZHIP_E_INVALID, "nzhip_avgpool2d: null pointer");
+    PoolArgs p;
+    if (int rc = pool_args(p, pool, stride, pad, batches, channels, H_in, W_in, H_out, W_out, "nzhip_avgpool2d")) return rc;
+    const size_t total = batches * channels * H_out * W_out;
+    if (total == 0) return NZHIP_OK;
+    if ((total + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_avgpool2d: extent too large");
+    hipLaunchKernelGGL(avgpool_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), out, in, p);
+    return check_launch("avgpool_kernel");
+}
+
+int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches,
+                             size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out, void* stream) {
+    if (!din || !dout) return set_error(NZHIP_E_INVALID, "nzhip_avgpool2d_backward: null pointer");
+    PoolArgs p;
+    if (int rc = pool_args(p, pool, stride, pad, batches, channels, H_in, W_in, H_out, W_out, "nzhip_avgpool2d_backward")) return rc;
+    const size_t total = batches * channels * H_in * W_in;
+    if (total == 0) return NZHIP_OK;
+    if ((total + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_avgpool2d_backward: extent too large");
+    hipLaunchKernelGGL(avgpool_backward_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), din,
+                       dout, p);
+    return check_launch("avgpool_backward_kernel");
+}
+
+int nzhip_bce_loss(float* loss, const float* predict, const float* real, size_t n, void* stream) {
+    if (!loss || ((!predict || !real) && n)) return set_error(NZHIP_E_INVALID, "nzhip_bce_loss: null pointer");
+    hipStream_t s = as_stream(stream);
+    size_t blocks = (n + 255) / 256;
+    if (blocks > (size_t)BCE_MAX_BLOCKS) blocks = BCE_MAX_BLOCKS;
+    if (blocks == 0) blocks = 1;                                  // n = 0: the sum of nothing
+    float* partial = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), blocks * sizeof(float), s)) return rc;
+    hipLaunchKernelGGL(bce_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, s, partial, predict, real, (long)n);
+    int rc = check_launch("bce_partial_kernel");
+    if (rc == NZHIP_OK) {
+        hipLaunchKernelGGL(bce_final_kernel, dim3(1), dim3(256), 0, s, loss, partial, (int)blocks);
+        rc = check_launch("bce_final_kernel");
+    }
+    const int rc2 = workspace_free(partial, s);
+    return rc ? rc : rc2;
+}
+
+int nzhip_bce_backward(float* grad, const float* predict, const float* real, size_t n, void* stream) {
+    if ((!grad || !predict || !real) && n) return set_error(NZHIP_E_INVALID, "nzhip_bce_backward: null pointer");
+    if (n == 0) return NZHIP_OK;
+    if ((n + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_bce_backward: extent too large");
+    hipLaunchKernelGGL(bce_backward_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), grad, predict,
+                       real, (long)n);
+    return check_launch("bce_backward_kernel");
+}
+
+int nzhip_expand(float* out, const float* in, size_t n, size_t batches, void* stream) {
+    if ((!out || !in) && n * batches) return set_error(NZHIP_E_INVALID, "nzhip_expand: null pointer");
+    const size_t total = n * batches;
+    if (total == 0) return NZHIP_OK;
+    if ((total + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_expand: extent too large");
+    hipLaunchKernelGGL(expand_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), out, in, (long)n,
+                       (long)total);
+    return check_launch("expand_kernel");
+}
+
+int nzhip_compress(float* out, const float* in, size_t n, size_t batches, void* stream) {
+    if ((!out || !in) && n * batches) return set_error(NZHIP_E_INVALID, "nzhip_compress: null pointer");
+    if (n == 0 || batches == 0) return NZHIP_OK;
+    if ((n + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_compress: extent too large");
+    hipLaunchKernelGGL(compress_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), out, in, (long)n,
+                       (long)batches);
+    return check_launch("compress_kernel");
+}
+
+}  // extern "C"

@@ -37,6 +37,7 @@ namespace nz::graph {
         void backward();
         void zeroGrad() const;                           // src/ComputeGraph.cu:434-438
         void update(opt::Optimizer* optimizer) const;    // one step() per node that requires gradients (:541-547)
+        [[nodiscard]] Tensor::value_type getLoss() const;      // of the first output node; throws std::runtime_error without one (:534-539)
         [[nodiscard]] io::OutputNode* getOutputNode() const;   // throws std::runtime_error without exactly one output
         void setFusion(bool enabled);
         [[nodiscard]] size_t fusedGroupCount() const { return fusedGroups; }

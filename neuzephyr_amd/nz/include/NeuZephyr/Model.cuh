@@ -25,6 +25,7 @@ namespace nz {
         data::Tensor& forward();
         void backward();                                 // reverse pass of the graph (src/Model.cu:17-19)
         void update(opt::Optimizer* optimizer) const;    // graph update, then zeroGrad (src/Model.cu:20-23)
+        [[nodiscard]] data::Tensor::value_type getLoss() const;   // loss of the last forward() (src/Model.cu:25-27)
         graph::ComputeGraph& graph() { return computeGraph; }
         // Parameters (weights, biases) in creation order, so that callers can inject values.
         [[nodiscard]] const std::vector<io::InputNode*>& parameters() const { return params; }
@@ -48,6 +49,13 @@ namespace nz {
         Node* Conv2d(Node* input, data::Tensor::size_type outChannels, data::Tensor::size_type kernelHeight,
                      data::Tensor::size_type kernelWidth, data::Tensor::size_type stride,
                      data::Tensor::size_type padding, bool bias = true);
+        // softmax over all of (c, h, w) per sample (the input is reshaped to [n, 1, c*h*w, 1] first; src/Model.cu:185-202)
+        Node* Softmax(Node* input);
+        // a batch-1 target repeated to `shape`'s batch; any other mismatch throws std::runtime_error (src/Model.cu:204-221)
+        Node* TargetExpand(Node* input, const data::Tensor::shape_type& shape);
+        Node* AvgPool2d(Node* input, data::Tensor::size_type poolSize, data::Tensor::size_type stride,
+                        data::Tensor::size_type padding = 0);
+        void BCELoss(Node* input, Node* target);         // terminates the graph (src/Model.cu:317-325)
         void defaultOutput(Node* input);
     };
 }

@@ -270,6 +270,11 @@ namespace nz::graph {
             if (node->output && node->output->requiresGrad()) node->output->zeroGrad();
     }
 
+    Tensor::value_type ComputeGraph::getLoss() const {
+        if (outputNodes.empty()) throw std::runtime_error("No output node");
+        return outputNodes[0]->getLoss();
+    }
+
     io::OutputNode* ComputeGraph::getOutputNode() const {
         if (outputNodes.empty()) throw std::runtime_error("No output node");
         if (outputNodes.size() > 1) throw std::runtime_error("Multiple output nodes");

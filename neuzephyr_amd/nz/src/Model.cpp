@@ -1,5 +1,7 @@
 #include "NeuZephyr/Model.cuh"
 
+#include <stdexcept>
+
 namespace nz {
     Model::Model() = default;
 
@@ -101,6 +103,39 @@ namespace nz {
         return Col2Img(result, (s.H() + 2 * padding - kernelHeight) / stride + 1,
                        (s.W() + 2 * padding - kernelWidth) / stride + 1);
     }
+
+    Node* Model::Softmax(Node* input) {
+        computeGraph.addNode(input);
+        const auto s = input->output->shape();
+        const size_t size = s[1] * s[2] * s[3];
+        Node* shaped = s[2] != size ? Reshape(input, {s[0], 1, size, 1}) : input;
+        return track(new calc::SoftmaxNode(shaped));
+    }
+
+    Node* Model::TargetExpand(Node* input, const data::Tensor::shape_type& shape) {
+        computeGraph.addNode(input);
+        const auto s = input->output->shape();
+        if (s == shape) return input;
+        if (s[0] != 1 || s[1] != shape[1] || s[2] != shape[2] || s[3] != shape[3])
+            throw std::runtime_error("The input data cannot be expanded.");
+        return track(new calc::ExpandNode(input, shape.N()));
+    }
+
+    Node* Model::AvgPool2d(Node* input, const data::Tensor::size_type poolSize, const data::Tensor::size_type stride,
+                           const data::Tensor::size_type padding) {
+        computeGraph.addNode(input);
+        return track(new calc::AveragePoolingNode(input, poolSize, stride, padding));
+    }
+
+    void Model::BCELoss(Node* input, Node* target) {
+        computeGraph.addNode(input);
+        Node* expanded = TargetExpand(target, input->output->shape());
+        auto* bce = new loss::BinaryCrossEntropyNode(input, expanded);
+        hiddenNodes.push_back(bce);
+        computeGraph.addOutput(bce);
+    }
+
+    data::Tensor::value_type Model::getLoss() const { return computeGraph.getLoss(); }
 
     void Model::defaultOutput(Node* input) {
         auto* output = new io::OutputNode(input);

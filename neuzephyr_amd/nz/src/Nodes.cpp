@@ -129,6 +129,46 @@ namespace nz::nodes {
             iSoftmaxBackward(inputs[0]->output->grad(), output->data(), output->grad(), s[2] * s[3], s[0] * s[1]);
         }
 
+        ExpandNode::ExpandNode(Node* input, const Tensor::size_type newBatch) : newBatch(newBatch) {
+            if (input->output->shape()[0] != 1) throw std::invalid_argument("ExpandNode: input must have batch size 1");
+            inputs.push_back(input);
+            const auto s = input->output->shape();
+            output = std::make_shared<Tensor>(Tensor::shape_type{newBatch, s[1], s[2], s[3]}, input->output->requiresGrad());
+            type = "Expand";
+        }
+
+        void ExpandNode::forward() { iExpand(output->data(), inputs[0]->output->data(), inputs[0]->output->size(), newBatch); }
+        void ExpandNode::backward() {                                  // src/Nodes.cu:594-603
+            if (inputs[0]->output->requiresGrad())
+                iCompress(inputs[0]->output->grad(), output->grad(), inputs[0]->output->size(), newBatch);
+        }
+
+        AveragePoolingNode::AveragePoolingNode(Node* input, const Tensor::size_type poolSize, const Tensor::size_type stride,
+                                               const Tensor::size_type padding)
+            : poolSize(poolSize), stride(stride), padding(padding) {
+            const auto s = input->output->shape();
+            if (poolSize == 0 || stride == 0 || s[2] + 2 * padding < poolSize || s[3] + 2 * padding < poolSize)
+                throw std::invalid_argument("AveragePoolingNode: window does not fit the padded input");
+            inputs.push_back(input);
+            output = std::make_shared<Tensor>(Tensor::shape_type{s[0], s[1], (s[2] + 2 * padding - poolSize) / stride + 1,
+                                                                 (s[3] + 2 * padding - poolSize) / stride + 1},
+                                              input->output->requiresGrad());
+            type = "AveragePooling";
+        }
+
+        void AveragePoolingNode::forward() {
+            const auto si = inputs[0]->output->shape(), so = output->shape();
+            iAveragePooling(output->data(), inputs[0]->output->data(), poolSize, stride, padding, si[0], si[1], si[2], si[3],
+                            so[2], so[3]);
+        }
+
+        void AveragePoolingNode::backward() {                          // src/Nodes.cu:684-690
+            if (!inputs[0]->output->requiresGrad()) return;
+            const auto si = inputs[0]->output->shape(), so = output->shape();
+            iAveragePoolingBackward(inputs[0]->output->grad(), output->grad(), poolSize, stride, padding, si[0], si[1], si[2],
+                                    si[3], so[2], so[3]);
+        }
+
         ReshapeNode::ReshapeNode(Node* input, const Tensor::shape_type& newShape) : newShape(newShape) {
             if (input->output->shape().size() != newShape.size()) {
                 throw std::invalid_argument("ReshapeNode: input and new shape must have the same number of dimensions");
@@ -190,6 +230,25 @@ namespace nz::nodes {
             if (inputs[0]->output->requiresGrad())
                 iCol2imgBackward(inputs[0]->output->grad(), output->grad(), outputHeight, outputWidth, outputChannels,
                                  inputs[0]->output->shape()[0]);
+        }
+    }
+
+    namespace loss {
+        BinaryCrossEntropyNode::BinaryCrossEntropyNode(Node* input1, Node* input2) : OutputNode(input1) {
+            if (input1->output->shape() != input2->output->shape())
+                throw std::invalid_argument("input1 and input2 should have the same shape");
+            inputs.push_back(input2);
+            type = "BinaryCrossEntropy";
+        }
+
+        void BinaryCrossEntropyNode::forward() {                       // src/Nodes.cu:822-840
+            OutputNode::forward();
+            loss = iBinaryCrossEntropy(inputs[0]->output->data(), inputs[1]->output->data(), output->size());
+        }
+
+        void BinaryCrossEntropyNode::backward() {                      // src/Nodes.cu:842-849
+            if (output->requiresGrad())
+                iBCEBackward(output->grad(), inputs[0]->output->data(), inputs[1]->output->data(), output->size());
         }
     }
 }

@@ -125,6 +125,44 @@ namespace nz::data {
         NZ_CHECK(nzhip_softmax_backward(dx, s, dy, n, batch, nzhip_default_stream()));
     }
 
+    void iAveragePooling(float* out, float* in, const size_t pool_size, const size_t stride, const size_t padding,
+                         const size_t batches, const size_t channels, const size_t H_in, const size_t W_in,
+                         const size_t H_out, const size_t W_out) {
+        NZ_CHECK(nzhip_avgpool2d(out, in, pool_size, stride, padding, batches, channels, H_in, W_in, H_out, W_out,
+                                 nzhip_default_stream()));
+    }
+
+    void iAveragePoolingBackward(float* out, float* in, const size_t pool_size, const size_t stride, const size_t padding,
+                                 const size_t batches, const size_t channels, const size_t H_in, const size_t W_in,
+                                 const size_t H_out, const size_t W_out) {
+        NZ_CHECK(nzhip_avgpool2d_backward(out, in, pool_size, stride, padding, batches, channels, H_in, W_in, H_out, W_out,
+                                          nzhip_default_stream()));
+    }
+
+    float iBinaryCrossEntropy(float* predict, float* real, const size_t n) {
+        void* dev = nullptr;
+        NZ_CHECK(nzhip_malloc(&dev, sizeof(float)));
+        float host = 0.f;
+        int rc = nzhip_bce_loss(static_cast<float*>(dev), predict, real, n, nzhip_default_stream());
+        if (rc == 0) rc = nzhip_memcpy_d2h(&host, dev, sizeof(float));      // blocks until the value is here
+        const int rc2 = nzhip_free(dev);
+        NZ_CHECK(rc);
+        NZ_CHECK(rc2);
+        return host;
+    }
+
+    void iBCEBackward(float* grad, float* predict, float* real, const size_t n) {
+        NZ_CHECK(nzhip_bce_backward(grad, predict, real, n, nzhip_default_stream()));
+    }
+
+    void iExpand(float* out, float* in, const size_t n, const size_t batches) {
+        NZ_CHECK(nzhip_expand(out, in, n, batches, nzhip_default_stream()));
+    }
+
+    void iCompress(float* out, float* in, const size_t n, const size_t batches) {
+        NZ_CHECK(nzhip_compress(out, in, n, batches, nzhip_default_stream()));
+    }
+
     void iConv2dForward(float* y, float* x, float* w, float* bias, const size_t N, const size_t C, const size_t H,
                         const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
                         const size_t pad, const size_t weightBatch, const long long biasPixelStride,

@@ -22,6 +22,7 @@ using namespace nz::data;
 using namespace nz::nodes;
 using namespace nz::nodes::io;
 using namespace nz::nodes::calc;
+using namespace nz::nodes::loss;
 
 static float f16(float x) { return _cvtsh_ss(_cvtss_sh(x, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC)); }
 
@@ -688,6 +689,159 @@ TEST(NodeBasic, SoftmaxForwardJacobianBackward) {
     EXPECT_TRUE(closeTo(input.output->hostGrad(), wantD, 1e-4));
     InputNode notVector({1, 1, 2, 2});
     EXPECT_THROW(SoftmaxNode bad(&notVector), std::invalid_argument);
+}
+
+// ---- pooling, loss, expand: the loop nests of the reference's tests (test/Test.cpp:3179-3385, 1937-1999, 2663-2730) ----
+TEST(NodeBasic, AveragePoolingForwardBackward) {
+    const size_t n = 2, c = 3, h = 9, w = 7, pool = 3, stride = 2, pad = 1;
+    const size_t Ho = (h + 2 * pad - pool) / stride + 1, Wo = (w + 2 * pad - pool) / stride + 1;
+    auto x = randomVec(n * c * h * w, 101, 0.1f, 0.9f), g = randomVec(n * c * Ho * Wo, 102, 0.1f, 0.9f);
+    std::vector<float> want(n * c * Ho * Wo, 0.f);
+    std::vector<double> wantGrad(n * c * h * w, 0.0);
+    for (size_t pl = 0; pl < n * c; pl++)
+        for (size_t k = 0; k < Ho; k++)
+            for (size_t l = 0; l < Wo; l++) {
+                const long long h0 = (long long)(k * stride) - (long long)pad, w0 = (long long)(l * stride) - (long long)pad;
+                size_t count = 0;
+                float sum = 0.f;
+                for (size_t r = 0; r < pool; r++)
+                    for (size_t q = 0; q < pool; q++) {
+                        const long long hi = h0 + (long long)r, wi = w0 + (long long)q;
+                        if (hi >= 0 && hi < (long long)h && wi >= 0 && wi < (long long)w) {
+                            sum += x[pl * h * w + hi * w + wi];
+                            count++;
+                        }
+                    }
+                want[pl * Ho * Wo + k * Wo + l] = count ? sum / static_cast<float>(count) : 0.f;
+                for (size_t r = 0; r < pool; r++)
+                    for (size_t q = 0; q < pool; q++) {
+                        const long long hi = h0 + (long long)r, wi = w0 + (long long)q;
+                        if (hi >= 0 && hi < (long long)h && wi >= 0 && wi < (long long)w)
+                            wantGrad[pl * h * w + hi * w + wi] += g[pl * Ho * Wo + k * Wo + l] / static_cast<float>(count);
+                    }
+            }
+    InputNode input({n, c, h, w}, true);
+    input.dataInject(x.begin(), x.end());
+    AveragePoolingNode poolNode(&input, pool, stride, pad);
+    poolNode.forward();
+    EXPECT_TRUE(poolNode.output->hostData() == want);
+    input.output->zeroGrad();
+    poolNode.output->dataInject(g.begin(), g.end(), true);
+    poolNode.backward();
+    EXPECT_TRUE(closeTo(input.output->hostGrad(), wantGrad, 1e-6));
+    Tensor t({n, c, h, w});
+    t.dataInject(x.begin(), x.end());
+    EXPECT_TRUE(tensorAveragePooling(t, pool, stride, pad).hostData() == want);
+    EXPECT_THROW(AveragePoolingNode bad(&input, 12, 1, 0), std::invalid_argument);
+}
+
+TEST(NodeLoss, BCEForwardBackward) {
+    const size_t n = 2, c = 3, h = 12, w = 5, total = n * c * h * w;
+    auto predict = randomVec(total, 103, 0.1f, 0.9f), target = randomVec(total, 104, 0.1f, 0.9f);
+    double lossWant = 0;
+    std::vector<double> gradWant(total);
+    for (size_t i = 0; i < total; i++) {
+        lossWant += -target[i] * std::log((double)predict[i]) - (1 - target[i]) * std::log(1.0 - predict[i]);
+        gradWant[i] = ((predict[i] - target[i]) / ((double)predict[i] * (1 - predict[i]))) / total;
+    }
+    lossWant /= total;
+    InputNode input1({n, c, h, w}, true), input2({n, c, h, w});
+    input1.dataInject(predict.begin(), predict.end());
+    input2.dataInject(target.begin(), target.end());
+    BinaryCrossEntropyNode bce(&input1, &input2);
+    bce.forward();
+    EXPECT_TRUE(std::fabs(bce.getLoss() - lossWant) < 1e-5 * lossWant);
+    bce.forward();                                            // the loss of a pass, not a running total
+    EXPECT_TRUE(std::fabs(bce.getLoss() - lossWant) < 1e-5 * lossWant);
+    bce.backward();
+    EXPECT_TRUE(closeTo(input1.output->hostGrad(), gradWant, 1e-6));
+    InputNode other({n, c, h, w + 1});
+    EXPECT_THROW(BinaryCrossEntropyNode bad(&input1, &other), std::invalid_argument);
+}
+
+TEST(NodeBasic, ExpandForwardBackward) {
+    const size_t c = 2, h = 3, w = 4, batch = 5, per = c * h * w;
+    auto x = randomVec(per, 105, -1.f, 1.f), g = randomVec(per * batch, 106, -1.f, 1.f);
+    InputNode input({1, c, h, w}, true);
+    input.dataInject(x.begin(), x.end());
+    ExpandNode expand(&input, batch);
+    expand.forward();
+    const auto out = expand.output->hostData();
+    for (size_t i = 0; i < per * batch; i++) EXPECT_TRUE(out[i] == x[i % per]);
+    input.output->zeroGrad();
+    expand.output->dataInject(g.begin(), g.end(), true);
+    expand.backward();
+    std::vector<double> want(per, 0.0);
+    for (size_t i = 0; i < per * batch; i++) want[i % per] += g[i];
+    EXPECT_TRUE(closeTo(input.output->hostGrad(), want, 1e-6));
+    InputNode batched({2, c, h, w});
+    EXPECT_THROW(ExpandNode bad(&batched, 3), std::invalid_argument);
+}
+
+// The network of the reference's README (README.md:62-90) at a reduced image size: Conv2d -> ReLU -> Conv2d ->
+// AvgPool2d -> Linear -> Softmax -> BCELoss, trained with Adam. The labels are given once and expanded to the batch.
+struct ReadmeModel : nz::Model {
+    InputNode input, target;
+    ReadmeModel(size_t n, size_t h, size_t w) : input({n, 3, h, w}), target({1, 1, 16, 1}) {
+        Node* x = Conv2d(&input, 1, 3, 3, 1, 1);
+        x = ReLU(x);
+        x = Conv2d(x, 1, 3, 3, 1, 1);
+        x = AvgPool2d(x, 5, 2);
+        x = Linear(x, 16);
+        x = Softmax(x);
+        BCELoss(x, &target);
+    }
+    Node* checkExpand(Node* t) { return TargetExpand(t, Tensor::shape_type{4, 1, 16, 1}); }
+};
+
+TEST(Model, ReadmeExampleTrains) {
+    const size_t n = 4, h = 40, w = 48;
+    ReadmeModel m(n, h, w);
+    auto x = randomVec(n * 3 * h * w, 111, 0.f, 1.f);
+    m.input.dataInject(x.begin(), x.end());
+    std::vector<float> labels(16, 0.02f);
+    labels[3] = 0.7f;
+    m.target.dataInject(labels.begin(), labels.end());
+    // small positive parameters keep the ReLU alive and the softmax away from saturation
+    unsigned seed = 120;
+    for (auto* p : m.parameters()) {
+        auto v = randomVec(p->output->size(), seed++, 0.0f, 0.05f);
+        p->dataInject(v.begin(), v.end());
+    }
+    nz::opt::Adam optimizer(0.01f, 0.9f, 0.999f);
+    m.forward();
+    const float first = m.getLoss();
+    EXPECT_TRUE(std::isfinite(first) && first > 0.f);
+    float last = first;
+    for (int epoch = 0; epoch < 8; ++epoch) {
+        m.backward();
+        m.update(&optimizer);
+        m.forward();
+        last = m.getLoss();
+        EXPECT_TRUE(std::isfinite(last));
+    }
+    EXPECT_TRUE(last < first);
+    // the same steps without the fused chains reach the same loss
+    ReadmeModel r(n, h, w);
+    r.graph().setFusion(false);
+    r.input.dataInject(x.begin(), x.end());
+    r.target.dataInject(labels.begin(), labels.end());
+    seed = 120;
+    for (auto* p : r.parameters()) {
+        auto v = randomVec(p->output->size(), seed++, 0.0f, 0.05f);
+        p->dataInject(v.begin(), v.end());
+    }
+    nz::opt::Adam optimizer2(0.01f, 0.9f, 0.999f);
+    r.forward();
+    EXPECT_TRUE(std::fabs(r.getLoss() - first) <= 1e-5f * first);
+    for (int epoch = 0; epoch < 8; ++epoch) {
+        r.backward();
+        r.update(&optimizer2);
+        r.forward();
+    }
+    EXPECT_TRUE(std::fabs(r.getLoss() - last) <= 2e-3f * std::fabs(last));
+    InputNode wrong({2, 1, 16, 1});
+    EXPECT_THROW(m.checkExpand(&wrong), std::runtime_error);
 }
 
 TEST(Runtime, AllocatorCachesAndErrorsSurfaceAsExceptions) {

@@ -655,6 +655,67 @@ void nzo_fill(float* dst, size_t n, uint64_t seed, int kind, double lo, double h
     }
 }
 
+void nzo_avgpool2d(float* out, const float* in, size_t pool, size_t stride, size_t pad, size_t batches,
+                   size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out) {
+    for (size_t pl = 0; pl < batches * channels; pl++)
+        for (size_t h = 0; h < H_out; h++)
+            for (size_t w = 0; w < W_out; w++) {
+                const long long h0 = (long long)(h * stride) - (long long)pad, w0 = (long long)(w * stride) - (long long)pad;
+                float sum = 0.0f;
+                size_t count = 0;
+                for (size_t i = 0; i < pool; i++)
+                    for (size_t j = 0; j < pool; j++) {
+                        const long long hi = h0 + (long long)i, wi = w0 + (long long)j;
+                        if (hi >= 0 && hi < (long long)H_in && wi >= 0 && wi < (long long)W_in) {
+                            sum += in[pl * H_in * W_in + (size_t)hi * W_in + (size_t)wi];
+                            count++;
+                        }
+                    }
+                out[pl * H_out * W_out + h * W_out + w] = count > 0 ? sum / (float)count : 0.0f;
+            }
+}
+
+void nzo_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches,
+                            size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out) {
+    for (size_t pl = 0; pl < batches * channels; pl++)
+        for (size_t h = 0; h < H_out; h++)
+            for (size_t w = 0; w < W_out; w++) {
+                const long long h0 = (long long)(h * stride) - (long long)pad, w0 = (long long)(w * stride) - (long long)pad;
+                size_t count = 0;
+                for (size_t i = 0; i < pool; i++)
+                    for (size_t j = 0; j < pool; j++) {
+                        const long long hi = h0 + (long long)i, wi = w0 + (long long)j;
+                        if (hi >= 0 && hi < (long long)H_in && wi >= 0 && wi < (long long)W_in) count++;
+                    }
+                const float g = dout[pl * H_out * W_out + h * W_out + w];
+                const float div = pad == 0 ? (float)(pool * pool) : (float)count;
+                for (size_t i = 0; i < pool; i++)
+                    for (size_t j = 0; j < pool; j++) {
+                        const long long hi = h0 + (long long)i, wi = w0 + (long long)j;
+                        if (hi >= 0 && hi < (long long)H_in && wi >= 0 && wi < (long long)W_in)
+                            din[pl * H_in * W_in + (size_t)hi * W_in + (size_t)wi] += g / div;
+                    }
+            }
+}
+
+float nzo_bce_loss(const float* predict, const float* real, size_t n) {
+    float loss = 0.0f;
+    for (size_t i = 0; i < n; i++) loss += -real[i] * logf(predict[i]) - (1 - real[i]) * logf(1 - predict[i]);
+    return n ? loss / (float)n : 0.0f;
+}
+
+void nzo_bce_backward(float* grad, const float* predict, const float* real, size_t n) {
+    for (size_t i = 0; i < n; i++) grad[i] = ((predict[i] - real[i]) / (predict[i] * (1 - predict[i]))) / (float)n;
+}
+
+void nzo_expand(float* out, const float* in, size_t n, size_t batches) {
+    for (size_t i = 0; i < n * batches; i++) out[i] = in[i % n];
+}
+
+void nzo_compress(float* out, const float* in, size_t n, size_t batches) {
+    for (size_t i = 0; i < n * batches; i++) out[i % n] += in[i];
+}
+
 int nzo_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

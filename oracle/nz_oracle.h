@@ -159,6 +159,26 @@ void nzo_sgd_step(float* data, const float* grad, float lr, size_t n);
 void nzo_adam_step(float* data, float* m, float* v, const float* grad, float lr, float beta1, float beta2,
                    float eps, int t, size_t n);
 
+/* ---- average pooling, binary cross-entropy, expand / compress -----------------
+ * AveragePoolingKernel (src/OperationKernels.cu:1404-1429), which is also the loop nest of the reference's
+ * own test (test/Test.cpp:3179-3246): mean over the window cells inside the image, row by row. */
+void nzo_avgpool2d(float* out, const float* in, size_t pool, size_t stride, size_t pad, size_t batches,
+                   size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out);
+/* AveragePoolingBackwardKernel (:1439-1486) run serially in ascending output index: din += dout / divisor
+ * (pool^2 without padding, the in-image cell count with padding). The reference's atomicAdd order is not
+ * defined; a serial run is one of its possible orders. */
+void nzo_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches,
+                            size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out);
+/* Mean binary cross-entropy as the reference's test states it (test/Test.cpp:1955-1958): the terms summed in
+ * ascending order with logf, then divided by n. The kernel (:648-685) divides every term by n, uses __logf
+ * and a tree sum: last bits are PARITY UNPINNED (the reference's test compares at 1e-2). */
+float nzo_bce_loss(const float* predict, const float* real, size_t n);
+/* BCEBackwardKernel (:692-699; test/Test.cpp:1985-1987): ((p - t) / (p (1 - p))) / n. */
+void nzo_bce_backward(float* grad, const float* predict, const float* real, size_t n);
+/* ExpandKernel / CompressKernel (:1282-1301), the latter run serially in ascending index. */
+void nzo_expand(float* out, const float* in, size_t n, size_t batches);
+void nzo_compress(float* out, const float* in, size_t n, size_t batches);
+
 /* max over i of |got-truth| / max(|truth|, floor) and Frobenius ||got-truth|| / ||truth|| */
 void nzo_errors_f32_vs_f64(const float* got, const double* truth, size_t n, double floor_abs,
                            double* max_rel, double* frob_rel);

@@ -85,6 +85,12 @@ _conv_bwd_data = _sig("nzo_conv2d_backward_data", None, _f32p, _f32p, _f32p, *([
 _conv_bwd_w = _sig("nzo_conv2d_backward_weights", None, _f32p, _f32p, _f32p, *([_sz] * 9))
 _softmax = _sig("nzo_softmax", None, _f32p, _f32p, _sz, _sz)
 _softmax_jac = _sig("nzo_softmax_jacobian", None, _f32p, _f32p, _sz, _sz)
+_avgpool = _sig("nzo_avgpool2d", None, _f32p, _f32p, *([_sz] * 9))
+_avgpool_bwd = _sig("nzo_avgpool2d_backward", None, _f32p, _f32p, *([_sz] * 9))
+_bce = _sig("nzo_bce_loss", C.c_float, _f32p, _f32p, _sz)
+_bce_bwd = _sig("nzo_bce_backward", None, _f32p, _f32p, _f32p, _sz)
+_expand = _sig("nzo_expand", None, _f32p, _f32p, _sz, _sz)
+_compress = _sig("nzo_compress", None, _f32p, _f32p, _sz, _sz)
 _sgd = _sig("nzo_sgd_step", None, _f32p, _f32p, C.c_float, _sz)
 _adam = _sig("nzo_adam_step", None, _f32p, _f32p, _f32p, _f32p, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, _sz)
 _conv_graph = _sig("nzo_conv2d_graph", None, _f32p, _f32p, _f32p, C.c_void_p, *([_sz] * 10), C.c_int)
@@ -317,6 +323,48 @@ def softmax_backward(s: np.ndarray, dy: np.ndarray) -> np.ndarray:
     """SoftmaxNode::backward (src/Nodes.cu:538-548): Jacobian times gradient through the fp16 GEMM."""
     jac = softmax_jacobian(s)
     return tensorcore_gemm(jac, dy) if s.shape[2] > s.shape[3] else tensorcore_gemm(dy, jac)
+
+
+def avgpool2d(x: np.ndarray, pool: int, stride: int, pad: int) -> np.ndarray:
+    x = _c(x)
+    N, Cc, H, W = x.shape
+    Ho, Wo = (H + 2 * pad - pool) // stride + 1, (W + 2 * pad - pool) // stride + 1
+    out = np.empty((N, Cc, Ho, Wo), np.float32)
+    _avgpool(out.reshape(-1), x.reshape(-1), pool, stride, pad, N, Cc, H, W, Ho, Wo)
+    return out
+
+
+def avgpool2d_backward(dx: np.ndarray, dy: np.ndarray, pool: int, stride: int, pad: int) -> np.ndarray:
+    """Returns dx + gradient (dx has the input's shape)."""
+    dx, dy = _c(dx).copy(), _c(dy)
+    N, Cc, H, W = dx.shape
+    _avgpool_bwd(dx.reshape(-1), dy.reshape(-1), pool, stride, pad, N, Cc, H, W, dy.shape[2], dy.shape[3])
+    return dx
+
+
+def bce_loss(predict: np.ndarray, real: np.ndarray) -> float:
+    p, t = _c(predict), _c(real)
+    return float(_bce(p.reshape(-1), t.reshape(-1), p.size))
+
+
+def bce_backward(predict: np.ndarray, real: np.ndarray) -> np.ndarray:
+    p, t = _c(predict), _c(real)
+    g = np.empty_like(p)
+    _bce_bwd(g.reshape(-1), p.reshape(-1), t.reshape(-1), p.size)
+    return g
+
+
+def expand(x: np.ndarray, batches: int) -> np.ndarray:
+    x = _c(x)
+    out = np.empty((batches,) + x.shape[1:], np.float32)
+    _expand(out.reshape(-1), x.reshape(-1), x.size, batches)
+    return out
+
+
+def compress(out: np.ndarray, x: np.ndarray) -> np.ndarray:
+    out, x = _c(out).copy(), _c(x)
+    _compress(out.reshape(-1), x.reshape(-1), out.size, x.shape[0])
+    return out
 
 
 def sgd_step(data, grad, lr):

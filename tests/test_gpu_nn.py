@@ -1,0 +1,82 @@
+"""Average pooling, binary cross-entropy and expand / compress on the GPU against the CPU oracle, through
+the C-ABI. Pooling, its gradient, the loss gradient and expand / compress are compared bit for bit (same
+additions in the same order, correctly rounded divisions); the loss value uses the fast logarithm and a
+tree sum and is compared at 1e-5 relative."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+POOL_CASES = [((2, 3, 4, 5), 2, 2, 0), ((1, 2, 9, 7), 3, 1, 1), ((2, 1, 10, 10), 5, 2, 0), ((1, 1, 6, 8), 4, 3, 2),
+              ((1, 3, 5, 5), 5, 1, 2), ((2, 2, 7, 3), 1, 1, 0), ((1, 1, 8, 8), 3, 2, 1), ((3, 5, 33, 47), 3, 2, 1),
+              ((1, 1, 70, 300), 5, 2, 0), ((2, 2, 16, 16), 2, 2, 0), ((1, 1, 9, 9), 4, 5, 3)]
+
+
+@pytest.fixture(scope="module")
+def nz():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from neuzephyr_amd import capi
+    capi.load()
+    return capi
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def host(t):
+    return t.cpu().numpy()
+
+
+@pytest.mark.parametrize("shape,pool,stride,pad", POOL_CASES)
+def test_avgpool_forward_and_backward_bit_exact(nz, oracle, shape, pool, stride, pad):
+    rng = np.random.default_rng(sum(shape) + pool + stride)
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    want = oracle.avgpool2d(x, pool, stride, pad)
+    got = host(nz.avgpool2d(dev(x), pool, stride, pad))
+    assert got.shape == want.shape and np.array_equal(got, want)
+    dy = rng.uniform(-1, 1, want.shape).astype(np.float32)
+    base = rng.uniform(-1, 1, shape).astype(np.float32)
+    dx = dev(base)
+    nz.avgpool2d_backward(dx, dev(dy), pool, stride, pad)
+    assert np.array_equal(host(dx), oracle.avgpool2d_backward(base, dy, pool, stride, pad))
+
+
+def test_avgpool_rejects_bad_geometry(nz):
+    x = dev(np.zeros((1, 1, 4, 4)))
+    with pytest.raises(nz.NzHipError):
+        nz.avgpool2d(x, 5, 1, 0)                                   # window larger than the input
+    with pytest.raises(nz.NzHipError):
+        nz.avgpool2d(x, 2, 0, 0)                                   # zero stride
+    with pytest.raises(nz.NzHipError):
+        nz.avgpool2d_backward(x, dev(np.zeros((1, 1, 3, 3))), 2, 2, 0)   # dy extent does not match
+
+
+def test_bce_loss_and_backward(nz, oracle):
+    rng = np.random.default_rng(11)
+    for n in (1, 7, 360, 4097, 300001):
+        p = rng.uniform(0.1, 0.9, n).astype(np.float32)
+        t = rng.uniform(0.1, 0.9, n).astype(np.float32)
+        want = oracle.bce_loss(p, t)
+        got = float(host(nz.bce_loss(dev(p), dev(t)))[0])
+        p64, t64 = p.astype(np.float64), t.astype(np.float64)
+        truth = float(np.mean(-t64 * np.log(p64) - (1 - t64) * np.log1p(-p64)))
+        assert abs(got - truth) <= 1e-5 * truth and abs(want - truth) <= 1e-4 * truth, n
+        assert np.array_equal(host(nz.bce_backward(dev(p), dev(t))), oracle.bce_backward(p, t)), n
+    # the loss value does not depend on scheduling: the same input gives the same bits
+    a = host(nz.bce_loss(dev(p), dev(t)))
+    b = host(nz.bce_loss(dev(p), dev(t)))
+    assert np.array_equal(a, b)
+
+
+def test_expand_and_compress_bit_exact(nz, oracle):
+    rng = np.random.default_rng(12)
+    x = rng.normal(size=(1, 3, 16, 5)).astype(np.float32)
+    assert np.array_equal(host(nz.expand(dev(x), 7)), oracle.expand(x, 7))
+    g = rng.normal(size=(7, 3, 16, 5)).astype(np.float32)
+    base = rng.normal(size=(1, 3, 16, 5)).astype(np.float32)
+    out = dev(base)
+    nz.compress(out, dev(g))
+    assert np.array_equal(host(out), oracle.compress(base, g))
