@@ -1399,6 +1399,117 @@ __global__ __launch_bounds__(256) void conv_dw_reduce_kernel(float* __restrict__
     dW[(long)b * group_stride_dW + ((long)c0 * 9 + row) * O + o0 + col] += sum;
 }
 
+// ---- weight gradient of the 3x3, stride 1, pad 1 convolution with a handful of channels -------------
+// With C <= 4 and O <= 2 the gradient has at most 72 entries per weight copy, each a sum over every pixel:
+// a stream over x and dy, not a matrix product. Same thread mapping as the forward stream kernel (a lane
+// owns 4 adjacent columns of a 16-row strip, three rounded x rows in a rolling register window, halo
+// columns from the neighbour lanes), and C*9*O running sums per lane:
+//     acc[(c, r, s)][o] += f16(x[c][h + r - 1][w + s - 1]) * f16(dy[o][h][w]).
+// A wave adds its lanes in a fixed tree and writes one partial vector per strip; small_dw_reduce_kernel
+// adds the strips (and, for shared weights, the images) in ascending order.
+template <int O_T, int C_T>
+__global__ __launch_bounds__(256) void conv3x3_dw_stream_kernel(float* __restrict__ partial, const float* __restrict__ x,
+                                                                const float* __restrict__ dy, int H, int W) {
+    constexpr int Q = C_T * 9 * O_T;
+    int bx, by, b;
+    xcd_contiguous_block(bx, by, b);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int w0 = (bx * 64 + lane) * 4;
+    const int strip = by * 4 + wave, n_strips = gridDim.y * 4;
+    const int h0 = strip * ST_ROWS;
+    float acc[Q];
+#pragma unroll
+    for (int q = 0; q < Q; q++) acc[q] = 0.f;
+    if (h0 < H) {                                                // uniform over the wave
+        const bool col_ok = w0 < W;                              // W % 4 == 0: a lane's quad is all in or all out
+        const int wq = col_ok ? w0 : 0;
+        const bool has_l = col_ok && w0 > 0, has_r = col_ok && w0 + 4 < W;
+        const int wx = lane == 0 ? (has_l ? w0 - 1 : wq) : (lane == 63 && has_r ? w0 + 4 : wq);
+        const float* xb = x + (long)b * C_T * H * W;
+        const float* gb = dy + (long)b * O_T * H * W;
+        const long plane = (long)H * W;
+        const int rows = (H - h0) < ST_ROWS ? (H - h0) : ST_ROWS;
+        const int T = rows + 2;
+        float win[3][C_T][6];
+        for (int t0 = 0; t0 < T; t0 += 3) {
+#pragma unroll
+            for (int u = 0; u < 3; u++) {
+                const int t = t0 + u;
+                if (t >= T) break;
+                const int hi = h0 - 1 + t;
+                const bool in_img = hi >= 0 && hi < H;
+                const float* row = xb + (long)(in_img ? hi : 0) * W;
+#pragma unroll
+                for (int c = 0; c < C_T; c++) {
+                    const floatx4 qv = *reinterpret_cast<const floatx4*>(row + c * plane + wq);
+                    const float ex = row[c * plane + wx];
+                    float r5[5];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r5[e] = (in_img && col_ok) ? round_f16(qv[e]) : 0.f;
+                    r5[4] = in_img ? round_f16(ex) : 0.f;
+                    const float below = from_lane_below(r5[3]), above = from_lane_above(r5[0]);
+                    win[u][c][0] = has_l ? (lane == 0 ? r5[4] : below) : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) win[u][c][1 + e] = r5[e];
+                    win[u][c][5] = has_r ? (lane == 63 ? r5[4] : above) : 0.f;
+                }
+                if (t < 2) continue;
+                const int ho = h0 + t - 2;                       // rows t-2, t-1, t are the window of output row ho
+                float g[O_T][4];
+#pragma unroll
+                for (int o = 0; o < O_T; o++) {
+                    const floatx4 gv = *reinterpret_cast<const floatx4*>(gb + (long)o * plane + (long)ho * W + wq);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) g[o][e] = col_ok ? round_f16(gv[e]) : 0.f;
+                }
+#pragma unroll
+                for (int c = 0; c < C_T; c++)
+#pragma unroll
+                    for (int r = 0; r < 3; r++) {
+                        const int slot = (u + 1 + r) % 3;        // step t-2+r lives in slot (t-2+r) % 3, and t % 3 == u
+#pragma unroll
+                        for (int s2 = 0; s2 < 3; s2++)
+#pragma unroll
+                            for (int o = 0; o < O_T; o++)
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    acc[((c * 3 + r) * 3 + s2) * O_T + o] =
+                                        __builtin_fmaf(win[slot][c][e + s2], g[o][e], acc[((c * 3 + r) * 3 + s2) * O_T + o]);
+                    }
+            }
+        }
+    }
+    float* dst = partial + (((long)b * n_strips + strip) * gridDim.x + bx) * Q;
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+        float v = acc[q];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off);
+        if (lane == 0) dst[q] = v;
+    }
+}
+
+// dW[g][q] += sum over the S partial vectors of group g (a weight copy), in a fixed order: eight threads per
+// entry add a contiguous eighth each in ascending order, then the eight sums are added in ascending order.
+__global__ __launch_bounds__(256) void small_dw_reduce_kernel(float* __restrict__ dW, const float* __restrict__ P, int S,
+                                                              int Q) {
+    __shared__ float part[8][32];
+    const int k = threadIdx.x >> 5, tl = threadIdx.x & 31;
+    const int q = blockIdx.x * 32 + tl, g = blockIdx.y;
+    const bool live = q < Q;
+    const float* src = P + (long)g * S * Q + q;
+    const int per = (S + 7) / 8, s0 = k * per, s1 = (s0 + per) < S ? (s0 + per) : S;
+    float sum = 0.f;
+    if (live)
+        for (int s = s0; s < s1; s++) sum += src[(long)s * Q];
+    part[k][tl] = sum;
+    __syncthreads();
+    if (k != 0 || !live) return;
+#pragma unroll
+    for (int j = 1; j < 8; j++) sum += part[j][tl];
+    dW[(long)g * Q + q] += sum;
+}
+
 // Weights of the data-gradient convolution: the gradient with respect to x of a stride-1 convolution is
 // itself a stride-1 convolution of dy (O channels in, C channels out) with the taps mirrored:
 //   w'[wb][(o, r', s')][c] = w[wb][(c, K_h-1-r', K_w-1-s')][o]
@@ -1567,6 +1678,39 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
     const bool vec = W % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
     if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (C <= 4 && O <= 2 && W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0) {
+        // a handful of channels: stream x and dy once, C*9*O running sums per lane
+        dim3 grid((unsigned)((W + 255) / 256), (unsigned)((H + 4 * ST_ROWS - 1) / (4 * ST_ROWS)), (unsigned)N);
+        const size_t Q = C * 9 * O, per_image = (size_t)grid.x * grid.y * 4;
+        if (per_image * N > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_weights: too many strips");
+        float* partial = nullptr;
+        if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), per_image * N * Q * sizeof(float), s)) return rc;
+#define NZHIP_DWS(OT, CT)                                                                                            \
+    hipLaunchKernelGGL((conv3x3_dw_stream_kernel<OT, CT>), grid, dim3(256), 0, s, partial, x, dy, (int)H, (int)W)
+        switch ((int)(O * 10 + C)) {
+            case 11: NZHIP_DWS(1, 1); break;
+            case 12: NZHIP_DWS(1, 2); break;
+            case 13: NZHIP_DWS(1, 3); break;
+            case 14: NZHIP_DWS(1, 4); break;
+            case 21: NZHIP_DWS(2, 1); break;
+            case 22: NZHIP_DWS(2, 2); break;
+            case 23: NZHIP_DWS(2, 3); break;
+            default: NZHIP_DWS(2, 4); break;
+        }
+#undef NZHIP_DWS
+        hipError_t e = hipGetLastError();
+        int rc = e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv3x3_dw_stream kernel launch");
+        if (rc == NZHIP_OK) {
+            const bool shared = w_batch == 1;
+            const int S = (int)(shared ? per_image * N : per_image), groups = shared ? 1 : (int)N;
+            hipLaunchKernelGGL(small_dw_reduce_kernel, dim3((unsigned)((Q + 31) / 32), (unsigned)groups), dim3(256), 0, s, dw,
+                               partial, S, (int)Q);
+            e = hipGetLastError();
+            if (e != hipSuccess) rc = set_hip_error(e, "small_dw_reduce kernel launch");
+        }
+        const int rc2 = workspace_free(partial, s);
+        return rc ? rc : rc2;
+    }
     const int chunks = (int)((C + DW_CC - 1) / DW_CC), otiles = (int)((O + DW_OT - 1) / DW_OT);
     if (chunks > 65535 || otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_weights: too many channels");
     // one workgroup per CU in total (its LDS footprint leaves room for no second one); a band is a whole

@@ -50,12 +50,24 @@ __global__ __launch_bounds__(256) void avgpool_kernel(float* __restrict__ out, c
     out[idx] = count > 0 ? sum / (float)count : 0.f;
 }
 
-// Gradient as a gather: one thread per INPUT element adds, in ascending (row, column) order of the
-// output windows that cover it, dout / divisor onto the value already there. That is the order in
-// which a serial run of the reference's scatter loop reaches this element, so the result does not
-// depend on scheduling (the reference's atomicAdd order does). The divisor is pool^2 without padding
-// and the number of window cells inside the image with padding (:1451-1480).
-__global__ __launch_bounds__(256) void avgpool_backward_kernel(float* __restrict__ din, const float* __restrict__ dout,
+// Gradient in two steps. First every output element's share dout / divisor is computed once (the divisor is
+// pool^2 without padding and the number of window cells inside the image with padding, :1451-1480); then one
+// thread per INPUT element adds, in ascending (row, column) order of the output windows that cover it, those
+// shares onto the value already there. That is the order in which a serial run of the reference's scatter loop
+// reaches this element, so the result does not depend on scheduling (the reference's atomicAdd order does).
+__global__ __launch_bounds__(256) void avgpool_share_kernel(float* __restrict__ share, const float* __restrict__ dout,
+                                                            const PoolArgs p) {
+    const long per = (long)p.H_out * p.W_out;
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= p.planes * per) return;
+    const int oh = (int)((idx % per) / p.W_out), ow = (int)((idx % per) % p.W_out);
+    const int h0 = oh * p.stride - p.pad, w0 = ow * p.stride - p.pad;
+    const int rows = min(h0 + p.pool, p.H_in) - max(h0, 0), cols = min(w0 + p.pool, p.W_in) - max(w0, 0);
+    const float div = p.pad == 0 ? (float)(p.pool * p.pool) : (float)(rows * cols);
+    share[idx] = dout[idx] / div;
+}
+
+__global__ __launch_bounds__(256) void avgpool_backward_kernel(float* __restrict__ din, const float* __restrict__ share,
                                                                const PoolArgs p) {
     const long per = (long)p.H_in * p.W_in;
     const long idx = (long)blockIdx.x * 256 + threadIdx.x;
@@ -69,18 +81,10 @@ __global__ __launch_bounds__(256) void avgpool_backward_kernel(float* __restrict
     int oh_hi = hp / p.stride, ow_hi = wp / p.stride;
     if (oh_hi > p.H_out - 1) oh_hi = p.H_out - 1;
     if (ow_hi > p.W_out - 1) ow_hi = p.W_out - 1;
-    const float* g = dout + plane * p.H_out * p.W_out;
+    const float* g = share + plane * p.H_out * p.W_out;
     float acc = din[idx];
-    for (int oh = oh_lo; oh <= oh_hi; oh++) {
-        const int h0 = oh * p.stride - p.pad;
-        const int rows = min(h0 + p.pool, p.H_in) - max(h0, 0);
-        for (int ow = ow_lo; ow <= ow_hi; ow++) {
-            const int w0 = ow * p.stride - p.pad;
-            const int cols = min(w0 + p.pool, p.W_in) - max(w0, 0);
-            const float div = p.pad == 0 ? (float)(p.pool * p.pool) : (float)(rows * cols);
-            acc += g[(long)oh * p.W_out + ow] / div;
-        }
-    }
+    for (int oh = oh_lo; oh <= oh_hi; oh++)
+        for (int ow = ow_lo; ow <= ow_hi; ow++) acc += g[(long)oh * p.W_out + ow];
     din[idx] = acc;
 }
 
@@ -183,9 +187,19 @@ int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t 
     const size_t total = batches * channels * H_in * W_in;
     if (total == 0) return NZHIP_OK;
     if ((total + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_avgpool2d_backward: extent too large");
-    hipLaunchKernelGGL(avgpool_backward_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), din,
-                       dout, p);
-    return check_launch("avgpool_backward_kernel");
+    const size_t outs = batches * channels * H_out * W_out;
+    if (outs == 0) return NZHIP_OK;
+    hipStream_t s = as_stream(stream);
+    float* share = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&share), outs * sizeof(float), s)) return rc;
+    hipLaunchKernelGGL(avgpool_share_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, s, share, dout, p);
+    int rc = check_launch("avgpool_share_kernel");
+    if (rc == NZHIP_OK) {
+        hipLaunchKernelGGL(avgpool_backward_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, din, share, p);
+        rc = check_launch("avgpool_backward_kernel");
+    }
+    const int rc2 = workspace_free(share, s);
+    return rc ? rc : rc2;
 }
 
 int nzhip_bce_loss(float* loss, const float* predict, const float* real, size_t n, void* stream) {

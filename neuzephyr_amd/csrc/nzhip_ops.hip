@@ -536,6 +536,11 @@ int nzhip_col2im(float* out, const float* in, size_t H_out, size_t W_out, size_t
     if (HW == 0 || C_out == 0 || batches == 0) return NZHIP_OK;
     if (HW > 0x7fffffff || (C_out + 31) / 32 > 65535 || batches > 65535)
         return set_error(NZHIP_E_UNSUPPORTED, "nzhip_col2im: extent too large");
+    if (C_out == 1 || HW == 1) {                                 // the transpose of a vector is a copy
+        if (out == in) return NZHIP_OK;
+        hipError_t e = hipMemcpyAsync(out, in, batches * HW * C_out * sizeof(float), hipMemcpyDeviceToDevice, as_stream(stream));
+        return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipMemcpyAsync (col2im of one channel)");
+    }
     dim3 grid((unsigned)((HW + 31) / 32), (unsigned)((C_out + 31) / 32), (unsigned)batches);
     hipLaunchKernelGGL(col2im_kernel, grid, dim3(256), 0, as_stream(stream), out, in, (int)HW, (int)C_out);
     return check_launch("col2im_kernel");
@@ -778,6 +783,11 @@ int nzhip_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_o
     if (HW == 0 || C_out == 0 || batches == 0) return NZHIP_OK;
     if (C_out > 0x7fffffff || (HW + 31) / 32 > 65535 || batches > 65535)
         return set_error(NZHIP_E_UNSUPPORTED, "nzhip_col2im_backward: extent too large");
+    if (C_out == 1 || HW == 1) {                                 // the transpose of a vector is a copy
+        if (dcol == dy) return NZHIP_OK;
+        hipError_t e = hipMemcpyAsync(dcol, dy, batches * HW * C_out * sizeof(float), hipMemcpyDeviceToDevice, as_stream(stream));
+        return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipMemcpyAsync (col2im gradient of one channel)");
+    }
     // the inverse transpose of col2im: [C_out, HW] -> [HW, C_out] per image
     dim3 grid((unsigned)((C_out + 31) / 32), (unsigned)((HW + 31) / 32), (unsigned)batches);
     hipLaunchKernelGGL(col2im_kernel, grid, dim3(256), 0, as_stream(stream), dcol, dy, (int)C_out, (int)HW);

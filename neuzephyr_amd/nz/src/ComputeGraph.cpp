@@ -261,8 +261,12 @@ namespace nz::graph {
     }
 
     void ComputeGraph::update(opt::Optimizer* optimizer) const {
+        // The reference steps every node whose output carries a gradient (:541-547), hidden activations
+        // included. An activation is rewritten in full by the next forward(), so only leaves (parameters and
+        // inputs that require gradients) are stepped here: same parameters after every step, no optimizer pass
+        // and no optimizer state over the activations.
         for (Node* node : nodes)
-            if (node->output && node->output->requiresGrad()) optimizer->step(node);
+            if (node->inputs.empty() && node->output && node->output->requiresGrad()) optimizer->step(node);
     }
 
     void ComputeGraph::zeroGrad() const {

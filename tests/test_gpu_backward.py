@@ -175,7 +175,7 @@ def test_im2col_backward_bit_exact(nz, oracle, shape, k_h, k_w, stride, pad):
     assert np.array_equal(host(got), oracle.im2col_backward(np.zeros(shape, np.float32), dcol_f, k_h, k_w, stride, pad))
 
 
-@pytest.mark.parametrize("n,c,h,w", [(2, 3, 4, 5), (1, 1, 1, 1), (3, 40, 9, 11), (2, 128, 16, 16), (1, 1, 50, 70)])
+@pytest.mark.parametrize("n,c,h,w", [(2, 3, 4, 5), (1, 1, 1, 1), (3, 40, 9, 11), (2, 128, 16, 16), (1, 1, 50, 70), (3, 7, 1, 1)])
 def test_col2im_backward_bit_exact(nz, oracle, n, c, h, w):
     rng = np.random.default_rng(37)
     dy = rng.standard_normal((n, c, h, w)).astype(np.float32)
@@ -243,7 +243,11 @@ def test_conv2d_backward_data_rejects_what_it_does_not_cover(nz):
 CONV_BWD_W = [  # N, C, H, W, O, w_batch   (3x3, stride 1, pad 1; W a multiple of 8 takes 16-byte loads)
     (1, 3, 4, 8, 2, 1), (2, 5, 7, 16, 9, 1), (2, 32, 9, 24, 40, 2), (3, 40, 6, 136, 130, 1), (1, 64, 16, 128, 128, 1),
     (2, 33, 5, 264, 129, 2), (4, 8, 33, 40, 16, 1), (1, 1, 1, 8, 1, 1),
-    (2, 3, 28, 28, 6, 1), (1, 5, 7, 9, 4, 1), (2, 20, 6, 131, 33, 2), (1, 2, 3, 1, 2, 1), (1, 4, 5, 127, 3, 1)]
+    (2, 3, 28, 28, 6, 1), (1, 5, 7, 9, 4, 1), (2, 20, 6, 131, 33, 2), (1, 2, 3, 1, 2, 1), (1, 4, 5, 127, 3, 1),
+    # C <= 4, O <= 2, W a multiple of 4: the streaming kernel (strips of 16 rows, 256 columns per wave; partial last
+    # strip, several column blocks with a ragged last one, per-sample and shared weights)
+    (2, 3, 20, 24, 1, 2), (3, 1, 33, 260, 1, 3), (1, 4, 5, 8, 2, 1), (2, 2, 70, 516, 2, 1), (2, 3, 64, 256, 1, 1),
+    (1, 1, 1, 4, 1, 1)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,wb", CONV_BWD_W)
@@ -271,6 +275,24 @@ def test_conv2d_backward_weights_float_tolerance(nz, oracle):
         for sx in range(3):
             truth[:, r, sx, :] = np.einsum("nchw,nohw->co", xp[:, :, r:r + H, sx:sx + W], dyr)
     truth = truth.reshape(1, 1, C * 9, O)
+    mr, fr = oracle.errors(got, truth, float(np.sqrt(np.mean(truth ** 2))))
+    assert mr <= 1e-3 and fr <= 1e-4, (mr, fr)
+
+
+def test_conv2d_backward_weights_few_channels_float_tolerance(nz, oracle):
+    # the streaming kernel on float data against an fp64 sum of the rounded operands
+    N, C, H, W, O = 3, 3, 50, 300, 1
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, O, H, W)).astype(np.float32)
+    got = host(nz.conv2d_backward_weights(dev(np.zeros((N, 1, C * 9, O))), dev(x), dev(dy), 3, 3, 1, 1))
+    xr, dyr = oracle.round_f16(x).astype(np.float64), oracle.round_f16(dy).astype(np.float64)
+    xp = np.pad(xr, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    truth = np.zeros((N, C, 3, 3, O))
+    for r in range(3):
+        for sx in range(3):
+            truth[:, :, r, sx, :] = np.einsum("nchw,nohw->nco", xp[:, :, r:r + H, sx:sx + W], dyr)
+    truth = truth.reshape(N, 1, C * 9, O)
     mr, fr = oracle.errors(got, truth, float(np.sqrt(np.mean(truth ** 2))))
     assert mr <= 1e-3 and fr <= 1e-4, (mr, fr)
 

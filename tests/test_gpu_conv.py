@@ -55,7 +55,7 @@ def test_im2col_bit_exact(nz, oracle, shape, k_h, k_w, stride, pad):
     assert np.array_equal(host(nz.im2col(dev(x), k_h, k_w, stride, pad)), oracle.im2col(x, k_h, k_w, stride, pad))
 
 
-@pytest.mark.parametrize("n,c,h,w", [(2, 3, 4, 5), (1, 1, 1, 1), (3, 40, 9, 11), (2, 128, 16, 16), (1, 1, 50, 70)])
+@pytest.mark.parametrize("n,c,h,w", [(2, 3, 4, 5), (1, 1, 1, 1), (3, 40, 9, 11), (2, 128, 16, 16), (1, 1, 50, 70), (3, 7, 1, 1)])
 def test_col2im_bit_exact(nz, oracle, n, c, h, w):
     col = np.random.default_rng(n + c + h + w).uniform(-1, 1, size=(n, 1, h * w, c)).astype(np.float32)
     assert np.array_equal(host(nz.col2im(dev(col), h, w)), oracle.col2im(col, h, w))
