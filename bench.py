@@ -466,6 +466,20 @@ def main():
                 extra[name]["frac_fp32_vector_peak"] = w2.flops / ms2 / 1e9 / PEAK_TFLOPS_FP32
             del w2
 
+    if args.workload == "gemm8192" and not args.no_extra:
+        # the reference's README network (batch 10 x 3 x 1024 x 1024) through the C++ nz:: layer, one Adam
+        # training step; a child process of its own (host wall clock around a device synchronisation)
+        exe = os.path.join(ROOT, "neuzephyr_amd", "nz", "examples", "readme_example")
+        if os.path.exists(exe):
+            torch.cuda.empty_cache()
+            import subprocess
+            try:
+                out = subprocess.run([exe, "10", "3"], capture_output=True, text=True, timeout=120)
+                extra["readme_example_training_step"] = (json.loads(out.stdout.strip().splitlines()[-1]) if out.returncode == 0
+                                                         else {"error": out.stderr[-300:]})
+            except (subprocess.TimeoutExpired, ValueError, IndexError) as e:
+                extra["readme_example_training_step"] = {"error": str(e)[:300]}
+
     cpu = None
     if args.workload == "gemm8192" and not args.no_cpu_baseline:
         cpu = cpu_baseline_gemm(orc, *host_ops)

@@ -51,8 +51,10 @@ int main(int argc, char** argv) {
             for (auto& e : v) e = init(gen);
             p->dataInject(v.begin(), v.end());
         }
-        // a fan-in of 260 100 into the Linear layer: every Adam step moves each logit by about fan-in x lr x mean input
-        nz::opt::Adam optimizer(1e-6f, 0.9f, 0.999f);
+        // Adam moves every weight by about lr per step whatever the gradient's size, so a logit of the Linear
+        // layer moves by about fan-in x lr x mean input; keep that near 0.1 (fan-in 260 100 at full size)
+        const size_t fanIn = ((h + 2 - 3 + 1 - 5) / 2 + 1) * ((w + 2 - 3 + 1 - 5) / 2 + 1);
+        nz::opt::Adam optimizer(0.25f / static_cast<float>(fanIn), 0.9f, 0.999f);
         model.forward();
         const float first = model.getLoss();
         auto step = [&] {

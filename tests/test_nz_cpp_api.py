@@ -28,3 +28,17 @@ def test_host_layer_without_gpu():
 @pytest.mark.gpu
 def test_cpp_api_on_gpu():
     _run("test_gpu", 300)
+
+
+@pytest.mark.gpu
+def test_readme_example_runs_and_learns():
+    """The reference's README network on the nz:: layer (reduced image size): finite loss that goes down."""
+    import json
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "neuzephyr_amd", "nz", "examples",
+                       "readme_example")
+    assert os.path.exists(exe), "build the host layer first (python -m neuzephyr_amd.build)"
+    p = subprocess.run([exe, "6", "1", "4", "96", "128"], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, p.stderr[-2000:]
+    line = json.loads(p.stdout.strip().splitlines()[-1])
+    assert line["fused_groups"] == 3
+    assert 0.0 < line["loss_last"] < line["loss_first"]
