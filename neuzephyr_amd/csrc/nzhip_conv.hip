@@ -205,7 +205,10 @@ __device__ __forceinline__ float from_lane_above(float v) {
                                                                  0x130 /* wave_shl:1 */, 0xf, 0xf, false));
 }
 
-template <int O_T, int C_T, bool PIX_BIAS>
+// PIX_BIAS: 0 none or per channel; 1 per pixel with any strides; 2 per pixel in the layout of the
+// reference's Bias node ([pixel][channel], 16-byte aligned), where a lane's 4 pixels x O_T channels are one
+// contiguous run fetched with 16-byte loads.
+template <int O_T, int C_T, int PIX_BIAS>
 __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__ y, const float* __restrict__ x,
                                                              const float* __restrict__ w_ref,
                                                              const float* __restrict__ bias, int H, int W,
@@ -256,10 +259,20 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
             // the bias of the output row a step completes travels with that step's input row, so its
             // wait never drains the rows requested after it
             const int hb = (t >= 2 && t < T) ? out_row(t) : h0;
+            if (PIX_BIAS == 2) {
+                const floatx4* run = reinterpret_cast<const floatx4*>(bias + ((long)hb * W + w0) * O_T);
 #pragma unroll
-            for (int o = 0; o < O_T; o++)
+                for (int k = 0; k < O_T; k++) {
+                    const floatx4 v = run[k];                    // elements 4k..4k+3 of the run: (pixel, channel) = (i / O_T, i % O_T)
 #pragma unroll
-                for (int e = 0; e < 4; e++) bdst[o][e] = bias[((long)hb * W + w0 + e) * bias_sp + (long)o * bias_sc];
+                    for (int j = 0; j < 4; j++) bdst[(4 * k + j) % O_T][(4 * k + j) / O_T] = v[j];
+                }
+            } else {
+#pragma unroll
+                for (int o = 0; o < O_T; o++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) bdst[o][e] = bias[((long)hb * W + w0 + e) * bias_sp + (long)o * bias_sc];
+            }
         }
 #pragma unroll
         for (int c = 0; c < C_T; c++) {
@@ -364,13 +377,18 @@ static int conv_direct(float* y, const float* x, const float* w_ref, const float
     if (vec && C <= 4 && O <= 2 && H >= 8) {
         dim3 sgrid((unsigned)((W + 255) / 256), (unsigned)((H + 4 * ST_ROWS - 1) / (4 * ST_ROWS)), (unsigned)N);
         const bool pixb = bias && bias_sp != 0;
+        // the reference's Bias node: [pixel][channel], so the bias of a lane's 4 pixels is one aligned run
+        const bool pixrun = pixb && bias_sp == (int64_t)O && bias_sc == 1 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
 #define NZHIP_ST(OT, CT)                                                                                             \
     do {                                                                                                             \
-        if (pixb)                                                                                                    \
-            hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT, true>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H, \
+        if (pixrun)                                                                                                  \
+            hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT, 2>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H,  \
+                               (int)W, wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU);                   \
+        else if (pixb)                                                                                               \
+            hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT, 1>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H,  \
                                (int)W, wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU);                   \
         else                                                                                                         \
-            hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT, false>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H, \
+            hipLaunchKernelGGL((conv3x3_stream_kernel<OT, CT, 0>), sgrid, dim3(256), 0, s, y, x, w_ref, bias, (int)H,  \
                                (int)W, wbs, (long)bias_sp, (long)bias_sc, act == NZHIP_ACT_RELU);                   \
     } while (0)
         switch ((int)(O * 10 + C)) {

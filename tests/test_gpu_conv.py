@@ -125,6 +125,22 @@ def test_conv2d_per_pixel_bias_like_the_reference_parameter(nz, oracle):
     assert np.max(np.abs(got - ref)) <= 1e-4
 
 
+@pytest.mark.parametrize("N,C,H,W,O", [(2, 3, 40, 264, 1), (1, 2, 20, 8, 2), (2, 4, 17, 260, 2), (1, 1, 9, 12, 1)])
+def test_stream_conv_with_the_reference_bias_layout_is_bit_exact(nz, oracle, N, C, H, W, O):
+    """Few channels (the streaming kernel) with the bias parameter the reference's Model::Conv2d creates,
+    [1, 1, H*W, O]: fetched as aligned runs of 4 pixels x O channels, or element by element when the bias
+    pointer is not 16-byte aligned; both equal the im2col -> GEMM -> bias -> col2im -> ReLU graph bit for bit."""
+    x = oracle.fill((N, C, H, W), 71, "uniform", 0.0, 1.0)
+    w_ref = oracle.weights_oihw_to_ref(oracle.fill((O, C, 3, 3), 72, "normal", 0.0, 0.3))
+    bias_px = oracle.fill((1, 1, H * W, O), 73, "uniform", -0.5, 0.5)
+    want = np.maximum(oracle.conv2d_graph(x, w_ref, bias_px, 3, 3, 1, 1), 0)
+    got = host(nz.conv2d_forward(dev(x), dev(w_ref), dev(bias_px), 3, 3, 1, 1, bias_strides=(O, 1), relu=True))
+    assert np.array_equal(got, want)
+    shifted = dev(np.concatenate([[0.0], bias_px.reshape(-1)]))[1:]              # 4-byte aligned only
+    got2 = host(nz.conv2d_forward(dev(x), dev(w_ref), shifted, 3, 3, 1, 1, bias_strides=(O, 1), relu=True))
+    assert np.array_equal(got2, want)
+
+
 def test_config4a_conv_64_to_128_channels(nz, oracle):
     N, C, H, W, O = 16, 64, 128, 128, 128
     x = oracle.fill((N, C, H, W), 4, "normal", 0.0, 1.0)
