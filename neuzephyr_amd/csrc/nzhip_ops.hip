@@ -313,6 +313,26 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(nzhip_gemm_desc d, c
     d.C[bn * d.c_stride_n + m * d.ldc + n] = x;
 }
 
+// Very few outputs and many chunks (a Linear layer with a huge fan-in): one wave per output. Lane l adds
+// chunks l, l + 64, ... in ascending order, then the 64 sums are added in a fixed shuffle tree.
+__global__ __launch_bounds__(256) void splitk_reduce_wave_kernel(nzhip_gemm_desc d, const float* __restrict__ P, int S) {
+    const long mn = d.M * d.N;
+    const long bn = blockIdx.y;
+    P += bn * S * mn;
+    const int lane = threadIdx.x & 63;
+    const long t = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= mn) return;                                          // uniform over the wave
+    float x = 0.f;
+    for (int s = lane; s < S; s += 64) x += P[(long)s * mn + t];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off);
+    if (lane != 0) return;
+    const long m = t / d.N, n = t % d.N;
+    if (d.bias) x += d.bias[bn * d.bias_stride_n + m * d.bias_stride_row + n * d.bias_stride_col];
+    if (d.activation == NZHIP_ACT_RELU) x = x > 0.f ? x : 0.f;
+    d.C[bn * d.c_stride_n + m * d.ldc + n] = x;
+}
+
 // The same sum for few chunks and many outputs: one thread per output adds its chunks in ascending
 // order (coalesced along the outputs).
 __global__ __launch_bounds__(256) void splitk_reduce_wide_kernel(nzhip_gemm_desc d, const float* __restrict__ P, int S) {
@@ -383,7 +403,10 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
                 g.bias = nullptr; g.activation = NZHIP_ACT_NONE;
                 int rc = gemm_mfma_dispatch(g, s, 0, d.K);
                 if (rc == NZHIP_OK) {
-                    if (parts > 16 || d.M * d.N < (1 << 18)) {                  // few outputs: spread each over eight lanes
+                    if (parts >= 64 && d.M * d.N <= 4096) {                     // a handful of outputs: one wave each
+                        const long groups = (d.M * d.N + 3) / 4;
+                        hipLaunchKernelGGL(splitk_reduce_wave_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
+                    } else if (parts > 16 || d.M * d.N < (1 << 18)) {           // few outputs: spread each over eight lanes
                         const long groups = (d.M * d.N + 31) / 32;               // 32 outputs x 8 chunk lanes per workgroup
                         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
                     } else {

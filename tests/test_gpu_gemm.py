@@ -94,7 +94,8 @@ def test_skinny_products_are_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans
     assert np.array_equal(got, expect)
 
 
-SPLITK = [(130, 9000, 70), (576, 16384, 128), (64, 4096, 64), (33, 20001, 300), (128, 8192, 129)]
+SPLITK = [(130, 9000, 70), (576, 16384, 128), (64, 4096, 64), (33, 20001, 300), (128, 8192, 129),
+          (10, 70000, 16), (16, 33000, 10)]       # a handful of outputs, hundreds of chunks: one wave per output adds them
 
 
 @pytest.mark.parametrize("M,K,N", SPLITK)
