@@ -243,6 +243,12 @@ int nzhip_bce_loss(float* loss, const float* predict, const float* real, size_t 
  * grad_i = ((p_i - t_i) / (p_i (1 - p_i))) / n, overwriting grad. */
 int nzhip_bce_backward(float* grad, const float* predict, const float* real, size_t n, void* stream);
 
+/* MeanSquaredErrorNode::forward / backward (src/Nodes.cu:785-811; MeanSquaredErrorKernel, MSEBackwardKernel,
+ * src/OperationKernels.cu:579-627): *loss (device memory) = sum_i (p_i - t_i)^2 / n with the summation order of
+ * nzhip_bce_loss; grad_i = 2 (p_i - t_i) / n, overwriting grad. */
+int nzhip_mse_loss(float* loss, const float* predict, const float* real, size_t n, void* stream);
+int nzhip_mse_backward(float* grad, const float* predict, const float* real, size_t n, void* stream);
+
 /* ExpandNode::forward / backward (src/Nodes.cu:585-603; ExpandKernel, CompressKernel, :1282-1301):
  * out[b*n + j] = in[j] for b < batches; and out[j] += sum_b in[b*n + j] in ascending b. */
 int nzhip_expand(float* out, const float* in, size_t n, size_t batches, void* stream);

@@ -20,7 +20,7 @@ EXPORTS = [
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
     "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
-    "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_expand", "nzhip_compress",
+    "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_mse_loss", "nzhip_mse_backward", "nzhip_expand", "nzhip_compress",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
@@ -94,6 +94,8 @@ def load() -> C.CDLL:
     lib.nzhip_avgpool2d_backward.argtypes = [vp, vp] + [sz] * 9 + [vp]
     lib.nzhip_bce_loss.argtypes = [vp, vp, vp, sz, vp]
     lib.nzhip_bce_backward.argtypes = [vp, vp, vp, sz, vp]
+    lib.nzhip_mse_loss.argtypes = [vp, vp, vp, sz, vp]
+    lib.nzhip_mse_backward.argtypes = [vp, vp, vp, sz, vp]
     lib.nzhip_expand.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_compress.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_adam_step.argtypes = [vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, sz, vp]
@@ -412,6 +414,22 @@ def bce_backward(predict, real, stream=None):
     lib = load()
     grad = torch.empty_like(predict)
     check(lib.nzhip_bce_backward(_dev(grad), _dev(predict), _dev(real), predict.numel(), _stream_handle(stream)))
+    return grad
+
+
+def mse_loss(predict, real, stream=None):
+    import torch
+    lib = load()
+    loss = torch.empty(1, dtype=torch.float32, device=predict.device)
+    check(lib.nzhip_mse_loss(_dev(loss), _dev(predict), _dev(real), predict.numel(), _stream_handle(stream)))
+    return loss
+
+
+def mse_backward(predict, real, stream=None):
+    import torch
+    lib = load()
+    grad = torch.empty_like(predict)
+    check(lib.nzhip_mse_backward(_dev(grad), _dev(predict), _dev(real), predict.numel(), _stream_handle(stream)))
     return grad
 
 

@@ -115,6 +115,25 @@ __global__ __launch_bounds__(256) void bce_partial_kernel(float* __restrict__ pa
     if (threadIdx.x == 0) partial[blockIdx.x] = total;
 }
 
+// Mean squared error with the same two-step summation: sum_i (p_i - t_i)^2 / n (MeanSquaredErrorKernel, :579-619).
+__global__ __launch_bounds__(256) void mse_partial_kernel(float* __restrict__ partial, const float* __restrict__ predict,
+                                                          const float* __restrict__ real, long n) {
+    __shared__ float part[4];
+    float s = 0.f;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        const float d = predict[i] - real[i];
+        s += d * d / (float)n;
+    }
+    const float total = block_sum_256(s, part);
+    if (threadIdx.x == 0) partial[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(256) void mse_backward_kernel(float* __restrict__ grad, const float* __restrict__ predict,
+                                                           const float* __restrict__ real, long n) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) grad[i] = 2 * (predict[i] - real[i]) / (float)n;
+}
+
 __global__ __launch_bounds__(256) void bce_final_kernel(float* __restrict__ loss, const float* __restrict__ partial, int m) {
     __shared__ float part[4];
     float s = 0.f;
@@ -202,22 +221,40 @@ int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t 
     return rc ? rc : rc2;
 }
 
-int nzhip_bce_loss(float* loss, const float* predict, const float* real, size_t n, void* stream) {
-    if (!loss || ((!predict || !real) && n)) return set_error(NZHIP_E_INVALID, "nzhip_bce_loss: null pointer");
+static int mean_loss(float* loss, const float* predict, const float* real, size_t n, void* stream, bool bce, const char* who) {
+    if (!loss || ((!predict || !real) && n)) return set_error(NZHIP_E_INVALID, "%s: null pointer", who);
     hipStream_t s = as_stream(stream);
     size_t blocks = (n + 255) / 256;
     if (blocks > (size_t)BCE_MAX_BLOCKS) blocks = BCE_MAX_BLOCKS;
     if (blocks == 0) blocks = 1;                                  // n = 0: the sum of nothing
     float* partial = nullptr;
     if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), blocks * sizeof(float), s)) return rc;
-    hipLaunchKernelGGL(bce_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, s, partial, predict, real, (long)n);
-    int rc = check_launch("bce_partial_kernel");
+    if (bce) hipLaunchKernelGGL(bce_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, s, partial, predict, real, (long)n);
+    else hipLaunchKernelGGL(mse_partial_kernel, dim3((unsigned)blocks), dim3(256), 0, s, partial, predict, real, (long)n);
+    int rc = check_launch("loss partial kernel");
     if (rc == NZHIP_OK) {
         hipLaunchKernelGGL(bce_final_kernel, dim3(1), dim3(256), 0, s, loss, partial, (int)blocks);
         rc = check_launch("bce_final_kernel");
     }
     const int rc2 = workspace_free(partial, s);
     return rc ? rc : rc2;
+}
+
+int nzhip_bce_loss(float* loss, const float* predict, const float* real, size_t n, void* stream) {
+    return mean_loss(loss, predict, real, n, stream, true, "nzhip_bce_loss");
+}
+
+int nzhip_mse_loss(float* loss, const float* predict, const float* real, size_t n, void* stream) {
+    return mean_loss(loss, predict, real, n, stream, false, "nzhip_mse_loss");
+}
+
+int nzhip_mse_backward(float* grad, const float* predict, const float* real, size_t n, void* stream) {
+    if ((!grad || !predict || !real) && n) return set_error(NZHIP_E_INVALID, "nzhip_mse_backward: null pointer");
+    if (n == 0) return NZHIP_OK;
+    if ((n + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_mse_backward: extent too large");
+    hipLaunchKernelGGL(mse_backward_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), grad, predict,
+                       real, (long)n);
+    return check_launch("mse_backward_kernel");
 }
 
 int nzhip_bce_backward(float* grad, const float* predict, const float* real, size_t n, void* stream) {

@@ -55,6 +55,7 @@ namespace nz {
         Node* TargetExpand(Node* input, const data::Tensor::shape_type& shape);
         Node* AvgPool2d(Node* input, data::Tensor::size_type poolSize, data::Tensor::size_type stride,
                         data::Tensor::size_type padding = 0);
+        void MSELoss(Node* input, Node* target);         // terminates the graph (src/Model.cu:307-315)
         void BCELoss(Node* input, Node* target);         // terminates the graph (src/Model.cu:317-325)
         void defaultOutput(Node* input);
     };

@@ -127,6 +127,14 @@ namespace nz {
         return track(new calc::AveragePoolingNode(input, poolSize, stride, padding));
     }
 
+    void Model::MSELoss(Node* input, Node* target) {
+        computeGraph.addNode(input);
+        Node* expanded = TargetExpand(target, input->output->shape());
+        auto* mse = new loss::MeanSquaredErrorNode(input, expanded);
+        hiddenNodes.push_back(mse);
+        computeGraph.addOutput(mse);
+    }
+
     void Model::BCELoss(Node* input, Node* target) {
         computeGraph.addNode(input);
         Node* expanded = TargetExpand(target, input->output->shape());

@@ -234,6 +234,23 @@ namespace nz::nodes {
     }
 
     namespace loss {
+        MeanSquaredErrorNode::MeanSquaredErrorNode(Node* input1, Node* input2) : OutputNode(input1) {
+            if (input1->output->shape() != input2->output->shape())
+                throw std::invalid_argument("input1 and input2 should have the same shape");
+            inputs.push_back(input2);
+            type = "MeanSquaredError";
+        }
+
+        void MeanSquaredErrorNode::forward() {                         // src/Nodes.cu:785-802
+            OutputNode::forward();
+            loss = iMeanSquaredError(inputs[0]->output->data(), inputs[1]->output->data(), output->size());
+        }
+
+        void MeanSquaredErrorNode::backward() {                        // src/Nodes.cu:804-811
+            if (output->requiresGrad())
+                iMSEBackward(output->grad(), inputs[0]->output->data(), inputs[1]->output->data(), output->size());
+        }
+
         BinaryCrossEntropyNode::BinaryCrossEntropyNode(Node* input1, Node* input2) : OutputNode(input1) {
             if (input1->output->shape() != input2->output->shape())
                 throw std::invalid_argument("input1 and input2 should have the same shape");

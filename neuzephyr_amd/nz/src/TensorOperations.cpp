@@ -139,16 +139,24 @@ namespace nz::data {
                                           nzhip_default_stream()));
     }
 
-    float iBinaryCrossEntropy(float* predict, float* real, const size_t n) {
+    static float meanLoss(float* predict, float* real, const size_t n, const bool bce) {
         void* dev = nullptr;
         NZ_CHECK(nzhip_malloc(&dev, sizeof(float)));
         float host = 0.f;
-        int rc = nzhip_bce_loss(static_cast<float*>(dev), predict, real, n, nzhip_default_stream());
+        int rc = bce ? nzhip_bce_loss(static_cast<float*>(dev), predict, real, n, nzhip_default_stream())
+                     : nzhip_mse_loss(static_cast<float*>(dev), predict, real, n, nzhip_default_stream());
         if (rc == 0) rc = nzhip_memcpy_d2h(&host, dev, sizeof(float));      // blocks until the value is here
         const int rc2 = nzhip_free(dev);
         NZ_CHECK(rc);
         NZ_CHECK(rc2);
         return host;
+    }
+
+    float iBinaryCrossEntropy(float* predict, float* real, const size_t n) { return meanLoss(predict, real, n, true); }
+    float iMeanSquaredError(float* predict, float* real, const size_t n) { return meanLoss(predict, real, n, false); }
+
+    void iMSEBackward(float* grad, float* predict, float* real, const size_t n) {
+        NZ_CHECK(nzhip_mse_backward(grad, predict, real, n, nzhip_default_stream()));
     }
 
     void iBCEBackward(float* grad, float* predict, float* real, const size_t n) {

@@ -759,6 +759,60 @@ TEST(NodeLoss, BCEForwardBackward) {
     EXPECT_THROW(BinaryCrossEntropyNode bad(&input1, &other), std::invalid_argument);
 }
 
+TEST(NodeLoss, MSEForwardBackward) {                       // test/Test.cpp:1872-1935
+    const size_t n = 2, c = 3, h = 12, w = 5, total = n * c * h * w;
+    auto predict = randomVec(total, 107, 0.1f, 0.9f), target = randomVec(total, 108, 0.1f, 0.9f);
+    double lossWant = 0;
+    std::vector<double> gradWant(total);
+    for (size_t i = 0; i < total; i++) {
+        lossWant += ((double)predict[i] - target[i]) * ((double)predict[i] - target[i]);
+        gradWant[i] = 2 * ((double)predict[i] - target[i]) / total;
+    }
+    lossWant /= total;
+    InputNode input1({n, c, h, w}, true), input2({n, c, h, w});
+    input1.dataInject(predict.begin(), predict.end());
+    input2.dataInject(target.begin(), target.end());
+    MeanSquaredErrorNode mse(&input1, &input2);
+    mse.forward();
+    EXPECT_TRUE(std::fabs(mse.getLoss() - lossWant) < 1e-5 * lossWant);
+    mse.backward();
+    EXPECT_TRUE(closeTo(input1.output->hostGrad(), gradWant, 1e-6));
+}
+
+// Linear -> ReLU -> Linear with an MSE loss against a target given once for the whole batch
+struct RegressionModel : nz::Model {
+    InputNode input, target;
+    RegressionModel() : input({8, 1, 64, 1}), target({1, 1, 4, 1}) {
+        Node* x = Linear(&input, 32);
+        x = ReLU(x);
+        x = Linear(x, 4);
+        MSELoss(x, &target);
+    }
+};
+
+TEST(Model, MSELossTrainingLowersTheLoss) {
+    RegressionModel m;
+    auto x = randomVec(8 * 64, 131, -1.f, 1.f);
+    m.input.dataInject(x.begin(), x.end());
+    m.target.dataInject({0.5f, -0.25f, 1.0f, 0.0f});
+    unsigned seed = 140;
+    for (auto* p : m.parameters()) {
+        auto v = randomVec(p->output->size(), seed++, -0.2f, 0.2f);
+        p->dataInject(v.begin(), v.end());
+    }
+    nz::opt::SGD optimizer(0.05f);
+    m.forward();
+    float before = m.getLoss();
+    EXPECT_TRUE(before > 0.f);
+    for (int step = 0; step < 10; ++step) {
+        m.backward();
+        m.update(&optimizer);
+        m.forward();
+        EXPECT_TRUE(m.getLoss() < before);
+        before = m.getLoss();
+    }
+}
+
 TEST(NodeBasic, ExpandForwardBackward) {
     const size_t c = 2, h = 3, w = 4, batch = 5, per = c * h * w;
     auto x = randomVec(per, 105, -1.f, 1.f), g = randomVec(per * batch, 106, -1.f, 1.f);

@@ -708,6 +708,16 @@ void nzo_bce_backward(float* grad, const float* predict, const float* real, size
     for (size_t i = 0; i < n; i++) grad[i] = ((predict[i] - real[i]) / (predict[i] * (1 - predict[i]))) / (float)n;
 }
 
+float nzo_mse_loss(const float* predict, const float* real, size_t n) {
+    float loss = 0.0f;
+    for (size_t i = 0; i < n; i++) loss += (predict[i] - real[i]) * (predict[i] - real[i]);
+    return n ? loss / (float)n : 0.0f;
+}
+
+void nzo_mse_backward(float* grad, const float* predict, const float* real, size_t n) {
+    for (size_t i = 0; i < n; i++) grad[i] = 2 * (predict[i] - real[i]) / (float)n;
+}
+
 void nzo_expand(float* out, const float* in, size_t n, size_t batches) {
     for (size_t i = 0; i < n * batches; i++) out[i] = in[i % n];
 }

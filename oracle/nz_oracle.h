@@ -175,6 +175,11 @@ void nzo_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t s
 float nzo_bce_loss(const float* predict, const float* real, size_t n);
 /* BCEBackwardKernel (:692-699; test/Test.cpp:1985-1987): ((p - t) / (p (1 - p))) / n. */
 void nzo_bce_backward(float* grad, const float* predict, const float* real, size_t n);
+/* Mean squared error as the reference's test states it (test/Test.cpp:1890-1893): squared differences summed in
+ * ascending order, then divided by n (the kernel, :579-619, divides every term and sums in a tree: last bits
+ * PARITY UNPINNED, the test compares at 1e-2); MSEBackwardKernel (:621-627): 2 (p - t) / n. */
+float nzo_mse_loss(const float* predict, const float* real, size_t n);
+void nzo_mse_backward(float* grad, const float* predict, const float* real, size_t n);
 /* ExpandKernel / CompressKernel (:1282-1301), the latter run serially in ascending index. */
 void nzo_expand(float* out, const float* in, size_t n, size_t batches);
 void nzo_compress(float* out, const float* in, size_t n, size_t batches);

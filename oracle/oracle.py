@@ -40,9 +40,11 @@ def _load() -> C.CDLL:
     order = ["libnz_oracle_v4.so", "libnz_oracle_v3.so"] if all(f in flags for f in _AVX512) else ["libnz_oracle_v3.so"]
     if os.environ.get("NZ_ORACLE_ISA") == "v3":
         order = ["libnz_oracle_v3.so"]
+    sources = [os.path.join(_HERE, f) for f in ("nz_oracle.c", "nz_oracle.h", "Makefile")]
+    newest = max(os.path.getmtime(f) for f in sources if os.path.exists(f))
     for name in order:
         path = os.path.join(_HERE, name)
-        if os.path.exists(path):
+        if os.path.exists(path) and os.path.getmtime(path) >= newest:       # built, and not older than its sources
             return C.CDLL(path)
     build()
     return C.CDLL(os.path.join(_HERE, order[-1]))
@@ -89,6 +91,8 @@ _avgpool = _sig("nzo_avgpool2d", None, _f32p, _f32p, *([_sz] * 9))
 _avgpool_bwd = _sig("nzo_avgpool2d_backward", None, _f32p, _f32p, *([_sz] * 9))
 _bce = _sig("nzo_bce_loss", C.c_float, _f32p, _f32p, _sz)
 _bce_bwd = _sig("nzo_bce_backward", None, _f32p, _f32p, _f32p, _sz)
+_mse = _sig("nzo_mse_loss", C.c_float, _f32p, _f32p, _sz)
+_mse_bwd = _sig("nzo_mse_backward", None, _f32p, _f32p, _f32p, _sz)
 _expand = _sig("nzo_expand", None, _f32p, _f32p, _sz, _sz)
 _compress = _sig("nzo_compress", None, _f32p, _f32p, _sz, _sz)
 _sgd = _sig("nzo_sgd_step", None, _f32p, _f32p, C.c_float, _sz)
@@ -351,6 +355,18 @@ def bce_backward(predict: np.ndarray, real: np.ndarray) -> np.ndarray:
     p, t = _c(predict), _c(real)
     g = np.empty_like(p)
     _bce_bwd(g.reshape(-1), p.reshape(-1), t.reshape(-1), p.size)
+    return g
+
+
+def mse_loss(predict: np.ndarray, real: np.ndarray) -> float:
+    p, t = _c(predict), _c(real)
+    return float(_mse(p.reshape(-1), t.reshape(-1), p.size))
+
+
+def mse_backward(predict: np.ndarray, real: np.ndarray) -> np.ndarray:
+    p, t = _c(predict), _c(real)
+    g = np.empty_like(p)
+    _mse_bwd(g.reshape(-1), p.reshape(-1), t.reshape(-1), p.size)
     return g
 
 

@@ -71,6 +71,17 @@ def test_bce_loss_and_backward(nz, oracle):
     assert np.array_equal(a, b)
 
 
+def test_mse_loss_and_backward(nz, oracle):
+    rng = np.random.default_rng(13)
+    for n in (1, 9, 360, 70001):
+        p = rng.uniform(-2, 2, n).astype(np.float32)
+        t = rng.uniform(-2, 2, n).astype(np.float32)
+        truth = float(np.mean((p.astype(np.float64) - t.astype(np.float64)) ** 2))
+        got = float(host(nz.mse_loss(dev(p), dev(t)))[0])
+        assert abs(got - truth) <= 1e-5 * truth and abs(oracle.mse_loss(p, t) - truth) <= 1e-4 * truth, n
+        assert np.array_equal(host(nz.mse_backward(dev(p), dev(t))), oracle.mse_backward(p, t)), n
+
+
 def test_expand_and_compress_bit_exact(nz, oracle):
     rng = np.random.default_rng(12)
     x = rng.normal(size=(1, 3, 16, 5)).astype(np.float32)

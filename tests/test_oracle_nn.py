@@ -84,6 +84,25 @@ def test_bce_loss_and_gradient(oracle):
     assert np.array_equal(oracle.bce_backward(t, t), np.zeros_like(t))
 
 
+def test_mse_loss_and_gradient(oracle):
+    rng = np.random.default_rng(8)
+    p = rng.uniform(0.1, 0.9, (2, 3, 12, 5)).astype(np.float32)       # the reference test's shape (Test.cpp:1873-1876)
+    t = rng.uniform(0.1, 0.9, p.shape).astype(np.float32)
+    p64, t64 = p.astype(np.float64), t.astype(np.float64)
+    want = float(np.mean((p64 - t64) ** 2))
+    assert abs(oracle.mse_loss(p, t) - want) <= 1e-5 * want
+    assert oracle.mse_loss(t, t) == 0.0
+    assert abs(oracle.mse_loss(np.full(7, 3.0, np.float32), np.full(7, 1.0, np.float32)) - 4.0) < 1e-6
+    g = oracle.mse_backward(p, t)
+    assert np.allclose(g, 2 * (p64 - t64) / p.size, rtol=1e-6, atol=0)
+    # the loss is quadratic: its gradient is exact under central differences
+    hi, lo = p64.copy(), p64.copy()
+    hi[1, 2, 3, 4] += 1e-3
+    lo[1, 2, 3, 4] -= 1e-3
+    fd = (np.mean((hi - t64) ** 2) - np.mean((lo - t64) ** 2)) / 2e-3
+    assert abs(g[1, 2, 3, 4] - fd) <= 1e-5 * abs(fd)
+
+
 def test_expand_and_compress(oracle):
     rng = np.random.default_rng(6)
     x = rng.integers(-9, 10, (1, 2, 3, 4)).astype(np.float32)
