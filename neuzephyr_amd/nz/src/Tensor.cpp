@@ -142,7 +142,8 @@ namespace nz::data {
     }
 
     void Tensor::zeroGrad() const {
-        if (_requires_grad && _size) NZ_CHECK(nzhip_memset(grad(), 0, _size * sizeof(value_type)));
+        // a gradient nobody has asked for yet is not allocated, and is cleared when it is (grad())
+        if (_requires_grad && _size && _grad) NZ_CHECK(nzhip_memset(_grad, 0, _size * sizeof(value_type)));
     }
 
     void Tensor::clear() const {
