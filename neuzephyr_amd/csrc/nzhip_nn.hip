@@ -20,18 +20,19 @@ static int check_launch(const char* what) {
 struct PoolArgs {
     int pool, stride, pad;
     int H_in, W_in, H_out, W_out;
-    long planes;            // batches * channels
+    int wblocks, wblocks_in;    // 256-column blocks per output row / per input row
+    long planes;                // batches * channels
 };
 
 // One thread per output element: the window is summed row by row, left to right (the reference's
 // loop order), and divided by the number of window cells inside the image.
 __global__ __launch_bounds__(256) void avgpool_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                       const PoolArgs p) {
-    const long per = (long)p.H_out * p.W_out;
-    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= p.planes * per) return;
-    const long plane = idx / per;
-    const int h = (int)((idx % per) / p.W_out), w = (int)((idx % per) % p.W_out);
+    // grid: x = (output row, 256-column block), y and z = plane; nothing here divides per thread
+    const int h = blockIdx.x / p.wblocks, w = (blockIdx.x % p.wblocks) * 256 + threadIdx.x;
+    const long plane = blockIdx.y + (long)gridDim.y * blockIdx.z;
+    if (w >= p.W_out || plane >= p.planes) return;
+    const long idx = (plane * p.H_out + h) * p.W_out + w;
     const int h0 = h * p.stride - p.pad, w0 = w * p.stride - p.pad;
     const float* src = in + plane * p.H_in * p.W_in;
     float sum = 0.f;
@@ -57,10 +58,10 @@ __global__ __launch_bounds__(256) void avgpool_kernel(float* __restrict__ out, c
 // reaches this element, so the result does not depend on scheduling (the reference's atomicAdd order does).
 __global__ __launch_bounds__(256) void avgpool_share_kernel(float* __restrict__ share, const float* __restrict__ dout,
                                                             const PoolArgs p) {
-    const long per = (long)p.H_out * p.W_out;
-    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= p.planes * per) return;
-    const int oh = (int)((idx % per) / p.W_out), ow = (int)((idx % per) % p.W_out);
+    const int oh = blockIdx.x / p.wblocks, ow = (blockIdx.x % p.wblocks) * 256 + threadIdx.x;
+    const long plane = blockIdx.y + (long)gridDim.y * blockIdx.z;
+    if (ow >= p.W_out || plane >= p.planes) return;
+    const long idx = (plane * p.H_out + oh) * p.W_out + ow;
     const int h0 = oh * p.stride - p.pad, w0 = ow * p.stride - p.pad;
     const int rows = min(h0 + p.pool, p.H_in) - max(h0, 0), cols = min(w0 + p.pool, p.W_in) - max(w0, 0);
     const float div = p.pad == 0 ? (float)(p.pool * p.pool) : (float)(rows * cols);
@@ -69,16 +70,19 @@ __global__ __launch_bounds__(256) void avgpool_share_kernel(float* __restrict__ 
 
 __global__ __launch_bounds__(256) void avgpool_backward_kernel(float* __restrict__ din, const float* __restrict__ share,
                                                                const PoolArgs p) {
-    const long per = (long)p.H_in * p.W_in;
-    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= p.planes * per) return;
-    const long plane = idx / per;
-    const int h = (int)((idx % per) / p.W_in), w = (int)((idx % per) % p.W_in);
-    // windows with oh*stride - pad <= h <= oh*stride - pad + pool - 1
+    // grid: x = (input row, 256-column block; wblocks_in blocks per row), y and z = plane
+    const int h = blockIdx.x / p.wblocks_in, w = (blockIdx.x % p.wblocks_in) * 256 + threadIdx.x;
+    const long plane = blockIdx.y + (long)gridDim.y * blockIdx.z;
+    if (w >= p.W_in || plane >= p.planes) return;
+    const long idx = (plane * p.H_in + h) * p.W_in + w;
+    // windows with oh*stride - pad <= h <= oh*stride - pad + pool - 1. The row bounds are the same for the
+    // whole workgroup; the column bounds divide in fp32, which is exact for these magnitudes (< 2^24).
     const int hp = h + p.pad, wp = w + p.pad;
     int oh_lo = hp - p.pool + 1 <= 0 ? 0 : (hp - p.pool + p.stride) / p.stride;
-    int ow_lo = wp - p.pool + 1 <= 0 ? 0 : (wp - p.pool + p.stride) / p.stride;
-    int oh_hi = hp / p.stride, ow_hi = wp / p.stride;
+    int oh_hi = hp / p.stride;
+    const float fs = (float)p.stride;
+    int ow_lo = wp - p.pool + 1 <= 0 ? 0 : (int)((float)(wp - p.pool + p.stride) / fs);
+    int ow_hi = (int)((float)wp / fs);
     if (oh_hi > p.H_out - 1) oh_hi = p.H_out - 1;
     if (ow_hi > p.W_out - 1) ow_hi = p.W_out - 1;
     const float* g = share + plane * p.H_out * p.W_out;
@@ -177,7 +181,18 @@ static int pool_args(PoolArgs& p, size_t pool, size_t stride, size_t pad, size_t
     p.pool = (int)pool; p.stride = (int)stride; p.pad = (int)pad;
     p.H_in = (int)H_in; p.W_in = (int)W_in; p.H_out = (int)H_out; p.W_out = (int)W_out;
     p.planes = (long)(batches * channels);
+    p.wblocks = (int)((W_out + 255) / 256);
+    p.wblocks_in = (int)((W_in + 255) / 256);
+    if (W_in + pad + stride >= (1u << 24) || (size_t)p.wblocks_in * H_in > 0x7fffffffull ||
+        (size_t)p.wblocks * H_out > 0x7fffffffull || batches * channels > 65535ull * 65535ull)
+        return set_error(NZHIP_E_UNSUPPORTED, "%s: extent too large", who);
     return NZHIP_OK;
+}
+
+// x = rows x column blocks, planes folded into y (up to 65535) and z
+static dim3 pool_grid(int wblocks, int rows, long planes) {
+    const long gy = planes < 65535 ? planes : 65535;
+    return dim3((unsigned)((long)wblocks * rows), (unsigned)gy, (unsigned)((planes + gy - 1) / gy));
 }
 
 }  // namespace nzhip
@@ -193,8 +208,7 @@ int nzhip_avgpool2d(float* out, const float* in, size_t pool, size_t stride, siz
     if (int rc = pool_args(p, pool, stride, pad, batches, channels, H_in, W_in, H_out, W_out, "nzhip_avgpool2d")) return rc;
     const size_t total = batches * channels * H_out * W_out;
     if (total == 0) return NZHIP_OK;
-    if ((total + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_avgpool2d: extent too large");
-    hipLaunchKernelGGL(avgpool_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, as_stream(stream), out, in, p);
+    hipLaunchKernelGGL(avgpool_kernel, pool_grid(p.wblocks, p.H_out, p.planes), dim3(256), 0, as_stream(stream), out, in, p);
     return check_launch("avgpool_kernel");
 }
 
@@ -205,16 +219,15 @@ int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t 
     if (int rc = pool_args(p, pool, stride, pad, batches, channels, H_in, W_in, H_out, W_out, "nzhip_avgpool2d_backward")) return rc;
     const size_t total = batches * channels * H_in * W_in;
     if (total == 0) return NZHIP_OK;
-    if ((total + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_avgpool2d_backward: extent too large");
     const size_t outs = batches * channels * H_out * W_out;
     if (outs == 0) return NZHIP_OK;
     hipStream_t s = as_stream(stream);
     float* share = nullptr;
     if (int rc = workspace_alloc(reinterpret_cast<void**>(&share), outs * sizeof(float), s)) return rc;
-    hipLaunchKernelGGL(avgpool_share_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, s, share, dout, p);
+    hipLaunchKernelGGL(avgpool_share_kernel, pool_grid(p.wblocks, p.H_out, p.planes), dim3(256), 0, s, share, dout, p);
     int rc = check_launch("avgpool_share_kernel");
     if (rc == NZHIP_OK) {
-        hipLaunchKernelGGL(avgpool_backward_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, din, share, p);
+        hipLaunchKernelGGL(avgpool_backward_kernel, pool_grid(p.wblocks_in, p.H_in, p.planes), dim3(256), 0, s, din, share, p);
         rc = check_launch("avgpool_backward_kernel");
     }
     const int rc2 = workspace_free(share, s);
