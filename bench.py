@@ -436,7 +436,7 @@ def main():
             traffic = json.load(f).get(args.workload, {}).get("bytes_per_step")
     except OSError:
         pass
-    scope = ("whole step = every kernel the call launches (for gemm8192: two fp16 rounding kernels + the MFMA "
+    scope = ("whole step = every kernel the call launches (for gemm8192: the fp16 rounding kernel + the MFMA "
              "kernel); per-kernel durations are in profiles/")
     if wl.bound == "mfma":
         roofline = {"bound": "mfma", "achieved": tflops, "peak": PEAK_TFLOPS_FP16, "unit": "TFLOP/s",
