@@ -25,6 +25,9 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int waves = 
 // Bandwidth-bound kernels for M <= 8 (nzhip_skinny.hip).
 int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
 bool gemm_skinny_applicable(const nzhip_gemm_desc& d);
+// short contraction (K <= 32), one extent <= 16, the other long: streamed, one lane per long index
+bool gemm_thin_applicable(const nzhip_gemm_desc& d);
+int gemm_thin_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
 
 // Stream-ordered workspace from the caching allocator (nzhip_runtime.cpp).
 int workspace_alloc(void** ptr, size_t bytes, hipStream_t stream);

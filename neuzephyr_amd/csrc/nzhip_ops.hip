@@ -366,6 +366,7 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
         hipLaunchKernelGGL(fill_bias_act_kernel, grid, dim3(256), 0, s, d);
         return check_launch("fill_bias_act_kernel");
     }
+    if (gemm_thin_applicable(d)) return gemm_thin_dispatch(d, s);
     if (gemm_skinny_applicable(d)) return gemm_skinny_dispatch(d, s);
     // One matrix with few output tiles (weight gradients with K = batch x pixels, mid-size products):
     // a workgroup's k loop is latency-bound (about 0.55 us per 32-wide k tile with 16-byte loads, 2 us

@@ -321,4 +321,88 @@ int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream) {
     return rc;
 }
 
+// ---- thin products: a short contraction and one narrow extent --------------------------------------
+// K <= 32 and min(M, N) <= 16 with the other extent long (a Linear layer with a huge fan-in seen from its
+// backward: dW[16 x 260100] = dy[16 x batch] x^T, dx[260100 x batch] = W^T dy). The output and the long
+// operand are streamed once; a 128 x 128 MFMA tile would be empty to seven eighths. One lane owns one
+// index l of the long extent and keeps the T <= 16 outputs of its row (column) in registers; the narrow
+// operand sits in LDS, rounded, and is read as broadcasts. Every output is one chain of FMAs over
+// ascending k of fp16-rounded operands: the k-ascending fp32 sum of the CPU restatement, bit for bit.
+struct ThinArgs {
+    const float* X;         // long operand: element (l, k) at X[l * x_sl + k * x_sk]
+    const float* S;         // narrow operand: element (t, k) at S[t * s_st + k * s_sk]
+    float* C;               // element (l, t) at C[l * c_sl + t * c_st]
+    const float* bias;      // element (l, t) at bias[l * b_sl + t * b_st], or null
+    long L, x_sl, x_sk, s_st, s_sk, c_sl, c_st, b_sl, b_st;
+    int T, K, relu;
+};
+
+constexpr int THIN_MAX_T = 16, THIN_MAX_K = 32;
+
+template <int T_T>
+__global__ __launch_bounds__(256) void gemm_thin_kernel(const ThinArgs p) {
+    __shared__ float s_lds[THIN_MAX_T * THIN_MAX_K];             // [t][k], rounded to fp16
+    for (int i = threadIdx.x; i < T_T * p.K; i += 256) {
+        const int t = i / p.K, k = i % p.K;
+        s_lds[t * THIN_MAX_K + k] = t < p.T ? (float)(_Float16)p.S[t * p.s_st + k * p.s_sk] : 0.f;
+    }
+    __syncthreads();
+    const long l = (long)blockIdx.x * 256 + threadIdx.x;
+    if (l >= p.L) return;
+    float acc[T_T];
+#pragma unroll
+    for (int t = 0; t < T_T; t++) acc[t] = 0.f;
+    const float* xr = p.X + l * p.x_sl;
+    for (int k = 0; k < p.K; k++) {
+        const float x = (float)(_Float16)xr[k * p.x_sk];
+#pragma unroll
+        for (int t = 0; t < T_T; t++) acc[t] = __builtin_fmaf(x, s_lds[t * THIN_MAX_K + k], acc[t]);
+    }
+#pragma unroll
+    for (int t = 0; t < T_T; t++) {
+        if (t >= p.T) break;
+        float v = acc[t];
+        if (p.bias) v += p.bias[l * p.b_sl + t * p.b_st];
+        if (p.relu) v = v > 0.f ? v : 0.f;
+        p.C[l * p.c_sl + t * p.c_st] = v;
+    }
+}
+
+bool gemm_thin_applicable(const nzhip_gemm_desc& d) {
+    static const char* env = getenv("NZHIP_THIN");               // benchmarking only: 0 switches the route off
+    if (env && atoi(env) == 0) return false;
+    const int64_t lo = d.M < d.N ? d.M : d.N, hi = d.M < d.N ? d.N : d.M;
+    return d.batch_n * d.batch_c == 1 && d.K >= 1 && d.K <= THIN_MAX_K && lo <= THIN_MAX_T && hi >= 2048;
+}
+
+int gemm_thin_dispatch(const nzhip_gemm_desc& d, hipStream_t stream) {
+    ThinArgs p;
+    const bool long_n = d.N >= d.M;
+    // strides of A(m, k) and B(k, n) as stored
+    const long a_sm = d.a_layout == NZHIP_LAYOUT_ROW ? d.lda : 1, a_sk = d.a_layout == NZHIP_LAYOUT_ROW ? 1 : d.lda;
+    const long b_sk = d.b_layout == NZHIP_LAYOUT_ROW ? d.ldb : 1, b_sn = d.b_layout == NZHIP_LAYOUT_ROW ? 1 : d.ldb;
+    if (long_n) {
+        p.X = d.B; p.x_sl = b_sn; p.x_sk = b_sk;
+        p.S = d.A; p.s_st = a_sm; p.s_sk = a_sk;
+        p.L = d.N; p.T = (int)d.M;
+        p.c_sl = 1; p.c_st = d.ldc;
+        p.b_sl = d.bias_stride_col; p.b_st = d.bias_stride_row;
+    } else {
+        p.X = d.A; p.x_sl = a_sm; p.x_sk = a_sk;
+        p.S = d.B; p.s_st = b_sn; p.s_sk = b_sk;
+        p.L = d.M; p.T = (int)d.N;
+        p.c_sl = d.ldc; p.c_st = 1;
+        p.b_sl = d.bias_stride_row; p.b_st = d.bias_stride_col;
+    }
+    p.C = d.C; p.bias = d.bias; p.K = (int)d.K; p.relu = d.activation == NZHIP_ACT_RELU;
+    const long blocks = (p.L + 255) / 256;
+    if (blocks > 0x7fffffffL) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_gemm: long extent too large");
+    dim3 grid((unsigned)blocks);
+    if (p.T <= 4) hipLaunchKernelGGL(gemm_thin_kernel<4>, grid, dim3(256), 0, stream, p);
+    else if (p.T <= 8) hipLaunchKernelGGL(gemm_thin_kernel<8>, grid, dim3(256), 0, stream, p);
+    else hipLaunchKernelGGL(gemm_thin_kernel<16>, grid, dim3(256), 0, stream, p);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "thin GEMM kernel launch");
+}
+
 }  // namespace nzhip

@@ -276,6 +276,28 @@ def test_batched_products_with_few_tiles_split_the_contraction(nz, sa, sb):
     assert np.array_equal(host(nz.tensorcore_gemm(dev(A), dev(B))), expect)
 
 
+@pytest.mark.parametrize("M,K,N", [(16, 10, 5000), (5000, 16, 10), (3, 32, 4099), (2500, 1, 16), (9, 7, 2048), (2049, 31, 13)])
+@pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
+def test_thin_products_short_contraction_one_narrow_extent(nz, oracle, M, K, N, a_trans, b_trans):
+    """K <= 32, one extent <= 16 and the other long (Linear-layer gradients with a huge fan-in): the streaming
+    kernel, exact on integers with bias and ReLU, and bit-identical to the k-ascending oracle on float data."""
+    rng = np.random.default_rng(M + 3 * K + 7 * N)
+    A = rng.integers(-4, 5, size=(K, M) if a_trans else (M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, size=(N, K) if b_trans else (K, N)).astype(np.float32)
+    bias = rng.integers(-5, 6, size=(M, N)).astype(np.float32)
+    P = (A.T if a_trans else A).astype(np.int64) @ (B.T if b_trans else B).astype(np.int64)
+    got = host(nz.gemm(dev(A), dev(B), a_trans=a_trans, b_trans=b_trans, bias=dev(bias), bias_strides=(N, 1), relu=True))
+    assert np.array_equal(got, np.maximum(P + bias, 0).astype(np.float32))
+    Af = rng.standard_normal(A.shape).astype(np.float32)
+    Bf = rng.standard_normal(B.shape).astype(np.float32)
+    want = oracle.gemm(np.ascontiguousarray(Af.T if a_trans else Af), np.ascontiguousarray(Bf.T if b_trans else Bf))
+    assert np.array_equal(host(nz.gemm(dev(Af), dev(Bf), a_trans=a_trans, b_trans=b_trans)), want)
+    # accumulate in place: the bias operand is the output itself
+    out = dev(bias)
+    nz.gemm(dev(A), dev(B), a_trans=a_trans, b_trans=b_trans, bias=out, bias_strides=(N, 1), out=out)
+    assert np.array_equal(host(out), (P + bias).astype(np.float32))
+
+
 def test_bias_forms_and_relu_special_values(nz, oracle):
     M, K, N = 40, 24, 52
     rng = np.random.default_rng(1)
