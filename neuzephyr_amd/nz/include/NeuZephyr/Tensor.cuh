@@ -46,6 +46,8 @@ namespace nz::data {
 
         [[nodiscard]] value_type* data() const;                    // device pointer (allocates on first use)
         [[nodiscard]] value_type* grad() const;                    // throws std::runtime_error without gradients
+        // the same buffer for a caller that is about to write EVERY element of it (contents undefined on return)
+        [[nodiscard]] value_type* gradOverwrite() const;
         [[nodiscard]] std::vector<value_type> hostData() const;    // blocks
         [[nodiscard]] std::vector<value_type> hostGrad() const;    // blocks
 
@@ -85,6 +87,9 @@ namespace nz::data {
         shape_type _shape;
         mutable value_type* _data;
         mutable value_type* _grad;
+        // zeroGrad() only notes that the gradient is zero; the clear runs when somebody reads or adds to it
+        // (grad()) and is skipped when the next user overwrites every element (gradOverwrite())
+        mutable bool _gradZeroPending = false;
         bool _requires_grad;
     };
 }

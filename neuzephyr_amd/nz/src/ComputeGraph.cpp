@@ -145,8 +145,9 @@ namespace nz::graph {
                         back = [=] {
                             float* dZ = last->output->grad();
                             if (relu) {
-                                iReLUBackward(c2i->output->grad(), last->output->data(), dZ, last->output->size());
-                                dZ = c2i->output->grad();
+                                float* masked = c2i->output->gradOverwrite();     // every element written
+                                iReLUBackward(masked, last->output->data(), dZ, last->output->size());
+                                dZ = masked;
                             }
                             const bool needW = rhs->output->requiresGrad();
                             const bool needB = biasNode && biasNode->output->requiresGrad();
@@ -155,7 +156,7 @@ namespace nz::graph {
                                                                                  xs[1], xs[2], xs[3], O, i2c->kernelHeight,
                                                                                  i2c->kernelWidth, i2c->stride, i2c->padding, ws[0]);
                             if ((needW && !directW) || needB)
-                                iCol2imgBackward(pre->output->grad(), dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
+                                iCol2imgBackward(pre->output->gradOverwrite(), dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
                             if (needB)
                                 iAddBackward(biasNode->output->grad(), pre->output->grad(), biasNode->output->shape(),
                                              pre->output->shape());

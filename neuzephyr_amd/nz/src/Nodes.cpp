@@ -72,7 +72,12 @@ namespace nz::nodes {
         void AddNode::forward() { tensorMatrixAdd(*output, *inputs[0]->output, *inputs[1]->output); }
         void AddNode::backward() {                                     // src/Nodes.cu:99-146
             for (Node* in : inputs)
-                if (in->output->requiresGrad()) iAddBackward(in->output->grad(), output->grad(), in->output->shape(), output->shape());
+                if (in->output->requiresGrad()) {
+                    // equal shapes: a plain copy of the gradient (every element written); broadcast inputs accumulate
+                    const bool copies = in->output->shape() == output->shape();
+                    iAddBackward(copies ? in->output->gradOverwrite() : in->output->grad(), output->grad(), in->output->shape(),
+                                 output->shape());
+                }
         }
 
         MatMulNode::MatMulNode(Node* input_left, Node* input_right) {
@@ -106,7 +111,7 @@ namespace nz::nodes {
         void ReLUNode::forward() { iRELU(output->data(), inputs[0]->output->data(), output->size()); }
         void ReLUNode::backward() {                                    // src/Nodes.cu:357-364
             if (inputs[0]->output->requiresGrad())
-                iReLUBackward(inputs[0]->output->grad(), inputs[0]->output->data(), output->grad(), output->size());
+                iReLUBackward(inputs[0]->output->gradOverwrite(), inputs[0]->output->data(), output->grad(), output->size());
         }
 
         SoftmaxNode::SoftmaxNode(Node* input) {
@@ -126,7 +131,7 @@ namespace nz::nodes {
             // both are the same sums) with fp16-rounded operands like the GEMM the reference calls, fused so
             // that the n x n Jacobian never reaches memory
             const auto& s = output->shape();
-            iSoftmaxBackward(inputs[0]->output->grad(), output->data(), output->grad(), s[2] * s[3], s[0] * s[1]);
+            iSoftmaxBackward(inputs[0]->output->gradOverwrite(), output->data(), output->grad(), s[2] * s[3], s[0] * s[1]);
         }
 
         ExpandNode::ExpandNode(Node* input, const Tensor::size_type newBatch) : newBatch(newBatch) {
@@ -183,7 +188,8 @@ namespace nz::nodes {
         }
         void ReshapeNode::backward() {                                 // src/Nodes.cu:565-571
             if (inputs[0]->output->requiresGrad())
-                NZ_CHECK(nzhip_memcpy_d2d(inputs[0]->output->grad(), output->grad(), output->size() * sizeof(Tensor::value_type)));
+                NZ_CHECK(nzhip_memcpy_d2d(inputs[0]->output->gradOverwrite(), output->grad(),
+                                          output->size() * sizeof(Tensor::value_type)));
         }
 
         Img2ColNode::Img2ColNode(Node* input, const Tensor::size_type kernelHeight, const Tensor::size_type kernelWidth,
@@ -228,7 +234,7 @@ namespace nz::nodes {
         }
         void Col2ImgNode::backward() {                                 // src/Nodes.cu:660-665
             if (inputs[0]->output->requiresGrad())
-                iCol2imgBackward(inputs[0]->output->grad(), output->grad(), outputHeight, outputWidth, outputChannels,
+                iCol2imgBackward(inputs[0]->output->gradOverwrite(), output->grad(), outputHeight, outputWidth, outputChannels,
                                  inputs[0]->output->shape()[0]);
         }
     }
@@ -248,7 +254,7 @@ namespace nz::nodes {
 
         void MeanSquaredErrorNode::backward() {                        // src/Nodes.cu:804-811
             if (output->requiresGrad())
-                iMSEBackward(output->grad(), inputs[0]->output->data(), inputs[1]->output->data(), output->size());
+                iMSEBackward(output->gradOverwrite(), inputs[0]->output->data(), inputs[1]->output->data(), output->size());
         }
 
         BinaryCrossEntropyNode::BinaryCrossEntropyNode(Node* input1, Node* input2) : OutputNode(input1) {
@@ -265,7 +271,7 @@ namespace nz::nodes {
 
         void BinaryCrossEntropyNode::backward() {                      // src/Nodes.cu:842-849
             if (output->requiresGrad())
-                iBCEBackward(output->grad(), inputs[0]->output->data(), inputs[1]->output->data(), output->size());
+                iBCEBackward(output->gradOverwrite(), inputs[0]->output->data(), inputs[1]->output->data(), output->size());
         }
     }
 }

@@ -52,12 +52,14 @@ namespace nz::data {
 
     Tensor::Tensor(const Tensor& other) : Tensor(other._shape, other._requires_grad) {
         if (other._data) NZ_CHECK(nzhip_memcpy_d2d(data(), other._data, _size * sizeof(value_type)));
-        if (_requires_grad && other._grad) NZ_CHECK(nzhip_memcpy_d2d(grad(), other._grad, _size * sizeof(value_type)));
+        if (_requires_grad && other._grad) NZ_CHECK(nzhip_memcpy_d2d(gradOverwrite(), other.grad(), _size * sizeof(value_type)));
     }
 
     Tensor::Tensor(Tensor&& other) noexcept
         : _size(other._size), _shape(other._shape), _data(other._data), _grad(other._grad),
           _requires_grad(other._requires_grad) {
+        _gradZeroPending = other._gradZeroPending;
+        other._gradZeroPending = false;
         other._data = nullptr;
         other._grad = nullptr;
         other._size = 0;
@@ -80,6 +82,8 @@ namespace nz::data {
         _data = other._data;
         _grad = other._grad;
         _requires_grad = other._requires_grad;
+        _gradZeroPending = other._gradZeroPending;
+        other._gradZeroPending = false;
         other._data = nullptr;
         other._grad = nullptr;
         other._size = 0;
@@ -102,6 +106,7 @@ namespace nz::data {
         if (!requires_grad && _grad) {
             nzhip_free_async(_grad);
             _grad = nullptr;
+            _gradZeroPending = false;
         }
         _requires_grad = requires_grad;
     }
@@ -115,8 +120,19 @@ namespace nz::data {
         if (!_requires_grad) throw std::runtime_error("Tensor does not require gradients");
         if (!_grad && _size) {
             _grad = deviceAlloc(_size);
+            _gradZeroPending = true;
+        }
+        if (_gradZeroPending) {
+            _gradZeroPending = false;
             NZ_CHECK(nzhip_memset(_grad, 0, _size * sizeof(value_type)));
         }
+        return _grad;
+    }
+
+    Tensor::value_type* Tensor::gradOverwrite() const {
+        if (!_requires_grad) throw std::runtime_error("Tensor does not require gradients");
+        if (!_grad && _size) _grad = deviceAlloc(_size);
+        _gradZeroPending = false;
         return _grad;
     }
 
@@ -143,7 +159,7 @@ namespace nz::data {
 
     void Tensor::zeroGrad() const {
         // a gradient nobody has asked for yet is not allocated, and is cleared when it is (grad())
-        if (_requires_grad && _size && _grad) NZ_CHECK(nzhip_memset(_grad, 0, _size * sizeof(value_type)));
+        if (_requires_grad && _size && _grad) _gradZeroPending = true;
     }
 
     void Tensor::clear() const {

@@ -898,6 +898,37 @@ TEST(Model, ReadmeExampleTrains) {
     EXPECT_THROW(m.checkExpand(&wrong), std::runtime_error);
 }
 
+TEST(TensorBasic, ZeroGradIsLazyButObservable) {
+    // zeroGrad() defers the clear; every reader still sees zeros, and a full overwrite replaces it
+    Tensor t({1, 1, 2, 3}, true);
+    std::vector<float> g = {1, 2, 3, 4, 5, 6};
+    t.dataInject(g.begin(), g.end(), true);
+    EXPECT_TRUE(t.hostGrad() == g);
+    t.zeroGrad();
+    EXPECT_TRUE(t.hostGrad() == std::vector<float>(6, 0.f));
+    t.dataInject(g.begin(), g.end(), true);
+    t.zeroGrad();
+    std::vector<float> h = {6, 5, 4, 3, 2, 1};
+    EXPECT_EQ(nzhip_memcpy_h2d(t.gradOverwrite(), h.data(), 6 * sizeof(float)), 0);
+    EXPECT_TRUE(t.hostGrad() == h);                           // the pending clear did not run over the new values
+    t.zeroGrad();
+    Tensor copy(t);                                           // a copy of a cleared gradient is cleared
+    EXPECT_TRUE(copy.hostGrad() == std::vector<float>(6, 0.f));
+    // accumulation after zeroGrad starts from zero: d(relu)/dx of ones through a node that adds (MatMul)
+    InputNode a({1, 1, 2, 2}, true), b({1, 1, 2, 2}, true);
+    a.dataInject({1, 2, 3, 4});
+    b.dataInject({1, 0, 0, 1});
+    MatMulNode mm(&a, &b);
+    mm.forward();
+    for (int pass = 0; pass < 2; ++pass) {
+        a.output->zeroGrad();
+        b.output->zeroGrad();
+        mm.output->dataInject({1, 1, 1, 1}, true);
+        mm.backward();
+        EXPECT_TRUE(a.output->hostGrad() == (std::vector<float>{1, 1, 1, 1}));   // dC * B^T, not twice that on pass 2
+    }
+}
+
 TEST(Runtime, AllocatorCachesAndErrorsSurfaceAsExceptions) {
     size_t inUse0 = 0, cached0 = 0, allocs0 = 0, inUse1 = 0, cached1 = 0, allocs1 = 0;
     {
