@@ -155,16 +155,19 @@ namespace nz::graph {
                             const bool directW = needW && iConv2dBackwardWeights(rhs->output->grad(), x->output->data(), dZ, xs[0],
                                                                                  xs[1], xs[2], xs[3], O, i2c->kernelHeight,
                                                                                  i2c->kernelWidth, i2c->stride, i2c->padding, ws[0]);
-                            if ((needW && !directW) || needB)
-                                iCol2imgBackward(pre->output->gradOverwrite(), dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
+                            // gradient in the layout of the matmul result, [n][pixel][channel]: with one output
+                            // channel that is dZ itself, otherwise its per-image transpose
+                            float* dPre = dZ;
+                            if (O != 1 && ((needW && !directW) || needB)) {
+                                dPre = pre->output->gradOverwrite();
+                                iCol2imgBackward(dPre, dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
+                            }
                             if (needB)
-                                iAddBackward(biasNode->output->grad(), pre->output->grad(), biasNode->output->shape(),
-                                             pre->output->shape());
+                                iAddBackward(biasNode->output->grad(), dPre, biasNode->output->shape(), pre->output->shape());
                             if (needW && !directW) {
                                 i2c->forward();                      // the column matrix the fused forward never wrote
-                                iMatMulBackward(nullptr, rhs->output->grad(), i2c->output->data(), rhs->output->data(),
-                                                pre->output->grad(), i2c->output->shape(), rhs->output->shape(),
-                                                mm->output->shape());
+                                iMatMulBackward(nullptr, rhs->output->grad(), i2c->output->data(), rhs->output->data(), dPre,
+                                                i2c->output->shape(), rhs->output->shape(), mm->output->shape());
                             }
                             if (x->output->requiresGrad())
                                 iConv2dBackwardData(x->output->grad(), dZ, rhs->output->data(), xs[0], xs[1], xs[2], xs[3], O,
