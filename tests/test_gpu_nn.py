@@ -91,3 +91,37 @@ def test_expand_and_compress_bit_exact(nz, oracle):
     out = dev(base)
     nz.compress(out, dev(g))
     assert np.array_equal(host(out), oracle.compress(base, g))
+
+
+def test_readme_network_sizes_through_size_independent_properties(nz):
+    """The pooling and loss operators at the README network's sizes (10 x 1 x 1024 x 1024 -> 510 x 510), where the
+    CPU oracle would take too long: a constant image stays constant, pooling and its gradient are adjoint
+    (<pool(x), dy> = <x, pool^T(dy)>), the gradient hands out exactly what it receives (no padding), and the loss
+    and its gradient agree with fp64 formulas evaluated by torch on the same data."""
+    import torch
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    x = torch.rand((10, 1, 1024, 1024), device="cuda", generator=gen)
+    y = nz.avgpool2d(x, 5, 2, 0)
+    assert tuple(y.shape) == (10, 1, 510, 510)
+    const = nz.avgpool2d(torch.full_like(x, 0.375), 5, 2, 0)              # 0.375 * 25 and / 25 are exact
+    assert bool((const == 0.375).all())
+    dy = torch.rand(y.shape, device="cuda", generator=gen) - 0.5
+    dx = torch.zeros_like(x)
+    nz.avgpool2d_backward(dx, dy, 5, 2, 0)
+    lhs = float((y.double() * dy.double()).sum())
+    rhs = float((x.double() * dx.double()).sum())
+    assert abs(lhs - rhs) <= 1e-5 * max(1.0, abs(lhs))
+    assert abs(float(dx.double().sum()) - float(dy.double().sum())) <= 1e-4 * max(1.0, abs(float(dy.double().sum())))
+    # torch's own pooling (count_include_pad irrelevant without padding) as a third opinion on the values
+    ref = torch.nn.functional.avg_pool2d(x.double(), 5, 2).float()
+    assert float((y - ref).abs().max()) <= 2e-6
+    p = torch.rand(10 * 1024 * 1024, device="cuda", generator=gen) * 0.8 + 0.1
+    t = torch.rand(p.shape, device="cuda", generator=gen) * 0.8 + 0.1
+    truth = float((-(t.double()) * torch.log(p.double()) - (1 - t.double()) * torch.log1p(-p.double())).mean())
+    assert abs(float(nz.bce_loss(p, t)[0]) - truth) <= 1e-5 * truth
+    g = nz.bce_backward(p, t)
+    gt = ((p.double() - t.double()) / (p.double() * (1 - p.double())) / p.numel())
+    assert float(((g.double() - gt).abs() / gt.abs().clamp_min(1e-12)).max()) <= 1e-5
+    mse_truth = float(((p.double() - t.double()) ** 2).mean())
+    assert abs(float(nz.mse_loss(p, t)[0]) - mse_truth) <= 1e-5 * mse_truth
+
