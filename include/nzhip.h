@@ -218,6 +218,13 @@ int nzhip_softmax_jacobian(float* out, const float* in, size_t n, size_t batch, 
  * additions (the Jacobian is symmetric, so column and row vectors are the same sums). dx is overwritten. */
 int nzhip_softmax_backward(float* dx, const float* s, const float* dy, size_t n, size_t batch, void* stream);
 
+/* Gradient of the bias parameter of the reference's Conv2d ([1,1,H_out*W_out,O]: per pixel and channel, added to the
+ * matmul result): dbias[p*O + o] += sum over n of dz[(n*O + o)*HW + p]. Replaces Col2ImgNode::backward (a transposed
+ * copy of the whole gradient) + AddNode::backward (sum over the batch), src/Nodes.cu:660-665, 99-146; the images are
+ * added in ascending order onto the value already in dbias, like that chain (which, for a batch of one, copies
+ * instead of adding: AddNode::backward with equal shapes; callers keep that case on the two-step path). */
+int nzhip_conv2d_backward_bias(float* dbias, const float* dz, size_t N, size_t O, size_t HW, void* stream);
+
 /* ---- the rest of the reference's example network (README.md:62-90): pooling, loss, target expansion ---- */
 /* nz::data::iAveragePooling (AveragePoolingKernel, src/OperationKernels.cu:1404-1429; AveragePoolingNode::forward,
  * src/Nodes.cu:678-682): square window, out = mean over the window cells inside the image (cells in the

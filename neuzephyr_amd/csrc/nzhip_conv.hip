@@ -1528,6 +1528,55 @@ __global__ __launch_bounds__(256) void small_dw_reduce_kernel(float* __restrict_
     dW[(long)g * Q + q] += sum;
 }
 
+// Gradient of the per-pixel, per-channel bias the reference's Conv2d adds to the matmul result ([1,1,HW,O]):
+//   dbias[p][o] += sum over n of dz[n][o][p]   (dz in NCHW),
+// i.e. Col2ImgNode::backward (a transpose of the whole gradient) followed by AddNode::backward (a sum over the
+// batch) without the transposed copy. A workgroup owns 64 pixels x 32 channels: it starts from the values
+// already in dbias and adds the images in ascending order (the order of the two-step chain), reading dz
+// along pixels and writing dbias along channels; the tile is turned in LDS on the way in and on the way out.
+__global__ __launch_bounds__(256) void conv_bias_grad_kernel(float* __restrict__ dbias, const float* __restrict__ dz, int N,
+                                                             int O, long HW) {
+    __shared__ float tile[64][33];                               // [pixel][channel]
+    const long p0 = (long)blockIdx.x * 64;
+    const int o0 = blockIdx.y * 32;
+    {   // in: rows of dbias (channels contiguous)
+        const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+        for (int r = 0; r < 64; r += 8) {
+            const long p = p0 + ty + r;
+            const int o = o0 + tx;
+            tile[ty + r][tx] = (p < HW && o < O) ? dbias[p * O + o] : 0.f;
+        }
+    }
+    __syncthreads();
+    const int px = threadIdx.x & 63, oy = threadIdx.x >> 6;      // this thread's pixel, and channels oy, oy + 4, ...
+    const long p = p0 + px;
+    float acc[8];
+#pragma unroll
+    for (int r = 0; r < 8; r++) acc[r] = tile[px][oy + r * 4];
+    if (p < HW)
+        for (int n = 0; n < N; n++) {
+#pragma unroll
+            for (int r = 0; r < 8; r++) {
+                const int o = o0 + oy + r * 4;
+                if (o < O) acc[r] += dz[((long)n * O + o) * HW + p];
+            }
+        }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 8; r++) tile[px][oy + r * 4] = acc[r];
+    __syncthreads();
+    {   // out: rows of dbias again
+        const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+        for (int r = 0; r < 64; r += 8) {
+            const long pp = p0 + ty + r;
+            const int o = o0 + tx;
+            if (pp < HW && o < O) dbias[pp * O + o] = tile[ty + r][tx];
+        }
+    }
+}
+
 // Weights of the data-gradient convolution: the gradient with respect to x of a stride-1 convolution is
 // itself a stride-1 convolution of dy (O channels in, C channels out) with the taps mirrored:
 //   w'[wb][(o, r', s')][c] = w[wb][(c, K_h-1-r', K_w-1-s')][o]
@@ -1678,6 +1727,21 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     int rc2 = tmp ? workspace_free(tmp, s) : NZHIP_OK;
     int rc3 = workspace_free(wflip, s);
     return rc ? rc : (rc2 ? rc2 : rc3);
+}
+
+/* Gradient of the reference's Conv2d bias parameter ([1,1,H_out*W_out,O], added to the matmul result before
+ * Col2Img): dbias[p][o] += sum over n of dz[n][o][p], dz being the gradient of the convolution output in NCHW.
+ * One kernel for Col2ImgNode::backward + AddNode::backward (src/Nodes.cu:660-665, 99-146). */
+extern "C" int nzhip_conv2d_backward_bias(float* dbias, const float* dz, size_t N, size_t O, size_t HW, void* stream) {
+    if (!dbias || !dz) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_bias: null pointer");
+    if (N == 0 || O == 0 || HW == 0) return NZHIP_OK;
+    if (N > 0x7fffffff || O > 0x7fffffff || (O + 31) / 32 > 65535 || (HW + 63) / 64 > 0x7fffffffull)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_bias: extent too large");
+    dim3 grid((unsigned)((HW + 63) / 64), (unsigned)((O + 31) / 32));
+    hipLaunchKernelGGL(conv_bias_grad_kernel, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream), dbias, dz, (int)N,
+                       (int)O, (long)HW);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv_bias_grad kernel launch");
 }
 
 /* Gradient of nzhip_conv2d_forward with respect to the weights, without the column matrix the reference's

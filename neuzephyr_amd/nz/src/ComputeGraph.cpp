@@ -157,12 +157,20 @@ namespace nz::graph {
                                                                                  i2c->kernelWidth, i2c->stride, i2c->padding, ws[0]);
                             // gradient in the layout of the matmul result, [n][pixel][channel]: with one output
                             // channel that is dZ itself, otherwise its per-image transpose
+                            // the Conv2d bias is [1, 1, pixels, O]: its gradient comes straight from dZ in one kernel
+                            const auto bshape = biasNode ? biasNode->output->shape() : Tensor::shape_type{0, 0, 0, 0};
+                            // (with one channel dZ already has that layout and the plain batch sum below reads it)
+                            // and with a batch of one Add.backward copies instead of adding: left to the node's own path)
+                            const bool fusedB = needB && O != 1 && xs[0] > 1 && bshape[0] == 1 && bshape[1] == 1 &&
+                                                bshape[2] == c2i->outputHeight * c2i->outputWidth && bshape[3] == O;
                             float* dPre = dZ;
-                            if (O != 1 && ((needW && !directW) || needB)) {
+                            if (O != 1 && ((needW && !directW) || (needB && !fusedB))) {
                                 dPre = pre->output->gradOverwrite();
                                 iCol2imgBackward(dPre, dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
                             }
-                            if (needB)
+                            if (fusedB)
+                                iConv2dBackwardBias(biasNode->output->grad(), dZ, xs[0], O, c2i->outputHeight * c2i->outputWidth);
+                            else if (needB)
                                 iAddBackward(biasNode->output->grad(), dPre, biasNode->output->shape(), pre->output->shape());
                             if (needW && !directW) {
                                 i2c->forward();                      // the column matrix the fused forward never wrote

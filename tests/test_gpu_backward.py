@@ -297,6 +297,19 @@ def test_conv2d_backward_weights_few_channels_float_tolerance(nz, oracle):
     assert mr <= 1e-3 and fr <= 1e-4, (mr, fr)
 
 
+@pytest.mark.parametrize("N,O,H,W", [(1, 1, 1, 1), (3, 5, 7, 9), (2, 40, 9, 30), (4, 128, 16, 24), (5, 1, 30, 70), (2, 33, 1, 130)])
+def test_conv2d_backward_bias_equals_the_two_step_chain_bit_for_bit(nz, oracle, N, O, H, W):
+    """One kernel for Col2Img.backward (transpose) + Add.backward (sum over the batch onto the gradient already
+    there): the same additions in the same order, so float data agree bit for bit with the oracle's chain."""
+    rng = np.random.default_rng(N + 3 * O + 5 * H + 7 * W)
+    dz = rng.standard_normal((N, O, H, W)).astype(np.float32)
+    base = rng.standard_normal((1, 1, H * W, O)).astype(np.float32)
+    # with a batch of one the reference's Add.backward copies instead of adding (equal shapes); the kernel always adds
+    want = oracle.add_backward(base, oracle.col2im_backward(dz)) if N > 1 else base + oracle.col2im_backward(dz)
+    got = host(nz.conv2d_backward_bias(dev(base), dev(dz)))
+    assert np.array_equal(got, want)
+
+
 def test_conv2d_backward_weights_rejects_what_it_does_not_cover(nz):
     from neuzephyr_amd.capi import NzHipError
     with pytest.raises(NzHipError):      # stride 2
