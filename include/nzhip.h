@@ -225,6 +225,12 @@ int nzhip_softmax_backward(float* dx, const float* s, const float* dy, size_t n,
  * instead of adding: AddNode::backward with equal shapes; callers keep that case on the two-step path). */
 int nzhip_conv2d_backward_bias(float* dbias, const float* dz, size_t N, size_t O, size_t HW, void* stream);
 
+/* The same for a Conv2d followed by ReLU, with ReLUNode::backward (src/Nodes.cu:357-364) in front: writes
+ * dz[i] = y[i] > 0 ? dy[i] : 0 over the whole [N,O,HW] gradient and adds its batch sum, transposed, onto dbias in the
+ * same pass. dz must not overlap y or dy. */
+int nzhip_conv2d_backward_relu_bias(float* dz, float* dbias, const float* y, const float* dy, size_t N, size_t O,
+                                    size_t HW, void* stream);
+
 /* ---- the rest of the reference's example network (README.md:62-90): pooling, loss, target expansion ---- */
 /* nz::data::iAveragePooling (AveragePoolingKernel, src/OperationKernels.cu:1404-1429; AveragePoolingNode::forward,
  * src/Nodes.cu:678-682): square window, out = mean over the window cells inside the image (cells in the

@@ -18,7 +18,7 @@ EXPORTS = [
     "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_tensorcore_gemm",
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
-    "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
+    "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
     "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
     "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_mse_loss", "nzhip_mse_backward", "nzhip_expand", "nzhip_compress",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
@@ -91,6 +91,7 @@ def load() -> C.CDLL:
     lib.nzhip_softmax_jacobian.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_softmax_backward.argtypes = [vp, vp, vp, sz, sz, vp]
     lib.nzhip_conv2d_backward_bias.argtypes = [vp, vp, sz, sz, sz, vp]
+    lib.nzhip_conv2d_backward_relu_bias.argtypes = [vp, vp, vp, vp, sz, sz, sz, vp]
     lib.nzhip_avgpool2d.argtypes = [vp, vp] + [sz] * 9 + [vp]
     lib.nzhip_avgpool2d_backward.argtypes = [vp, vp] + [sz] * 9 + [vp]
     lib.nzhip_bce_loss.argtypes = [vp, vp, vp, sz, vp]
@@ -387,6 +388,16 @@ def conv2d_backward_bias(dbias, dz, stream=None):
     N, O, H, W = dz.shape
     check(lib.nzhip_conv2d_backward_bias(_dev(dbias), _dev(dz), N, O, H * W, _stream_handle(stream)))
     return dbias
+
+
+def conv2d_backward_relu_bias(dbias, y, dy, stream=None):
+    """Returns dz = dy where y > 0 else 0, and adds its transposed batch sum onto dbias [1,1,HW,O] in place."""
+    import torch
+    lib = load()
+    N, O, H, W = dy.shape
+    dz = torch.empty_like(dy)
+    check(lib.nzhip_conv2d_backward_relu_bias(_dev(dz), _dev(dbias), _dev(y), _dev(dy), N, O, H * W, _stream_handle(stream)))
+    return dz
 
 
 def avgpool2d(x, pool, stride, pad, stream=None):

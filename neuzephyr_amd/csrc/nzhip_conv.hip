@@ -1534,8 +1534,12 @@ __global__ __launch_bounds__(256) void small_dw_reduce_kernel(float* __restrict_
 // batch) without the transposed copy. A workgroup owns 64 pixels x 32 channels: it starts from the values
 // already in dbias and adds the images in ascending order (the order of the two-step chain), reading dz
 // along pixels and writing dbias along channels; the tile is turned in LDS on the way in and on the way out.
+// MASK: dz is not given but made here, dz[n][o][p] = y[n][o][p] > 0 ? dy[n][o][p] : 0 (the gradient through the ReLU
+// that follows the convolution, ReLUNode::backward), written out for the other gradient kernels and summed on the way.
+template <bool MASK>
 __global__ __launch_bounds__(256) void conv_bias_grad_kernel(float* __restrict__ dbias, const float* __restrict__ dz, int N,
-                                                             int O, long HW) {
+                                                             int O, long HW, float* __restrict__ dz_out,
+                                                             const float* __restrict__ y) {
     __shared__ float tile[64][33];                               // [pixel][channel]
     const long p0 = (long)blockIdx.x * 64;
     const int o0 = blockIdx.y * 32;
@@ -1559,7 +1563,15 @@ __global__ __launch_bounds__(256) void conv_bias_grad_kernel(float* __restrict__
 #pragma unroll
             for (int r = 0; r < 8; r++) {
                 const int o = o0 + oy + r * 4;
-                if (o < O) acc[r] += dz[((long)n * O + o) * HW + p];
+                if (o < O) {
+                    const long at = ((long)n * O + o) * HW + p;
+                    float g = dz[at];
+                    if (MASK) {
+                        g = y[at] > 0.f ? g : 0.f;
+                        dz_out[at] = g;
+                    }
+                    acc[r] += g;
+                }
             }
         }
     __syncthreads();
@@ -1738,10 +1750,26 @@ extern "C" int nzhip_conv2d_backward_bias(float* dbias, const float* dz, size_t 
     if (N > 0x7fffffff || O > 0x7fffffff || (O + 31) / 32 > 65535 || (HW + 63) / 64 > 0x7fffffffull)
         return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_bias: extent too large");
     dim3 grid((unsigned)((HW + 63) / 64), (unsigned)((O + 31) / 32));
-    hipLaunchKernelGGL(conv_bias_grad_kernel, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream), dbias, dz, (int)N,
-                       (int)O, (long)HW);
+    hipLaunchKernelGGL(conv_bias_grad_kernel<false>, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream), dbias, dz,
+                       (int)N, (int)O, (long)HW, static_cast<float*>(nullptr), static_cast<const float*>(nullptr));
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv_bias_grad kernel launch");
+}
+
+/* The same with the ReLU gradient in front (Conv2d followed by ReLU): dz[n][o][p] = y[n][o][p] > 0 ? dy[n][o][p] : 0
+ * is written out (ReLUNode::backward, src/Nodes.cu:357-364) and dbias[p][o] += sum over n of dz[n][o][p] in the same
+ * pass, so the masked gradient is not read back for the bias. dz must not overlap y or dy. */
+extern "C" int nzhip_conv2d_backward_relu_bias(float* dz, float* dbias, const float* y, const float* dy, size_t N, size_t O,
+                                               size_t HW, void* stream) {
+    if (!dz || !dbias || !y || !dy) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_relu_bias: null pointer");
+    if (N == 0 || O == 0 || HW == 0) return NZHIP_OK;
+    if (N > 0x7fffffff || O > 0x7fffffff || (O + 31) / 32 > 65535 || (HW + 63) / 64 > 0x7fffffffull)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_relu_bias: extent too large");
+    dim3 grid((unsigned)((HW + 63) / 64), (unsigned)((O + 31) / 32));
+    hipLaunchKernelGGL(conv_bias_grad_kernel<true>, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream), dbias, dy,
+                       (int)N, (int)O, (long)HW, dz, y);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv_bias_grad (masked) kernel launch");
 }
 
 /* Gradient of nzhip_conv2d_forward with respect to the weights, without the column matrix the reference's

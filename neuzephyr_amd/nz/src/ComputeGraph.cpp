@@ -143,34 +143,43 @@ namespace nz::graph {
                     if (i2c->stride == 1 && i2c->kernelHeight == i2c->kernelWidth && i2c->padding <= i2c->kernelHeight - 1) {
                         Node* pre = add ? static_cast<Node*>(add) : static_cast<Node*>(mm);   // holds [N,1,HW,O] gradients
                         back = [=] {
-                            float* dZ = last->output->grad();
-                            if (relu) {
-                                float* masked = c2i->output->gradOverwrite();     // every element written
-                                iReLUBackward(masked, last->output->data(), dZ, last->output->size());
-                                dZ = masked;
-                            }
                             const bool needW = rhs->output->requiresGrad();
                             const bool needB = biasNode && biasNode->output->requiresGrad();
+                            const size_t pixels = c2i->outputHeight * c2i->outputWidth;
+                            // The Conv2d bias is [1, 1, pixels, O]: its gradient is the batch sum of the transposed
+                            // output gradient and comes straight from the NCHW gradient in one kernel. (With one
+                            // channel the gradient already has that layout and the plain batch sum reads it; with a
+                            // batch of one Add.backward copies instead of adding: both stay on the node's own path.)
+                            const auto bshape = biasNode ? biasNode->output->shape() : Tensor::shape_type{0, 0, 0, 0};
+                            const bool fusedB = needB && O != 1 && xs[0] > 1 && bshape[0] == 1 && bshape[1] == 1 &&
+                                                bshape[2] == pixels && bshape[3] == O;
+                            float* dZ = last->output->grad();
+                            bool biasDone = false;
+                            if (relu) {
+                                float* masked = c2i->output->gradOverwrite();     // every element written
+                                if (fusedB) {                                     // mask and bias gradient in one pass
+                                    iConv2dBackwardReluBias(masked, biasNode->output->grad(), last->output->data(), dZ, xs[0], O,
+                                                            pixels);
+                                    biasDone = true;
+                                } else {
+                                    iReLUBackward(masked, last->output->data(), dZ, last->output->size());
+                                }
+                                dZ = masked;
+                            }
                             // weights straight from x and dZ where the geometry allows, else through the column matrix
                             const bool directW = needW && iConv2dBackwardWeights(rhs->output->grad(), x->output->data(), dZ, xs[0],
                                                                                  xs[1], xs[2], xs[3], O, i2c->kernelHeight,
                                                                                  i2c->kernelWidth, i2c->stride, i2c->padding, ws[0]);
                             // gradient in the layout of the matmul result, [n][pixel][channel]: with one output
                             // channel that is dZ itself, otherwise its per-image transpose
-                            // the Conv2d bias is [1, 1, pixels, O]: its gradient comes straight from dZ in one kernel
-                            const auto bshape = biasNode ? biasNode->output->shape() : Tensor::shape_type{0, 0, 0, 0};
-                            // (with one channel dZ already has that layout and the plain batch sum below reads it)
-                            // and with a batch of one Add.backward copies instead of adding: left to the node's own path)
-                            const bool fusedB = needB && O != 1 && xs[0] > 1 && bshape[0] == 1 && bshape[1] == 1 &&
-                                                bshape[2] == c2i->outputHeight * c2i->outputWidth && bshape[3] == O;
                             float* dPre = dZ;
                             if (O != 1 && ((needW && !directW) || (needB && !fusedB))) {
                                 dPre = pre->output->gradOverwrite();
                                 iCol2imgBackward(dPre, dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
                             }
-                            if (fusedB)
-                                iConv2dBackwardBias(biasNode->output->grad(), dZ, xs[0], O, c2i->outputHeight * c2i->outputWidth);
-                            else if (needB)
+                            if (fusedB && !biasDone)
+                                iConv2dBackwardBias(biasNode->output->grad(), dZ, xs[0], O, pixels);
+                            else if (needB && !fusedB)
                                 iAddBackward(biasNode->output->grad(), dPre, biasNode->output->shape(), pre->output->shape());
                             if (needW && !directW) {
                                 i2c->forward();                      // the column matrix the fused forward never wrote

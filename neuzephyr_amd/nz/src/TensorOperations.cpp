@@ -129,6 +129,10 @@ namespace nz::data {
         NZ_CHECK(nzhip_conv2d_backward_bias(dbias, dz, N, O, HW, nzhip_default_stream()));
     }
 
+    void iConv2dBackwardReluBias(float* dz, float* dbias, float* y, float* dy, const size_t N, const size_t O, const size_t HW) {
+        NZ_CHECK(nzhip_conv2d_backward_relu_bias(dz, dbias, y, dy, N, O, HW, nzhip_default_stream()));
+    }
+
     void iAveragePooling(float* out, float* in, const size_t pool_size, const size_t stride, const size_t padding,
                          const size_t batches, const size_t channels, const size_t H_in, const size_t W_in,
                          const size_t H_out, const size_t W_out) {

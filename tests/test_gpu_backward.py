@@ -310,6 +310,19 @@ def test_conv2d_backward_bias_equals_the_two_step_chain_bit_for_bit(nz, oracle, 
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("N,O,H,W", [(3, 5, 7, 9), (2, 40, 9, 30), (4, 128, 16, 24), (2, 33, 1, 130)])
+def test_conv2d_backward_relu_bias_equals_relu_backward_then_bias(nz, oracle, N, O, H, W):
+    rng = np.random.default_rng(2 * N + 3 * O + 5 * H + 7 * W)
+    y = np.maximum(rng.standard_normal((N, O, H, W)), 0).astype(np.float32)       # a ReLU output: zeros and positives
+    dy = rng.standard_normal((N, O, H, W)).astype(np.float32)
+    base = rng.standard_normal((1, 1, H * W, O)).astype(np.float32)
+    dz_want = oracle.relu_backward(y, dy)
+    db_want = oracle.add_backward(base, oracle.col2im_backward(dz_want))
+    db = dev(base)
+    dz = nz.conv2d_backward_relu_bias(db, dev(y), dev(dy))
+    assert np.array_equal(host(dz), dz_want) and np.array_equal(host(db), db_want)
+
+
 def test_conv2d_backward_weights_rejects_what_it_does_not_cover(nz):
     from neuzephyr_amd.capi import NzHipError
     with pytest.raises(NzHipError):      # stride 2
