@@ -27,11 +27,20 @@ typedef float floatx2 __attribute__((ext_vector_type(2)));
 // The workspace is NOT a row-major matrix. It is a sequence of 16 KiB blocks, one per
 // (256-row block rb, 32-wide k tile kt), stored at block index rb * (Kp/32) + kt, and each
 // block is the exact image the GEMM wants in LDS: physical row pr (see phys_row_of) at byte
-// pr*64, chunk c (8 halfs) of that row at chunk position c ^ ((pr>>2)&3). The GEMM's
+// pr*64, chunk c (8 halfs) of that row at chunk position c ^ chunk_swizzle(pr). The GEMM's
 // global->LDS copies are therefore plain contiguous 1 KiB reads, consecutive k tiles are
 // consecutive 16 KiB blocks (no power-of-two row pitch, so all memory channels stay busy),
 // and rows/columns beyond the operand are zero.
 constexpr int CVT_ROWS = 256, CVT_K = 32, CVT_BLOCK_BYTES = CVT_ROWS * CVT_K * 2;
+
+// Chunk swizzle of a 64-byte LDS row. A 128-bit LDS read is served 16 lanes per pass, and the passes
+// are NOT lanes 0-15, 16-31, ...: lanes {0-3, 12-15, 20-23, 24-27} share one pass, {4-7, 8-11, 16-19,
+// 28-31} the next (and the same again for lanes 32-63). In a 16x16x32 fragment read lane l takes
+// chunk l>>4 of row l&15, so one pass mixes row quads 0 and 3 at chunk q with row quads 1 and 2 at
+// chunk q^1. With f(quad) = -quad mod 4 the four (quad, chunk) pairs of every pass land on four
+// different 16-byte bank groups; the plainer f(quad) = quad puts them on two, and every read takes
+// 1.6 times as long (measured per instruction: 7.1 against 4.4 clocks).
+__device__ __forceinline__ int chunk_swizzle(int row) { return (-(row >> 2)) & 3; }
 
 // Physical LDS row of logical tile row r when a wave owns FR consecutive 32-row MFMA blocks of the
 // 256-row tile (FR = 4: two waves along that dimension, FR = 2: four). The rows of a wave are
@@ -77,7 +86,7 @@ __device__ __forceinline__ void cvt_block(char* img, const CvtOperand& o, int K,
             }
             half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
             const int pr = phys_row_of(lr, fr, blk);
-            const int pos = (k4 >> 1) ^ ((pr >> 2) & 3);
+            const int pos = (k4 >> 1) ^ chunk_swizzle(pr);
             *reinterpret_cast<half4_t*>(img + pr * 64 + pos * 16 + (k4 & 1) * 8) = h;
         }
     } else {
@@ -100,7 +109,7 @@ __device__ __forceinline__ void cvt_block(char* img, const CvtOperand& o, int K,
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 const int pr = phys_row_of(lr + e, fr, blk);
-                const int pos = (kk >> 3) ^ ((pr >> 2) & 3);
+                const int pos = (kk >> 3) ^ chunk_swizzle(pr);
                 *reinterpret_cast<_Float16*>(img + pr * 64 + pos * 16 + (kk & 7) * 2) = (_Float16)v[e];
             }
         }
@@ -161,8 +170,8 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC
 
 // BM x BN x 32 tiles in an NSTAGE-deep LDS ring. One LDS row = 32 halfs = 64 bytes = 4 chunks of
 // 16 bytes. LDS has 64 banks x 4 B, so a 256-byte bank row spans four tile rows; chunk c of row r
-// is stored at chunk position  c ^ ((r>>2)&3), which puts the 16 rows that one pass of a
-// 128-bit fragment read touches on 16 different 16-byte bank groups.
+// is stored at chunk position  c ^ chunk_swizzle(r), which puts the 16 lanes that share one pass of a
+// 128-bit fragment read on 16 different 16-byte bank groups.
 template <int BM, int BN, int WM, int WN, int NSTAGE>
 __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16_kernel(const H16Args p) {
     static_assert((BM == CVT_ROWS || BM * 2 == CVT_ROWS) && BN == CVT_ROWS, "must match the workspace block image");
@@ -246,10 +255,10 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    // fragment addressing: physical row = block*32 + li; chunk position (2*ks + lh) ^ ((row>>2)&3)
+    // fragment addressing: physical row = block*32 + li; chunk position (2*ks + lh) ^ chunk_swizzle(row)
     const int a_row_off = ((wm * FM) * 32 + li) * ROWB;
     const int b_row_off = A_BYTES + ((wn * FN) * 32 + li) * ROWB;
-    const int sw = (li >> 2) & 3;
+    const int sw = chunk_swizzle(li);
 
     half8_t af[2][FM], bf[2][FN];
     auto read_frags = [&](const char* base, int ks, int buf) {
@@ -467,8 +476,8 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
         for (int r = 0; r < 4; r++) acc[t][r] = 0.f;
 
     // fragment addressing: physical row = block*16 + l16, the lane's 8 k values are chunk lq,
-    // stored at chunk position lq ^ ((row>>2)&3)
-    const int frag_off = l16 * ROWB + ((lq ^ ((l16 >> 2) & 3)) << 4);
+    // stored at chunk position lq ^ chunk_swizzle(row)
+    const int frag_off = l16 * ROWB + ((lq ^ chunk_swizzle(l16)) << 4);
     const int a_off = (wm * FM) * 16 * ROWB + frag_off;
     const int b_off = A_BYTES + (wn * FN) * 16 * ROWB + frag_off;
 
