@@ -82,6 +82,28 @@ typedef struct nzhip_gemm_desc {
 
 int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream);
 
+/* nzhip_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose GEMM
+ * driver allocates three temporaries per call (src/OperationKernels.cu:885-912).
+ * Same arguments, same kernels and bit-identical results, but every workspace the routes use
+ * (fp16 operand images of the two-pass route, split-contraction partial sums) lives in a static
+ * device array of NZHIP_STATIC_SCRATCH_BYTES that each GPU holds from library load until the
+ * process ends; the call performs no hipMalloc / hipFree and never touches the caching pool.
+ * A product whose workspace would not fit is rejected with NZHIP_E_UNSUPPORTED before anything
+ * is enqueued (nzhip_last_error() names the size).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race; serialise them. */
+#define NZHIP_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int nzhip_gemm_static(const nzhip_gemm_desc* desc, void* stream);
+size_t nzhip_static_scratch_bytes(void);
+
+/* Test and benchmark hook (no counterpart in the reference): nzhip_gemm with the kernel chosen by the
+ * caller instead of by the shape, so that every kernel can be checked on every shape.
+ * tile 128 / 256: the fused convert-on-load kernel with that square tile; 16 / 18 / 12: the two-pass
+ * fp16 route with 256x256 tiles on 4 waves / 256x256 tiles on 8 waves / 128x256 tiles, 16x16x32 MFMAs;
+ * 316 / 318 / 312: the same three with 32x32x16 MFMAs.  Any other value: NZHIP_E_INVALID. */
+int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream);
+
 /* Drop-in for nz::data::iTensorCoreGEMM (include/NeuZephyr/TensorOperations.cuh:1021-1022,
  * src/TensorOperations.cu:112-115 -> krnl::TensorCoreGEMMParallel, src/OperationKernels.cu:914-1026):
  * M = A.h, N = B.w, K = A.w; loops over C's (n,c); an operand whose n (or c) is 1 is

@@ -15,7 +15,8 @@ ACT_NONE, ACT_RELU = 0, 1
 LAYOUT_ROW, LAYOUT_TRANS = 0, 1
 
 EXPORTS = [
-    "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_tensorcore_gemm",
+    "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_gemm_static",
+    "nzhip_static_scratch_bytes", "nzhip_gemm_force_tile", "nzhip_tensorcore_gemm",
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
@@ -70,6 +71,8 @@ def load() -> C.CDLL:
     lib.nzhip_last_error.restype = C.c_char_p
     lib.nzhip_device_info.argtypes = [C.POINTER(C.c_int), C.POINTER(sz), C.c_char_p, sz]
     lib.nzhip_gemm.argtypes = [C.POINTER(GemmDesc), vp]
+    lib.nzhip_gemm_static.argtypes = [C.POINTER(GemmDesc), vp]
+    lib.nzhip_static_scratch_bytes.restype = sz
     lib.nzhip_gemm_force_tile.argtypes = [C.POINTER(GemmDesc), C.c_int, vp]
     lib.nzhip_tensorcore_gemm.argtypes = [vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_im2col.argtypes = [vp, vp] + [sz] * 10 + [vp]
@@ -139,9 +142,10 @@ def _dev(t):
 
 
 def gemm(A, B, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), relu=False, out=None,
-         force_tile=0, stream=None):
+         force_tile=0, stream=None, static=False):
     """C = act(f16(A) @ f16(B) + bias) for 2-D tensors. a_trans: A holds K x M; b_trans: B holds N x K.
-    bias_strides = (row stride, column stride) in elements."""
+    bias_strides = (row stride, column stride) in elements. static: through nzhip_gemm_static (the
+    entry point that allocates nothing); `out` must then be given."""
     import torch
     lib = load()
     M, K = (A.shape[1], A.shape[0]) if a_trans else A.shape
@@ -160,7 +164,9 @@ def gemm(A, B, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), 
         d.bias = _dev(bias)
         d.bias_stride_row, d.bias_stride_col = bias_strides
     d.activation = ACT_RELU if relu else ACT_NONE
-    if force_tile:
+    if static:
+        check(lib.nzhip_gemm_static(C.byref(d), _stream_handle(stream)))
+    elif force_tile:
         check(lib.nzhip_gemm_force_tile(C.byref(d), force_tile, _stream_handle(stream)))
     else:
         check(lib.nzhip_gemm(C.byref(d), _stream_handle(stream)))

@@ -77,13 +77,59 @@ private:
     PoolAllocator<HipBackend> pool_;
 };
 
+// ---- static scratch: the workspace of the entry point that allocates nothing -----------------
+// One array per GPU, held from the moment the library is loaded until the process ends. In host code
+// the array's name is only a stand-in for the symbol: the device address comes from
+// hipGetSymbolAddress, once per device with that device current, and only that address is ever
+// handed to kernels.
+constexpr size_t STATIC_SCRATCH_BYTES = NZHIP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+static int static_scratch_base(unsigned char** base) {
+    static std::mutex mu;
+    static unsigned char* per_device[64] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return set_hip_error(e, "hipGetDevice");
+    if (dev < 0 || dev >= 64) return set_error(NZHIP_E_UNSUPPORTED, "static scratch: device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!per_device[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return set_hip_error(e, "hipGetSymbolAddress(static scratch)");
+        per_device[dev] = static_cast<unsigned char*>(p);
+    }
+    *base = per_device[dev];
+    return NZHIP_OK;
+}
+
+// While a thread is inside nzhip_gemm_static its workspace requests are served from the current
+// device's static scratch (bump allocation, nothing is ever returned) instead of the pool.
+struct StaticArena {
+    unsigned char* base = nullptr;
+    size_t used = 0;
+    bool active = false;
+};
+static thread_local StaticArena t_arena;
+
 int workspace_alloc(void** ptr, size_t bytes, hipStream_t s) {
+    if (t_arena.active) {
+        const size_t at = (t_arena.used + 255) & ~(size_t)255;
+        if (bytes > STATIC_SCRATCH_BYTES || at > STATIC_SCRATCH_BYTES - bytes)
+            return set_error(NZHIP_E_UNSUPPORTED,
+                             "nzhip_gemm_static: this product needs %zu bytes of workspace, the static scratch holds %zu",
+                             at + bytes, STATIC_SCRATCH_BYTES);
+        *ptr = t_arena.base + at;
+        t_arena.used = at + bytes;
+        return NZHIP_OK;
+    }
     int rc = Runtime::instance().pool().allocate(ptr, bytes, reinterpret_cast<uintptr_t>(s));
     if (rc != 0) return set_error(NZHIP_E_NOMEM, "workspace allocation of %zu bytes failed (hipError_t %d)", bytes, rc);
     return NZHIP_OK;
 }
 
 int workspace_free(void* ptr, hipStream_t s) {
+    if (t_arena.active) return NZHIP_OK;                      // the arena is reset by the next call
     return Runtime::instance().pool().free_async(ptr, reinterpret_cast<uintptr_t>(s)) == 0
                ? NZHIP_OK
                : set_error(NZHIP_E_INVALID, "workspace_free: unknown pointer");
@@ -210,6 +256,19 @@ int nzhip_sync_all(void) {
     hipError_t e = hipDeviceSynchronize();
     return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipDeviceSynchronize");
 }
+
+int nzhip_gemm_static(const nzhip_gemm_desc* desc, void* stream) {
+    unsigned char* base = nullptr;
+    if (int rc = static_scratch_base(&base)) return rc;
+    t_arena.base = base;
+    t_arena.used = 0;
+    t_arena.active = true;
+    const int rc = nzhip_gemm(desc, stream);
+    t_arena.active = false;
+    return rc;
+}
+
+size_t nzhip_static_scratch_bytes(void) { return STATIC_SCRATCH_BYTES; }
 
 int nzhip_allocator_stats(size_t* bytes_in_use, size_t* bytes_cached, size_t* device_allocs) {
     const PoolStats s = Runtime::instance().pool().stats();
