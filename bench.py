@@ -46,8 +46,11 @@ def dev(a):
 class Workload:
     """name, algorithmic flops and bytes per step, a run() closure, and a verify() closure."""
 
-    def __init__(self, name, flops, bytes_, run, verify, bound, desc):
+    def __init__(self, name, flops, bytes_, run, verify, bound, desc, another=None):
         self.name, self.flops, self.bytes, self.run, self.verify, self.bound, self.desc = name, flops, bytes_, run, verify, bound, desc
+        # another(): allocates one more independent set of the large operands and the output (same values)
+        # and returns a run() closure over it -- for the rotated-buffer timing of the memory-bound workloads
+        self.another = another
 
 
 def tolerance(orc, got, truth, tag):
@@ -108,8 +111,11 @@ def make_workload(name, orc, capi):
             truth = np.maximum(orc.gemm_f64(X[:256], Wt, trans_b=True) + bias[None, :].astype(np.float64), 0)
             return tolerance(orc, out[:256].cpu().numpy(), truth, name)
 
+        def another():
+            return capi.prepare_gemm(Xd.clone(), Wd.clone(), torch.empty_like(out), b_trans=True, bias=bd, bias_strides=(0, 1), relu=True)
+
         return Workload(name, 2.0 * Nb * IN * OUT, 4.0 * (Nb * IN + IN * OUT + OUT + Nb * OUT), run, verify, "mfma",
-                        "Linear X[4096,1024] W[4096,1024]^T + bias, ReLU"), None
+                        "Linear X[4096,1024] W[4096,1024]^T + bias, ReLU", another), None
     if name == "linear_bwd":
         # backward of Model::Linear at the L config: W[1,1,OUT,IN] * x[n,1,IN,1] -> dW += dY^T X, dx += dY W
         Nb, IN, OUT = 4096, 1024, 4096
@@ -226,8 +232,11 @@ def make_workload(name, orc, capi):
         def verify():
             return tolerance(orc, out.cpu().numpy(), orc.gemm_f64(a, Bm), name)
 
+        def another():
+            return capi.prepare_gemm(ad.clone(), Bd.clone(), torch.empty_like(out))
+
         return Workload(name, 2.0 * 4096 * 4096, 4.0 * (4096 + 4096 * 4096 + 4096), run, verify, "hbm",
-                        "A[1,4096] * B[4096,4096]"), None
+                        "A[1,4096] * B[4096,4096]", another), None
     if name == "ragged":
         A = orc.fill((1000, 777), 3, "uniform", -1.0, 1.0)
         B = orc.fill((777, 513), 1003, "uniform", -1.0, 1.0)
@@ -260,10 +269,17 @@ def make_workload(name, orc, capi):
             truth = orc.conv2d_direct_f64(x[:1], w, bias, 1, 1, relu=True)
             return tolerance(orc, out[:1].cpu().numpy(), truth, name)
 
+        def another():
+            x2, out2 = xd.clone(), torch.empty_like(out)
+
+            def run2():
+                capi.conv2d_forward(x2, wd, bd, 3, 3, 1, 1, bias_strides=(0, 1), relu=True, out=out2)
+            return run2
+
         flops = 2.0 * N * H * W * C * 9 * O
         bytes_ = 4.0 * (N * C * H * W + O * C * 9 + O + N * O * H * W)
         return Workload(name, flops, bytes_, run, verify, "hbm",
-                        f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},3,3] s1 p1 + bias + ReLU"), None
+                        f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},3,3] s1 p1 + bias + ReLU", another), None
     if name == "adam":
         # opt::Adam::step over 2^26 parameters: data, m, v read and written, the gradient read
         n = 1 << 26
@@ -351,10 +367,26 @@ def make_workload(name, orc, capi):
     raise ValueError(name)
 
 
+SETTLE_SECONDS = 0.25
+
+
+def settle(run, seconds=SETTLE_SECONDS):
+    """Untimed: keeps the GPU on the workload for a quarter of a second before the warm-up steps. After an
+    idle period the power management first overshoots and then throttles (the 8192^3 kernel runs 0.93, 1.18,
+    ... ms over its first twenty calls before it levels out at 0.90 ms); the metric is the steady rate."""
+    import torch
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            run()
+        torch.cuda.synchronize()
+
+
 def time_steps(wl, steps, warmup):
     """Times exactly `steps` runs with HIP events recorded on the stream the kernels are
     launched on (torch's current stream), bracketed by device synchronisation."""
     import torch
+    settle(wl.run)
     for _ in range(warmup):
         wl.run()
     torch.cuda.synchronize()
@@ -367,6 +399,42 @@ def time_steps(wl, steps, warmup):
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     return start.elapsed_time(stop) / steps, wall * 1e3 / steps      # ms per step (device events, host wall)
+
+
+ROTATE_MIN_BYTES = 640 << 20
+
+
+def time_rotated(wl, steps, warmup):
+    """Steady-state loop over k >= 4 independent operand/output sets, more than 640 MiB in total, used round
+    robin: by the time a set comes round again every byte of it has left the 32 MiB of L2 and the 256 MiB
+    memory-side cache, so the rate is that of HBM. Returns (ms per step, k)."""
+    import torch
+    k = max(4, int(ROTATE_MIN_BYTES // wl.bytes) + 1)
+    runs = [wl.run] + [wl.another() for _ in range(k - 1)]
+    steps = max(steps, 2 * k)
+    for i in range(max(warmup, k)):
+        runs[i % k]()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        runs[i % k]()
+    stop.record()
+    torch.cuda.synchronize()
+    del runs
+    return start.elapsed_time(stop) / steps, k
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or "unknown"
 
 
 def time_cold(wl, iters=10):
@@ -404,7 +472,7 @@ def cpu_baseline_gemm(orc, A, B, rows=8192):
         dt = time.perf_counter() - t0
         best = dt if best is None or dt < best else best
     return {"value": 2.0 * rows * n * B.shape[1] / best / 1e12, "unit": "TFLOP/s", "cores": orc.num_threads(),
-            "kind": "port", "sample": f"the whole 8192^3 GEMM ({rows}x8192x8192 incl. rounding both operands), best of 3, {best:.2f} s each"}
+            "cpu_model": cpu_model(), "kind": "port", "sample": f"the whole 8192^3 GEMM ({rows}x8192x8192 incl. rounding both operands), best of 3, {best:.2f} s each"}
 
 
 def main():
@@ -450,7 +518,7 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "linear", "gemv", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "adam",
+        for name in ("conv_b", "conv_a", "linear", "gemv", "ragged", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "adam",
                      "softmax_bwd", "matmul_f32"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)
@@ -461,6 +529,17 @@ def main():
                            "TFLOP/s": w2.flops / ms2 / 1e9, "GB/s": w2.bytes / ms2 / 1e6,
                            "frac_mfma_peak": w2.flops / ms2 / 1e9 / PEAK_TFLOPS_FP16,
                            "frac_hbm_peak": w2.bytes / ms2 / 1e6 / PEAK_HBM_GBPS, "verified": v2, "workload": w2.desc}
+            if w2.another is not None:
+                # the HBM figure proper: operands rotated through more memory than the caches hold; the
+                # same-buffer loop above re-reads a working set that the 256 MiB memory-side cache can serve
+                ms_rot, k = time_rotated(w2, max(10, args.steps // 2), max(3, args.warmup // 2))
+                e = extra[name]
+                e["frac_hbm_peak_same_buffers"] = e["frac_hbm_peak"]
+                e.update({"ms_rotated_buffers": ms_rot, "rotated_sets": k, "rotated_bytes": k * w2.bytes,
+                          "GB/s_rotated_buffers": w2.bytes / ms_rot / 1e6,
+                          "frac_hbm_peak": w2.bytes / ms_rot / 1e6 / PEAK_HBM_GBPS,
+                          "frac_mfma_peak_rotated_buffers": w2.flops / ms_rot / 1e9 / PEAK_TFLOPS_FP16})
+                torch.cuda.empty_cache()
             if w2.bound == "valu_fp32":
                 del extra[name]["frac_mfma_peak"]
                 extra[name]["frac_fp32_vector_peak"] = w2.flops / ms2 / 1e9 / PEAK_TFLOPS_FP32
@@ -490,6 +569,7 @@ def main():
         "unit": "GB/s" if wl.bound == "hbm" else "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_dev, "ms_per_step_host_wall": ms_wall,
+        "untimed_settle_s_before_warmup": SETTLE_SECONDS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "dtype_note": "fp32 operands rounded to fp16 (RNE), fp16 MFMA, fp32 accumulate and output",
         "data": "synthetic",

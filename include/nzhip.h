@@ -291,9 +291,18 @@ int nzhip_compress(float* out, const float* in, size_t n, size_t batches, void* 
 
 /* ---- runtime: device allocator + stream manager -------------------------- */
 /* Replace cuStrm::StreamManager<float> (include/NeuZephyr/StreamManager.cuh:131-911) and
- * EventPool (EventPool.cuh:165-457).  One ordered compute stream carries every kernel and
- * every stream-ordered allocation, so producer/consumer order needs no per-buffer events;
- * nzhip_sync_ptr / nzhip_sync_all are the only blocking calls. */
+ * EventPool (EventPool.cuh:165-457).  One ordered compute stream, nzhip_default_stream(), carries
+ * the runtime's copies, memsets and stream-ordered allocations, so producer/consumer order on
+ * it needs no per-buffer events.
+ *
+ * Precondition: the runtime only knows about work on ITS stream.  Memory from nzhip_malloc is
+ * handed out, cached and re-issued in the order of that stream, and nzhip_sync_ptr,
+ * nzhip_memcpy_* and nzhip_memset are ordered on it.  A caller that passes another stream to a
+ * compute entry point whose operands came from nzhip_malloc must call nzhip_stream_wait(stream)
+ * before it frees, copies, clears or synchronises those operands through the runtime (and must
+ * order the other direction itself, e.g. by synchronising before the compute call).  The nz::
+ * C++ layer always computes on nzhip_default_stream() and needs none of this.  Workspaces the
+ * library takes internally are tagged with the caller's stream and never migrate. */
 void* nzhip_default_stream(void);                 /* the manager's compute stream (hipStream_t) */
 int nzhip_malloc(void** ptr, size_t bytes);       /* StreamManager::malloc (:230-240); size in BYTES */
 int nzhip_free_async(void* ptr);                  /* StreamManager::freeAsync (:325-335): stream-ordered, cached */
@@ -302,7 +311,14 @@ int nzhip_memset(void* ptr, int value, size_t bytes);                 /* :360 */
 int nzhip_memcpy_h2d(void* dst, const void* src, size_t bytes);       /* :391, async w.r.t. device */
 int nzhip_memcpy_d2d(void* dst, const void* src, size_t bytes);
 int nzhip_memcpy_d2h(void* dst, const void* src, size_t bytes);       /* blocks until the copy landed */
-int nzhip_sync_ptr(const void* ptr);              /* StreamManager::syncData (:714): wait for work touching ptr */
+/* StreamManager::syncData (:714).  Blocks until nzhip_default_stream() has drained, which covers
+ * every piece of work that touches ptr provided the precondition above is kept; ptr itself is
+ * not looked at. */
+int nzhip_sync_ptr(const void* ptr);
+/* StreamManager::streamWait (:840-850), per stream instead of per buffer: everything enqueued
+ * later on nzhip_default_stream() (frees and the re-issue of freed blocks, copies, memsets,
+ * kernels) runs after everything enqueued so far on `stream`.  Does not block the host. */
+int nzhip_stream_wait(void* stream);
 int nzhip_sync_all(void);                         /* StreamManager::sync (:671) */
 /* allocator statistics (bytes handed out, bytes cached, hipMalloc calls so far) */
 int nzhip_allocator_stats(size_t* bytes_in_use, size_t* bytes_cached, size_t* device_allocs);

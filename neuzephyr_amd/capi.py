@@ -23,7 +23,7 @@ EXPORTS = [
     "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
     "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_mse_loss", "nzhip_mse_backward", "nzhip_expand", "nzhip_compress",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
-    "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_sync_all",
+    "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_stream_wait", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
 ]
 
@@ -112,6 +112,7 @@ def load() -> C.CDLL:
     for n in ("nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h"):
         getattr(lib, n).argtypes = [vp, vp, sz]
     lib.nzhip_sync_ptr.argtypes = [vp]
+    lib.nzhip_stream_wait.argtypes = [vp]
     lib.nzhip_allocator_stats.argtypes = [C.POINTER(sz), C.POINTER(sz), C.POINTER(sz)]
     _LIB = lib
     return lib

@@ -518,18 +518,24 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
         }
         wait_vmcnt<(NSTAGE - 2) * LOADS>();    // tile kt+1 has landed (this wave's share)
         wait_lgkmcnt0();                        // this wave's reads of slot kt are complete
+#ifndef ABL_NOBARRIER
         __syncthreads();
+#endif
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = PRE; t < NPOS; t++) {
             mfma_at(t);
+#ifndef ABL_NOLOAD
             if (t - PRE < LOADS) issue_load(kt + NSTAGE, kt % NSTAGE, t - PRE);
+#endif
+#ifndef ABL_NOFRAG
             // last use of B block jj of the first half: position HALF - 4 + jj
             if (t >= HALF - 4 && t < HALF) read_b(nxt, t - (HALF - 4));
             // last use of A block i: position HALF + 4 i + 3
             if (t >= HALF && (t & 3) == 3) read_a(nxt, (t - HALF) / 4);
             // last use of B block 4 + jj: position NPOS - 4 + jj
             if (t >= NPOS - 4) read_b(nxt, 4 + t - (NPOS - 4));
+#endif
             __builtin_amdgcn_sched_barrier(0);
         }
     }

@@ -247,9 +247,24 @@ int nzhip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
 }
 
 int nzhip_sync_ptr(const void* ptr) {
-    (void)ptr;   // one ordered stream: everything that touches ptr is ahead of this point in it
+    (void)ptr;   // everything that touches ptr is ahead of this point in the runtime's stream (see nzhip.h)
     hipError_t e = hipStreamSynchronize(Runtime::instance().stream());
     return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipStreamSynchronize");
+}
+
+int nzhip_stream_wait(void* stream) {
+    Runtime& rt = Runtime::instance();
+    if (int rc = rt.ensure_stream()) return rc;
+    hipStream_t other = static_cast<hipStream_t>(stream);
+    if (other == rt.stream()) return NZHIP_OK;
+    hipEvent_t ev = nullptr;
+    hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+    if (e != hipSuccess) return set_hip_error(e, "hipEventCreateWithFlags");
+    e = hipEventRecord(ev, other);
+    if (e == hipSuccess) e = hipStreamWaitEvent(rt.stream(), ev, 0);
+    const hipError_t e2 = hipEventDestroy(ev);          // released by the runtime once the event has completed
+    if (e != hipSuccess) return set_hip_error(e, "nzhip_stream_wait");
+    return e2 == hipSuccess ? NZHIP_OK : set_hip_error(e2, "hipEventDestroy");
 }
 
 int nzhip_sync_all(void) {

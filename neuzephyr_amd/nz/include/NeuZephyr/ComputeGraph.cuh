@@ -36,7 +36,7 @@ namespace nz::graph {
         // last forward() fused node chains, the skipped intermediates are recomputed first.
         void backward();
         void zeroGrad() const;                           // src/ComputeGraph.cu:434-438
-        void update(opt::Optimizer* optimizer) const;    // one step() per leaf node that requires gradients (:541-547 steps hidden activations too)
+        void update(opt::Optimizer* optimizer) const;    // step() per leaf that requires gradients, skip() per other node the reference would step (:541-547)
         [[nodiscard]] Tensor::value_type getLoss() const;      // of the first output node; throws std::runtime_error without one (:534-539)
         [[nodiscard]] io::OutputNode* getOutputNode() const;   // throws std::runtime_error without exactly one output
         void setFusion(bool enabled);

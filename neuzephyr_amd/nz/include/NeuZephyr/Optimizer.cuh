@@ -20,6 +20,10 @@ namespace nz::opt {
         explicit Optimizer() = default;
         virtual ~Optimizer() = default;
         virtual void step(Node* input) = 0;              // updates input->output from its gradient
+        // Account for a step() the reference would make on `input` without touching its tensor:
+        // ComputeGraph::update calls this for nodes whose output the next forward() overwrites, so that
+        // whatever the optimizer counts per step() call advances exactly as in the reference.
+        virtual void skip(Node* input) { (void)input; }
     };
 
     class DL_API SGD : public Optimizer {
@@ -32,6 +36,7 @@ namespace nz::opt {
     public:
         explicit Adam(Tensor::value_type learning_rate, Tensor::value_type beta1, Tensor::value_type beta2);
         void step(Node* input) override;
+        void skip(Node* input) override;                 // advances the step count only
 
     private:
         Tensor::value_type beta1, beta2;

@@ -283,11 +283,16 @@ namespace nz::graph {
 
     void ComputeGraph::update(opt::Optimizer* optimizer) const {
         // The reference steps every node whose output carries a gradient (:541-547), hidden activations
-        // included. An activation is rewritten in full by the next forward(), so only leaves (parameters and
-        // inputs that require gradients) are stepped here: same parameters after every step, no optimizer pass
-        // and no optimizer state over the activations.
-        for (Node* node : nodes)
-            if (node->inputs.empty() && node->output && node->output->requiresGrad()) optimizer->step(node);
+        // and the output node included. An activation is rewritten in full by the next forward(), so only
+        // leaves (parameters and inputs that require gradients) are stepped here; the others are passed to
+        // skip(), which keeps an optimizer's per-call state in step with the reference: Adam's bias
+        // corrections use the number of step() calls so far (src/Optimizer.cu:86-101), so a leaf must see
+        // the same count as it would there.
+        for (Node* node : nodes) {
+            if (!node->output || !node->output->requiresGrad()) continue;
+            if (node->inputs.empty()) optimizer->step(node);
+            else optimizer->skip(node);
+        }
     }
 
     void ComputeGraph::zeroGrad() const {

@@ -16,6 +16,11 @@ namespace nz::opt {
         this->learning_rate = learning_rate;
     }
 
+    void Adam::skip(Node* input) {
+        (void)input;
+        it++;                                            // the reference counts every step() call (src/Optimizer.cu:87)
+    }
+
     void Adam::step(Node* input) {
         it++;                                            // src/Optimizer.cu:87: one count per call, shared by all nodes
         for (auto* moments : {&m, &v}) {

@@ -609,6 +609,57 @@ TEST(Model, SGDOptimize) {
     EXPECT_EQ(expected, *model.input1.output);                   // gradient was reset by update()
 }
 
+TEST(Model, AdamThroughUpdateCountsStepsLikeTheReference) {
+    // ComputeGraph::update of the reference calls Adam::step for EVERY node whose output carries a gradient
+    // (src/ComputeGraph.cu:541-547), and Adam counts calls, not updates (src/Optimizer.cu:86-101): the t of
+    // a parameter's bias corrections is its position among those nodes, plus their number per earlier update.
+    // Restated here on the host for the two parameters of a Linear layer over two updates.
+    const size_t batch = 6, in = 20, out = 12;
+    LinearModel m(batch, in, out, true);
+    auto x = randomVec(batch * in, 301, -1.f, 1.f), W = randomVec(out * in, 302, -0.5f, 0.5f), b = randomVec(out, 303, -0.3f, 0.3f);
+    m.input.dataInject(x.begin(), x.end());
+    m.parameters()[0]->dataInject(W.begin(), W.end());
+    m.parameters()[1]->dataInject(b.begin(), b.end());
+    const float lr = 0.01f, beta1 = 0.9f, beta2 = 0.999f, eps = 1e-6f;
+    nz::opt::Adam optimizer(lr, beta1, beta2);
+    const auto& nodes = m.graph().getNodes();
+    size_t per_update = 0;
+    std::vector<std::vector<float>> data = {W, b}, mo = {std::vector<float>(W.size(), 0.f), std::vector<float>(b.size(), 0.f)}, ve = mo;
+    for (int update = 0; update < 2; ++update) {
+        m.forward();
+        m.backward();
+        if (update == 0) {                                       // counted once the graph has run: every node has its output
+            for (Node* n : nodes) per_update += n->output && n->output->requiresGrad();
+            EXPECT_TRUE(per_update > 2);                         // hidden activations and the output node count too
+        }
+        std::vector<std::vector<float>> grads;
+        for (int k = 0; k < 2; ++k) grads.push_back(m.parameters()[k]->output->hostGrad());
+        int t = update * (int)per_update;
+        for (Node* n : nodes) {                                   // the reference's loop
+            if (!(n->output && n->output->requiresGrad())) continue;
+            ++t;
+            for (int k = 0; k < 2; ++k) {
+                if (n != m.parameters()[k]) continue;
+                const float c1 = 1.0f - std::pow(beta1, (float)t), c2 = 1.0f - std::pow(beta2, (float)t);
+                for (size_t i = 0; i < data[k].size(); ++i) {
+                    const float g = grads[k][i];
+                    mo[k][i] = mo[k][i] * beta1 + g * (1 - beta1);
+                    ve[k][i] = ve[k][i] * beta2 + g * g * (1 - beta2);
+                    data[k][i] -= lr * (mo[k][i] / c1) / (std::sqrt(ve[k][i] / c2) + eps);
+                }
+            }
+        }
+        m.update(&optimizer);
+    }
+    for (int k = 0; k < 2; ++k) {
+        const auto got = m.parameters()[k]->output->hostData();
+        double worst = 0;
+        for (size_t i = 0; i < got.size(); ++i) worst = std::max(worst, (double)std::fabs(got[i] - data[k][i]));
+        // counting only the stepped leaves instead (t = 2 where the reference has 3) moves entries by about 4e-3
+        EXPECT_TRUE(worst < 2e-5);
+    }
+}
+
 TEST(Model, LinearTrainingStepLowersTheOutputSum) {
     // forward -> backward (d(sum of outputs)) -> SGD: the sum of the outputs must go down
     LinearModel m(16, 40, 24, false);
