@@ -101,8 +101,15 @@ size_t nzhip_static_scratch_bytes(void);
  * caller instead of by the shape, so that every kernel can be checked on every shape.
  * tile 128 / 256: the fused convert-on-load kernel with that square tile; 16 / 18 / 12: the two-pass
  * fp16 route with 256x256 tiles on 4 waves / 256x256 tiles on 8 waves / 128x256 tiles, 16x16x32 MFMAs;
- * 316 / 318 / 312: the same three with 32x32x16 MFMAs.  Any other value: NZHIP_E_INVALID. */
+ * 316 / 318 / 312: the same three with 32x32x16 MFMAs; 28: the single-kernel route for very large
+ * products (rounding overlapped with the MFMA loop; NZHIP_E_UNSUPPORTED unless M and N are multiples of
+ * 4096 and K of 1024).  Any other value: NZHIP_E_INVALID. */
 int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream);
+/* Diagnostic (no counterpart in the reference): in the single-kernel route workgroups wait for each
+ * other's rounding work with a bounded number of polls; *count receives how many waits have run out
+ * since the library was loaded.  Anything but 0 means a product may be wrong (a device with fewer than
+ * 256 free compute units).  Blocks until the device is idle. */
+int nzhip_gemm_coop_timeouts(unsigned* count);
 
 /* Drop-in for nz::data::iTensorCoreGEMM (include/NeuZephyr/TensorOperations.cuh:1021-1022,
  * src/TensorOperations.cu:112-115 -> krnl::TensorCoreGEMMParallel, src/OperationKernels.cu:914-1026):

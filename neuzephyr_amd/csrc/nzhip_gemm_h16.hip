@@ -518,24 +518,18 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
         }
         wait_vmcnt<(NSTAGE - 2) * LOADS>();    // tile kt+1 has landed (this wave's share)
         wait_lgkmcnt0();                        // this wave's reads of slot kt are complete
-#ifndef ABL_NOBARRIER
         __syncthreads();
-#endif
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = PRE; t < NPOS; t++) {
             mfma_at(t);
-#ifndef ABL_NOLOAD
             if (t - PRE < LOADS) issue_load(kt + NSTAGE, kt % NSTAGE, t - PRE);
-#endif
-#ifndef ABL_NOFRAG
             // last use of B block jj of the first half: position HALF - 4 + jj
             if (t >= HALF - 4 && t < HALF) read_b(nxt, t - (HALF - 4));
             // last use of A block i: position HALF + 4 i + 3
             if (t >= HALF && (t & 3) == 3) read_a(nxt, (t - HALF) / 4);
             // last use of B block 4 + jj: position NPOS - 4 + jj
             if (t >= NPOS - 4) read_b(nxt, 4 + t - (NPOS - 4));
-#endif
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -591,6 +585,345 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
     }
 }
 
+// ---- both passes in one kernel for very large products --------------------------------------------
+// The rounding pass is memory-bound and the MFMA pass leaves most of the HBM bandwidth idle, so for
+// products with many tiles the two are overlapped: the workgroups of the GEMM round, inside their k
+// loops, the operand blocks that will be needed NEXT, and counters in memory tell a workgroup when
+// the blocks it is about to request have been written by everybody.
+//
+// Schedule. The grid is cut into waves of 256 workgroups (one per CU); wave w computes the 16 x 16
+// tile block (sbm, sbn) of C, the blocks taken in boustrophedon order so that consecutive waves
+// share the A rows or the B columns. A k loop is cut into panels of COOP_KP k tiles. Stage (w, p) is
+// the set of fp16 image blocks that wave w needs in panel p and that no earlier wave needed (the A
+// blocks of a tile-block row when it is entered, the B blocks only in the first tile-block row).
+// Stage (0, 0) is rounded by coop_prologue_kernel; every other stage is rounded by the 256
+// workgroups of the wave that runs just before it is needed: stage (w, p + 1) during panel p of
+// wave w, stage (w + 1, 0) during the last panel of wave w. A stage has at most 32 x COOP_KP blocks,
+// i.e. at most 4 per workgroup, 16 fp32 values per thread and block.
+//
+// A block goes global fp32 -> registers -> fp16 in a 16 KiB LDS staging area (the same image layout
+// as cvt_block writes) -> linear 16-byte stores, spread over four k tiles. The stores carry the sc1
+// bit (device scope: they are written through the L2 of the writing XCD, which the other XCDs do
+// not snoop); once a wave's stores have completed (vmcnt 0) and the workgroup has met at the k
+// loop's barrier, one lane adds 1 to the stage's counter with a device-scope atomic. A consumer reads
+// the counter with a device-scope load a few k tiles before it needs the stage and, in the normal
+// case, finds 256 there; otherwise it sleeps and polls, at most spin_limit times (then it counts a
+// time-out in g_coop_timeouts and goes on, so every wave always reaches the end of the kernel). No
+// cache invalidation is needed on the consumer side: a block's lines cannot be in a cache before
+// they are first requested, they are first requested after the counter has been seen complete, and
+// all caches are invalidated at kernel boundaries.
+// Completion of stage (w, 0) implies completion of every earlier stage (its producers have passed
+// the checks of all stages before it), so the one check a workgroup makes before its first request
+// covers the operand blocks that earlier waves rounded.
+// Progress: a workgroup only waits for workgroups with a smaller wave number or of its own wave, and
+// workgroups are dispatched in order, so with one workgroup per CU and at least 256 CUs nobody waits
+// for a workgroup that cannot start.
+constexpr int COOP_KP = 32, COOP_SB = 16, COOP_WG = COOP_SB * COOP_SB;
+
+struct CoopArgs {
+    H16Args g;
+    const float* srcA;
+    const float* srcB;
+    long lda, ldb;
+    unsigned* flags;            // one arrival counter per stage; zeroed by coop_prologue_kernel
+    int sn;                     // tile blocks along N
+    int waves, panels;
+    unsigned spin_limit;
+};
+
+__device__ unsigned g_coop_timeouts;   // polls that gave up (0 unless the device is shared or smaller than assumed)
+
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) void coop_prologue_kernel(CvtOperand a, CvtOperand b, int a_blocks, int K, int nkt,
+                                                            unsigned* flags, int n_flags) {
+    __shared__ __attribute__((aligned(16))) char img[CVT_BLOCK_BYTES];
+    if (blockIdx.x == 0 && blockIdx.y == 0)
+        for (int i = threadIdx.x; i < n_flags; i += 256) flags[i] = 0;
+    const int rb = blockIdx.y;
+    if (rb < a_blocks)
+        cvt_block<A_KC>(img, a, K, nkt, 16, blockIdx.x, rb, 0);
+    else
+        cvt_block<B_KC>(img, b, K, nkt, 16, blockIdx.x, rb - a_blocks, 0);
+}
+
+// phys_row_of for 16-row blocks and fr = 1 << lg blocks per wave tile
+__device__ __forceinline__ int phys_row16(int r, int lg) {
+    const int w = r >> (4 + lg), l = r & ((16 << lg) - 1);
+    return (((w << lg) + (l & ((1 << lg) - 1))) << 4) + (l >> lg);
+}
+
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
+    constexpr int BM = 256, BN = 256, WN = 2, NSTAGE = 4, ROWB = 64;
+    constexpr int TM = 64, TN = 128, FM = TM / 16, FN = TN / 16;
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int A_LOADS = 2, B_LOADS = 2, LOADS = A_LOADS + B_LOADS;
+    constexpr int RING = NSTAGE * STAGE;
+    const H16Args& p = q.g;
+
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    char* const stg = lds + RING;                              // 32 KiB staging area of the rounding work
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+    const int l16 = lane & 15, lq = lane >> 4;
+
+    // wave of workgroups, slot in it, tile
+    const int wv = blockIdx.x / COOP_WG, slot = blockIdx.x % COOP_WG;
+    auto block_of = [&](int w, int& sbm, int& sbn, bool& new_a, bool& new_b) {
+        sbm = w / q.sn;
+        const int j = w - sbm * q.sn;
+        sbn = (sbm & 1) ? q.sn - 1 - j : j;
+        new_a = j == 0;
+        new_b = sbm == 0;
+    };
+    int sbm, sbn;
+    bool unused_a, unused_b;
+    block_of(wv, sbm, sbn, unused_a, unused_b);
+    const int xcd = slot & 7, sq = slot >> 3;                  // workgroups go to the XCDs round-robin: 4 x 8 tiles per XCD
+    const int tile_m = sbm * COOP_SB + (xcd & 3) * 4 + (sq & 3);
+    const int tile_n = sbn * COOP_SB + (xcd >> 2) * 8 + (sq >> 2);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    const _Float16* __restrict__ A = p.A;
+    const _Float16* __restrict__ B = p.B;
+    float* __restrict__ C = p.C;
+    const int nk = p.Kp / CVT_K;
+    const char* a_tile = reinterpret_cast<const char*>(A) + (long)tile_m * nk * A_BYTES + wave * A_LOADS * 1024 + lane * 16;
+    const char* b_tile = reinterpret_cast<const char*>(B) + (long)tile_n * nk * B_BYTES + wave * B_LOADS * 1024 + lane * 16;
+
+    auto issue_load = [&](int kt, int stage, int r) {
+        const int kc = kt < nk ? kt : nk - 1;
+        const bool is_a = r < A_LOADS;
+        const int j = is_a ? r : r - A_LOADS;
+        char* dst = lds + stage * STAGE + (is_a ? 0 : A_BYTES) + (wave * (is_a ? A_LOADS : B_LOADS) + j) * 1024;
+        const char* src = is_a ? a_tile + (long)kc * A_BYTES + j * 1024 : b_tile + (long)kc * B_BYTES + j * 1024;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    };
+
+    constexpr int HALF = FM * 4, NPOS = 2 * HALF;
+    floatx4 acc[NPOS];
+#pragma unroll
+    for (int t = 0; t < NPOS; t++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[t][r] = 0.f;
+
+    const int frag_off = l16 * ROWB + ((lq ^ chunk_swizzle(l16)) << 4);
+    const int a_off = (wm * FM) * 16 * ROWB + frag_off;
+    const int b_off = A_BYTES + (wn * FN) * 16 * ROWB + frag_off;
+    half8_t af[FM], bf[FN];
+    auto read_a = [&](const char* base, int i) { af[i] = *reinterpret_cast<const half8_t*>(base + a_off + i * 16 * ROWB); };
+    auto read_b = [&](const char* base, int j) { bf[j] = *reinterpret_cast<const half8_t*>(base + b_off + j * 16 * ROWB); };
+    auto mfma_at = [&](int t) {
+        const int h = t / HALF, i = (t % HALF) / 4, j = 4 * h + (t & 3);
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[t]) : "v"(af[i]), "v"(bf[j]));
+    };
+
+    // ---- stage counters -------------------------------------------------------------------------
+    auto flag_of = [&](int w, int pn) { return q.flags + (long)w * q.panels + pn; };
+    auto wait_stage = [&](unsigned seen, unsigned* flag) {      // wave 0 only; seen: an earlier reading of *flag
+        unsigned v = __builtin_amdgcn_readfirstlane(seen);
+        unsigned polls = 0;
+        while (v < (unsigned)COOP_WG) {
+            __builtin_amdgcn_s_sleep(16);
+            v = __builtin_amdgcn_readfirstlane(__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            if (++polls > q.spin_limit) {
+                if (lane == 0) atomicAdd(&g_coop_timeouts, 1u);
+                break;
+            }
+        }
+    };
+
+    // ---- rounding work of this workgroup --------------------------------------------------------
+    // Per panel up to four blocks, one every four k tiles. k tile it, it & 3 == 0: the block's 32 KiB of
+    // fp32 are requested straight into the staging area (global_load_lds, four 1 KiB pieces per wave: rows
+    // of 32 k values when k is contiguous in the source, k rows of 256 values otherwise); the requests sit
+    // in front of that k tile's ring requests; requests complete in order, so the ring's own wait three k
+    // tiles later (at most 8 requests outstanding) covers them, and the two waits in between allow 12.
+    // it & 3 == 3: every thread reads the 8 values of one 16-byte piece of the image from the staging area,
+    // rounds them and stores the piece, twice; thread t takes pieces t and 512 + t of the block, so a wave
+    // writes 1 KiB runs.
+    char* cv_dst = nullptr;                                   // image block in hand (uniform), null = none
+    const char* cv_src = nullptr;                             // this lane's first 16 source bytes of it
+    long cv_step = 0;                                         // bytes between the wave's four pieces
+    int cv_kc = 0, cv_lg = 2;                                 // k contiguous in the source; log2(blocks per wave tile)
+    int t_w = 0, t_p = 0, t_na = 0, t_nb = 0, t_sbm = 0, t_sbn = 0;   // the stage being produced in this panel
+    bool t_any = false;
+    auto begin_panel = [&](int pn) {                          // which stage do we produce during panel pn?
+        t_any = false;
+        if (pn + 1 < q.panels) { t_w = wv; t_p = pn + 1; t_any = true; }
+        else if (wv + 1 < q.waves) { t_w = wv + 1; t_p = 0; t_any = true; }
+        if (t_any) {
+            bool na, nb;
+            block_of(t_w, t_sbm, t_sbn, na, nb);
+            t_na = na ? COOP_SB : 0;
+            t_nb = nb ? COOP_SB : 0;
+        }
+    };
+    auto begin_block = [&](int n) {                            // n-th block of this workgroup in the stage (uniform)
+        const int i = slot + COOP_WG * n;
+        cv_dst = nullptr;
+        if (!t_any || i >= (t_na + t_nb) * COOP_KP) return;
+        const int r = i / COOP_KP, kt = t_p * COOP_KP + i % COOP_KP;
+        const bool is_a = r < t_na;
+        auto setup = [&](const float* S, const long ld, const _Float16* img, const int rb, const bool kc, const int lg) {
+            cv_kc = kc;
+            cv_lg = lg;
+            const long r0 = (long)rb * CVT_ROWS, k0 = (long)kt * CVT_K;
+            if (kc) {       // piece j of wave v: rows 32 v + 8 j .. + 8, lane l -> row + l / 8, k + 4 (l & 7)
+                cv_src = reinterpret_cast<const char*>(S + (r0 + wave * 32 + (lane >> 3)) * ld + k0 + 4 * (lane & 7));
+                cv_step = 8 * ld * 4;
+            } else {        // piece j of wave v: k row 4 v + j, lane l -> 4 rows from 4 l
+                cv_src = reinterpret_cast<const char*>(S + (k0 + wave * 4) * ld + r0 + 4 * lane);
+                cv_step = ld * 4;
+            }
+            cv_dst = const_cast<char*>(reinterpret_cast<const char*>(img)) + ((long)rb * nk + kt) * CVT_BLOCK_BYTES;
+        };
+        // FM = 4 and FN = 8 blocks of 16 rows per wave tile: the images interleave their rows accordingly
+        if (is_a) setup(q.srcA, q.lda, A, t_sbm * COOP_SB + r, A_KC, 2);
+        else setup(q.srcB, q.ldb, B, t_sbn * COOP_SB + (r - t_na), B_KC, 3);
+    };
+    auto cv_request = [&]() {                                  // 4 KiB per wave: staging bytes [4096 v, 4096 v + 4096)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(cv_src + j * cv_step),
+                                             (__attribute__((address_space(3))) void*)(stg + wave * 4096 + j * 1024), 16, 0, 2);   // aux 2 = nt: streamed once, keep it from displacing the tiles in L2
+    };
+    auto cv_round = [&](int j) {                               // image piece 512 j + t: staging -> registers -> memory
+        const int c = j * 512 + tid, pr = c >> 2;
+        const int chunk = (c & 3) ^ chunk_swizzle(pr);         // logical 8-wide k chunk held at this position
+        // logical row of physical row pr (inverse of phys_row16)
+        const int blk16 = pr >> 4, in_blk = pr & 15;
+        const int lr = ((blk16 >> cv_lg) << (4 + cv_lg)) + (in_blk << cv_lg) + (blk16 & ((1 << cv_lg) - 1));
+        float x[8];
+        if (cv_kc) {
+            const floatx4 lo = *reinterpret_cast<const floatx4*>(stg + lr * 128 + chunk * 32);
+            const floatx4 hi = *reinterpret_cast<const floatx4*>(stg + lr * 128 + chunk * 32 + 16);
+#pragma unroll
+            for (int e = 0; e < 4; e++) { x[e] = lo[e]; x[4 + e] = hi[e]; }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = *reinterpret_cast<const float*>(stg + (chunk * 8 + e) * 1024 + lr * 4);
+        }
+        half8_t h;
+#pragma unroll
+        for (int e = 0; e < 8; e++) h[e] = (_Float16)x[e];
+        // device-scope store (sc1): written through the L2 of this XCD. The no-op keeps the data registers
+        // untouched for the cycles in which the store still reads them.
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(cv_dst + c * 16), "v"(h) : "memory");
+    };
+
+    // ---- prologue ---------------------------------------------------------------------------------
+    if (wv > 0 && wave == 0)
+        wait_stage(__hip_atomic_load(flag_of(wv, 0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), flag_of(wv, 0));
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < NSTAGE; t++)
+#pragma unroll
+        for (int r = 0; r < LOADS; r++) issue_load(t, t, r);
+    wait_vmcnt<(NSTAGE - 1) * LOADS>();
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < FN; j++) read_b(lds, j);
+#pragma unroll
+    for (int i = 0; i < FM; i++) read_a(lds, i);
+
+    // ---- k loop -----------------------------------------------------------------------------------
+    // it: k tile within the panel. DRAIN_IT: every wave waits for its stores, then (behind the barrier)
+    // one lane signals; POLL_IT: wave 0 reads the counter of the next panel's stage; CHECK_IT: the k
+    // tile in which the first requests of the next panel are issued.
+    constexpr int PRE = HALF - 4 - LOADS;
+    constexpr int DRAIN_IT = 18, POLL_IT = COOP_KP - 7, CHECK_IT = COOP_KP - NSTAGE;
+    static_assert(DRAIN_IT > 16 && DRAIN_IT < POLL_IT && POLL_IT + 2 < CHECK_IT, "schedule");
+    unsigned polled = 0;
+    auto k_tile = [&](const int kt, const int slot_c, const int ph) {   // slot_c = kt % NSTAGE, ph = kt & 3 (compile time)
+        const int it = kt & (COOP_KP - 1), pn = kt / COOP_KP;
+        const char* nxt = lds + ((slot_c + 1) % NSTAGE) * STAGE;
+#pragma unroll
+        for (int t = 0; t < PRE; t++) {
+            mfma_at(t);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (it == DRAIN_IT) wait_vmcnt<0>();                  // this wave's image stores are in memory
+        else if ((ph == 1 || ph == 2) && it < 16 && cv_dst) wait_vmcnt<(NSTAGE - 2) * LOADS + 4>();   // + the staging requests of this block
+        else wait_vmcnt<(NSTAGE - 2) * LOADS>();              // tile kt+1 has landed (this wave's share)
+        wait_lgkmcnt0();
+        if (it == CHECK_IT && pn + 1 < q.panels && wave == 0) wait_stage(polled, flag_of(wv, pn + 1));
+        // A bare barrier: the waits above name exactly what has to be complete. __syncthreads() would add a
+        // workgroup fence, which here (ordinary global loads and stores are in flight) drains every request.
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        if (it == DRAIN_IT && t_any && tid == 0)
+            __hip_atomic_fetch_add(flag_of(t_w, t_p), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (it == POLL_IT && pn + 1 < q.panels && wave == 0)
+            polled = __hip_atomic_load(flag_of(wv, pn + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (ph == 0 && it < 16) {                             // in front of this k tile's ring requests
+            if (it == 0) begin_panel(pn);
+            begin_block(it >> 2);
+            if (cv_dst) cv_request();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int t = PRE; t < NPOS; t++) {
+            mfma_at(t);
+            if (t - PRE < LOADS) issue_load(kt + NSTAGE, slot_c, t - PRE);
+            if (t >= HALF - 4 && t < HALF) read_b(nxt, t - (HALF - 4));
+            if (t >= HALF && (t & 3) == 3) read_a(nxt, (t - HALF) / 4);
+            if (t >= NPOS - 4) read_b(nxt, 4 + t - (NPOS - 4));
+            __builtin_amdgcn_sched_barrier(0);
+            if ((t == PRE + LOADS || t == HALF + 5) && ph == 3 && it < 16 && cv_dst) {
+                cv_round(t == PRE + LOADS ? 0 : 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    for (int kt = 0; kt < nk; kt += 4) {
+        k_tile(kt, 0, 0);
+        k_tile(kt + 1, 1, 1);
+        k_tile(kt + 2, 2, 2);
+        k_tile(kt + 3, 3, 3);
+    }
+    wait_vmcnt<0>();
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue (whole tiles only: M and N are multiples of the tile) -----------------------------
+    const float* bias = p.bias;
+    const int gn = n0 + wn * TN + l16 * FN;
+    float bcol[FN];
+    const bool bias_rowless = bias && p.bias_sm == 0;
+#pragma unroll
+    for (int j = 0; j < FN; j++) bcol[j] = bias_rowless ? bias[(long)(gn + j) * p.bias_sk] : 0.f;
+#pragma unroll
+    for (int i = 0; i < FM; i++) {
+        float bv[4][FN];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int gm = m0 + wm * TM + (lq * 4 + r) * FM + i;
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                bv[r][j] = (bias && !bias_rowless) ? bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk] : bcol[j];
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int gm = m0 + wm * TM + (lq * 4 + r) * FM + i;
+            float v[FN];
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                float x = acc[(j >> 2) * HALF + i * 4 + (j & 3)][r] + bv[r][j];
+                if (p.relu) x = x > 0.f ? x : 0.f;
+                v[j] = x;
+            }
+            float* dst = C + (long)gm * p.ldc + gn;
+            floatx4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
+            *reinterpret_cast<floatx4*>(dst) = o0;
+            *reinterpret_cast<floatx4*>(dst + 4) = o1;
+        }
+    }
+}
+
 // ---- host side -----------------------------------------------------------------------------
 static inline long round_up(long v, long q) { return (v + q - 1) / q * q; }
 
@@ -608,6 +941,86 @@ bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
     const bool whole_tiles = d.M % 256 == 0 && d.N % 256 == 0 && d.K % 32 == 0 && d.lda % 4 == 0 && d.ldb % 4 == 0 &&
                              d.ldc % 4 == 0;
     return flops / cvt_bytes >= (whole_tiles ? 512.0 : 300.0);
+}
+
+// The single-kernel route wants one unbatched product of whole 16 x 16 tile blocks and whole panels, 16-byte
+// accesses everywhere, at least two stages to overlap, and a device on which a wave of 256 workgroups is
+// resident at once (one workgroup per CU).
+bool gemm_h16_coop_applicable(const nzhip_gemm_desc& d) {
+    constexpr int64_t BLOCK = (int64_t)COOP_SB * 256, PANEL = (int64_t)COOP_KP * CVT_K;
+    if (d.batch_n * d.batch_c != 1) return false;
+    if (d.M < BLOCK || d.N < BLOCK || d.M % BLOCK || d.N % BLOCK || d.K % PANEL) return false;
+    const int64_t waves = (d.M / BLOCK) * (d.N / BLOCK), panels = d.K / PANEL;
+    if (waves * panels < 2 || waves > 16384) return false;
+    if (d.lda % 4 || d.ldb % 4 || d.ldc % 4) return false;
+    if ((reinterpret_cast<uintptr_t>(d.A) | reinterpret_cast<uintptr_t>(d.B) | reinterpret_cast<uintptr_t>(d.C)) & 15) return false;
+    return device_cu_count() == COOP_WG;
+}
+
+int gemm_h16_coop_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
+    const long Mp = d.M, Np = d.N, Kp = d.K;
+    const bool a_kc = d.a_layout != NZHIP_LAYOUT_TRANS, b_kc = d.b_layout == NZHIP_LAYOUT_TRANS;
+    const size_t a_elems = (size_t)Mp * Kp, b_elems = (size_t)Np * Kp;
+    const int nkt = (int)(Kp / CVT_K), panels = nkt / COOP_KP;
+    const int sm = (int)(Mp / (COOP_SB * 256)), sn = (int)(Np / (COOP_SB * 256)), waves = sm * sn;
+    const int n_flags = waves * panels;
+    const size_t img_bytes = (a_elems + b_elems) * sizeof(_Float16);
+    char* ws = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&ws), img_bytes + (size_t)n_flags * sizeof(unsigned), s)) return rc;
+    _Float16* Ah = reinterpret_cast<_Float16*>(ws);
+    _Float16* Bh = Ah + a_elems;
+    unsigned* flags = reinterpret_cast<unsigned*>(ws + img_bytes);
+
+    auto operand = [&](_Float16* dst, const float* src, long R, long ld, int fr) {
+        CvtOperand o;
+        o.dst = dst; o.src = src; o.R = (int)R; o.ld = ld;
+        o.src_batch = 0; o.dst_batch = 0; o.vec = 1; o.fr = fr;
+        return o;
+    };
+    const CvtOperand oa = operand(Ah, d.A, d.M, d.lda, 4), ob = operand(Bh, d.B, d.N, d.ldb, 8);
+    CoopArgs a;
+    H16Args& g = a.g;
+    g.A = Ah; g.B = Bh; g.C = d.C; g.bias = d.bias;
+    g.M = (int)d.M; g.N = (int)d.N; g.Kp = (int)Kp; g.ldc = d.ldc;
+    g.batch_c = 1; g.batch = 1; g.a_batch = g.b_batch = 0;
+    g.a_bcast_n = g.a_bcast_c = g.b_bcast_n = g.b_bcast_c = 1;
+    g.a_cn = g.b_cn = 1;
+    g.c_sn = g.c_sc = g.bias_sn = g.bias_sc = 0;
+    g.bias_sm = d.bias_stride_row; g.bias_sk = d.bias_stride_col;
+    g.relu = d.activation == NZHIP_ACT_RELU;
+    g.tiles_m = (int)(Mp / 256); g.tiles_n = (int)(Np / 256); g.group_m = 4;
+    a.srcA = d.A; a.srcB = d.B; a.lda = d.lda; a.ldb = d.ldb;
+    a.flags = flags; a.sn = sn; a.waves = waves; a.panels = panels;
+    a.spin_limit = 200000;                                             // x (16 sleeps + one read): a few hundred ms
+
+    // stage (0, 0): the first 16 row blocks of both operands over the first panel; also clears the counters
+    dim3 pgrid((unsigned)COOP_KP, (unsigned)(2 * COOP_SB), 1);
+    constexpr size_t lds_bytes = 4 * (256 + 256) * 64 + 2 * CVT_BLOCK_BYTES;   // ring + fp32 staging = all 160 KiB
+    int rc = NZHIP_OK;
+#define NZHIP_COOP(AK, BK)                                                                                         \
+    do {                                                                                                           \
+        hipLaunchKernelGGL((coop_prologue_kernel<AK, BK>), pgrid, dim3(256), 0, s, oa, ob, COOP_SB, (int)d.K, nkt, \
+                           flags, n_flags);                                                                        \
+        auto kfn = gemm_h16c_kernel<AK, BK>;                                                                       \
+        rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(gemm_h16c)"); \
+        if (rc == NZHIP_OK) hipLaunchKernelGGL(kfn, dim3((unsigned)(waves * COOP_WG)), dim3(512), lds_bytes, s, a); \
+    } while (0)
+    if (a_kc && b_kc) NZHIP_COOP(true, true);
+    else if (a_kc) NZHIP_COOP(true, false);
+    else if (b_kc) NZHIP_COOP(false, true);
+    else NZHIP_COOP(false, false);
+#undef NZHIP_COOP
+    if (rc == NZHIP_OK) {
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "gemm_h16c kernel launch");
+    }
+    int rc2 = workspace_free(ws, s);
+    return rc ? rc : rc2;
+}
+
+int gemm_h16_coop_timeouts(unsigned* count) {
+    hipError_t e = hipMemcpyFromSymbol(count, HIP_SYMBOL(g_coop_timeouts), sizeof(unsigned));
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipMemcpyFromSymbol(g_coop_timeouts)");
 }
 
 int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mfma) {

@@ -22,6 +22,10 @@ bool gemm_h16_applicable(const nzhip_gemm_desc& d);
 bool gemm_vec_legal(const nzhip_gemm_desc& d);   // 16-byte global accesses are legal for A, B and C
 // waves: 0 = choose, else 2 / 4 / 8; mfma: 0 = choose, else 16 (16x16x32) / 32 (32x32x16)
 int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int waves = 0, int mfma = 0);
+// Both passes in one kernel (rounding overlapped with the MFMA loop) for products of whole 4096 x 4096 x 1024 blocks.
+bool gemm_h16_coop_applicable(const nzhip_gemm_desc& d);
+int gemm_h16_coop_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
+int gemm_h16_coop_timeouts(unsigned* count);     // polls that gave up since the library was loaded (expected: 0)
 // Bandwidth-bound kernels for M <= 8 (nzhip_skinny.hip).
 int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
 bool gemm_skinny_applicable(const nzhip_gemm_desc& d);

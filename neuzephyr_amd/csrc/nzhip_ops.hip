@@ -424,6 +424,9 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
     // NZHIP_GEMM_ROUTE=fused|h16 overrides the route choice (benchmarking only).
     static const char* route = getenv("NZHIP_GEMM_ROUTE");
     const bool force_fused = route && route[0] == 'f', force_h16 = route && route[0] == 'h';
+    static const char* coop_env = getenv("NZHIP_H16_COOP");              // 0: never the single-kernel route (benchmarking only)
+    const bool allow_coop = !(coop_env && atoi(coop_env) == 0);
+    if (!force_fused && allow_coop && gemm_h16_coop_applicable(d)) return gemm_h16_coop_dispatch(d, s);
     if (!force_fused && (force_h16 || gemm_h16_applicable(d))) return gemm_h16_dispatch(d, s);
     return gemm_mfma_dispatch(d, s, 0);
 }
@@ -435,15 +438,25 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
 int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream) {
     if (!desc) return set_error(NZHIP_E_INVALID, "nzhip_gemm: null descriptor");
     const int base = tile > 300 ? tile - 300 : tile;
-    if (tile != 128 && tile != 256 && base != 16 && base != 18 && base != 12)
-        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128, 256, 16, 18, 12, 316, 318 or 312");
+    if (tile != 128 && tile != 256 && tile != 28 && base != 16 && base != 18 && base != 12)
+        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128, 256, 16, 18, 12, 28, 316, 318 or 312");
     if (int rc = validate_gemm(*desc)) return rc;
     if (desc->M == 0 || desc->N == 0 || desc->K == 0) return nzhip_gemm(desc, stream);
     const int mfma = tile > 300 ? 32 : 16;
+    if (tile == 28) {
+        if (!gemm_h16_coop_applicable(*desc))
+            return set_error(NZHIP_E_UNSUPPORTED, "nzhip_gemm_force_tile: the single-kernel route needs one product of whole 4096 x 4096 x 1024 blocks");
+        return gemm_h16_coop_dispatch(*desc, as_stream(stream));
+    }
     if (base == 16) return gemm_h16_dispatch(*desc, as_stream(stream), 4, mfma);
     if (base == 18) return gemm_h16_dispatch(*desc, as_stream(stream), 8, mfma);
     if (base == 12) return gemm_h16_dispatch(*desc, as_stream(stream), 2, mfma);
     return gemm_mfma_dispatch(*desc, as_stream(stream), tile);
+}
+
+int nzhip_gemm_coop_timeouts(unsigned* count) {
+    if (!count) return set_error(NZHIP_E_INVALID, "nzhip_gemm_coop_timeouts: null pointer");
+    return gemm_h16_coop_timeouts(count);
 }
 
 int nzhip_tensorcore_gemm(const float* A, const float* B, float* C, const size_t sA[4], const size_t sB[4],

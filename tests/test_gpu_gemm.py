@@ -113,6 +113,39 @@ def test_long_contractions_with_few_tiles_are_bit_exact_on_integers(nz, M, K, N,
     assert np.array_equal(got, expect)
 
 
+COOP = [(4096, 2048, 4096), (8192, 1024, 4096), (4096, 1024, 8192), (8192, 2048, 8192)]
+
+
+@pytest.mark.parametrize("M,K,N", COOP)
+@pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
+def test_single_kernel_route_is_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans):
+    # the route for very large products (rounding done inside the k loops of the GEMM, stage counters between
+    # workgroups): one wave of tiles with two panels; two waves that share B, or A; four waves in boustrophedon
+    # order. Bias matrix and ReLU ride along; no wait may have run out.
+    import ctypes as C
+    import torch
+    gen = torch.Generator(device="cuda").manual_seed(M + 3 * K + 7 * N + 2 * a_trans + b_trans)
+    A = torch.randint(-4, 5, (K, M) if a_trans else (M, K), generator=gen, device="cuda").float()
+    B = torch.randint(-4, 5, (N, K) if b_trans else (K, N), generator=gen, device="cuda").float()
+    bias = torch.randint(-50, 51, (M, N), generator=gen, device="cuda").float()
+    expect = torch.relu(((A.T if a_trans else A).double() @ (B.T if b_trans else B).double()).float() + bias)   # |sums| < 2^24: exact
+    got = nz.gemm(A, B, a_trans=a_trans, b_trans=b_trans, bias=bias, bias_strides=(N, 1), relu=True, force_tile=28)
+    assert torch.equal(got, expect)
+    again = nz.gemm(A, B, a_trans=a_trans, b_trans=b_trans, bias=bias, bias_strides=(N, 1), relu=True)      # default route: the same one
+    assert torch.equal(again, expect)
+    n = C.c_uint(123)
+    nz.check(nz.load().nzhip_gemm_coop_timeouts(C.byref(n)))
+    assert n.value == 0
+
+
+def test_single_kernel_route_rejects_other_shapes(nz):
+    import torch
+    A, B = torch.zeros((4096, 1000), device="cuda"), torch.zeros((1000, 4096), device="cuda")
+    with pytest.raises(nz.NzHipError) as e:
+        nz.gemm(A, B, force_tile=28)
+    assert e.value.status == -3
+
+
 def _route_sweep_cases():
     # seeded shapes aimed at the boundaries of the route choice: skinny extents 1..9 on either side,
     # long contractions with few tiles (split or not, vectorisable or not), mid-size and ragged shapes,
