@@ -218,13 +218,23 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
     int bx, by, b;
     xcd_contiguous_block(bx, by, b);
     const float* wb = w_ref + (long)b * w_batch_stride;
-    for (int i = threadIdx.x; i < C_T * 9 * O_T; i += 256) wsm[i] = round_f16(wb[i]);   // [q][o]
-    __syncthreads();
+    static_assert(C_T * 9 * O_T <= 128, "one weight per thread");
+    // requested now, parked in LDS after the first input rows have been requested (the rows then do not
+    // queue up behind the round trip of the weights)
+    const float w_mine = threadIdx.x < C_T * 9 * O_T ? wb[threadIdx.x] : 0.f;
+    auto park_weights = [&]() {
+        if (threadIdx.x < C_T * 9 * O_T) wsm[threadIdx.x] = round_f16(w_mine);   // [q][o]
+        __syncthreads();
+    };
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int strip = by * 4 + wave;
     const int w0 = (bx * 64 + lane) * 4;
-    const int h0 = (by * 4 + wave) * ST_ROWS;
-    if (w0 >= W || h0 >= H) return;
+    const int h0 = strip * ST_ROWS;
+    if (w0 >= W || h0 >= H) {                                    // nothing to do but the workgroup's one barrier
+        park_weights();
+        return;
+    }
     const float* xb = x + (long)b * C_T * H * W;
     float* yb = y + (long)b * O_T * H * W;
     const long plane = (long)H * W;
@@ -238,7 +248,7 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
     // start, or both at the end of their walk), so the second request finds it in L2. Walking all
     // strips downwards puts a whole strip's duration between the two uses and the row comes from
     // memory twice. The walk is instantiated once per direction and a wave runs one of the two.
-    const bool rev = ((by * 4 + wave) & 1) != 0;
+    const bool rev = (strip & 1) != 0;
     auto walk = [&](auto upwards) {
     constexpr bool UP = decltype(upwards)::value;
     const int row_first = UP ? h0 + rows : h0 - 1, row_step = UP ? -1 : 1;
@@ -287,6 +297,7 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
 
 #pragma unroll
     for (int t = 0; t < ST_AHEAD; t++) request(t, raw[t], braw[t]);
+    park_weights();
 
     static_assert(ST_AHEAD % 3 == 0, "the request ring must be a whole number of windows");
     for (int t0 = 0; t0 < T; t0 += ST_AHEAD) {
