@@ -34,6 +34,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary (conv / linear) measurements")
     ap.add_argument("--no-verify", action="store_true")
+    ap.add_argument("--no-settle", action="store_true",
+                    help="profiling runs: skip the untimed settle phase, so that a kernel trace holds warm-up + timed steps only")
     return ap.parse_args()
 
 
@@ -382,11 +384,12 @@ def settle(run, seconds=SETTLE_SECONDS):
         torch.cuda.synchronize()
 
 
-def time_steps(wl, steps, warmup):
+def time_steps(wl, steps, warmup, do_settle=True):
     """Times exactly `steps` runs with HIP events recorded on the stream the kernels are
     launched on (torch's current stream), bracketed by device synchronisation."""
     import torch
-    settle(wl.run)
+    if do_settle:
+        settle(wl.run)
     for _ in range(warmup):
         wl.run()
     torch.cuda.synchronize()
@@ -491,7 +494,7 @@ def main():
     capi.load()
 
     wl, host_ops = make_workload(args.workload, orc, capi)
-    ms_dev, ms_wall = time_steps(wl, args.steps, args.warmup)
+    ms_dev, ms_wall = time_steps(wl, args.steps, args.warmup, not args.no_settle)
     verified = None if args.no_verify else wl.verify()
 
     tflops = wl.flops / (ms_dev * 1e-3) / 1e12
@@ -569,7 +572,7 @@ def main():
         "unit": "GB/s" if wl.bound == "hbm" else "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_dev, "ms_per_step_host_wall": ms_wall,
-        "untimed_settle_s_before_warmup": SETTLE_SECONDS,
+        "untimed_settle_s_before_warmup": 0.0 if args.no_settle else SETTLE_SECONDS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "dtype_note": "fp32 operands rounded to fp16 (RNE), fp16 MFMA, fp32 accumulate and output",
         "data": "synthetic",

@@ -143,6 +143,7 @@ namespace nz::graph {
                     if (i2c->stride == 1 && i2c->kernelHeight == i2c->kernelWidth && i2c->padding <= i2c->kernelHeight - 1) {
                         Node* pre = add ? static_cast<Node*>(add) : static_cast<Node*>(mm);   // holds [N,1,HW,O] gradients
                         back = [=] {
+                            if (!last->output->requiresGrad()) return;     // nothing in the chain carries a gradient
                             const bool needW = rhs->output->requiresGrad();
                             const bool needB = biasNode && biasNode->output->requiresGrad();
                             const size_t pixels = c2i->outputHeight * c2i->outputWidth;
@@ -217,10 +218,30 @@ namespace nz::graph {
                     const size_t batch = rs[0], in = ls[3], out = ls[2];
                     std::vector<Node*> members = {mm, add};
                     if (relu) members.push_back(last);
+                    // Backward of the whole chain from the fused output alone: the activation mask comes from y
+                    // (y > 0 exactly where the ReLU's input was), the bias gradient is the batch sum of the masked
+                    // gradient (Add.backward), and MatMul.backward takes it as dC directly. The node chain would
+                    // first have to recompute the MatMul and Add outputs the fused forward never wrote.
+                    std::function<void()> back = [=] {
+                        if (!last->output->requiresGrad()) return;
+                        float* dZ = last->output->grad();
+                        if (relu) {
+                            float* masked = add->output->gradOverwrite();     // every element written
+                            iReLUBackward(masked, last->output->data(), dZ, last->output->size());
+                            dZ = masked;
+                        }
+                        if (biasNode->output->requiresGrad())
+                            iAddBackward(biasNode->output->grad(), dZ, biasNode->output->shape(), add->output->shape());
+                        const bool needW = lhs->output->requiresGrad(), needX = rhs->output->requiresGrad();
+                        if (needW || needX)
+                            iMatMulBackward(needW ? lhs->output->grad() : nullptr, needX ? rhs->output->grad() : nullptr,
+                                            lhs->output->data(), rhs->output->data(), dZ, lhs->output->shape(),
+                                            rhs->output->shape(), mm->output->shape());
+                    };
                     addGroup(std::move(members), [=] {
                         iLinearForward(last->output->data(), rhs->output->data(), lhs->output->data(),
                                        biasNode->output->data(), batch, in, out, relu);
-                    });
+                    }, std::move(back));
                 }
             }
         }

@@ -149,12 +149,12 @@ namespace nz::data {
 
     static float meanLoss(float* predict, float* real, const size_t n, const bool bce) {
         void* dev = nullptr;
-        NZ_CHECK(nzhip_malloc(&dev, sizeof(float)));
+        NZ_CHECK(nzhip_malloc(&dev, sizeof(float)));                         // from the pool's cache after the first call
         float host = 0.f;
         int rc = bce ? nzhip_bce_loss(static_cast<float*>(dev), predict, real, n, nzhip_default_stream())
                      : nzhip_mse_loss(static_cast<float*>(dev), predict, real, n, nzhip_default_stream());
         if (rc == 0) rc = nzhip_memcpy_d2h(&host, dev, sizeof(float));      // blocks until the value is here
-        const int rc2 = nzhip_free(dev);
+        const int rc2 = nzhip_free_async(dev);                               // the copy has completed: back to the cache, no device-wide sync
         NZ_CHECK(rc);
         NZ_CHECK(rc2);
         return host;
@@ -200,8 +200,10 @@ namespace nz::data {
                                 const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
                                 const size_t pad, const size_t weightBatch) {
         if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1) return false;
-        NZ_CHECK(nzhip_conv2d_backward_weights(dw, x, dy, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch,
-                                               nzhip_default_stream()));
+        const int rc = nzhip_conv2d_backward_weights(dw, x, dy, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch,
+                                                     nzhip_default_stream());
+        if (rc == NZHIP_E_UNSUPPORTED) return false;      // extents beyond the fused kernel: the caller takes the column-matrix route
+        NZ_CHECK(rc);
         return true;
     }
 

@@ -518,6 +518,54 @@ TEST(Model, Conv2dFusedBackwardEqualsNodeChain) {
     convBackwardFusedEqualsChain(2, 40, 10, 136, 36, 3, 1, 1, true);  // W a multiple of 8: weights without the column matrix
 }
 
+struct LinearGradModel : nz::Model {
+    InputNode input;
+    LinearGradModel(size_t batch, size_t features, size_t out, bool relu) : input({batch, 1, features, 1}, true) {
+        Node* x = Linear(&input, out);
+        if (relu) x = ReLU(x);
+        defaultOutput(x);
+    }
+};
+
+TEST(Model, LinearFusedBackwardEqualsNodeChain) {
+    // integer-valued data: every gradient is exact, so the fused backward (mask from y, bias gradient and
+    // MatMul.backward straight from the masked gradient) must equal the node-by-node backward bit for bit,
+    // twice in a row (gradients are cleared in between)
+    for (const bool relu : {true, false}) {
+        const size_t batch = 9, in = 40, out = 24;
+        LinearGradModel m(batch, in, out, relu);
+        auto ints = [](size_t count, unsigned seed, int lo, int hi) {
+            auto v = randomVec(count, seed, static_cast<float>(lo), static_cast<float>(hi) + 0.999f);
+            for (auto& e : v) e = std::floor(e);
+            return v;
+        };
+        auto x = ints(batch * in, 71, -3, 3), W = ints(out * in, 72, -2, 2), b = ints(out, 73, -4, 4);
+        m.input.dataInject(x.begin(), x.end());
+        m.parameters()[0]->dataInject(W.begin(), W.end());
+        m.parameters()[1]->dataInject(b.begin(), b.end());
+        std::vector<float> dx, dW, db;
+        for (int pass = 0; pass < 2; ++pass) {
+            m.graph().zeroGrad();
+            m.forward();
+            EXPECT_EQ(m.graph().fusedGroupCount(), 1u);
+            m.backward();
+            dx = m.input.output->hostGrad();
+            dW = m.parameters()[0]->output->hostGrad();
+            db = m.parameters()[1]->output->hostGrad();
+        }
+        m.graph().setFusion(false);
+        m.graph().zeroGrad();
+        m.forward();
+        m.backward();
+        EXPECT_TRUE(m.input.output->hostGrad() == dx);
+        EXPECT_TRUE(m.parameters()[0]->output->hostGrad() == dW);
+        EXPECT_TRUE(m.parameters()[1]->output->hostGrad() == db);
+        bool any = false;
+        for (float v : dW) any = any || v != 0.f;
+        EXPECT_TRUE(any);
+    }
+}
+
 // ---- fp32 matmul and optimizers (test/Test.cpp:119-184, 2230-2265, 2398-2452, 2816-2878) ------------
 TEST(TensorBasic, TensorMultiplicationTest) {
     Tensor tensor1({2, 1, 2, 3});
