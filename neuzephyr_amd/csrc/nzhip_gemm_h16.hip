@@ -49,6 +49,11 @@ __device__ __forceinline__ int phys_row_of(int r, int fr, int blk) {
     const int tr = blk * fr, w = r / tr, l = r % tr;
     return (w * fr + (l % fr)) * blk + (l / fr);
 }
+// the inverse: logical tile row held at physical row pr
+__device__ __forceinline__ int logical_row_of(int pr, int fr, int blk) {
+    const int b = pr / blk, in = pr % blk;
+    return (b / fr) * (blk * fr) + in * fr + (b % fr);
+}
 
 // K_CONTIG: source element (r, k) at src[r*ld + k]; otherwise at src[k*ld + r].
 struct CvtOperand {
@@ -68,11 +73,14 @@ __device__ __forceinline__ void cvt_block(char* img, const CvtOperand& o, int K,
     const int t = threadIdx.x;
     const int r0 = rb * CVT_ROWS, k0 = kt * CVT_K;
     if (K_CONTIG) {
-        // 8 threads per row (one float4 each), 32 rows per pass
+        // 8 threads per row (one float4 each), 32 rows per pass. The threads walk the PHYSICAL rows of the
+        // image, so a wave's 8-byte stores cover 512 contiguous bytes of LDS (conflict-free); walking the
+        // logical rows puts rows 16 apart (1 KiB, the same banks) into one store instruction. In global
+        // memory a row's 32 values are one 128-byte line either way.
         const int k4 = t & 7, rr = t >> 3;
 #pragma unroll
         for (int pass = 0; pass < 8; pass++) {
-            const int lr = rr + pass * 32, r = r0 + lr, k = k0 + k4 * 4;
+            const int pr_ = rr + pass * 32, lr = logical_row_of(pr_, fr, blk), r = r0 + lr, k = k0 + k4 * 4;
             floatx4 v = {0.f, 0.f, 0.f, 0.f};
             const float* q = s + (long)r * ld + k;
             if (r < R) {
@@ -85,7 +93,7 @@ __device__ __forceinline__ void cvt_block(char* img, const CvtOperand& o, int K,
                 }
             }
             half4_t h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-            const int pr = phys_row_of(lr, fr, blk);
+            const int pr = pr_;
             const int pos = (k4 >> 1) ^ chunk_swizzle(pr);
             *reinterpret_cast<half4_t*>(img + pr * 64 + pos * 16 + (k4 & 1) * 8) = h;
         }
