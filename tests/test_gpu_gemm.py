@@ -138,6 +138,22 @@ def test_single_kernel_route_is_bit_exact_on_integers(nz, M, K, N, a_trans, b_tr
     assert n.value == 0
 
 
+def test_single_kernel_route_bias_forms(nz):
+    # no bias; a per-column vector (the Linear layer's form); a per-row vector; all against the two-kernel route,
+    # which must give the same bits (same tiles, same k order)
+    import torch
+    M, K, N = 4096, 2048, 4096
+    gen = torch.Generator(device="cuda").manual_seed(99)
+    A = (torch.rand((M, K), generator=gen, device="cuda") - 0.5)
+    B = (torch.rand((K, N), generator=gen, device="cuda") - 0.5)
+    col = torch.rand((N,), generator=gen, device="cuda") - 0.5
+    row = torch.rand((M,), generator=gen, device="cuda") - 0.5
+    for kw in (dict(), dict(bias=col, bias_strides=(0, 1), relu=True), dict(bias=row, bias_strides=(1, 0))):
+        one = nz.gemm(A, B, force_tile=28, **kw)
+        two = nz.gemm(A, B, force_tile=18, **kw)
+        assert torch.equal(one, two), kw.keys()
+
+
 def test_single_kernel_route_rejects_other_shapes(nz):
     import torch
     A, B = torch.zeros((4096, 1000), device="cuda"), torch.zeros((1000, 4096), device="cuda")
