@@ -94,6 +94,32 @@ def test_skinny_products_are_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans
     assert np.array_equal(got, expect)
 
 
+def test_skinny_split_contraction_back_to_back(nz):
+    # the streaming kernel's blocks leave partial sums in a pooled workspace that a second kernel adds: calls of
+    # different shapes, queued without a wait between them on two streams, must not see each other's partials
+    import torch
+    shapes = [(1, 4096, 4096), (2, 3000, 700), (1, 4096, 4096), (1, 777, 513), (2, 1024, 260)]
+    side = torch.cuda.Stream()
+    todo = []
+    for rep in range(3):
+        for i, (M, K, N) in enumerate(shapes):
+            rng = np.random.default_rng(rep * 100 + i)
+            A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+            B = rng.integers(-8, 9, size=(K, N)).astype(np.float32)
+            todo.append((dev(A), dev(B), (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)))
+    torch.cuda.synchronize()
+    outs = []
+    for j, (Ad, Bd, _) in enumerate(todo):
+        if j % 2:
+            with torch.cuda.stream(side):
+                outs.append(nz.gemm(Ad, Bd, stream=side))
+        else:
+            outs.append(nz.gemm(Ad, Bd))
+    torch.cuda.synchronize()
+    for (_, _, expect), got in zip(todo, outs):
+        assert np.array_equal(host(got), expect)
+
+
 SPLITK = [(130, 9000, 70), (576, 16384, 128), (64, 4096, 64), (33, 20001, 300), (128, 8192, 129),
           (10, 70000, 16), (16, 33000, 10)]       # a handful of outputs, hundreds of chunks: one wave per output adds them
 
