@@ -314,6 +314,12 @@ void* nzhip_default_stream(void);                 /* the manager's compute strea
 int nzhip_malloc(void** ptr, size_t bytes);       /* StreamManager::malloc (:230-240); size in BYTES */
 int nzhip_free_async(void* ptr);                  /* StreamManager::freeAsync (:325-335): stream-ordered, cached */
 int nzhip_free(void* ptr);                        /* StreamManager::free (:263): blocks until users finished */
+/* Page-locked host memory mapped into the device, the storage of nz::data::MappedTensor
+ * (src/MappedTensor.cu:88-96: cudaMallocHost; StreamManager::freeHost, StreamManager.cuh:299-302).
+ * The pointer is valid on the host and as an operand of every compute entry point; kernels then
+ * read and write it over the host link. nzhip_host_free waits for nzhip_default_stream() first. */
+int nzhip_host_malloc(void** ptr, size_t bytes);
+int nzhip_host_free(void* ptr);
 int nzhip_memset(void* ptr, int value, size_t bytes);                 /* :360 */
 int nzhip_memcpy_h2d(void* dst, const void* src, size_t bytes);       /* :391, async w.r.t. device */
 int nzhip_memcpy_d2d(void* dst, const void* src, size_t bytes);

@@ -22,7 +22,7 @@ EXPORTS = [
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
     "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
     "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_mse_loss", "nzhip_mse_backward", "nzhip_expand", "nzhip_compress",
-    "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_memset",
+    "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_host_malloc", "nzhip_host_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_stream_wait", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
 ]
@@ -109,6 +109,8 @@ def load() -> C.CDLL:
     lib.nzhip_malloc.argtypes = [C.POINTER(vp), sz]
     lib.nzhip_free_async.argtypes = [vp]
     lib.nzhip_free.argtypes = [vp]
+    lib.nzhip_host_malloc.argtypes = [C.POINTER(vp), sz]
+    lib.nzhip_host_free.argtypes = [vp]
     lib.nzhip_memset.argtypes = [vp, C.c_int, sz]
     for n in ("nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h"):
         getattr(lib, n).argtypes = [vp, vp, sz]
@@ -139,7 +141,9 @@ def _stream_handle(stream=None) -> int:
 
 def _dev(t):
     import torch
-    assert t.is_cuda and t.dtype == torch.float32 and t.is_contiguous(), "expects contiguous fp32 CUDA tensors"
+    # page-locked host tensors are mapped into the device at the same address and are legal operands
+    assert (t.is_cuda or t.is_pinned()) and t.dtype == torch.float32 and t.is_contiguous(), \
+        "expects contiguous fp32 CUDA (or pinned host) tensors"
     return t.data_ptr()
 
 

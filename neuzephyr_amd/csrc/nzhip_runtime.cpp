@@ -217,6 +217,28 @@ int nzhip_free(void* ptr) {
     return NZHIP_OK;
 }
 
+int nzhip_host_malloc(void** ptr, size_t bytes) {
+    if (!ptr) return set_error(NZHIP_E_INVALID, "nzhip_host_malloc: null out-pointer");
+    *ptr = nullptr;
+    if (bytes == 0) return NZHIP_OK;
+    if (int rc = Runtime::instance().ensure_stream()) return rc;
+    // page-locked and mapped: the same address is valid on the host and in kernels
+    hipError_t e = hipHostMalloc(ptr, bytes, hipHostMallocMapped | hipHostMallocPortable);
+    if (e != hipSuccess) {
+        *ptr = nullptr;
+        return set_error(NZHIP_E_NOMEM, "nzhip_host_malloc: %zu bytes: hipError_t %d", bytes, (int)e);
+    }
+    return NZHIP_OK;
+}
+
+int nzhip_host_free(void* ptr) {
+    if (!ptr) return NZHIP_OK;
+    hipError_t e = hipStreamSynchronize(Runtime::instance().stream());     // kernels may still read or write it
+    if (e != hipSuccess) return set_hip_error(e, "hipStreamSynchronize");
+    e = hipHostFree(ptr);
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipHostFree");
+}
+
 int nzhip_memset(void* ptr, int value, size_t bytes) {
     if (!ptr && bytes) return set_error(NZHIP_E_INVALID, "nzhip_memset: null pointer");
     hipError_t e = hipMemsetAsync(ptr, value, bytes, Runtime::instance().stream());

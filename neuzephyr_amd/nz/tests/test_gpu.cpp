@@ -65,6 +65,117 @@ TEST(TensorCore, TensorCoreGEMMTest) {
     EXPECT_TRUE(result.hostData() == kExpected);             // exact, not merely within 1e-5
 }
 
+// MappedTensor operands: the kernels of the path read and write page-locked host memory through the same
+// pointers the host iterates over (reference: test/Test.cpp:2571-2598 computes its expectation this way).
+TEST(MappedTensorPath, TensorCoreGEMMOnMappedOperands) {
+    MappedTensor a({2, 1, 2, 3}), b({1, 3, 3, 2}), c({2, 3, 2, 2});
+    a.dataInject(kData1.begin(), kData1.end());
+    b.dataInject(kData2.begin(), kData2.end());
+    GEMMTensorCore(c, a, b);
+    std::vector<float> got(c.begin(), c.end());               // begin() waits for the kernel
+    EXPECT_TRUE(got == kExpected);
+    for (size_t i = 0; i < kExpected.size(); ++i) EXPECT_EQ(c[i], kExpected[i]);
+    // the same through a device-resident Tensor
+    Tensor ta({2, 1, 2, 3}), tb({1, 3, 3, 2}), tc({2, 3, 2, 2});
+    ta.dataInject(a.begin(), a.end());
+    tb.dataInject(b.begin(), b.end());
+    GEMMTensorCore(tc, ta, tb);
+    EXPECT_TRUE(tc.hostData() == got);
+}
+
+TEST(MappedTensorPath, MatMulReluAddChainEqualsTheNodeGraph) {
+    // the chain of test/Test.cpp:2594-2597: GEMMTensorCore -> ReLU -> + on mapped tensors against the nodes
+    MappedTensor x({2, 3, 4, 5}), w({1, 3, 5, 1}), bias({2, 3, 4, 1});
+    const auto xv = randomVec(x.size(), 11, -10.f, 10.f), wv = randomVec(w.size(), 12, -10.f, 10.f),
+               bv = randomVec(bias.size(), 13, -10.f, 10.f);
+    x.dataInject(xv.begin(), xv.end());
+    w.dataInject(wv.begin(), wv.end());
+    bias.dataInject(bv.begin(), bv.end());
+    MappedTensor product({2, 3, 4, 1});
+    GEMMTensorCore(product, x, w);
+    auto activated = ReLU(product);
+    auto sum = activated + bias;
+
+    InputNode in({2, 3, 4, 5}), wn({1, 3, 5, 1}), bn({2, 3, 4, 1});
+    in.dataInject(xv.begin(), xv.end());
+    wn.dataInject(wv.begin(), wv.end());
+    bn.dataInject(bv.begin(), bv.end());
+    MatMulNode mm(&in, &wn);
+    ReLUNode relu(&mm);
+    AddNode add(&relu, &bn);
+    mm.forward();
+    relu.forward();
+    add.forward();
+    EXPECT_TRUE(add.output->hostData() == std::vector<float>(sum.begin(), sum.end()));
+    // and against the host: fp16-rounded operands, wide accumulation
+    std::vector<double> want(sum.size());
+    for (size_t n = 0; n < 2; ++n)
+        for (size_t c = 0; c < 3; ++c)
+            for (size_t h = 0; h < 4; ++h) {
+                double acc = 0;
+                for (size_t k = 0; k < 5; ++k) acc += double(f16(xv[((n * 3 + c) * 4 + h) * 5 + k])) * f16(wv[c * 5 + k]);
+                want[(n * 3 + c) * 4 + h] = std::max(acc, 0.0) + bv[(n * 3 + c) * 4 + h];
+            }
+    EXPECT_TRUE(closeTo(std::vector<float>(sum.begin(), sum.end()), want, 1e-5));
+}
+
+TEST(MappedTensorPath, Img2colCol2imgAndHostMembers) {
+    MappedTensor image({2, 3, 5, 4});
+    const auto iv = randomVec(image.size(), 21, -1.f, 1.f);
+    image.dataInject(iv.begin(), iv.end());
+    auto cols = tensorImg2col(image, 3, 3, 1, 1);
+    Tensor dimage({2, 3, 5, 4});
+    dimage.dataInject(iv.begin(), iv.end());
+    auto dcols = tensorImg2col(dimage, 3, 3, 1, 1);
+    EXPECT_TRUE(dcols.hostData() == std::vector<float>(cols.begin(), cols.end()));
+    auto back = tensorCol2img(cols, 5, 4);                    // [2,1,20,27] read as 5 x 4 pixels of 27 channels
+    auto dback = tensorCol2img(dcols, 5, 4);
+    EXPECT_TRUE(dback.hostData() == std::vector<float>(back.begin(), back.end()));
+
+    // fp32-exact product and the host-side members
+    MappedTensor p({1, 1, 2, 3}), q({1, 1, 3, 2});
+    p.dataInject({1, 2, 3, 4, 5, 6});
+    q.dataInject({1, 2, 3, 4, 5, 6});
+    auto pq = p * q;
+    EXPECT_TRUE(std::vector<float>(pq.begin(), pq.end()) == (std::vector<float>{22, 28, 49, 64}));
+    MappedTensor pt(p);
+    pt.transpose();
+    EXPECT_TRUE(pt.shape() == Dimension(1, 1, 3, 2));
+    EXPECT_TRUE(std::vector<float>(pt.begin(), pt.end()) == (std::vector<float>{1, 4, 2, 5, 3, 6}));
+    EXPECT_EQ((p - p).sum(), 0.f);
+    EXPECT_EQ(p.sum(), 21.f);
+    EXPECT_EQ(p.sum(0, 0), 21.f);
+    auto ratio = p / p;
+    EXPECT_TRUE(std::vector<float>(ratio.begin(), ratio.end()) == std::vector<float>(6, 1.f));
+    auto neg = -p;
+    EXPECT_EQ(neg[5], -6.f);
+    EXPECT_TRUE(p == MappedTensor(p));
+    EXPECT_TRUE(p != neg);
+    EXPECT_THROW(p[6], std::out_of_range);
+    EXPECT_THROW(p.grad(), std::invalid_argument);
+    EXPECT_THROW(p.clearGrad(), std::runtime_error);
+    p.setRequiresGrad(true);
+    p.fill(2.f, true);
+    EXPECT_EQ(p.grad()[3], 2.f);
+    p.fillMatrix(7.f, 0, 0);
+    EXPECT_EQ(p[0], 7.f);
+    p.reshape({1, 1, 2, 4});
+    EXPECT_EQ(p[5], 7.f);
+    EXPECT_EQ(p[7], 0.f);
+    p.randomize(5);
+    for (float v : p) EXPECT_TRUE(v > 0.f && v <= 1.f);
+    std::istringstream text("1 2 3 4 5 6 7 8");
+    text >> p;
+    EXPECT_EQ(p[7], 8.f);
+    std::ostringstream os;
+    os << p;
+    EXPECT_TRUE(os.str().find("Gradient: ") != std::string::npos);
+    MappedTensor moved(std::move(p));
+    EXPECT_EQ(p.size(), 0u);
+    EXPECT_EQ(moved.size(), 8u);
+    EXPECT_THROW(MappedTensor({1, 1, 2, 3}) + MappedTensor({1, 1, 3, 2}), std::invalid_argument);
+}
+
 TEST(NodeBasic, MatMulForward) {
     InputNode input1({2, 1, 2, 3}), input2({1, 3, 3, 2});
     input1.dataInject(kData1.begin(), kData1.end());

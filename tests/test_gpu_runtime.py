@@ -63,3 +63,37 @@ def test_product_on_a_second_stream_then_free_and_reissue_through_the_runtime(nz
     # waiting for the runtime's own stream is a no-op, a null handle means HIP's null stream
     nz.check(lib.nzhip_stream_wait(lib.nzhip_default_stream()))
     nz.check(lib.nzhip_stream_wait(None))
+
+
+def test_pinned_host_operands(nz):
+    # page-locked host memory is mapped into the device at the same address: the kernels take it as any operand
+    # (the storage of nz::data::MappedTensor); host-memory result == device-memory result, bit for bit
+    import ctypes as C
+    import numpy as np
+    import torch
+    lib = nz.load()
+    rng = np.random.default_rng(5)
+    for (M, K, N) in [(64, 96, 48), (1, 300, 130), (130, 70, 257)]:
+        A = torch.from_numpy(rng.standard_normal((M, K)).astype(np.float32))
+        B = torch.from_numpy(rng.standard_normal((K, N)).astype(np.float32))
+        bias = torch.from_numpy(rng.standard_normal((N,)).astype(np.float32))
+        want = nz.gemm(A.cuda(), B.cuda(), bias=bias.cuda(), bias_strides=(0, 1), relu=True)
+        out = torch.empty((M, N), dtype=torch.float32).pin_memory()
+        got = nz.gemm(A.pin_memory(), B.pin_memory(), bias=bias.pin_memory(), bias_strides=(0, 1), relu=True, out=out)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want.cpu())
+    # the runtime's own host allocator
+    p = C.c_void_p()
+    nz.check(lib.nzhip_host_malloc(C.byref(p), 4096 * 4))
+    host = (C.c_float * 4096).from_address(p.value)
+    for i in range(4096):
+        host[i] = float(i % 17) - 8.0
+    nz.check(lib.nzhip_relu(p, p, 4096, lib.nzhip_default_stream()))
+    nz.check(lib.nzhip_sync_ptr(p))
+    assert all(host[i] == max(float(i % 17) - 8.0, 0.0) for i in range(4096))
+    nz.check(lib.nzhip_relu(p, p, 4096, lib.nzhip_default_stream()))
+    nz.check(lib.nzhip_host_free(p))                            # waits for the kernel, then releases
+    q = C.c_void_p(1)
+    nz.check(lib.nzhip_host_malloc(C.byref(q), 0))
+    assert q.value is None
+    nz.check(lib.nzhip_host_free(None))
