@@ -34,6 +34,7 @@ extern "C" {
 #define NZHIP_E_SHAPE (-2)        /* shapes are not broadcast compatible */
 #define NZHIP_E_UNSUPPORTED (-3)  /* valid request outside implemented limits */
 #define NZHIP_E_NOMEM (-4)        /* device allocation failed */
+#define NZHIP_E_TIMEOUT (-5)      /* an earlier single-kernel product ran out of polls; see nzhip_gemm_coop_timeouts */
 
 #define NZHIP_ACT_NONE 0
 #define NZHIP_ACT_RELU 1          /* x > 0 ? x : 0  (NaN -> 0, -0 -> +0) */
@@ -108,8 +109,14 @@ int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream);
 /* Diagnostic (no counterpart in the reference): in the single-kernel route workgroups wait for each
  * other's rounding work with a bounded number of polls; *count receives how many waits have run out
  * since the library was loaded.  Anything but 0 means a product may be wrong (a device with fewer than
- * 256 free compute units).  Blocks until the device is idle. */
+ * 256 free compute units).  Blocks until the device is idle.
+ * The runtime looks at the same count by itself: the first nzhip_sync_ptr, nzhip_sync_all or
+ * nzhip_memcpy_d2h that has drained the stream of such a product returns NZHIP_E_TIMEOUT once if the
+ * count went up, and from then on nzhip_gemm keeps to the two-kernel route in this process. */
 int nzhip_gemm_coop_timeouts(unsigned* count);
+/* Test hook for that report: adds `inject` to the device-side count as if that many waits had run out
+ * (no kernel misbehaves), or, with inject == 0, forgets earlier time-outs and allows the route again. */
+int nzhip_gemm_coop_reset(unsigned inject);
 
 /* Drop-in for nz::data::iTensorCoreGEMM (include/NeuZephyr/TensorOperations.cuh:1021-1022,
  * src/TensorOperations.cu:112-115 -> krnl::TensorCoreGEMMParallel, src/OperationKernels.cu:914-1026):

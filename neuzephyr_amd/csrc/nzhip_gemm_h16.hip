@@ -11,6 +11,9 @@
 // to fp32 summation order.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <mutex>
+
 #include <cstdlib>
 
 #include "nzhip_internal.h"
@@ -954,7 +957,17 @@ bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
 // The single-kernel route wants one unbatched product of whole 16 x 16 tile blocks and whole panels, 16-byte
 // accesses everywhere, at least two stages to overlap, and a device on which a wave of 256 workgroups is
 // resident at once (one workgroup per CU).
+// Host-side bookkeeping of the bounded waits: which stream the products enqueued since the last look went to,
+// how many time-outs had been seen by then, and whether the route has been given up.
+static std::mutex g_coop_mu;
+static unsigned g_coop_pending = 0;              // single-kernel products enqueued since the last look
+static hipStream_t g_coop_stream = nullptr;      // the stream they all went to ...
+static bool g_coop_mixed = false;                // ... unless they went to several
+static unsigned g_coop_seen = 0;                 // value of g_coop_timeouts at the last look
+static std::atomic<bool> g_coop_off{false};
+
 bool gemm_h16_coop_applicable(const nzhip_gemm_desc& d) {
+    if (g_coop_off.load(std::memory_order_relaxed)) return false;
     constexpr int64_t BLOCK = (int64_t)COOP_SB * 256, PANEL = (int64_t)COOP_KP * CVT_K;
     if (d.batch_n * d.batch_c != 1) return false;
     if (d.M < BLOCK || d.N < BLOCK || d.M % BLOCK || d.N % BLOCK || d.K % PANEL) return false;
@@ -1022,8 +1035,53 @@ int gemm_h16_coop_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "gemm_h16c kernel launch");
     }
+    {
+        std::lock_guard<std::mutex> lock(g_coop_mu);
+        if (g_coop_pending && g_coop_stream != s) g_coop_mixed = true;
+        g_coop_stream = s;
+        g_coop_pending++;
+    }
     int rc2 = workspace_free(ws, s);
     return rc ? rc : rc2;
+}
+
+int gemm_h16_coop_check(hipStream_t drained, bool whole_device) {
+    std::lock_guard<std::mutex> lock(g_coop_mu);
+    if (!g_coop_pending) return NZHIP_OK;
+    if (!whole_device && (g_coop_mixed || g_coop_stream != drained)) return NZHIP_OK;   // may still be running
+    unsigned count = 0;
+    hipError_t e = hipMemcpyFromSymbol(&count, HIP_SYMBOL(g_coop_timeouts), sizeof(unsigned));
+    if (e != hipSuccess) return set_hip_error(e, "hipMemcpyFromSymbol(g_coop_timeouts)");
+    g_coop_pending = 0;
+    g_coop_mixed = false;
+    if (count == g_coop_seen) return NZHIP_OK;
+    const unsigned fresh = count - g_coop_seen;
+    g_coop_seen = count;
+    g_coop_off.store(true, std::memory_order_relaxed);
+    return set_error(NZHIP_E_TIMEOUT,
+                     "nzhip_gemm: %u bounded waits of the single-kernel route ran out (is the device shared?): the result of "
+                     "that product may be wrong; this process uses the two-kernel route from now on",
+                     fresh);
+}
+
+int gemm_h16_coop_reset(unsigned inject) {
+    std::lock_guard<std::mutex> lock(g_coop_mu);
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return set_hip_error(e, "hipDeviceSynchronize");
+    unsigned count = 0;
+    e = hipMemcpyFromSymbol(&count, HIP_SYMBOL(g_coop_timeouts), sizeof(unsigned));
+    if (e != hipSuccess) return set_hip_error(e, "hipMemcpyFromSymbol(g_coop_timeouts)");
+    if (inject) {
+        count += inject;
+        e = hipMemcpyToSymbol(HIP_SYMBOL(g_coop_timeouts), &count, sizeof(unsigned));
+        if (e != hipSuccess) return set_hip_error(e, "hipMemcpyToSymbol(g_coop_timeouts)");
+    } else {
+        g_coop_seen = count;
+        g_coop_pending = 0;
+        g_coop_mixed = false;
+        g_coop_off.store(false, std::memory_order_relaxed);
+    }
+    return NZHIP_OK;
 }
 
 int gemm_h16_coop_timeouts(unsigned* count) {

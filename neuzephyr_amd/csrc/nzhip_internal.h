@@ -25,6 +25,10 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int waves = 
 // Both passes in one kernel (rounding overlapped with the MFMA loop) for products of whole 4096 x 4096 x 1024 blocks.
 bool gemm_h16_coop_applicable(const nzhip_gemm_desc& d);
 int gemm_h16_coop_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
+// After `drained` (or, with whole_device, every stream) has been synchronised: NZHIP_E_TIMEOUT once if a
+// single-kernel product that has finished by now ran out of polls; the route is switched off from then on.
+int gemm_h16_coop_check(hipStream_t drained, bool whole_device);
+int gemm_h16_coop_reset(unsigned inject);
 int gemm_h16_coop_timeouts(unsigned* count);     // polls that gave up since the library was loaded (expected: 0)
 // Bandwidth-bound kernels for M <= 8 (nzhip_skinny.hip).
 int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);

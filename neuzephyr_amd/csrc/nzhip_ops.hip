@@ -445,7 +445,7 @@ int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream) {
     const int mfma = tile > 300 ? 32 : 16;
     if (tile == 28) {
         if (!gemm_h16_coop_applicable(*desc))
-            return set_error(NZHIP_E_UNSUPPORTED, "nzhip_gemm_force_tile: the single-kernel route needs one product of whole 4096 x 4096 x 1024 blocks");
+            return set_error(NZHIP_E_UNSUPPORTED, "nzhip_gemm_force_tile: the single-kernel route needs one product of whole 4096 x 4096 x 1024 blocks (and is off after a time-out)");
         return gemm_h16_coop_dispatch(*desc, as_stream(stream));
     }
     if (base == 16) return gemm_h16_dispatch(*desc, as_stream(stream), 4, mfma);
@@ -458,6 +458,8 @@ int nzhip_gemm_coop_timeouts(unsigned* count) {
     if (!count) return set_error(NZHIP_E_INVALID, "nzhip_gemm_coop_timeouts: null pointer");
     return gemm_h16_coop_timeouts(count);
 }
+
+int nzhip_gemm_coop_reset(unsigned inject) { return gemm_h16_coop_reset(inject); }
 
 int nzhip_tensorcore_gemm(const float* A, const float* B, float* C, const size_t sA[4], const size_t sB[4],
                           const size_t sC[4], void* stream) {

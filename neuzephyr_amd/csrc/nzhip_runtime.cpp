@@ -265,13 +265,17 @@ int nzhip_memcpy_d2h(void* dst, const void* src, size_t bytes) {
     int rc = copy(dst, src, bytes, hipMemcpyDeviceToHost, "nzhip_memcpy_d2h");
     if (rc) return rc;
     hipError_t e = hipStreamSynchronize(Runtime::instance().stream());
+    if (e == hipSuccess) {
+        if (int late = gemm_h16_coop_check(Runtime::instance().stream(), false)) return late;
+    }
     return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipStreamSynchronize");
 }
 
 int nzhip_sync_ptr(const void* ptr) {
     (void)ptr;   // everything that touches ptr is ahead of this point in the runtime's stream (see nzhip.h)
     hipError_t e = hipStreamSynchronize(Runtime::instance().stream());
-    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipStreamSynchronize");
+    if (e != hipSuccess) return set_hip_error(e, "hipStreamSynchronize");
+    return gemm_h16_coop_check(Runtime::instance().stream(), false);
 }
 
 int nzhip_stream_wait(void* stream) {
@@ -291,7 +295,8 @@ int nzhip_stream_wait(void* stream) {
 
 int nzhip_sync_all(void) {
     hipError_t e = hipDeviceSynchronize();
-    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipDeviceSynchronize");
+    if (e != hipSuccess) return set_hip_error(e, "hipDeviceSynchronize");
+    return gemm_h16_coop_check(nullptr, true);
 }
 
 int nzhip_gemm_static(const nzhip_gemm_desc* desc, void* stream) {

@@ -14,6 +14,7 @@ namespace nz::detail {
         if (status == NZHIP_E_SHAPE) throw std::invalid_argument(text && *text ? text : "Shapes are not broadcast compatible.");
         if (status == NZHIP_E_INVALID || status == NZHIP_E_UNSUPPORTED) throw std::invalid_argument(text ? text : "invalid argument");
         if (status == NZHIP_E_NOMEM) throw std::bad_alloc();
+        if (status == NZHIP_E_TIMEOUT) throw std::runtime_error(text && *text ? text : "a GEMM's bounded waits ran out");
         throw nz::CudaException(file, line, status, expr, text);
     }
 }

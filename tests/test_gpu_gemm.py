@@ -188,6 +188,49 @@ def test_single_kernel_route_rejects_other_shapes(nz):
     assert e.value.status == -3
 
 
+def test_single_kernel_route_reports_waits_that_ran_out(nz):
+    # A bounded wait that runs out leaves a product that may be wrong. No kernel is made to misbehave here: the
+    # device-side count is raised from the host after a (correct) product, and the runtime must then say so at
+    # the first blocking call that has drained the product's stream, once, and stop taking the route.
+    import ctypes as C
+    import torch
+    lib = nz.load()
+    M, K, N = 4096, 2048, 4096
+    rng = np.random.default_rng(3)
+    A = dev(rng.integers(-4, 5, size=(M, K)).astype(np.float32))
+    B = dev(rng.integers(-4, 5, size=(K, N)).astype(np.float32))
+    want = nz.gemm(A, B, force_tile=18)
+    torch.cuda.synchronize()
+    nz.check(lib.nzhip_gemm_coop_reset(0))
+    rt = torch.cuda.ExternalStream(lib.nzhip_default_stream())
+    try:
+        got = nz.gemm(A, B, force_tile=28, stream=rt)          # on the runtime's stream: nzhip_sync_ptr covers it
+        nz.check(lib.nzhip_sync_ptr(None))                         # nothing ran out: no complaint
+        assert torch.equal(got, want)
+        got = nz.gemm(A, B, force_tile=28, stream=rt)
+        nz.check(lib.nzhip_gemm_coop_reset(2))                     # "two waits ran out"
+        with pytest.raises(nz.NzHipError) as e:
+            nz.check(lib.nzhip_sync_ptr(None))
+        assert e.value.status == -5 and "2 bounded waits" in str(e.value)
+        nz.check(lib.nzhip_sync_ptr(None))                         # reported once
+        with pytest.raises(nz.NzHipError) as e:                    # the route is off now ...
+            nz.gemm(A, B, force_tile=28)
+        assert e.value.status == -3
+        assert torch.equal(nz.gemm(A, B), want)                    # ... and the default route still multiplies
+        # a product on another stream is only looked at once the whole device has been drained
+        nz.check(lib.nzhip_gemm_coop_reset(0))
+        got = nz.gemm(A, B, force_tile=28)                         # torch's current stream
+        nz.check(lib.nzhip_gemm_coop_reset(1))
+        nz.check(lib.nzhip_sync_ptr(None))
+        with pytest.raises(nz.NzHipError) as e:
+            nz.check(lib.nzhip_sync_all())
+        assert e.value.status == -5
+    finally:
+        nz.check(lib.nzhip_gemm_coop_reset(0))
+    torch.cuda.synchronize()
+    assert torch.equal(nz.gemm(A, B, force_tile=28), want)
+
+
 def _route_sweep_cases():
     # seeded shapes aimed at the boundaries of the route choice: skinny extents 1..9 on either side,
     # long contractions with few tiles (split or not, vectorisable or not), mid-size and ragged shapes,
