@@ -100,7 +100,7 @@ size_t nzhip_static_scratch_bytes(void);
 
 /* Test and benchmark hook (no counterpart in the reference): nzhip_gemm with the kernel chosen by the
  * caller instead of by the shape, so that every kernel can be checked on every shape.
- * tile 128 / 256: the fused convert-on-load kernel with that square tile; 16 / 18 / 12: the two-pass
+ * tile 64 / 128 / 256: the fused convert-on-load kernel with that square tile; 16 / 18 / 12: the two-pass
  * fp16 route with 256x256 tiles on 4 waves / 256x256 tiles on 8 waves / 128x256 tiles, 16x16x32 MFMAs;
  * 316 / 318 / 312: the same three with 32x32x16 MFMAs; 28: the single-kernel route for very large
  * products (rounding overlapped with the MFMA loop; NZHIP_E_UNSUPPORTED unless M and N are multiples of

@@ -40,6 +40,7 @@ struct GemmKernelArgs {
     int tiles_m, tiles_n;
     int group_m;                      // tile rows per rasterisation group
     int k_total;                      // > 0: member j of the inner batch contracts min(K, k_total - j*K) (split-k chunks)
+    int c_vec;                        // 16-byte stores to C are legal (alignment, ldc and N multiples of 4)
 };
 
 // Physical LDS row of logical tile row r. A wave owns TR = 32*FR logical rows; its MFMA
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     // the bias does not vary along rows) so the stores never wait on one load each.
     const float* bias = p.bias ? p.bias + bi * p.bias_sn + bj * p.bias_sc : nullptr;
     const int gn = n0 + wn * TN + li * FN;                // first of this lane's FN columns
-    const bool vec_store = FULL || (VEC && (FN == 2 || FN == 4) && (gn + FN <= p.N));
+    const bool vec_store = FULL || (VEC && p.c_vec && (FN == 2 || FN == 4) && (gn + FN <= p.N));
     float bcol[FN];
     const bool bias_rowless = bias && p.bias_sm == 0;
 #pragma unroll
@@ -387,7 +388,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
 // ---- host-side selection -------------------------------------------------------------------
 template <int BM, int BN, int BK, int WM, int WN>
 static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool vec, int batch, hipStream_t s) {
-    const bool full = vec && a.M % BM == 0 && a.N % BN == 0 && a.K % BK == 0 && (a.k_total <= 0 || a.k_total % a.K == 0);
+    const bool full = vec && a.c_vec && a.M % BM == 0 && a.N % BN == 0 && a.K % BK == 0 && (a.k_total <= 0 || a.k_total % a.K == 0);
     constexpr int ROWB = BK * 2 + 16;
     constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * ROWB;
     dim3 grid((unsigned)((int64_t)a.tiles_m * a.tiles_n * batch), 1, 1), block(WM * WN * 64, 1, 1);
@@ -424,17 +425,76 @@ static int launch_cfg(const GemmKernelArgs& a, bool a_trans, bool b_trans, bool 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // 16-byte accesses are legal when every row start is 16-byte aligned and the contiguous extent is
-// a multiple of 4, for every batch member.
-bool gemm_vec_legal(const nzhip_gemm_desc& d) {
-    const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
+// a multiple of 4, for every batch member: the operands decide which kernel instance loads them,
+// C only whether the epilogue may use vector stores.
+bool gemm_operand_vec_legal(const float* X, int64_t ld, int64_t contig, int64_t stride_n, int64_t stride_c) {
     auto ok4 = [](int64_t v) { return (v & 3) == 0; };
-    const int64_t a_contig = a_trans ? d.M : d.K, b_contig = b_trans ? d.K : d.N;
-    return aligned16(d.A) && aligned16(d.B) && aligned16(d.C) && ok4(d.lda) && ok4(d.ldb) && ok4(d.ldc) &&
-           ok4(a_contig) && ok4(b_contig) && ok4(d.N) && ok4(d.a_stride_n) && ok4(d.a_stride_c) &&
-           ok4(d.b_stride_n) && ok4(d.b_stride_c) && ok4(d.c_stride_n) && ok4(d.c_stride_c);
+    return aligned16(X) && ok4(ld) && ok4(contig) && ok4(stride_n) && ok4(stride_c);
 }
 
-int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile, int64_t k_total) {
+// padded: bit 0 / bit 1 = the rows of A / B are readable up to the next multiple of 4 elements and hold
+// zeros there (the library's own padded copies), so their contiguous extent need not be a multiple of 4
+bool gemm_operands_vec_legal(const nzhip_gemm_desc& d, int padded) {
+    const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
+    return gemm_operand_vec_legal(d.A, d.lda, (padded & 1) ? 0 : (a_trans ? d.M : d.K), d.a_stride_n, d.a_stride_c) &&
+           gemm_operand_vec_legal(d.B, d.ldb, (padded & 2) ? 0 : (b_trans ? d.K : d.N), d.b_stride_n, d.b_stride_c);
+}
+
+bool gemm_c_vec_legal(const nzhip_gemm_desc& d) {
+    return gemm_operand_vec_legal(d.C, d.ldc, d.N, d.c_stride_n, d.c_stride_c);
+}
+
+bool gemm_vec_legal(const nzhip_gemm_desc& d) { return gemm_operands_vec_legal(d, 0) && gemm_c_vec_legal(d); }
+
+// ---- tile and split choice for products that do not fill the device -------------------------------
+// The fused kernel's k loop is bound by the rate at which one CU takes fp32 tiles in through its L1
+// (about 50 GB/s per CU with 16-byte loads, 36 GB/s when they carry predicates, 9 GB/s element by element), so the time of a launch is
+// the bytes the busiest CU streams: rounds of workgroups x (tile rows + tile columns) x chunk length
+// x 4 bytes. 64 x 64 tiles stream twice the bytes of 128 x 128 tiles in total but put four times
+// as many CUs to work (1024^3: 23.6 us -> 14.2 us); a split contraction adds a pass over the partial sums.
+static double fused_cost_us(const nzhip_gemm_desc& d, int tile, int64_t parts, int64_t Kc, bool vec) {
+    const double cus = (double)device_cu_count();
+    const int64_t tiles = ((d.M + tile - 1) / tile) * ((d.N + tile - 1) / tile) * d.batch_n * d.batch_c * parts;
+    const double rounds = (double)((tiles + (int64_t)cus - 1) / (int64_t)cus);
+    const bool full = vec && gemm_c_vec_legal(d) && d.M % tile == 0 && d.N % tile == 0 && Kc % 32 == 0 && d.K % 32 == 0;   // unpredicated instance
+    const double stream = rounds * 2.0 * tile * (double)Kc * 4.0 / (full ? 50e3 : vec ? 36e3 : 9e3);   // bytes / (bytes per us)
+    const double out = (double)d.M * d.N * d.batch_n * 4.0;
+    const double reduce = parts > 1 ? 6.0 + (double)(parts + 1) * out / 3e6 : 0.0;
+    return 3.0 + stream + reduce;
+}
+
+GemmPlan gemm_fused_plan(const nzhip_gemm_desc& d, int padded) {
+    GemmPlan best = {128, 1, d.K, 0.0};
+    const bool vec = gemm_operands_vec_legal(d, padded);
+    double best_cost = fused_cost_us(d, 128, 1, d.K, vec);
+    auto consider = [&](int tile, int64_t parts, int64_t Kc) {
+        const double c = fused_cost_us(d, tile, parts, Kc, vec);
+        if (c < best_cost * 0.97) { best_cost = c; best = {tile, parts, Kc, 0.0}; }    // keep the plainer plan on a near tie
+    };
+    consider(64, 1, d.K);
+    // a batch over n alone (batch_c == 1) can be split as well: the chunks take the c dimension of the launch
+    if (d.batch_c == 1 && d.batch_n <= 65535 && d.K >= 512) {
+        const bool narrow = d.M <= 64 || d.N <= 64;                // padded tiles: the k loop is shorter per byte
+        const int64_t min_chunk = vec && !narrow ? 512 : 128;
+        for (int64_t S = 2; S <= 1024 && S <= d.K / min_chunk; S += (S < 32 ? 1 : S / 8)) {
+            const int64_t Kc = ((d.K + S - 1) / S + 31) / 32 * 32;              // chunk length, whole 32-wide k tiles
+            const int64_t parts = (d.K + Kc - 1) / Kc;                           // the last one may be shorter
+            if (parts < 2) continue;
+            consider(128, parts, Kc);
+            consider(64, parts, Kc);
+        }
+    }
+    best.cost_us = best_cost;
+    return best;
+}
+
+bool gemm_small_tile(const nzhip_gemm_desc& d, int padded) {
+    // called with the descriptor of the launch itself (split chunks are its inner batch)
+    const bool vec = gemm_operands_vec_legal(d, padded);
+    return fused_cost_us(d, 64, 1, d.K, vec) < 0.97 * fused_cost_us(d, 128, 1, d.K, vec);
+}
+
+int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile, int64_t k_total, int padded) {
     GemmKernelArgs a;
     a.A = d.A;
     a.B = d.B;
@@ -462,17 +522,18 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
     a.k_total = (int)k_total;
 
     const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
-    const bool vec = gemm_vec_legal(d);
+    const bool vec = gemm_operands_vec_legal(d, padded);
+    a.c_vec = gemm_c_vec_legal(d);
     const int64_t batch = d.batch_n * d.batch_c;
 
     // Tile choice: 256x256 tiles need enough of them to fill the 256 CUs and pay only in their
     // unpredicated instance (5000x1000x5000: 379 us with predicated 256x256 tiles, 156 us with
     // 128x128 tiles).
     const int64_t t256 = ((d.M + 255) / 256) * ((d.N + 255) / 256) * batch;
-    const bool whole256 = vec && d.M % 256 == 0 && d.N % 256 == 0 && d.K % 32 == 0 && (k_total <= 0 || k_total % d.K == 0);
+    const bool whole256 = vec && a.c_vec && d.M % 256 == 0 && d.N % 256 == 0 && d.K % 32 == 0 && (k_total <= 0 || k_total % d.K == 0);
     static const char* tile_env = getenv("NZHIP_GEMM_TILE");         // 128 | 256: benchmarking only
     if (!force_tile && tile_env && (atoi(tile_env) == 128 || atoi(tile_env) == 256)) force_tile = atoi(tile_env);
-    int tile = force_tile ? force_tile : (t256 >= 192 && whole256 ? 256 : 128);
+    int tile = force_tile ? force_tile : (t256 >= 192 && whole256 ? 256 : gemm_small_tile(d, padded) ? 64 : 128);
     const int bm = tile, bn = tile;
     a.tiles_m = (int)((d.M + bm - 1) / bm);
     a.tiles_n = (int)((d.N + bn - 1) / bn);
@@ -487,6 +548,7 @@ int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_t
     if (tile == 256 && waves_env && atoi(waves_env) == 4)
         return launch_cfg<256, 256, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
     if (tile == 256) return launch_cfg<256, 256, 32, 4, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
+    if (tile == 64) return launch_cfg<64, 64, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
     return launch_cfg<128, 128, 32, 2, 2>(a, a_trans, b_trans, vec, (int)batch, stream);
 }
 

@@ -954,9 +954,6 @@ bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
     return flops / cvt_bytes >= (whole_tiles ? 512.0 : 300.0);
 }
 
-// The single-kernel route wants one unbatched product of whole 16 x 16 tile blocks and whole panels, 16-byte
-// accesses everywhere, at least two stages to overlap, and a device on which a wave of 256 workgroups is
-// resident at once (one workgroup per CU).
 // Host-side bookkeeping of the bounded waits: which stream the products enqueued since the last look went to,
 // how many time-outs had been seen by then, and whether the route has been given up.
 static std::mutex g_coop_mu;
@@ -966,6 +963,9 @@ static bool g_coop_mixed = false;                // ... unless they went to seve
 static unsigned g_coop_seen = 0;                 // value of g_coop_timeouts at the last look
 static std::atomic<bool> g_coop_off{false};
 
+// The single-kernel route wants one unbatched product of whole 16 x 16 tile blocks and whole panels, 16-byte
+// accesses everywhere, at least two stages to overlap, and a device on which a wave of 256 workgroups is
+// resident at once (one workgroup per CU).
 bool gemm_h16_coop_applicable(const nzhip_gemm_desc& d) {
     if (g_coop_off.load(std::memory_order_relaxed)) return false;
     constexpr int64_t BLOCK = (int64_t)COOP_SB * 256, PANEL = (int64_t)COOP_KP * CVT_K;

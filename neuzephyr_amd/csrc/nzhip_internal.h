@@ -15,11 +15,18 @@ int set_hip_error(hipError_t e, const char* what);
 // MFMA tile kernels (nzhip_gemm.hip). force_tile: 0 = choose, 128 / 256 = that square tile.
 // k_total > 0: the inner batch members are consecutive chunks of one contraction of that length
 // (d.K is the chunk length; the last member contracts what is left)
-int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile, int64_t k_total = 0);
+int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile, int64_t k_total = 0, int padded = 0);
+// Tile (64 or 128) and number of contraction chunks (1 = no split) for a product that goes to the fused kernel.
+struct GemmPlan { int tile; int64_t parts; int64_t Kc; double cost_us; };
+GemmPlan gemm_fused_plan(const nzhip_gemm_desc& d, int padded = 0);
+bool gemm_small_tile(const nzhip_gemm_desc& d, int padded = 0);
 // Two-pass route for large products: fp16 rounding pass + fp16 GEMM fed by direct-to-LDS loads
 // (nzhip_gemm_h16.hip).
 bool gemm_h16_applicable(const nzhip_gemm_desc& d);
 bool gemm_vec_legal(const nzhip_gemm_desc& d);   // 16-byte global accesses are legal for A, B and C
+bool gemm_operand_vec_legal(const float* X, int64_t ld, int64_t contig, int64_t stride_n, int64_t stride_c);
+bool gemm_operands_vec_legal(const nzhip_gemm_desc& d, int padded = 0);   // ... for A and B (decides the kernel instance)
+bool gemm_c_vec_legal(const nzhip_gemm_desc& d);          // ... for C (decides the epilogue's stores)
 // waves: 0 = choose, else 2 / 4 / 8; mfma: 0 = choose, else 16 (16x16x32) / 32 (32x32x16)
 int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int waves = 0, int mfma = 0);
 // Both passes in one kernel (rounding overlapped with the MFMA loop) for products of whole 4096 x 4096 x 1024 blocks.

@@ -4,6 +4,7 @@
 // working; the fused route is nzhip_conv2d_forward / nzhip_gemm with bias and activation.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdlib>
 
 #include "nzhip_internal.h"
@@ -353,14 +354,81 @@ __global__ __launch_bounds__(256) void splitk_reduce_wide_kernel(nzhip_gemm_desc
 
 using namespace nzhip;
 
+// ---- operands that do not allow 16-byte loads ----------------------------------------------------
+// Rows that start off a 16-byte boundary or whose contiguous extent is not a multiple of 4 (1000 x 777 x 513)
+// make the fused kernel load element by element, which more than halves the rate at which a CU takes
+// tiles in. For a product big enough to notice, such an operand is first copied into a workspace with the
+// same layout and rows padded with zeros to a multiple of 4 elements (one launch for both operands).
+struct RepackOperand {
+    const float* src;
+    float* dst;
+    long rows, cols, ld_src, ld_dst;          // rows == 0: nothing to do
+};
+
+__global__ __launch_bounds__(256) void repack_pair_kernel(const RepackOperand a, const RepackOperand b) {
+    const RepackOperand& q = blockIdx.y ? b : a;
+    const long per_row = q.ld_dst / 4, total = q.rows * per_row;
+    for (long idx = (long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long)gridDim.x * 256) {
+        const long r = idx / per_row, c = (idx - r * per_row) * 4;
+        const float* src = q.src + r * q.ld_src + c;
+        floatx4 v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = c + e < q.cols ? src[e] : 0.f;
+        *reinterpret_cast<floatx4*>(q.dst + r * q.ld_dst + c) = v;
+    }
+}
+
+static int gemm_routed(const nzhip_gemm_desc& d, hipStream_t s, int padded = 0);
+
+// Returns NZHIP_OK and sets *done when the product was computed from padded copies; leaves *done false when
+// the copies would not pay (or the workspace is not to be had) and the caller goes on with the operands as given.
+static int gemm_try_repacked(const nzhip_gemm_desc& d, hipStream_t s, bool* done) {
+    *done = false;
+    if (d.batch_n * d.batch_c != 1) return NZHIP_OK;
+    const bool a_trans = d.a_layout == NZHIP_LAYOUT_TRANS, b_trans = d.b_layout == NZHIP_LAYOUT_TRANS;
+    const int64_t a_rows = a_trans ? d.K : d.M, a_cols = a_trans ? d.M : d.K;
+    const int64_t b_rows = b_trans ? d.N : d.K, b_cols = b_trans ? d.K : d.N;
+    const bool a_ok = gemm_operand_vec_legal(d.A, d.lda, a_cols, 0, 0), b_ok = gemm_operand_vec_legal(d.B, d.ldb, b_cols, 0, 0);
+    if (a_ok && b_ok) return NZHIP_OK;
+    const int64_t a_ld = (a_cols + 3) / 4 * 4, b_ld = (b_cols + 3) / 4 * 4;
+    const size_t a_bytes = a_ok ? 0 : (size_t)a_rows * a_ld * sizeof(float), b_bytes = b_ok ? 0 : (size_t)b_rows * b_ld * sizeof(float);
+    nzhip_gemm_desc g = d;
+    const int padded = (a_ok ? 0 : 1) | (b_ok ? 0 : 2);
+    // stand-in addresses for the cost estimate: only alignment and leading dimensions matter to it
+    if (!a_ok) { g.A = nullptr; g.lda = a_ld; }
+    if (!b_ok) { g.B = nullptr; g.ldb = b_ld; }
+    const double copy_us = 3.0 + 2.0 * (double)(a_bytes + b_bytes) / 3e6;
+    if (gemm_fused_plan(g, padded).cost_us + copy_us >= 0.9 * gemm_fused_plan(d).cost_us) return NZHIP_OK;
+    const size_t a_off = (a_bytes + 255) & ~(size_t)255;
+    char* ws = nullptr;
+    if (workspace_alloc(reinterpret_cast<void**>(&ws), a_off + b_bytes, s) != NZHIP_OK) return NZHIP_OK;   // no room: as given
+    RepackOperand ra = {d.A, reinterpret_cast<float*>(ws), a_ok ? 0 : a_rows, a_cols, d.lda, a_ld};
+    RepackOperand rb = {d.B, reinterpret_cast<float*>(ws + a_off), b_ok ? 0 : b_rows, b_cols, d.ldb, b_ld};
+    if (!a_ok) g.A = ra.dst;
+    if (!b_ok) g.B = rb.dst;
+    const long units = std::max(ra.rows * (ra.ld_dst / 4), rb.rows * (rb.ld_dst / 4));
+    const unsigned blocks = (unsigned)std::min<long>((units + 255) / 256, 4096);
+    hipLaunchKernelGGL(repack_pair_kernel, dim3(blocks, 2), dim3(256), 0, s, ra, rb);
+    int rc = check_launch("repack_pair_kernel");
+    if (rc == NZHIP_OK) rc = gemm_routed(g, s, padded);
+    const int rc2 = workspace_free(ws, s);
+    *done = true;
+    return rc ? rc : rc2;
+}
+
 extern "C" {
 
 int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
     if (!desc) return set_error(NZHIP_E_INVALID, "nzhip_gemm: null descriptor");
-    const nzhip_gemm_desc& d = *desc;
-    if (int rc = validate_gemm(d)) return rc;
-    if (d.M == 0 || d.N == 0) return NZHIP_OK;
-    hipStream_t s = as_stream(stream);
+    if (int rc = validate_gemm(*desc)) return rc;
+    if (desc->M == 0 || desc->N == 0) return NZHIP_OK;
+    return gemm_routed(*desc, as_stream(stream));
+}
+
+}  // extern "C"
+
+// The route choice behind nzhip_gemm, for a validated descriptor with M, N > 0.
+static int gemm_routed(const nzhip_gemm_desc& d, hipStream_t s, int padded) {
     if (d.K == 0) {
         dim3 grid((unsigned)((d.M * d.N + 255) / 256), (unsigned)(d.batch_n * d.batch_c));
         hipLaunchKernelGGL(fill_bias_act_kernel, grid, dim3(256), 0, s, d);
@@ -368,78 +436,77 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
     }
     if (gemm_thin_applicable(d)) return gemm_thin_dispatch(d, s);
     if (gemm_skinny_applicable(d)) return gemm_skinny_dispatch(d, s);
-    // One matrix with few output tiles (weight gradients with K = batch x pixels, mid-size products):
-    // a workgroup's k loop is latency-bound (about 0.55 us per 32-wide k tile with 16-byte loads, 2 us
-    // without), so cut K into chunks that run as a batch into a workspace, then add the chunks in
-    // order. The extra pass over the partial sums costs 5..15 us, so a chunk keeps at least 512 of
-    // the contraction when loads are vectorised (1024^3: 23 us unsplit, 31 us in two chunks;
-    // 1024x4096x1024: 71 us unsplit, 39 us in eight chunks) and 128 otherwise.
-    // A batch over n alone (batch_c == 1: shared-weight layers, the conv column-matrix route) splits the
-    // same way; its chunks take the c dimension of the launch.
-    if (d.batch_c == 1 && d.batch_n <= 65535 && d.K >= 512) {
-        const int cus = device_cu_count();
-        const int64_t tiles = ((d.M + 127) / 128) * ((d.N + 127) / 128) * d.batch_n;
-        if (tiles * 2 <= cus) {
-            const bool narrow = d.M <= 64 || d.N <= 64;            // padded tiles: the k loop is shorter per byte
-            const int64_t min_chunk = gemm_vec_legal(d) && !narrow ? 512 : 128;
-            int64_t S = (2 * cus + tiles - 1) / tiles;
-            if (S > d.K / min_chunk) S = d.K / min_chunk;
-            if (S > 1024) S = 1024;
-            static const char* sk_env = getenv("NZHIP_SPLITK");                  // benchmarking only
-            if (sk_env && atoi(sk_env) >= 1) S = atoi(sk_env);
-            if (S < 1) S = 1;
-            const int64_t Kc = ((d.K + S - 1) / S + 31) / 32 * 32;          // chunk length, whole 32-wide k tiles
-            const int parts = (int)((d.K + Kc - 1) / Kc);                    // the last one may be shorter
-            if (parts >= 2) {
-                float* P = nullptr;
-                if (int rc = workspace_alloc(reinterpret_cast<void**>(&P), (size_t)d.batch_n * parts * d.M * d.N * sizeof(float), s))
-                    return rc;
-                nzhip_gemm_desc g = d;
-                g.C = P; g.ldc = d.N; g.K = Kc;
-                g.batch_c = parts;
-                g.c_stride_n = (int64_t)parts * d.M * d.N;
-                g.a_stride_c = d.a_layout == NZHIP_LAYOUT_ROW ? Kc : Kc * d.lda;   // next chunk of A / B
-                g.b_stride_c = d.b_layout == NZHIP_LAYOUT_ROW ? Kc * d.ldb : Kc;
-                g.c_stride_c = d.M * d.N;
-                g.bias = nullptr; g.activation = NZHIP_ACT_NONE;
-                int rc = gemm_mfma_dispatch(g, s, 0, d.K);
-                if (rc == NZHIP_OK) {
-                    if (parts >= 64 && d.M * d.N <= 4096) {                     // a handful of outputs: one wave each
-                        const long groups = (d.M * d.N + 3) / 4;
-                        hipLaunchKernelGGL(splitk_reduce_wave_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
-                    } else if (parts > 16 || d.M * d.N < (1 << 18)) {           // few outputs: spread each over eight lanes
-                        const long groups = (d.M * d.N + 31) / 32;               // 32 outputs x 8 chunk lanes per workgroup
-                        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
-                    } else {
-                        const long groups = (d.M * d.N + 255) / 256;
-                        hipLaunchKernelGGL(splitk_reduce_wide_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
-                    }
-                    rc = check_launch("splitk_reduce_kernel");
-                }
-                const int rc2 = workspace_free(P, s);
-                return rc ? rc : rc2;
-            }
-        }
-    }
-    // NZHIP_GEMM_ROUTE=fused|h16 overrides the route choice (benchmarking only).
-    static const char* route = getenv("NZHIP_GEMM_ROUTE");
+    // Products that leave CUs idle with 128 x 128 tiles (weight gradients with K = batch x pixels, mid-size
+    // products): smaller tiles, or the contraction cut into chunks that run as a batch into a workspace and are
+    // then added in order, whichever the cost model in gemm_fused_plan prefers. A chunk keeps at least 512 of the
+    // contraction when loads are vectorised and 128 otherwise. A batch over n alone (batch_c == 1: shared-weight
+    // layers, the conv column-matrix route) splits the same way; its chunks take the c dimension of the launch.
+    static const char* route = getenv("NZHIP_GEMM_ROUTE");         // fused | h16: overrides the route choice (benchmarking only)
     const bool force_fused = route && route[0] == 'f', force_h16 = route && route[0] == 'h';
     static const char* coop_env = getenv("NZHIP_H16_COOP");              // 0: never the single-kernel route (benchmarking only)
     const bool allow_coop = !(coop_env && atoi(coop_env) == 0);
     if (!force_fused && allow_coop && gemm_h16_coop_applicable(d)) return gemm_h16_coop_dispatch(d, s);
     if (!force_fused && (force_h16 || gemm_h16_applicable(d))) return gemm_h16_dispatch(d, s);
-    return gemm_mfma_dispatch(d, s, 0);
+    {
+        static const char* repack_env = getenv("NZHIP_REPACK");          // 0: never copy operands (benchmarking only)
+        bool done = false;
+        if (!padded && !(repack_env && atoi(repack_env) == 0)) {
+            const int rc = gemm_try_repacked(d, s, &done);
+            if (done || rc) return rc;
+        }
+    }
+    GemmPlan plan = gemm_fused_plan(d, padded);
+    static const char* sk_env = getenv("NZHIP_SPLITK");                  // benchmarking only: number of chunks
+    if (sk_env && atoi(sk_env) >= 1 && d.batch_c == 1 && d.batch_n <= 65535) {
+        const int64_t S = atoi(sk_env);
+        plan.Kc = ((d.K + S - 1) / S + 31) / 32 * 32;
+        plan.parts = (d.K + plan.Kc - 1) / plan.Kc;
+    }
+    if (plan.parts >= 2) {
+        const int parts = (int)plan.parts;
+        const int64_t Kc = plan.Kc;
+        float* P = nullptr;
+        if (int rc = workspace_alloc(reinterpret_cast<void**>(&P), (size_t)d.batch_n * parts * d.M * d.N * sizeof(float), s))
+            return rc;
+        nzhip_gemm_desc g = d;
+        g.C = P; g.ldc = d.N; g.K = Kc;
+        g.batch_c = parts;
+        g.c_stride_n = (int64_t)parts * d.M * d.N;
+        g.a_stride_c = d.a_layout == NZHIP_LAYOUT_ROW ? Kc : Kc * d.lda;   // next chunk of A / B
+        g.b_stride_c = d.b_layout == NZHIP_LAYOUT_ROW ? Kc * d.ldb : Kc;
+        g.c_stride_c = d.M * d.N;
+        g.bias = nullptr; g.activation = NZHIP_ACT_NONE;
+        int rc = gemm_mfma_dispatch(g, s, plan.tile, d.K, padded);
+        if (rc == NZHIP_OK) {
+            if (parts >= 64 && d.M * d.N <= 4096) {                     // a handful of outputs: one wave each
+                const long groups = (d.M * d.N + 3) / 4;
+                hipLaunchKernelGGL(splitk_reduce_wave_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
+            } else if (parts > 16 || d.M * d.N < (1 << 18)) {           // few outputs: spread each over eight lanes
+                const long groups = (d.M * d.N + 31) / 32;               // 32 outputs x 8 chunk lanes per workgroup
+                hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
+            } else {
+                const long groups = (d.M * d.N + 255) / 256;
+                hipLaunchKernelGGL(splitk_reduce_wide_kernel, dim3((unsigned)groups, (unsigned)d.batch_n), dim3(256), 0, s, d, P, parts);
+            }
+            rc = check_launch("splitk_reduce_kernel");
+        }
+        const int rc2 = workspace_free(P, s);
+        return rc ? rc : rc2;
+    }
+    return gemm_mfma_dispatch(d, s, 0, 0, padded);
 }
 
-/* Test hook: pick the kernel instead of letting the shape decide. tile 128 / 256: the fused
+extern "C" {
+
+/* Test hook: pick the kernel instead of letting the shape decide. tile 64 / 128 / 256: the fused
  * convert-on-load kernel with that square tile; tile 16 / 18 / 12: the two-pass fp16 route with
  * 256x256 tiles and 4 waves / 256x256 tiles and 8 waves / 128x256 tiles, 16x16x32 MFMAs;
  * tile 316 / 318 / 312: the same three with 32x32x16 MFMAs. */
 int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream) {
     if (!desc) return set_error(NZHIP_E_INVALID, "nzhip_gemm: null descriptor");
     const int base = tile > 300 ? tile - 300 : tile;
-    if (tile != 128 && tile != 256 && tile != 28 && base != 16 && base != 18 && base != 12)
-        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 128, 256, 16, 18, 12, 28, 316, 318 or 312");
+    if (tile != 64 && tile != 128 && tile != 256 && tile != 28 && base != 16 && base != 18 && base != 12)
+        return set_error(NZHIP_E_INVALID, "nzhip_gemm_force_tile: tile must be 64, 128, 256, 16, 18, 12, 28, 316, 318 or 312");
     if (int rc = validate_gemm(*desc)) return rc;
     if (desc->M == 0 || desc->N == 0 || desc->K == 0) return nzhip_gemm(desc, stream);
     const int mfma = tile > 300 ? 32 : 16;

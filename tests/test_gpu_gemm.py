@@ -63,7 +63,7 @@ SHAPES = [(1, 1, 1), (3, 5, 2), (16, 16, 16), (17, 33, 15), (64, 100, 132), (130
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
 @pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("tile", [128, 256, 16, 18, 12, 316, 318, 312])  # fused kernels with that tile; 16 / 18 / 12 = two-pass fp16 route variants (16x16x32 MFMAs), 3xx = the same with 32x32x16
+@pytest.mark.parametrize("tile", [64, 128, 256, 16, 18, 12, 316, 318, 312])  # fused kernels with that tile; 16 / 18 / 12 = two-pass fp16 route variants (16x16x32 MFMAs), 3xx = the same with 32x32x16
 def test_integer_operands_are_bit_exact(nz, M, K, N, a_trans, b_trans, tile):
     rng = np.random.default_rng(M * 7919 + K * 31 + N)
     A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
@@ -281,6 +281,51 @@ def test_skinny_batched_linear_single_sample(nz, oracle):
     assert np.max(np.abs(got - ref)) <= 1e-4
 
 
+@pytest.mark.parametrize("M,K,N", [(1000, 777, 513), (700, 701, 333), (999, 1001, 1003), (516, 1030, 520)])
+@pytest.mark.parametrize("a_trans,b_trans", [(False, False), (False, True), (True, False), (True, True)])
+def test_operands_without_16_byte_rows_are_bit_exact_on_integers(nz, M, K, N, a_trans, b_trans):
+    # products big enough for it are computed from zero-padded copies of the operands whose rows do not allow
+    # 16-byte loads; rows are embedded in NaN-filled storage with a leading dimension of their own and an odd base
+    # offset, so a read past a row's end or a missing zero in the padding poisons the result
+    import ctypes as C
+    import torch
+    rng = np.random.default_rng(M + 3 * K + 7 * N)
+    A = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+    B = rng.integers(-8, 9, size=(K, N)).astype(np.float32)
+    bias = rng.integers(-50, 51, size=(M, N)).astype(np.float32)
+    expect = np.maximum((A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32) + bias, 0)
+
+    def embed(X, ld, off):
+        rows, cols = X.shape
+        buf = torch.full((rows * ld + off + 8,), float("nan"), device="cuda")
+        view = buf[off:off + rows * ld].view(rows, ld)
+        view[:, :cols] = torch.from_numpy(X).cuda()
+        return buf, view.data_ptr()
+
+    As = A.T.copy() if a_trans else A
+    Bs = B.T.copy() if b_trans else B
+    lda, ldb, ldc = As.shape[1] + 2, Bs.shape[1] + 1, N + 3
+    bufA, pa = embed(As, lda, 1)
+    bufB, pb = embed(Bs, ldb, 3)
+    out = torch.full((M * ldc + 1,), float("nan"), device="cuda")
+    bd = dev(bias)
+    d = nz.GemmDesc()
+    d.A, d.B, d.C = pa, pb, out.data_ptr() + 4
+    d.M, d.N, d.K = M, N, K
+    d.lda, d.ldb, d.ldc = lda, ldb, ldc
+    d.a_layout = nz.LAYOUT_TRANS if a_trans else nz.LAYOUT_ROW
+    d.b_layout = nz.LAYOUT_TRANS if b_trans else nz.LAYOUT_ROW
+    d.batch_n = d.batch_c = 1
+    d.bias = bd.data_ptr()
+    d.bias_stride_row, d.bias_stride_col = N, 1
+    d.activation = nz.ACT_RELU
+    nz.check(nz.load().nzhip_gemm(C.byref(d), None))
+    torch.cuda.synchronize()
+    got = out[1:].view(M, ldc).cpu().numpy()
+    assert np.array_equal(got[:, :N], expect)
+    assert np.all(np.isnan(got[:, N:]))                            # nothing written between the rows of C
+
+
 def test_unaligned_base_pointers_take_the_scalar_path(nz):
     import torch
     rng = np.random.default_rng(5)
@@ -319,7 +364,7 @@ def test_config1_gemm_256_uniform(nz, oracle):
     A = oracle.fill((256, 256), 0, "uniform", -1.0, 1.0)
     B = oracle.fill((256, 256), 1000, "uniform", -1.0, 1.0)
     truth = oracle.gemm_f64(A, B)
-    for tile in (128, 256, 16):
+    for tile in (64, 128, 256, 16):
         got = host(nz.gemm(dev(A), dev(B), force_tile=tile))
         check_tolerance(oracle, got, truth, f"G1 tile {tile}")
         # and against the fp32 sequential oracle: same rounding, only the sum order differs

@@ -36,6 +36,7 @@ ROUTES = {
     "split contraction": [(256, 4096, 256), (128, 2048, 192)],
     "streamed skinny": [(1, 4096, 4096), (1, 1024, 512)],
     "two-pass fp16": [(3072, 768, 3072), (2000, 800, 2000)],
+    "padded operand copies": [(1000, 777, 513), (333, 331, 335)],
     "no workspace": [(300, 100, 200), (17, 33, 15)],
 }
 
