@@ -350,9 +350,6 @@ __global__ __launch_bounds__(256) void splitk_reduce_wide_kernel(nzhip_gemm_desc
     d.C[bn * d.c_stride_n + m * d.ldc + n] = x;
 }
 
-}  // namespace nzhip
-
-using namespace nzhip;
 
 // ---- operands that do not allow 16-byte loads ----------------------------------------------------
 // Rows that start off a 16-byte boundary or whose contiguous extent is not a multiple of 4 (1000 x 777 x 513)
@@ -377,6 +374,10 @@ __global__ __launch_bounds__(256) void repack_pair_kernel(const RepackOperand a,
         *reinterpret_cast<floatx4*>(q.dst + r * q.ld_dst + c) = v;
     }
 }
+
+}  // namespace nzhip
+
+using namespace nzhip;
 
 static int gemm_routed(const nzhip_gemm_desc& d, hipStream_t s, int padded = 0);
 
