@@ -326,6 +326,75 @@ def test_operands_without_16_byte_rows_are_bit_exact_on_integers(nz, M, K, N, a_
     assert np.all(np.isnan(got[:, N:]))                            # nothing written between the rows of C
 
 
+def _embedded_cases():
+    rng = np.random.default_rng(777)
+    cases = []
+    for i in range(96):
+        big = i % 3 == 0
+        M = int(rng.integers(1, 1200 if big else 200))
+        N = int(rng.integers(1, 1200 if big else 200))
+        K = int(rng.integers(1, 2500 if big else 400))
+        cases.append((M, K, N, bool(rng.integers(2)), bool(rng.integers(2)), [int(v) for v in rng.integers(0, 6, size=3)],
+                      [int(v) for v in rng.integers(0, 4, size=3)], int(rng.integers(4)), 1000 + i))
+    return cases
+
+
+@pytest.mark.parametrize("M,K,N,a_trans,b_trans,slack,offset,bias_form,seed", _embedded_cases())
+def test_embedded_operands_random_sweep(nz, M, K, N, a_trans, b_trans, slack, offset, bias_form, seed):
+    # random shapes, layouts, leading dimensions and base offsets through the default route choice (streaming,
+    # thin, split, 64 / 128 tiles, padded copies): exact on integers, nothing read or written outside the rows
+    import ctypes as C
+    import torch
+    rng = np.random.default_rng(seed)
+    A = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, size=(K, N)).astype(np.float32)
+    expect = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)
+    bias = None
+    if bias_form == 1:                                              # one value per column
+        bias = rng.integers(-50, 51, size=(N,)).astype(np.float32)
+        expect = expect + bias[None, :]
+        strides = (0, 1)
+    elif bias_form == 2:                                            # one value per row
+        bias = rng.integers(-50, 51, size=(M,)).astype(np.float32)
+        expect = expect + bias[:, None]
+        strides = (1, 0)
+    elif bias_form == 3:                                            # a full matrix, and ReLU
+        bias = rng.integers(-50, 51, size=(M, N)).astype(np.float32)
+        expect = np.maximum(expect + bias, 0)
+        strides = (N, 1)
+
+    def embed(X, ld, off):
+        rows, cols = X.shape
+        buf = torch.full((rows * ld + off + 8,), float("nan"), device="cuda")
+        buf[off:off + rows * ld].view(rows, ld)[:, :cols] = torch.from_numpy(X).cuda()
+        return buf, buf.data_ptr() + 4 * off
+
+    As = A.T.copy() if a_trans else A
+    Bs = B.T.copy() if b_trans else B
+    lda, ldb, ldc = As.shape[1] + slack[0], Bs.shape[1] + slack[1], N + slack[2]
+    bufA, pa = embed(As, lda, offset[0])
+    bufB, pb = embed(Bs, ldb, offset[1])
+    out = torch.full((M * ldc + offset[2] + 8,), float("nan"), device="cuda")
+    d = nz.GemmDesc()
+    d.A, d.B, d.C = pa, pb, out.data_ptr() + 4 * offset[2]
+    d.M, d.N, d.K = M, N, K
+    d.lda, d.ldb, d.ldc = lda, ldb, ldc
+    d.a_layout = nz.LAYOUT_TRANS if a_trans else nz.LAYOUT_ROW
+    d.b_layout = nz.LAYOUT_TRANS if b_trans else nz.LAYOUT_ROW
+    d.batch_n = d.batch_c = 1
+    if bias is not None:
+        bd = dev(bias)
+        d.bias = bd.data_ptr()
+        d.bias_stride_row, d.bias_stride_col = strides
+        d.activation = nz.ACT_RELU if bias_form == 3 else nz.ACT_NONE
+    nz.check(nz.load().nzhip_gemm(C.byref(d), None))
+    torch.cuda.synchronize()
+    flat = out.cpu().numpy()
+    got = flat[offset[2]:offset[2] + M * ldc].reshape(M, ldc)
+    assert np.array_equal(got[:, :N], expect)
+    assert np.all(np.isnan(got[:, N:])) and np.all(np.isnan(flat[:offset[2]])) and np.all(np.isnan(flat[offset[2] + M * ldc:]))
+
+
 def test_unaligned_base_pointers_take_the_scalar_path(nz):
     import torch
     rng = np.random.default_rng(5)
