@@ -507,8 +507,9 @@ def main():
             traffic = json.load(f).get(args.workload, {}).get("bytes_per_step")
     except OSError:
         pass
-    scope = ("whole step = every kernel the call launches (for gemm8192: the fp16 rounding kernel + the MFMA "
-             "kernel); per-kernel durations are in profiles/")
+    scope = ("whole step = every kernel the call launches (for gemm8192: the kernel that rounds the first stage of "
+             "the operands + the MFMA kernel, which rounds the rest inside its k loops); per-kernel durations are "
+             "in profiles/")
     if wl.bound == "mfma":
         roofline = {"bound": "mfma", "achieved": tflops, "peak": PEAK_TFLOPS_FP16, "unit": "TFLOP/s",
                     "frac": tflops / PEAK_TFLOPS_FP16, "traffic": traffic, "scope": scope}
