@@ -67,7 +67,9 @@ struct CvtOperand {
     int vec, fr;
 };
 
-template <bool K_CONTIG>
+// WHOLE: the block lies inside the operand and 16-byte loads are legal, so the eight requests of a thread carry no
+// condition and are all in flight before the first is used (a launch of few blocks is bound by that latency).
+template <bool K_CONTIG, bool WHOLE = false>
 __device__ __forceinline__ void cvt_block(char* img, const CvtOperand& o, int K, int nkt, int blk, int kt, int rb, int member) {
     _Float16* dst = o.dst;
     const int R = o.R, vec = o.vec, fr = o.fr;
@@ -81,12 +83,20 @@ __device__ __forceinline__ void cvt_block(char* img, const CvtOperand& o, int K,
         // logical rows puts rows 16 apart (1 KiB, the same banks) into one store instruction. In global
         // memory a row's 32 values are one 128-byte line either way.
         const int k4 = t & 7, rr = t >> 3;
+        floatx4 whole[8];
+        if (WHOLE) {
+#pragma unroll
+            for (int pass = 0; pass < 8; pass++)
+                whole[pass] = *reinterpret_cast<const floatx4*>(s + (long)(r0 + logical_row_of(rr + pass * 32, fr, blk)) * ld + k0 + k4 * 4);
+        }
 #pragma unroll
         for (int pass = 0; pass < 8; pass++) {
             const int pr_ = rr + pass * 32, lr = logical_row_of(pr_, fr, blk), r = r0 + lr, k = k0 + k4 * 4;
             floatx4 v = {0.f, 0.f, 0.f, 0.f};
             const float* q = s + (long)r * ld + k;
-            if (r < R) {
+            if (WHOLE) {
+                v = whole[pass];
+            } else if (r < R) {
                 if (vec && k + 4 <= K) {
                     v = *reinterpret_cast<const floatx4*>(q);
                 } else {
@@ -103,12 +113,20 @@ __device__ __forceinline__ void cvt_block(char* img, const CvtOperand& o, int K,
     } else {
         // 64 threads per k row (one float4 of 4 rows each), 4 k rows per pass
         const int r4 = t & 63, kk0 = t >> 6;
+        floatx4 whole[8];
+        if (WHOLE) {
+#pragma unroll
+            for (int pass = 0; pass < 8; pass++)
+                whole[pass] = *reinterpret_cast<const floatx4*>(s + (long)(k0 + kk0 + pass * 4) * ld + r0 + r4 * 4);
+        }
 #pragma unroll
         for (int pass = 0; pass < 8; pass++) {
             const int kk = kk0 + pass * 4, k = k0 + kk, lr = r4 * 4, r = r0 + lr;
             floatx4 v = {0.f, 0.f, 0.f, 0.f};
             const float* q = s + (long)k * ld + r;
-            if (k < K) {
+            if (WHOLE) {
+                v = whole[pass];
+            } else if (k < K) {
                 if (vec && r + 4 <= R) {
                     v = *reinterpret_cast<const floatx4*>(q);
                 } else {
@@ -652,9 +670,9 @@ __global__ __launch_bounds__(256) void coop_prologue_kernel(CvtOperand a, CvtOpe
         for (int i = threadIdx.x; i < n_flags; i += 256) flags[i] = 0;
     const int rb = blockIdx.y;
     if (rb < a_blocks)
-        cvt_block<A_KC>(img, a, K, nkt, 16, blockIdx.x, rb, 0);
+        cvt_block<A_KC, true>(img, a, K, nkt, 16, blockIdx.x, rb, 0);
     else
-        cvt_block<B_KC>(img, b, K, nkt, 16, blockIdx.x, rb - a_blocks, 0);
+        cvt_block<B_KC, true>(img, b, K, nkt, 16, blockIdx.x, rb - a_blocks, 0);
 }
 
 // phys_row_of for 16-row blocks and fr = 1 << lg blocks per wave tile
