@@ -1044,6 +1044,340 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     }
 }
 
+// ---- resident weights, two halo buffers (3x3, 64-pixel-wide patches, 16-byte image rows) --------------
+// The kernel above spends a quarter of every work item between its two barriers: the halo is stored, the
+// workgroup meets, multiplies, meets again. With a second halo buffer the next item's halo is stored in the
+// middle of the current item's MFMAs and one barrier per item is left. LDS has no room for it beside nine
+// taps of weights (144 KiB for 128 channels x 64 x 9), so the ninth tap is not resident: a wave requests the
+// 16 bytes per lane and 32 output channels it needs of it one item ahead, from L2, into registers. The other
+// eight taps make rows of exactly 256 bytes; their sixteen 16-byte slots (tap, channel half) are stored at
+// slot ^ (row & 15), so the sixteen rows of a read pass fall on sixteen different bank groups.
+// Image of one channel tile: [chunk][BN rows][256 B] for taps 0..7, then [chunk][BN rows][32 B] for tap 8.
+template <int BN>
+__global__ __launch_bounds__(256) void conv_weight_image_db_kernel(_Float16* __restrict__ dst, const float* __restrict__ w_ref,
+                                                                   int C, int O, int n_chunks, int n_otiles) {
+    const int slab = blockIdx.y;                               // o_tile * n_chunks + chunk
+    const int chunk = slab % n_chunks, o_tile = slab / n_chunks;
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    const int o_l = t % BN, rest = t / BN;
+    if (rest >= 9 * IG_CC) return;
+    const int cc = rest % IG_CC, tap = rest / IG_CC;
+    const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
+    float v = 0.f;
+    if (c < C && o < O) v = w_ref[((long)c * 9 + tap) * O + o];
+    _Float16* tile = dst + (long)o_tile * n_chunks * BN * 144;   // 288 bytes per (chunk, row)
+    const int half = cc >> 3;
+    if (tap < 8) {
+        const int slot = (tap * 2 + half) ^ (o_l & 15);
+        tile[((long)chunk * BN + o_l) * 128 + slot * 8 + (cc & 7)] = (_Float16)v;
+    } else {
+        tile[(long)n_chunks * BN * 128 + ((long)chunk * BN + o_l) * 16 + half * 8 + (cc & 7)] = (_Float16)v;
+    }
+}
+
+// NCH: channel chunks of 16 (= ceil(C / 16), even, so that an item's parity is its chunk's). Work item k (one chunk of one patch) multiplies out of halo buffer k & 1; behind its
+// first four taps it requests item k + 2 into the register set item k's halo came from, behind its sixth tap
+// it rounds item k + 1's set into the other halo buffer, and it ends with the only barrier.
+constexpr int CONV_DB_PLANE = 6 * 66 * 16 + 96;               // halo plane pitch of the kernel below: 6432 = 25 * 256 + 32
+template <bool PIX_BIAS, int NI, int NCH>
+__global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArgs p, const int n_patches) {
+    using G = IgemmGeom<3, 3, 64, 128>;
+    constexpr int TW = 64, KW = 3;
+    constexpr int BN = 64 * NI, WCH = 32 * NI, CB = TW / 32, FP = 2, NW = 8;
+    constexpr int W_CHUNK = BN * 256;
+    static_assert(NCH % 2 == 0, "items come in pairs");
+    // A halo buffer is two planes (channels 0..7 and 8..15 of the chunk), 16 bytes per pixel. Fragment reads
+    // (32 adjacent pixels of one plane per half-wave) and the staging stores below are then conflict-free
+    // without a swizzle; the plane pitch is 32 bytes past a multiple of 256 so that the two planes a 16-lane
+    // group of stores touches use different banks.
+    constexpr int H_PLANE = CONV_DB_PLANE, H_BYTES = 2 * H_PLANE;
+    static_assert(H_PLANE >= G::HH * G::WW * 16 && H_PLANE % 256 == 32, "plane pitch");
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    char* lds_w = lds;
+    char* lds_h0 = lds + NCH * W_CHUNK;
+    char* lds_h1 = lds_h0 + H_BYTES;
+    float* lds_bias = reinterpret_cast<float*>(lds_h1 + H_BYTES);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+    const int o_tile = blockIdx.y;
+    const int patches_per_image = p.tiles_w * p.tiles_h;
+    const long plane = (long)p.H * p.W;
+
+    const char* wtile = reinterpret_cast<const char*>(p.wimg) + (long)o_tile * NCH * BN * 288;
+    {
+        const char* wsrc = wtile + lane * 16;
+        constexpr int pieces = NCH * (W_CHUNK / 1024);
+        for (int j = wave; j < pieces; j += NW)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc + (long)j * 1024),
+                                             (__attribute__((address_space(3))) void*)(lds_w + j * 1024), 16, 0, 0);
+    }
+    // tap 8 of this wave's channels: the set of the chunk in hand and the set of the next chunk, requested one
+    // item ahead from the image (it stays in L2: every workgroup reads the same 16 KiB)
+    half8_t w8[2][NI];
+    const char* w8_src = wtile + (long)NCH * W_CHUNK + ((wn * WCH + li) * 32 + lh * 16);
+    auto request_w8 = [&](half8_t (&dst)[NI], const int c) {
+#pragma unroll
+        for (int i = 0; i < NI; i++) dst[i] = *reinterpret_cast<const half8_t*>(w8_src + (c * BN + i * 32) * 32);
+    };
+    request_w8(w8[0], 0);
+    float my_bias = 0.f;
+    if (!PIX_BIAS && p.bias && tid < BN && o_tile * BN + tid < p.O) my_bias = p.bias[(long)(o_tile * BN + tid) * p.bias_sc];
+
+    // staging task of this thread: 4 adjacent pixels x 4 channels (core) or one halo-column pixel x 4 channels
+    // (edge). A wave takes one halo row; its lanes are (channel quarter, pixel quad) with the quarter fastest, so
+    // the 16 lanes of a store pass write the four quarters of four quads: 16 different 8-byte bank pairs.
+    constexpr int W4 = TW / 4;
+    constexpr int CORE_TASKS = 4 * G::HH * W4, EDGE_TASKS = 4 * G::HH * (KW - 1);
+    static_assert(CORE_TASKS + EDGE_TASKS <= 512 && W4 == 16, "one task per thread, one halo row per wave");
+    const bool is_core = tid < CORE_TASKS, is_edge = !is_core && tid < CORE_TASKS + EDGE_TASKS;
+    int t_q4, t_hh, t_ww;
+    if (is_core) {
+        t_q4 = tid & 3;
+        t_hh = tid >> 6;
+        t_ww = p.pad + 4 * ((tid >> 2) & 15);
+    } else {
+        const int e = tid - CORE_TASKS;
+        const int ecol = e % (KW - 1);
+        t_hh = (e / (KW - 1)) % G::HH;
+        t_q4 = e / ((KW - 1) * G::HH);
+        t_ww = ecol < p.pad ? ecol : TW + ecol;
+    }
+    t_q4 &= 3;
+    auto halo_slot = [&](char* hb, int hh, int ww) {
+        return hb + (t_q4 >> 1) * H_PLANE + (hh * G::WW + ww) * 16 + (t_q4 & 1) * 8;
+    };
+
+    int first_patch = blockIdx.x, patch_stride = gridDim.x;
+    int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    if (p.patch_map != 0 && gridDim.x % 8 == 0) {               // the workgroups of an XCD sweep a contiguous eighth
+        const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3, nq = gridDim.x >> 3;
+        const int lo = (int)((long)n_patches * xcd / 8), hi = (int)((long)n_patches * (xcd + 1) / 8);
+        first_patch = lo + q;
+        patch_stride = nq;
+        my_patches = q < hi - lo ? (hi - lo - q + nq - 1) / nq : 0;
+    }
+    const int total = my_patches * NCH;
+
+    // requests: unconditional loads from clamped addresses, zeroed at consumption through nv[]
+    floatx4 raw[2][4];
+    int nv[2] = {0, 0};
+    const int t_comp = (t_ww - p.pad) & 3;
+    int ld_patch = first_patch, ld_chunk = 0, ld_it = 0;
+    const float* ld_src = p.x;
+    bool ld_ok = false;
+    int ld_hin = 0, ld_win = 0;
+    const float* ld_cur = p.x;
+    int ld_n = 0, ld_c0 = 0;
+    auto load_begin = [&](int& nvalid) {
+        if (ld_chunk == 0) {
+            const bool live = ld_it < total;
+            const int patch = live ? ld_patch : 0;
+            const int b = patch / patches_per_image, r = patch % patches_per_image;
+            const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
+            ld_hin = th0 + t_hh - p.pad;
+            ld_win = tw0 + t_ww - p.pad;
+            const bool row_ok = live && (is_core || is_edge) && ld_hin >= 0 && ld_hin < p.H;
+            ld_ok = row_ok && ld_win >= 0 && ld_win < p.W;       // W % 4 == 0: a quad is all in or all out
+            ld_src = p.x + ((long)b * p.C + t_q4 * 4) * plane + (ld_ok ? (long)ld_hin * p.W + (ld_win & ~3) : 0);
+        }
+        ld_c0 = ld_chunk * IG_CC + t_q4 * 4;
+        int n = p.C - ld_c0;
+        n = n < 0 ? 0 : (n > 4 ? 4 : n);
+        ld_n = ld_ok ? n : 0;
+        nvalid = ld_n;
+        ld_cur = ld_n > 0 ? ld_src + (long)ld_chunk * IG_CC * plane : p.x;
+    };
+    auto load_one = [&](floatx4 (&dst)[4], const int e) {
+        dst[e] = *reinterpret_cast<const floatx4*>(ld_cur);
+        ld_cur += plane & -(long)(e + 1 < ld_n);
+    };
+    auto load_end = [&]() {
+        ld_it++;
+        if (++ld_chunk == NCH) { ld_chunk = 0; ld_patch += patch_stride; }
+    };
+    auto load_item = [&](floatx4 (&dst)[4], int& nvalid) {
+        load_begin(nvalid);
+#pragma unroll
+        for (int e = 0; e < 4; e++) load_one(dst, e);
+        load_end();
+    };
+    auto store_halo = [&](const floatx4 (&src)[4], const int nvalid, char* hb) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) asm volatile("" ::"v"(src[e]));   // every lane takes delivery of the set
+        if (!(is_core || is_edge)) return;
+        if (is_core) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                half4_t h;
+#pragma unroll
+                for (int e = 0; e < 4; e++) h[e] = e < nvalid ? (_Float16)src[e][q] : (_Float16)0.f;
+                *reinterpret_cast<half4_t*>(halo_slot(hb, t_hh, t_ww + q)) = h;
+            }
+        } else {
+            half4_t h;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float f = src[e][0];
+                f = t_comp == 1 ? src[e][1] : f;
+                f = t_comp == 2 ? src[e][2] : f;
+                f = t_comp == 3 ? src[e][3] : f;
+                h[e] = e < nvalid ? (_Float16)f : (_Float16)0.f;
+            }
+            *reinterpret_cast<half4_t*>(halo_slot(hb, t_hh, t_ww)) = h;
+        }
+    };
+
+    floatx16 acc[NI][FP];
+    auto init_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < NI; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const floatx4 bq = *reinterpret_cast<const floatx4*>(lds_bias + wn * WCH + i * 32 + g * 8 + lh * 4);
+#pragma unroll
+                for (int j = 0; j < FP; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) acc[i][j][g * 4 + q] = bq[q];
+            }
+    };
+
+    // chunk c out of halo buffer hb, ninth tap out of w9; after_tap(tap) runs behind the MFMAs of each tap
+    auto compute = [&](const int c, const char* hb, const half8_t (&w9)[NI], auto after_tap) {
+        const char* wrow = lds_w + c * W_CHUNK + (wn * WCH + li) * 256;
+        const int sw = li & 15;
+        half8_t wf[2][NI], pf[2][FP];
+        auto read_frags = [&](const int tap, half8_t (&w)[NI], half8_t (&x)[FP]) {
+            const int kh = tap / KW, kw = tap % KW;
+#pragma unroll
+            for (int i = 0; i < NI; i++)
+                w[i] = tap < 8 ? *reinterpret_cast<const half8_t*>(wrow + i * 32 * 256 + (((tap * 2 + lh) ^ sw) << 4)) : w9[i];
+#pragma unroll
+            for (int j = 0; j < FP; j++) {
+                const int blk = wm * FP + j;
+                const int col = (blk % CB) * 32 + li + kw;
+                x[j] = *reinterpret_cast<const half8_t*>(hb + lh * H_PLANE + ((blk / CB + kh) * G::WW + col) * 16);
+            }
+        };
+        read_frags(0, wf[0], pf[0]);
+#pragma unroll
+        for (int tap = 0; tap < 9; tap++) {
+            if (tap + 1 < 9) read_frags(tap + 1, wf[(tap + 1) & 1], pf[(tap + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);                   // requests stay ahead of the MFMAs below
+#pragma unroll
+            for (int i = 0; i < NI; i++)
+#pragma unroll
+                for (int j = 0; j < FP; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf[tap & 1][i], pf[tap & 1][j], acc[i][j], 0, 0, 0);
+            after_tap(tap);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    const int o_wave = o_tile * BN + wn * WCH;
+    const bool o_full = o_tile * BN + BN <= p.O;
+    const long hw_out = (long)p.H_out * p.W_out;
+    auto flush_unit = [&](const int j, const int i, const int patch) {
+        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
+        const int blk = wm * FP + j;
+        const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
+        const bool inside = o_full && th0 + G::TH <= p.H_out && tw0 + TW <= p.W_out;   // uniform
+        const bool pix_ok = inside || (ho < p.H_out && wo < p.W_out);
+        const long pix = pix_ok ? (long)ho * p.W_out + wo : 0;
+        const unsigned lane_bytes = (unsigned)((pix + (long)lh * 4 * hw_out) * 4);
+        char* pl = reinterpret_cast<char*>(p.y + ((long)b * p.O + o_wave + i * 32) * hw_out);
+        const int o_lane = o_wave + i * 32 + lh * 4;
+        float bv[16];
+        if (PIX_BIAS) {
+#pragma unroll
+            for (int rr = 0; rr < 16; rr++) {
+                const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
+                bv[rr] = p.bias[(long)b * p.bias_sn + pix * p.bias_sp + (long)((o_full || o < p.O) ? o : 0) * p.bias_sc];
+            }
+        }
+        auto finished = [&](const int rr) {
+            float v = acc[i][j][rr];
+            if (PIX_BIAS) v += bv[rr];
+            return fmaxf(v, p.relu ? 0.f : v);                  // NaN -> 0 under ReLU, like x > 0 ? x : 0
+        };
+        int step_lo = __builtin_amdgcn_readfirstlane((int)(hw_out * 4)),
+            step_hi = __builtin_amdgcn_readfirstlane((int)((hw_out * 4) >> 32));
+        asm volatile("" : "+s"(step_lo), "+s"(step_hi));        // plane addresses are stepped, not kept in registers
+        const long step1 = ((long)step_hi << 32) | (unsigned)step_lo, step5 = step1 * 5;
+        if (inside) {
+#pragma unroll
+            for (int rr = 0; rr < 16; rr++) {
+                *reinterpret_cast<float*>(pl + lane_bytes) = finished(rr);
+                pl += (rr & 3) == 3 ? step5 : step1;
+            }
+        } else {
+#pragma unroll
+            for (int rr = 0; rr < 16; rr++) {
+                const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
+                const float v = finished(rr);
+                if (pix_ok && o < p.O) *reinterpret_cast<float*>(pl + lane_bytes) = v;
+                pl += (rr & 3) == 3 ? step5 : step1;
+            }
+        }
+    };
+
+    auto lds_barrier = []() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    // Item k multiplies out of halo buffer k & 1. Register set (k + 1) & 1 holds item k + 1, requested two items
+    // ago: behind tap 4 (waves 0..3) or tap 6 (waves 4..7: the two waves of a SIMD, w and w + 4, do not round at
+    // the same time) it is rounded into the other halo buffer, and the set is at once requested again for item
+    // k + 3, one load behind each of the following taps. One barrier ends the item.
+    auto item = [&](floatx4 (&nxt)[4], int& n_nxt, const int c, const char* hb_cur, char* hb_next, const half8_t (&w9)[NI],
+                    half8_t (&w9_next)[NI]) {
+        compute(c, hb_cur, w9, [&](const int tap) {
+            if (tap == 3) request_w8(w9_next, c + 1 < NCH ? c + 1 : 0);
+            if (wave < 4) {
+                if (tap == 4) {
+                    store_halo(nxt, n_nxt, hb_next);
+                    load_begin(n_nxt);
+                }
+                if (tap >= 5) load_one(nxt, tap - 5);
+            } else {
+                if (tap == 6) {
+                    store_halo(nxt, n_nxt, hb_next);
+                    load_begin(n_nxt);
+                    load_one(nxt, 0);
+                    load_one(nxt, 1);
+                }
+                if (tap == 7) load_one(nxt, 2);
+                if (tap == 8) load_one(nxt, 3);
+            }
+        });
+        load_end();
+        lds_barrier();                                           // next halo complete, this one free again
+    };
+
+    load_item(raw[0], nv[0]);
+    load_item(raw[1], nv[1]);
+    if (tid < BN) lds_bias[tid] = my_bias;
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);                 // vmcnt(0): resident weights and both sets landed
+    store_halo(raw[0], nv[0], lds_h0);
+    load_item(raw[0], nv[0]);                                    // item 2
+    lds_barrier();
+    for (int pi = 0; pi < my_patches; pi++) {
+        init_acc();
+#pragma unroll 1
+        for (int c = 0; c < NCH; c += 2) {
+            item(raw[1], nv[1], c, lds_h0, lds_h1, w8[0], w8[1]);
+            item(raw[0], nv[0], c + 1, lds_h1, lds_h0, w8[1], w8[0]);
+        }
+        const int patch = first_patch + pi * patch_stride;
+#pragma unroll
+        for (int j = 0; j < FP; j++)
+#pragma unroll
+            for (int i = 0; i < NI; i++) flush_unit(j, i, patch);
+    }
+    // the requests issued for items past the end are still in flight
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);
+}
+
 static bool conv_igemm_applicable(size_t C, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t N) {
     (void)O;
     // pad <= K_w - 1 keeps the 32 aligned core columns of a tile inside its halo
@@ -1057,6 +1391,50 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     using G = IgemmGeom<KH, KW, TW, BN>;
     const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
     if (n_otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many output channels");
+    // Resident weights with two halo buffers: 3x3, 64-wide patches, 16-byte image rows, and exactly the chunk count
+    // the kernel is built for (64 input channels with a 128-channel tile, 128 with a 64-channel tile).
+    if constexpr (KH == 3 && KW == 3 && TW == 64) {
+        constexpr int NI = BN / 64, NCH = NI == 2 ? 4 : 8;
+        static const char* db_env = getenv("NZHIP_CONV_DB");     // 0: the single-buffer kernel (benchmarking only)
+        const bool vec4r = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+        const bool pixb = bias && bias_sp != 0;                  // per-pixel bias with a 128-channel tile: out of registers
+        if (!(db_env && atoi(db_env) == 0) && w_batch == 1 && n_chunks == NCH && vec4r && !(pixb && NI == 2)) {
+            constexpr size_t lds_need = (size_t)NCH * BN * 256 + 4 * CONV_DB_PLANE + 128 * sizeof(float);
+            static_assert(lds_need <= 160 * 1024 - 512, "LDS budget");
+            _Float16* wres = nullptr;
+            const size_t bytes = (size_t)n_otiles * NCH * BN * 288;
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&wres), bytes, s)) return rc;
+            dim3 pg((unsigned)((BN * 9 * IG_CC + 255) / 256), (unsigned)(n_otiles * NCH));
+            hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles);
+            IgemmArgs a;
+            a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
+            a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.H_out = (int)H_out; a.W_out = (int)W_out;
+            a.pad = (int)pad; a.n_chunks = NCH; a.n_otiles = n_otiles;
+            a.tiles_w = (int)((W_out + TW - 1) / TW);
+            a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
+            a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
+            a.patch_map = 1;
+            const long n_patches = (long)N * a.tiles_w * a.tiles_h;
+            int rc = NZHIP_OK;
+            if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
+            auto kdb = conv3x3_resident_db_kernel<false, NI, NCH>;
+            if constexpr (NI == 1) {
+                if (pixb) kdb = conv3x3_resident_db_kernel<true, NI, NCH>;
+            }
+            if (rc == NZHIP_OK)
+                rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kdb), (int)lds_need, "hipFuncSetAttribute(conv3x3_resident_db)");
+            if (rc == NZHIP_OK) {
+                const int cus = device_cu_count();
+                int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
+                if ((long)per_tile > n_patches) per_tile = (int)n_patches;
+                hipLaunchKernelGGL(kdb, dim3((unsigned)per_tile, (unsigned)n_otiles, 1), dim3(512), lds_need, s, a, (int)n_patches);
+                hipError_t e = hipGetLastError();
+                if (e != hipSuccess) rc = set_hip_error(e, "conv3x3_resident_db kernel launch");
+            }
+            int rc2 = workspace_free(wres, s);
+            return rc ? rc : rc2;
+        }
+    }
     // Resident-weight route: shared weights whose fp16 image (unpadded) plus one halo fit in LDS.
     {
         constexpr size_t W_CHUNK_R = BN * (size_t)G::TAPS * 32;
