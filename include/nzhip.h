@@ -87,11 +87,15 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream);
  * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose GEMM
  * driver allocates three temporaries per call (src/OperationKernels.cu:885-912).
  * Same arguments, same kernels and bit-identical results, but every workspace the routes use
- * (fp16 operand images of the two-pass route, split-contraction partial sums) lives in a static
- * device array of NZHIP_STATIC_SCRATCH_BYTES that each GPU holds from library load until the
- * process ends; the call performs no hipMalloc / hipFree and never touches the caching pool.
- * A product whose workspace would not fit is rejected with NZHIP_E_UNSUPPORTED before anything
- * is enqueued (nzhip_last_error() names the size).
+ * (fp16 operand images of the two-pass route, split-contraction partial sums, padded copies of
+ * operands whose rows do not allow 16-byte loads) lives in a static device array of
+ * NZHIP_STATIC_SCRATCH_BYTES that each GPU holds from library load until the process ends; the
+ * call performs no hipMalloc / hipFree and never touches the caching pool.
+ * A product whose workspace would not fit is rejected with NZHIP_E_UNSUPPORTED
+ * (nzhip_last_error() names the size) and leaves C untouched.  The one workspace that is only
+ * an optimisation, the padded operand copies, is given up instead when it does not fit: the
+ * product is then computed from the operands as given, and its sums may be grouped differently
+ * from nzhip_gemm's (same tolerance, not the same last bits).
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
  * streams, two threads) race; serialise them. */
 #define NZHIP_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
