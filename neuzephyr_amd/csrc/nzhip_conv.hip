@@ -1056,22 +1056,28 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
 template <int BN>
 __global__ __launch_bounds__(256) void conv_weight_image_db_kernel(_Float16* __restrict__ dst, const float* __restrict__ w_ref,
                                                                    int C, int O, int n_chunks, int n_otiles) {
+    // One thread per (row, tap) of a slab: 16 reads that are contiguous across the threads of a wave (adjacent
+    // output channels) and two 16-byte stores, instead of one 2-byte store per element.
     const int slab = blockIdx.y;                               // o_tile * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = slab / n_chunks;
     const int t = blockIdx.x * 256 + threadIdx.x;
-    const int o_l = t % BN, rest = t / BN;
-    if (rest >= 9 * IG_CC) return;
-    const int cc = rest % IG_CC, tap = rest / IG_CC;
-    const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
-    float v = 0.f;
-    if (c < C && o < O) v = w_ref[((long)c * 9 + tap) * O + o];
+    const int o_l = t % BN, tap = t / BN;
+    if (tap >= 9) return;
+    const int o = o_tile * BN + o_l;
+    half8_t h[2];
+#pragma unroll
+    for (int cc = 0; cc < IG_CC; cc++) {
+        const int c = chunk * IG_CC + cc;
+        const bool ok = c < C && o < O;
+        const float v = w_ref[ok ? ((long)c * 9 + tap) * O + o : 0];
+        h[cc >> 3][cc & 7] = ok ? (_Float16)v : (_Float16)0.f;
+    }
     _Float16* tile = dst + (long)o_tile * n_chunks * BN * 144;   // 288 bytes per (chunk, row)
-    const int half = cc >> 3;
-    if (tap < 8) {
-        const int slot = (tap * 2 + half) ^ (o_l & 15);
-        tile[((long)chunk * BN + o_l) * 128 + slot * 8 + (cc & 7)] = (_Float16)v;
-    } else {
-        tile[(long)n_chunks * BN * 128 + ((long)chunk * BN + o_l) * 16 + half * 8 + (cc & 7)] = (_Float16)v;
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        _Float16* q = tap < 8 ? tile + ((long)chunk * BN + o_l) * 128 + (((tap * 2 + half) ^ (o_l & 15)) << 3)
+                              : tile + (long)n_chunks * BN * 128 + ((long)chunk * BN + o_l) * 16 + half * 8;
+        *reinterpret_cast<half8_t*>(q) = h[half];
     }
 }
 
@@ -1404,7 +1410,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             _Float16* wres = nullptr;
             const size_t bytes = (size_t)n_otiles * NCH * BN * 288;
             if (int rc = workspace_alloc(reinterpret_cast<void**>(&wres), bytes, s)) return rc;
-            dim3 pg((unsigned)((BN * 9 * IG_CC + 255) / 256), (unsigned)(n_otiles * NCH));
+            dim3 pg((unsigned)((BN * 9 + 255) / 256), (unsigned)(n_otiles * NCH));
             hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles);
             IgemmArgs a;
             a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
