@@ -87,6 +87,14 @@ CONV_CASES = [
     (1, 9, 33, 36, 140, 3, 3, 1, 2, 1),     # padding 2: both halo columns on the left
     (2, 20, 16, 64, 64, 3, 3, 1, 1, 2),     # per-sample weights
     (1, 16, 12, 40, 8, 3, 3, 1, 3, 1),      # padding larger than the kernel reach: workspace route
+    # resident weights with two halo buffers (64 channels -> 128-channel tile, 128 -> 64-channel tile, 64-wide patches)
+    (1, 64, 9, 64, 128, 3, 3, 1, 1, 1),     # rows not a multiple of the 4-row patch
+    (2, 50, 12, 72, 100, 3, 3, 1, 1, 1),    # last chunk with 2 of 16 channels, part of a channel tile, ragged second patch
+    (1, 64, 8, 68, 130, 3, 3, 1, 0, 1),     # no padding, two channel tiles (the second with 2 channels)
+    (1, 64, 6, 64, 128, 3, 3, 1, 2, 1),     # padding 2
+    (2, 128, 10, 64, 64, 3, 3, 1, 1, 1),    # eight chunks, 64-channel tile
+    (1, 120, 7, 128, 40, 3, 3, 1, 1, 1),    # eight chunks, the last partial, 40 of 64 channels
+    (33, 64, 32, 64, 128, 3, 3, 1, 1, 1),   # 264 patches for 256 workgroups: uneven patch counts
 ]
 
 
@@ -111,8 +119,8 @@ def test_conv2d_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, 
     assert np.array_equal(host(y), got)
 
 
-def test_conv2d_per_pixel_bias_like_the_reference_parameter(nz, oracle):
-    N, C, H, W, O = 2, 5, 10, 9, 6
+@pytest.mark.parametrize("N,C,H,W,O", [(2, 5, 10, 9, 6), (1, 128, 9, 64, 64), (1, 64, 8, 64, 128)])
+def test_conv2d_per_pixel_bias_like_the_reference_parameter(nz, oracle, N, C, H, W, O):
     x = oracle.fill((N, C, H, W), 61, "normal", 0.0, 1.0)
     w = oracle.fill((O, C, 3, 3), 62, "normal", 0.0, 0.2)
     Ho, Wo = oracle.out_hw(H, W, 3, 3, 1, 1)
