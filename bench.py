@@ -28,7 +28,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
-                    choices=["gemm8192", "gemm_batched", "linear", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "gemv", "ragged", "conv_a", "conv_b",
+                    choices=["gemm8192", "gemm256", "gemm1024", "gemm_batched", "linear", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "gemv", "ragged", "conv_a", "conv_b",
                              "adam", "softmax_bwd", "matmul_f32",
                              "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -239,6 +239,19 @@ def make_workload(name, orc, capi):
 
         return Workload(name, 2.0 * 4096 * 4096, 4.0 * (4096 + 4096 * 4096 + 4096), run, verify, "hbm",
                         "A[1,4096] * B[4096,4096]", another), None
+    if name in ("gemm256", "gemm1024"):
+        n = 256 if name == "gemm256" else 1024
+        A = orc.fill((n, n), 0, "uniform", -1.0, 1.0)
+        B = orc.fill((n, n), 1000, "uniform", -1.0, 1.0)
+        Ad, Bd = dev(A), dev(B)
+        out = torch.empty((n, n), device="cuda")
+
+        run = capi.prepare_gemm(Ad, Bd, out)
+
+        def verify():
+            return tolerance(orc, out.cpu().numpy(), orc.gemm_f64(A, B), name)
+
+        return Workload(name, 2.0 * n ** 3, 4.0 * 3 * n * n, run, verify, "mfma", f"A[{n},{n}] * B[{n},{n}], U[-1,1]"), None
     if name == "ragged":
         A = orc.fill((1000, 777), 3, "uniform", -1.0, 1.0)
         B = orc.fill((777, 513), 1003, "uniform", -1.0, 1.0)
@@ -522,7 +535,7 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "linear", "gemv", "ragged", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "adam",
+        for name in ("conv_b", "conv_a", "linear", "gemv", "ragged", "gemm256", "gemm1024", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "adam",
                      "softmax_bwd", "matmul_f32"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)
