@@ -449,34 +449,52 @@ bool gemm_vec_legal(const nzhip_gemm_desc& d) { return gemm_operands_vec_legal(d
 // ---- tile and split choice for products that do not fill the device -------------------------------
 // The fused kernel's k loop is bound by the rate at which one CU takes fp32 tiles in through its L1
 // (about 50 GB/s per CU with 16-byte loads, 36 GB/s when they carry predicates, 9 GB/s element by element), so the time of a launch is
-// the bytes the busiest CU streams: rounds of workgroups x (tile rows + tile columns) x chunk length
-// x 4 bytes. 64 x 64 tiles stream twice the bytes of 128 x 128 tiles in total but put four times
+// the bytes the busiest CU streams: rounds of workgroups x (tile rows + tile columns, as far as the
+// operands reach) x chunk length x 4 bytes. 64 x 64 tiles stream twice the bytes of 128 x 128 tiles in total but put four times
 // as many CUs to work (1024^3: 23.6 us -> 14.2 us); a split contraction adds a pass over the partial sums.
-static double fused_cost_us(const nzhip_gemm_desc& d, int tile, int64_t parts, int64_t Kc, bool vec) {
-    const double cus = (double)device_cu_count();
-    const int64_t tiles = ((d.M + tile - 1) / tile) * ((d.N + tile - 1) / tile) * d.batch_n * d.batch_c * parts;
-    const double rounds = (double)((tiles + (int64_t)cus - 1) / (int64_t)cus);
-    const bool full = vec && gemm_c_vec_legal(d) && d.M % tile == 0 && d.N % tile == 0 && Kc % 32 == 0 && d.K % 32 == 0;   // unpredicated instance
-    const double stream = rounds * 2.0 * tile * (double)Kc * 4.0 / (full ? 50e3 : vec ? 36e3 : 9e3);   // bytes / (bytes per us)
-    const double out = (double)d.M * d.N * d.batch_n * 4.0;
+struct FusedCostInput {
+    int64_t M, N, K, members;       // members: batch_n * batch_c of the product as given
+    double cus;
+    bool vec, c_vec;
+};
+
+static double fused_cost_us(const FusedCostInput& q, int tile, int64_t parts, int64_t Kc) {
+    const int64_t tiles = ((q.M + tile - 1) / tile) * ((q.N + tile - 1) / tile) * q.members * parts;
+    const double rounds = (double)((tiles + (int64_t)q.cus - 1) / (int64_t)q.cus);
+    const bool full = q.vec && q.c_vec && q.M % tile == 0 && q.N % tile == 0 && Kc % 32 == 0 && q.K % 32 == 0;   // unpredicated instance
+    // rows past the operand's extent are predicated off, not loaded: a narrow operand costs what it has
+    const double rows = (double)(q.M < tile ? q.M : tile) + (double)(q.N < tile ? q.N : tile);
+    // two or more workgroups on a CU overlap their waits: the CU takes in up to 1.3 x what one workgroup draws
+    // (16 x 8192 x 8192: 50 us in eight chunks, two workgroups per CU, against 57 us in four)
+    const double per_cu = (double)tiles / q.cus;
+    const double overlap = per_cu >= 2.0 ? 1.3 : per_cu > 1.0 ? 1.0 + 0.3 * (per_cu - 1.0) : 1.0;
+    const double stream = rounds * rows * (double)Kc * 4.0 / ((full ? 50e3 : q.vec ? 36e3 : 9e3) * overlap);   // bytes / (bytes per us)
+    const double out = (double)q.M * q.N * q.members * 4.0;
     const double reduce = parts > 1 ? 6.0 + (double)(parts + 1) * out / 3e6 : 0.0;
-    return 3.0 + stream + reduce;
+    // what a workgroup spends outside its k loop (first requests, predicated epilogue): 17 x 33 x 15 takes 10 us with a
+    // 128 x 128 tile and 5 us with a 64 x 64 tile; rounds that share a CU pay it side by side
+    const double ends = (tile == 64 ? 1.5 : 4.0) * (rounds > 2.0 ? rounds / 2.0 : 1.0);
+    return 3.0 + ends + stream + reduce;
+}
+
+static FusedCostInput fused_cost_input(const nzhip_gemm_desc& d, int padded) {
+    return {d.M, d.N, d.K, d.batch_n * d.batch_c, (double)device_cu_count(), gemm_operands_vec_legal(d, padded), gemm_c_vec_legal(d)};
 }
 
 GemmPlan gemm_fused_plan(const nzhip_gemm_desc& d, int padded) {
+    const FusedCostInput q = fused_cost_input(d, padded);
     GemmPlan best = {128, 1, d.K, 0.0};
-    const bool vec = gemm_operands_vec_legal(d, padded);
-    double best_cost = fused_cost_us(d, 128, 1, d.K, vec);
+    double best_cost = fused_cost_us(q, 128, 1, d.K);
     auto consider = [&](int tile, int64_t parts, int64_t Kc) {
-        const double c = fused_cost_us(d, tile, parts, Kc, vec);
+        const double c = fused_cost_us(q, tile, parts, Kc);
         if (c < best_cost * 0.97) { best_cost = c; best = {tile, parts, Kc, 0.0}; }    // keep the plainer plan on a near tie
     };
     consider(64, 1, d.K);
     // a batch over n alone (batch_c == 1) can be split as well: the chunks take the c dimension of the launch
     if (d.batch_c == 1 && d.batch_n <= 65535 && d.K >= 512) {
         const bool narrow = d.M <= 64 || d.N <= 64;                // padded tiles: the k loop is shorter per byte
-        const int64_t min_chunk = vec && !narrow ? 512 : 128;
-        for (int64_t S = 2; S <= 1024 && S <= d.K / min_chunk; S += (S < 32 ? 1 : S / 8)) {
+        const int64_t min_chunk = q.vec && !narrow ? 512 : 128;
+        for (int64_t S = 2; S <= 1024 && S <= d.K / min_chunk; S += (S < 8 ? 1 : S / 4)) {   // about 25 candidates
             const int64_t Kc = ((d.K + S - 1) / S + 31) / 32 * 32;              // chunk length, whole 32-wide k tiles
             const int64_t parts = (d.K + Kc - 1) / Kc;                           // the last one may be shorter
             if (parts < 2) continue;
@@ -490,8 +508,8 @@ GemmPlan gemm_fused_plan(const nzhip_gemm_desc& d, int padded) {
 
 bool gemm_small_tile(const nzhip_gemm_desc& d, int padded) {
     // called with the descriptor of the launch itself (split chunks are its inner batch)
-    const bool vec = gemm_operands_vec_legal(d, padded);
-    return fused_cost_us(d, 64, 1, d.K, vec) < 0.97 * fused_cost_us(d, 128, 1, d.K, vec);
+    const FusedCostInput q = fused_cost_input(d, padded);
+    return fused_cost_us(q, 64, 1, d.K) < 0.97 * fused_cost_us(q, 128, 1, d.K);
 }
 
 int gemm_mfma_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int force_tile, int64_t k_total, int padded) {

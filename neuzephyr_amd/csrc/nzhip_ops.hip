@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 
 #include "nzhip_internal.h"
@@ -398,8 +399,8 @@ static int gemm_try_repacked(const nzhip_gemm_desc& d, hipStream_t s, bool* done
     // stand-in addresses for the cost estimate: only alignment and leading dimensions matter to it
     if (!a_ok) { g.A = nullptr; g.lda = a_ld; }
     if (!b_ok) { g.B = nullptr; g.ldb = b_ld; }
-    const double copy_us = 3.0 + 2.0 * (double)(a_bytes + b_bytes) / 3e6;
-    if (gemm_fused_plan(g, padded).cost_us + copy_us >= 0.9 * gemm_fused_plan(d).cost_us) return NZHIP_OK;
+    const double copy_us = 5.0 + 2.0 * (double)(a_bytes + b_bytes) / 3e6;      // launch and latency of the copy kernel, then its traffic
+    if (gemm_fused_plan(g, padded).cost_us + copy_us >= 0.9 * gemm_fused_plan(d).cost_us) return NZHIP_OK;   // two plans, ~50 estimates each
     const size_t a_off = (a_bytes + 255) & ~(size_t)255;
     char* ws = nullptr;
     if (workspace_alloc(reinterpret_cast<void**>(&ws), a_off + b_bytes, s) != NZHIP_OK) return NZHIP_OK;   // no room: as given
@@ -457,6 +458,11 @@ static int gemm_routed(const nzhip_gemm_desc& d, hipStream_t s, int padded) {
         }
     }
     GemmPlan plan = gemm_fused_plan(d, padded);
+    static const char* trace_env = getenv("NZHIP_TRACE");               // 1: one line per product on stderr (debugging only)
+    if (trace_env && atoi(trace_env))
+        fprintf(stderr, "nzhip_gemm %ld x %ld x %ld batch %ld x %ld%s: fused kernel, %d^2 tiles, %ld chunk(s) of %ld, model %.1f us\n",
+                (long)d.M, (long)d.K, (long)d.N, (long)d.batch_n, (long)d.batch_c, padded ? " (padded copies)" : "", plan.tile,
+                (long)plan.parts, (long)plan.Kc, plan.cost_us);
     static const char* sk_env = getenv("NZHIP_SPLITK");                  // benchmarking only: number of chunks
     if (sk_env && atoi(sk_env) >= 1 && d.batch_c == 1 && d.batch_n <= 65535) {
         const int64_t S = atoi(sk_env);
