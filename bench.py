@@ -19,7 +19,7 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS_FP16 = 2500.0      # MI355X dense fp16 MFMA
 PEAK_HBM_GBPS = 8000.0         # MI355X HBM3E
-PEAK_TFLOPS_FP32 = 157.3      # MI355X fp32 vector (counts packed FMAs)
+PEAK_TFLOPS_FP32 = 157.3      # MI355X fp32: vector (counts packed FMAs) and dense matrix peaks are the same figure
 
 
 def parse_args():
@@ -362,8 +362,8 @@ def make_workload(name, orc, capi):
                 raise SystemExit("VERIFY FAILED matmul_f32")
             return {"bit_exact": True}
 
-        return Workload(name, 2.0 * M ** 3, 12.0 * M * M, run, verify, "valu_fp32",
-                        "fp32-exact A[2048,2048] * B[2048,2048] (fp32 VALU kernel; fp32 vector peak 157.3 TFLOP/s)"), None
+        return Workload(name, 2.0 * M ** 3, 12.0 * M * M, run, verify, "mfma_fp32",
+                        "fp32-exact A[2048,2048] * B[2048,2048] (fp32 MFMA kernel; fp32 matrix peak 157.3 TFLOP/s)"), None
     if name == "copy":
         # Calibration only: a plain device copy of known size (1 GiB read + 1 GiB written), so that
         # rocprofv3's FETCH_SIZE / WRITE_SIZE readings can be scaled to bytes.
@@ -526,8 +526,8 @@ def main():
     if wl.bound == "mfma":
         roofline = {"bound": "mfma", "achieved": tflops, "peak": PEAK_TFLOPS_FP16, "unit": "TFLOP/s",
                     "frac": tflops / PEAK_TFLOPS_FP16, "traffic": traffic, "scope": scope}
-    elif wl.bound == "valu_fp32":        # the two fp32 vector kernels (not the default workload)
-        roofline = {"bound": "valu_fp32", "achieved": tflops, "peak": PEAK_TFLOPS_FP32, "unit": "TFLOP/s",
+    elif wl.bound in ("valu_fp32", "mfma_fp32"):        # the fp32 kernels (not the default workload)
+        roofline = {"bound": wl.bound, "achieved": tflops, "peak": PEAK_TFLOPS_FP32, "unit": "TFLOP/s",
                     "frac": tflops / PEAK_TFLOPS_FP32, "traffic": traffic, "scope": scope}
     else:
         roofline = {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s",
@@ -557,9 +557,10 @@ def main():
                           "frac_hbm_peak": w2.bytes / ms_rot / 1e6 / PEAK_HBM_GBPS,
                           "frac_mfma_peak_rotated_buffers": w2.flops / ms_rot / 1e9 / PEAK_TFLOPS_FP16})
                 torch.cuda.empty_cache()
-            if w2.bound == "valu_fp32":
+            if w2.bound in ("valu_fp32", "mfma_fp32"):
                 del extra[name]["frac_mfma_peak"]
-                extra[name]["frac_fp32_vector_peak"] = w2.flops / ms2 / 1e9 / PEAK_TFLOPS_FP32
+                key = "frac_fp32_vector_peak" if w2.bound == "valu_fp32" else "frac_fp32_matrix_peak"
+                extra[name][key] = w2.flops / ms2 / 1e9 / PEAK_TFLOPS_FP32
             del w2
 
     if args.workload == "gemm8192" and not args.no_extra:

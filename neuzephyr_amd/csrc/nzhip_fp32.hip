@@ -11,6 +11,7 @@
 namespace nzhip {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 
 static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
@@ -22,10 +23,12 @@ static int check_launch(const char* what) {
 }
 
 // ---- fp32 matmul --------------------------------------------------------------------------------
-// 128 x 128 output tile per workgroup, 16 x 16 threads with an 8 x 8 register block each, k in
-// steps of 16 through LDS (A stored k-major so that both fragment reads are contiguous). Every
-// output is one chain of FMAs in ascending k, the same arithmetic as a scalar loop
-// `sum = fma(a[k], b[k], sum)`, so integer data and the CPU restatement match bit for bit.
+// 128 x 128 output tile per workgroup, four waves of 64 x 64 (2 x 2 blocks of v_mfma_f32_32x32x2_f32),
+// k in steps of 16 through LDS (A stored k-major so that both fragment reads are 32 adjacent
+// floats). The fp32 MFMA adds its two products to the accumulator one after the other, each as a
+// fused multiply-add, in ascending k (checked on the device against a scalar chain over operands
+// of widely different magnitudes: 1024 of 1024 outputs identical), so every output is the chain
+// `sum = fma(a[k], b[k], sum)` of the CPU restatement, bit for bit; the tests hold it to that.
 struct F32Args {
     const float* A;
     const float* B;
@@ -41,7 +44,7 @@ constexpr int F32_BM = 128, F32_BN = 128, F32_BK = 16;
 __global__ __launch_bounds__(256) void matmul_f32_kernel(const F32Args p) {
     __shared__ __attribute__((aligned(16))) float As[2][F32_BK][F32_BM + 4];   // [k][m]
     __shared__ __attribute__((aligned(16))) float Bs[2][F32_BK][F32_BN + 4];   // [k][n]
-    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int tid = threadIdx.x;
     const int m0 = blockIdx.y * F32_BM, n0 = blockIdx.x * F32_BN;
     const int bi = blockIdx.z / p.batch_c, bj = blockIdx.z % p.batch_c;
     const float* __restrict__ A = p.A + bi * p.a_sn + bj * p.a_sc;
@@ -92,11 +95,15 @@ __global__ __launch_bounds__(256) void matmul_f32_kernel(const F32Args p) {
         }
     };
 
-    float acc[8][8];
+    const int lane = tid & 63, wave = tid >> 6, li = lane & 31, lh = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    floatx16 acc[2][2];
 #pragma unroll
-    for (int i = 0; i < 8; i++)
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) acc[i][j] = 0.f;
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
     const int nk = (p.K + F32_BK - 1) / F32_BK;
     fetch(0);
@@ -106,32 +113,34 @@ __global__ __launch_bounds__(256) void matmul_f32_kernel(const F32Args p) {
         const int buf = kt & 1;
         if (kt + 1 < nk) fetch((kt + 1) * F32_BK);
 #pragma unroll
-        for (int k = 0; k < F32_BK; k++) {
-            // rows ty*4..+3 and 64+ty*4..+3, columns tx*4..+3 and 64+tx*4..+3
-            const floatx4 a0 = *reinterpret_cast<const floatx4*>(&As[buf][k][ty * 4]);
-            const floatx4 a1 = *reinterpret_cast<const floatx4*>(&As[buf][k][64 + ty * 4]);
-            const floatx4 b0 = *reinterpret_cast<const floatx4*>(&Bs[buf][k][tx * 4]);
-            const floatx4 b1 = *reinterpret_cast<const floatx4*>(&Bs[buf][k][64 + tx * 4]);
+        for (int k = 0; k < F32_BK; k += 2) {
+            // lane (li, lh) brings row / column li of its blocks at k + lh; zero rows past K add fma(0, 0, sum) = sum
+            float a[2], b[2];
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const float a = i < 4 ? a0[i] : a1[i - 4];
+            for (int i = 0; i < 2; i++) a[i] = As[buf][k + lh][wm * 64 + i * 32 + li];
 #pragma unroll
-                for (int j = 0; j < 8; j++) acc[i][j] = __builtin_fmaf(a, j < 4 ? b0[j] : b1[j - 4], acc[i][j]);
-            }
+            for (int j = 0; j < 2; j++) b[j] = Bs[buf][k + lh][wn * 64 + j * 32 + li];
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
         }
         if (kt + 1 < nk) stash(buf ^ 1);
         __syncthreads();
     }
+    // accumulator register r of lane (li, lh): row (r / 4) * 8 + lh * 4 + r % 4, column li of the 32 x 32 block
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int m = m0 + (i < 4 ? ty * 4 + i : 64 + ty * 4 + i - 4);
-        if (m >= p.M) continue;
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int n = n0 + (j < 4 ? tx * 4 + j : 64 + tx * 4 + j - 4);
-            if (n < p.N) C[(long)m * p.N + n] = acc[i][j];
+        for (int r = 0; r < 16; r++) {
+            const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+            if (m >= p.M) continue;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int n = n0 + wn * 64 + j * 32 + li;
+                if (n < p.N) C[(long)m * p.N + n] = acc[i][j][r];
+            }
         }
-    }
 }
 
 // ---- optimizer steps ----------------------------------------------------------------------------

@@ -47,6 +47,19 @@ def test_matmul_f32_bit_identical_to_the_oracle(nz, oracle, sa, sb):
     assert np.array_equal(got, oracle.general_matmul(A, B))
 
 
+def test_matmul_f32_is_one_fma_chain_in_ascending_k(nz, oracle):
+    # operands spread over 20 binades: a different order of the additions, or products rounded before they are added,
+    # would change most outputs (the kernel's fp32 MFMAs must behave like the scalar chain)
+    rng = np.random.default_rng(99)
+    A = (rng.standard_normal((1, 1, 160, 777)) * np.exp2(rng.integers(-10, 11, size=(1, 1, 160, 777)))).astype(np.float32)
+    B = (rng.standard_normal((1, 1, 777, 200)) * np.exp2(rng.integers(-10, 11, size=(1, 1, 777, 200)))).astype(np.float32)
+    got = host(nz.matmul_f32(dev(A), dev(B)))
+    want = oracle.general_matmul(A, B)
+    assert np.array_equal(got, want)
+    # and the chain is not what numpy's pairwise float32 product gives: the check above can tell orders apart
+    assert not np.array_equal(want[0, 0], A[0, 0] @ B[0, 0])
+
+
 def test_matmul_f32_rejects_bad_shapes(nz):
     with pytest.raises(nz.NzHipError):
         nz.matmul_f32(dev(np.zeros((1, 1, 2, 3))), dev(np.zeros((1, 1, 4, 2))))
