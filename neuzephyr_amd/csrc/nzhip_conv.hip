@@ -1397,48 +1397,56 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     using G = IgemmGeom<KH, KW, TW, BN>;
     const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
     if (n_otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many output channels");
-    // Resident weights with two halo buffers: 3x3, 64-wide patches, 16-byte image rows, and exactly the chunk count
-    // the kernel is built for (64 input channels with a 128-channel tile, 128 with a 64-channel tile).
+    // Resident weights with two halo buffers: 3x3, 64-wide patches, 16-byte image rows, and one of the chunk counts
+    // the kernel is built for (2 or 4 chunks of 16 input channels with a 128-channel tile; 2, 4 or 8 with a 64-channel
+    // tile, whose eight chunks still fit LDS).
     if constexpr (KH == 3 && KW == 3 && TW == 64) {
-        constexpr int NI = BN / 64, NCH = NI == 2 ? 4 : 8;
+        constexpr int NI = BN / 64;
         static const char* db_env = getenv("NZHIP_CONV_DB");     // 0: the single-buffer kernel (benchmarking only)
         const bool vec4r = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
         const bool pixb = bias && bias_sp != 0;                  // per-pixel bias with a 128-channel tile: out of registers
-        if (!(db_env && atoi(db_env) == 0) && w_batch == 1 && n_chunks == NCH && vec4r && !(pixb && NI == 2)) {
-            constexpr size_t lds_need = (size_t)NCH * BN * 256 + 4 * CONV_DB_PLANE + 128 * sizeof(float);
-            static_assert(lds_need <= 160 * 1024 - 512, "LDS budget");
-            _Float16* wres = nullptr;
-            const size_t bytes = (size_t)n_otiles * NCH * BN * 288;
-            if (int rc = workspace_alloc(reinterpret_cast<void**>(&wres), bytes, s)) return rc;
-            dim3 pg((unsigned)((BN * 9 + 255) / 256), (unsigned)(n_otiles * NCH));
-            hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles);
-            IgemmArgs a;
-            a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
-            a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.H_out = (int)H_out; a.W_out = (int)W_out;
-            a.pad = (int)pad; a.n_chunks = NCH; a.n_otiles = n_otiles;
-            a.tiles_w = (int)((W_out + TW - 1) / TW);
-            a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
-            a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
-            a.patch_map = 1;
-            const long n_patches = (long)N * a.tiles_w * a.tiles_h;
-            int rc = NZHIP_OK;
-            if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
-            auto kdb = conv3x3_resident_db_kernel<false, NI, NCH>;
-            if constexpr (NI == 1) {
-                if (pixb) kdb = conv3x3_resident_db_kernel<true, NI, NCH>;
-            }
-            if (rc == NZHIP_OK)
-                rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kdb), (int)lds_need, "hipFuncSetAttribute(conv3x3_resident_db)");
-            if (rc == NZHIP_OK) {
-                const int cus = device_cu_count();
-                int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
-                if ((long)per_tile > n_patches) per_tile = (int)n_patches;
-                hipLaunchKernelGGL(kdb, dim3((unsigned)per_tile, (unsigned)n_otiles, 1), dim3(512), lds_need, s, a, (int)n_patches);
-                hipError_t e = hipGetLastError();
-                if (e != hipSuccess) rc = set_hip_error(e, "conv3x3_resident_db kernel launch");
-            }
-            int rc2 = workspace_free(wres, s);
-            return rc ? rc : rc2;
+        const bool count_ok = n_chunks == 2 || n_chunks == 4 || (n_chunks == 8 && NI == 1);
+        if (!(db_env && atoi(db_env) == 0) && w_batch == 1 && count_ok && vec4r && !(pixb && NI == 2)) {
+            auto run = [&](auto nch_tag) -> int {
+                constexpr int NCH = decltype(nch_tag)::value;
+                constexpr size_t lds_need = (size_t)NCH * BN * 256 + 4 * CONV_DB_PLANE + 128 * sizeof(float);
+                static_assert(lds_need <= 160 * 1024 - 512, "LDS budget");
+                _Float16* wres = nullptr;
+                const size_t bytes = (size_t)n_otiles * NCH * BN * 288;
+                if (int rc = workspace_alloc(reinterpret_cast<void**>(&wres), bytes, s)) return rc;
+                dim3 pg((unsigned)((BN * 9 + 255) / 256), (unsigned)(n_otiles * NCH));
+                hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles);
+                IgemmArgs a;
+                a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
+                a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.H_out = (int)H_out; a.W_out = (int)W_out;
+                a.pad = (int)pad; a.n_chunks = NCH; a.n_otiles = n_otiles;
+                a.tiles_w = (int)((W_out + TW - 1) / TW);
+                a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
+                a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
+                a.patch_map = 1;
+                const long n_patches = (long)N * a.tiles_w * a.tiles_h;
+                int rc = NZHIP_OK;
+                if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
+                auto kdb = conv3x3_resident_db_kernel<false, NI, NCH>;
+                if constexpr (NI == 1) {
+                    if (pixb) kdb = conv3x3_resident_db_kernel<true, NI, NCH>;
+                }
+                if (rc == NZHIP_OK)
+                    rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kdb), (int)lds_need, "hipFuncSetAttribute(conv3x3_resident_db)");
+                if (rc == NZHIP_OK) {
+                    const int cus = device_cu_count();
+                    int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
+                    if ((long)per_tile > n_patches) per_tile = (int)n_patches;
+                    hipLaunchKernelGGL(kdb, dim3((unsigned)per_tile, (unsigned)n_otiles, 1), dim3(512), lds_need, s, a, (int)n_patches);
+                    hipError_t e = hipGetLastError();
+                    if (e != hipSuccess) rc = set_hip_error(e, "conv3x3_resident_db kernel launch");
+                }
+                int rc2 = workspace_free(wres, s);
+                return rc ? rc : rc2;
+            };
+            if (n_chunks == 2) return run(std::integral_constant<int, 2>{});
+            if (n_chunks == 4) return run(std::integral_constant<int, 4>{});
+            if constexpr (NI == 1) return run(std::integral_constant<int, 8>{});
         }
     }
     // Resident-weight route: shared weights whose fp16 image (unpadded) plus one halo fit in LDS.

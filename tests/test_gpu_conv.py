@@ -95,6 +95,11 @@ CONV_CASES = [
     (2, 128, 10, 64, 64, 3, 3, 1, 1, 1),    # eight chunks, 64-channel tile
     (1, 120, 7, 128, 40, 3, 3, 1, 1, 1),    # eight chunks, the last partial, 40 of 64 channels
     (33, 64, 32, 64, 128, 3, 3, 1, 1, 1),   # 264 patches for 256 workgroups: uneven patch counts
+    (2, 32, 10, 64, 128, 3, 3, 1, 1, 1),    # two chunks, 128-channel tile
+    (1, 20, 9, 72, 100, 3, 3, 1, 1, 1),     # two chunks, the second with 4 of 16 channels, part of a channel tile
+    (2, 64, 10, 64, 64, 3, 3, 1, 1, 1),     # four chunks, 64-channel tile
+    (1, 30, 7, 128, 40, 3, 3, 1, 0, 1),     # two chunks, 64-channel tile, no padding
+    (3, 17, 5, 64, 200, 3, 3, 1, 2, 1),     # two chunks (1 channel in the second), two channel tiles, padding 2
 ]
 
 
@@ -119,7 +124,7 @@ def test_conv2d_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, 
     assert np.array_equal(host(y), got)
 
 
-@pytest.mark.parametrize("N,C,H,W,O", [(2, 5, 10, 9, 6), (1, 128, 9, 64, 64), (1, 64, 8, 64, 128)])
+@pytest.mark.parametrize("N,C,H,W,O", [(2, 5, 10, 9, 6), (1, 128, 9, 64, 64), (1, 64, 8, 64, 128), (2, 64, 7, 64, 48), (1, 32, 8, 128, 64)])
 def test_conv2d_per_pixel_bias_like_the_reference_parameter(nz, oracle, N, C, H, W, O):
     x = oracle.fill((N, C, H, W), 61, "normal", 0.0, 1.0)
     w = oracle.fill((O, C, 3, 3), 62, "normal", 0.0, 0.2)
