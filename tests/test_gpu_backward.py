@@ -262,6 +262,39 @@ def test_conv2d_backward_weights_is_bit_exact_on_integers(nz, oracle, N, C, H, W
     assert np.array_equal(got, expect)
 
 
+def _conv_grad_sweep_cases(seed, count):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        C = int(rng.choice([1, 2, 3, 4, 8, 17, 32, 40, 64, 70, 128]))
+        O = int(rng.choice([1, 2, 5, 33, 64, 100, 128, 130]))
+        H = int(rng.integers(1, 20))
+        W = int(rng.choice([int(rng.integers(1, 40)), 8, 24, 64, 68, 72, 128, 136, 260]))
+        N = int(rng.integers(1, 4))
+        wb = int(rng.choice([1, 1, N]))
+        if N * O * H * W * C * 9 > 3e8:
+            continue
+        cases.append((N, C, H, W, O, wb))
+    return cases
+
+
+@pytest.mark.parametrize("N,C,H,W,O,wb", _conv_grad_sweep_cases(20252, 48))
+def test_conv2d_gradients_random_sweep_integers_bit_exact(nz, oracle, N, C, H, W, O, wb):
+    # 3x3, stride 1, padding 1 (what the fused gradients cover): both gradients against the node chain's sums
+    rng = np.random.default_rng(N * 5 + C * 7 + H * 11 + W * 13 + O * 17 + wb)
+    x = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    dy = rng.integers(-3, 4, size=(N, O, H, W)).astype(np.float32)
+    w = rng.integers(-3, 4, size=(wb, 1, C * 9, O)).astype(np.float32)
+    dw0 = rng.integers(-5, 6, size=(wb, 1, C * 9, O)).astype(np.float32)
+    expect_dw = oracle.conv2d_backward_weights(dw0.copy(), x, dy, 3, 3, 1)
+    got_dw = host(nz.conv2d_backward_weights(dev(dw0), dev(x), dev(dy), 3, 3, 1, 1))
+    assert np.array_equal(got_dw, expect_dw)
+    dx0 = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    expect_dx = oracle.conv2d_backward_data(dx0.copy(), dy, w, 3, 3, 1)
+    got_dx = host(nz.conv2d_backward_data(dev(dx0), dev(dy), dev(w), 3, 3, 1, 1, accumulate=True))
+    assert np.array_equal(got_dx, expect_dx)
+
+
 def test_conv2d_backward_weights_float_tolerance(nz, oracle):
     N, C, H, W, O = 2, 48, 20, 72, 80
     rng = np.random.default_rng(9)

@@ -124,6 +124,44 @@ def test_conv2d_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, 
     assert np.array_equal(host(y), got)
 
 
+def _conv_sweep_cases(seed, count):
+    """Random geometries over every route: direct / streaming (few channels), implicit GEMM with 32- and 64-wide
+    patches and both channel tiles, resident weights (single and double halo buffers), the column-matrix route
+    (strides, 2x3 / 5x5 kernels), per-sample weights."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        k = int(rng.choice([1, 2, 3, 3, 3, 5]))
+        k_w = 3 if k == 2 else k
+        stride = int(rng.choice([1, 1, 1, 2]))
+        pad = int(rng.integers(0, k_w))
+        C = int(rng.choice([1, 3, 8, 17, 32, 50, 64, 70, 128]))
+        O = int(rng.choice([1, 2, 5, 40, 64, 100, 128, 130]))
+        H = int(rng.integers(max(k, 1), 20))
+        W = int(rng.choice([int(rng.integers(max(k_w, 1), 40)), 64, 68, 72, 128, 132]))
+        N = int(rng.integers(1, 4))
+        wb = int(rng.choice([1, 1, 1, N]))
+        Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k_w) // stride + 1
+        if Ho < 1 or Wo < 1 or N * O * Ho * Wo * C * k * k_w > 3e8:
+            continue
+        cases.append((N, C, H, W, O, k, k_w, stride, pad, wb))
+    return cases
+
+
+@pytest.mark.parametrize("N,C,H,W,O,k_h,k_w,stride,pad,w_batch", _conv_sweep_cases(20251, 64))
+def test_conv2d_random_sweep_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, pad, w_batch):
+    rng = np.random.default_rng(N * 7 + C * 11 + H * 13 + W * 17 + O * 19 + k_h + stride + pad)
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    bias = rng.integers(-2, 3, size=(O,)).astype(np.float32)
+    ws = [rng.integers(-3, 4, size=(O, C, k_h, k_w)).astype(np.float32) for _ in range(w_batch)]
+    w_ref = np.concatenate([oracle.weights_oihw_to_ref(w) for w in ws], axis=0)
+    got = host(nz.conv2d_forward(dev(x), dev(w_ref), dev(bias), k_h, k_w, stride, pad, bias_strides=(0, 1), relu=True))
+    for n in range(N):
+        w = ws[n if w_batch > 1 else 0]
+        truth = oracle.conv2d_direct_f64(x[n:n + 1], w, bias, stride, pad, relu=True)
+        assert np.array_equal(got[n:n + 1].astype(np.float64), truth), (n,)
+
+
 @pytest.mark.parametrize("N,C,H,W,O", [(2, 5, 10, 9, 6), (1, 128, 9, 64, 64), (1, 64, 8, 64, 128), (2, 64, 7, 64, 48), (1, 32, 8, 128, 64)])
 def test_conv2d_per_pixel_bias_like_the_reference_parameter(nz, oracle, N, C, H, W, O):
     x = oracle.fill((N, C, H, W), 61, "normal", 0.0, 1.0)
