@@ -170,7 +170,8 @@ int nzhip_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, s
  * Img2ColNode::forward wrote (:605-630) and dC the pixel-major gradient from Col2ImgNode::backward (:660-665):
  *   dw[wb][(c,r,s)][o] += sum over h, w (and n, for shared weights) of
  *                         f16(x[n][c][h+r-pad][w+s-pad]) * f16(dy[n][o][h][w])
- * Supported: 3x3, stride 1, pad 1; anything else returns NZHIP_E_UNSUPPORTED and the caller runs the chain. */
+ * Supported: 3x3, stride 1, pad 1, and 1x1, stride 1, pad 0 (whose column matrix is x itself: one batched product);
+ * anything else returns NZHIP_E_UNSUPPORTED and the caller runs the chain. */
 int nzhip_conv2d_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H,
                                   size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
                                   size_t w_batch, void* stream);

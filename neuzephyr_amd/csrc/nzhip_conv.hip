@@ -2175,6 +2175,49 @@ extern "C" int nzhip_conv2d_backward_relu_bias(float* dz, float* dbias, const fl
     return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv_bias_grad (masked) kernel launch");
 }
 
+// dw[i] += P[0][i] + P[1][i] + ... (ascending, then added to dw once): the per-image products of the 1x1 weight gradient
+__global__ __launch_bounds__(256) void dw_add_members_kernel(float* __restrict__ dw, const float* __restrict__ P, int members, long n) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float sum = 0.f;
+    for (int m = 0; m < members; m++) sum += P[(long)m * n + i];
+    dw[i] += sum;
+}
+
+// Weight gradient of a 1x1, stride 1, unpadded convolution: its column matrix is x itself with pixels and channels
+// swapped, so MatMulNode::backward's dB += A^T * dC (src/Nodes.cu:169-182) is, per image,
+//   dw[c][o] += sum over pixels of f16(x[n][c][pixel]) * f16(dy[n][o][pixel]),
+// a product of two operands that both have the contraction contiguous. Per-sample weights: one batched product that
+// reads dw as its bias matrix and writes it back (every element is read and written by the same thread). Shared
+// weights: the per-image products go to a workspace and are added in ascending image order.
+static int conv1x1_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t HW, size_t O,
+                                    bool shared, hipStream_t s) {
+    nzhip_gemm_desc g = {};
+    g.A = x; g.M = (int64_t)C; g.K = (int64_t)HW; g.lda = (int64_t)HW; g.a_layout = NZHIP_LAYOUT_ROW;
+    g.B = dy; g.N = (int64_t)O; g.ldb = (int64_t)HW; g.b_layout = NZHIP_LAYOUT_TRANS;     // dy[n] is [O, pixels]: B^T as stored
+    g.ldc = (int64_t)O;
+    g.batch_n = (int64_t)N; g.batch_c = 1;
+    g.a_stride_n = (int64_t)(C * HW); g.b_stride_n = (int64_t)(O * HW); g.c_stride_n = (int64_t)(C * O);
+    g.activation = NZHIP_ACT_NONE;
+    if (!shared || N == 1) {
+        g.C = dw;
+        g.bias = dw; g.bias_stride_n = (int64_t)(C * O); g.bias_stride_row = (int64_t)O; g.bias_stride_col = 1;
+        return nzhip_gemm(&g, s);
+    }
+    float* P = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&P), N * C * O * sizeof(float), s)) return rc;
+    g.C = P;
+    int rc = nzhip_gemm(&g, s);
+    if (rc == NZHIP_OK) {
+        const long n = (long)(C * O);
+        hipLaunchKernelGGL(dw_add_members_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, dw, P, (int)N, n);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "dw_add_members kernel launch");
+    }
+    const int rc2 = workspace_free(P, s);
+    return rc ? rc : rc2;
+}
+
 /* Gradient of nzhip_conv2d_forward with respect to the weights, without the column matrix the reference's
  * chain needs (Img2ColNode::forward output as A in MatMulNode::backward, dB += A^T * dC, src/Nodes.cu:169-182):
  *   dW[wb][(c, r, s)][o] += sum over h, w (and over n when the weights are shared) of
@@ -2184,10 +2227,15 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
                                              size_t w_batch, void* stream) {
     if (!dw || !x || !dy) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_weights: null pointer");
     if (w_batch != 1 && w_batch != N) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
+    if (K_h == 1 && K_w == 1 && stride == 1 && pad == 0 && H > 0 && W > 0 && H * W < 0x3fffffff && C < 0x3fffffff &&
+        O < 0x3fffffff && N <= 65535 && N * C * O < 0x7fffffffull) {
+        if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
+        return conv1x1_backward_weights(dw, x, dy, N, C, H * W, O, w_batch == 1, reinterpret_cast<hipStream_t>(stream));
+    }
     if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1 || H == 0 || W == 0 || H > 0x3fffffff || W > 0x3fffffff ||
         C > 0x3fffffff || O > 0x3fffffff || N > 65535)
         return set_error(NZHIP_E_UNSUPPORTED,
-                         "nzhip_conv2d_backward_weights: only 3x3, stride 1, pad 1 (use the column-matrix chain)");
+                         "nzhip_conv2d_backward_weights: only 3x3, stride 1, pad 1 and 1x1, stride 1, pad 0 (use the column-matrix chain)");
     const bool vec = W % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
     if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);

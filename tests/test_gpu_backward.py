@@ -295,6 +295,42 @@ def test_conv2d_gradients_random_sweep_integers_bit_exact(nz, oracle, N, C, H, W
     assert np.array_equal(got_dx, expect_dx)
 
 
+CONV1X1_BWD_W = [  # N, C, H, W, O, w_batch   (1x1, stride 1, no padding: one batched product, no column matrix)
+    (1, 1, 1, 1, 1, 1), (1, 3, 4, 5, 2, 1), (2, 5, 7, 9, 6, 1), (3, 16, 8, 8, 24, 3), (2, 64, 16, 16, 128, 1), (4, 70, 9, 11, 33, 1),
+    (2, 128, 12, 20, 64, 2), (5, 3, 30, 33, 1, 1), (1, 256, 8, 8, 256, 1), (6, 8, 5, 5, 8, 6)]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,wb", CONV1X1_BWD_W)
+def test_conv1x1_backward_weights_is_bit_exact_on_integers(nz, oracle, N, C, H, W, O, wb):
+    rng = np.random.default_rng(N * 31 + C * 17 + H * 7 + W + O * 3 + wb)
+    x = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    dy = rng.integers(-3, 4, size=(N, O, H, W)).astype(np.float32)
+    dw0 = rng.integers(-5, 6, size=(wb, 1, C, O)).astype(np.float32)
+    expect = oracle.conv2d_backward_weights(dw0.copy(), x, dy, 1, 1, 0)
+    got = host(nz.conv2d_backward_weights(dev(dw0), dev(x), dev(dy), 1, 1, 1, 0))
+    assert np.array_equal(got, expect)
+    # the node chain's own product gives the same numbers: dB of MatMul.backward with the column matrix of a 1x1 kernel
+    col = host(nz.im2col(dev(x), 1, 1, 1, 0))                                     # [N, 1, HW, C]
+    dcol = np.ascontiguousarray(dy.reshape(N, 1, O, H * W).transpose(0, 1, 3, 2))  # [N, 1, HW, O]
+    chain = dw0.astype(np.float64).copy()
+    for n in range(N):
+        chain[n if wb > 1 else 0, 0] += col[n, 0].astype(np.float64).T @ dcol[n, 0].astype(np.float64)
+    assert np.array_equal(got.astype(np.float64), chain)
+
+
+def test_conv1x1_backward_weights_float_tolerance(nz, oracle):
+    N, C, H, W, O = 3, 96, 20, 28, 80
+    rng = np.random.default_rng(19)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, O, H, W)).astype(np.float32)
+    dw0 = rng.standard_normal((1, 1, C, O)).astype(np.float32)
+    got = host(nz.conv2d_backward_weights(dev(dw0), dev(x), dev(dy), 1, 1, 1, 0))
+    xr, dyr = oracle.round_f16(x).astype(np.float64), oracle.round_f16(dy).astype(np.float64)
+    truth = dw0.astype(np.float64) + np.einsum("nchw,nohw->co", xr, dyr).reshape(1, 1, C, O)
+    mr, fr = oracle.errors(got, truth, float(np.sqrt(np.mean(truth ** 2))))
+    assert mr <= 1e-3 and fr <= 1e-4, (mr, fr)
+
+
 def test_conv2d_backward_weights_float_tolerance(nz, oracle):
     N, C, H, W, O = 2, 48, 20, 72, 80
     rng = np.random.default_rng(9)
