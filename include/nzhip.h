@@ -112,15 +112,26 @@ size_t nzhip_static_scratch_bytes(void);
 int nzhip_gemm_force_tile(const nzhip_gemm_desc* desc, int tile, void* stream);
 /* Diagnostic (no counterpart in the reference): in the single-kernel route workgroups wait for each
  * other's rounding work with a bounded number of polls; *count receives how many waits have run out
- * since the library was loaded.  Anything but 0 means a product may be wrong (a device with fewer than
- * 256 free compute units).  Blocks until the device is idle.
- * The runtime looks at the same count by itself: the first nzhip_sync_ptr, nzhip_sync_all or
- * nzhip_memcpy_d2h that has drained the stream of such a product returns NZHIP_E_TIMEOUT once if the
- * count went up, and from then on nzhip_gemm keeps to the two-kernel route in this process. */
+ * since the library was loaded (expected: 0; anything else means a device with fewer than 256 free
+ * compute units, e.g. one shared with another process or stream).  Blocks until the device is idle.
+ * What C holds after a wait ran out: every workgroup looks at the launch's own count of such waits in
+ * front of its result stores, and from the first one on every 256 x 256 tile of C is written as NaN
+ * (tiles stored before it are complete and correct).  A product of this route can therefore be wrong
+ * only visibly, whichever stream it ran on and however the caller synchronises.
+ * The runtime looks at the process-wide count by itself as well: the first nzhip_sync_ptr,
+ * nzhip_sync_all or nzhip_memcpy_d2h that has drained the stream of such a product returns
+ * NZHIP_E_TIMEOUT once if the count went up (the copy or wait itself has been carried out: after
+ * nzhip_memcpy_d2h the destination is filled), and from then on nzhip_gemm keeps to the two-kernel
+ * route in this process. */
 int nzhip_gemm_coop_timeouts(unsigned* count);
 /* Test hook for that report: adds `inject` to the device-side count as if that many waits had run out
- * (no kernel misbehaves), or, with inject == 0, forgets earlier time-outs and allows the route again. */
+ * (no kernel misbehaves), or, with inject == 0, forgets earlier time-outs (the count reads 0 again) and allows the route again. */
 int nzhip_gemm_coop_reset(unsigned inject);
+/* Test hook for the waits themselves: spin_limit polls per wait (0 = the default, a few hundred ms) and,
+ * with mute != 0, workgroups that keep their arrivals to themselves, so that every wait of the following
+ * single-kernel products runs out after spin_limit polls.  All waves still run to the end of the kernel;
+ * the product comes out as NaN.  Always returns NZHIP_OK. */
+int nzhip_gemm_coop_test_mode(unsigned spin_limit, int mute);
 
 /* Drop-in for nz::data::iTensorCoreGEMM (include/NeuZephyr/TensorOperations.cuh:1021-1022,
  * src/TensorOperations.cu:112-115 -> krnl::TensorCoreGEMMParallel, src/OperationKernels.cu:914-1026):

@@ -654,10 +654,12 @@ struct CoopArgs {
     const float* srcA;
     const float* srcB;
     long lda, ldb;
-    unsigned* flags;            // one arrival counter per stage; zeroed by coop_prologue_kernel
+    unsigned* flags;            // one arrival counter per stage, then the launch's own count of waits that ran out;
+                                // zeroed by coop_prologue_kernel
     int sn;                     // tile blocks along N
     int waves, panels;
     unsigned spin_limit;
+    int mute;                   // test hook: producers keep their arrivals to themselves, so every wait runs out
 };
 
 __device__ unsigned g_coop_timeouts;   // polls that gave up (0 unless the device is shared or smaller than assumed)
@@ -753,6 +755,7 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
 
     // ---- stage counters -------------------------------------------------------------------------
     auto flag_of = [&](int w, int pn) { return q.flags + (long)w * q.panels + pn; };
+    unsigned* const launch_timeouts = q.flags + (long)q.waves * q.panels;
     auto wait_stage = [&](unsigned seen, unsigned* flag) {      // wave 0 only; seen: an earlier reading of *flag
         unsigned v = __builtin_amdgcn_readfirstlane(seen);
         unsigned polls = 0;
@@ -760,7 +763,15 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
             __builtin_amdgcn_s_sleep(16);
             v = __builtin_amdgcn_readfirstlane(__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
             if (++polls > q.spin_limit) {
-                if (lane == 0) atomicAdd(&g_coop_timeouts, 1u);
+                // Give up, but leave a mark that nobody can miss: the launch's own count (read by every workgroup
+                // in front of its result stores, which then write NaN) and the process-wide one (read by the host).
+                // The returning atomic is waited for, so the mark is in memory before this workgroup signals
+                // anything else.
+                if (lane == 0) {
+                    atomicAdd(&g_coop_timeouts, 1u);
+                    unsigned was = __hip_atomic_fetch_add(launch_timeouts, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    asm volatile("s_waitcnt vmcnt(0)" ::"v"(was) : "memory");
+                }
                 break;
             }
         }
@@ -885,7 +896,7 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
         // workgroup fence, which here (ordinary global loads and stores are in flight) drains every request.
         asm volatile("s_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
-        if (it == DRAIN_IT && t_any && tid == 0)
+        if (it == DRAIN_IT && t_any && tid == 0 && !q.mute)
             __hip_atomic_fetch_add(flag_of(t_w, t_p), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (it == POLL_IT && pn + 1 < q.panels && wave == 0)
             polled = __hip_atomic_load(flag_of(wv, pn + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -919,6 +930,11 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
     // ---- epilogue (whole tiles only: M and N are multiples of the tile) -----------------------------
+    // A wait that ran out anywhere in this launch before this point may have let somebody multiply image blocks
+    // that were not complete (this workgroup, or one whose arrival others relied on): the tile is then written
+    // as NaN, so that the product cannot be mistaken for a result.
+    const bool poisoned =
+        __builtin_amdgcn_readfirstlane(__hip_atomic_load(launch_timeouts, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) != 0;
     const float* bias = p.bias;
     const int gn = n0 + wn * TN + l16 * FN;
     float bcol[FN];
@@ -943,7 +959,7 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
             for (int j = 0; j < FN; j++) {
                 float x = acc[(j >> 2) * HALF + i * 4 + (j & 3)][r] + bv[r][j];
                 if (p.relu) x = x > 0.f ? x : 0.f;
-                v[j] = x;
+                v[j] = poisoned ? __builtin_nanf("") : x;
             }
             float* dst = C + (long)gm * p.ldc + gn;
             floatx4 o0 = {v[0], v[1], v[2], v[3]}, o1 = {v[4], v[5], v[6], v[7]};
@@ -980,6 +996,8 @@ static hipStream_t g_coop_stream = nullptr;      // the stream they all went to 
 static bool g_coop_mixed = false;                // ... unless they went to several
 static unsigned g_coop_seen = 0;                 // value of g_coop_timeouts at the last look
 static std::atomic<bool> g_coop_off{false};
+static std::atomic<unsigned> g_coop_spin_limit{200000};   // x (16 sleeps + one read): a few hundred ms
+static std::atomic<int> g_coop_mute{0};                   // test hook, see CoopArgs::mute
 
 // The single-kernel route wants one unbatched product of whole 16 x 16 tile blocks and whole panels, 16-byte
 // accesses everywhere, at least two stages to overlap, and a device on which a wave of 256 workgroups is
@@ -1002,7 +1020,7 @@ int gemm_h16_coop_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
     const size_t a_elems = (size_t)Mp * Kp, b_elems = (size_t)Np * Kp;
     const int nkt = (int)(Kp / CVT_K), panels = nkt / COOP_KP;
     const int sm = (int)(Mp / (COOP_SB * 256)), sn = (int)(Np / (COOP_SB * 256)), waves = sm * sn;
-    const int n_flags = waves * panels;
+    const int n_flags = waves * panels + 1;                             // stage counters + the launch's time-out count
     const size_t img_bytes = (a_elems + b_elems) * sizeof(_Float16);
     char* ws = nullptr;
     if (int rc = workspace_alloc(reinterpret_cast<void**>(&ws), img_bytes + (size_t)n_flags * sizeof(unsigned), s)) return rc;
@@ -1030,7 +1048,8 @@ int gemm_h16_coop_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
     g.tiles_m = (int)(Mp / 256); g.tiles_n = (int)(Np / 256); g.group_m = 4;
     a.srcA = d.A; a.srcB = d.B; a.lda = d.lda; a.ldb = d.ldb;
     a.flags = flags; a.sn = sn; a.waves = waves; a.panels = panels;
-    a.spin_limit = 200000;                                             // x (16 sleeps + one read): a few hundred ms
+    a.spin_limit = g_coop_spin_limit.load(std::memory_order_relaxed);
+    a.mute = g_coop_mute.load(std::memory_order_relaxed);
 
     // stage (0, 0): the first 16 row blocks of both operands over the first panel; also clears the counters
     dim3 pgrid((unsigned)COOP_KP, (unsigned)(2 * COOP_SB), 1);
@@ -1077,8 +1096,8 @@ int gemm_h16_coop_check(hipStream_t drained, bool whole_device) {
     g_coop_seen = count;
     g_coop_off.store(true, std::memory_order_relaxed);
     return set_error(NZHIP_E_TIMEOUT,
-                     "nzhip_gemm: %u bounded waits of the single-kernel route ran out (is the device shared?): the result of "
-                     "that product may be wrong; this process uses the two-kernel route from now on",
+                     "nzhip_gemm: %u bounded waits of the single-kernel route ran out (is the device shared?): that product "
+                     "holds NaN in every tile stored after the first of them; this process uses the two-kernel route from now on",
                      fresh);
 }
 
@@ -1094,12 +1113,20 @@ int gemm_h16_coop_reset(unsigned inject) {
         e = hipMemcpyToSymbol(HIP_SYMBOL(g_coop_timeouts), &count, sizeof(unsigned));
         if (e != hipSuccess) return set_hip_error(e, "hipMemcpyToSymbol(g_coop_timeouts)");
     } else {
-        g_coop_seen = count;
+        count = 0;
+        e = hipMemcpyToSymbol(HIP_SYMBOL(g_coop_timeouts), &count, sizeof(unsigned));
+        if (e != hipSuccess) return set_hip_error(e, "hipMemcpyToSymbol(g_coop_timeouts)");
+        g_coop_seen = 0;
         g_coop_pending = 0;
         g_coop_mixed = false;
         g_coop_off.store(false, std::memory_order_relaxed);
     }
     return NZHIP_OK;
+}
+
+void gemm_h16_coop_test_mode(unsigned spin_limit, int mute) {
+    g_coop_spin_limit.store(spin_limit ? spin_limit : 200000u, std::memory_order_relaxed);
+    g_coop_mute.store(mute, std::memory_order_relaxed);
 }
 
 int gemm_h16_coop_timeouts(unsigned* count) {

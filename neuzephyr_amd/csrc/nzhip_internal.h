@@ -36,6 +36,7 @@ int gemm_h16_coop_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
 // single-kernel product that has finished by now ran out of polls; the route is switched off from then on.
 int gemm_h16_coop_check(hipStream_t drained, bool whole_device);
 int gemm_h16_coop_reset(unsigned inject);
+void gemm_h16_coop_test_mode(unsigned spin_limit, int mute);   // test hook: bound of the waits (0 = default), producers that do not signal
 int gemm_h16_coop_timeouts(unsigned* count);     // polls that gave up since the library was loaded (expected: 0)
 // Bandwidth-bound kernels for M <= 8 (nzhip_skinny.hip).
 int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);

@@ -535,6 +535,11 @@ int nzhip_gemm_coop_timeouts(unsigned* count) {
 
 int nzhip_gemm_coop_reset(unsigned inject) { return gemm_h16_coop_reset(inject); }
 
+int nzhip_gemm_coop_test_mode(unsigned spin_limit, int mute) {
+    gemm_h16_coop_test_mode(spin_limit, mute);
+    return NZHIP_OK;
+}
+
 int nzhip_tensorcore_gemm(const float* A, const float* B, float* C, const size_t sA[4], const size_t sB[4],
                           const size_t sC[4], void* stream) {
     if (!A || !B || !C || !sA || !sB || !sC) return set_error(NZHIP_E_INVALID, "nzhip_tensorcore_gemm: null argument");

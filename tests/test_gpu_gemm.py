@@ -231,6 +231,59 @@ def test_single_kernel_route_reports_waits_that_ran_out(nz):
     assert torch.equal(nz.gemm(A, B, force_tile=28), want)
 
 
+def test_single_kernel_route_writes_nan_when_a_wait_runs_out(nz):
+    # The waits are made to run out from the host: producers keep their arrivals to themselves and a wait gives
+    # up after one poll. Every wave still runs to the end of the kernel; the product must then be NaN all over
+    # (never a plausible wrong number), the runtime must say so at the next blocking call, and the route must
+    # work again once the hook is off.
+    import torch
+    lib = nz.load()
+    M, K, N = 4096, 2048, 4096
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    A = torch.randint(-4, 5, (M, K), generator=gen, device="cuda").float()
+    B = torch.randint(-4, 5, (K, N), generator=gen, device="cuda").float()
+    want = nz.gemm(A, B, force_tile=18)
+    torch.cuda.synchronize()
+    nz.check(lib.nzhip_gemm_coop_reset(0))
+    try:
+        nz.check(lib.nzhip_gemm_coop_test_mode(1, 1))
+        got = torch.zeros((M, N), device="cuda")
+        nz.gemm(A, B, out=got, force_tile=28)
+        torch.cuda.synchronize()
+        assert bool(torch.isnan(got).all())
+        with pytest.raises(nz.NzHipError) as e:
+            nz.check(lib.nzhip_sync_all())
+        assert e.value.status == -5 and "NaN" in str(e.value)
+    finally:
+        nz.check(lib.nzhip_gemm_coop_test_mode(0, 0))
+        nz.check(lib.nzhip_gemm_coop_reset(0))
+    assert torch.equal(nz.gemm(A, B, force_tile=28), want)
+
+
+@pytest.mark.parametrize("b_trans", [False, True])
+def test_single_kernel_route_equals_two_kernel_route_at_8192_cubed(nz, b_trans):
+    # the benchmarked shape in full (four waves of workgroups, eight panels), float data: both routes run the
+    # same tiles in the same k order, so every one of the 2^26 outputs must have the same bits; and a sample of
+    # rows agrees with fp64 accumulation of the rounded operands
+    import ctypes as C
+    import torch
+    n = 8192
+    gen = torch.Generator(device="cuda").manual_seed(8192 + b_trans)
+    A = torch.randn((n, n), generator=gen, device="cuda") / n ** 0.5
+    B = torch.randn((n, n), generator=gen, device="cuda") / n ** 0.5
+    one = nz.gemm(A, B, b_trans=b_trans, force_tile=28)
+    two = nz.gemm(A, B, b_trans=b_trans, force_tile=18)
+    assert torch.equal(one, two)
+    rows = torch.arange(0, n, 257, device="cuda")
+    Ah, Bh = A[rows].half().double(), B.half().double()
+    truth = Ah @ (Bh.T if b_trans else Bh)
+    err = (one[rows].double() - truth).abs().max() / truth.pow(2).mean().sqrt()
+    assert float(err) <= 1e-3
+    cnt = C.c_uint(123)
+    nz.check(nz.load().nzhip_gemm_coop_timeouts(C.byref(cnt)))
+    assert cnt.value == 0
+
+
 def _route_sweep_cases():
     # seeded shapes aimed at the boundaries of the route choice: skinny extents 1..9 on either side,
     # long contractions with few tiles (split or not, vectorisable or not), mid-size and ragged shapes,
