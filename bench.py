@@ -417,6 +417,150 @@ def time_steps(wl, steps, warmup, do_settle=True):
     return start.elapsed_time(stop) / steps, wall * 1e3 / steps      # ms per step (device events, host wall)
 
 
+def per_step_stats(wl, steps):
+    """A second loop of `steps` runs with an event between every two of them: median, min and max of the
+    single steps in ms. The event packets sit between the kernels of neighbouring steps, so for steps of a
+    few microseconds these figures carry that gap; the mean of time_steps() (one event pair around the whole
+    loop) does not and stays the reported `ms_per_step`."""
+    import torch
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    ev[0].record()
+    for i in range(steps):
+        wl.run()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    ts = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
+    return {"median_ms": ts[len(ts) // 2], "min_ms": ts[0], "max_ms": ts[-1], "steps": steps}
+
+
+class PowerClockSampler:
+    """Best effort: reads the GPU's package power and shader clock from sysfs in a background thread while a
+    loop runs (amdgpu's hwmon power1_input / power1_average, pp_dpm_sclk). Figures are None where the files are
+    not there or not readable."""
+
+    def __init__(self):
+        import glob
+        dev = "/sys/class/drm/card*/device/"
+        self.pw = (glob.glob(dev + "hwmon/hwmon*/power1_input") + glob.glob(dev + "hwmon/hwmon*/power1_average"))[:1]
+        self.cap = glob.glob(dev + "hwmon/hwmon*/power1_cap")[:1]
+        self.ck = glob.glob(dev + "pp_dpm_sclk")[:1]
+        self.power, self.clock, self._stop, self._th = [], [], False, None
+
+    def _loop(self):
+        while not self._stop:
+            try:
+                if self.pw:
+                    self.power.append(int(open(self.pw[0]).read()) / 1e6)
+                if self.ck:
+                    cur = [l for l in open(self.ck[0]).read().splitlines() if "*" in l]
+                    if cur:
+                        self.clock.append(float(cur[0].split(":")[1].lower().replace("mhz", "").replace("*", "").strip()))
+            except (OSError, ValueError, IndexError):
+                pass
+            time.sleep(0.01)
+
+    def __enter__(self):
+        import threading
+        self.power, self.clock, self._stop = [], [], False
+        self._th = threading.Thread(target=self._loop, daemon=True)
+        self._th.start()
+        return self
+
+    def __exit__(self, *a):
+        self._stop = True
+        self._th.join()
+
+    @staticmethod
+    def _median(v):
+        v = sorted(v)
+        return v[len(v) // 2] if v else None
+
+    def result(self, skip=0.25):
+        """medians over the samples after the first quarter (the ramp after an idle period)"""
+        p, c = self.power[int(len(self.power) * skip):], self.clock[int(len(self.clock) * skip):]
+        cap = None
+        try:
+            cap = int(open(self.cap[0]).read()) / 1e6 if self.cap else None
+        except (OSError, ValueError):
+            pass
+        return {"power_W": self._median(p), "sclk_MHz": self._median(c), "power_cap_W": cap, "samples": len(p)}
+
+
+def box_ceilings(capi, wl_run):
+    """What this box sustains: (i) a register-only MFMA loop (random fp16 operands; zeros for comparison) with the
+    clock the chip held under it, (ii) a plain 16-byte copy over rotated buffers (nothing served by the caches)
+    and over the same buffers, (iii) package power and shader clock while the headline workload runs back to
+    back for about a second."""
+    import ctypes as C
+    import torch
+    lib = capi.load()
+    out = {}
+    ws = torch.zeros(65536 // 4, dtype=torch.float32, device="cuda")
+    stream = C.c_void_p(int(torch.cuda.current_stream().cuda_stream))
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    passes = 4000
+    for zero, key in ((0, "mfma_loop_random_operands"), (1, "mfma_loop_zero_operands")):
+        for _ in range(4):                                            # settle: ~40 ms of the loop
+            capi.check(lib.nzhip_probe_mfma(passes, zero, ws.data_ptr(), 65536, stream))
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 10
+        e0.record()
+        for _ in range(reps):
+            capi.check(lib.nzhip_probe_mfma(passes, zero, ws.data_ptr(), 65536, stream))
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        st = ws[: 2 * cus * 2].view(torch.int64).cpu().tolist()       # (shader ticks, 100 MHz ticks) per workgroup
+        ratios = sorted(st[2 * i] / st[2 * i + 1] for i in range(cus) if st[2 * i + 1] > 0)
+        out[key] = {"TFLOP/s": cus * 4 * passes * 64 * 16384.0 / ms / 1e9,
+                    "clock_MHz": 100.0 * ratios[len(ratios) // 2] if ratios else None,
+                    "desc": f"{cus} workgroups x 4 waves x {passes} x 64 v_mfma_f32_16x16x32_f16 from registers"}
+    # copy: 4 source/destination pairs of 256 MiB each (2 GiB in all) used round robin, and one pair reused
+    n = 1 << 26
+    pairs = [(torch.rand(n, device="cuda"), torch.empty(n, device="cuda")) for _ in range(4)]
+
+    def copy_loop(k, reps):
+        for i in range(8):
+            capi.check(lib.nzhip_probe_copy(pairs[i % k][1].data_ptr(), pairs[i % k][0].data_ptr(), 4 * n, stream))
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(reps):
+            capi.check(lib.nzhip_probe_copy(pairs[i % k][1].data_ptr(), pairs[i % k][0].data_ptr(), 4 * n, stream))
+        e1.record()
+        torch.cuda.synchronize()
+        return 8.0 * n * reps / (e0.elapsed_time(e1) * 1e-3) / 1e9
+
+    out["copy_rotated_GB/s"] = copy_loop(4, 40)
+    assert torch.equal(pairs[3][1], pairs[3][0])
+    del pairs[1:]
+    out["copy_same_buffers_256MiB_GB/s"] = copy_loop(1, 40)
+    n_small = 1 << 24                                                  # 64 MiB + 64 MiB: fits the memory-side cache
+    src, dst = pairs[0][0][:n_small], pairs[0][1][:n_small]
+    for _ in range(8):
+        capi.check(lib.nzhip_probe_copy(dst.data_ptr(), src.data_ptr(), 4 * n_small, stream))
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(100):
+        capi.check(lib.nzhip_probe_copy(dst.data_ptr(), src.data_ptr(), 4 * n_small, stream))
+    e1.record()
+    torch.cuda.synchronize()
+    out["copy_same_buffers_64MiB_GB/s"] = 8.0 * n_small * 100 / (e0.elapsed_time(e1) * 1e-3) / 1e9
+    del pairs, src, dst
+    torch.cuda.empty_cache()
+    with PowerClockSampler() as smp:
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 1.0:
+            for _ in range(16):
+                wl_run()
+            torch.cuda.synchronize()
+    out["under_headline_workload"] = smp.result()
+    return out
+
+
 ROTATE_MIN_BYTES = 640 << 20
 
 
@@ -508,6 +652,7 @@ def main():
 
     wl, host_ops = make_workload(args.workload, orc, capi)
     ms_dev, ms_wall = time_steps(wl, args.steps, args.warmup, not args.no_settle)
+    step_stats = per_step_stats(wl, args.steps)
     verified = None if args.no_verify else wl.verify()
 
     tflops = wl.flops / (ms_dev * 1e-3) / 1e12
@@ -540,9 +685,10 @@ def main():
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)
             ms2, _ = time_steps(w2, max(10, args.steps // 2), max(3, args.warmup // 2))
+            st2 = per_step_stats(w2, max(10, args.steps // 2))
             v2 = None if args.no_verify else w2.verify()
             ms_cold = time_cold(w2)
-            extra[name] = {"ms": ms2, "ms_cold_caches": ms_cold, "GB/s_cold_caches": w2.bytes / ms_cold / 1e6,
+            extra[name] = {"ms": ms2, "per_step_events": st2, "ms_cold_caches": ms_cold, "GB/s_cold_caches": w2.bytes / ms_cold / 1e6,
                            "TFLOP/s": w2.flops / ms2 / 1e9, "GB/s": w2.bytes / ms2 / 1e6,
                            "frac_mfma_peak": w2.flops / ms2 / 1e9 / PEAK_TFLOPS_FP16,
                            "frac_hbm_peak": w2.bytes / ms2 / 1e6 / PEAK_HBM_GBPS, "verified": v2, "workload": w2.desc}
@@ -577,6 +723,18 @@ def main():
             except (subprocess.TimeoutExpired, ValueError, IndexError) as e:
                 extra["readme_example_training_step"] = {"error": str(e)[:300]}
 
+    ceilings = None
+    if args.workload == "gemm8192" and not args.no_extra:
+        torch.cuda.empty_cache()
+        ceilings = box_ceilings(capi, wl.run)
+        mf, cp = ceilings["mfma_loop_random_operands"]["TFLOP/s"], ceilings["copy_rotated_GB/s"]
+        roofline["frac_of_box_mfma_loop"] = tflops / mf
+        for e in extra.values():
+            if isinstance(e, dict) and "TFLOP/s" in e and "frac_mfma_peak" in e:
+                e["frac_of_box_mfma_loop"] = e["TFLOP/s"] / mf
+            if isinstance(e, dict) and "GB/s_rotated_buffers" in e:
+                e["frac_of_box_copy_rotated"] = e["GB/s_rotated_buffers"] / cp
+
     cpu = None
     if args.workload == "gemm8192" and not args.no_cpu_baseline:
         cpu = cpu_baseline_gemm(orc, *host_ops)
@@ -586,7 +744,7 @@ def main():
         "value": gbps if wl.bound == "hbm" else tflops,
         "unit": "GB/s" if wl.bound == "hbm" else "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_dev, "ms_per_step_host_wall": ms_wall,
+        "ms_per_step": ms_dev, "ms_per_step_host_wall": ms_wall, "per_step_events": step_stats,
         "untimed_settle_s_before_warmup": 0.0 if args.no_settle else SETTLE_SECONDS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "dtype_note": "fp32 operands rounded to fp16 (RNE), fp16 MFMA, fp32 accumulate and output",
@@ -595,6 +753,7 @@ def main():
                    "algorithmic_bytes": wl.bytes},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "box_ceilings": ceilings,
         "verified": verified,
         "conv_and_other_configs": extra,
     }

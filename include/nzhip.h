@@ -61,7 +61,10 @@ int nzhip_device_info(int* cu_count, size_t* lds_bytes_per_cu, char* arch_name, 
  * Strides are in elements; a batch stride of 0 broadcasts that operand.
  * bias may be NULL; its element for output (m,n) of batch (i,j) is
  *     bias[i*bias_stride_n_batch + j*bias_stride_c_batch + m*bias_stride_row + n*bias_stride_col]
- * so a per-row vector, a per-column vector and a full [M,N] matrix are all expressible. */
+ * so a per-row vector, a per-column vector and a full [M,N] matrix are all expressible.
+ * bias may be C itself with C's strides ("C += A*B", how the backward entry points accumulate): on every
+ * route the thread that stores C(m,n) is the one that read bias(m,n) before.  Any other overlap of bias
+ * and C, and any overlap of A or B with C, is undefined. */
 typedef struct nzhip_gemm_desc {
     const float* A;
     const float* B;
@@ -83,8 +86,11 @@ typedef struct nzhip_gemm_desc {
 
 int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream);
 
-/* nzhip_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight
- * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose GEMM
+/* nzhip_gemm for callers that cannot allocate device memory (tight serving loops, harnesses that
+ * forbid hipMalloc, code that is to run under HIP graph capture -- not tested under capture here; the first
+ * call on a device looks up the static array's address and raises kernels' dynamic-LDS limits, which are
+ * driver calls, so make one call of each shape class outside a capture first).  No counterpart in the
+ * reference, whose GEMM
  * driver allocates three temporaries per call (src/OperationKernels.cu:885-912).
  * Same arguments, same kernels and bit-identical results, but every workspace the routes use
  * (fp16 operand images of the two-pass route, split-contraction partial sums, padded copies of
@@ -132,6 +138,21 @@ int nzhip_gemm_coop_reset(unsigned inject);
  * single-kernel products runs out after spin_limit polls.  All waves still run to the end of the kernel;
  * the product comes out as NaN.  Always returns NZHIP_OK. */
 int nzhip_gemm_coop_test_mode(unsigned spin_limit, int mute);
+
+/* Measurement hooks (no counterpart in the reference; not used by any product path): what the GPU at hand
+ * sustains with only its matrix pipes, or only its memory system, at work -- the two figures a benchmark
+ * sets a kernel's rate against, next to the published peaks.
+ * nzhip_probe_mfma: one workgroup of four waves per compute unit; every wave issues `passes` x 64
+ * v_mfma_f32_16x16x32_f16 on fragments held in registers (a fixed pseudo-random fp16 pattern, or zeros with
+ * zero_operands != 0), i.e. cu_count x 4 x passes x 64 x 16384 flop per call; time it with events on
+ * `stream`.  `workspace`: device memory of NZHIP_PROBE_MFMA_WORKSPACE_BYTES, 16-byte aligned; after the call
+ * its first 2 x cu_count 64-bit words hold, per workgroup, the elapsed shader-clock ticks and the elapsed ticks
+ * of the constant 100 MHz counter of the loop (ticks ratio x 100 MHz = the clock the chip held under the loop).
+ * nzhip_probe_copy: dst[0, bytes) = src[0, bytes) with 16-byte accesses (both 16-byte aligned, bytes a
+ * multiple of 16): 2 x bytes of memory traffic per call. */
+#define NZHIP_PROBE_MFMA_WORKSPACE_BYTES ((size_t)65536)
+int nzhip_probe_mfma(int passes, int zero_operands, void* workspace, size_t workspace_bytes, void* stream);
+int nzhip_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
 
 /* Drop-in for nz::data::iTensorCoreGEMM (include/NeuZephyr/TensorOperations.cuh:1021-1022,
  * src/TensorOperations.cu:112-115 -> krnl::TensorCoreGEMMParallel, src/OperationKernels.cu:914-1026):

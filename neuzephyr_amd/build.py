@@ -11,7 +11,7 @@ LIB = os.path.join(HERE, "libnzhip.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 SOURCES = ["nzhip_gemm.hip", "nzhip_gemm_h16.hip", "nzhip_skinny.hip", "nzhip_conv.hip", "nzhip_ops.hip", "nzhip_fp32.hip",
-           "nzhip_nn.hip",
+           "nzhip_nn.hip", "nzhip_probe.hip",
            "nzhip_runtime.cpp"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=default",

@@ -16,7 +16,7 @@ LAYOUT_ROW, LAYOUT_TRANS = 0, 1
 
 EXPORTS = [
     "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_gemm_static",
-    "nzhip_static_scratch_bytes", "nzhip_gemm_force_tile", "nzhip_gemm_coop_timeouts", "nzhip_gemm_coop_reset", "nzhip_gemm_coop_test_mode", "nzhip_tensorcore_gemm",
+    "nzhip_static_scratch_bytes", "nzhip_gemm_force_tile", "nzhip_gemm_coop_timeouts", "nzhip_gemm_coop_reset", "nzhip_gemm_coop_test_mode", "nzhip_probe_mfma", "nzhip_probe_copy", "nzhip_tensorcore_gemm",
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
@@ -77,6 +77,8 @@ def load() -> C.CDLL:
     lib.nzhip_gemm_coop_timeouts.argtypes = [C.POINTER(C.c_uint)]
     lib.nzhip_gemm_coop_reset.argtypes = [C.c_uint]
     lib.nzhip_gemm_coop_test_mode.argtypes = [C.c_uint, C.c_int]
+    lib.nzhip_probe_mfma.argtypes = [C.c_int, C.c_int, vp, sz, vp]
+    lib.nzhip_probe_copy.argtypes = [vp, vp, sz, vp]
     lib.nzhip_tensorcore_gemm.argtypes = [vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_im2col.argtypes = [vp, vp] + [sz] * 10 + [vp]
     lib.nzhip_col2im.argtypes = [vp, vp, sz, sz, sz, sz, vp]

@@ -229,12 +229,15 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int strip = by * 4 + wave;
-    const int w0 = (bx * 64 + lane) * 4;
     const int h0 = strip * ST_ROWS;
-    if (w0 >= W || h0 >= H) {                                    // nothing to do but the workgroup's one barrier
+    if (h0 >= H) {                                               // a whole wave with nothing to do but the workgroup's one barrier
         park_weights();
         return;
     }
+    // Lanes past the last column stay in the walk (the barrier in park_weights() must not sit in a branch that
+    // only some lanes of a wave take): they work on the image's last quad of columns and store nothing.
+    const bool active = (bx * 64 + lane) * 4 < W;
+    const int w0 = active ? (bx * 64 + lane) * 4 : W - 4;
     const float* xb = x + (long)b * C_T * H * W;
     float* yb = y + (long)b * O_T * H * W;
     const long plane = (long)H * W;
@@ -366,7 +369,7 @@ __global__ __launch_bounds__(256) void conv3x3_stream_kernel(float* __restrict__
                     if (relu) a = a > 0.f ? a : 0.f;
                     ov[e] = a;
                 }
-                *reinterpret_cast<floatx4*>(yb + ((long)o * H + ho) * W + w0) = ov;
+                if (active) *reinterpret_cast<floatx4*>(yb + ((long)o * H + ho) * W + w0) = ov;
             }
         }
     }

@@ -8,6 +8,8 @@
 #include <iterator>
 #include <vector>
 
+#include <exception>
+
 #include "NeuZephyr/NeuZephyrCudaErrorHandling.cuh"
 #include "NeuZephyr/TensorOperations.cuh"
 #include "nzhip.h"
@@ -130,7 +132,14 @@ namespace nz::data {
         return *this;
     }
 
-    MappedTensor::~MappedTensor() noexcept(false) { release(); }
+    MappedTensor::~MappedTensor() noexcept(false) {
+        try {
+            release();
+        } catch (...) {
+            // a second exception during stack unwinding would end the process: report only when nothing else is in flight
+            if (std::uncaught_exceptions() == 0) throw;
+        }
+    }
 
     void MappedTensor::release() {
         // nzhip_host_free waits for the compute stream: a kernel may still be using the memory

@@ -297,7 +297,10 @@ def test_conv2d_gradients_random_sweep_integers_bit_exact(nz, oracle, N, C, H, W
 
 CONV1X1_BWD_W = [  # N, C, H, W, O, w_batch   (1x1, stride 1, no padding: one batched product, no column matrix)
     (1, 1, 1, 1, 1, 1), (1, 3, 4, 5, 2, 1), (2, 5, 7, 9, 6, 1), (3, 16, 8, 8, 24, 3), (2, 64, 16, 16, 128, 1), (4, 70, 9, 11, 33, 1),
-    (2, 128, 12, 20, 64, 2), (5, 3, 30, 33, 1, 1), (1, 256, 8, 8, 256, 1), (6, 8, 5, 5, 8, 6)]
+    (2, 128, 12, 20, 64, 2), (5, 3, 30, 33, 1, 1), (1, 256, 8, 8, 256, 1), (6, 8, 5, 5, 8, 6),
+    # per-sample weights (dw is read and written in place as the product's bias matrix) with a long contraction
+    # that is split into chunks, with pixel rows that forbid 16-byte loads (padded copies), and on the two-pass route
+    (2, 40, 32, 40, 24, 2), (2, 24, 31, 35, 40, 2), (3, 130, 45, 23, 70, 3), (2, 512, 48, 48, 512, 2)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,wb", CONV1X1_BWD_W)

@@ -139,6 +139,21 @@ def test_long_contractions_with_few_tiles_are_bit_exact_on_integers(nz, M, K, N,
     assert np.array_equal(got, expect)
 
 
+@pytest.mark.parametrize("M,K,N", [(300, 1000, 260), (130, 9000, 70), (999, 777, 513), (1024, 2048, 1024), (64, 64, 64)])
+@pytest.mark.parametrize("force", [0, 64, 128, 256, 18, 12])
+def test_bias_may_alias_the_output(nz, M, K, N, force):
+    # "C += A B": the bias operand is C itself, element for element. Every route reads bias(m, n) in the
+    # thread that writes C(m, n), also behind a split contraction or padded operand copies.
+    rng = np.random.default_rng(M + 3 * K + 5 * N + force)
+    A = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, size=(K, N)).astype(np.float32)
+    C0 = rng.integers(-100, 101, size=(M, N)).astype(np.float32)
+    expect = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32) + C0
+    Cd = dev(C0)
+    nz.gemm(dev(A), dev(B), bias=Cd, bias_strides=(N, 1), out=Cd, force_tile=force)
+    assert np.array_equal(host(Cd), expect)
+
+
 COOP = [(4096, 2048, 4096), (8192, 1024, 4096), (4096, 1024, 8192), (8192, 2048, 8192)]
 
 
