@@ -28,7 +28,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
-                    choices=["gemm8192", "gemm256", "gemm1024", "gemm_batched", "linear", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "gemv", "ragged", "conv_a", "conv_b",
+                    choices=["gemm8192", "gemm256", "gemm1024", "gemm_batched", "linear", "linear_prepared", "conv_a_prepared", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "gemv", "ragged", "conv_a", "conv_b",
                              "adam", "softmax_bwd", "matmul_f32",
                              "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -98,7 +98,7 @@ def make_workload(name, orc, capi):
 
         return Workload(name, 2.0 * 128 * 1024 ** 3, 3.0 * 128 * 1024 * 1024 * 4, run, verify, "mfma",
                         "[8,16,1024,1024] x [8,16,1024,1024] batched over (N,C)"), None
-    if name == "linear":
+    if name in ("linear", "linear_prepared"):
         Nb, IN, OUT = 4096, 1024, 4096
         X = orc.fill((Nb, IN), 2, "normal", 0.0, 1.0)
         bound = float(np.sqrt(6.0 / IN))
@@ -107,17 +107,22 @@ def make_workload(name, orc, capi):
         Xd, Wd, bd = dev(X), dev(Wt), dev(bias)
         out = torch.empty((Nb, OUT), device="cuda")
 
-        run = capi.prepare_gemm(Xd, Wd, out, b_trans=True, bias=bd, bias_strides=(0, 1), relu=True)
+        # "_prepared": the fp16 image of W kept in a prepared-operand handle between the calls (a layer whose
+        # weights do not change between forward passes)
+        handle = capi.Prepared() if name == "linear_prepared" else None
+        run = capi.prepare_gemm(Xd, Wd, out, b_trans=True, bias=bd, bias_strides=(0, 1), relu=True, prepared_b=handle)
 
         def verify():
             truth = np.maximum(orc.gemm_f64(X[:256], Wt, trans_b=True) + bias[None, :].astype(np.float64), 0)
             return tolerance(orc, out[:256].cpu().numpy(), truth, name)
 
         def another():
-            return capi.prepare_gemm(Xd.clone(), Wd.clone(), torch.empty_like(out), b_trans=True, bias=bd, bias_strides=(0, 1), relu=True)
+            return capi.prepare_gemm(Xd.clone(), Wd.clone(), torch.empty_like(out), b_trans=True, bias=bd, bias_strides=(0, 1), relu=True,
+                                     prepared_b=capi.Prepared() if handle is not None else None)
 
         return Workload(name, 2.0 * Nb * IN * OUT, 4.0 * (Nb * IN + IN * OUT + OUT + Nb * OUT), run, verify, "mfma",
-                        "Linear X[4096,1024] W[4096,1024]^T + bias, ReLU", another), None
+                        "Linear X[4096,1024] W[4096,1024]^T + bias, ReLU" + (", fp16 image of W kept between calls" if handle else ""),
+                        another), None
     if name == "linear_bwd":
         # backward of Model::Linear at the L config: W[1,1,OUT,IN] * x[n,1,IN,1] -> dW += dY^T X, dx += dY W
         Nb, IN, OUT = 4096, 1024, 4096
@@ -265,20 +270,21 @@ def make_workload(name, orc, capi):
 
         return Workload(name, 2.0 * 1000 * 777 * 513, 4.0 * (1000 * 777 + 777 * 513 + 1000 * 513), run, verify, "mfma",
                         "A[1000,777] * B[777,513]"), None
-    if name in ("conv_a", "conv_b"):
-        if name == "conv_a":
+    if name in ("conv_a", "conv_b", "conv_a_prepared"):
+        prepared = capi.Prepared() if name == "conv_a_prepared" else None
+        if name != "conv_b":
             N, C, H, W, O = 16, 64, 128, 128, 128
             x = orc.fill((N, C, H, W), 4, "normal", 0.0, 1.0)
         else:
             N, C, H, W, O = 10, 3, 1024, 1024, 1
             x = orc.fill((N, C, H, W), 14, "uniform", 0.0, 1.0)
-        w = orc.fill((O, C, 3, 3), 1004 if name == "conv_a" else 1014, "normal", 0.0, float(np.sqrt(2.0 / (C * 9))))
-        bias = orc.fill((O,), 2004 if name == "conv_a" else 2014, "uniform", -0.03, 0.03)
+        w = orc.fill((O, C, 3, 3), 1004 if name != "conv_b" else 1014, "normal", 0.0, float(np.sqrt(2.0 / (C * 9))))
+        bias = orc.fill((O,), 2004 if name != "conv_b" else 2014, "uniform", -0.03, 0.03)
         xd, wd, bd = dev(x), dev(orc.weights_oihw_to_ref(w)), dev(bias)
         out = torch.empty((N, O, H, W), device="cuda")
 
         def run():
-            capi.conv2d_forward(xd, wd, bd, 3, 3, 1, 1, bias_strides=(0, 1), relu=True, out=out)
+            capi.conv2d_forward(xd, wd, bd, 3, 3, 1, 1, bias_strides=(0, 1), relu=True, out=out, prepared_w=prepared)
 
         def verify():
             truth = orc.conv2d_direct_f64(x[:1], w, bias, 1, 1, relu=True)
@@ -288,13 +294,14 @@ def make_workload(name, orc, capi):
             x2, out2 = xd.clone(), torch.empty_like(out)
 
             def run2():
-                capi.conv2d_forward(x2, wd, bd, 3, 3, 1, 1, bias_strides=(0, 1), relu=True, out=out2)
+                capi.conv2d_forward(x2, wd, bd, 3, 3, 1, 1, bias_strides=(0, 1), relu=True, out=out2, prepared_w=prepared)
             return run2
 
         flops = 2.0 * N * H * W * C * 9 * O
         bytes_ = 4.0 * (N * C * H * W + O * C * 9 + O + N * O * H * W)
         return Workload(name, flops, bytes_, run, verify, "hbm",
-                        f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},3,3] s1 p1 + bias + ReLU", another), None
+                        f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},3,3] s1 p1 + bias + ReLU" +
+                        (", fp16 image of the weights kept between calls" if prepared else ""), another), None
     if name == "adam":
         # opt::Adam::step over 2^26 parameters: data, m, v read and written, the gradient read
         n = 1 << 26
@@ -680,7 +687,7 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "linear", "gemv", "ragged", "gemm256", "gemm1024", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "adam",
+        for name in ("conv_b", "conv_a", "conv_a_prepared", "linear", "linear_prepared", "gemv", "ragged", "gemm256", "gemm1024", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "adam",
                      "softmax_bwd", "matmul_f32"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)
@@ -722,6 +729,19 @@ def main():
                                                          else {"error": out.stderr[-300:]})
             except (subprocess.TimeoutExpired, ValueError, IndexError) as e:
                 extra["readme_example_training_step"] = {"error": str(e)[:300]}
+
+    if args.workload == "gemm8192" and not args.no_extra:
+        # single layers through the C++ nz:: API (Model::forward()), with and without the kept weight images
+        exe = os.path.join(ROOT, "neuzephyr_amd", "nz", "examples", "layer_bench")
+        if os.path.exists(exe):
+            torch.cuda.empty_cache()
+            import subprocess
+            try:
+                out = subprocess.run([exe, "200", "20"], capture_output=True, text=True, timeout=120)
+                extra["layers_through_model_forward"] = (json.loads(out.stdout.strip().splitlines()[-1]) if out.returncode == 0
+                                                         else {"error": out.stderr[-300:]})
+            except (subprocess.TimeoutExpired, ValueError, IndexError) as e:
+                extra["layers_through_model_forward"] = {"error": str(e)[:300]}
 
     ceilings = None
     if args.workload == "gemm8192" and not args.no_extra:

@@ -139,6 +139,29 @@ int nzhip_gemm_coop_reset(unsigned inject);
  * the product comes out as NaN.  Always returns NZHIP_OK. */
 int nzhip_gemm_coop_test_mode(unsigned spin_limit, int mute);
 
+/* ---- prepared operands ---------------------------------------------------------------------------------
+ * No counterpart in the reference, which rounds and pads both operands anew on every call
+ * (src/OperationKernels.cu:940-975).  Several routes first turn an operand into an fp16 image: the two-pass
+ * GEMM route its B operand, the implicit-GEMM convolution kernels their weights.  A layer's weights do not
+ * change between forward calls, so a caller may keep that image in a handle: the first call through a handle
+ * builds the image into memory the handle owns, later calls with the same operand (address, extents, layout,
+ * and a route that wants the same image) skip the conversion kernel; anything else rebuilds it.  Routes
+ * without an image (skinny, fused convert-on-load, single-kernel, direct and column-matrix convolutions)
+ * ignore the handle.  Results are bit-identical with and without a handle.
+ * The library cannot see writes to the operand: after the weights change, call nzhip_prepared_invalidate
+ * before the next product (a stale image gives the product of the OLD weights, silently).
+ * A handle's image is filled on the stream of the call that builds it; use a handle on one stream at a time
+ * (or synchronise that stream before using the handle elsewhere).  nzhip_prepared_destroy returns the image
+ * to the pool in the order of that stream.  nzhip_prepared_fills: how often an image has been built through
+ * the handle (tests, tuning). */
+typedef struct nzhip_prepared nzhip_prepared;
+int nzhip_prepared_create(nzhip_prepared** handle);
+int nzhip_prepared_invalidate(nzhip_prepared* handle);
+int nzhip_prepared_fills(const nzhip_prepared* handle, unsigned long long* count);
+int nzhip_prepared_destroy(nzhip_prepared* handle);
+/* nzhip_gemm with the image of B kept in b_image (NULL: plain nzhip_gemm). */
+int nzhip_gemm_prepared_b(const nzhip_gemm_desc* desc, nzhip_prepared* b_image, void* stream);
+
 /* Measurement hooks (no counterpart in the reference; not used by any product path): what the GPU at hand
  * sustains with only its matrix pipes, or only its memory system, at work -- the two figures a benchmark
  * sets a kernel's rate against, next to the published peaks.
@@ -186,6 +209,12 @@ int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref, const flo
                          size_t N, size_t C, size_t H, size_t W, size_t O, size_t K_h, size_t K_w,
                          size_t stride, size_t pad, size_t w_batch, int64_t bias_stride_pixel,
                          int64_t bias_stride_channel, int activation, void* stream);
+/* nzhip_conv2d_forward with the fp16 image of the weights kept in w_image (see "prepared operands"; NULL:
+ * plain nzhip_conv2d_forward). */
+int nzhip_conv2d_forward_prepared(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
+                                  size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                                  size_t w_batch, int64_t bias_stride_pixel, int64_t bias_stride_channel, int activation,
+                                  nzhip_prepared* w_image, void* stream);
 
 /* Gradient of nzhip_conv2d_forward with respect to x, as one call. In the reference this is the chain
  * Col2ImgNode::backward (src/Nodes.cu:660-665) -> MatMulNode::backward, dA += dC * B^T (:169-182) ->

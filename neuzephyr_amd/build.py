@@ -75,6 +75,7 @@ def build_host_layer(verbose: bool = False) -> str:
     run([CXX, "-O2", "-mf16c", os.path.join(tests, "test_gpu.cpp"), "-o", os.path.join(tests, "test_gpu"), *common])
     examples = os.path.join(NZ, "examples")
     run([CXX, "-O2", os.path.join(examples, "readme_example.cpp"), "-o", os.path.join(examples, "readme_example"), *common])
+    run([CXX, "-O2", os.path.join(examples, "layer_bench.cpp"), "-o", os.path.join(examples, "layer_bench"), *common])
     return NZ_LIB
 
 

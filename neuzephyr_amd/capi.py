@@ -16,7 +16,8 @@ LAYOUT_ROW, LAYOUT_TRANS = 0, 1
 
 EXPORTS = [
     "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_gemm_static",
-    "nzhip_static_scratch_bytes", "nzhip_gemm_force_tile", "nzhip_gemm_coop_timeouts", "nzhip_gemm_coop_reset", "nzhip_gemm_coop_test_mode", "nzhip_probe_mfma", "nzhip_probe_copy", "nzhip_tensorcore_gemm",
+    "nzhip_static_scratch_bytes", "nzhip_gemm_force_tile", "nzhip_gemm_coop_timeouts", "nzhip_gemm_coop_reset", "nzhip_gemm_coop_test_mode", "nzhip_probe_mfma", "nzhip_probe_copy", "nzhip_prepared_create", "nzhip_prepared_invalidate", "nzhip_prepared_fills",
+    "nzhip_prepared_destroy", "nzhip_gemm_prepared_b", "nzhip_conv2d_forward_prepared", "nzhip_tensorcore_gemm",
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
@@ -79,6 +80,12 @@ def load() -> C.CDLL:
     lib.nzhip_gemm_coop_test_mode.argtypes = [C.c_uint, C.c_int]
     lib.nzhip_probe_mfma.argtypes = [C.c_int, C.c_int, vp, sz, vp]
     lib.nzhip_probe_copy.argtypes = [vp, vp, sz, vp]
+    lib.nzhip_prepared_create.argtypes = [C.POINTER(vp)]
+    lib.nzhip_prepared_invalidate.argtypes = [vp]
+    lib.nzhip_prepared_fills.argtypes = [vp, C.POINTER(C.c_ulonglong)]
+    lib.nzhip_prepared_destroy.argtypes = [vp]
+    lib.nzhip_gemm_prepared_b.argtypes = [C.POINTER(GemmDesc), vp, vp]
+    lib.nzhip_conv2d_forward_prepared.argtypes = [vp, vp, vp, vp] + [sz] * 10 + [i64, i64, C.c_int, vp, vp]
     lib.nzhip_tensorcore_gemm.argtypes = [vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_im2col.argtypes = [vp, vp] + [sz] * 10 + [vp]
     lib.nzhip_col2im.argtypes = [vp, vp, sz, sz, sz, sz, vp]
@@ -151,8 +158,39 @@ def _dev(t):
     return t.data_ptr()
 
 
+class Prepared:
+    """A prepared-operand handle (nzhip_prepared): owns the fp16 image of a weight operand between calls."""
+
+    def __init__(self):
+        self._h = C.c_void_p()
+        check(load().nzhip_prepared_create(C.byref(self._h)))
+
+    @property
+    def handle(self):
+        return self._h
+
+    def invalidate(self):
+        check(load().nzhip_prepared_invalidate(self._h))
+
+    def fills(self) -> int:
+        n = C.c_ulonglong(0)
+        check(load().nzhip_prepared_fills(self._h, C.byref(n)))
+        return n.value
+
+    def close(self):
+        if self._h:
+            check(load().nzhip_prepared_destroy(self._h))
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def gemm(A, B, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), relu=False, out=None,
-         force_tile=0, stream=None, static=False):
+         force_tile=0, stream=None, static=False, prepared_b=None):
     """C = act(f16(A) @ f16(B) + bias) for 2-D tensors. a_trans: A holds K x M; b_trans: B holds N x K.
     bias_strides = (row stride, column stride) in elements. static: through nzhip_gemm_static (the
     entry point that allocates nothing); `out` must then be given."""
@@ -174,7 +212,9 @@ def gemm(A, B, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), 
         d.bias = _dev(bias)
         d.bias_stride_row, d.bias_stride_col = bias_strides
     d.activation = ACT_RELU if relu else ACT_NONE
-    if static:
+    if prepared_b is not None:
+        check(lib.nzhip_gemm_prepared_b(C.byref(d), prepared_b.handle, _stream_handle(stream)))
+    elif static:
         check(lib.nzhip_gemm_static(C.byref(d), _stream_handle(stream)))
     elif force_tile:
         check(lib.nzhip_gemm_force_tile(C.byref(d), force_tile, _stream_handle(stream)))
@@ -183,7 +223,8 @@ def gemm(A, B, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), 
     return out
 
 
-def prepare_gemm(A, B, out, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), relu=False, stream=None):
+def prepare_gemm(A, B, out, *, a_trans=False, b_trans=False, bias=None, bias_strides=(0, 0), relu=False, stream=None,
+                 prepared_b=None):
     """Build the descriptor once and return a zero-argument callable that only enqueues the
     product (for timing loops, where per-call Python work would otherwise dominate small shapes)."""
     lib = load()
@@ -201,6 +242,14 @@ def prepare_gemm(A, B, out, *, a_trans=False, b_trans=False, bias=None, bias_str
         d.bias_stride_row, d.bias_stride_col = bias_strides
     d.activation = ACT_RELU if relu else ACT_NONE
     ref, h, fn = C.byref(d), C.c_void_p(_stream_handle(stream)), lib.nzhip_gemm
+    if prepared_b is not None:
+        pb, fp = prepared_b.handle, lib.nzhip_gemm_prepared_b
+
+        def call_prepared(_keep=(d, A, B, out, bias, prepared_b)):
+            st = fp(ref, pb, h)
+            if st:
+                check(st)
+        return call_prepared
 
     def call(_keep=(d, A, B, out, bias)):
         st = fn(ref, h)
@@ -241,7 +290,8 @@ def col2im(col, Ho, Wo, stream=None):
     return out
 
 
-def conv2d_forward(x, w_ref, bias, K_h, K_w, stride, pad, *, bias_strides=(0, 1), relu=False, out=None, stream=None):
+def conv2d_forward(x, w_ref, bias, K_h, K_w, stride, pad, *, bias_strides=(0, 1), relu=False, out=None, stream=None,
+                   prepared_w=None):
     """x [N,C,H,W]; w_ref [Wb,1,C*Kh*Kw,O]; bias_strides = (pixel stride, channel stride)."""
     import torch
     lib = load()
@@ -251,6 +301,11 @@ def conv2d_forward(x, w_ref, bias, K_h, K_w, stride, pad, *, bias_strides=(0, 1)
     Ho, Wo = (H + 2 * pad - K_h) // stride + 1, (W + 2 * pad - K_w) // stride + 1
     if out is None:
         out = torch.empty((N, O, Ho, Wo), dtype=torch.float32, device=x.device)
+    if prepared_w is not None:
+        check(lib.nzhip_conv2d_forward_prepared(_dev(out), _dev(x), _dev(w_ref), None if bias is None else _dev(bias), N, Cc,
+                                                H, W, O, K_h, K_w, stride, pad, Wb, bias_strides[0], bias_strides[1],
+                                                ACT_RELU if relu else ACT_NONE, prepared_w.handle, _stream_handle(stream)))
+        return out
     check(lib.nzhip_conv2d_forward(_dev(out), _dev(x), _dev(w_ref), None if bias is None else _dev(bias), N, Cc, H, W,
                                    O, K_h, K_w, stride, pad, Wb, bias_strides[0], bias_strides[1],
                                    ACT_RELU if relu else ACT_NONE, _stream_handle(stream)))

@@ -1393,6 +1393,15 @@ static bool conv_igemm_applicable(size_t C, size_t O, size_t K_h, size_t K_w, si
     return stride == 1 && ((K_h == 3 && K_w == 3) || (K_h == 1 && K_w == 1)) && pad <= K_w - 1 && C >= 8 && N <= 65535;
 }
 
+// Key of a weight image: everything the conversion kernel's output depends on (image kind, tile shape, source and extents).
+static void conv_image_key(uint64_t (&key)[PREPARED_KEY_WORDS], int kind, int kh, int kw, int bn, const float* w_ref, size_t C,
+                           size_t O, int n_chunks, int n_otiles, size_t w_batch) {
+    for (auto& k : key) k = 0;
+    key[0] = (uint64_t)kind | ((uint64_t)kh << 8) | ((uint64_t)kw << 16) | ((uint64_t)bn << 24);
+    key[1] = reinterpret_cast<uintptr_t>(w_ref);
+    key[2] = C; key[3] = O; key[4] = (uint64_t)n_chunks; key[5] = (uint64_t)n_otiles; key[6] = w_batch;
+}
+
 template <int KH, int KW, int TW, int BN>
 static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
                              size_t H, size_t W, size_t O, size_t pad, size_t w_batch, int64_t bias_sp,
@@ -1414,11 +1423,15 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                 constexpr int NCH = decltype(nch_tag)::value;
                 constexpr size_t lds_need = (size_t)NCH * BN * 256 + 4 * CONV_DB_PLANE + 128 * sizeof(float);
                 static_assert(lds_need <= 160 * 1024 - 512, "LDS budget");
-                _Float16* wres = nullptr;
                 const size_t bytes = (size_t)n_otiles * NCH * BN * 288;
-                if (int rc = workspace_alloc(reinterpret_cast<void**>(&wres), bytes, s)) return rc;
+                uint64_t key[PREPARED_KEY_WORDS];
+                conv_image_key(key, 1, 3, 3, BN, w_ref, C, O, NCH, n_otiles, w_batch);
+                ImageLease lease;
+                if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
+                _Float16* wres = static_cast<_Float16*>(lease.ptr);
                 dim3 pg((unsigned)((BN * 9 + 255) / 256), (unsigned)(n_otiles * NCH));
-                hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles);
+                if (lease.fill)
+                    hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles);
                 IgemmArgs a;
                 a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
                 a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.H_out = (int)H_out; a.W_out = (int)W_out;
@@ -1444,7 +1457,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                     hipError_t e = hipGetLastError();
                     if (e != hipSuccess) rc = set_hip_error(e, "conv3x3_resident_db kernel launch");
                 }
-                int rc2 = workspace_free(wres, s);
+                int rc2 = image_release(lease, s);
                 return rc ? rc : rc2;
             };
             if (n_chunks == 2) return run(std::integral_constant<int, 2>{});
@@ -1460,12 +1473,16 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         static const char* res_env = getenv("NZHIP_CONV_RESIDENT");
         const bool allow = res_env ? atoi(res_env) != 0 : true;
         if (allow && w_batch == 1 && lds_need <= 160 * 1024 - 512) {
-            _Float16* wres = nullptr;
             const size_t bytes = (size_t)n_otiles * n_chunks * W_CHUNK_R;
-            if (int rc = workspace_alloc(reinterpret_cast<void**>(&wres), bytes, s)) return rc;
+            uint64_t key[PREPARED_KEY_WORDS];
+            conv_image_key(key, 2, KH, KW, BN, w_ref, C, O, n_chunks, n_otiles, w_batch);
+            ImageLease lease;
+            if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
+            _Float16* wres = static_cast<_Float16*>(lease.ptr);
             dim3 pg((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)(n_otiles * n_chunks));
-            hipLaunchKernelGGL((conv_weight_image_resident_kernel<KH, KW, BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C,
-                               (int)O, n_chunks, n_otiles);
+            if (lease.fill)
+                hipLaunchKernelGGL((conv_weight_image_resident_kernel<KH, KW, BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C,
+                                   (int)O, n_chunks, n_otiles);
             IgemmArgs a;
             a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
             a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.H_out = (int)H_out; a.W_out = (int)W_out;
@@ -1495,23 +1512,23 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                 hipError_t e = hipGetLastError();
                 if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm_resident kernel launch");
             }
-            int rc2 = workspace_free(wres, s);
+            int rc2 = image_release(lease, s);
             return rc ? rc : rc2;
         }
     }
     const size_t slabs = (size_t)w_batch * n_otiles * n_chunks;
-    _Float16* wimg = nullptr;
-    if (int rc = workspace_alloc(reinterpret_cast<void**>(&wimg), slabs * G::W_BYTES, s)) return rc;
+    if (slabs > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: weight set too large for the fused route");
+    uint64_t key[PREPARED_KEY_WORDS];
+    conv_image_key(key, 3, KH, KW, BN, w_ref, C, O, n_chunks, n_otiles, w_batch);
+    ImageLease lease;
+    if (int rc = image_acquire(PREPARED_CONV_W, key, slabs * G::W_BYTES, s, &lease)) return rc;
+    _Float16* wimg = static_cast<_Float16*>(lease.ptr);
     int rc = NZHIP_OK;
-    {
+    if (lease.fill) {
         // pad bytes of the slabs are never read as data; no need to clear them
         dim3 grid((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)slabs);
-        if (slabs > 65535) {
-            rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: weight set too large for the fused route");
-        } else {
-            hipLaunchKernelGGL((conv_weight_image_kernel<KH, KW, BN>), grid, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O,
-                               n_chunks, n_otiles);
-        }
+        hipLaunchKernelGGL((conv_weight_image_kernel<KH, KW, BN>), grid, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O,
+                           n_chunks, n_otiles);
     }
     if (rc == NZHIP_OK) {
         IgemmArgs a;
@@ -1547,7 +1564,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm kernel launch");
         }
     }
-    int rc2 = workspace_free(wimg, s);
+    int rc2 = image_release(lease, s);
     return rc ? rc : rc2;
 }
 

@@ -1143,10 +1143,44 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mf
     const long b_n = d.b_stride_n ? d.batch_n : 1, b_c = d.b_stride_c ? d.batch_c : 1;
     const size_t a_elems = (size_t)Mp * Kp, b_elems = (size_t)Np * Kp;
     const size_t a_total = a_elems * a_n * a_c, b_total = b_elems * b_n * b_c;
-    _Float16* ws = nullptr;
-    if (int rc = workspace_alloc(reinterpret_cast<void**>(&ws), (a_total + b_total) * sizeof(_Float16), s)) return rc;
-    _Float16* Ah = ws;
-    _Float16* Bh = ws + a_total;
+    // Kernel variants (waves: 0 = choose, 4 / 8 / 2 = force):
+    //   8: 256 x 256 tile, 4 x 2 waves (two per SIMD, 128 accumulators each): the memory instructions of one
+    //      wave issue under the MFMAs of the other (8192^3 with 16x16x32: 1.08 ms against 1.10 ms with 4 waves)
+    //   4: 256 x 256 tile, 2 x 2 waves (one wave per SIMD, 256 accumulators), 4-stage ring, 1 workgroup per CU
+    //   2: 128 x 256 tile, 2 x 2 waves, 3-stage ring of 72 KiB: two workgroups share a CU, so the output
+    //      stores and ring fill of one overlap the MFMAs of the other -- for products with few tiles
+    // mfma: 0 = choose (16), 16 = v_mfma_f32_16x16x32_f16, 32 = v_mfma_f32_32x32x16_f16 (8192^3: 1.10 / 1.13 ms
+    // with 4 waves; the 32x32x16 loop is kept for comparison).
+    static const char* waves_env = getenv("NZHIP_H16_WAVES");
+    if (waves == 0 && waves_env) waves = atoi(waves_env);
+    static const char* mfma_env = getenv("NZHIP_H16_MFMA");             // 16 | 32: benchmarking only
+    if (mfma == 0 && mfma_env) mfma = atoi(mfma_env);
+    const bool mf16 = mfma != 32;
+    if (waves != 2 && waves != 4 && waves != 8) {
+        const long t256 = (Mp / 256) * (Np / 256) * d.batch_n * d.batch_c;
+        waves = t256 < 2 * device_cu_count() ? 2 : (mf16 ? 8 : 4);
+    }
+    const bool half_m = waves == 2;
+    const int wm_waves = waves == 8 ? 4 : 2;
+    const int blk = mf16 ? 16 : 32;                                     // rows per MFMA block
+    const int fr_a = (half_m ? 64 : 256 / wm_waves) / blk, fr_b = 128 / blk;   // blocks per wave tile
+
+    // The image of A comes from the pooled workspace. The image of B may belong to a prepared-operand handle
+    // (nzhip_gemm_prepared_b): its layout does not depend on the kernel variant beyond the MFMA block height, so an
+    // image built by an earlier call with the same operand is used as it is and B's rounding pass is skipped.
+    _Float16* Ah = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&Ah), a_total * sizeof(_Float16), s)) return rc;
+    uint64_t key[PREPARED_KEY_WORDS] = {};
+    key[0] = 4u | ((uint64_t)blk << 8) | ((uint64_t)fr_b << 16) | ((uint64_t)(b_trans ? 1 : 0) << 24);
+    key[1] = reinterpret_cast<uintptr_t>(d.B);
+    key[2] = (uint64_t)d.N; key[3] = (uint64_t)d.K; key[4] = (uint64_t)d.ldb;
+    key[5] = (uint64_t)b_n; key[6] = (uint64_t)b_c; key[7] = (uint64_t)d.b_stride_n; key[8] = (uint64_t)d.b_stride_c;
+    ImageLease b_lease;
+    if (int rc = image_acquire(PREPARED_GEMM_B, key, b_total * sizeof(_Float16), s, &b_lease)) {
+        workspace_free(Ah, s);
+        return rc;
+    }
+    _Float16* Bh = static_cast<_Float16*>(b_lease.ptr);
 
     const int nkt = (int)(Kp / BK);
     auto operand = [&](_Float16* dst, const float* src, long R, long ld, long sc, size_t elems, int fr) {
@@ -1189,33 +1223,12 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mf
         hipError_t e = hipGetLastError();
         return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "fp16 rounding pass launch");
     };
-    // Kernel variants (waves: 0 = choose, 4 / 8 / 2 = force):
-    //   8: 256 x 256 tile, 4 x 2 waves (two per SIMD, 128 accumulators each): the memory instructions of one
-    //      wave issue under the MFMAs of the other (8192^3 with 16x16x32: 1.08 ms against 1.10 ms with 4 waves)
-    //   4: 256 x 256 tile, 2 x 2 waves (one wave per SIMD, 256 accumulators), 4-stage ring, 1 workgroup per CU
-    //   2: 128 x 256 tile, 2 x 2 waves, 3-stage ring of 72 KiB: two workgroups share a CU, so the output
-    //      stores and ring fill of one overlap the MFMAs of the other -- for products with few tiles
-    // mfma: 0 = choose (16), 16 = v_mfma_f32_16x16x32_f16, 32 = v_mfma_f32_32x32x16_f16 (8192^3: 1.10 / 1.13 ms
-    // with 4 waves; the 32x32x16 loop is kept for comparison).
-    static const char* waves_env = getenv("NZHIP_H16_WAVES");
-    if (waves == 0 && waves_env) waves = atoi(waves_env);
-    static const char* mfma_env = getenv("NZHIP_H16_MFMA");             // 16 | 32: benchmarking only
-    if (mfma == 0 && mfma_env) mfma = atoi(mfma_env);
-    const bool mf16 = mfma != 32;
-    if (waves != 2 && waves != 4 && waves != 8) {
-        const long t256 = (Mp / 256) * (Np / 256) * d.batch_n * d.batch_c;
-        waves = t256 < 2 * device_cu_count() ? 2 : (mf16 ? 8 : 4);
-    }
-    const bool half_m = waves == 2;
-    const int wm_waves = waves == 8 ? 4 : 2;
-    const int blk = mf16 ? 16 : 32;                                     // rows per MFMA block
-    const int fr_a = (half_m ? 64 : 256 / wm_waves) / blk, fr_b = 128 / blk;   // blocks per wave tile
     int rc;
-    if (a_n == 1 && b_n == 1 && a_c == b_c && (Mp + Np) / CVT_ROWS <= 65535) {
+    if (b_lease.fill && a_n == 1 && b_n == 1 && a_c == b_c && (Mp + Np) / CVT_ROWS <= 65535) {
         rc = convert_pair(fr_a, fr_b, blk);
     } else {
         rc = convert(Ah, d.A, d.M, Mp, !a_trans, d.lda, a_n, a_c, d.a_stride_n, d.a_stride_c, a_elems, fr_a, blk);
-        if (rc == NZHIP_OK)
+        if (rc == NZHIP_OK && b_lease.fill)
             rc = convert(Bh, d.B, d.N, Np, b_trans, d.ldb, b_n, b_c, d.b_stride_n, d.b_stride_c, b_elems, fr_b, blk);
     }
     if (rc == NZHIP_OK) {
@@ -1265,7 +1278,9 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mf
             if (e != hipSuccess) rc = set_hip_error(e, "gemm_h16 kernel launch");
         }
     }
-    int rc2 = workspace_free(ws, s);
+    int rc2 = workspace_free(Ah, s);
+    const int rc3 = image_release(b_lease, s);
+    if (!rc2) rc2 = rc3;
     return rc ? rc : rc2;
 }
 

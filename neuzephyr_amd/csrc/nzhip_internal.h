@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
+
 #include "../../include/nzhip.h"
 
 namespace nzhip {
@@ -48,6 +50,23 @@ int gemm_thin_dispatch(const nzhip_gemm_desc& d, hipStream_t stream);
 // Stream-ordered workspace from the caching allocator (nzhip_runtime.cpp).
 int workspace_alloc(void** ptr, size_t bytes, hipStream_t stream);
 int workspace_free(void* ptr, hipStream_t stream);
+
+// ---- prepared operand images (nzhip_prepared) -------------------------------------------------------------
+// A kernel route that first turns an operand into an fp16 image (the two-pass GEMM's B image, the conv kernels'
+// weight images) asks image_acquire() for the memory instead of workspace_alloc(). Outside a *_prepared entry
+// point that is a pooled workspace and *fill is always true. Inside one (the calling thread carries the handle),
+// the memory belongs to the handle: when the handle already holds an image built from the same key (operand
+// address, extents, image kind) *fill comes back false and the conversion kernel is skipped.
+// kind: which entry point the site belongs to; a handle is only honoured by sites of the kind it was passed for.
+constexpr int PREPARED_GEMM_B = 1, PREPARED_CONV_W = 2;
+constexpr int PREPARED_KEY_WORDS = 12;
+struct ImageLease {
+    void* ptr = nullptr;
+    bool fill = true;           // the caller must (re)build the image
+    bool persistent = false;    // owned by a handle: image_release leaves it alone
+};
+int image_acquire(int kind, const uint64_t key[PREPARED_KEY_WORDS], size_t bytes, hipStream_t s, ImageLease* out);
+int image_release(const ImageLease& lease, hipStream_t s);
 
 // Compute units of the current device (queried once per device, then cached).
 int device_cu_count();

@@ -13,6 +13,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <new>
 #include <utility>
 
 #include "nz_pool_allocator.hpp"
@@ -133,6 +134,68 @@ int workspace_free(void* ptr, hipStream_t s) {
     return Runtime::instance().pool().free_async(ptr, reinterpret_cast<uintptr_t>(s)) == 0
                ? NZHIP_OK
                : set_error(NZHIP_E_INVALID, "workspace_free: unknown pointer");
+}
+
+// ---- prepared operand images ----------------------------------------------------------------------------------
+}  // namespace nzhip
+
+struct nzhip_prepared {
+    std::mutex mu;
+    void* image = nullptr;
+    size_t bytes = 0;
+    bool valid = false;
+    uint64_t key[nzhip::PREPARED_KEY_WORDS] = {};
+    uintptr_t stream_tag = 0;                       // pool tag the image was allocated under
+    unsigned long long fills = 0;                   // how often an image was (re)built through this handle
+};
+
+namespace nzhip {
+
+struct PreparedScope {
+    nzhip_prepared* handle = nullptr;
+    int kind = 0;
+};
+static thread_local PreparedScope t_prepared;
+
+int image_acquire(int kind, const uint64_t key[PREPARED_KEY_WORDS], size_t bytes, hipStream_t s, ImageLease* out) {
+    nzhip_prepared* h = (t_prepared.handle && t_prepared.kind == kind && !t_arena.active) ? t_prepared.handle : nullptr;
+    if (!h) {
+        out->fill = true;
+        out->persistent = false;
+        return workspace_alloc(&out->ptr, bytes, s);
+    }
+    std::lock_guard<std::mutex> lock(h->mu);
+    out->persistent = true;
+    if (h->valid && h->bytes == bytes && memcmp(h->key, key, sizeof(h->key)) == 0) {
+        out->ptr = h->image;
+        out->fill = false;
+        return NZHIP_OK;
+    }
+    if (h->image && h->bytes != bytes) {            // another operand or another route: start over
+        Runtime::instance().pool().free_async(h->image, h->stream_tag);
+        h->image = nullptr;
+    }
+    if (!h->image) {
+        const int rc = Runtime::instance().pool().allocate(&h->image, bytes, reinterpret_cast<uintptr_t>(s));
+        if (rc != 0) {
+            h->image = nullptr;
+            h->valid = false;
+            return set_error(NZHIP_E_NOMEM, "prepared image of %zu bytes: allocation failed (hipError_t %d)", bytes, rc);
+        }
+        h->stream_tag = reinterpret_cast<uintptr_t>(s);
+    }
+    h->bytes = bytes;
+    memcpy(h->key, key, sizeof(h->key));
+    h->valid = true;
+    h->fills++;
+    out->ptr = h->image;
+    out->fill = true;
+    return NZHIP_OK;
+}
+
+int image_release(const ImageLease& lease, hipStream_t s) {
+    if (lease.persistent || !lease.ptr) return NZHIP_OK;
+    return workspace_free(lease.ptr, s);
 }
 
 int device_cu_count() {
@@ -296,6 +359,56 @@ int nzhip_sync_all(void) {
     hipError_t e = hipDeviceSynchronize();
     if (e != hipSuccess) return set_hip_error(e, "hipDeviceSynchronize");
     return gemm_h16_coop_check(nullptr, true);
+}
+
+int nzhip_prepared_create(nzhip_prepared** handle) {
+    if (!handle) return set_error(NZHIP_E_INVALID, "nzhip_prepared_create: null pointer");
+    *handle = new (std::nothrow) nzhip_prepared();
+    return *handle ? NZHIP_OK : set_error(NZHIP_E_NOMEM, "nzhip_prepared_create: out of host memory");
+}
+
+int nzhip_prepared_invalidate(nzhip_prepared* handle) {
+    if (!handle) return set_error(NZHIP_E_INVALID, "nzhip_prepared_invalidate: null handle");
+    std::lock_guard<std::mutex> lock(handle->mu);
+    handle->valid = false;
+    return NZHIP_OK;
+}
+
+int nzhip_prepared_fills(const nzhip_prepared* handle, unsigned long long* count) {
+    if (!handle || !count) return set_error(NZHIP_E_INVALID, "nzhip_prepared_fills: null argument");
+    std::lock_guard<std::mutex> lock(const_cast<nzhip_prepared*>(handle)->mu);
+    *count = handle->fills;
+    return NZHIP_OK;
+}
+
+int nzhip_prepared_destroy(nzhip_prepared* handle) {
+    if (!handle) return NZHIP_OK;
+    int rc = NZHIP_OK;
+    if (handle->image && Runtime::instance().pool().free_async(handle->image, handle->stream_tag) != 0)
+        rc = set_error(NZHIP_E_INVALID, "nzhip_prepared_destroy: the image is not a pool allocation");
+    delete handle;
+    return rc;
+}
+
+int nzhip_gemm_prepared_b(const nzhip_gemm_desc* desc, nzhip_prepared* b_image, void* stream) {
+    if (!b_image) return nzhip_gemm(desc, stream);
+    t_prepared.handle = b_image;
+    t_prepared.kind = PREPARED_GEMM_B;
+    const int rc = nzhip_gemm(desc, stream);
+    t_prepared = PreparedScope();
+    return rc;
+}
+
+int nzhip_conv2d_forward_prepared(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C, size_t H,
+                                  size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t w_batch,
+                                  int64_t bias_stride_pixel, int64_t bias_stride_channel, int activation,
+                                  nzhip_prepared* w_image, void* stream) {
+    t_prepared.handle = w_image;
+    t_prepared.kind = PREPARED_CONV_W;
+    const int rc = nzhip_conv2d_forward(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
+                                        bias_stride_channel, activation, stream);
+    t_prepared = PreparedScope();
+    return rc;
 }
 
 int nzhip_gemm_static(const nzhip_gemm_desc* desc, void* stream) {

@@ -1,0 +1,89 @@
+// Forward passes of single layers through the nz:: API (Model::forward()), timed on the host around a device
+// synchronisation: Linear 4096 x 1024 -> 4096 + ReLU, and Conv2d 16 x 64 x 128 x 128 -> 128 (3x3, stride 1, pad 1)
+// + ReLU with the reference's parameters (one weight copy per sample, per-pixel bias; src/Model.cu:244-263).
+// Each layer twice: weights untouched between the passes (the fused layers keep the fp16 image of their weights),
+// and weights rewritten before every pass (the image is rebuilt every time). Prints one JSON line.
+//   layer_bench [steps] [warmup]
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <vector>
+
+#include "NeuZephyr/Model.cuh"
+#include "nzhip.h"
+
+using namespace nz::nodes;
+using namespace nz::nodes::io;
+
+struct LinearLayer : nz::Model {
+    InputNode input;
+    LinearLayer(size_t batch, size_t in, size_t out) : input({batch, 1, in, 1}) { defaultOutput(ReLU(Linear(&input, out))); }
+};
+
+struct ConvLayer : nz::Model {
+    InputNode input;
+    ConvLayer(size_t n, size_t c, size_t h, size_t w, size_t o) : input({n, c, h, w}) {
+        defaultOutput(ReLU(Conv2d(&input, o, 3, 3, 1, 1)));
+    }
+};
+
+template <typename M>
+static void fill(M& model, std::mt19937& gen, float scale) {
+    std::uniform_real_distribution<float> u(-1.f, 1.f);
+    std::vector<float> x(model.input.output->size());
+    for (auto& v : x) v = u(gen);
+    model.input.dataInject(x.begin(), x.end());
+    for (auto* p : model.parameters()) {
+        std::vector<float> v(p->output->size());
+        for (auto& e : v) e = u(gen) * scale;
+        p->dataInject(v.begin(), v.end());
+    }
+}
+
+template <typename M>
+static double timeForward(M& model, int steps, int warmup, bool touchWeights) {
+    auto pass = [&] {
+        if (touchWeights) (void)model.parameters()[0]->output->data();     // a writable pointer was handed out
+        model.forward();
+    };
+    for (int i = 0; i < warmup; ++i) pass();
+    nzhip_sync_all();
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; ++i) pass();
+    nzhip_sync_all();
+    return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
+}
+
+int main(int argc, char** argv) {
+    const int steps = argc > 1 ? atoi(argv[1]) : 200, warmup = argc > 2 ? atoi(argv[2]) : 20;
+    try {
+        std::mt19937 gen(11);
+        double linKept, linRebuilt, convKept, convRebuilt;
+        unsigned long long linBuilds, convBuilds;
+        {
+            LinearLayer m(4096, 1024, 4096);
+            fill(m, gen, 0.0765f);
+            linKept = timeForward(m, steps, warmup, false);
+            linBuilds = m.graph().weightImageBuilds();
+            linRebuilt = timeForward(m, steps, warmup, true);
+        }
+        {
+            ConvLayer m(16, 64, 128, 128, 128);
+            fill(m, gen, 0.06f);
+            convKept = timeForward(m, steps, warmup, false);
+            convBuilds = m.graph().weightImageBuilds();
+            convRebuilt = timeForward(m, steps, warmup, true);
+        }
+        printf("{\"workload\": \"single layers through nz::Model::forward(), host wall clock per pass\", \"steps\": %d, \"warmup\": %d, "
+               "\"linear_4096x1024_to_4096_relu\": {\"ms_weight_image_kept\": %.4f, \"ms_weight_image_rebuilt_every_pass\": %.4f, "
+               "\"image_builds_in_kept_loop\": %llu}, "
+               "\"conv2d_16x64x128x128_to_128_relu_per_sample_weights_per_pixel_bias\": {\"ms_weight_image_kept\": %.4f, "
+               "\"ms_weight_image_rebuilt_every_pass\": %.4f, \"image_builds_in_kept_loop\": %llu}}\n",
+               steps, warmup, linKept, linRebuilt, linBuilds, convKept, convRebuilt, convBuilds);
+    } catch (const std::exception& e) {
+        fprintf(stderr, "layer_bench: %s\n", e.what());
+        return 1;
+    }
+    return 0;
+}

@@ -7,12 +7,14 @@
 #ifndef NZ_COMPUTE_GRAPH_CUH
 #define NZ_COMPUTE_GRAPH_CUH
 #include <functional>
+#include <memory>
 #include <iosfwd>
 #include <string>
 #include <vector>
 
 #include "Nodes.cuh"
 #include "Optimizer.cuh"
+#include "TensorOperations.cuh"
 #include "dl_export.cuh"
 
 namespace nz::graph {
@@ -41,6 +43,9 @@ namespace nz::graph {
         [[nodiscard]] io::OutputNode* getOutputNode() const;   // throws std::runtime_error without exactly one output
         void setFusion(bool enabled);
         [[nodiscard]] size_t fusedGroupCount() const { return fusedGroups; }
+        // how often the fused layers have built the fp16 image of their weights so far (once per layer while the
+        // weights stay untouched, again after every change)
+        [[nodiscard]] unsigned long long weightImageBuilds() const;
         [[nodiscard]] const std::vector<Node*>& getNodes() const { return nodes; }
 
     private:
@@ -56,6 +61,7 @@ namespace nz::graph {
         bool fusion = true;
         bool planned = false;
         size_t fusedGroups = 0;
+        std::vector<std::shared_ptr<PreparedOperand>> weightImages;   // one per fused layer of the current plan
     };
 }
 #endif

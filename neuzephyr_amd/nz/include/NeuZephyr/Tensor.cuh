@@ -45,6 +45,12 @@ namespace nz::data {
         void setRequiresGrad(bool requires_grad);
 
         [[nodiscard]] value_type* data() const;                    // device pointer (allocates on first use)
+        // The same pointer for a caller that only reads. data() hands out a writable pointer and therefore counts
+        // as a possible write: version() goes up with every data() call (and so with every member that writes),
+        // never with constData(). Whoever keeps something derived from the contents (the fused layers keep the
+        // fp16 image of their weights between forward passes) compares version() to know whether it is still good.
+        [[nodiscard]] const value_type* constData() const;
+        [[nodiscard]] unsigned long long version() const noexcept { return _version; }
         [[nodiscard]] value_type* grad() const;                    // throws std::runtime_error without gradients
         // the same buffer for a caller that is about to write EVERY element of it (contents undefined on return)
         [[nodiscard]] value_type* gradOverwrite() const;
@@ -90,6 +96,7 @@ namespace nz::data {
         // zeroGrad() only notes that the gradient is zero; the clear runs when somebody reads or adds to it
         // (grad()) and is skipped when the next user overwrites every element (gradOverwrite())
         mutable bool _gradZeroPending = false;
+        mutable unsigned long long _version = 0;
         bool _requires_grad;
     };
 }

@@ -78,6 +78,7 @@ namespace nz::graph {
     void ComputeGraph::buildPlan() {
         plan.clear();
         fusedGroups = 0;
+        weightImages.clear();
         std::unordered_map<Node*, std::vector<Node*>> consumers;
         for (Node* node : nodes)
             for (Node* input : node->inputs) consumers[input].push_back(node);
@@ -192,11 +193,21 @@ namespace nz::graph {
                                                     i2c->kernelHeight, i2c->kernelWidth, i2c->stride, i2c->padding, ws[0]);
                         };
                     }
+                    // The fp16 image of the weights survives between forward passes while nobody has asked the
+                    // weight tensor for a writable pointer (Tensor::version()).
+                    auto image = std::make_shared<PreparedOperand>();
+                    weightImages.push_back(image);
+                    auto seen = std::make_shared<unsigned long long>(~0ull);
                     addGroup(std::move(members), [=] {
-                        iConv2dForward(last->output->data(), x->output->data(), rhs->output->data(),
+                        const float* w = rhs->output->constData();
+                        if (rhs->output->version() != *seen) {
+                            image->invalidate();
+                            *seen = rhs->output->version();
+                        }
+                        iConv2dForward(last->output->data(), x->output->data(), w,
                                        biasNode ? biasNode->output->data() : nullptr, xs[0], xs[1], xs[2], xs[3], O,
                                        i2c->kernelHeight, i2c->kernelWidth, i2c->stride, i2c->padding, ws[0],
-                                       static_cast<long long>(O), 1, relu);
+                                       static_cast<long long>(O), 1, relu, image.get());
                     }, std::move(back));
                     continue;
                 }
@@ -238,9 +249,17 @@ namespace nz::graph {
                                             lhs->output->data(), rhs->output->data(), dZ, lhs->output->shape(),
                                             rhs->output->shape(), mm->output->shape());
                     };
+                    auto image = std::make_shared<PreparedOperand>();
+                    weightImages.push_back(image);
+                    auto seen = std::make_shared<unsigned long long>(~0ull);
                     addGroup(std::move(members), [=] {
-                        iLinearForward(last->output->data(), rhs->output->data(), lhs->output->data(),
-                                       biasNode->output->data(), batch, in, out, relu);
+                        const float* w = lhs->output->constData();
+                        if (lhs->output->version() != *seen) {
+                            image->invalidate();
+                            *seen = lhs->output->version();
+                        }
+                        iLinearForward(last->output->data(), rhs->output->data(), w, biasNode->output->data(), batch, in, out,
+                                       relu, image.get());
                     }, std::move(back));
                 }
             }
@@ -314,6 +333,12 @@ namespace nz::graph {
             if (node->inputs.empty()) optimizer->step(node);
             else optimizer->skip(node);
         }
+    }
+
+    unsigned long long ComputeGraph::weightImageBuilds() const {
+        unsigned long long n = 0;
+        for (const auto& image : weightImages) n += image->fills();
+        return n;
     }
 
     void ComputeGraph::zeroGrad() const {

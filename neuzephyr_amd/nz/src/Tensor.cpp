@@ -114,6 +114,12 @@ namespace nz::data {
 
     Tensor::value_type* Tensor::data() const {
         if (!_data && _size) _data = deviceAlloc(_size);
+        ++_version;
+        return _data;
+    }
+
+    const Tensor::value_type* Tensor::constData() const {
+        if (!_data && _size) _data = deviceAlloc(_size);
         return _data;
     }
 

@@ -179,12 +179,30 @@ namespace nz::data {
         NZ_CHECK(nzhip_compress(out, in, n, batches, nzhip_default_stream()));
     }
 
-    void iConv2dForward(float* y, float* x, float* w, float* bias, const size_t N, const size_t C, const size_t H,
+    PreparedOperand::PreparedOperand() {
+        nzhip_prepared* p = nullptr;
+        NZ_CHECK(nzhip_prepared_create(&p));
+        h = p;
+    }
+
+    PreparedOperand::~PreparedOperand() { nzhip_prepared_destroy(static_cast<nzhip_prepared*>(h)); }
+
+    void PreparedOperand::invalidate() const { NZ_CHECK(nzhip_prepared_invalidate(static_cast<nzhip_prepared*>(h))); }
+
+    unsigned long long PreparedOperand::fills() const {
+        unsigned long long n = 0;
+        NZ_CHECK(nzhip_prepared_fills(static_cast<const nzhip_prepared*>(h), &n));
+        return n;
+    }
+
+    void iConv2dForward(float* y, float* x, const float* w, float* bias, const size_t N, const size_t C, const size_t H,
                         const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
                         const size_t pad, const size_t weightBatch, const long long biasPixelStride,
-                        const long long biasChannelStride, const bool relu) {
-        NZ_CHECK(nzhip_conv2d_forward(y, x, w, bias, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch, biasPixelStride,
-                                      biasChannelStride, relu ? NZHIP_ACT_RELU : NZHIP_ACT_NONE, nzhip_default_stream()));
+                        const long long biasChannelStride, const bool relu, const PreparedOperand* weightImage) {
+        NZ_CHECK(nzhip_conv2d_forward_prepared(y, x, w, bias, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch, biasPixelStride,
+                                               biasChannelStride, relu ? NZHIP_ACT_RELU : NZHIP_ACT_NONE,
+                                               weightImage ? static_cast<nzhip_prepared*>(weightImage->handle()) : nullptr,
+                                               nzhip_default_stream()));
     }
 
     bool iConv2dBackwardData(float* dx, float* dy, float* w, const size_t N, const size_t C, const size_t H,
@@ -208,8 +226,8 @@ namespace nz::data {
         return true;
     }
 
-    void iLinearForward(float* y, float* x, float* wOutIn, float* bias, const size_t batch, const size_t in,
-                        const size_t out, const bool relu) {
+    void iLinearForward(float* y, float* x, const float* wOutIn, float* bias, const size_t batch, const size_t in,
+                        const size_t out, const bool relu, const PreparedOperand* weightImage) {
         nzhip_gemm_desc d = {};
         d.A = x;
         d.B = wOutIn;
@@ -227,6 +245,7 @@ namespace nz::data {
         d.bias_stride_row = 0;
         d.bias_stride_col = 1;
         d.activation = relu ? NZHIP_ACT_RELU : NZHIP_ACT_NONE;
-        NZ_CHECK(nzhip_gemm(&d, nzhip_default_stream()));
+        NZ_CHECK(nzhip_gemm_prepared_b(&d, weightImage ? static_cast<nzhip_prepared*>(weightImage->handle()) : nullptr,
+                                       nzhip_default_stream()));
     }
 }

@@ -678,6 +678,54 @@ TEST(Model, LinearFusedBackwardEqualsNodeChain) {
     }
 }
 
+// ---- weight images kept between forward passes ------------------------------------------------------------
+TEST(Model, WeightImagesAreKeptWhileWeightsStayUntouchedAndRebuiltAfterAChange) {
+    // Linear at a size that takes the two-pass route (the fp16 image of W is its B operand), and a Conv2d on the
+    // implicit-GEMM kernels: three forward passes build each image once and give the same values; new weights
+    // (dataInject, an optimizer step) are seen by the very next forward pass, which must equal the unfused graph.
+    {
+        const size_t batch = 4096, in = 1024, out = 4096;
+        LinearModel m(batch, in, out, true);
+        auto x = randomVec(batch * in, 11, -1.f, 1.f), W = randomVec(out * in, 12, -0.08f, 0.08f), b = randomVec(out, 13, -0.03f, 0.03f);
+        m.input.dataInject(x.begin(), x.end());
+        m.parameters()[0]->dataInject(W.begin(), W.end());
+        m.parameters()[1]->dataInject(b.begin(), b.end());
+        const auto first = m.forward().hostData();
+        EXPECT_EQ(m.graph().weightImageBuilds(), 1ull);
+        EXPECT_TRUE(m.forward().hostData() == first);
+        EXPECT_TRUE(m.forward().hostData() == first);
+        EXPECT_EQ(m.graph().weightImageBuilds(), 1ull);
+        auto W2 = randomVec(out * in, 14, -0.08f, 0.08f);
+        m.parameters()[0]->dataInject(W2.begin(), W2.end());
+        const auto second = m.forward().hostData();
+        EXPECT_EQ(m.graph().weightImageBuilds(), 2ull);
+        EXPECT_TRUE(second != first);
+        m.graph().setFusion(false);
+        EXPECT_TRUE(closeTo(m.forward().hostData(), std::vector<double>(second.begin(), second.end()), 1e-5));
+    }
+    {
+        ConvModel m(8, 16, 64, 64, 32, 3, 1, 1, true);           // enough patches for the implicit-GEMM kernel
+        auto x = randomVec(8 * 16 * 64 * 64, 21, -1.f, 1.f);
+        m.input.dataInject(x.begin(), x.end());
+        auto W = randomVec(8 * 16 * 9 * 32, 22, -0.2f, 0.2f), b = randomVec(64 * 64 * 32, 23, -0.1f, 0.3f);
+        m.parameters()[0]->dataInject(W.begin(), W.end());
+        m.parameters()[1]->dataInject(b.begin(), b.end());
+        const auto first = m.forward().hostData();
+        EXPECT_EQ(m.graph().fusedGroupCount(), 1u);
+        EXPECT_EQ(m.graph().weightImageBuilds(), 1ull);
+        EXPECT_TRUE(m.forward().hostData() == first);
+        EXPECT_EQ(m.graph().weightImageBuilds(), 1ull);
+        m.backward();
+        nz::opt::SGD optimizer(0.05f);
+        m.update(&optimizer);
+        const auto second = m.forward().hostData();
+        EXPECT_EQ(m.graph().weightImageBuilds(), 2ull);
+        EXPECT_TRUE(second != first);
+        m.graph().setFusion(false);
+        EXPECT_TRUE(closeTo(m.forward().hostData(), std::vector<double>(second.begin(), second.end()), 1e-5));
+    }
+}
+
 // ---- fp32 matmul and optimizers (test/Test.cpp:119-184, 2230-2265, 2398-2452, 2816-2878) ------------
 TEST(TensorBasic, TensorMultiplicationTest) {
     Tensor tensor1({2, 1, 2, 3});
