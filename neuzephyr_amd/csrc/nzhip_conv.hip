@@ -2238,6 +2238,167 @@ static int conv1x1_backward_weights(float* dw, const float* x, const float* dy, 
     return rc ? rc : rc2;
 }
 
+// ---- weight gradient for any kernel extent, stride and padding ---------------------------------------------------
+// dW[(c, r, s)][o] = sum over pixels of f16(x[c][ho*stride - pad + r][wo*stride - pad + s]) * f16(dy[o][ho][wo]): a product
+// whose contraction runs over the output pixels, with the column matrix of the reference's chain (Img2ColNode::forward,
+// src/Nodes.cu:605-630, as A of MatMulNode::backward's dB += A^T dC, :169-182) gathered from LDS instead of written to
+// memory. A workgroup owns up to 128 (channel, tap) rows (as many whole channels as fit) x 64 output channels and a band
+// of output rows of one image; per output row and per segment of 128 pixels it stages the K_h input rows of its channels
+// (the 127 * stride + K_w columns the segment touches, zero outside the image) and the dy segment in LDS as fp16, then
+// runs eight 32x32x16 MFMA steps per wave. The A fragment of a lane is eight pixels of one (c, r, s) row, `stride`
+// elements apart in the staged input row: eight 16-bit LDS reads, which is what makes every tap offset and stride
+// one code path. Band sums go to a workspace and are added in ascending order by conv_dwg_reduce_kernel.
+constexpr int DWG_PX = 128, DWG_OT = 64, DWG_ROWS = 128, DWG_ZPITCH = DWG_PX + 8;
+
+struct ConvDwGenArgs {
+    const float* x;        // [N, C, H, W]
+    const float* dy;       // [N, O, Ho, Wo]
+    float* partial;        // [chunk][o_tile][image][band][DWG_ROWS][DWG_OT]
+    int C, H, W, O, Ho, Wo, Kh, Kw, stride, pad;
+    int cc;                // channels per workgroup
+    int pw;                // staged columns per input row: (DWG_PX - 1) * stride + Kw, rounded up to an odd count
+    int bands, band_rows, n_images;
+};
+
+__global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    _Float16* xs = reinterpret_cast<_Float16*>(lds);                                   // [cc * Kh][pw]
+    _Float16* zs = xs + ((p.cc * p.Kh * p.pw + 7) & ~7);                                // [DWG_OT][DWG_ZPITCH]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const int band = blockIdx.x % p.bands, img = blockIdx.x / p.bands;
+    const int c0 = blockIdx.y * p.cc, o0 = blockIdx.z * DWG_OT;
+    const int taps = p.Kh * p.Kw;
+    const int nch = (p.C - c0) < p.cc ? (p.C - c0) : p.cc;
+    const int h_begin = band * p.band_rows;
+    const int h_end = (h_begin + p.band_rows) < p.Ho ? (h_begin + p.band_rows) : p.Ho;
+    const float* ximg = p.x + ((long)img * p.C + c0) * p.H * p.W;
+    const float* zimg = p.dy + ((long)img * p.O + o0) * p.Ho * p.Wo;
+
+    floatx16 acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+
+    // this lane's row of the tile: (channel, tap row, tap column); rows past the last channel multiply zeros
+    const int m = wave * 32 + li;
+    const bool row_live = m < nch * taps;
+    const int mc = row_live ? m / taps : 0, mt = row_live ? m % taps : 0;
+    const int a_base = (mc * p.Kh + mt / p.Kw) * p.pw + mt % p.Kw + 8 * lh * p.stride;
+    const int rows_staged = nch * p.Kh, n_stage = rows_staged * p.pw;
+    const int segs = (p.Wo + DWG_PX - 1) / DWG_PX;
+
+    for (int ho = h_begin; ho < h_end; ho++) {
+        for (int seg = 0; seg < segs; seg++) {
+            const int wo0 = seg * DWG_PX;
+            const int w_first = wo0 * p.stride - p.pad;                       // image column of staged column 0
+            for (int e = tid; e < n_stage; e += 256) {
+                const int row = e / p.pw, col = e - row * p.pw;
+                const int c = row / p.Kh, r = row - c * p.Kh;
+                const int h = ho * p.stride - p.pad + r, w = w_first + col;
+                const bool in = h >= 0 && h < p.H && w >= 0 && w < p.W;
+                const float v = ximg[((long)c * p.H + (in ? h : 0)) * p.W + (in ? w : 0)];
+                xs[e] = (_Float16)(in ? v : 0.f);
+            }
+            for (int e = tid; e < DWG_OT * DWG_PX; e += 256) {
+                const int o = e / DWG_PX, k = e % DWG_PX;
+                const bool in = o0 + o < p.O && wo0 + k < p.Wo;
+                const float v = zimg[((long)(in ? o : 0) * p.Ho + ho) * p.Wo + (in ? wo0 + k : 0)];
+                zs[o * DWG_ZPITCH + k] = (_Float16)(in ? v : 0.f);
+            }
+            __syncthreads();
+#pragma unroll 2
+            for (int ks = 0; ks < DWG_PX / 16; ks++) {
+                half8_t af;
+                const _Float16* ap = xs + a_base + ks * 16 * p.stride;
+#pragma unroll
+                for (int j = 0; j < 8; j++) af[j] = row_live ? ap[j * p.stride] : (_Float16)0.f;
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const half8_t bf = *reinterpret_cast<const half8_t*>(zs + (j * 32 + li) * DWG_ZPITCH + ks * 16 + lh * 8);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc[j], 0, 0, 0);
+                }
+            }
+            __syncthreads();
+        }
+    }
+    // accumulator (block j, register r): row 32 wave + (r >> 2) * 8 + lh * 4 + (r & 3), column 32 j + li
+    float* out = p.partial + ((((long)blockIdx.y * gridDim.z + blockIdx.z) * p.n_images + img) * p.bands + band) * (DWG_ROWS * DWG_OT);
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int row = wave * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+            out[row * DWG_OT + j * 32 + li] = acc[j][r];
+        }
+}
+
+// dW[b][(c0 + c) * taps + t][o0 + o] += the S partial regions of weight copy b, in ascending order (per-sample weights:
+// the bands of image b; shared weights: images x bands).
+__global__ __launch_bounds__(256) void conv_dwg_reduce_kernel(float* __restrict__ dW, const float* __restrict__ P, int S, int C, int O,
+                                                              int taps, int cc, int n_otiles, long group_stride_P, long group_stride_dW) {
+    const int chunk = blockIdx.y / n_otiles, ot = blockIdx.y % n_otiles, b = blockIdx.z;
+    const int c0 = chunk * cc, o0 = ot * DWG_OT;
+    const int nch = (C - c0) < cc ? (C - c0) : cc;
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    const int row = t / DWG_OT, col = t % DWG_OT;
+    if (row >= nch * taps || o0 + col >= O) return;
+    const float* src = P + (long)blockIdx.y * gridDim.z * group_stride_P + (long)b * group_stride_P + t;
+    float sum = 0.f;
+    for (int s = 0; s < S; s++) sum += src[(long)s * (DWG_ROWS * DWG_OT)];
+    dW[(long)b * group_stride_dW + ((long)c0 * taps + row) * O + o0 + col] += sum;
+}
+
+static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W, size_t O,
+                           size_t K_h, size_t K_w, size_t stride, size_t pad, bool shared, hipStream_t s) {
+    const size_t taps = K_h * K_w;
+    const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
+    int cc = (int)(DWG_ROWS / taps);
+    if (cc > (int)C) cc = (int)C;
+    int pw = (int)((DWG_PX - 1) * stride + K_w) | 1;                 // odd: consecutive staged rows start on different banks
+    // staged input rows + dy segment must fit the 64 KiB a workgroup may take without crowding out its neighbours
+    while (cc > 1 && ((size_t)cc * K_h * pw + 8) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2 > 64 * 1024) cc--;
+    const size_t lds_bytes = (((size_t)cc * K_h * pw + 7) & ~(size_t)7) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2;
+    if (lds_bytes > 64 * 1024) return NZHIP_E_UNSUPPORTED;
+    const int chunks = (int)((C + cc - 1) / cc), otiles = (int)((O + DWG_OT - 1) / DWG_OT);
+    if (chunks > 65535 || otiles > 65535) return NZHIP_E_UNSUPPORTED;
+    // about four workgroups per CU in total; a band is a whole number of output rows of one image
+    const long units = (long)chunks * otiles * (long)N;
+    long want = (4L * device_cu_count() + units - 1) / units;
+    if (want < 1) want = 1;
+    if (want > (long)Ho) want = (long)Ho;
+    const int band_rows = (int)((Ho + want - 1) / want), bands = (int)((Ho + band_rows - 1) / band_rows);
+    if (N * (size_t)bands > 0x7fffffffull) return NZHIP_E_UNSUPPORTED;
+    const size_t regions = (size_t)chunks * otiles * N * bands;
+    float* partial = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), regions * DWG_ROWS * DWG_OT * sizeof(float), s)) return rc;
+    ConvDwGenArgs a;
+    a.x = x; a.dy = dy; a.partial = partial;
+    a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.Ho = (int)Ho; a.Wo = (int)Wo;
+    a.Kh = (int)K_h; a.Kw = (int)K_w; a.stride = (int)stride; a.pad = (int)pad;
+    a.cc = cc; a.pw = pw; a.bands = bands; a.band_rows = band_rows; a.n_images = (int)N;
+    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(conv_dwg_kernel), (int)lds_bytes, "hipFuncSetAttribute(conv_dwg)");
+    if (rc == NZHIP_OK) {
+        hipLaunchKernelGGL(conv_dwg_kernel, dim3((unsigned)(N * bands), (unsigned)chunks, (unsigned)otiles), dim3(256), lds_bytes, s, a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg kernel launch");
+    }
+    if (rc == NZHIP_OK) {
+        const int S = shared ? (int)(N * bands) : bands, groups = shared ? 1 : (int)N;
+        const long per_group = (long)S * DWG_ROWS * DWG_OT;
+        // partial regions of one (chunk, o_tile) are contiguous: [image][band]; a weight copy's regions start at b * S
+        dim3 grid((unsigned)((DWG_ROWS * DWG_OT + 255) / 256), (unsigned)(chunks * otiles), (unsigned)groups);
+        hipLaunchKernelGGL(conv_dwg_reduce_kernel, grid, dim3(256), 0, s, dw, partial, S, (int)C, (int)O, (int)taps, cc, otiles,
+                           per_group, (long)(C * taps * O));
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg_reduce kernel launch");
+    }
+    const int rc2 = workspace_free(partial, s);
+    return rc ? rc : rc2;
+}
+
 /* Gradient of nzhip_conv2d_forward with respect to the weights, without the column matrix the reference's
  * chain needs (Img2ColNode::forward output as A in MatMulNode::backward, dB += A^T * dC, src/Nodes.cu:169-182):
  *   dW[wb][(c, r, s)][o] += sum over h, w (and over n when the weights are shared) of
@@ -2252,10 +2413,24 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
         if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
         return conv1x1_backward_weights(dw, x, dy, N, C, H * W, O, w_batch == 1, reinterpret_cast<hipStream_t>(stream));
     }
-    if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1 || H == 0 || W == 0 || H > 0x3fffffff || W > 0x3fffffff ||
-        C > 0x3fffffff || O > 0x3fffffff || N > 65535)
-        return set_error(NZHIP_E_UNSUPPORTED,
-                         "nzhip_conv2d_backward_weights: only 3x3, stride 1, pad 1 and 1x1, stride 1, pad 0 (use the column-matrix chain)");
+    if (stride == 0 || K_h == 0 || K_w == 0) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_weights: zero stride or kernel extent");
+    if (H + 2 * pad < K_h || W + 2 * pad < K_w)
+        return set_error(NZHIP_E_SHAPE, "nzhip_conv2d_backward_weights: kernel larger than the padded input");
+    if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1) {
+        // any other geometry: the gather kernel (up to 128 taps, stride up to 4, extents that fit its index arithmetic)
+        const bool fits = K_h * K_w <= (size_t)DWG_ROWS && stride <= 4 && pad < 0x10000 && H < 0x3fffffff && W < 0x3fffffff &&
+                          C < 0x3fffffff && O < 0x3fffffff && N <= 65535 && H * W < 0x3fffffffull;
+        if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
+        const int rc = fits ? conv_dw_generic(dw, x, dy, N, C, H, W, O, K_h, K_w, stride, pad, w_batch == 1,
+                                              reinterpret_cast<hipStream_t>(stream))
+                            : NZHIP_E_UNSUPPORTED;
+        if (rc == NZHIP_E_UNSUPPORTED)
+            return set_error(NZHIP_E_UNSUPPORTED,
+                             "nzhip_conv2d_backward_weights: more than 128 taps, a stride above 4 or extents beyond the fused kernels (use the column-matrix chain)");
+        return rc;
+    }
+    if (H == 0 || W == 0 || H > 0x3fffffff || W > 0x3fffffff || C > 0x3fffffff || O > 0x3fffffff || N > 65535)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_weights: extents beyond the fused kernels (use the column-matrix chain)");
     const bool vec = W % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
     if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);

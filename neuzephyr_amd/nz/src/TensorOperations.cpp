@@ -217,8 +217,6 @@ namespace nz::data {
     bool iConv2dBackwardWeights(float* dw, float* x, float* dy, const size_t N, const size_t C, const size_t H,
                                 const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
                                 const size_t pad, const size_t weightBatch) {
-        const bool three = K_h == 3 && K_w == 3 && stride == 1 && pad == 1, one = K_h == 1 && K_w == 1 && stride == 1 && pad == 0;
-        if (!three && !one) return false;
         const int rc = nzhip_conv2d_backward_weights(dw, x, dy, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch,
                                                      nzhip_default_stream());
         if (rc == NZHIP_E_UNSUPPORTED) return false;      // extents beyond the fused kernel: the caller takes the column-matrix route

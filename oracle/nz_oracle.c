@@ -435,14 +435,15 @@ void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, si
     free(wr);
 }
 
-/* Weight gradient of the Model::Conv2d graph in one statement (stride 1): MatMulNode::backward's
+/* Weight gradient of the Model::Conv2d graph in one statement: MatMulNode::backward's
  * dB += A^T * dC (src/Nodes.cu:169-182) with A the column matrix of Img2ColNode::forward (:605-630,
- * img2colKernel src/OperationKernels.cu:1308-1328) and dC the pixel-major gradient of
- * Col2ImgNode::backward (:660-665); fp16-rounded operands, fp32 accumulation over the pixels in
- * ascending order (and over the images, for shared weights). */
-void nzo_conv2d_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W,
-                                 size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch) {
-    const size_t H_out = H + 2 * pad - K_h + 1, W_out = W + 2 * pad - K_w + 1, CKK = C * K_h * K_w;
+ * img2colKernel src/OperationKernels.cu:1308-1328: h = ho*stride - pad + r, w = wo*stride - pad + s) and dC the
+ * pixel-major gradient of Col2ImgNode::backward (:660-665); fp16-rounded operands, fp32 accumulation over the
+ * pixels in ascending order (and over the images, for shared weights). */
+void nzo_conv2d_backward_weights_strided(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H,
+                                         size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                                         size_t w_batch) {
+    const size_t H_out = (H + 2 * pad - K_h) / stride + 1, W_out = (W + 2 * pad - K_w) / stride + 1, CKK = C * K_h * K_w;
     float* xr = (float*)malloc(sizeof(float) * N * C * H * W);
     float* dyr = (float*)malloc(sizeof(float) * N * O * H_out * W_out);
     nzo_round_f16_array(xr, x, N * C * H * W);
@@ -456,7 +457,8 @@ void nzo_conv2d_backward_weights(float* dw, const float* x, const float* dy, siz
                 for (size_t b = (w_batch > 1 ? wb : 0); b < (w_batch > 1 ? wb + 1 : N); b++)
                     for (size_t ho = 0; ho < H_out; ho++)
                         for (size_t wo = 0; wo < W_out; wo++) {
-                            const long long h = (long long)(ho + r) - (long long)pad, w = (long long)(wo + s) - (long long)pad;
+                            const long long h = (long long)(ho * stride + r) - (long long)pad,
+                                            w = (long long)(wo * stride + s) - (long long)pad;
                             if (h < 0 || h >= (long long)H || w < 0 || w >= (long long)W) continue;
                             acc += xr[((b * C + c) * H + (size_t)h) * W + (size_t)w] * dyr[((b * O + o) * H_out + ho) * W_out + wo];
                         }
@@ -465,6 +467,11 @@ void nzo_conv2d_backward_weights(float* dw, const float* x, const float* dy, siz
         }
     free(xr);
     free(dyr);
+}
+
+void nzo_conv2d_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W,
+                                 size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch) {
+    nzo_conv2d_backward_weights_strided(dw, x, dy, N, C, H, W, O, K_h, K_w, 1, pad, w_batch);
 }
 
 /* ------------------------------------------------------------------------- */

@@ -139,6 +139,9 @@ void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_ou
  * statement); dy [N,O,H_out,W_out], w_ref [w_batch,1,C*K_h*K_w,O], dx [N,C,H,W]. */
 /* dw += weight gradient of the stride-1 Conv2d graph (Nodes.cu:169-182 on the column matrix of :605-630);
  * x [N,C,H,W], dy [N,O,H_out,W_out], dw [w_batch,1,C*K_h*K_w,O]. */
+void nzo_conv2d_backward_weights_strided(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H,
+                                         size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                                         size_t w_batch);
 void nzo_conv2d_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W,
                                  size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch);
 void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,

@@ -84,7 +84,7 @@ _add_bwd = _sig("nzo_add_backward", None, _f32p, _f32p, _Shape, _Shape)
 _im2col_bwd = _sig("nzo_im2col_backward", None, _f32p, _f32p, *([_sz] * 10))
 _col2im_bwd = _sig("nzo_col2im_backward", None, _f32p, _f32p, _sz, _sz, _sz, _sz)
 _conv_bwd_data = _sig("nzo_conv2d_backward_data", None, _f32p, _f32p, _f32p, *([_sz] * 9))
-_conv_bwd_w = _sig("nzo_conv2d_backward_weights", None, _f32p, _f32p, _f32p, *([_sz] * 9))
+_conv_bwd_w = _sig("nzo_conv2d_backward_weights_strided", None, _f32p, _f32p, _f32p, *([_sz] * 10))
 _softmax = _sig("nzo_softmax", None, _f32p, _f32p, _sz, _sz)
 _softmax_jac = _sig("nzo_softmax_jacobian", None, _f32p, _f32p, _sz, _sz)
 _avgpool = _sig("nzo_avgpool2d", None, _f32p, _f32p, *([_sz] * 9))
@@ -285,14 +285,15 @@ def col2im_backward(dy: np.ndarray) -> np.ndarray:
     return out
 
 
-def conv2d_backward_weights(dw: np.ndarray, x: np.ndarray, dy: np.ndarray, K_h: int, K_w: int, pad: int) -> np.ndarray:
-    """dw += gradient of the stride-1 Conv2d graph with respect to its weights (in place, returns dw)."""
+def conv2d_backward_weights(dw: np.ndarray, x: np.ndarray, dy: np.ndarray, K_h: int, K_w: int, pad: int, stride: int = 1) -> np.ndarray:
+    """dw += gradient of the Conv2d graph with respect to its weights (in place, returns dw)."""
     x, dy = _c(x), _c(dy)
     assert dw.dtype == np.float32 and dw.flags.c_contiguous
     N, Cc, H, W = x.shape
     O = dy.shape[1]
-    assert dy.shape == (N, O, H + 2 * pad - K_h + 1, W + 2 * pad - K_w + 1) and dw.shape[1:] == (1, Cc * K_h * K_w, O)
-    _conv_bwd_w(dw.reshape(-1), x.reshape(-1), dy.reshape(-1), N, Cc, H, W, O, K_h, K_w, pad, dw.shape[0])
+    assert dy.shape == (N, O, (H + 2 * pad - K_h) // stride + 1, (W + 2 * pad - K_w) // stride + 1)
+    assert dw.shape[1:] == (1, Cc * K_h * K_w, O)
+    _conv_bwd_w(dw.reshape(-1), x.reshape(-1), dy.reshape(-1), N, Cc, H, W, O, K_h, K_w, stride, pad, dw.shape[0])
     return dw
 
 

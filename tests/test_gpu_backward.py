@@ -321,6 +321,51 @@ def test_conv1x1_backward_weights_is_bit_exact_on_integers(nz, oracle, N, C, H, 
     assert np.array_equal(got.astype(np.float64), chain)
 
 
+CONV_GEN_BWD_W = [  # N, C, H, W, O, Kh, Kw, stride, pad, w_batch: every geometry but 3x3 s1 p1 and 1x1 s1 p0
+    (2, 3, 9, 8, 4, 3, 3, 2, 1, 1), (1, 2, 11, 13, 3, 5, 5, 1, 2, 1), (2, 2, 10, 9, 2, 5, 3, 2, 0, 2), (1, 3, 12, 12, 2, 7, 7, 3, 3, 1),
+    (3, 1, 6, 7, 5, 2, 4, 1, 1, 3), (2, 20, 16, 300, 70, 5, 5, 1, 2, 1),      # several 128-pixel segments per row, two o tiles, 4 chunks
+    (2, 40, 33, 37, 100, 3, 3, 2, 1, 1), (2, 7, 20, 20, 9, 3, 3, 1, 0, 1), (1, 5, 40, 260, 6, 3, 3, 4, 2, 1), (2, 3, 30, 30, 3, 11, 11, 4, 5, 2),
+    (1, 130, 12, 12, 8, 1, 1, 2, 0, 1)]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", CONV_GEN_BWD_W)
+def test_conv_backward_weights_any_geometry_is_bit_exact_on_integers(nz, oracle, N, C, H, W, O, Kh, Kw, stride, pad, wb):
+    rng = np.random.default_rng(N * 31 + C * 17 + H * 7 + W + O * 3 + Kh + 5 * stride)
+    Ho, Wo = (H + 2 * pad - Kh) // stride + 1, (W + 2 * pad - Kw) // stride + 1
+    x = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    dy = rng.integers(-3, 4, size=(N, O, Ho, Wo)).astype(np.float32)
+    dw0 = rng.integers(-5, 6, size=(wb, 1, C * Kh * Kw, O)).astype(np.float32)
+    expect = oracle.conv2d_backward_weights(dw0.copy(), x, dy, Kh, Kw, pad, stride)
+    got = host(nz.conv2d_backward_weights(dev(dw0), dev(x), dev(dy), Kh, Kw, stride, pad))
+    assert np.array_equal(got, expect)
+
+
+def test_conv_backward_weights_any_geometry_float_tolerance(nz, oracle):
+    N, C, H, W, O, K, stride, pad = 2, 24, 40, 72, 48, 5, 2, 2
+    Ho, Wo = (H + 2 * pad - K) // stride + 1, (W + 2 * pad - K) // stride + 1
+    rng = np.random.default_rng(29)
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    dy = rng.standard_normal((N, O, Ho, Wo)).astype(np.float32)
+    got = host(nz.conv2d_backward_weights(dev(np.zeros((1, 1, C * K * K, O))), dev(x), dev(dy), K, K, stride, pad))
+    xr = np.pad(oracle.round_f16(x).astype(np.float64), ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+    dyr = oracle.round_f16(dy).astype(np.float64)
+    truth = np.zeros((C, K, K, O))
+    for r in range(K):
+        for s2 in range(K):
+            patch = xr[:, :, r:r + stride * Ho:stride, s2:s2 + stride * Wo:stride]
+            truth[:, r, s2, :] = np.einsum("nchw,nohw->co", patch, dyr)
+    mr, fr = oracle.errors(got.reshape(-1), truth.reshape(-1), float(np.sqrt(np.mean(truth ** 2))))
+    assert mr <= 1e-3 and fr <= 1e-4, (mr, fr)
+
+
+def test_conv_backward_weights_rejects_what_the_kernels_do_not_take(nz):
+    import torch
+    x, dy = torch.zeros((1, 1, 40, 40), device="cuda"), torch.zeros((1, 1, 29, 29), device="cuda")
+    with pytest.raises(nz.NzHipError) as e:                      # 12 x 12 = 144 taps
+        nz.conv2d_backward_weights(torch.zeros((1, 1, 144, 1), device="cuda"), x, dy, 12, 12, 1, 0)
+    assert e.value.status == -3
+
+
 def test_conv1x1_backward_weights_float_tolerance(nz, oracle):
     N, C, H, W, O = 3, 96, 20, 28, 80
     rng = np.random.default_rng(19)
@@ -397,7 +442,9 @@ def test_conv2d_backward_relu_bias_equals_relu_backward_then_bias(nz, oracle, N,
 
 def test_conv2d_backward_weights_rejects_what_it_does_not_cover(nz):
     from neuzephyr_amd.capi import NzHipError
-    with pytest.raises(NzHipError):      # stride 2
-        nz.conv2d_backward_weights(dev(np.zeros((1, 1, 18, 3))), dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 4, 4))), 3, 3, 2, 1)
-    with pytest.raises(NzHipError):      # 5x5
-        nz.conv2d_backward_weights(dev(np.zeros((1, 1, 50, 3))), dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 8, 8))), 5, 5, 1, 2)
+    with pytest.raises(NzHipError) as e:      # stride 5
+        nz.conv2d_backward_weights(dev(np.zeros((1, 1, 18, 3))), dev(np.zeros((1, 2, 11, 11))), dev(np.zeros((1, 3, 3, 3))), 3, 3, 5, 1)
+    assert e.value.status == -3
+    with pytest.raises(NzHipError) as e:      # a kernel larger than the padded input
+        nz.conv2d_backward_weights(dev(np.zeros((1, 1, 50, 3))), dev(np.zeros((1, 2, 2, 2))), dev(np.zeros((1, 3, 1, 1))), 5, 5, 1, 0)
+    assert e.value.status == -2

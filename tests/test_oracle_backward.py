@@ -161,3 +161,19 @@ def test_conv2d_backward_weights_equals_the_pinned_chain(oracle, N, C, H, W, O, 
     got = oracle.conv2d_backward_weights(dw0.copy(), x, dy, K, K, pad)
     _, want = oracle.matmul_backward(oracle.im2col(x, K, K, 1, pad), dw0, oracle.col2im_backward(dy), dB0=dw0)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", [(2, 3, 9, 8, 4, 3, 3, 2, 1, 1), (1, 2, 11, 13, 3, 5, 5, 1, 2, 1),
+                                                            (2, 2, 10, 9, 2, 5, 3, 2, 0, 2), (1, 3, 12, 12, 2, 7, 7, 3, 3, 1),
+                                                            (3, 1, 6, 7, 5, 2, 4, 1, 1, 3)])
+def test_strided_conv2d_backward_weights_equals_the_pinned_chain(oracle, N, C, H, W, O, Kh, Kw, stride, pad, wb):
+    # any kernel extent and stride: the one-statement gradient == Img2Col.forward (whose index formula carries the
+    # stride) -> MatMul.backward (dB); exact on integers, so a wrong stride, tap or padding term shows
+    rng = np.random.default_rng(N + 10 * C + 100 * H + O + 7 * stride + Kh)
+    Ho, Wo = (H + 2 * pad - Kh) // stride + 1, (W + 2 * pad - Kw) // stride + 1
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    dy = rng.integers(-4, 5, size=(N, O, Ho, Wo)).astype(np.float32)
+    dw0 = rng.integers(-3, 4, size=(wb, 1, C * Kh * Kw, O)).astype(np.float32)
+    got = oracle.conv2d_backward_weights(dw0.copy(), x, dy, Kh, Kw, pad, stride)
+    _, want = oracle.matmul_backward(oracle.im2col(x, Kh, Kw, stride, pad), dw0, oracle.col2im_backward(dy), dB0=dw0)
+    assert np.array_equal(got, want)
