@@ -28,7 +28,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
-                    choices=["gemm8192", "gemm256", "gemm1024", "gemm_batched", "linear", "linear_prepared", "conv_a_prepared", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "gemv", "ragged", "conv_a", "conv_b",
+                    choices=["gemm8192", "gemm256", "gemm1024", "gemm_batched", "linear", "linear_prepared", "conv_a_prepared", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "conv_dwx_5x5", "gemv", "ragged", "conv_a", "conv_b",
                              "adam", "softmax_bwd", "matmul_f32",
                              "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -179,6 +179,30 @@ def make_workload(name, orc, capi):
 
         return Workload(name, 2.0 * N * H * W * C * 9 * O, 4.0 * (N * O * H * W + O * C * 9 + 2 * N * C * H * W), run, verify,
                         "hbm", "Conv2d data gradient: dx[16,64,128,128] += dy[16,128,128,128] (*) mirrored w[128,64,3,3]"), None
+    if name == "conv_dwx_5x5":
+        # weight gradient of a 5x5 convolution of the CA shape straight from x and dy (the gather kernel)
+        N, C, H, W, O, K = 16, 64, 128, 128, 128, 5
+        x = orc.fill((N, C, H, W), 4, "normal", 0.0, 1.0)
+        dy = orc.fill((N, O, H, W), 4104, "normal", 0.0, 1.0)
+        xd, dyd = dev(x), dev(dy)
+        dwd = torch.zeros((1, 1, C * K * K, O), device="cuda")
+
+        def run():
+            capi.conv2d_backward_weights(dwd, xd, dyd, K, K, 1, 2)
+
+        def verify():
+            dwd.zero_()
+            run()
+            xr = np.pad(orc.round_f16(x[:, :2]).astype(np.float64), ((0, 0), (0, 0), (2, 2), (2, 2)))
+            dyr = orc.round_f16(dy).astype(np.float64)
+            truth = np.zeros((2, K, K, O))
+            for r in range(K):
+                for sx in range(K):
+                    truth[:, r, sx, :] = np.einsum("nchw,nohw->co", xr[:, :, r:r + H, sx:sx + W], dyr)
+            return tolerance(orc, dwd.reshape(C, K * K, O)[:2].cpu().numpy().reshape(-1), truth.reshape(-1), name)
+
+        return Workload(name, 2.0 * N * H * W * C * K * K * O, 4.0 * (N * C * H * W + N * O * H * W + 2 * C * K * K * O), run, verify,
+                        "hbm", "Conv2d weight gradient, 5x5 s1 p2: dW[1600,128] += x[16,64,128,128] (*) dy[16,128,128,128], no column matrix"), None
     if name == "conv_dwx":
         # weight gradient of the CA convolution straight from x and dy (no column matrix)
         N, C, H, W, O = 16, 64, 128, 128, 128
@@ -687,7 +711,7 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "conv_a_prepared", "linear", "linear_prepared", "gemv", "ragged", "gemm256", "gemm1024", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "adam",
+        for name in ("conv_b", "conv_a", "conv_a_prepared", "linear", "linear_prepared", "gemv", "ragged", "gemm256", "gemm1024", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "conv_dwx_5x5", "adam",
                      "softmax_bwd", "matmul_f32"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)

@@ -2243,12 +2243,12 @@ static int conv1x1_backward_weights(float* dw, const float* x, const float* dy, 
 // whose contraction runs over the output pixels, with the column matrix of the reference's chain (Img2ColNode::forward,
 // src/Nodes.cu:605-630, as A of MatMulNode::backward's dB += A^T dC, :169-182) gathered from LDS instead of written to
 // memory. A workgroup owns up to 128 (channel, tap) rows (as many whole channels as fit) x 64 output channels and a band
-// of output rows of one image; per output row and per segment of 128 pixels it stages the K_h input rows of its channels
-// (the 127 * stride + K_w columns the segment touches, zero outside the image) and the dy segment in LDS as fp16, then
-// runs eight 32x32x16 MFMA steps per wave. The A fragment of a lane is eight pixels of one (c, r, s) row, `stride`
+// of output rows of one image; per segment of 128 output pixels (SR rows x SW columns, SW the power of two from 16 to 128
+// that covers the output width or 128) it stages the input rows of its channels that the segment touches (zero outside
+// the image) and the dy segment in LDS as fp16, then runs eight 32x32x16 MFMA steps per wave. The A fragment of a lane is eight pixels of one (c, r, s) row, `stride`
 // elements apart in the staged input row: eight 16-bit LDS reads, which is what makes every tap offset and stride
 // one code path. Band sums go to a workspace and are added in ascending order by conv_dwg_reduce_kernel.
-constexpr int DWG_PX = 128, DWG_OT = 64, DWG_ROWS = 128, DWG_ZPITCH = DWG_PX + 8;
+constexpr int DWG_PX = 128, DWG_OT = 128, DWG_ROWS = 128, DWG_ZPITCH = DWG_PX + 8, DWG_NB = DWG_OT / 32;
 
 struct ConvDwGenArgs {
     const float* x;        // [N, C, H, W]
@@ -2256,14 +2256,20 @@ struct ConvDwGenArgs {
     float* partial;        // [chunk][o_tile][image][band][DWG_ROWS][DWG_OT]
     int C, H, W, O, Ho, Wo, Kh, Kw, stride, pad;
     int cc;                // channels per workgroup
-    int pw;                // staged columns per input row: (DWG_PX - 1) * stride + Kw, rounded up to an odd count
+    int pw;                // staged columns per input row (a multiple of 4 for the vector path)
+    int shift;             // staged column 0 is image column wo0 * stride - pad - shift (vector path: 16-byte aligned)
+    int sw_log;            // log2 of the segment width SW; a segment is 128 / SW output rows x SW output columns
+    int span;              // staged input rows per channel: (128 / SW - 1) * stride + Kh
     int bands, band_rows, n_images;
 };
 
+// VEC: W and Wo are multiples of 4 and x, dy are 16-byte aligned: rows are staged with 16-byte loads (a group of four
+// columns is then wholly inside or wholly outside the image) and 8-byte LDS stores; otherwise element by element.
+template <bool VEC>
 __global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     _Float16* xs = reinterpret_cast<_Float16*>(lds);                                   // [cc * Kh][pw]
-    _Float16* zs = xs + ((p.cc * p.Kh * p.pw + 7) & ~7);                                // [DWG_OT][DWG_ZPITCH]
+    _Float16* zs = xs + ((p.cc * p.span * p.pw + 7) & ~7);                              // [DWG_OT][DWG_ZPITCH]
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, lh = lane >> 5;
@@ -2276,9 +2282,9 @@ __global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
     const float* ximg = p.x + ((long)img * p.C + c0) * p.H * p.W;
     const float* zimg = p.dy + ((long)img * p.O + o0) * p.Ho * p.Wo;
 
-    floatx16 acc[2];
+    floatx16 acc[DWG_NB];
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < DWG_NB; j++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
@@ -2286,37 +2292,64 @@ __global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
     const int m = wave * 32 + li;
     const bool row_live = m < nch * taps;
     const int mc = row_live ? m / taps : 0, mt = row_live ? m % taps : 0;
-    const int a_base = (mc * p.Kh + mt / p.Kw) * p.pw + mt % p.Kw + 8 * lh * p.stride;
-    const int rows_staged = nch * p.Kh, n_stage = rows_staged * p.pw;
-    const int segs = (p.Wo + DWG_PX - 1) / DWG_PX;
+    const int a_base = (mc * p.span + mt / p.Kw) * p.pw + mt % p.Kw + p.shift + 8 * lh * p.stride;
+    const int rows_staged = nch * p.span;
+    const int SW = 1 << p.sw_log, SR = DWG_PX >> p.sw_log;
+    const int segs = (p.Wo + SW - 1) >> p.sw_log;
 
-    for (int ho = h_begin; ho < h_end; ho++) {
+    for (int ho = h_begin; ho < h_end; ho += SR) {
         for (int seg = 0; seg < segs; seg++) {
-            const int wo0 = seg * DWG_PX;
-            const int w_first = wo0 * p.stride - p.pad;                       // image column of staged column 0
-            for (int e = tid; e < n_stage; e += 256) {
-                const int row = e / p.pw, col = e - row * p.pw;
-                const int c = row / p.Kh, r = row - c * p.Kh;
-                const int h = ho * p.stride - p.pad + r, w = w_first + col;
-                const bool in = h >= 0 && h < p.H && w >= 0 && w < p.W;
-                const float v = ximg[((long)c * p.H + (in ? h : 0)) * p.W + (in ? w : 0)];
-                xs[e] = (_Float16)(in ? v : 0.f);
-            }
-            for (int e = tid; e < DWG_OT * DWG_PX; e += 256) {
-                const int o = e / DWG_PX, k = e % DWG_PX;
-                const bool in = o0 + o < p.O && wo0 + k < p.Wo;
-                const float v = zimg[((long)(in ? o : 0) * p.Ho + ho) * p.Wo + (in ? wo0 + k : 0)];
-                zs[o * DWG_ZPITCH + k] = (_Float16)(in ? v : 0.f);
+            const int wo0 = seg * SW;
+            const int w_first = wo0 * p.stride - p.pad - p.shift;               // image column of staged column 0
+            if (VEC) {
+                const int pw4 = p.pw >> 2, n4 = rows_staged * pw4;
+                for (int e = tid; e < n4; e += 256) {
+                    const int row = e / pw4, q = e - row * pw4;
+                    const int c = row / p.span, r = row - c * p.span;
+                    const int h = ho * p.stride - p.pad + r, w = w_first + 4 * q;
+                    const bool in = h >= 0 && h < p.H && w >= 0 && w < p.W;
+                    const floatx4 v = *reinterpret_cast<const floatx4*>(ximg + ((long)c * p.H + (in ? h : 0)) * p.W + (in ? w : 0));
+                    half4_t hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+                    const half4_t zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+                    *reinterpret_cast<half4_t*>(xs + row * p.pw + 4 * q) = in ? hv : zero;
+                }
+                for (int e = tid; e < DWG_OT * DWG_PX / 4; e += 256) {
+                    const int o = e / (DWG_PX / 4), k = (e % (DWG_PX / 4)) * 4;
+                    const int kr = k >> p.sw_log, kc = k & (SW - 1);
+                    const bool in = o0 + o < p.O && wo0 + kc < p.Wo && ho + kr < h_end;
+                    const floatx4 v = *reinterpret_cast<const floatx4*>(zimg + ((long)(in ? o : 0) * p.Ho + (in ? ho + kr : 0)) * p.Wo + (in ? wo0 + kc : 0));
+                    half4_t hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+                    const half4_t zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+                    *reinterpret_cast<half4_t*>(zs + o * DWG_ZPITCH + k) = in ? hv : zero;
+                }
+            } else {
+                const int n_stage = rows_staged * p.pw;
+                for (int e = tid; e < n_stage; e += 256) {
+                    const int row = e / p.pw, col = e - row * p.pw;
+                    const int c = row / p.span, r = row - c * p.span;
+                    const int h = ho * p.stride - p.pad + r, w = w_first + col;
+                    const bool in = h >= 0 && h < p.H && w >= 0 && w < p.W;
+                    const float v = ximg[((long)c * p.H + (in ? h : 0)) * p.W + (in ? w : 0)];
+                    xs[e] = (_Float16)(in ? v : 0.f);
+                }
+                for (int e = tid; e < DWG_OT * DWG_PX; e += 256) {
+                    const int o = e / DWG_PX, k = e % DWG_PX;
+                    const int kr = k >> p.sw_log, kc = k & (SW - 1);
+                    const bool in = o0 + o < p.O && wo0 + kc < p.Wo && ho + kr < h_end;
+                    const float v = zimg[((long)(in ? o : 0) * p.Ho + (in ? ho + kr : 0)) * p.Wo + (in ? wo0 + kc : 0)];
+                    zs[o * DWG_ZPITCH + k] = (_Float16)(in ? v : 0.f);
+                }
             }
             __syncthreads();
 #pragma unroll 2
             for (int ks = 0; ks < DWG_PX / 16; ks++) {
                 half8_t af;
-                const _Float16* ap = xs + a_base + ks * 16 * p.stride;
+                // pixels 16 ks .. 16 ks + 15 of the segment: output row (16 ks) / SW, columns from (16 ks) % SW
+                const _Float16* ap = xs + a_base + (((ks * 16) >> p.sw_log) * p.pw + ((ks * 16) & (SW - 1))) * p.stride;
 #pragma unroll
                 for (int j = 0; j < 8; j++) af[j] = row_live ? ap[j * p.stride] : (_Float16)0.f;
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
+                for (int j = 0; j < DWG_NB; j++) {
                     const half8_t bf = *reinterpret_cast<const half8_t*>(zs + (j * 32 + li) * DWG_ZPITCH + ks * 16 + lh * 8);
                     acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc[j], 0, 0, 0);
                 }
@@ -2327,7 +2360,7 @@ __global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
     // accumulator (block j, register r): row 32 wave + (r >> 2) * 8 + lh * 4 + (r & 3), column 32 j + li
     float* out = p.partial + ((((long)blockIdx.y * gridDim.z + blockIdx.z) * p.n_images + img) * p.bands + band) * (DWG_ROWS * DWG_OT);
 #pragma unroll
-    for (int j = 0; j < 2; j++)
+    for (int j = 0; j < DWG_NB; j++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int row = wave * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
@@ -2357,10 +2390,19 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
     int cc = (int)(DWG_ROWS / taps);
     if (cc > (int)C) cc = (int)C;
-    int pw = (int)((DWG_PX - 1) * stride + K_w) | 1;                 // odd: consecutive staged rows start on different banks
+    const bool vec = W % 4 == 0 && Wo % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0;
+    // vector path: the staged window starts at a multiple of four columns, `shift` columns left of the first one needed
+    // (128 * stride is a multiple of 4, so the shift is the same for every segment)
+    const int shift = vec ? (int)(((4 - (long)(pad % 4)) % 4 + 4) % 4) : 0;
+    int sw_log = 7;                                                   // segment width: 16 .. 128, covering the output width
+    while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= Wo) sw_log--;
+    const int SW = 1 << sw_log, SR = DWG_PX / SW;
+    const int span = (int)((SR - 1) * stride + K_h);
+    int pw = (int)((SW - 1) * stride + K_w) + shift;
+    pw = vec ? (pw + 3) / 4 * 4 : (pw | 1);                           // scalar path: odd, rows start on different banks
     // staged input rows + dy segment must fit the 64 KiB a workgroup may take without crowding out its neighbours
-    while (cc > 1 && ((size_t)cc * K_h * pw + 8) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2 > 64 * 1024) cc--;
-    const size_t lds_bytes = (((size_t)cc * K_h * pw + 7) & ~(size_t)7) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2;
+    while (cc > 1 && ((size_t)cc * span * pw + 8) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2 > 64 * 1024) cc--;
+    const size_t lds_bytes = (((size_t)cc * span * pw + 7) & ~(size_t)7) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2;
     if (lds_bytes > 64 * 1024) return NZHIP_E_UNSUPPORTED;
     const int chunks = (int)((C + cc - 1) / cc), otiles = (int)((O + DWG_OT - 1) / DWG_OT);
     if (chunks > 65535 || otiles > 65535) return NZHIP_E_UNSUPPORTED;
@@ -2369,7 +2411,9 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     long want = (4L * device_cu_count() + units - 1) / units;
     if (want < 1) want = 1;
     if (want > (long)Ho) want = (long)Ho;
-    const int band_rows = (int)((Ho + want - 1) / want), bands = (int)((Ho + band_rows - 1) / band_rows);
+    int band_rows = (int)((Ho + want - 1) / want);
+    band_rows = (band_rows + SR - 1) / SR * SR;                       // whole segments: a segment never straddles two bands
+    const int bands = (int)((Ho + band_rows - 1) / band_rows);
     if (N * (size_t)bands > 0x7fffffffull) return NZHIP_E_UNSUPPORTED;
     const size_t regions = (size_t)chunks * otiles * N * bands;
     float* partial = nullptr;
@@ -2378,10 +2422,11 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     a.x = x; a.dy = dy; a.partial = partial;
     a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.Ho = (int)Ho; a.Wo = (int)Wo;
     a.Kh = (int)K_h; a.Kw = (int)K_w; a.stride = (int)stride; a.pad = (int)pad;
-    a.cc = cc; a.pw = pw; a.bands = bands; a.band_rows = band_rows; a.n_images = (int)N;
-    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(conv_dwg_kernel), (int)lds_bytes, "hipFuncSetAttribute(conv_dwg)");
+    a.cc = cc; a.pw = pw; a.shift = shift; a.sw_log = sw_log; a.span = span; a.bands = bands; a.band_rows = band_rows; a.n_images = (int)N;
+    auto kfn = vec ? conv_dwg_kernel<true> : conv_dwg_kernel<false>;
+    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(conv_dwg)");
     if (rc == NZHIP_OK) {
-        hipLaunchKernelGGL(conv_dwg_kernel, dim3((unsigned)(N * bands), (unsigned)chunks, (unsigned)otiles), dim3(256), lds_bytes, s, a);
+        hipLaunchKernelGGL(kfn, dim3((unsigned)(N * bands), (unsigned)chunks, (unsigned)otiles), dim3(256), lds_bytes, s, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg kernel launch");
     }
