@@ -657,7 +657,11 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
 // Progress: a workgroup only waits for workgroups with a smaller wave number or of its own wave, and
 // workgroups are dispatched in order, so with one workgroup per CU and at least 256 CUs nobody waits
 // for a workgroup that cannot start.
-constexpr int COOP_KP = 32, COOP_SB = 16, COOP_WG = COOP_SB * COOP_SB;
+#ifndef NZHIP_COOP_KP
+#define NZHIP_COOP_KP 32
+#endif
+constexpr int COOP_KP = NZHIP_COOP_KP, COOP_SB = 16, COOP_WG = COOP_SB * COOP_SB;
+constexpr int COOP_RND = COOP_KP / 2;           // k tiles of a panel in which rounding work is scheduled (a block every four)
 
 struct CoopArgs {
     H16Args g;
@@ -886,8 +890,8 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
     // one lane signals; POLL_IT: wave 0 reads the counter of the next panel's stage; CHECK_IT: the k
     // tile in which the first requests of the next panel are issued.
     constexpr int PRE = HALF - 4 - LOADS;
-    constexpr int DRAIN_IT = 18, POLL_IT = COOP_KP - 7, CHECK_IT = COOP_KP - NSTAGE;
-    static_assert(DRAIN_IT > 16 && DRAIN_IT < POLL_IT && POLL_IT + 2 < CHECK_IT, "schedule");
+    constexpr int DRAIN_IT = COOP_RND + 2, POLL_IT = COOP_KP - 7, CHECK_IT = COOP_KP - NSTAGE;
+    static_assert(DRAIN_IT > COOP_RND && DRAIN_IT < POLL_IT && POLL_IT + 2 < CHECK_IT, "schedule");
     unsigned polled = 0;
     auto k_tile = [&](const int kt, const int slot_c, const int ph) {   // slot_c = kt % NSTAGE, ph = kt & 3 (compile time)
         const int it = kt & (COOP_KP - 1), pn = kt / COOP_KP;
@@ -898,7 +902,7 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
             __builtin_amdgcn_sched_barrier(0);
         }
         if (it == DRAIN_IT) wait_vmcnt<0>();                  // this wave's image stores are in memory
-        else if ((ph == 1 || ph == 2) && it < 16 && cv_dst) wait_vmcnt<(NSTAGE - 2) * LOADS + 4>();   // + the staging requests of this block
+        else if ((ph == 1 || ph == 2) && it < COOP_RND && cv_dst) wait_vmcnt<(NSTAGE - 2) * LOADS + 4>();   // + the staging requests of this block
         else wait_vmcnt<(NSTAGE - 2) * LOADS>();              // tile kt+1 has landed (this wave's share)
         wait_lgkmcnt0();
         if (it == CHECK_IT && pn + 1 < q.panels && wave == 0) wait_stage(polled, flag_of(wv, pn + 1));
@@ -910,7 +914,7 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
             __hip_atomic_fetch_add(flag_of(t_w, t_p), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (it == POLL_IT && pn + 1 < q.panels && wave == 0)
             polled = __hip_atomic_load(flag_of(wv, pn + 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (ph == 0 && it < 16) {                             // in front of this k tile's ring requests
+        if (ph == 0 && it < COOP_RND) {                             // in front of this k tile's ring requests
             if (it == 0) begin_panel(pn);
             begin_block(it >> 2);
             if (cv_dst) cv_request();
@@ -924,7 +928,7 @@ __global__ __launch_bounds__(512, 1) void gemm_h16c_kernel(const CoopArgs q) {
             if (t >= HALF && (t & 3) == 3) read_a(nxt, (t - HALF) / 4);
             if (t >= NPOS - 4) read_b(nxt, 4 + t - (NPOS - 4));
             __builtin_amdgcn_sched_barrier(0);
-            if ((t == PRE + LOADS || t == HALF + 5) && ph == 3 && it < 16 && cv_dst) {
+            if ((t == PRE + LOADS || t == HALF + 5) && ph == 3 && it < COOP_RND && cv_dst) {
                 cv_round(t == PRE + LOADS ? 0 : 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
