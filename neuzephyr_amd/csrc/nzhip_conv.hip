@@ -507,8 +507,27 @@ struct IgemmArgs {
     int w_batched;
     long bias_sp, bias_sc, bias_sn;   // bias element of (image b, pixel, channel o): bias[b*bias_sn + pixel*bias_sp + o*bias_sc]
     int relu;
-    int patch_map;                    // resident kernel: 0 strided by the grid, 1 XCD-contiguous, 2 XCD-contiguous runs
+    int patch_map;                    // resident kernels: 0 strided by the grid, 1 XCD-contiguous, 2 XCD-contiguous runs,
+                                      // 3 image-major (per-sample weights: every workgroup stays inside one image)
+    int n_images;                     // patch_map 3: images of the batch (the grid is a multiple of it wide)
+    long w_image_bytes;               // patch_map 3: bytes from one image's weight image to the next
 };
+
+// Patches of a workgroup of the resident kernels under patch_map 3, for the reference's Conv2d parameter with one
+// weight copy per sample (src/Model.cu:248-252): the grid's G workgroups are split evenly over the images (G / n_images
+// each, neighbours in XCD-major order, so that an image's workgroups share an L2 when the counts divide), and a
+// workgroup walks its image's patches with that stride. Its weights are those of its image.
+__device__ __forceinline__ void image_major_patches(const IgemmArgs& p, int patches_per_image, int& image, int& first_patch,
+                                                    int& patch_stride, int& my_patches) {
+    const int G = gridDim.x;
+    const int u = (G % 8 == 0) ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+    const int wpi = G / p.n_images;
+    image = u / wpi;
+    const int j = u - image * wpi;
+    first_patch = image * patches_per_image + j;
+    patch_stride = wpi;
+    my_patches = j < patches_per_image ? (patches_per_image - j + wpi - 1) / wpi : 0;
+}
 
 template <int KH, int KW, int TW, int BN, bool VEC4>
 __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(const IgemmArgs p) {
@@ -698,6 +717,9 @@ __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float1
                                                                          const float* __restrict__ w_ref, int C,
                                                                          int O, int n_chunks, int n_otiles) {
     constexpr int TAPS = KH * KW;
+    // blockIdx.z: weight copy (one per sample for the reference's Conv2d parameter); images follow each other
+    w_ref += (long)blockIdx.z * C * TAPS * O;
+    dst += (long)blockIdx.z * n_otiles * n_chunks * (BN * TAPS * IG_CC);
     const int slab = blockIdx.y;                               // o_tile * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = slab / n_chunks;
     const int t = blockIdx.x * 256 + threadIdx.x;
@@ -743,9 +765,14 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     const int patches_per_image = p.tiles_w * p.tiles_h;
     const long plane = (long)p.H * p.W;
 
+    int w_image = 0, first_patch = blockIdx.x, patch_stride = gridDim.x;
+    int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    if (p.patch_map == 3) image_major_patches(p, patches_per_image, w_image, first_patch, patch_stride, my_patches);
+
     // resident weights: n_chunks * W_CHUNK bytes, 1 KiB per wave-wide request
     {
-        const char* wsrc = reinterpret_cast<const char*>(p.wimg) + (long)o_tile * p.n_chunks * W_CHUNK + lane * 16;
+        const char* wsrc = reinterpret_cast<const char*>(p.wimg) + (long)w_image * p.w_image_bytes +
+                           (long)o_tile * p.n_chunks * W_CHUNK + lane * 16;
         const int pieces = p.n_chunks * (W_CHUNK / 1024);
         for (int j = wave; j < pieces; j += NW)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc + (long)j * 1024),
@@ -783,9 +810,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     // is a multiple of 8 wide) the workgroups of one XCD share a contiguous eighth of the patches: halo
     // rows and columns that neighbouring patches have in common are then found in that L2 instead of
     // being fetched again from memory.
-    int first_patch = blockIdx.x, patch_stride = gridDim.x;
-    int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-    if (p.patch_map != 0 && gridDim.x % 8 == 0) {
+    if (p.patch_map != 0 && p.patch_map != 3 && gridDim.x % 8 == 0) {
         const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3, nq = gridDim.x >> 3;
         const int lo = (int)((long)n_patches * xcd / 8), hi = (int)((long)n_patches * (xcd + 1) / 8);
         if (p.patch_map == 1) {                                  // the XCD's workgroups sweep its range side by side
@@ -1061,6 +1086,9 @@ __global__ __launch_bounds__(256) void conv_weight_image_db_kernel(_Float16* __r
                                                                    int C, int O, int n_chunks, int n_otiles) {
     // One thread per (row, tap) of a slab: 16 reads that are contiguous across the threads of a wave (adjacent
     // output channels) and two 16-byte stores, instead of one 2-byte store per element.
+    // blockIdx.z: weight copy (one per sample for the reference's Conv2d parameter); images follow each other
+    w_ref += (long)blockIdx.z * C * 9 * O;
+    dst += (long)blockIdx.z * n_otiles * n_chunks * BN * 144;
     const int slab = blockIdx.y;                               // o_tile * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = slab / n_chunks;
     const int t = blockIdx.x * 256 + threadIdx.x;
@@ -1115,7 +1143,11 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
     const int patches_per_image = p.tiles_w * p.tiles_h;
     const long plane = (long)p.H * p.W;
 
-    const char* wtile = reinterpret_cast<const char*>(p.wimg) + (long)o_tile * NCH * BN * 288;
+    int w_image = 0, first_patch = blockIdx.x, patch_stride = gridDim.x;
+    int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
+    if (p.patch_map == 3) image_major_patches(p, patches_per_image, w_image, first_patch, patch_stride, my_patches);
+
+    const char* wtile = reinterpret_cast<const char*>(p.wimg) + (long)w_image * p.w_image_bytes + (long)o_tile * NCH * BN * 288;
     {
         const char* wsrc = wtile + lane * 16;
         constexpr int pieces = NCH * (W_CHUNK / 1024);
@@ -1159,9 +1191,7 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
         return hb + (t_q4 >> 1) * H_PLANE + (hh * G::WW + ww) * 16 + (t_q4 & 1) * 8;
     };
 
-    int first_patch = blockIdx.x, patch_stride = gridDim.x;
-    int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-    if (p.patch_map != 0 && gridDim.x % 8 == 0) {               // the workgroups of an XCD sweep a contiguous eighth
+    if (p.patch_map != 0 && p.patch_map != 3 && gridDim.x % 8 == 0) {   // the workgroups of an XCD sweep a contiguous eighth
         const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3, nq = gridDim.x >> 3;
         const int lo = (int)((long)n_patches * xcd / 8), hi = (int)((long)n_patches * (xcd + 1) / 8);
         first_patch = lo + q;
@@ -1393,6 +1423,14 @@ static bool conv_igemm_applicable(size_t C, size_t O, size_t K_h, size_t K_w, si
     return stride == 1 && ((K_h == 3 && K_w == 3) || (K_h == 1 && K_w == 1)) && pad <= K_w - 1 && C >= 8 && N <= 65535;
 }
 
+// Per-sample weights (one copy per image) on the resident kernels: the grid must split evenly over the images, at
+// least one workgroup each. Returns the grid width (0: not possible, the per-patch slab kernel takes the layer).
+static int resident_grid_per_sample(size_t N, int n_otiles) {
+    const int per_tile = device_cu_count() / n_otiles;
+    if (N == 0 || N > (size_t)per_tile) return 0;
+    return (int)(per_tile / (int)N * (int)N);
+}
+
 // Key of a weight image: everything the conversion kernel's output depends on (image kind, tile shape, source and extents).
 static void conv_image_key(uint64_t (&key)[PREPARED_KEY_WORDS], int kind, int kh, int kw, int bn, const float* w_ref, size_t C,
                            size_t O, int n_chunks, int n_otiles, size_t w_batch) {
@@ -1418,18 +1456,19 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         const bool vec4r = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
         const bool pixb = bias && bias_sp != 0;                  // per-pixel bias with a 128-channel tile: out of registers
         const bool count_ok = n_chunks == 2 || n_chunks == 4 || (n_chunks == 8 && NI == 1);
-        if (!(db_env && atoi(db_env) == 0) && w_batch == 1 && count_ok && vec4r && !(pixb && NI == 2)) {
+        const int grid_ps = w_batch > 1 ? resident_grid_per_sample(N, n_otiles) : 0;
+        if (!(db_env && atoi(db_env) == 0) && (w_batch == 1 || grid_ps > 0) && count_ok && vec4r && !(pixb && NI == 2)) {
             auto run = [&](auto nch_tag) -> int {
                 constexpr int NCH = decltype(nch_tag)::value;
                 constexpr size_t lds_need = (size_t)NCH * BN * 256 + 4 * CONV_DB_PLANE + 128 * sizeof(float);
                 static_assert(lds_need <= 160 * 1024 - 512, "LDS budget");
-                const size_t bytes = (size_t)n_otiles * NCH * BN * 288;
+                const size_t image_bytes = (size_t)n_otiles * NCH * BN * 288, bytes = image_bytes * w_batch;
                 uint64_t key[PREPARED_KEY_WORDS];
                 conv_image_key(key, 1, 3, 3, BN, w_ref, C, O, NCH, n_otiles, w_batch);
                 ImageLease lease;
                 if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
                 _Float16* wres = static_cast<_Float16*>(lease.ptr);
-                dim3 pg((unsigned)((BN * 9 + 255) / 256), (unsigned)(n_otiles * NCH));
+                dim3 pg((unsigned)((BN * 9 + 255) / 256), (unsigned)(n_otiles * NCH), (unsigned)w_batch);
                 if (lease.fill)
                     hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles);
                 IgemmArgs a;
@@ -1439,7 +1478,8 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                 a.tiles_w = (int)((W_out + TW - 1) / TW);
                 a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
                 a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
-                a.patch_map = 1;
+                a.patch_map = w_batch > 1 ? 3 : 1;
+                a.n_images = (int)N; a.w_image_bytes = (long)image_bytes;
                 const long n_patches = (long)N * a.tiles_w * a.tiles_h;
                 int rc = NZHIP_OK;
                 if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
@@ -1453,6 +1493,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                     const int cus = device_cu_count();
                     int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
                     if ((long)per_tile > n_patches) per_tile = (int)n_patches;
+                    if (w_batch > 1) per_tile = grid_ps;                          // a whole number of workgroups per image
                     hipLaunchKernelGGL(kdb, dim3((unsigned)per_tile, (unsigned)n_otiles, 1), dim3(512), lds_need, s, a, (int)n_patches);
                     hipError_t e = hipGetLastError();
                     if (e != hipSuccess) rc = set_hip_error(e, "conv3x3_resident_db kernel launch");
@@ -1472,14 +1513,15 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         const size_t lds_need = (size_t)n_chunks * W_CHUNK_R + G::HALO_BYTES + 128 * sizeof(float);   // + bias
         static const char* res_env = getenv("NZHIP_CONV_RESIDENT");
         const bool allow = res_env ? atoi(res_env) != 0 : true;
-        if (allow && w_batch == 1 && lds_need <= 160 * 1024 - 512) {
-            const size_t bytes = (size_t)n_otiles * n_chunks * W_CHUNK_R;
+        const int grid_ps = w_batch > 1 ? resident_grid_per_sample(N, n_otiles) : 0;
+        if (allow && (w_batch == 1 || grid_ps > 0) && lds_need <= 160 * 1024 - 512) {
+            const size_t image_bytes = (size_t)n_otiles * n_chunks * W_CHUNK_R, bytes = image_bytes * w_batch;
             uint64_t key[PREPARED_KEY_WORDS];
             conv_image_key(key, 2, KH, KW, BN, w_ref, C, O, n_chunks, n_otiles, w_batch);
             ImageLease lease;
             if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
             _Float16* wres = static_cast<_Float16*>(lease.ptr);
-            dim3 pg((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)(n_otiles * n_chunks));
+            dim3 pg((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)(n_otiles * n_chunks), (unsigned)w_batch);
             if (lease.fill)
                 hipLaunchKernelGGL((conv_weight_image_resident_kernel<KH, KW, BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C,
                                    (int)O, n_chunks, n_otiles);
@@ -1491,7 +1533,8 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             a.tiles_h = (int)((H_out + G::TH - 1) / G::TH);
             a.w_batched = 0; a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
             static const char* map_env = getenv("NZHIP_CONV_PATCH_MAP");
-            a.patch_map = map_env ? atoi(map_env) : 1;
+            a.patch_map = w_batch > 1 ? 3 : (map_env ? atoi(map_env) : 1);
+            a.n_images = (int)N; a.w_image_bytes = (long)image_bytes;
             const long n_patches = (long)N * a.tiles_w * a.tiles_h;
             int rc = NZHIP_OK;
             if (n_patches > 0x7fffffffL) rc = set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many patches");
@@ -1507,6 +1550,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                 const int cus = device_cu_count();
                 int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
                 if ((long)per_tile > n_patches) per_tile = (int)n_patches;
+                if (w_batch > 1) per_tile = grid_ps;                          // a whole number of workgroups per image
                 dim3 grid((unsigned)per_tile, (unsigned)n_otiles, 1);
                 hipLaunchKernelGGL(kres, grid, dim3(512), lds_need, s, a, (int)n_patches);
                 hipError_t e = hipGetLastError();
@@ -1553,6 +1597,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         a.bias_sn = bias_sn;
         a.relu = act == NZHIP_ACT_RELU;
         a.patch_map = 0;
+        a.n_images = (int)N; a.w_image_bytes = 0;
         const bool vec4 = (W % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
         auto kfn = vec4 ? conv_igemm_kernel<KH, KW, TW, BN, true> : conv_igemm_kernel<KH, KW, TW, BN, false>;
         if (rc == NZHIP_OK)
@@ -2082,7 +2127,7 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
         const size_t tw = wide ? 64 : 32, th = 256 / tw, bn = bn128 ? 128 : 64;
         const size_t units = N * ((W_out + tw - 1) / tw) * ((H_out + th - 1) / th) * ((O + bn - 1) / bn);
         const size_t w_lds = ((C + IG_CC - 1) / IG_CC) * bn * K_h * K_w * 32;       // fp16 weight image of one channel tile
-        const bool resident = w_batch == 1 && w_lds <= 148 * 1024;
+        const bool resident = (w_batch == 1 || N * ((O + bn - 1) / bn) <= (size_t)device_cu_count()) && w_lds <= 148 * 1024;
         few_patches = !resident && units * 4 <= (size_t)device_cu_count();
     }
     if (!force_ws && !few_patches && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL) {

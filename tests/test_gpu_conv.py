@@ -124,6 +124,38 @@ def test_conv2d_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, 
     assert np.array_equal(host(y), got)
 
 
+PER_SAMPLE = [  # N, C, H, W, O, k, pad, per-pixel bias: one weight copy per image, every copy different
+    (4, 32, 12, 64, 128, 3, 1, False),    # two halo buffers, 128-channel tile, 64 workgroups per image
+    (3, 64, 9, 64, 64, 3, 1, True),       # two halo buffers, 64-channel tile, per-pixel bias; 255 of 256 workgroups used
+    (16, 64, 16, 64, 128, 3, 1, False),   # sixteen images, 16 workgroups each
+    (5, 48, 10, 72, 100, 3, 1, False),    # three chunks: the single-buffer resident kernel
+    (2, 64, 8, 64, 128, 3, 1, True),      # per-pixel bias with a 128-channel tile: the single-buffer resident kernel
+    (6, 40, 9, 40, 70, 1, 0, False),      # 1x1, 32-wide patches, two channel tiles
+    (2, 160, 8, 64, 128, 3, 1, False),    # weights beyond LDS: the per-patch slab kernel
+    (300, 16, 4, 32, 16, 3, 1, False),    # more images than workgroups: the per-patch slab kernel
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,k,pad,pix", PER_SAMPLE)
+def test_conv2d_per_sample_weights_that_differ_between_images(nz, oracle, N, C, H, W, O, k, pad, pix):
+    # the reference's Conv2d parameter holds one weight copy per sample (src/Model.cu:248-252); here every copy is
+    # different, so a kernel that multiplied image b by another image's weights would be found out
+    rng = np.random.default_rng(N + 3 * C + 5 * H + W + O + k)
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    w = rng.integers(-3, 4, size=(N, O, C, k, k)).astype(np.float32)
+    Ho, Wo = oracle.out_hw(H, W, k, k, 1, pad)
+    if pix:
+        bias = rng.integers(-2, 3, size=(1, 1, Ho * Wo, O)).astype(np.float32)
+        strides, badd = (O, 1), bias.reshape(Ho, Wo, O).transpose(2, 0, 1)[None].astype(np.float64)
+    else:
+        bias = rng.integers(-2, 3, size=(O,)).astype(np.float32)
+        strides, badd = (0, 1), bias.reshape(1, O, 1, 1).astype(np.float64)
+    w_ref = np.concatenate([oracle.weights_oihw_to_ref(w[b]) for b in range(N)], axis=0)
+    truth = np.concatenate([oracle.conv2d_direct_f64(x[b:b + 1], w[b], None, 1, pad) for b in range(N)], axis=0) + badd
+    got = host(nz.conv2d_forward(dev(x), dev(w_ref), dev(bias), k, k, 1, pad, bias_strides=strides, relu=False))
+    assert np.array_equal(got.astype(np.float64), truth)
+
+
 def _conv_sweep_cases(seed, count):
     """Random geometries over every route: direct / streaming (few channels), implicit GEMM with 32- and 64-wide
     patches and both channel tiles, resident weights (single and double halo buffers), the column-matrix route
