@@ -187,7 +187,6 @@ struct H16Args {
     long c_sn, c_sc, bias_sn, bias_sc, bias_sm, bias_sk;
     int relu;
     int tiles_m, tiles_n, group_m;
-    int cus;                            // compute units of the device (workgroups are dealt out in rounds of that many)
 };
 
 // s_waitcnt on the vector-memory counter only (expcnt / lgkmcnt left at "don't wait").
@@ -462,15 +461,6 @@ __global__ __launch_bounds__(WM* WN * 64, (BM < CVT_ROWS ? 2 : 1)) void gemm_h16
     const char* a_tile = reinterpret_cast<const char*>(A) + (long)(tile_m / A_PER_BLOCK) * nk * A_BLOCK +
                          (tile_m % A_PER_BLOCK) * A_BYTES + wave * A_LOADS * 1024 + lane * 16;
     const char* b_tile = reinterpret_cast<const char*>(B) + (long)tile_n * nk * B_BYTES + wave * B_LOADS * 1024 + lane * 16;
-
-    // Two workgroups share a CU (BM = 128). Workgroups are dealt out in rounds of one per CU, so the two on a CU come
-    // from rounds of different parity. The even round's waves get issue priority: that workgroup runs its k loop at
-    // the full MFMA rate while the other one fills the gaps, and its result stores then fall under the other's k loop
-    // instead of both storing at once with idle matrix pipes.
-    // (4096 x 1024 x 4096: 57.9 -> 52.5 us in one process; a wave's priority, not a stream's.)
-    if constexpr (BM < CVT_ROWS) {
-        if (((blockIdx.x / (unsigned)p.cus) & 1) == 0) __builtin_amdgcn_s_setprio(3);
-    }
 
     // Past the end the last tile is requested again (into a slot nobody reads any more) so that
     // the number of loads in flight, which the vmcnt waits count on, is the same in every step.
@@ -1060,7 +1050,6 @@ int gemm_h16_coop_dispatch(const nzhip_gemm_desc& d, hipStream_t s) {
     g.bias_sm = d.bias_stride_row; g.bias_sk = d.bias_stride_col;
     g.relu = d.activation == NZHIP_ACT_RELU;
     g.tiles_m = (int)(Mp / 256); g.tiles_n = (int)(Np / 256); g.group_m = 4;
-    g.cus = device_cu_count();
     a.srcA = d.A; a.srcB = d.B; a.lda = d.lda; a.ldb = d.ldb;
     a.flags = flags; a.sn = sn; a.waves = waves; a.panels = panels;
     a.spin_limit = g_coop_spin_limit.load(std::memory_order_relaxed);
@@ -1276,7 +1265,6 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mf
         a.tiles_m = (int)(Mp / (half_m ? 128 : BM));
         a.tiles_n = (int)(Np / BN);
         a.group_m = half_m ? 8 : 4;
-        a.cus = device_cu_count();
         const size_t lds_bytes = half_m ? (size_t)3 * (128 + BN) * 64 : (size_t)NSTAGE * (BM + BN) * 64;
         void (*kfn)(const H16Args) = half_m          ? gemm_h16_kernel<128, BN, 2, 2, 3>
                                      : wm_waves == 4 ? gemm_h16_kernel<BM, BN, 4, 2, NSTAGE>
