@@ -2241,7 +2241,7 @@ extern "C" int nzhip_conv2d_backward_relu_bias(float* dz, float* dbias, const fl
 }
 
 // dw[i] += P[0][i] + P[1][i] + ... (ascending, then added to dw once): the per-image products of the 1x1 weight gradient
-__global__ __launch_bounds__(256) void dw_add_members_kernel(float* __restrict__ dw, const float* __restrict__ P, int members, long n) {
+static __global__ __launch_bounds__(256) void dw_add_members_kernel(float* __restrict__ dw, const float* __restrict__ P, int members, long n) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     float sum = 0.f;
@@ -2282,6 +2282,8 @@ static int conv1x1_backward_weights(float* dw, const float* x, const float* dy, 
     const int rc2 = workspace_free(P, s);
     return rc ? rc : rc2;
 }
+
+namespace nzhip {
 
 // ---- weight gradient for any kernel extent, stride and padding ---------------------------------------------------
 // dW[(c, r, s)][o] = sum over pixels of f16(x[c][ho*stride - pad + r][wo*stride - pad + s]) * f16(dy[o][ho][wo]): a product
@@ -2488,6 +2490,8 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     const int rc2 = workspace_free(partial, s);
     return rc ? rc : rc2;
 }
+
+}  // namespace nzhip
 
 /* Gradient of nzhip_conv2d_forward with respect to the weights, without the column matrix the reference's
  * chain needs (Img2ColNode::forward output as A in MatMulNode::backward, dB += A^T * dC, src/Nodes.cu:169-182):

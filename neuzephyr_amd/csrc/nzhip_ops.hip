@@ -714,7 +714,7 @@ struct BwdOperand {
 // Reductions are folded into the contraction (K' = members x K, one launch) when both operands are
 // laid out so that the member index continues the k index; otherwise the members are added one
 // launch after the other, which fixes the summation order.
-int accumulate_products(float* C, int64_t ldc, int64_t c_sn, int64_t c_sc, BwdOperand A, BwdOperand B, int64_t M,
+static int accumulate_products(float* C, int64_t ldc, int64_t c_sn, int64_t c_sc, BwdOperand A, BwdOperand B, int64_t M,
                         int64_t N, int64_t K, int64_t bn, int64_t bc, void* stream) {
     if (bn == 0 || bc == 0 || M == 0 || N == 0) return NZHIP_OK;
     auto launch = [&](const float* a, const float* b, float* c, int64_t k, int la, int64_t lda, int lb, int64_t ldb,
