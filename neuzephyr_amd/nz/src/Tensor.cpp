@@ -90,6 +90,7 @@ namespace nz::data {
         other._size = 0;
         other._shape = Dimension(0, 0, 0, 0);
         other._requires_grad = false;
+        ++_version;   // new contents, possibly at an address this tensor held before
         return *this;
     }
 
