@@ -2310,9 +2310,7 @@ struct ConvDwGenArgs {
     int bands, band_rows, n_images;
 };
 
-// VEC: W and Wo are multiples of 4 and x, dy are 16-byte aligned: rows are staged with 16-byte loads (a group of four
-// columns is then wholly inside or wholly outside the image) and 8-byte LDS stores; otherwise element by element.
-template <bool VEC>
+// Rows that do not allow 16-byte loads: staged element by element, four waves, 128 rows per workgroup.
 __global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     _Float16* xs = reinterpret_cast<_Float16*>(lds);                                   // [cc * Kh][pw]
@@ -2348,28 +2346,7 @@ __global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
         for (int seg = 0; seg < segs; seg++) {
             const int wo0 = seg * SW;
             const int w_first = wo0 * p.stride - p.pad - p.shift;               // image column of staged column 0
-            if (VEC) {
-                const int pw4 = p.pw >> 2, n4 = rows_staged * pw4;
-                for (int e = tid; e < n4; e += 256) {
-                    const int row = e / pw4, q = e - row * pw4;
-                    const int c = row / p.span, r = row - c * p.span;
-                    const int h = ho * p.stride - p.pad + r, w = w_first + 4 * q;
-                    const bool in = h >= 0 && h < p.H && w >= 0 && w < p.W;
-                    const floatx4 v = *reinterpret_cast<const floatx4*>(ximg + ((long)c * p.H + (in ? h : 0)) * p.W + (in ? w : 0));
-                    half4_t hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-                    const half4_t zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
-                    *reinterpret_cast<half4_t*>(xs + row * p.pw + 4 * q) = in ? hv : zero;
-                }
-                for (int e = tid; e < DWG_OT * DWG_PX / 4; e += 256) {
-                    const int o = e / (DWG_PX / 4), k = (e % (DWG_PX / 4)) * 4;
-                    const int kr = k >> p.sw_log, kc = k & (SW - 1);
-                    const bool in = o0 + o < p.O && wo0 + kc < p.Wo && ho + kr < h_end;
-                    const floatx4 v = *reinterpret_cast<const floatx4*>(zimg + ((long)(in ? o : 0) * p.Ho + (in ? ho + kr : 0)) * p.Wo + (in ? wo0 + kc : 0));
-                    half4_t hv = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-                    const half4_t zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
-                    *reinterpret_cast<half4_t*>(zs + o * DWG_ZPITCH + k) = in ? hv : zero;
-                }
-            } else {
+            {
                 const int n_stage = rows_staged * p.pw;
                 for (int e = tid; e < n_stage; e += 256) {
                     const int row = e / p.pw, col = e - row * p.pw;
@@ -2415,10 +2392,173 @@ __global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
         }
 }
 
+// The same product for rows that allow 16-byte loads (W and Wo multiples of 4, x and dy 16-byte aligned), on eight
+// waves: a workgroup owns up to 256 rows (channel, tap) x 128 output channels, so a dy segment is fetched half as
+// often, and the requests for the NEXT segment are issued before the current one multiplies. A thread's share of a
+// segment is a fixed set of 16-byte pieces (DWG8_XMAX of the input rows, 8 of dy) whose place in the tile does not
+// depend on the segment, so the index arithmetic is done once; per segment only the image row and column move.
+// Requests are unconditional (clamped addresses, zero selected when the piece is stored), so the compiler's waits
+// stay exact; the last step requests its own segment once more instead of branching.
+constexpr int DWG8_ROWS = 256, DWG8_XMAX = 7, DWG8_THREADS = 512;
+
+// XP: 16-byte pieces of the staged input rows per thread (the tile has at most 512 XP of them)
+// S1: stride 1. A lane's eight pixels are then eight consecutive halfs of a staged row: five dword reads and four
+// v_alignbit (by 0 or 16 bits, the parity of the lane's tap column) instead of eight 16-bit reads.
+template <int XP, bool S1>
+__global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGenArgs p) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    _Float16* xs = reinterpret_cast<_Float16*>(lds);                                   // [cc * span][pw]
+    _Float16* zs = xs + ((p.cc * p.span * p.pw + 7) & ~7);                              // [DWG_OT][DWG_ZPITCH]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const int band = blockIdx.x % p.bands, img = blockIdx.x / p.bands;
+    const int c0 = blockIdx.y * p.cc, o0 = blockIdx.z * DWG_OT;
+    const int taps = p.Kh * p.Kw;
+    const int nch = (p.C - c0) < p.cc ? (p.C - c0) : p.cc;
+    const int h_begin = band * p.band_rows;
+    const int h_end = (h_begin + p.band_rows) < p.Ho ? (h_begin + p.band_rows) : p.Ho;
+    const float* ximg = p.x + ((long)img * p.C + c0) * p.H * p.W;
+    const float* zimg = p.dy + ((long)img * p.O + o0) * p.Ho * p.Wo;
+
+    floatx16 acc[DWG_NB];
+#pragma unroll
+    for (int j = 0; j < DWG_NB; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+
+    const int m = wave * 32 + li;
+    const bool row_live = m < nch * taps;
+    const int mc = row_live ? m / taps : 0, mt = row_live ? m % taps : 0;
+    const int a_base = (mc * p.span + mt / p.Kw) * p.pw + mt % p.Kw + p.shift + 8 * lh * p.stride;
+    const bool wave_live = wave * 32 < nch * taps;                                     // wave-uniform
+    const int SW = 1 << p.sw_log, SR = DWG_PX >> p.sw_log;
+    const int segs = (p.Wo + SW - 1) >> p.sw_log;
+
+    // this thread's pieces of the staged input rows: piece e = tid + 512 k is 4 columns of staged row e / pw4
+    const int pw4 = p.pw >> 2, n4 = nch * p.span * pw4;
+    int xoff[XP], xrq[XP];
+#pragma unroll
+    for (int k = 0; k < XP; k++) {
+        const int e = tid + DWG8_THREADS * k;
+        const int row = e / pw4, q = e - row * pw4;
+        const int c = row / p.span, r = row - c * p.span;
+        xoff[k] = (c * p.H + r) * p.W + 4 * q;
+        xrq[k] = e < n4 ? (r | (q << 16)) : -1;
+    }
+    // ... and of the dy segment: output channel tid / 32 + 16 k, pixels 4 (tid % 32) .. + 3 of the segment
+    const int zo = tid >> 5, zk = (tid & 31) * 4;
+    const int zkr = zk >> p.sw_log, zkc = zk & (SW - 1);
+
+    const int xn = (n4 + DWG8_THREADS - 1) / DWG8_THREADS;                             // pieces per thread that exist at all (uniform)
+    floatx4 xr[XP], zr[8];
+    unsigned xin = 0, zin = 0;                                                         // which pieces lie inside the images
+    auto request = [&](int ho, int wo0) {
+        const int hb = ho * p.stride - p.pad, wf = wo0 * p.stride - p.pad - p.shift;
+        const int corner = hb * p.W + wf;
+        xin = 0; zin = 0;
+#pragma unroll
+        for (int k = 0; k < XP; k++) {
+            if (k < xn) {
+                const int h = hb + (xrq[k] & 0xffff), w = wf + 4 * (xrq[k] >> 16);
+                const bool in = xrq[k] >= 0 && h >= 0 && h < p.H && w >= 0 && w < p.W;
+                xr[k] = *reinterpret_cast<const floatx4*>(ximg + (in ? xoff[k] + corner : 0));
+                xin |= (in ? 1u : 0u) << k;
+            }
+        }
+        const bool zpix = wo0 + zkc < p.Wo && ho + zkr < h_end;
+        const long zpos = zpix ? (long)(ho + zkr) * p.Wo + wo0 + zkc : 0;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int o = zo + 16 * k;
+            const bool in = zpix && o0 + o < p.O;
+            zr[k] = *reinterpret_cast<const floatx4*>(zimg + (in ? (long)o * p.Ho * p.Wo + zpos : 0));
+            zin |= (in ? 1u : 0u) << k;
+        }
+    };
+    auto deposit = [&]() {
+        const half4_t zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+#pragma unroll
+        for (int k = 0; k < XP; k++) {
+            if (k < xn) {
+                const half4_t hv = {(_Float16)xr[k][0], (_Float16)xr[k][1], (_Float16)xr[k][2], (_Float16)xr[k][3]};
+                if (xrq[k] >= 0) *reinterpret_cast<half4_t*>(xs + 4 * (tid + DWG8_THREADS * k)) = (xin >> k & 1) ? hv : zero;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const half4_t hv = {(_Float16)zr[k][0], (_Float16)zr[k][1], (_Float16)zr[k][2], (_Float16)zr[k][3]};
+            *reinterpret_cast<half4_t*>(zs + (zo + 16 * k) * DWG_ZPITCH + zk) = (zin >> k & 1) ? hv : zero;
+        }
+    };
+
+    const int n_steps = (h_end - h_begin + SR - 1) / SR * segs;
+    int ho = h_begin, seg = 0;
+    if (n_steps > 0) request(ho, 0);
+    for (int step = 0; step < n_steps; step++) {
+        deposit();
+        __syncthreads();
+        {   // the next segment (the last step asks for its own again: no branch around the requests)
+            int nseg = seg + 1, nho = ho;
+            if (nseg == segs) { nseg = 0; nho += SR; }
+            if (step + 1 == n_steps) { nseg = seg; nho = ho; }
+            request(nho, nseg * SW);
+            seg = nseg; ho = nho;
+        }
+        if (wave_live) {
+            // two fragment sets: the reads of k step ks + 1 are issued before the MFMAs of step ks
+            half8_t af[2], bf[2][DWG_NB];
+            auto fragments = [&](int ks, int set) {
+                if (S1) {
+                    // (segment row) * pw and the column of the k step are even, so the parity is a_base's
+                    const int eo = a_base + ((ks * 16) >> p.sw_log) * p.pw + ((ks * 16) & (SW - 1));
+                    const unsigned* dp = reinterpret_cast<const unsigned*>(xs) + (eo >> 1);
+                    const unsigned sh = (a_base & 1) * 16;
+                    unsigned d[5];
+#pragma unroll
+                    for (int j = 0; j < 5; j++) d[j] = dp[j];
+                    union { unsigned u[4]; half8_t h; } pack;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) pack.u[j] = __builtin_amdgcn_alignbit(d[j + 1], d[j], sh);
+                    af[set] = pack.h;
+                } else {
+                    const _Float16* ap = xs + a_base + (((ks * 16) >> p.sw_log) * p.pw + ((ks * 16) & (SW - 1))) * p.stride;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) af[set][j] = ap[j * p.stride];
+                }
+#pragma unroll
+                for (int j = 0; j < DWG_NB; j++)
+                    bf[set][j] = *reinterpret_cast<const half8_t*>(zs + (j * 32 + li) * DWG_ZPITCH + ks * 16 + lh * 8);
+            };
+            fragments(0, 0);
+#pragma unroll
+            for (int ks = 0; ks < DWG_PX / 16; ks++) {
+                if (ks + 1 < DWG_PX / 16) fragments(ks + 1, (ks + 1) & 1);
+#pragma unroll
+                for (int j = 0; j < DWG_NB; j++)
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks & 1], bf[ks & 1][j], acc[j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    // accumulator (block j, register r): row 32 wave + (r >> 2) * 8 + lh * 4 + (r & 3), column 32 j + li
+    float* out = p.partial + ((((long)blockIdx.y * gridDim.z + blockIdx.z) * p.n_images + img) * p.bands + band) * (DWG8_ROWS * DWG_OT);
+    if (wave_live) {
+#pragma unroll
+        for (int j = 0; j < DWG_NB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = wave * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                out[row * DWG_OT + j * 32 + li] = acc[j][r];
+            }
+    }
+}
+
 // dW[b][(c0 + c) * taps + t][o0 + o] += the S partial regions of weight copy b, in ascending order (per-sample weights:
 // the bands of image b; shared weights: images x bands).
 __global__ __launch_bounds__(256) void conv_dwg_reduce_kernel(float* __restrict__ dW, const float* __restrict__ P, int S, int C, int O,
-                                                              int taps, int cc, int n_otiles, long group_stride_P, long group_stride_dW) {
+                                                              int taps, int cc, int n_otiles, long group_stride_P, long group_stride_dW,
+                                                              int region_rows) {
     const int chunk = blockIdx.y / n_otiles, ot = blockIdx.y % n_otiles, b = blockIdx.z;
     const int c0 = chunk * cc, o0 = ot * DWG_OT;
     const int nch = (C - c0) < cc ? (C - c0) : cc;
@@ -2427,17 +2567,36 @@ __global__ __launch_bounds__(256) void conv_dwg_reduce_kernel(float* __restrict_
     if (row >= nch * taps || o0 + col >= O) return;
     const float* src = P + (long)blockIdx.y * gridDim.z * group_stride_P + (long)b * group_stride_P + t;
     float sum = 0.f;
-    for (int s = 0; s < S; s++) sum += src[(long)s * (DWG_ROWS * DWG_OT)];
+    for (int s = 0; s < S; s++) sum += src[(long)s * region_rows * DWG_OT];
     dW[(long)b * group_stride_dW + ((long)c0 * taps + row) * O + o0 + col] += sum;
+}
+
+// Row bands per image for the weight-gradient kernels: with `units` (chunk, output tile, image) triples and `resident`
+// workgroups running at a time, the number of bands that minimises rounds x (segments of a band + the cost of a
+// workgroup's result stores, in segment times). More bands even the rounds out, fewer keep the partial sums small.
+static int dwg_pick_bands(long units, long resident, long row_steps, long segs, double store_cost) {
+    int best = 1;
+    double best_cost = 1e300;
+    const long max_bands = row_steps < 64 ? row_steps : 64;
+    for (long b = 1; b <= max_bands; b++) {
+        const long steps = (row_steps + b - 1) / b;                   // row steps of the largest band
+        const long bands = (row_steps + steps - 1) / steps;
+        if (bands != b) continue;                                     // the same split as a smaller count
+        const long rounds = (units * bands + resident - 1) / resident;
+        const double cost = (double)rounds * ((double)steps * (double)segs + store_cost);
+        if (cost < best_cost - 1e-9) { best_cost = cost; best = (int)b; }
+    }
+    return best;
 }
 
 static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W, size_t O,
                            size_t K_h, size_t K_w, size_t stride, size_t pad, bool shared, hipStream_t s) {
     const size_t taps = K_h * K_w;
     const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
-    int cc = (int)(DWG_ROWS / taps);
-    if (cc > (int)C) cc = (int)C;
     const bool vec = W % 4 == 0 && Wo % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0;
+    const int region_rows = vec ? DWG8_ROWS : DWG_ROWS;
+    int cc = (int)(region_rows / taps);
+    if (cc > (int)C) cc = (int)C;
     // vector path: the staged window starts at a multiple of four columns, `shift` columns left of the first one needed
     // (128 * stride is a multiple of 4, so the shift is the same for every segment)
     const int shift = vec ? (int)(((4 - (long)(pad % 4)) % 4 + 4) % 4) : 0;
@@ -2447,43 +2606,52 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     const int span = (int)((SR - 1) * stride + K_h);
     int pw = (int)((SW - 1) * stride + K_w) + shift;
     pw = vec ? (pw + 3) / 4 * 4 : (pw | 1);                           // scalar path: odd, rows start on different banks
-    // staged input rows + dy segment must fit the 64 KiB a workgroup may take without crowding out its neighbours
-    while (cc > 1 && ((size_t)cc * span * pw + 8) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2 > 64 * 1024) cc--;
+    // staged input rows + dy segment: at most 64 KiB for the four-wave kernel (two workgroups share a CU), 96 KiB and
+    // DWG8_XMAX 16-byte pieces per thread for the eight-wave one
+    const size_t lds_limit = vec ? 96 * 1024 : 64 * 1024;
+    auto too_big = [&](int c) {
+        if (((size_t)c * span * pw + 8) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2 > lds_limit) return true;
+        return vec && (size_t)c * span * (pw / 4) > (size_t)DWG8_THREADS * DWG8_XMAX;
+    };
+    while (cc > 1 && too_big(cc)) cc--;
+    if (too_big(cc)) return NZHIP_E_UNSUPPORTED;
+    if (vec && (size_t)cc * H * W + (size_t)(stride * DWG_PX + K_h) * W >= 0x7fffffffull) return NZHIP_E_UNSUPPORTED;   // int offsets in the kernel
     const size_t lds_bytes = (((size_t)cc * span * pw + 7) & ~(size_t)7) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2;
-    if (lds_bytes > 64 * 1024) return NZHIP_E_UNSUPPORTED;
     const int chunks = (int)((C + cc - 1) / cc), otiles = (int)((O + DWG_OT - 1) / DWG_OT);
     if (chunks > 65535 || otiles > 65535) return NZHIP_E_UNSUPPORTED;
-    // about four workgroups per CU in total; a band is a whole number of output rows of one image
+    // a band is a whole number of segment rows of one image
     const long units = (long)chunks * otiles * (long)N;
-    long want = (4L * device_cu_count() + units - 1) / units;
-    if (want < 1) want = 1;
-    if (want > (long)Ho) want = (long)Ho;
-    int band_rows = (int)((Ho + want - 1) / want);
-    band_rows = (band_rows + SR - 1) / SR * SR;                       // whole segments: a segment never straddles two bands
+    const long row_steps = ((long)Ho + SR - 1) / SR, segs = ((long)Wo + SW - 1) / SW;
+    const long resident = (long)device_cu_count() * (vec ? 1 : 2);
+    const int want = dwg_pick_bands(units, resident, row_steps, segs, vec ? 3.0 : 1.0);
+    const int band_rows = (int)((row_steps + want - 1) / want) * SR;
     const int bands = (int)((Ho + band_rows - 1) / band_rows);
     if (N * (size_t)bands > 0x7fffffffull) return NZHIP_E_UNSUPPORTED;
     const size_t regions = (size_t)chunks * otiles * N * bands;
     float* partial = nullptr;
-    if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), regions * DWG_ROWS * DWG_OT * sizeof(float), s)) return rc;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), regions * region_rows * DWG_OT * sizeof(float), s)) return rc;
     ConvDwGenArgs a;
     a.x = x; a.dy = dy; a.partial = partial;
     a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.Ho = (int)Ho; a.Wo = (int)Wo;
     a.Kh = (int)K_h; a.Kw = (int)K_w; a.stride = (int)stride; a.pad = (int)pad;
     a.cc = cc; a.pw = pw; a.shift = shift; a.sw_log = sw_log; a.span = span; a.bands = bands; a.band_rows = band_rows; a.n_images = (int)N;
-    auto kfn = vec ? conv_dwg_kernel<true> : conv_dwg_kernel<false>;
+    const size_t x_pieces = ((size_t)cc * span * (pw / 4) + DWG8_THREADS - 1) / DWG8_THREADS;
+    auto kfn = !vec ? conv_dwg_kernel
+               : stride == 1 ? (x_pieces <= 4 ? conv_dwg8_kernel<4, true> : conv_dwg8_kernel<DWG8_XMAX, true>)
+                             : (x_pieces <= 4 ? conv_dwg8_kernel<4, false> : conv_dwg8_kernel<DWG8_XMAX, false>);
     int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(conv_dwg)");
     if (rc == NZHIP_OK) {
-        hipLaunchKernelGGL(kfn, dim3((unsigned)(N * bands), (unsigned)chunks, (unsigned)otiles), dim3(256), lds_bytes, s, a);
+        hipLaunchKernelGGL(kfn, dim3((unsigned)(N * bands), (unsigned)chunks, (unsigned)otiles), dim3(vec ? DWG8_THREADS : 256), lds_bytes, s, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg kernel launch");
     }
     if (rc == NZHIP_OK) {
         const int S = shared ? (int)(N * bands) : bands, groups = shared ? 1 : (int)N;
-        const long per_group = (long)S * DWG_ROWS * DWG_OT;
+        const long per_group = (long)S * region_rows * DWG_OT;
         // partial regions of one (chunk, o_tile) are contiguous: [image][band]; a weight copy's regions start at b * S
-        dim3 grid((unsigned)((DWG_ROWS * DWG_OT + 255) / 256), (unsigned)(chunks * otiles), (unsigned)groups);
+        dim3 grid((unsigned)((region_rows * DWG_OT + 255) / 256), (unsigned)(chunks * otiles), (unsigned)groups);
         hipLaunchKernelGGL(conv_dwg_reduce_kernel, grid, dim3(256), 0, s, dw, partial, S, (int)C, (int)O, (int)taps, cc, otiles,
-                           per_group, (long)(C * taps * O));
+                           per_group, (long)(C * taps * O), region_rows);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg_reduce kernel launch");
     }

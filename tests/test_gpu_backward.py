@@ -325,7 +325,10 @@ CONV_GEN_BWD_W = [  # N, C, H, W, O, Kh, Kw, stride, pad, w_batch: every geometr
     (2, 3, 9, 8, 4, 3, 3, 2, 1, 1), (1, 2, 11, 13, 3, 5, 5, 1, 2, 1), (2, 2, 10, 9, 2, 5, 3, 2, 0, 2), (1, 3, 12, 12, 2, 7, 7, 3, 3, 1),
     (3, 1, 6, 7, 5, 2, 4, 1, 1, 3), (2, 20, 16, 300, 70, 5, 5, 1, 2, 1),      # several 128-pixel segments per row, two o tiles, 4 chunks
     (2, 40, 33, 37, 100, 3, 3, 2, 1, 1), (2, 7, 20, 20, 9, 3, 3, 1, 0, 1), (1, 5, 40, 260, 6, 3, 3, 4, 2, 1), (2, 3, 30, 30, 3, 11, 11, 4, 5, 2),
-    (1, 130, 12, 12, 8, 1, 1, 2, 0, 1), (2, 6, 40, 50, 5, 3, 3, 1, 0, 1), (1, 4, 70, 64, 130, 5, 5, 1, 2, 1)]   # segment widths 64 and (two rows of) 64
+    (1, 130, 12, 12, 8, 1, 1, 2, 0, 1), (2, 6, 40, 50, 5, 3, 3, 1, 0, 1), (1, 4, 70, 64, 130, 5, 5, 1, 2, 1),   # segment widths 64 and (two rows of) 64
+    # rows that allow 16-byte loads (the eight-wave kernel): stride 2 with seven pieces of input rows per thread and two chunks,
+    # per-sample weights, stride 2 over three segments per row, stride 1 with seven pieces per thread
+    (2, 40, 32, 64, 100, 3, 3, 2, 1, 1), (2, 6, 16, 16, 5, 5, 5, 1, 2, 2), (1, 8, 12, 520, 12, 3, 3, 2, 1, 1), (1, 70, 10, 128, 8, 2, 1, 1, 0, 1)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", CONV_GEN_BWD_W)
