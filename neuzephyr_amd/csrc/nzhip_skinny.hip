@@ -129,6 +129,88 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const SkinnyArgs p) 
     }
 }
 
+// ---- KL, whole contraction in one workgroup -------------------------------------------------------
+// For one long, wide L (a GEMV against a 4096 x 4096 matrix): a workgroup owns 16 adjacent columns l and the
+// WHOLE contraction, so no partial sums leave the chip and no second kernel runs. Eight waves; a thread owns
+// four columns (lane & 3) of the rows k = (tid >> 2) + 128 j, so a wave load is sixteen 64-byte row pieces; the
+// neighbour workgroup that uses the other half of those 128-byte lines runs on the same XCD (workgroups are
+// dealt to the XCDs round-robin, so workgroup i takes column group (i % 8) * (G / 8) + i / 8) and finds them in
+// its L2. A thread keeps two sets of U loads in flight (8 waves x 2 U KiB per CU). The 128 row lanes are folded
+// through LDS in a fixed order.
+constexpr int KLC_COLS = 16, KLC_ROWS = 128, KLC_THREADS = 512, KLC_U = 8;
+
+template <int SR>
+__global__ __launch_bounds__(KLC_THREADS) void skinny_kl_cols_kernel(const SkinnyArgs p) {
+    __shared__ float red[SR][KLC_ROWS][KLC_COLS + 1];
+    const int tid = threadIdx.x, q = tid & 3, rl = tid >> 2;
+    const int G = gridDim.x;
+    const int g = (G % 8 == 0) ? (blockIdx.x % 8) * (G / 8) + blockIdx.x / 8 : blockIdx.x;
+    const int l0 = g * KLC_COLS + q * 4;
+    const float* __restrict__ S = p.S;
+    const float* __restrict__ Lp = p.L + l0;
+
+    float acc[SR][4];
+#pragma unroll
+    for (int s = 0; s < SR; s++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[s][e] = 0.f;
+
+    // two register sets: the loads of chunk c + 1 are issued before chunk c is added up
+    floatx4 v[2][KLC_U];
+    float a[2][SR][KLC_U];
+    auto request = [&](int kb, int set) {
+#pragma unroll
+        for (int u = 0; u < KLC_U; u++) {
+            const int k = kb + KLC_ROWS * u;
+            const int kc = k < p.K ? k : rl;                                   // clamped: a row this thread owns anyway
+            v[set][u] = *reinterpret_cast<const floatx4*>(Lp + (long)kc * p.ldl);
+#pragma unroll
+            for (int s = 0; s < SR; s++) a[set][s][u] = S[s * p.s_ss + kc * p.s_sk];
+        }
+    };
+    auto add_up = [&](int kb, int set) {
+#pragma unroll
+        for (int u = 0; u < KLC_U; u++) {
+            const bool live = kb + KLC_ROWS * u < p.K;
+#pragma unroll
+            for (int s = 0; s < SR; s++) {
+                const float as = live ? rnd16(a[set][s][u]) : 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[s][e] = __builtin_fmaf(as, rnd16(v[set][u][e]), acc[s][e]);
+            }
+        }
+    };
+    constexpr int STEP = KLC_ROWS * KLC_U;
+    request(rl, 0);
+    for (int kb = rl; kb < p.K; kb += 2 * STEP) {
+        request(kb + STEP, 1);                                                 // past the end: clamped loads, nothing added
+        add_up(kb, 0);
+        request(kb + 2 * STEP, 0);
+        add_up(kb + STEP, 1);
+    }
+#pragma unroll
+    for (int s = 0; s < SR; s++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) red[s][rl][q * 4 + e] = acc[s][e];
+    __syncthreads();
+    // output (s, c): eight lanes add sixteen row lanes each, ascending, then fold 8 -> 1 in a fixed tree
+    if (tid < SR * KLC_COLS * 8) {
+        const int part = tid & 7, oc = tid >> 3, s = oc / KLC_COLS, c = oc % KLC_COLS;
+        float x = 0.f;
+#pragma unroll
+        for (int r = 0; r < KLC_ROWS / 8; r++) x += red[s][part * (KLC_ROWS / 8) + r][c];
+        x += __shfl_xor(x, 1);
+        x += __shfl_xor(x, 2);
+        x += __shfl_xor(x, 4);
+        if (part == 0) {
+            const int l = g * KLC_COLS + c;
+            if (p.bias) x += p.bias[s * p.b_ss + l * p.b_sl];
+            if (p.relu) x = x > 0.f ? x : 0.f;
+            p.out[s * p.o_ss + l * p.o_sl] = x;
+        }
+    }
+}
+
 // ---- LK: rows of L are dot products ------------------------------------------------------------
 template <int SR>
 __global__ __launch_bounds__(256) void skinny_lk_kernel(const SkinnyArgs p) {
@@ -276,7 +358,15 @@ int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream) {
     const int sr_t = p.SR <= 1 ? 1 : (p.SR <= 2 ? 2 : (p.SR <= 4 ? 4 : 8));
     int rc = NZHIP_OK;
     float* partial = nullptr;
-    if (l_is_kl) {
+    static const char* klc_env = getenv("NZHIP_SKINNY_COLS");           // benchmarking only: 0 keeps the split-contraction kernels
+    const bool klc_on = !klc_env || atoi(klc_env) != 0;
+    if (l_is_kl && klc_on && batch == 1 && p.SR <= 2 && p.vec && p.LN % KLC_COLS == 0 && p.LN >= 128 * KLC_COLS && p.K >= 1024 &&
+        (long)p.K * p.ldl < 0x7fffffffL) {
+        // enough column groups to occupy the chip, a contraction long enough to stream: one kernel, no partial sums
+        dim3 grid((unsigned)(p.LN / KLC_COLS));
+        if (sr_t == 1) hipLaunchKernelGGL(skinny_kl_cols_kernel<1>, grid, dim3(KLC_THREADS), 0, stream, p);
+        else hipLaunchKernelGGL(skinny_kl_cols_kernel<2>, grid, dim3(KLC_THREADS), 0, stream, p);
+    } else if (l_is_kl) {
         const unsigned lblocks = (unsigned)((p.LN + 255) / 256);
         // split k until ~4 blocks per CU are in flight, keeping at least 64 k per block
         int ksplit = (int)(1024 / ((long)lblocks * batch));

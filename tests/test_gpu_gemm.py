@@ -76,7 +76,10 @@ def test_integer_operands_are_bit_exact(nz, M, K, N, a_trans, b_trans, tile):
 
 
 SKINNY = [(1, 1, 1), (1, 4096, 64), (1, 777, 513), (3, 300, 1000), (8, 64, 260), (5, 1000, 7), (1000, 77, 3),
-          (300, 40, 1), (2049, 130, 8), (7, 9, 4100), (1, 5, 3)]
+          (300, 40, 1), (2049, 130, 8), (7, 9, 4100), (1, 5, 3),
+          # long and wide enough for the kernel that keeps the whole contraction in one workgroup (when the long
+          # operand has its long extent contiguous): K a multiple of its row step and not, one and two skinny rows
+          (1, 4096, 4096), (2, 1500, 2064), (2048, 1100, 2), (4096, 1024, 1)]
 
 
 @pytest.mark.parametrize("M,K,N", SKINNY)
