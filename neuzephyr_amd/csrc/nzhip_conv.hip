@@ -1498,7 +1498,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                     hipError_t e = hipGetLastError();
                     if (e != hipSuccess) rc = set_hip_error(e, "conv3x3_resident_db kernel launch");
                 }
-                int rc2 = image_release(lease, s);
+                int rc2 = image_release(lease, s, rc == NZHIP_OK);
                 return rc ? rc : rc2;
             };
             if (n_chunks == 2) return run(std::integral_constant<int, 2>{});
@@ -1556,7 +1556,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                 hipError_t e = hipGetLastError();
                 if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm_resident kernel launch");
             }
-            int rc2 = image_release(lease, s);
+            int rc2 = image_release(lease, s, rc == NZHIP_OK);
             return rc ? rc : rc2;
         }
     }
@@ -1609,7 +1609,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm kernel launch");
         }
     }
-    int rc2 = image_release(lease, s);
+    int rc2 = image_release(lease, s, rc == NZHIP_OK);
     return rc ? rc : rc2;
 }
 

@@ -1283,7 +1283,7 @@ int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t s, int waves, int mf
         }
     }
     int rc2 = workspace_free(Ah, s);
-    const int rc3 = image_release(b_lease, s);
+    const int rc3 = image_release(b_lease, s, rc == NZHIP_OK);
     if (!rc2) rc2 = rc3;
     return rc ? rc : rc2;
 }

@@ -63,10 +63,13 @@ constexpr int PREPARED_KEY_WORDS = 12;
 struct ImageLease {
     void* ptr = nullptr;
     bool fill = true;           // the caller must (re)build the image
-    bool persistent = false;    // owned by a handle: image_release leaves it alone
+    bool persistent = false;    // owned by a handle: image_release leaves the memory alone
+    void* owner = nullptr;      // that handle
 };
 int image_acquire(int kind, const uint64_t key[PREPARED_KEY_WORDS], size_t bytes, hipStream_t s, ImageLease* out);
-int image_release(const ImageLease& lease, hipStream_t s);
+// `enqueued`: every launch between acquire and release went through. A handle whose image was to be rebuilt under this
+// lease is only then marked as holding it; otherwise the next call rebuilds.
+int image_release(const ImageLease& lease, hipStream_t s, bool enqueued);
 
 // Compute units of the current device (queried once per device, then cached).
 int device_cu_count();

@@ -186,16 +186,25 @@ int image_acquire(int kind, const uint64_t key[PREPARED_KEY_WORDS], size_t bytes
     }
     h->bytes = bytes;
     memcpy(h->key, key, sizeof(h->key));
-    h->valid = true;
-    h->fills++;
+    h->valid = false;                               // until the release says that the image was built
     out->ptr = h->image;
     out->fill = true;
+    out->owner = h;
     return NZHIP_OK;
 }
 
-int image_release(const ImageLease& lease, hipStream_t s) {
-    if (lease.persistent || !lease.ptr) return NZHIP_OK;
-    return workspace_free(lease.ptr, s);
+int image_release(const ImageLease& lease, hipStream_t s, bool enqueued) {
+    if (!lease.ptr) return NZHIP_OK;
+    if (!lease.persistent) return workspace_free(lease.ptr, s);
+    if (lease.fill && lease.owner) {
+        nzhip_prepared* h = static_cast<nzhip_prepared*>(lease.owner);
+        std::lock_guard<std::mutex> lock(h->mu);
+        if (enqueued && h->image == lease.ptr) {
+            h->valid = true;
+            h->fills++;
+        }
+    }
+    return NZHIP_OK;
 }
 
 int device_cu_count() {
