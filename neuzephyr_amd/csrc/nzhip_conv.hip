@@ -2131,9 +2131,27 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
         few_patches = !resident && units * 4 <= (size_t)device_cu_count();
     }
     if (!force_ws && !few_patches && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL) {
+        // The reference's bias parameter is pixel-major ([1,1,H_out*W_out,O], src/Model.cu:252-256), while the kernels'
+        // lanes are adjacent pixels: read as it lies, every bias load touches 64 lines 4 O bytes apart. One pass turns it
+        // into channel planes (the layout of y), and the bias loads look like the result stores.
+        const float* bias_use = bias;
+        int64_t bsp = bias_stride_pixel, bsc = bias_stride_channel;
+        float* bias_planes = nullptr;
+        if (bias && bias_stride_image == 0 && bsc == 1 && bsp == (int64_t)O && O >= 8 && H_out * W_out >= 64) {
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&bias_planes), O * H_out * W_out * sizeof(float), s)) return rc;
+            if (int rc = nzhip_col2im(bias_planes, bias, H_out, W_out, O, 1, s)) {
+                workspace_free(bias_planes, s);
+                return rc;
+            }
+            bias_use = bias_planes; bsp = 1; bsc = (int64_t)(H_out * W_out);
+        }
+        auto finish = [&](int rc) {
+            const int rc2 = bias_planes ? workspace_free(bias_planes, s) : NZHIP_OK;
+            return rc ? rc : rc2;
+        };
 #define NZHIP_IG(KH_, TW_, BN_)                                                                                      \
-    return conv_igemm_launch<KH_, KH_, TW_, BN_>(y, x, w_ref, bias, N, C, H, W, O, pad, w_batch, bias_stride_pixel, \
-                                                 bias_stride_channel, bias_stride_image, activation, H_out, W_out, s)
+    return finish(conv_igemm_launch<KH_, KH_, TW_, BN_>(y, x, w_ref, bias_use, N, C, H, W, O, pad, w_batch, bsp, bsc, \
+                                                        bias_stride_image, activation, H_out, W_out, s))
         if (K_h == 3) {
             if (wide && bn128) NZHIP_IG(3, 64, 128);
             if (wide) NZHIP_IG(3, 64, 64);
