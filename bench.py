@@ -762,10 +762,10 @@ def main():
             import subprocess
             try:
                 out = subprocess.run([exe, "200", "20"], capture_output=True, text=True, timeout=120)
-                extra["layers_through_model_forward"] = (json.loads(out.stdout.strip().splitlines()[-1]) if out.returncode == 0
+                extra["layers_through_model"] = (json.loads(out.stdout.strip().splitlines()[-1]) if out.returncode == 0
                                                          else {"error": out.stderr[-300:]})
             except (subprocess.TimeoutExpired, ValueError, IndexError) as e:
-                extra["layers_through_model_forward"] = {"error": str(e)[:300]}
+                extra["layers_through_model"] = {"error": str(e)[:300]}
 
     ceilings = None
     if args.workload == "gemm8192" and not args.no_extra:

@@ -243,6 +243,10 @@ int nzhip_conv2d_backward_weights(float* dw, const float* x, const float* dy, si
 int nzhip_add_broadcast(float* out, const float* a, const float* b, const size_t shapeOut[4],
                         const size_t shapeA[4], const size_t shapeB[4], void* stream);
 
+/* Tensor::fill (src/Tensor.cu:306-314 -> krnl::Fill, FillKernel, src/OperationKernels.cu:1146-1156):
+ * data[0, n) = value, on the device (OutputNode::backward seeds the output gradient with it, src/Nodes.cu:62-66). */
+int nzhip_fill(float* data, float value, size_t n, void* stream);
+
 /* nz::data::iRELU (TensorOperations.cuh:19; RectifiedLinearUnitKernel, OperationKernels.cu:230-235). */
 int nzhip_relu(float* out, const float* in, size_t n, void* stream);
 

@@ -18,7 +18,7 @@ EXPORTS = [
     "nzhip_version", "nzhip_last_error", "nzhip_device_info", "nzhip_gemm", "nzhip_gemm_static",
     "nzhip_static_scratch_bytes", "nzhip_gemm_force_tile", "nzhip_gemm_coop_timeouts", "nzhip_gemm_coop_reset", "nzhip_gemm_coop_test_mode", "nzhip_probe_mfma", "nzhip_probe_copy", "nzhip_prepared_create", "nzhip_prepared_invalidate", "nzhip_prepared_fills",
     "nzhip_prepared_destroy", "nzhip_gemm_prepared_b", "nzhip_conv2d_forward_prepared", "nzhip_tensorcore_gemm",
-    "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu",
+    "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu", "nzhip_fill",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
     "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
@@ -94,6 +94,7 @@ def load() -> C.CDLL:
     lib.nzhip_conv2d_backward_weights.argtypes = [vp, vp, vp] + [sz] * 10 + [vp]
     lib.nzhip_add_broadcast.argtypes = [vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_relu.argtypes = [vp, vp, sz, vp]
+    lib.nzhip_fill.argtypes = [vp, C.c_float, sz, vp]
     lib.nzhip_gemm_backward.argtypes = [vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_matmul_backward.argtypes = [vp, vp, vp, vp, vp, shape, shape, shape, vp]
     lib.nzhip_relu_backward.argtypes = [vp, vp, vp, sz, vp]
@@ -320,6 +321,12 @@ def add_broadcast(a, b, stream=None):
     check(lib.nzhip_add_broadcast(_dev(out), _dev(a), _dev(b), shape4(so), shape4(a.shape), shape4(b.shape),
                                   _stream_handle(stream)))
     return out
+
+
+def fill(a, value, stream=None):
+    lib = load()
+    check(lib.nzhip_fill(_dev(a), float(value), a.numel(), _stream_handle(stream)))
+    return a
 
 
 def relu(a, stream=None):

@@ -218,6 +218,70 @@ __global__ __launch_bounds__(256) void grad_reduce_kernel(float* __restrict__ di
     *dst = acc;
 }
 
+// The same sum when hundreds of members map onto one element (the bias of a Linear layer: one vector against a batch
+// of thousands): a chain of that length in one thread is a millisecond of load latency. The members are cut into chunks;
+// a thread adds one chunk in ascending order, eight loads in flight, into a partial sum, and a second kernel adds the
+// partial sums onto din in ascending chunk order. Fixed order, but not the single chain of the kernel above, so it is
+// used only from GRAD_CHUNK_MIN members on. Members of one element are `stride` floats apart.
+constexpr int GRAD_CHUNK_MIN = 128;
+
+__global__ __launch_bounds__(256) void grad_partial_kernel(float* __restrict__ partial, const float* __restrict__ dout, long hw,
+                                                           int in_n, int in_c, int out_n, int out_c, int chunk) {
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= hw) return;
+    const int i0 = blockIdx.y / in_c, j0 = blockIdx.y % in_c;
+    // members in ascending (n, c): n and c both broadcast -> consecutive planes; only c -> the planes of image i0;
+    // only n -> plane j0 of every image
+    const long members = (in_n > 1 ? 1L : out_n) * (in_c > 1 ? 1L : out_c);
+    const long first = ((long)(in_n > 1 ? i0 : 0) * out_c + (in_c > 1 ? j0 : 0)) * hw;
+    const long stride = (in_c > 1 ? (long)out_c : 1L) * hw;
+    const long m_lo = (long)blockIdx.z * chunk, m_hi = m_lo + chunk < members ? m_lo + chunk : members;
+    const float* src = dout + first + m_lo * stride + t;
+    float acc = 0.f;
+    long m = m_lo;
+    for (; m + 8 <= m_hi; m += 8, src += 8 * stride) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = src[u * stride];
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc += v[u];
+    }
+    for (; m < m_hi; m++, src += stride) acc += *src;
+    partial[((long)blockIdx.y * gridDim.z + blockIdx.z) * hw + t] = acc;
+}
+
+__global__ __launch_bounds__(256) void grad_partial_sum_kernel(float* __restrict__ din, const float* __restrict__ partial, long hw,
+                                                               int chunks) {
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= hw) return;
+    float acc = din[(long)blockIdx.y * hw + t];
+    const float* src = partial + (long)blockIdx.y * chunks * hw + t;
+    int p = 0;
+    for (; p + 8 <= chunks; p += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = src[(long)(p + u) * hw];
+#pragma unroll
+        for (int u = 0; u < 8; u++) acc += v[u];
+    }
+    for (; p < chunks; p++) acc += src[(long)p * hw];
+    din[(long)blockIdx.y * hw + t] = acc;
+}
+
+__global__ __launch_bounds__(256) void fill_kernel(float* __restrict__ data, float value, long n, int vec) {
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec) {
+        if (t * 4 + 3 < n) {
+            const floatx4 v = {value, value, value, value};
+            reinterpret_cast<floatx4*>(data)[t] = v;
+        } else {
+            for (long k = t * 4; k < n; k++) data[k] = value;
+        }
+    } else if (t < n) {
+        data[t] = value;
+    }
+}
+
 // img2colBackwardKernel (src/OperationKernels.cu:1337-1355) as a gather: one thread owns one image
 // gradient element and adds the column-matrix gradient entries that were copied from it, in
 // ascending pixel order (the order in which the reference's element index visits them); no atomics.
@@ -687,6 +751,16 @@ int nzhip_add_broadcast(float* out, const float* a, const float* b, const size_t
     return check_launch("add_bcast_kernel");
 }
 
+int nzhip_fill(float* data, float value, size_t n, void* stream) {
+    if (!data && n) return set_error(NZHIP_E_INVALID, "nzhip_fill: null pointer");
+    if (n == 0) return NZHIP_OK;
+    const int vec = aligned16(data);
+    const size_t threads = vec ? (n + 3) / 4 : n;
+    if ((threads + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_fill: more than 2^39 elements");
+    hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, as_stream(stream), data, value, (long)n, vec);
+    return check_launch("fill_kernel");
+}
+
 int nzhip_relu(float* out, const float* in, size_t n, void* stream) {
     if ((!out || !in) && n) return set_error(NZHIP_E_INVALID, "nzhip_relu: null pointer");
     if (n == 0) return NZHIP_OK;
@@ -873,6 +947,30 @@ int nzhip_add_backward(float* din, const float* dout, const size_t sIn[4], const
     if (sIn[0] * sIn[1] > 65535 || sOut[0] > 0x7fffffff || sOut[1] > 0x7fffffff)
         return set_error(NZHIP_E_UNSUPPORTED, "nzhip_add_backward: more than 65535 (n,c) planes");
     dim3 grid((unsigned)((hw + 255) / 256), (unsigned)(sIn[0] * sIn[1]));
+    const size_t members = (sIn[0] > 1 ? 1 : sOut[0]) * (sIn[1] > 1 ? 1 : sOut[1]);
+    if (members >= (size_t)GRAD_CHUNK_MIN) {
+        // enough chunks to put every CU to work, at least 16 members each
+        const size_t threads = hw * sIn[0] * sIn[1];
+        size_t chunks = ((size_t)device_cu_count() * 1024 + threads - 1) / threads;
+        if (chunks > members / 16) chunks = members / 16;
+        if (chunks > 1024) chunks = 1024;
+        if (chunks >= 2) {
+            const int chunk = (int)((members + chunks - 1) / chunks);
+            chunks = (members + chunk - 1) / chunk;
+            float* partial = nullptr;
+            hipStream_t s = as_stream(stream);
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), chunks * threads * sizeof(float), s)) return rc;
+            hipLaunchKernelGGL(grad_partial_kernel, dim3(grid.x, grid.y, (unsigned)chunks), dim3(256), 0, s, partial, dout, (long)hw,
+                               (int)sIn[0], (int)sIn[1], (int)sOut[0], (int)sOut[1], chunk);
+            int rc = check_launch("grad_partial_kernel");
+            if (rc == NZHIP_OK) {
+                hipLaunchKernelGGL(grad_partial_sum_kernel, grid, dim3(256), 0, s, din, partial, (long)hw, (int)chunks);
+                rc = check_launch("grad_partial_sum_kernel");
+            }
+            const int rc2 = workspace_free(partial, s);
+            return rc ? rc : rc2;
+        }
+    }
     hipLaunchKernelGGL(grad_reduce_kernel, grid, dim3(256), 0, as_stream(stream), din, dout, (long)hw, (int)sIn[0],
                        (int)sIn[1], (int)sOut[0], (int)sOut[1]);
     return check_launch("grad_reduce_kernel");

@@ -176,8 +176,8 @@ namespace nz::data {
 
     void Tensor::fill(const value_type value, const bool isGrad) const {
         if (_size == 0) return;
-        std::vector<value_type> host(_size, value);
-        NZ_CHECK(nzhip_memcpy_h2d(isGrad ? grad() : data(), host.data(), _size * sizeof(value_type)));
+        // on the device, like the reference's Fill kernel: OutputNode::backward fills the whole output gradient on every pass
+        NZ_CHECK(nzhip_fill(isGrad ? gradOverwrite() : data(), value, _size, nzhip_default_stream()));
     }
 
     void Tensor::randomize(const unsigned long long seed) const {

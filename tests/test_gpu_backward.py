@@ -155,6 +155,36 @@ def test_add_backward_bit_exact(nz, oracle):
         nz.add_backward(dev(np.zeros((2, 1, 3, 3))), dev(np.zeros((3, 1, 3, 3))))
 
 
+def test_add_backward_with_hundreds_of_members_per_element(nz, oracle):
+    # a Linear layer's bias against a batch of thousands: the members are added in chunks (fixed order, not the single
+    # ascending chain of the oracle): exact on integers, a few ulp on floats, the same bits on every run
+    rng = np.random.default_rng(31)
+    for s_in, s_out in [((1, 1, 300, 1), (1000, 1, 300, 1)), ((1, 1, 50, 3), (20, 9, 50, 3)), ((1, 3, 70, 1), (400, 3, 70, 1)),
+                        ((2, 1, 33, 2), (2, 130, 33, 2))]:
+        din0, dout = ints(rng, s_in, -9, 10), ints(rng, s_out, -9, 10)
+        assert np.array_equal(host(nz.add_backward(dev(din0), dev(dout))), oracle.add_backward(din0, dout)), (s_in, s_out)
+    din0 = rng.standard_normal((1, 1, 300, 1)).astype(np.float32)
+    dout = rng.standard_normal((1000, 1, 300, 1)).astype(np.float32)
+    a = host(nz.add_backward(dev(din0), dev(dout)))
+    b = host(nz.add_backward(dev(din0), dev(dout)))
+    assert np.array_equal(a, b)
+    truth = din0.astype(np.float64) + dout.astype(np.float64).sum(axis=0, keepdims=True)
+    assert np.abs(a - truth).max() <= 1e-5 * np.abs(dout).sum(axis=0).max()
+
+
+def test_fill_writes_every_element(nz):
+    import torch
+    for n in (1, 3, 4, 1023, 4096, 100003):
+        t = torch.full((n + 9,), 7.0, device="cuda")
+        nz.fill(t[4:4 + n], -2.5)                      # 16-byte aligned start
+        want = np.full(n + 9, 7.0, np.float32); want[4:4 + n] = -2.5
+        assert np.array_equal(host(t), want)
+        t = torch.full((n + 9,), 7.0, device="cuda")
+        nz.fill(t[1:1 + n], 0.125)                     # unaligned start
+        want = np.full(n + 9, 7.0, np.float32); want[1:1 + n] = 0.125
+        assert np.array_equal(host(t), want)
+
+
 IM2COL_CASES = [((2, 3, 4, 5), 3, 3, 1, 1), ((1, 1, 1, 1), 1, 1, 1, 0), ((2, 2, 7, 6), 3, 2, 2, 0),
                 ((1, 3, 8, 9), 2, 4, 2, 2), ((3, 1, 5, 5), 5, 5, 1, 2), ((2, 4, 6, 6), 1, 1, 3, 0),
                 ((2, 5, 33, 47), 3, 3, 1, 1), ((1, 2, 9, 9), 3, 3, 3, 1)]
