@@ -2227,6 +2227,81 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     return rc ? rc : (rc2 ? rc2 : rc3);
 }
 
+namespace nzhip {
+
+// The same tile with 16-byte accesses (HW a multiple of 4, 16-byte aligned tensors): a thread owns four adjacent pixels
+// of channels oc and oc + 16, every element still one chain over ascending n (the same sums, bit for bit); two images'
+// loads are in flight at a time.
+template <bool MASK>
+__global__ __launch_bounds__(256) void conv_bias_grad_vec_kernel(float* __restrict__ dbias, const float* __restrict__ dz, int N,
+                                                                 int O, long HW, float* __restrict__ dz_out,
+                                                                 const float* __restrict__ y) {
+    __shared__ float tile[64][33];                               // [pixel][channel]
+    const long p0 = (long)blockIdx.x * 64;
+    const int o0 = blockIdx.y * 32;
+    {
+        const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+        for (int r = 0; r < 64; r += 8) {
+            const long p = p0 + ty + r;
+            const int o = o0 + tx;
+            tile[ty + r][tx] = (p < HW && o < O) ? dbias[p * O + o] : 0.f;
+        }
+    }
+    __syncthreads();
+    const int pq = threadIdx.x & 15, oc = threadIdx.x >> 4;      // pixels 4 pq .. 4 pq + 3, channels oc and oc + 16
+    const long p = p0 + 4 * pq;
+    float acc[2][4];
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[h][e] = tile[4 * pq + e][oc + 16 * h];
+    if (p < HW) {                                                // HW % 4 == 0: the four pixels are inside together
+        const bool live[2] = {o0 + oc < O, o0 + oc + 16 < O};
+        const long plane = HW, image = (long)O * HW;
+        const long at0 = (long)(o0 + oc) * plane + p;
+        auto step = [&](const int n) {
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                if (live[h]) {
+                    const long at = (long)n * image + at0 + (long)h * 16 * plane;
+                    floatx4 g = *reinterpret_cast<const floatx4*>(dz + at);
+                    if (MASK) {
+                        const floatx4 yy = *reinterpret_cast<const floatx4*>(y + at);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) g[e] = yy[e] > 0.f ? g[e] : 0.f;
+                        *reinterpret_cast<floatx4*>(dz_out + at) = g;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[h][e] += g[e];
+                }
+        };
+        int n = 0;
+        for (; n + 2 <= N; n += 2) {
+            step(n);
+            step(n + 1);
+        }
+        if (n < N) step(n);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) tile[4 * pq + e][oc + 16 * h] = acc[h][e];
+    __syncthreads();
+    {
+        const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+        for (int r = 0; r < 64; r += 8) {
+            const long pp = p0 + ty + r;
+            const int o = o0 + tx;
+            if (pp < HW && o < O) dbias[pp * O + o] = tile[ty + r][tx];
+        }
+    }
+}
+
+}  // namespace nzhip
+
 /* Gradient of the reference's Conv2d bias parameter ([1,1,H_out*W_out,O], added to the matmul result before
  * Col2Img): dbias[p][o] += sum over n of dz[n][o][p], dz being the gradient of the convolution output in NCHW.
  * One kernel for Col2ImgNode::backward + AddNode::backward (src/Nodes.cu:660-665, 99-146). */
@@ -2236,8 +2311,10 @@ extern "C" int nzhip_conv2d_backward_bias(float* dbias, const float* dz, size_t 
     if (N > 0x7fffffff || O > 0x7fffffff || (O + 31) / 32 > 65535 || (HW + 63) / 64 > 0x7fffffffull)
         return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_bias: extent too large");
     dim3 grid((unsigned)((HW + 63) / 64), (unsigned)((O + 31) / 32));
-    hipLaunchKernelGGL(conv_bias_grad_kernel<false>, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream), dbias, dz,
-                       (int)N, (int)O, (long)HW, static_cast<float*>(nullptr), static_cast<const float*>(nullptr));
+    const bool vec = HW % 4 == 0 && (reinterpret_cast<uintptr_t>(dz) & 15) == 0;
+    hipLaunchKernelGGL(vec ? conv_bias_grad_vec_kernel<false> : conv_bias_grad_kernel<false>, grid, dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), dbias, dz, (int)N, (int)O, (long)HW, static_cast<float*>(nullptr),
+                       static_cast<const float*>(nullptr));
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv_bias_grad kernel launch");
 }
@@ -2252,8 +2329,9 @@ extern "C" int nzhip_conv2d_backward_relu_bias(float* dz, float* dbias, const fl
     if (N > 0x7fffffff || O > 0x7fffffff || (O + 31) / 32 > 65535 || (HW + 63) / 64 > 0x7fffffffull)
         return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_relu_bias: extent too large");
     dim3 grid((unsigned)((HW + 63) / 64), (unsigned)((O + 31) / 32));
-    hipLaunchKernelGGL(conv_bias_grad_kernel<true>, grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream), dbias, dy,
-                       (int)N, (int)O, (long)HW, dz, y);
+    const bool vec = HW % 4 == 0 && ((reinterpret_cast<uintptr_t>(dz) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0;
+    hipLaunchKernelGGL(vec ? conv_bias_grad_vec_kernel<true> : conv_bias_grad_kernel<true>, grid, dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), dbias, dy, (int)N, (int)O, (long)HW, dz, y);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv_bias_grad (masked) kernel launch");
 }

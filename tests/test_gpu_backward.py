@@ -447,7 +447,7 @@ def test_conv2d_backward_weights_few_channels_float_tolerance(nz, oracle):
     assert mr <= 1e-3 and fr <= 1e-4, (mr, fr)
 
 
-@pytest.mark.parametrize("N,O,H,W", [(1, 1, 1, 1), (3, 5, 7, 9), (2, 40, 9, 30), (4, 128, 16, 24), (5, 1, 30, 70), (2, 33, 1, 130)])
+@pytest.mark.parametrize("N,O,H,W", [(1, 1, 1, 1), (3, 5, 7, 9), (2, 40, 9, 30), (4, 128, 16, 24), (5, 1, 30, 70), (2, 33, 1, 130), (3, 50, 6, 10), (7, 17, 8, 36)])
 def test_conv2d_backward_bias_equals_the_two_step_chain_bit_for_bit(nz, oracle, N, O, H, W):
     """One kernel for Col2Img.backward (transpose) + Add.backward (sum over the batch onto the gradient already
     there): the same additions in the same order, so float data agree bit for bit with the oracle's chain."""
