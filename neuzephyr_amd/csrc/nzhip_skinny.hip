@@ -229,7 +229,34 @@ __global__ __launch_bounds__(256) void skinny_lk_kernel(const SkinnyArgs p) {
         for (int r = 0; r < LR; r++) acc[s][r] = 0.f;
 
     const bool s_contig = p.s_sk == 1;
-    for (int k0 = lane * 4; k0 < p.K; k0 += 256) {
+    int k0 = lane * 4;
+    // Whole rows with 16-byte loads: U k steps at a time, their U x (SR + LR) loads issued before any is used -- a
+    // wave has only 64 KiB to stream, and one step per round trip to memory would leave it waiting for latency.
+    if (p.vec && s_contig && (p.SR == 1 || (p.s_ss & 3) == 0) && l0 + LR <= p.LN) {
+        constexpr int U = 4;
+        for (; k0 + 256 * (U - 1) + 4 <= p.K; k0 += 256 * U) {
+            floatx4 sv[U][SR], lv[U][LR];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+#pragma unroll
+                for (int s = 0; s < SR; s++) {
+                    const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                    sv[u][s] = s < p.SR ? *reinterpret_cast<const floatx4*>(S + s * p.s_ss + k0 + 256 * u) : zero;
+                }
+#pragma unroll
+                for (int r = 0; r < LR; r++) lv[u][r] = *reinterpret_cast<const floatx4*>(L + (long)(l0 + r) * p.ldl + k0 + 256 * u);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int r = 0; r < LR; r++)
+#pragma unroll
+                    for (int s = 0; s < SR; s++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[s][r] = __builtin_fmaf(rnd16(sv[u][s][e]), rnd16(lv[u][r][e]), acc[s][r]);
+        }
+    }
+    for (; k0 < p.K; k0 += 256) {
         const bool fullk = p.vec && (k0 + 4 <= p.K);
         floatx4 sv[SR];
 #pragma unroll
@@ -360,8 +387,7 @@ int gemm_skinny_dispatch(const nzhip_gemm_desc& d, hipStream_t stream) {
     float* partial = nullptr;
     static const char* klc_env = getenv("NZHIP_SKINNY_COLS");           // benchmarking only: 0 keeps the split-contraction kernels
     const bool klc_on = !klc_env || atoi(klc_env) != 0;
-    if (l_is_kl && klc_on && batch == 1 && p.SR <= 2 && p.vec && p.LN % KLC_COLS == 0 && p.LN >= 128 * KLC_COLS && p.K >= 1024 &&
-        (long)p.K * p.ldl < 0x7fffffffL) {
+    if (l_is_kl && klc_on && batch == 1 && p.SR <= 2 && p.vec && p.LN % KLC_COLS == 0 && p.LN >= 128 * KLC_COLS && p.K >= 1024) {
         // enough column groups to occupy the chip, a contraction long enough to stream: one kernel, no partial sums
         dim3 grid((unsigned)(p.LN / KLC_COLS));
         if (sr_t == 1) hipLaunchKernelGGL(skinny_kl_cols_kernel<1>, grid, dim3(KLC_THREADS), 0, stream, p);
