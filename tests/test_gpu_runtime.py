@@ -97,3 +97,64 @@ def test_pinned_host_operands(nz):
     nz.check(lib.nzhip_host_malloc(C.byref(q), 0))
     assert q.value is None
     nz.check(lib.nzhip_host_free(None))
+
+
+def test_entry_points_from_four_host_threads_at_once(nz):
+    """Thread-safe entry points (the reference's singleton manager is mutex-protected, StreamManager.cuh:799-805): four
+    host threads, each on its own stream, call products of every route family, a convolution through its own prepared
+    handle and a chunked broadcast gradient at the same time; every result must be the single-threaded one. What is
+    shared between them: the workspace pool, the per-kernel LDS limits, the error string (thread-local), the prepared
+    scope (thread-local). The single-kernel route for very large products needs the GPU to itself and is not part of
+    this."""
+    import threading
+    import torch
+    rng = np.random.default_rng(101)
+
+    def ints(shape, lo=-4, hi=5):
+        return torch.from_numpy(rng.integers(lo, hi, size=shape).astype(np.float32)).cuda()
+
+    gemms = [(300, 200, 100), (1024, 1024, 1024), (1, 4096, 4096), (2048, 1024, 2048), (64, 8192, 64), (1000, 777, 513)]
+    work = []
+    for M, K, N in gemms:
+        A, B = ints((M, K)), ints((K, N))
+        work.append(("gemm", (A, B), (A.double() @ B.double()).float()))
+    x, w = ints((4, 32, 64, 64)), ints((1, 1, 32 * 9, 64), -2, 3)
+    want_conv = nz.conv2d_forward(x, w, None, 3, 3, 1, 1)
+    dout = ints((600, 1, 256, 1))
+    want_bias = dout.sum(dim=0, keepdim=True)
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(tid):
+        try:
+            stream = torch.cuda.Stream()
+            handle = nz.Prepared()
+            with torch.cuda.stream(stream):
+                for rep in range(4):
+                    for i in range(len(work)):
+                        kind, (A, B), want = work[(i + tid) % len(work)]
+                        got = nz.gemm(A, B, stream=stream)
+                        stream.synchronize()
+                        if not torch.equal(got, want):
+                            errors.append((tid, rep, "gemm", tuple(A.shape), tuple(B.shape)))
+                    y = nz.conv2d_forward(x, w, None, 3, 3, 1, 1, stream=stream, prepared_w=handle)
+                    din = torch.zeros((1, 1, 256, 1), device="cuda")
+                    nz.add_backward(din, dout, stream=stream)
+                    stream.synchronize()
+                    if not torch.equal(y, want_conv):
+                        errors.append((tid, rep, "conv"))
+                    if not torch.equal(din, want_bias):
+                        errors.append((tid, rep, "add_backward"))
+            if handle.fills() != 1:
+                errors.append((tid, "fills", handle.fills()))
+            handle.close()
+        except Exception as e:                                        # noqa: BLE001 - reported below
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors[:5]
