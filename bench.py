@@ -28,7 +28,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="gemm8192",
-                    choices=["gemm8192", "gemm256", "gemm1024", "gemm_batched", "linear", "linear_prepared", "conv_a_prepared", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "conv_dwx_5x5", "gemv", "ragged", "conv_a", "conv_b",
+                    choices=["gemm8192", "gemm256", "gemm1024", "gemm_batched", "linear", "linear_prepared", "conv_a_prepared", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "conv_dwx_5x5", "gemv", "ragged", "conv_a", "conv_a_5x5", "conv_a_3x3s2", "conv_b",
                              "adam", "softmax_bwd", "matmul_f32",
                              "copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -326,6 +326,28 @@ def make_workload(name, orc, capi):
         return Workload(name, flops, bytes_, run, verify, "hbm",
                         f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},3,3] s1 p1 + bias + ReLU" +
                         (", fp16 image of the weights kept between calls" if prepared else ""), another), None
+    if name in ("conv_a_5x5", "conv_a_3x3s2"):
+        # the CA tensor through the kernel that takes any kernel extent and stride (no column matrix)
+        N, C, H, W, O = 16, 64, 128, 128, 128
+        K, stride, pad = (5, 1, 2) if name == "conv_a_5x5" else (3, 2, 1)
+        Ho, Wo = (H + 2 * pad - K) // stride + 1, (W + 2 * pad - K) // stride + 1
+        x = orc.fill((N, C, H, W), 4, "normal", 0.0, 1.0)
+        w = orc.fill((O, C, K, K), 1005, "normal", 0.0, float(np.sqrt(2.0 / (C * K * K))))
+        bias = orc.fill((O,), 2005, "uniform", -0.03, 0.03)
+        xd, wd, bd = dev(x), dev(orc.weights_oihw_to_ref(w)), dev(bias)
+        out = torch.empty((N, O, Ho, Wo), device="cuda")
+
+        def run():
+            capi.conv2d_forward(xd, wd, bd, K, K, stride, pad, bias_strides=(0, 1), relu=True, out=out)
+
+        def verify():
+            truth = orc.conv2d_direct_f64(x[:1], w, bias, stride, pad, relu=True)
+            return tolerance(orc, out[:1].cpu().numpy(), truth, name)
+
+        flops = 2.0 * N * Ho * Wo * C * K * K * O
+        bytes_ = 4.0 * (N * C * H * W + O * C * K * K + O + N * O * Ho * Wo)
+        return Workload(name, flops, bytes_, run, verify, "hbm",
+                        f"Conv2d x[{N},{C},{H},{W}] w[{O},{C},{K},{K}] s{stride} p{pad} + bias + ReLU"), None
     if name == "adam":
         # opt::Adam::step over 2^26 parameters: data, m, v read and written, the gradient read
         n = 1 << 26
@@ -711,7 +733,7 @@ def main():
 
     extra = {}
     if args.workload == "gemm8192" and not args.no_extra:
-        for name in ("conv_b", "conv_a", "conv_a_prepared", "linear", "linear_prepared", "gemv", "ragged", "gemm256", "gemm1024", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "conv_dwx_5x5", "adam",
+        for name in ("conv_b", "conv_a", "conv_a_prepared", "conv_a_5x5", "conv_a_3x3s2", "linear", "linear_prepared", "gemv", "ragged", "gemm256", "gemm1024", "gemm_batched", "linear_bwd", "conv_dw", "conv_dx", "conv_dwx", "conv_dwx_5x5", "adam",
                      "softmax_bwd", "matmul_f32"):
             torch.cuda.empty_cache()
             w2, _ = make_workload(name, orc, capi)

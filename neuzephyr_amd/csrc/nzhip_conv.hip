@@ -1613,6 +1613,280 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     return rc ? rc : rc2;
 }
 
+// ---- implicit GEMM for any kernel extent and stride ----------------------------------------------------------
+// The kernels above are built for 3x3 and 1x1 at stride 1 (halo geometry and tap loops are compile-time). Every other
+// geometry whose rows allow 16-byte loads -- 5x5, strides 2..4, rectangular kernels -- used to write its column matrix
+// (K_h K_w times the input) and read it back through the GEMM. This kernel keeps the same arithmetic without it:
+// a workgroup of eight waves owns a segment of 256 output pixels (256 / SW output rows x SW columns, SW the power of
+// two >= 16 that covers the output width) x BN output channels of one image. Per chunk of 16 input channels it
+// stages the input rows under the segment in LDS as fp16, channel-last (32 bytes per pixel, the two 16-byte halves
+// swapped every eight columns like the fixed-geometry kernels), and the chunk's weight slab (BN rows of taps x 32
+// bytes + 16, direct to LDS); a tap's B fragment is then one 16-byte read per lane at (row * stride + r,
+// column * stride + s). A thread's staging tasks -- four adjacent input columns x eight channels, transposed in
+// registers -- are fixed for the whole kernel; the next chunk's loads are in flight while this one multiplies.
+constexpr int CG_PX = 256, CG_THREADS = 512, CG_TP_MAX = 3;
+
+struct ConvGenArgs {
+    float* y;
+    const float* x;
+    const _Float16* wimg;   // [w copy][o tile][chunk][BN][w_pitch / 2]
+    const float* bias;
+    int C, H, W, O, Ho, Wo, Kh, Kw, stride, pad;
+    int n_chunks, n_otiles, w_batched;
+    int sw_log, span, pw, shift, segs_w;
+    int w_pitch, slab_bytes, halo_off;
+    long bias_sp, bias_sc, bias_sn;
+    int relu;
+};
+
+// Pre-pass: w_ref [wb][C * taps][O] fp32 -> fp16 slabs [wb][o tile][chunk][BN][taps * 16 + 8]
+__global__ __launch_bounds__(256) void conv_weight_image_gen_kernel(_Float16* __restrict__ dst, const float* __restrict__ w_ref, int C,
+                                                                    int O, int taps, int BN, int w_pitch_halfs, int n_chunks,
+                                                                    int n_otiles) {
+    const int slab = blockIdx.y;                               // (wb * n_otiles + o_tile) * n_chunks + chunk
+    const int chunk = slab % n_chunks, o_tile = (slab / n_chunks) % n_otiles, wb = slab / (n_chunks * n_otiles);
+    const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, o fastest
+    const int o_l = t % BN, rest = t / BN;
+    if (rest >= taps * IG_CC) return;
+    const int cc = rest % IG_CC, tap = rest / IG_CC;
+    const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
+    float v = 0.f;
+    if (c < C && o < O) v = w_ref[((long)wb * C * taps + (long)c * taps + tap) * O + o];
+    dst[(long)slab * BN * w_pitch_halfs + (long)o_l * w_pitch_halfs + tap * IG_CC + cc] = (_Float16)v;
+}
+
+// NO: 32-channel blocks per wave (BN / 64); every wave also owns two 32-pixel blocks. TP: staging tasks per thread.
+template <int NO, int TP>
+__global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGenArgs p) {
+    constexpr int BN = NO * 64;
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    char* lds_w = lds;
+    char* lds_h = lds + p.halo_off;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lh = lane >> 5;
+    const int wm = wave & 3, wn = wave >> 2;                    // pixel blocks 2 wm, 2 wm + 1; channel blocks NO wn ..
+    const int b = blockIdx.z, o_tile = blockIdx.y;
+    const int SW = 1 << p.sw_log, SR = CG_PX >> p.sw_log;
+    const int ho0 = (blockIdx.x / p.segs_w) * SR, wo0 = (blockIdx.x % p.segs_w) * SW;
+    const int hb = ho0 * p.stride - p.pad, wf = wo0 * p.stride - p.pad - p.shift;   // image position of staged (0, 0)
+    const int taps = p.Kh * p.Kw;
+    const long plane = (long)p.H * p.W;
+    const float* xb = p.x + (long)b * p.C * plane;
+    const char* wsrc = reinterpret_cast<const char*>(p.wimg) +
+                       ((long)(p.w_batched ? b : 0) * p.n_otiles + o_tile) * p.n_chunks * p.slab_bytes + lane * 16;
+
+    // staging tasks: task e = tid + 512 k is (8-channel half, staged row, column quad)
+    const int pw4 = p.pw >> 2, n_tasks = 2 * p.span * pw4;
+    int t_off[TP], t_dst[TP];                                   // image offset of the quad (or -1), LDS byte offset of its first pixel
+    int t_h8[TP];
+#pragma unroll
+    for (int k = 0; k < TP; k++) {
+        const int e = tid + CG_THREADS * k;
+        const int q = e % pw4, row = (e / pw4) % p.span, h8 = e / (pw4 * p.span);
+        const int h = hb + row, w = wf + 4 * q;
+        const bool in = e < n_tasks && h >= 0 && h < p.H && w >= 0 && w < p.W;     // W % 4 == 0 and w % 4 == 0: the whole quad
+        t_off[k] = in ? h * p.W + w : -1;
+        t_dst[k] = e < n_tasks ? (row * p.pw + 4 * q) * 32 : -1;
+        t_h8[k] = h8;
+    }
+
+    floatx16 acc[NO][2];
+#pragma unroll
+    for (int i = 0; i < NO; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    floatx4 raw[TP][8];                                          // [task][channel][pixel of the quad]
+    auto load_halo = [&](const int chunk) {
+#pragma unroll
+        for (int k = 0; k < TP; k++) {
+            const int c0 = chunk * IG_CC + t_h8[k] * 8;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const bool ok = t_off[k] >= 0 && c0 + e < p.C;
+                raw[k][e] = *reinterpret_cast<const floatx4*>(xb + (ok ? (long)(c0 + e) * plane + t_off[k] : 0));
+            }
+        }
+    };
+    auto store_halo = [&](const int chunk) {
+#pragma unroll
+        for (int k = 0; k < TP; k++) {
+            if (t_dst[k] < 0) continue;
+            const int c0 = chunk * IG_CC + t_h8[k] * 8;
+            const int col0 = (t_dst[k] >> 5) % p.pw;            // staged column of the quad's first pixel (a multiple of 4)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                half8_t h;
+#pragma unroll
+                for (int e = 0; e < 8; e++) h[e] = (t_off[k] >= 0 && c0 + e < p.C) ? (_Float16)raw[k][e][q] : (_Float16)0.f;
+                const int col = col0 + q;
+                *reinterpret_cast<half8_t*>(lds_h + t_dst[k] + q * 32 + ((t_h8[k] ^ ((col >> 3) & 1)) << 4)) = h;
+            }
+        }
+    };
+    auto load_slab = [&](const int chunk) {
+        const int pieces = p.slab_bytes >> 10;
+        for (int j = wave; j < pieces; j += CG_THREADS / 64)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void*)(wsrc + (long)chunk * p.slab_bytes + j * 1024),
+                (__attribute__((address_space(3))) void*)(lds_w + j * 1024), 16, 0, 0);
+    };
+
+    // this lane's two pixels: staged row and column of tap (0, 0)
+    int prow[2], pcol[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int px = (wm * 2 + j) * 32 + li;
+        prow[j] = (px >> p.sw_log) * p.stride;
+        pcol[j] = (px & (SW - 1)) * p.stride + p.shift;
+    }
+    const char* wrow[NO];
+#pragma unroll
+    for (int i = 0; i < NO; i++) wrow[i] = lds_w + ((wn * NO + i) * 32 + li) * p.w_pitch + lh * 16;
+
+    load_halo(0);
+    load_slab(0);
+    for (int chunk = 0; chunk < p.n_chunks; chunk++) {
+        store_halo(chunk);                                      // registers (chunk) -> LDS, fp16 channel-last
+        __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): this wave's slab pieces landed
+        __syncthreads();
+        load_halo(chunk + 1 < p.n_chunks ? chunk + 1 : chunk);  // lands while the MFMAs below run (the last: once more, unused)
+        // two fragment sets: the reads of tap t + 1 are issued before the MFMAs of tap t
+        half8_t wf_[2][NO], pf_[2][2];
+        auto fragments = [&](const int tap, const int r, const int sx, const int set) {
+#pragma unroll
+            for (int i = 0; i < NO; i++) wf_[set][i] = *reinterpret_cast<const half8_t*>(wrow[i] + tap * 32);
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int col = pcol[j] + sx;
+                pf_[set][j] = *reinterpret_cast<const half8_t*>(lds_h + ((prow[j] + r) * p.pw + col) * 32 + ((lh ^ ((col >> 3) & 1)) << 4));
+            }
+        };
+        int r = 0, sx = 0;
+        fragments(0, 0, 0, 0);
+        for (int tap = 0; tap < taps; tap += 2) {
+            {
+                int r1 = r, s1 = sx + 1;
+                if (s1 == p.Kw) { s1 = 0; r1++; }
+                if (tap + 1 < taps) fragments(tap + 1, r1, s1, 1);
+#pragma unroll
+                for (int i = 0; i < NO; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[0][i], pf_[0][j], acc[i][j], 0, 0, 0);
+                r = r1; sx = s1;
+            }
+            if (tap + 1 < taps) {
+                int r1 = r, s1 = sx + 1;
+                if (s1 == p.Kw) { s1 = 0; r1++; }
+                if (tap + 2 < taps) fragments(tap + 2, r1, s1, 0);
+#pragma unroll
+                for (int i = 0; i < NO; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[1][i], pf_[1][j], acc[i][j], 0, 0, 0);
+                r = r1; sx = s1;
+            }
+        }
+        __syncthreads();                                        // everyone is done reading this chunk's LDS
+        if (chunk + 1 < p.n_chunks) load_slab(chunk + 1);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);                // the halo requested once more after the last chunk
+
+    // ---- epilogue: bias + activation + NCHW store (lanes = adjacent pixels) ----
+    float* yb = p.y + (long)b * p.O * p.Ho * p.Wo;
+    const long hw_out = (long)p.Ho * p.Wo;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int px = (wm * 2 + j) * 32 + li;
+        const int ho = ho0 + (px >> p.sw_log), wo = wo0 + (px & (SW - 1));
+        if (ho >= p.Ho || wo >= p.Wo) continue;
+        const long pix = (long)ho * p.Wo + wo;
+#pragma unroll
+        for (int i = 0; i < NO; i++) {
+            const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
+            float bv[16];
+#pragma unroll
+            for (int rr = 0; rr < 16; rr++) {
+                const int o = o_base + (rr >> 2) * 8 + (rr & 3);
+                bv[rr] = (p.bias && o < p.O) ? p.bias[(long)b * p.bias_sn + pix * p.bias_sp + (long)o * p.bias_sc] : 0.f;
+            }
+#pragma unroll
+            for (int rr = 0; rr < 16; rr++) {
+                const int o = o_base + (rr >> 2) * 8 + (rr & 3);
+                float v = acc[i][j][rr] + bv[rr];
+                if (p.relu) v = v > 0.f ? v : 0.f;
+                if (o < p.O) yb[(long)o * hw_out + pix] = v;
+            }
+        }
+    }
+}
+
+static bool conv_igemm_gen_applicable(const float* x, size_t C, size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride,
+                                      size_t pad, size_t N) {
+    (void)O;
+    // (a strided 1x1 convolution has one tap per chunk to multiply between two barriers: its column matrix is the cheaper way)
+    return C >= 8 && W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && stride <= 4 && K_h * K_w >= 2 && K_h * K_w <= 64 && pad < 0x10000 &&
+           N <= 65535 && H * W < 0x7fffffffull && C * H * W < 0x7fffffffull;
+}
+
+// Returns NZHIP_E_UNSUPPORTED (nothing enqueued, no error text) when the tile does not fit LDS or a thread's staging share.
+static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C, size_t H,
+                                 size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t w_batch,
+                                 int64_t bias_sp, int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out,
+                                 hipStream_t s) {
+    const int taps = (int)(K_h * K_w);
+    const int BN = O > 64 ? 128 : 64;
+    int sw_log = 8;
+    while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
+    const int SW = 1 << sw_log, SR = CG_PX / SW;
+    const int shift = (int)(((4 - (long)(pad % 4)) % 4 + 4) % 4);   // staged column 0 is a multiple of four image columns
+    const int span = (int)((SR - 1) * stride + K_h);
+    int pw = (int)((SW - 1) * stride + K_w) + shift;
+    pw = (pw + 3) / 4 * 4;
+    const int w_pitch = taps * 32 + 16, slab_bytes = BN * w_pitch;
+    const int halo_off = (slab_bytes + 1023) / 1024 * 1024;
+    const size_t lds_need = (size_t)halo_off + (size_t)span * pw * 32;
+    const size_t tasks = (size_t)2 * span * (pw / 4);
+    if (lds_need > 160 * 1024 - 512 || tasks > (size_t)CG_THREADS * CG_TP_MAX) return NZHIP_E_UNSUPPORTED;
+    const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
+    const size_t seg_rows = (H_out + SR - 1) / SR, segs_w = (W_out + SW - 1) / SW;
+    if (n_otiles > 65535 || seg_rows * segs_w > 0x7fffffffull) return NZHIP_E_UNSUPPORTED;
+    const size_t image_bytes = (size_t)n_otiles * n_chunks * slab_bytes, bytes = image_bytes * w_batch;
+    uint64_t key[PREPARED_KEY_WORDS];
+    conv_image_key(key, 3, (int)K_h, (int)K_w, BN, w_ref, C, O, n_chunks, n_otiles, w_batch);
+    ImageLease lease;
+    if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
+    _Float16* wimg = static_cast<_Float16*>(lease.ptr);
+    if (lease.fill) {
+        dim3 pg((unsigned)((BN * taps * IG_CC + 255) / 256), (unsigned)(w_batch * n_otiles * n_chunks));
+        hipLaunchKernelGGL(conv_weight_image_gen_kernel, pg, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O, taps, BN, w_pitch / 2,
+                           n_chunks, n_otiles);
+    }
+    ConvGenArgs a;
+    a.y = y; a.x = x; a.wimg = wimg; a.bias = bias;
+    a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.Ho = (int)H_out; a.Wo = (int)W_out;
+    a.Kh = (int)K_h; a.Kw = (int)K_w; a.stride = (int)stride; a.pad = (int)pad;
+    a.n_chunks = n_chunks; a.n_otiles = n_otiles; a.w_batched = w_batch > 1;
+    a.sw_log = sw_log; a.span = span; a.pw = pw; a.shift = shift; a.segs_w = (int)segs_w;
+    a.w_pitch = w_pitch; a.slab_bytes = slab_bytes; a.halo_off = halo_off;
+    a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
+    const int tp = (int)((tasks + CG_THREADS - 1) / CG_THREADS);
+    auto kfn = BN == 128 ? (tp <= 1 ? conv_igemm_gen_kernel<2, 1> : tp == 2 ? conv_igemm_gen_kernel<2, 2> : conv_igemm_gen_kernel<2, 3>)
+                         : (tp <= 1 ? conv_igemm_gen_kernel<1, 1> : tp == 2 ? conv_igemm_gen_kernel<1, 2> : conv_igemm_gen_kernel<1, 3>);
+    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_need, "hipFuncSetAttribute(conv_igemm_gen)");
+    if (rc == NZHIP_OK) {
+        hipLaunchKernelGGL(kfn, dim3((unsigned)(seg_rows * segs_w), (unsigned)n_otiles, (unsigned)N), dim3(CG_THREADS), lds_need, s, a);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm_gen kernel launch");
+    }
+    const int rc2 = image_release(lease, s, rc == NZHIP_OK);
+    return rc ? rc : rc2;
+}
+
 // General route: column matrix in a pooled workspace, then ONE batched GEMM that computes the
 // transposed product  y_b[O, HW] = w_b^T[O, CKK] * col_b^T[CKK, HW]  so that bias, activation
 // and the col2im transpose (src/OperationKernels.cu:1364-1376) all happen in its epilogue and
@@ -2130,7 +2404,18 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
         const bool resident = (w_batch == 1 || N * ((O + bn - 1) / bn) <= (size_t)device_cu_count()) && w_lds <= 148 * 1024;
         few_patches = !resident && units * 4 <= (size_t)device_cu_count();
     }
-    if (!force_ws && !few_patches && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL) {
+    const bool fixed_geometry = !force_ws && !few_patches && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL;
+    // any other kernel extent or stride, when the rows allow 16-byte loads and the segments occupy at least a quarter of the CUs
+    bool any_geometry = false;
+    if (!fixed_geometry && !force_ws && bias_stride_image == 0 && !conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) &&
+        conv_igemm_gen_applicable(x, C, H, W, O, K_h, K_w, stride, pad, N) && (w_batch == 1 || w_batch * ((O + 63) / 64) * ((C + 15) / 16) <= 65535)) {
+        int sw_log = 8;
+        while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
+        const size_t sw = (size_t)1 << sw_log, sr = CG_PX / sw;
+        const size_t groups = N * ((H_out + sr - 1) / sr) * ((W_out + sw - 1) / sw) * ((O + 127) / 128);
+        any_geometry = groups * 4 >= (size_t)device_cu_count();
+    }
+    if (fixed_geometry || any_geometry) {
         // The reference's bias parameter is pixel-major ([1,1,H_out*W_out,O], src/Model.cu:252-256), while the kernels'
         // lanes are adjacent pixels: read as it lies, every bias load touches 64 lines 4 O bytes apart. One pass turns it
         // into channel planes (the layout of y), and the bias loads look like the result stores.
@@ -2149,6 +2434,14 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
             const int rc2 = bias_planes ? workspace_free(bias_planes, s) : NZHIP_OK;
             return rc ? rc : rc2;
         };
+        if (any_geometry) {
+            const int rc = conv_igemm_gen_launch(y, x, w_ref, bias_use, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bsp, bsc,
+                                                 bias_stride_image, activation, H_out, W_out, s);
+            const int rc_free = finish(rc == NZHIP_E_UNSUPPORTED ? NZHIP_OK : rc);
+            if (rc != NZHIP_E_UNSUPPORTED) return rc_free;
+            return conv2d_via_workspace(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
+                                        bias_stride_channel, activation, H_out, W_out, s);   // the tile does not fit: column matrix
+        }
 #define NZHIP_IG(KH_, TW_, BN_)                                                                                      \
     return finish(conv_igemm_launch<KH_, KH_, TW_, BN_>(y, x, w_ref, bias_use, N, C, H, W, O, pad, w_batch, bsp, bsc, \
                                                         bias_stride_image, activation, H_out, W_out, s))

@@ -124,6 +124,39 @@ def test_conv2d_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, 
     assert np.array_equal(host(y), got)
 
 
+CONV_ANY_GEOMETRY = [  # N, C, H, W, O, k_h, k_w, stride, pad, w_batch, per-pixel bias: enough 256-pixel segments for the
+    # implicit-GEMM kernel that takes any kernel extent and stride (rows that allow 16-byte loads)
+    (16, 16, 32, 32, 16, 5, 5, 1, 2, 1, False),     # 5x5, 32-wide segments of 8 rows, 64-channel tile
+    (32, 24, 33, 64, 70, 3, 3, 2, 1, 1, False),     # stride 2, two chunks (the second half empty), 128-channel tile with 70 channels
+    (16, 16, 48, 192, 8, 3, 3, 3, 1, 1, False),     # stride 3: three staging tasks per thread
+    (4, 8, 66, 260, 9, 3, 3, 2, 1, 1, False),       # 130 output columns: one row per segment, the second half of it empty
+    (40, 40, 20, 24, 130, 2, 3, 2, 0, 40, False),   # 2x3 kernel, no padding, per-sample weights, two channel tiles
+    (32, 32, 30, 40, 64, 5, 5, 2, 3, 1, True),      # padding 3, per-pixel bias (turned into channel planes first)
+    (64, 16, 14, 16, 32, 3, 3, 2, 1, 1, False),     # 7 x 8 outputs: a segment spans the whole image and more
+    (4, 16, 40, 128, 16, 5, 5, 4, 2, 1, False),     # stride 4 with 128-wide... the tile does not fit a thread's staging share: column matrix
+]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,k_h,k_w,stride,pad,w_batch,pix", CONV_ANY_GEOMETRY)
+def test_conv2d_any_geometry_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, pad, w_batch, pix):
+    rng = np.random.default_rng(N * 3 + C * 5 + H * 7 + W * 11 + O * 13 + k_h + stride)
+    Ho, Wo = oracle.out_hw(H, W, k_h, k_w, stride, pad)
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    ws = [rng.integers(-3, 4, size=(O, C, k_h, k_w)).astype(np.float32) for _ in range(w_batch)]
+    w_ref = np.concatenate([oracle.weights_oihw_to_ref(w) for w in ws], axis=0)
+    if pix:
+        bias = rng.integers(-2, 3, size=(1, 1, Ho * Wo, O)).astype(np.float32)
+        strides, badd = (O, 1), bias.reshape(Ho, Wo, O).transpose(2, 0, 1)[None].astype(np.float64)
+    else:
+        bias = rng.integers(-2, 3, size=(O,)).astype(np.float32)
+        strides, badd = (0, 1), bias.reshape(1, O, 1, 1).astype(np.float64)
+    got = host(nz.conv2d_forward(dev(x), dev(w_ref), dev(bias), k_h, k_w, stride, pad, bias_strides=strides, relu=True))
+    for n in range(N):
+        w = ws[n if w_batch > 1 else 0]
+        truth = np.maximum(oracle.conv2d_direct_f64(x[n:n + 1], w, None, stride, pad) + badd, 0)
+        assert np.array_equal(got[n:n + 1].astype(np.float64), truth), (n,)
+
+
 PER_SAMPLE = [  # N, C, H, W, O, k, pad, per-pixel bias: one weight copy per image, every copy different
     (4, 32, 12, 64, 128, 3, 1, False),    # two halo buffers, 128-channel tile, 64 workgroups per image
     (3, 64, 9, 64, 64, 3, 1, True),       # two halo buffers, 64-channel tile, per-pixel bias; 255 of 256 workgroups used
