@@ -1839,10 +1839,14 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
                                  int64_t bias_sp, int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out,
                                  hipStream_t s) {
     const int taps = (int)(K_h * K_w);
-    const int BN = O > 64 ? 128 : 64;
     int sw_log = 8;
     while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
     const int SW = 1 << sw_log, SR = CG_PX / SW;
+    // 128 output channels per workgroup, unless that leaves compute units without one (16 x 128 x 56 x 56 -> 128 at
+    // stride 2: 64 workgroups; with 64-channel tiles 128 of them, 40 against 49 us)
+    static const char* bn_env = getenv("NZHIP_CONV_BN");            // benchmarking only
+    const size_t groups128 = N * ((H_out + SR - 1) / SR) * ((W_out + SW - 1) / SW) * ((O + 127) / 128);
+    const int BN = bn_env ? (atoi(bn_env) == 128 ? 128 : 64) : (O > 64 && groups128 >= (size_t)device_cu_count() ? 128 : 64);
     const int shift = (int)(((4 - (long)(pad % 4)) % 4 + 4) % 4);   // staged column 0 is a multiple of four image columns
     const int span = (int)((SR - 1) * stride + K_h);
     int pw = (int)((SW - 1) * stride + K_w) + shift;
