@@ -1637,6 +1637,8 @@ struct ConvGenArgs {
     int w_pitch, slab_bytes, halo_off;
     long bias_sp, bias_sc, bias_sn;
     int relu;
+    int chunk_groups, chunks_per_group;   // the contraction split over groups of channel chunks (blockIdx.z = image * groups + group)
+    float* partial;                       // with more than one group: [group][image][O][Ho * Wo] sums without bias or activation
 };
 
 // Pre-pass: w_ref [wb][C * taps][O] fp32 -> fp16 slabs [wb][o tile][chunk][BN][taps * 16 + 8]
@@ -1666,7 +1668,9 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, lh = lane >> 5;
     const int wm = wave & 3, wn = wave >> 2;                    // pixel blocks 2 wm, 2 wm + 1; channel blocks NO wn ..
-    const int b = blockIdx.z, o_tile = blockIdx.y;
+    const int b = blockIdx.z / p.chunk_groups, group = blockIdx.z % p.chunk_groups, o_tile = blockIdx.y;
+    const int chunk_lo = group * p.chunks_per_group;
+    const int chunk_hi = chunk_lo + p.chunks_per_group < p.n_chunks ? chunk_lo + p.chunks_per_group : p.n_chunks;
     const int SW = 1 << p.sw_log, SR = CG_PX >> p.sw_log;
     const int ho0 = (blockIdx.x / p.segs_w) * SR, wo0 = (blockIdx.x % p.segs_w) * SW;
     const int hb = ho0 * p.stride - p.pad, wf = wo0 * p.stride - p.pad - p.shift;   // image position of staged (0, 0)
@@ -1747,13 +1751,13 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
 #pragma unroll
     for (int i = 0; i < NO; i++) wrow[i] = lds_w + ((wn * NO + i) * 32 + li) * p.w_pitch + lh * 16;
 
-    load_halo(0);
-    load_slab(0);
-    for (int chunk = 0; chunk < p.n_chunks; chunk++) {
+    load_halo(chunk_lo);
+    load_slab(chunk_lo);
+    for (int chunk = chunk_lo; chunk < chunk_hi; chunk++) {
         store_halo(chunk);                                      // registers (chunk) -> LDS, fp16 channel-last
         __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): this wave's slab pieces landed
         __syncthreads();
-        load_halo(chunk + 1 < p.n_chunks ? chunk + 1 : chunk);  // lands while the MFMAs below run (the last: once more, unused)
+        load_halo(chunk + 1 < chunk_hi ? chunk + 1 : chunk);    // lands while the MFMAs below run (the last: once more, unused)
         // two fragment sets: the reads of tap t + 1 are issued before the MFMAs of tap t
         half8_t wf_[2][NO], pf_[2][2];
         auto fragments = [&](const int tap, const int r, const int sx, const int set) {
@@ -1792,13 +1796,33 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
             }
         }
         __syncthreads();                                        // everyone is done reading this chunk's LDS
-        if (chunk + 1 < p.n_chunks) load_slab(chunk + 1);
+        if (chunk + 1 < chunk_hi) load_slab(chunk + 1);
     }
     __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);                // the halo requested once more after the last chunk
 
-    // ---- epilogue: bias + activation + NCHW store (lanes = adjacent pixels) ----
-    float* yb = p.y + (long)b * p.O * p.Ho * p.Wo;
+    // ---- epilogue: bias + activation + NCHW store (lanes = adjacent pixels), or the bare sums of this channel group ----
     const long hw_out = (long)p.Ho * p.Wo;
+    if (p.partial) {
+        float* pb = p.partial + ((long)group * (gridDim.z / p.chunk_groups) + b) * p.O * hw_out;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int px = (wm * 2 + j) * 32 + li;
+            const int ho = ho0 + (px >> p.sw_log), wo = wo0 + (px & (SW - 1));
+            if (ho >= p.Ho || wo >= p.Wo) continue;
+            const long pix = (long)ho * p.Wo + wo;
+#pragma unroll
+            for (int i = 0; i < NO; i++) {
+                const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
+#pragma unroll
+                for (int rr = 0; rr < 16; rr++) {
+                    const int o = o_base + (rr >> 2) * 8 + (rr & 3);
+                    if (o < p.O) pb[(long)o * hw_out + pix] = acc[i][j][rr];
+                }
+            }
+        }
+        return;
+    }
+    float* yb = p.y + (long)b * p.O * p.Ho * p.Wo;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int px = (wm * 2 + j) * 32 + li;
@@ -1823,6 +1847,22 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
             }
         }
     }
+}
+
+// y = act(bias + the channel groups' sums, added in ascending group order)
+__global__ __launch_bounds__(256) void conv_group_sum_kernel(float* __restrict__ y, const float* __restrict__ partial, const float* __restrict__ bias,
+                                                             int groups, int O, long hw, long per_group, long bias_sp, long bias_sc,
+                                                             long bias_sn, int relu) {
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;        // element of y: (image, channel, pixel)
+    if (t >= per_group) return;
+    float v = 0.f;
+    for (int g = 0; g < groups; g++) v += partial[(long)g * per_group + t];
+    if (bias) {
+        const long pix = t % hw, bo = t / hw;
+        v += bias[(bo / O) * bias_sn + pix * bias_sp + (bo % O) * bias_sc];
+    }
+    if (relu) v = v > 0.f ? v : 0.f;
+    y[t] = v;
 }
 
 static bool conv_igemm_gen_applicable(const float* x, size_t C, size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride,
@@ -1859,6 +1899,19 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
     const size_t seg_rows = (H_out + SR - 1) / SR, segs_w = (W_out + SW - 1) / SW;
     if (n_otiles > 65535 || seg_rows * segs_w > 0x7fffffffull) return NZHIP_E_UNSUPPORTED;
+    // Few segments and many channels (deep layers on small images): the contraction is split over groups of at least
+    // two channel chunks until every compute unit has a workgroup; a second kernel adds the groups' sums in order.
+    int chunk_groups = 1, chunks_per_group = n_chunks;
+    {
+        const size_t wgs = N * seg_rows * segs_w * n_otiles, cus = (size_t)device_cu_count();
+        if (wgs < cus && n_chunks >= 4) {
+            size_t want = (cus + wgs - 1) / wgs;
+            if (want > (size_t)n_chunks / 2) want = (size_t)n_chunks / 2;
+            chunks_per_group = (int)((n_chunks + want - 1) / want);
+            chunk_groups = (n_chunks + chunks_per_group - 1) / chunks_per_group;
+        }
+        if (N * (size_t)chunk_groups > 65535) return NZHIP_E_UNSUPPORTED;
+    }
     const size_t image_bytes = (size_t)n_otiles * n_chunks * slab_bytes, bytes = image_bytes * w_batch;
     uint64_t key[PREPARED_KEY_WORDS];
     conv_image_key(key, 3, (int)K_h, (int)K_w, BN, w_ref, C, O, n_chunks, n_otiles, w_batch);
@@ -1878,17 +1931,36 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     a.sw_log = sw_log; a.span = span; a.pw = pw; a.shift = shift; a.segs_w = (int)segs_w;
     a.w_pitch = w_pitch; a.slab_bytes = slab_bytes; a.halo_off = halo_off;
     a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
+    a.chunk_groups = chunk_groups; a.chunks_per_group = chunks_per_group; a.partial = nullptr;
+    const size_t per_group = N * O * H_out * W_out;
+    float* partial = nullptr;
+    if (chunk_groups > 1) {
+        if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), (size_t)chunk_groups * per_group * sizeof(float), s)) {
+            image_release(lease, s, true);
+            return rc;
+        }
+        a.partial = partial;
+    }
     const int tp = (int)((tasks + CG_THREADS - 1) / CG_THREADS);
     auto kfn = BN == 128 ? (tp <= 1 ? conv_igemm_gen_kernel<2, 1> : tp == 2 ? conv_igemm_gen_kernel<2, 2> : conv_igemm_gen_kernel<2, 3>)
                          : (tp <= 1 ? conv_igemm_gen_kernel<1, 1> : tp == 2 ? conv_igemm_gen_kernel<1, 2> : conv_igemm_gen_kernel<1, 3>);
     int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_need, "hipFuncSetAttribute(conv_igemm_gen)");
     if (rc == NZHIP_OK) {
-        hipLaunchKernelGGL(kfn, dim3((unsigned)(seg_rows * segs_w), (unsigned)n_otiles, (unsigned)N), dim3(CG_THREADS), lds_need, s, a);
+        hipLaunchKernelGGL(kfn, dim3((unsigned)(seg_rows * segs_w), (unsigned)n_otiles, (unsigned)(N * chunk_groups)), dim3(CG_THREADS),
+                           lds_need, s, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm_gen kernel launch");
     }
+    if (rc == NZHIP_OK && partial) {
+        hipLaunchKernelGGL(conv_group_sum_kernel, dim3((unsigned)((per_group + 255) / 256)), dim3(256), 0, s, y, partial, bias, chunk_groups,
+                           (int)O, (long)(H_out * W_out), (long)per_group, (long)bias_sp, (long)bias_sc, (long)bias_sn,
+                           act == NZHIP_ACT_RELU ? 1 : 0);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "conv_group_sum kernel launch");
+    }
+    const int rc3 = partial ? workspace_free(partial, s) : NZHIP_OK;
     const int rc2 = image_release(lease, s, rc == NZHIP_OK);
-    return rc ? rc : rc2;
+    return rc ? rc : (rc2 ? rc2 : rc3);
 }
 
 // General route: column matrix in a pooled workspace, then ONE batched GEMM that computes the
@@ -2400,24 +2472,35 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
     // patch per workgroup with the whole C x taps contraction inside, and there are too few patches to
     // fill the CUs (8 x 512 x 16 x 16 -> 512: 64 workgroups, 190 us). The column matrix of such a layer is
     // small; its batched GEMM splits the contraction over the idle CUs instead (83 us).
-    bool few_patches = false;
+    bool few_patches = false, sparse_patches = false;
     if (bias_stride_image == 0) {
         const size_t tw = wide ? 64 : 32, th = 256 / tw, bn = bn128 ? 128 : 64;
         const size_t units = N * ((W_out + tw - 1) / tw) * ((H_out + th - 1) / th) * ((O + bn - 1) / bn);
         const size_t w_lds = ((C + IG_CC - 1) / IG_CC) * bn * K_h * K_w * 32;       // fp16 weight image of one channel tile
         const bool resident = (w_batch == 1 || N * ((O + bn - 1) / bn) <= (size_t)device_cu_count()) && w_lds <= 148 * 1024;
         few_patches = !resident && units * 4 <= (size_t)device_cu_count();
+        // Weights beyond LDS and fewer than 1.75 patches per compute unit (16 x 256 x 28 x 28 -> 256: 128): the any-geometry
+        // kernel splits the channels over workgroups and is faster there (58 against 87 us; 16 x 512 x 16 x 16 -> 512: 75
+        // against 193 us), as long as its 256-pixel segments are at least half full (4 x 512 x 8 x 8: 37 against 29 us).
+        sparse_patches = !resident && units * 4 < 7 * (size_t)device_cu_count();
     }
-    const bool fixed_geometry = !force_ws && !few_patches && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL;
-    // any other kernel extent or stride, when the rows allow 16-byte loads and the segments occupy at least a quarter of the CUs
+    const bool force_gen = route_env && route_env[0] == 'g';        // "gen": the any-geometry kernel wherever it applies (benchmarking only)
+    bool fixed_geometry = !force_ws && !few_patches && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL;
+    // any other kernel extent or stride, when the rows allow 16-byte loads and the segments (times the channel groups the
+    // contraction can be split into) occupy at least a quarter of the CUs
     bool any_geometry = false;
-    if (!fixed_geometry && !force_ws && bias_stride_image == 0 && !conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) &&
+    if ((!fixed_geometry || force_gen || sparse_patches) && !force_ws && bias_stride_image == 0 &&
+        (force_gen || sparse_patches || !conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N)) &&
         conv_igemm_gen_applicable(x, C, H, W, O, K_h, K_w, stride, pad, N) && (w_batch == 1 || w_batch * ((O + 63) / 64) * ((C + 15) / 16) <= 65535)) {
         int sw_log = 8;
         while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
         const size_t sw = (size_t)1 << sw_log, sr = CG_PX / sw;
-        const size_t groups = N * ((H_out + sr - 1) / sr) * ((W_out + sw - 1) / sw) * ((O + 127) / 128);
-        any_geometry = groups * 4 >= (size_t)device_cu_count();
+        const size_t chunks = (C + IG_CC - 1) / IG_CC;
+        const size_t groups = N * ((H_out + sr - 1) / sr) * ((W_out + sw - 1) / sw) * ((O + 127) / 128) * (chunks >= 4 ? chunks / 2 : 1);
+        const size_t seg_rows = (H_out + sr - 1) / sr, segs_w = (W_out + sw - 1) / sw;
+        const bool half_full = H_out * W_out * 2 >= seg_rows * sr * segs_w * sw;
+        any_geometry = force_gen || (groups * 4 >= (size_t)device_cu_count() && (!sparse_patches || half_full || !conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N)));
+        if (any_geometry) fixed_geometry = false;
     }
     if (fixed_geometry || any_geometry) {
         // The reference's bias parameter is pixel-major ([1,1,H_out*W_out,O], src/Model.cu:252-256), while the kernels'

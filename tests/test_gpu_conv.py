@@ -127,13 +127,20 @@ def test_conv2d_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, k_w, stride, 
 CONV_ANY_GEOMETRY = [  # N, C, H, W, O, k_h, k_w, stride, pad, w_batch, per-pixel bias: enough 256-pixel segments for the
     # implicit-GEMM kernel that takes any kernel extent and stride (rows that allow 16-byte loads)
     (16, 16, 32, 32, 16, 5, 5, 1, 2, 1, False),     # 5x5, 32-wide segments of 8 rows, 64-channel tile
-    (32, 24, 33, 64, 70, 3, 3, 2, 1, 1, False),     # stride 2, two chunks (the second half empty), 128-channel tile with 70 channels
+    (32, 24, 33, 64, 70, 3, 3, 2, 1, 1, False),     # stride 2, two chunks (the second half empty), 70 channels in two 64-channel tiles
+    (256, 8, 32, 32, 70, 3, 3, 2, 1, 1, False),     # a workgroup for every compute unit: 128-channel tile with 70 channels
+    (64, 8, 32, 32, 65, 5, 5, 1, 2, 1, False),      # the same tile with one staging task per thread ...
+    (64, 8, 48, 192, 65, 3, 3, 3, 1, 1, False),     # ... and with three
     (16, 16, 48, 192, 8, 3, 3, 3, 1, 1, False),     # stride 3: three staging tasks per thread
     (4, 8, 66, 260, 9, 3, 3, 2, 1, 1, False),       # 130 output columns: one row per segment, the second half of it empty
     (40, 40, 20, 24, 130, 2, 3, 2, 0, 40, False),   # 2x3 kernel, no padding, per-sample weights, two channel tiles
     (32, 32, 30, 40, 64, 5, 5, 2, 3, 1, True),      # padding 3, per-pixel bias (turned into channel planes first)
     (64, 16, 14, 16, 32, 3, 3, 2, 1, 1, False),     # 7 x 8 outputs: a segment spans the whole image and more
     (4, 16, 40, 128, 16, 5, 5, 4, 2, 1, False),     # stride 4 with 128-wide... the tile does not fit a thread's staging share: column matrix
+    # few segments and many channels: the contraction split over groups of channel chunks, the groups' sums added by a
+    # second kernel (a 3x3 stride-1 layer whose weights are beyond LDS, and a 5x5 stride-2 one)
+    (16, 256, 16, 16, 64, 3, 3, 1, 1, 1, False),
+    (24, 96, 32, 32, 32, 5, 5, 2, 2, 1, True),
 ]
 
 
