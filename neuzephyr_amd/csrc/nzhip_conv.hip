@@ -1658,7 +1658,9 @@ __global__ __launch_bounds__(256) void conv_weight_image_gen_kernel(_Float16* __
 }
 
 // NO: 32-channel blocks per wave (BN / 64); every wave also owns two 32-pixel blocks. TP: staging tasks per thread.
-template <int NO, int TP>
+// VEC: image rows are whole 16-byte pieces (W a multiple of 4, aligned x): a task's four columns are one load per
+// channel and lie inside or outside the image together; otherwise (14 x 14 images ...) four loads with their own bounds.
+template <int NO, int TP, bool VEC>
 __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGenArgs p) {
     constexpr int BN = NO * 64;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -1682,17 +1684,20 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
 
     // staging tasks: task e = tid + 512 k is (8-channel half, staged row, column quad)
     const int pw4 = p.pw >> 2, n_tasks = 2 * p.span * pw4;
-    int t_off[TP], t_dst[TP];                                   // image offset of the quad (or -1), LDS byte offset of its first pixel
-    int t_h8[TP];
+    int t_off[TP], t_dst[TP];                                   // image offset of the quad's first column, LDS byte offset of its first pixel (or -1)
+    int t_h8[TP];                                               // bits 0..3: which of the four columns are inside the image; bit 4: the channel half
 #pragma unroll
     for (int k = 0; k < TP; k++) {
         const int e = tid + CG_THREADS * k;
         const int q = e % pw4, row = (e / pw4) % p.span, h8 = e / (pw4 * p.span);
         const int h = hb + row, w = wf + 4 * q;
-        const bool in = e < n_tasks && h >= 0 && h < p.H && w >= 0 && w < p.W;     // W % 4 == 0 and w % 4 == 0: the whole quad
-        t_off[k] = in ? h * p.W + w : -1;
+        const bool row_in = e < n_tasks && h >= 0 && h < p.H;
+        int mask = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) mask |= (row_in && w + j >= 0 && w + j < p.W) ? 1 << j : 0;     // VEC: all four or none
+        t_off[k] = h * p.W + w;
         t_dst[k] = e < n_tasks ? (row * p.pw + 4 * q) * 32 : -1;
-        t_h8[k] = h8;
+        t_h8[k] = mask | (h8 << 4);
     }
 
     floatx16 acc[NO][2];
@@ -1707,11 +1712,20 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
     auto load_halo = [&](const int chunk) {
 #pragma unroll
         for (int k = 0; k < TP; k++) {
-            const int c0 = chunk * IG_CC + t_h8[k] * 8;
+            const int c0 = chunk * IG_CC + (t_h8[k] >> 4) * 8;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const bool ok = t_off[k] >= 0 && c0 + e < p.C;
-                raw[k][e] = *reinterpret_cast<const floatx4*>(xb + (ok ? (long)(c0 + e) * plane + t_off[k] : 0));
+                const bool c_ok = c0 + e < p.C;
+                if (VEC) {
+                    const bool ok = (t_h8[k] & 1) && c_ok;
+                    raw[k][e] = *reinterpret_cast<const floatx4*>(xb + (ok ? (long)(c0 + e) * plane + t_off[k] : 0));
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const bool ok = (t_h8[k] >> j & 1) && c_ok;
+                        raw[k][e][j] = xb[ok ? (long)(c0 + e) * plane + t_off[k] + j : 0];
+                    }
+                }
             }
         }
     };
@@ -1719,15 +1733,16 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
 #pragma unroll
         for (int k = 0; k < TP; k++) {
             if (t_dst[k] < 0) continue;
-            const int c0 = chunk * IG_CC + t_h8[k] * 8;
+            const int h8 = t_h8[k] >> 4;
+            const int c0 = chunk * IG_CC + h8 * 8;
             const int col0 = (t_dst[k] >> 5) % p.pw;            // staged column of the quad's first pixel (a multiple of 4)
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 half8_t h;
 #pragma unroll
-                for (int e = 0; e < 8; e++) h[e] = (t_off[k] >= 0 && c0 + e < p.C) ? (_Float16)raw[k][e][q] : (_Float16)0.f;
+                for (int e = 0; e < 8; e++) h[e] = ((t_h8[k] >> q & 1) && c0 + e < p.C) ? (_Float16)raw[k][e][q] : (_Float16)0.f;
                 const int col = col0 + q;
-                *reinterpret_cast<half8_t*>(lds_h + t_dst[k] + q * 32 + ((t_h8[k] ^ ((col >> 3) & 1)) << 4)) = h;
+                *reinterpret_cast<half8_t*>(lds_h + t_dst[k] + q * 32 + ((h8 ^ ((col >> 3) & 1)) << 4)) = h;
             }
         }
     };
@@ -1869,7 +1884,8 @@ static bool conv_igemm_gen_applicable(const float* x, size_t C, size_t H, size_t
                                       size_t pad, size_t N) {
     (void)O;
     // (a strided 1x1 convolution has one tap per chunk to multiply between two barriers: its column matrix is the cheaper way)
-    return C >= 8 && W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && stride <= 4 && K_h * K_w >= 2 && K_h * K_w <= 64 && pad < 0x10000 &&
+    (void)x; (void)W;
+    return C >= 8 && stride <= 4 && K_h * K_w >= 2 && K_h * K_w <= 64 && pad < 0x10000 &&
            N <= 65535 && H * W < 0x7fffffffull && C * H * W < 0x7fffffffull;
 }
 
@@ -1942,8 +1958,13 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
         a.partial = partial;
     }
     const int tp = (int)((tasks + CG_THREADS - 1) / CG_THREADS);
-    auto kfn = BN == 128 ? (tp <= 1 ? conv_igemm_gen_kernel<2, 1> : tp == 2 ? conv_igemm_gen_kernel<2, 2> : conv_igemm_gen_kernel<2, 3>)
-                         : (tp <= 1 ? conv_igemm_gen_kernel<1, 1> : tp == 2 ? conv_igemm_gen_kernel<1, 2> : conv_igemm_gen_kernel<1, 3>);
+    const bool vec = W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    auto pick = [&](auto vec_tag) {
+        constexpr bool V = decltype(vec_tag)::value;
+        return BN == 128 ? (tp <= 1 ? conv_igemm_gen_kernel<2, 1, V> : tp == 2 ? conv_igemm_gen_kernel<2, 2, V> : conv_igemm_gen_kernel<2, 3, V>)
+                         : (tp <= 1 ? conv_igemm_gen_kernel<1, 1, V> : tp == 2 ? conv_igemm_gen_kernel<1, 2, V> : conv_igemm_gen_kernel<1, 3, V>);
+    };
+    auto kfn = vec ? pick(std::true_type{}) : pick(std::false_type{});
     int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_need, "hipFuncSetAttribute(conv_igemm_gen)");
     if (rc == NZHIP_OK) {
         hipLaunchKernelGGL(kfn, dim3((unsigned)(seg_rows * segs_w), (unsigned)n_otiles, (unsigned)(N * chunk_groups)), dim3(CG_THREADS),

@@ -141,6 +141,10 @@ CONV_ANY_GEOMETRY = [  # N, C, H, W, O, k_h, k_w, stride, pad, w_batch, per-pixe
     # second kernel (a 3x3 stride-1 layer whose weights are beyond LDS, and a 5x5 stride-2 one)
     (16, 256, 16, 16, 64, 3, 3, 1, 1, 1, False),
     (24, 96, 32, 32, 32, 5, 5, 2, 2, 1, True),
+    # rows that are not whole 16-byte pieces (14- and 30-wide images): staging with per-column bounds
+    (64, 16, 14, 14, 32, 5, 5, 1, 2, 1, False),
+    (64, 24, 21, 30, 70, 3, 3, 2, 1, 1, True),
+    (16, 256, 14, 14, 96, 3, 3, 1, 1, 1, False),    # ... with the contraction split (a 3x3 stride-1 layer, weights beyond LDS)
 ]
 
 
