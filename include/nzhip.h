@@ -219,9 +219,10 @@ int nzhip_conv2d_forward_prepared(float* y, const float* x, const float* w_ref, 
 /* Gradient of nzhip_conv2d_forward with respect to x, as one call. In the reference this is the chain
  * Col2ImgNode::backward (src/Nodes.cu:660-665) -> MatMulNode::backward, dA += dC * B^T (:169-182) ->
  * Img2ColNode::backward (:632-640; img2colBackwardKernel, src/OperationKernels.cu:1337-1362):
- *   dx[b][c][h][w] (+)= sum over r, s, o of f16(dy[b][o][h+pad-r][w+pad-s]) * f16(w_ref[wb][(c,r,s)][o])
- * accumulate != 0 adds into dx (what the chain does), 0 overwrites it. Supported: stride 1, K_h == K_w,
- * pad <= K_h - 1; anything else returns NZHIP_E_UNSUPPORTED and the caller runs the chain. */
+ *   dx[b][c][h][w] (+)= sum over r, s, o of f16(dy[b][o][ho][wo]) * f16(w_ref[wb][(c,r,s)][o])
+ *   with ho * stride = h + pad - r, wo * stride = w + pad - s
+ * accumulate != 0 adds into dx (what the chain does), 0 overwrites it. Supported: K_h == K_w, pad <= K_h - 1,
+ * stride <= 8; anything else returns NZHIP_E_UNSUPPORTED and the caller runs the chain. */
 int nzhip_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
                                size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
                                size_t w_batch, int accumulate, void* stream);

@@ -2575,10 +2575,44 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
                                bias_stride_channel, 0, activation, stream);
 }
 
-/* Gradient of nzhip_conv2d_forward with respect to x for stride 1: one convolution of dy with the
+namespace nzhip {
+// dst[plane][h][w] = src[plane][h / stride][w / stride] where both divide and the source pixel exists, else 0: the output
+// gradient of a strided convolution spread out to the positions its windows started at (H_up = H + 2 pad - K + 1 rows).
+// A thread writes four adjacent columns of one row (VEC: as one 16-byte store; Wu a multiple of 4, aligned dst).
+template <bool VEC>
+__global__ __launch_bounds__(256) void upsample_zero_kernel(float* __restrict__ dst, const float* __restrict__ src, long quads, int Ho,
+                                                            int Wo, int Hu, int Wu, int stride) {
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= quads) return;
+    const int wq = (Wu + 3) >> 2;
+    const int w0 = (int)(t % wq) * 4, h = (int)((t / wq) % Hu);
+    const long plane = t / ((long)wq * Hu);
+    const int ho = h / stride;
+    const bool row_hit = ho * stride == h && ho < Ho;
+    const float* srow = src + (plane * Ho + (row_hit ? ho : 0)) * Wo;
+    floatx4 v;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int w = w0 + j, wo = w / stride;
+        const bool hit = row_hit && wo * stride == w && wo < Wo;
+        v[j] = hit ? srow[wo] : 0.f;
+    }
+    float* drow = dst + (plane * Hu + h) * Wu + w0;
+    if (VEC) {
+        *reinterpret_cast<floatx4*>(drow) = v;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (w0 + j < Wu) drow[j] = v[j];
+    }
+}
+}  // namespace nzhip
+
+/* Gradient of nzhip_conv2d_forward with respect to x: one convolution of dy with the
  * mirrored weights instead of the reference's chain Col2ImgNode::backward -> MatMulNode::backward
  * (dA += dC * B^T) -> Img2ColNode::backward (src/Nodes.cu:660-665, 169-182, 632-640), which writes and
- * re-reads a column-matrix gradient of K_h*K_w times the size of x. */
+ * re-reads a column-matrix gradient of K_h*K_w times the size of x. With a stride above 1 the output gradient is first
+ * spread out with zeros between its pixels; the stride-1 convolution of that is the same sum. */
 extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
                                           size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
                                           size_t w_batch, int accumulate, void* stream) {
@@ -2588,11 +2622,27 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     if (w_batch != 1 && w_batch != N) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
     if (H + 2 * pad < K_h || W + 2 * pad < K_w)
         return set_error(NZHIP_E_SHAPE, "nzhip_conv2d_backward_data: kernel larger than the padded input");
-    if (stride != 1 || K_h != K_w || pad > K_h - 1)
+    if (stride > 8 || K_h != K_w || pad > K_h - 1)
         return set_error(NZHIP_E_UNSUPPORTED,
-                         "nzhip_conv2d_backward_data: only stride 1, square kernels and pad <= K-1 (use the column-matrix chain)");
+                         "nzhip_conv2d_backward_data: only square kernels, pad <= K-1 and stride <= 8 (use the column-matrix chain)");
     if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (stride > 1) {
+        const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
+        const size_t Hu = H + 2 * pad - K_h + 1, Wu = W + 2 * pad - K_w + 1, total = N * O * Hu * Wu;
+        const size_t quads = N * O * Hu * ((Wu + 3) / 4);
+        if (Hu > 0x3fffffff || Wu > 0x3fffffff || (quads + 255) / 256 > 0x7fffffffull)
+            return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_data: extents beyond the fused kernels (use the column-matrix chain)");
+        float* up = nullptr;
+        if (int rc = workspace_alloc(reinterpret_cast<void**>(&up), total * sizeof(float), s)) return rc;
+        hipLaunchKernelGGL(Wu % 4 == 0 ? upsample_zero_kernel<true> : upsample_zero_kernel<false>, dim3((unsigned)((quads + 255) / 256)),
+                           dim3(256), 0, s, up, dy, (long)quads, (int)Ho, (int)Wo, (int)Hu, (int)Wu, (int)stride);
+        hipError_t e = hipGetLastError();
+        int rc = e == hipSuccess ? NZHIP_OK : set_hip_error(e, "upsample_zero kernel launch");
+        if (rc == NZHIP_OK) rc = nzhip_conv2d_backward_data(dx, up, w_ref, N, C, H, W, O, K_h, K_w, 1, pad, w_batch, accumulate, stream);
+        const int rc2 = workspace_free(up, s);
+        return rc ? rc : rc2;
+    }
     const size_t H_out = H + 2 * pad - K_h + 1, W_out = W + 2 * pad - K_w + 1;
     const size_t w_elems = w_batch * C * K_h * K_w * O, x_elems = N * C * H * W;
     float* wflip = nullptr;

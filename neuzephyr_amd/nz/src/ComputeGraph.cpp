@@ -71,6 +71,23 @@ namespace nz::graph {
         T* as(Node* n, const char* type) {
             return (n && n->type == type) ? dynamic_cast<T*>(n) : nullptr;
         }
+
+        // Data gradient of a strided convolution: as ONE convolution it runs on the output gradient spread out with zeros,
+        // stride^2 times the multiply-adds; the column-matrix chain does the real ones but writes and re-reads a column
+        // gradient of K^2 / stride^2 times the input. Estimates in microseconds from rates measured on the MI355X
+        // (resident-weight convolution 600 TFLOP/s, otherwise 300; chain product 400 TFLOP/s; 4-5 TB/s of traffic); the
+        // estimates are both about half the measured times, and the convolution is favoured up to 1.5x because its
+        // measured side came out better than estimated on every shape tried (16x64x128x128 -> 128, 3x3 stride 2: 101
+        // against 269 us; 16x256x28x28 -> 512: 205 against 93 us, which this rule leaves to the chain).
+        bool stridedDataGradientAsConvolution(size_t N, size_t C, size_t H, size_t W, size_t O, size_t K, size_t stride, size_t pad) {
+            const double Ho = static_cast<double>((H + 2 * pad - K) / stride + 1), Wo = static_cast<double>((W + 2 * pad - K) / stride + 1);
+            const double Hu = static_cast<double>(H + 2 * pad - K + 1), Wu = static_cast<double>(W + 2 * pad - K + 1);
+            const double flops = 2.0 * N * Ho * Wo * C * K * K * O;
+            const bool resident = ((O + 15) / 16) * (C > 64 ? 128 : 64) * K * K * 32 <= 148 * 1024;
+            const double asConvolution = stride * stride * flops / (resident ? 600e6 : 300e6) + N * O * Hu * Wu * 4.0 / 5e6;
+            const double asChain = flops / 400e6 + 3.0 * N * Ho * Wo * C * K * K * 4.0 / 4e6;
+            return asConvolution < 1.5 * asChain;
+        }
     }
 
     // Turns the sorted node list into the list of calls forward() makes. A chain is fused only if
@@ -141,7 +158,14 @@ namespace nz::graph {
                     // Add.backward, MatMul.backward for B with the column matrix recomputed); the data gradient
                     // as one convolution of dZ. Same accumulate / overwrite behaviour as the node chain.
                     std::function<void()> back;
-                    if (i2c->stride == 1 && i2c->kernelHeight == i2c->kernelWidth && i2c->padding <= i2c->kernelHeight - 1) {
+                    // (the data gradient as one convolution needs a square kernel whose padding stays inside it and a stride up
+                    // to 8; a chain whose input carries no gradient does not need it at all)
+                    const bool dataGradientFused =
+                        i2c->kernelHeight == i2c->kernelWidth && i2c->padding <= i2c->kernelHeight - 1 && i2c->stride >= 1 &&
+                        i2c->stride <= 8 &&
+                        (i2c->stride == 1 || stridedDataGradientAsConvolution(xs[0], xs[1], xs[2], xs[3], O, i2c->kernelHeight,
+                                                                              i2c->stride, i2c->padding));
+                    {
                         Node* pre = add ? static_cast<Node*>(add) : static_cast<Node*>(mm);   // holds [N,1,HW,O] gradients
                         back = [=] {
                             if (!last->output->requiresGrad()) return;     // nothing in the chain carries a gradient
@@ -188,9 +212,24 @@ namespace nz::graph {
                                 iMatMulBackward(nullptr, rhs->output->grad(), i2c->output->data(), rhs->output->data(), dPre,
                                                 i2c->output->shape(), rhs->output->shape(), mm->output->shape());
                             }
-                            if (x->output->requiresGrad())
-                                iConv2dBackwardData(x->output->grad(), dZ, rhs->output->data(), xs[0], xs[1], xs[2], xs[3], O,
-                                                    i2c->kernelHeight, i2c->kernelWidth, i2c->stride, i2c->padding, ws[0]);
+                            if (x->output->requiresGrad()) {
+                                const bool asConvolution =
+                                    dataGradientFused && iConv2dBackwardData(x->output->grad(), dZ, const_cast<float*>(rhs->output->constData()),
+                                                                             xs[0], xs[1], xs[2], xs[3], O, i2c->kernelHeight, i2c->kernelWidth,
+                                                                             i2c->stride, i2c->padding, ws[0]);
+                                if (!asConvolution) {
+                                    // the reference's chain for this one gradient: dCol = dPre * W^T, then the gather into dx
+                                    if (O != 1 && dPre == dZ) {
+                                        dPre = pre->output->gradOverwrite();
+                                        iCol2imgBackward(dPre, dZ, c2i->outputHeight, c2i->outputWidth, O, xs[0]);
+                                    }
+                                    i2c->output->zeroGrad();
+                                    iMatMulBackward(i2c->output->grad(), nullptr, nullptr, const_cast<float*>(rhs->output->constData()), dPre, i2c->output->shape(),
+                                                    rhs->output->shape(), mm->output->shape());
+                                    iImg2colBackward(x->output->grad(), i2c->output->grad(), c2i->outputHeight, c2i->outputWidth, xs[1],
+                                                     i2c->kernelHeight, i2c->kernelWidth, i2c->stride, i2c->padding, xs[2], xs[3], xs[0]);
+                                }
+                            }
                         };
                     }
                     // The fp16 image of the weights survives between forward passes while nobody has asked the

@@ -208,7 +208,7 @@ namespace nz::data {
     bool iConv2dBackwardData(float* dx, float* dy, float* w, const size_t N, const size_t C, const size_t H,
                              const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
                              const size_t pad, const size_t weightBatch) {
-        if (stride != 1 || K_h != K_w || pad > K_h - 1) return false;
+        if (stride < 1 || stride > 8 || K_h != K_w || pad > K_h - 1) return false;
         NZ_CHECK(nzhip_conv2d_backward_data(dx, dy, w, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch, 1,
                                             nzhip_default_stream()));
         return true;

@@ -626,7 +626,10 @@ TEST(Model, Conv2dFusedBackwardEqualsNodeChain) {
     convBackwardFusedEqualsChain(1, 16, 12, 40, 24, 3, 1, 1, true);   // implicit-GEMM kernels
     convBackwardFusedEqualsChain(2, 4, 6, 6, 3, 1, 1, 0, false);      // 1x1, no activation
     convBackwardFusedEqualsChain(3, 20, 8, 10, 33, 1, 1, 0, true);    // 1x1: the weight gradient is one batched product of x and the gradient
-    convBackwardFusedEqualsChain(2, 3, 9, 8, 4, 3, 2, 1, true);       // stride 2: weights by the gather kernel; the data gradient falls back to the nodes
+    convBackwardFusedEqualsChain(2, 3, 9, 8, 4, 3, 2, 1, true);       // stride 2: weights by the gather kernel, the data gradient from the spread-out output gradient
+    convBackwardFusedEqualsChain(2, 5, 14, 12, 6, 5, 3, 2, true);     // stride 3, 5x5, rows and columns no window reaches
+    convBackwardFusedEqualsChain(1, 16, 20, 24, 8, 3, 2, 0, false);   // stride 2, no padding, no activation
+    convBackwardFusedEqualsChain(2, 128, 12, 12, 256, 3, 2, 1, true); // stride 2 with many channels on small images: the data gradient through the column-matrix gradient inside the fused backward
     convBackwardFusedEqualsChain(2, 6, 14, 20, 10, 5, 1, 2, true);    // 5x5: weights by the gather kernel
     convBackwardFusedEqualsChain(2, 40, 10, 136, 36, 3, 1, 1, true);  // W a multiple of 8: weights without the column matrix
 }

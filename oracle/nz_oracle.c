@@ -396,17 +396,18 @@ void nzo_col2im_backward(float* dcol, const float* dy, size_t H_out, size_t W_ou
     }
 }
 
-/* Data gradient of the Model::Conv2d graph in one statement (stride 1). The reference computes it
+/* Data gradient of the Model::Conv2d graph in one statement. The reference computes it
  * as the chain Col2ImgNode::backward (src/Nodes.cu:660-665) -> MatMulNode::backward, dA += dC * B^T
  * with fp16-rounded operands and fp32 accumulation (:169-182) -> Img2ColNode::backward (:632-640,
  * img2colBackwardKernel, src/OperationKernels.cu:1337-1362). Composed:
- *   dx[b][c][h][w] += sum over r, s, o of f16(dy[b][o][h+pad-r][w+pad-s]) * f16(W[wb][(c,r,s)][o])
- * for the (r, s) whose output position exists. Here o runs innermost in ascending order inside each
- * (r, s), then the taps in ascending (r, s): the grouping of the chain (a dot product over o per
- * column-matrix entry, then one addition per tap). */
-void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
-                              size_t W, size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch) {
-    const size_t H_out = H + 2 * pad - K_h + 1, W_out = W + 2 * pad - K_w + 1, CKK = C * K_h * K_w;
+ *   dx[b][c][h][w] += sum over r, s, o of f16(dy[b][o][ho][wo]) * f16(W[wb][(c,r,s)][o])
+ * for the (r, s) with ho * stride = h + pad - r and wo * stride = w + pad - s inside the output. Here o runs
+ * innermost in ascending order inside each (r, s), then the taps in ascending (r, s): the grouping of the
+ * chain (a dot product over o per column-matrix entry, then one addition per tap). */
+void nzo_conv2d_backward_data_strided(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
+                                      size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                                      size_t w_batch) {
+    const size_t H_out = (H + 2 * pad - K_h) / stride + 1, W_out = (W + 2 * pad - K_w) / stride + 1, CKK = C * K_h * K_w;
     float* dyr = (float*)malloc(sizeof(float) * N * O * H_out * W_out);
     float* wr = (float*)malloc(sizeof(float) * w_batch * CKK * O);
     nzo_round_f16_array(dyr, dy, N * O * H_out * W_out);
@@ -420,8 +421,10 @@ void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, si
                     float g = dx[((b * C + c) * H + h) * W + w];
                     for (size_t r = 0; r < K_h; r++)
                         for (size_t s = 0; s < K_w; s++) {
-                            const long long ho = (long long)(h + pad) - (long long)r, wo = (long long)(w + pad) - (long long)s;
-                            if (ho < 0 || ho >= (long long)H_out || wo < 0 || wo >= (long long)W_out) continue;
+                            const long long hs = (long long)(h + pad) - (long long)r, ws = (long long)(w + pad) - (long long)s;
+                            if (hs < 0 || ws < 0 || hs % (long long)stride || ws % (long long)stride) continue;
+                            const long long ho = hs / (long long)stride, wo = ws / (long long)stride;
+                            if (ho >= (long long)H_out || wo >= (long long)W_out) continue;
                             const float* wrow = wb + ((c * K_h + r) * K_w + s) * O;
                             float dot = 0.0f;
                             for (size_t o = 0; o < O; o++)
@@ -433,6 +436,11 @@ void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, si
         }
     free(dyr);
     free(wr);
+}
+
+void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
+                              size_t W, size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch) {
+    nzo_conv2d_backward_data_strided(dx, dy, w_ref, N, C, H, W, O, K_h, K_w, 1, pad, w_batch);
 }
 
 /* Weight gradient of the Model::Conv2d graph in one statement: MatMulNode::backward's

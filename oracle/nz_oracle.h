@@ -144,6 +144,10 @@ void nzo_conv2d_backward_weights_strided(float* dw, const float* x, const float*
                                          size_t w_batch);
 void nzo_conv2d_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W,
                                  size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch);
+/* dx += data gradient of the Conv2d graph (Nodes.cu:660-665, 169-182, 632-640); dy [N,O,H_out,W_out], dx [N,C,H,W]. */
+void nzo_conv2d_backward_data_strided(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
+                                      size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                                      size_t w_batch);
 void nzo_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
                               size_t W, size_t O, size_t K_h, size_t K_w, size_t pad, size_t w_batch);
 

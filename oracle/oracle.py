@@ -83,7 +83,7 @@ _relu_bwd = _sig("nzo_relu_backward", None, _f32p, _f32p, _f32p, _sz)
 _add_bwd = _sig("nzo_add_backward", None, _f32p, _f32p, _Shape, _Shape)
 _im2col_bwd = _sig("nzo_im2col_backward", None, _f32p, _f32p, *([_sz] * 10))
 _col2im_bwd = _sig("nzo_col2im_backward", None, _f32p, _f32p, _sz, _sz, _sz, _sz)
-_conv_bwd_data = _sig("nzo_conv2d_backward_data", None, _f32p, _f32p, _f32p, *([_sz] * 9))
+_conv_bwd_data = _sig("nzo_conv2d_backward_data_strided", None, _f32p, _f32p, _f32p, *([_sz] * 10))
 _conv_bwd_w = _sig("nzo_conv2d_backward_weights_strided", None, _f32p, _f32p, _f32p, *([_sz] * 10))
 _softmax = _sig("nzo_softmax", None, _f32p, _f32p, _sz, _sz)
 _softmax_jac = _sig("nzo_softmax_jacobian", None, _f32p, _f32p, _sz, _sz)
@@ -297,14 +297,14 @@ def conv2d_backward_weights(dw: np.ndarray, x: np.ndarray, dy: np.ndarray, K_h: 
     return dw
 
 
-def conv2d_backward_data(dx: np.ndarray, dy: np.ndarray, w_ref: np.ndarray, K_h: int, K_w: int, pad: int) -> np.ndarray:
-    """dx += gradient of the stride-1 Conv2d graph with respect to its input (in place, returns dx)."""
+def conv2d_backward_data(dx: np.ndarray, dy: np.ndarray, w_ref: np.ndarray, K_h: int, K_w: int, pad: int, stride: int = 1) -> np.ndarray:
+    """dx += gradient of the Conv2d graph with respect to its input (in place, returns dx)."""
     dy, w_ref = _c(dy), _c(w_ref)
     assert dx.dtype == np.float32 and dx.flags.c_contiguous
     N, Cc, H, W = dx.shape
     O = dy.shape[1]
-    assert dy.shape == (N, O, H + 2 * pad - K_h + 1, W + 2 * pad - K_w + 1) and w_ref.shape[2:] == (Cc * K_h * K_w, O)
-    _conv_bwd_data(dx.reshape(-1), dy.reshape(-1), w_ref.reshape(-1), N, Cc, H, W, O, K_h, K_w, pad, w_ref.shape[0])
+    assert dy.shape == (N, O, (H + 2 * pad - K_h) // stride + 1, (W + 2 * pad - K_w) // stride + 1) and w_ref.shape[2:] == (Cc * K_h * K_w, O)
+    _conv_bwd_data(dx.reshape(-1), dy.reshape(-1), w_ref.reshape(-1), N, Cc, H, W, O, K_h, K_w, stride, pad, w_ref.shape[0])
     return dx
 
 

@@ -263,11 +263,33 @@ def test_conv2d_backward_data_float_tolerance_and_adjoint(nz, oracle):
     assert abs(lhs - rhs) <= 1e-4 * max(abs(lhs), abs(rhs), 1.0)
 
 
+CONV_BWD_DATA_STRIDED = [  # N, C, H, W, O, K, stride, pad, w_batch: rows and columns no window reaches, strides 2..4, per-sample weights
+    (2, 3, 7, 8, 4, 3, 2, 1, 1), (1, 2, 9, 9, 3, 3, 2, 0, 1), (2, 2, 11, 10, 2, 5, 3, 2, 2), (1, 3, 8, 6, 2, 1, 2, 0, 1),
+    (2, 16, 21, 36, 24, 3, 2, 1, 1), (1, 64, 32, 64, 128, 3, 2, 1, 1), (3, 8, 17, 33, 70, 5, 2, 2, 3), (2, 24, 30, 40, 16, 3, 4, 1, 1),
+    (8, 32, 28, 28, 64, 3, 2, 1, 1)]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,K,stride,pad,wb", CONV_BWD_DATA_STRIDED)
+@pytest.mark.parametrize("accumulate", [True, False])
+def test_strided_conv2d_backward_data_is_exact_on_integers(nz, oracle, N, C, H, W, O, K, stride, pad, wb, accumulate):
+    rng = np.random.default_rng(N * 131 + C * 17 + H * 7 + W + O * 3 + K + stride)
+    Ho, Wo = (H + 2 * pad - K) // stride + 1, (W + 2 * pad - K) // stride + 1
+    dy = rng.integers(-4, 5, size=(N, O, Ho, Wo)).astype(np.float32)
+    w = rng.integers(-4, 5, size=(wb, 1, C * K * K, O)).astype(np.float32)
+    dx0 = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    expect = oracle.conv2d_backward_data(dx0.copy() if accumulate else np.zeros_like(dx0), dy, w, K, K, pad, stride)
+    got = host(nz.conv2d_backward_data(dev(dx0), dev(dy), dev(w), K, K, stride, pad, accumulate=accumulate))
+    assert np.array_equal(got, expect)
+
+
 def test_conv2d_backward_data_rejects_what_it_does_not_cover(nz):
     from neuzephyr_amd.capi import NzHipError
-    dx, dy, w = dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 4, 4))), dev(np.zeros((1, 1, 18, 3)))
+    dx, dy, w = dev(np.zeros((1, 2, 8, 8))), dev(np.zeros((1, 3, 7, 3))), dev(np.zeros((1, 1, 2 * 2 * 6, 3)))
     with pytest.raises(NzHipError):
-        nz.conv2d_backward_data(dx, dy, w, 3, 3, 2, 1)
+        nz.conv2d_backward_data(dx, dy, w, 2, 6, 1, 0)              # a kernel that is not square
+    dx, dy, w = dev(np.zeros((1, 2, 40, 40))), dev(np.zeros((1, 3, 5, 5))), dev(np.zeros((1, 1, 18, 3)))
+    with pytest.raises(NzHipError):
+        nz.conv2d_backward_data(dx, dy, w, 3, 3, 9, 1)              # stride above 8
 
 
 CONV_BWD_W = [  # N, C, H, W, O, w_batch   (3x3, stride 1, pad 1; W a multiple of 8 takes 16-byte loads)

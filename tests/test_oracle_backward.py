@@ -129,6 +129,25 @@ def test_col2im_backward_loop_nest_and_inverse(oracle):
     assert np.array_equal(oracle.col2im(got, h, w).reshape(-1), exp)   # inverse of the forward transpose
 
 
+@pytest.mark.parametrize("N,C,H,W,O,K,stride,pad,wb", [(2, 3, 7, 8, 4, 3, 2, 1, 1), (1, 2, 9, 9, 3, 3, 2, 0, 1), (2, 2, 11, 10, 2, 5, 3, 2, 2),
+                                                        (1, 3, 8, 6, 2, 1, 2, 0, 1), (2, 3, 10, 12, 3, 3, 4, 1, 1), (1, 2, 7, 7, 2, 2, 2, 1, 1)])
+def test_strided_conv2d_backward_data_equals_the_pinned_chain(oracle, N, C, H, W, O, K, stride, pad, wb):
+    # the strided form of the statement below against the same chain (Img2Col.backward takes the stride), including
+    # input rows and columns the strided windows never reach (their gradient stays what it was), and the adjoint identity
+    rng = np.random.default_rng(N + 10 * C + 100 * H + O + 7 * stride)
+    Ho, Wo = (H + 2 * pad - K) // stride + 1, (W + 2 * pad - K) // stride + 1
+    dy = rng.integers(-4, 5, size=(N, O, Ho, Wo)).astype(np.float32)
+    w = rng.integers(-4, 5, size=(wb, 1, C * K * K, O)).astype(np.float32)
+    dx0 = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    got = oracle.conv2d_backward_data(dx0.copy(), dy, w, K, K, pad, stride)
+    col = np.zeros((N, 1, Ho * Wo, C * K * K), np.float32)
+    dcol, _ = oracle.matmul_backward(col, w, oracle.col2im_backward(dy), dA0=np.zeros_like(col))
+    assert np.array_equal(got, oracle.im2col_backward(dx0, dcol, K, K, stride, pad))
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    y = oracle.col2im(oracle.tensorcore_gemm(oracle.im2col(x, K, K, stride, pad), w), Ho, Wo)
+    assert float((y.astype(np.float64) * dy).sum()) == float((x.astype(np.float64) * (got - dx0)).sum())
+
+
 @pytest.mark.parametrize("N,C,H,W,O,K,pad,wb", [(2, 3, 5, 6, 4, 3, 1, 1), (1, 2, 4, 4, 3, 3, 0, 1), (2, 2, 6, 5, 2, 3, 2, 2),
                                                  (1, 3, 5, 5, 2, 1, 0, 1), (3, 4, 7, 9, 5, 3, 1, 3)])
 def test_conv2d_backward_data_equals_the_pinned_chain(oracle, N, C, H, W, O, K, pad, wb):
