@@ -634,6 +634,46 @@ TEST(Model, Conv2dFusedBackwardEqualsNodeChain) {
     convBackwardFusedEqualsChain(2, 40, 10, 136, 36, 3, 1, 1, true);  // W a multiple of 8: weights without the column matrix
 }
 
+struct RectConvGradModel : nz::Model {
+    InputNode input;
+    RectConvGradModel(size_t n, size_t c, size_t h, size_t w, size_t o, size_t kh, size_t kw, size_t stride, size_t pad)
+        : input({n, c, h, w}, true) {
+        defaultOutput(ReLU(Conv2d(&input, o, kh, kw, stride, pad)));
+    }
+};
+
+TEST(Model, Conv2dFusedBackwardWithAKernelThatIsNotSquare) {
+    // 2 x 3 kernel, stride 2: weights by the gather kernel, bias in one pass, the data gradient through the column-matrix
+    // gradient inside the fused backward; all equal to the node chain on integers
+    const size_t n = 2, c = 5, h = 10, w = 12, o = 6, kh = 2, kw = 3, stride = 2, pad = 1;
+    RectConvGradModel m(n, c, h, w, o, kh, kw, stride, pad);
+    auto ints = [](size_t count, unsigned seed, int lo, int hi) {
+        auto v = randomVec(count, seed, static_cast<float>(lo), static_cast<float>(hi) + 0.999f);
+        for (auto& e : v) e = std::floor(e);
+        return v;
+    };
+    const size_t Ho = (h + 2 * pad - kh) / stride + 1, Wo = (w + 2 * pad - kw) / stride + 1;
+    auto x = ints(n * c * h * w, 81, -3, 3), W = ints(n * c * kh * kw * o, 82, -2, 2), b = ints(Ho * Wo * o, 83, -4, 4);
+    m.input.dataInject(x.begin(), x.end());
+    m.parameters()[0]->dataInject(W.begin(), W.end());
+    m.parameters()[1]->dataInject(b.begin(), b.end());
+    m.graph().zeroGrad();
+    m.forward();
+    EXPECT_EQ(m.graph().fusedGroupCount(), 1u);
+    m.backward();
+    const auto dx = m.input.output->hostGrad(), dW = m.parameters()[0]->output->hostGrad(), db = m.parameters()[1]->output->hostGrad();
+    m.graph().setFusion(false);
+    m.graph().zeroGrad();
+    m.forward();
+    m.backward();
+    EXPECT_TRUE(m.input.output->hostGrad() == dx);
+    EXPECT_TRUE(m.parameters()[0]->output->hostGrad() == dW);
+    EXPECT_TRUE(m.parameters()[1]->output->hostGrad() == db);
+    bool anyX = false;
+    for (float v : dx) anyX = anyX || v != 0.f;
+    EXPECT_TRUE(anyX);
+}
+
 struct LinearGradModel : nz::Model {
     InputNode input;
     LinearGradModel(size_t batch, size_t features, size_t out, bool relu) : input({batch, 1, features, 1}, true) {
