@@ -2855,93 +2855,11 @@ struct ConvDwGenArgs {
     int sw_log;            // log2 of the segment width SW; a segment is 128 / SW output rows x SW output columns
     int span;              // staged input rows per channel: (128 / SW - 1) * stride + Kh
     int bands, band_rows, n_images;
+    int ipw, n_groups;     // images per workgroup and groups of that many images (partial sums: one region per group and band)
 };
 
-// Rows that do not allow 16-byte loads: staged element by element, four waves, 128 rows per workgroup.
-__global__ __launch_bounds__(256) void conv_dwg_kernel(const ConvDwGenArgs p) {
-    extern __shared__ __attribute__((aligned(16))) char lds[];
-    _Float16* xs = reinterpret_cast<_Float16*>(lds);                                   // [cc * Kh][pw]
-    _Float16* zs = xs + ((p.cc * p.span * p.pw + 7) & ~7);                              // [DWG_OT][DWG_ZPITCH]
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int li = lane & 31, lh = lane >> 5;
-    const int band = blockIdx.x % p.bands, img = blockIdx.x / p.bands;
-    const int c0 = blockIdx.y * p.cc, o0 = blockIdx.z * DWG_OT;
-    const int taps = p.Kh * p.Kw;
-    const int nch = (p.C - c0) < p.cc ? (p.C - c0) : p.cc;
-    const int h_begin = band * p.band_rows;
-    const int h_end = (h_begin + p.band_rows) < p.Ho ? (h_begin + p.band_rows) : p.Ho;
-    const float* ximg = p.x + ((long)img * p.C + c0) * p.H * p.W;
-    const float* zimg = p.dy + ((long)img * p.O + o0) * p.Ho * p.Wo;
-
-    floatx16 acc[DWG_NB];
-#pragma unroll
-    for (int j = 0; j < DWG_NB; j++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
-
-    // this lane's row of the tile: (channel, tap row, tap column); rows past the last channel multiply zeros
-    const int m = wave * 32 + li;
-    const bool row_live = m < nch * taps;
-    const int mc = row_live ? m / taps : 0, mt = row_live ? m % taps : 0;
-    const int a_base = (mc * p.span + mt / p.Kw) * p.pw + mt % p.Kw + p.shift + 8 * lh * p.stride;
-    const int rows_staged = nch * p.span;
-    const int SW = 1 << p.sw_log, SR = DWG_PX >> p.sw_log;
-    const int segs = (p.Wo + SW - 1) >> p.sw_log;
-
-    for (int ho = h_begin; ho < h_end; ho += SR) {
-        for (int seg = 0; seg < segs; seg++) {
-            const int wo0 = seg * SW;
-            const int w_first = wo0 * p.stride - p.pad - p.shift;               // image column of staged column 0
-            {
-                const int n_stage = rows_staged * p.pw;
-                for (int e = tid; e < n_stage; e += 256) {
-                    const int row = e / p.pw, col = e - row * p.pw;
-                    const int c = row / p.span, r = row - c * p.span;
-                    const int h = ho * p.stride - p.pad + r, w = w_first + col;
-                    const bool in = h >= 0 && h < p.H && w >= 0 && w < p.W;
-                    const float v = ximg[((long)c * p.H + (in ? h : 0)) * p.W + (in ? w : 0)];
-                    xs[e] = (_Float16)(in ? v : 0.f);
-                }
-                for (int e = tid; e < DWG_OT * DWG_PX; e += 256) {
-                    const int o = e / DWG_PX, k = e % DWG_PX;
-                    const int kr = k >> p.sw_log, kc = k & (SW - 1);
-                    const bool in = o0 + o < p.O && wo0 + kc < p.Wo && ho + kr < h_end;
-                    const float v = zimg[((long)(in ? o : 0) * p.Ho + (in ? ho + kr : 0)) * p.Wo + (in ? wo0 + kc : 0)];
-                    zs[o * DWG_ZPITCH + k] = (_Float16)(in ? v : 0.f);
-                }
-            }
-            __syncthreads();
-#pragma unroll 2
-            for (int ks = 0; ks < DWG_PX / 16; ks++) {
-                half8_t af;
-                // pixels 16 ks .. 16 ks + 15 of the segment: output row (16 ks) / SW, columns from (16 ks) % SW
-                const _Float16* ap = xs + a_base + (((ks * 16) >> p.sw_log) * p.pw + ((ks * 16) & (SW - 1))) * p.stride;
-#pragma unroll
-                for (int j = 0; j < 8; j++) af[j] = row_live ? ap[j * p.stride] : (_Float16)0.f;
-#pragma unroll
-                for (int j = 0; j < DWG_NB; j++) {
-                    const half8_t bf = *reinterpret_cast<const half8_t*>(zs + (j * 32 + li) * DWG_ZPITCH + ks * 16 + lh * 8);
-                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf, acc[j], 0, 0, 0);
-                }
-            }
-            __syncthreads();
-        }
-    }
-    // accumulator (block j, register r): row 32 wave + (r >> 2) * 8 + lh * 4 + (r & 3), column 32 j + li
-    float* out = p.partial + ((((long)blockIdx.y * gridDim.z + blockIdx.z) * p.n_images + img) * p.bands + band) * (DWG_ROWS * DWG_OT);
-#pragma unroll
-    for (int j = 0; j < DWG_NB; j++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int row = wave * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-            out[row * DWG_OT + j * 32 + li] = acc[j][r];
-        }
-}
-
-// The same product for rows that allow 16-byte loads (W and Wo multiples of 4, x and dy 16-byte aligned), on eight
-// waves: a workgroup owns up to 256 rows (channel, tap) x 128 output channels, so a dy segment is fetched half as
-// often, and the requests for the NEXT segment are issued before the current one multiplies. A thread's share of a
+// Eight waves: a workgroup owns up to 256 rows (channel, tap) x 128 output channels, and the requests for the NEXT
+// segment are issued before the current one multiplies. A thread's share of a
 // segment is a fixed set of 16-byte pieces (DWG8_XMAX of the input rows, 8 of dy) whose place in the tile does not
 // depend on the segment, so the index arithmetic is done once; per segment only the image row and column move.
 // Requests are unconditional (clamped addresses, zero selected when the piece is stored), so the compiler's waits
@@ -2951,7 +2869,11 @@ constexpr int DWG8_ROWS = 256, DWG8_XMAX = 7, DWG8_THREADS = 512;
 // XP: 16-byte pieces of the staged input rows per thread (the tile has at most 512 XP of them)
 // S1: stride 1. A lane's eight pixels are then eight consecutive halfs of a staged row: five dword reads and four
 // v_alignbit (by 0 or 16 bits, the parity of the lane's tap column) instead of eight 16-bit reads.
-template <int XP, bool S1>
+// VEC: rows of x and dy are whole 16-byte pieces (W and Wo multiples of 4, aligned tensors); otherwise a piece's four
+// columns are loaded one by one with their own bounds (14-wide images ...).
+// A workgroup walks the segments of its band in p.ipw consecutive images (small images: one segment each, and one
+// set of partial sums per group of images instead of one per image).
+template <int XP, bool S1, bool VEC>
 __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGenArgs p) {
     extern __shared__ __attribute__((aligned(16))) char lds[];
     _Float16* xs = reinterpret_cast<_Float16*>(lds);                                   // [cc * span][pw]
@@ -2959,14 +2881,16 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, lh = lane >> 5;
-    const int band = blockIdx.x % p.bands, img = blockIdx.x / p.bands;
+    const int band = blockIdx.x % p.bands, group = blockIdx.x / p.bands;
+    const int img0 = group * p.ipw, n_img = (p.n_images - img0) < p.ipw ? (p.n_images - img0) : p.ipw;
     const int c0 = blockIdx.y * p.cc, o0 = blockIdx.z * DWG_OT;
     const int taps = p.Kh * p.Kw;
     const int nch = (p.C - c0) < p.cc ? (p.C - c0) : p.cc;
     const int h_begin = band * p.band_rows;
     const int h_end = (h_begin + p.band_rows) < p.Ho ? (h_begin + p.band_rows) : p.Ho;
-    const float* ximg = p.x + ((long)img * p.C + c0) * p.H * p.W;
-    const float* zimg = p.dy + ((long)img * p.O + o0) * p.Ho * p.Wo;
+    const long x_image = (long)p.C * p.H * p.W, z_image = (long)p.O * p.Ho * p.Wo;
+    const float* ximg0 = p.x + (long)c0 * p.H * p.W;
+    const float* zimg0 = p.dy + (long)o0 * p.Ho * p.Wo;
 
     floatx16 acc[DWG_NB];
 #pragma unroll
@@ -2999,8 +2923,10 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
 
     const int xn = (n4 + DWG8_THREADS - 1) / DWG8_THREADS;                             // pieces per thread that exist at all (uniform)
     floatx4 xr[XP], zr[8];
-    unsigned xin = 0, zin = 0;                                                         // which pieces lie inside the images
-    auto request = [&](int ho, int wo0) {
+    unsigned xin = 0, zin = 0;                            // four bits per piece: which of its columns lie inside the images
+    auto request = [&](int img, int ho, int wo0) {
+        const float* ximg = ximg0 + (long)img * x_image;
+        const float* zimg = zimg0 + (long)img * z_image;
         const int hb = ho * p.stride - p.pad, wf = wo0 * p.stride - p.pad - p.shift;
         const int corner = hb * p.W + wf;
         xin = 0; zin = 0;
@@ -3008,49 +2934,73 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
         for (int k = 0; k < XP; k++) {
             if (k < xn) {
                 const int h = hb + (xrq[k] & 0xffff), w = wf + 4 * (xrq[k] >> 16);
-                const bool in = xrq[k] >= 0 && h >= 0 && h < p.H && w >= 0 && w < p.W;
-                xr[k] = *reinterpret_cast<const floatx4*>(ximg + (in ? xoff[k] + corner : 0));
-                xin |= (in ? 1u : 0u) << k;
+                const bool row_in = xrq[k] >= 0 && h >= 0 && h < p.H;
+                if (VEC) {
+                    const bool in = row_in && w >= 0 && w < p.W;
+                    xr[k] = *reinterpret_cast<const floatx4*>(ximg + (in ? xoff[k] + corner : 0));
+                    xin |= (in ? 15u : 0u) << (4 * k);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const bool in = row_in && w + j >= 0 && w + j < p.W;
+                        xr[k][j] = ximg[in ? xoff[k] + corner + j : 0];
+                        xin |= (in ? 1u : 0u) << (4 * k + j);
+                    }
+                }
             }
         }
-        const bool zpix = wo0 + zkc < p.Wo && ho + zkr < h_end;
-        const long zpos = zpix ? (long)(ho + zkr) * p.Wo + wo0 + zkc : 0;
+        const bool zrow = ho + zkr < h_end;
+        const long zpos = (long)(zrow ? ho + zkr : 0) * p.Wo + wo0 + zkc;
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             const int o = zo + 16 * k;
-            const bool in = zpix && o0 + o < p.O;
-            zr[k] = *reinterpret_cast<const floatx4*>(zimg + (in ? (long)o * p.Ho * p.Wo + zpos : 0));
-            zin |= (in ? 1u : 0u) << k;
+            const bool o_in = zrow && o0 + o < p.O;
+            if (VEC) {
+                const bool in = o_in && wo0 + zkc < p.Wo;
+                zr[k] = *reinterpret_cast<const floatx4*>(zimg + (in ? (long)o * p.Ho * p.Wo + zpos : 0));
+                zin |= (in ? 15u : 0u) << (4 * k);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const bool in = o_in && wo0 + zkc + j < p.Wo;
+                    zr[k][j] = zimg[in ? (long)o * p.Ho * p.Wo + zpos + j : 0];
+                    zin |= (in ? 1u : 0u) << (4 * k + j);
+                }
+            }
         }
     };
     auto deposit = [&]() {
-        const half4_t zero = {(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
 #pragma unroll
         for (int k = 0; k < XP; k++) {
             if (k < xn) {
-                const half4_t hv = {(_Float16)xr[k][0], (_Float16)xr[k][1], (_Float16)xr[k][2], (_Float16)xr[k][3]};
-                if (xrq[k] >= 0) *reinterpret_cast<half4_t*>(xs + 4 * (tid + DWG8_THREADS * k)) = (xin >> k & 1) ? hv : zero;
+                half4_t hv;
+#pragma unroll
+                for (int j = 0; j < 4; j++) hv[j] = (xin >> (4 * k + (VEC ? 0 : j)) & 1) ? (_Float16)xr[k][j] : (_Float16)0.f;   // VEC: all four or none
+                if (xrq[k] >= 0) *reinterpret_cast<half4_t*>(xs + 4 * (tid + DWG8_THREADS * k)) = hv;
             }
         }
 #pragma unroll
         for (int k = 0; k < 8; k++) {
-            const half4_t hv = {(_Float16)zr[k][0], (_Float16)zr[k][1], (_Float16)zr[k][2], (_Float16)zr[k][3]};
-            *reinterpret_cast<half4_t*>(zs + (zo + 16 * k) * DWG_ZPITCH + zk) = (zin >> k & 1) ? hv : zero;
+            half4_t hv;
+#pragma unroll
+            for (int j = 0; j < 4; j++) hv[j] = (zin >> (4 * k + (VEC ? 0 : j)) & 1) ? (_Float16)zr[k][j] : (_Float16)0.f;
+            *reinterpret_cast<half4_t*>(zs + (zo + 16 * k) * DWG_ZPITCH + zk) = hv;
         }
     };
 
-    const int n_steps = (h_end - h_begin + SR - 1) / SR * segs;
-    int ho = h_begin, seg = 0;
-    if (n_steps > 0) request(ho, 0);
+    const int n_steps = n_img > 0 ? n_img * ((h_end - h_begin + SR - 1) / SR * segs) : 0;
+    int img = img0, ho = h_begin, seg = 0;
+    if (n_steps > 0) request(img, ho, 0);
     for (int step = 0; step < n_steps; step++) {
         deposit();
         __syncthreads();
         {   // the next segment (the last step asks for its own again: no branch around the requests)
-            int nseg = seg + 1, nho = ho;
+            int nseg = seg + 1, nho = ho, nimg = img;
             if (nseg == segs) { nseg = 0; nho += SR; }
-            if (step + 1 == n_steps) { nseg = seg; nho = ho; }
-            request(nho, nseg * SW);
-            seg = nseg; ho = nho;
+            if (nho >= h_end) { nho = h_begin; nimg++; }
+            if (step + 1 == n_steps) { nseg = seg; nho = ho; nimg = img; }
+            request(nimg, nho, nseg * SW);
+            seg = nseg; ho = nho; img = nimg;
         }
         if (wave_live) {
             // two fragment sets: the reads of k step ks + 1 are issued before the MFMAs of step ks
@@ -3077,19 +3027,30 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
                 for (int j = 0; j < DWG_NB; j++)
                     bf[set][j] = *reinterpret_cast<const half8_t*>(zs + (j * 32 + li) * DWG_ZPITCH + ks * 16 + lh * 8);
             };
-            fragments(0, 0);
+            if (VEC) {
+                fragments(0, 0);
 #pragma unroll
-            for (int ks = 0; ks < DWG_PX / 16; ks++) {
-                if (ks + 1 < DWG_PX / 16) fragments(ks + 1, (ks + 1) & 1);
+                for (int ks = 0; ks < DWG_PX / 16; ks++) {
+                    if (ks + 1 < DWG_PX / 16) fragments(ks + 1, (ks + 1) & 1);
 #pragma unroll
-                for (int j = 0; j < DWG_NB; j++)
-                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks & 1], bf[ks & 1][j], acc[j], 0, 0, 0);
+                    for (int j = 0; j < DWG_NB; j++)
+                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks & 1], bf[ks & 1][j], acc[j], 0, 0, 0);
+                }
+            } else {
+                // the per-column loads of this variant hold four address registers per piece: one fragment set
+#pragma unroll 2
+                for (int ks = 0; ks < DWG_PX / 16; ks++) {
+                    fragments(ks, 0);
+#pragma unroll
+                    for (int j = 0; j < DWG_NB; j++)
+                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0], bf[0][j], acc[j], 0, 0, 0);
+                }
             }
         }
         __syncthreads();
     }
     // accumulator (block j, register r): row 32 wave + (r >> 2) * 8 + lh * 4 + (r & 3), column 32 j + li
-    float* out = p.partial + ((((long)blockIdx.y * gridDim.z + blockIdx.z) * p.n_images + img) * p.bands + band) * (DWG8_ROWS * DWG_OT);
+    float* out = p.partial + ((((long)blockIdx.y * gridDim.z + blockIdx.z) * p.n_groups + group) * p.bands + band) * (DWG8_ROWS * DWG_OT);
     if (wave_live) {
 #pragma unroll
         for (int j = 0; j < DWG_NB; j++)
@@ -3141,10 +3102,9 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     const size_t taps = K_h * K_w;
     const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
     const bool vec = W % 4 == 0 && Wo % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0;
-    const int region_rows = vec ? DWG8_ROWS : DWG_ROWS;
-    int cc = (int)(region_rows / taps);
+    int cc = (int)(DWG8_ROWS / taps);
     if (cc > (int)C) cc = (int)C;
-    // vector path: the staged window starts at a multiple of four columns, `shift` columns left of the first one needed
+    // 16-byte pieces: the staged window starts at a multiple of four columns, `shift` columns left of the first one needed
     // (128 * stride is a multiple of 4, so the shift is the same for every segment)
     const int shift = vec ? (int)(((4 - (long)(pad % 4)) % 4 + 4) % 4) : 0;
     int sw_log = 7;                                                   // segment width: 16 .. 128, covering the output width
@@ -3152,53 +3112,67 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     const int SW = 1 << sw_log, SR = DWG_PX / SW;
     const int span = (int)((SR - 1) * stride + K_h);
     int pw = (int)((SW - 1) * stride + K_w) + shift;
-    pw = vec ? (pw + 3) / 4 * 4 : (pw | 1);                           // scalar path: odd, rows start on different banks
-    // staged input rows + dy segment: at most 64 KiB for the four-wave kernel (two workgroups share a CU), 96 KiB and
-    // DWG8_XMAX 16-byte pieces per thread for the eight-wave one
-    const size_t lds_limit = vec ? 96 * 1024 : 64 * 1024;
+    pw = (pw + 3) / 4 * 4;
+    // staged input rows + dy segment: at most 96 KiB, and DWG8_XMAX 16-byte pieces of input rows per thread
     auto too_big = [&](int c) {
-        if (((size_t)c * span * pw + 8) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2 > lds_limit) return true;
-        return vec && (size_t)c * span * (pw / 4) > (size_t)DWG8_THREADS * DWG8_XMAX;
+        if (((size_t)c * span * pw + 8) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2 > 96 * 1024) return true;
+        return (size_t)c * span * (pw / 4) > (size_t)DWG8_THREADS * DWG8_XMAX;
     };
     while (cc > 1 && too_big(cc)) cc--;
     if (too_big(cc)) return NZHIP_E_UNSUPPORTED;
-    if (vec && (size_t)cc * H * W + (size_t)(stride * DWG_PX + K_h) * W >= 0x7fffffffull) return NZHIP_E_UNSUPPORTED;   // int offsets in the kernel
+    if ((size_t)cc * H * W + (size_t)(stride * DWG_PX + K_h) * W >= 0x7fffffffull) return NZHIP_E_UNSUPPORTED;   // int offsets in the kernel
     const size_t lds_bytes = (((size_t)cc * span * pw + 7) & ~(size_t)7) * 2 + (size_t)DWG_OT * DWG_ZPITCH * 2;
     const int chunks = (int)((C + cc - 1) / cc), otiles = (int)((O + DWG_OT - 1) / DWG_OT);
     if (chunks > 65535 || otiles > 65535) return NZHIP_E_UNSUPPORTED;
-    // a band is a whole number of segment rows of one image
-    const long units = (long)chunks * otiles * (long)N;
+    // A workgroup takes a band of segment rows of one image, or -- small images, shared weights -- all segments of several
+    // images: whichever split minimises rounds x (segments per workgroup + the cost of its result stores).
     const long row_steps = ((long)Ho + SR - 1) / SR, segs = ((long)Wo + SW - 1) / SW;
-    const long resident = (long)device_cu_count() * (vec ? 1 : 2);
-    const int want = dwg_pick_bands(units, resident, row_steps, segs, vec ? 3.0 : 1.0);
-    const int band_rows = (int)((row_steps + want - 1) / want) * SR;
-    const int bands = (int)((Ho + band_rows - 1) / band_rows);
-    if (N * (size_t)bands > 0x7fffffffull) return NZHIP_E_UNSUPPORTED;
-    const size_t regions = (size_t)chunks * otiles * N * bands;
+    const long resident = (long)device_cu_count();
+    const long tiles = (long)chunks * otiles;
+    int bands = dwg_pick_bands(tiles * (long)N, resident, row_steps, segs, 3.0), ipw = 1;
+    if (shared && N > 1) {
+        const double steps1 = (double)((row_steps + bands - 1) / bands) * (double)segs;
+        double best = (double)((tiles * (long)N * bands + resident - 1) / resident) * (steps1 + 3.0);
+        for (long g = 2; g <= (long)N && g <= 64; g++) {
+            const long groups = ((long)N + g - 1) / g;
+            if ((groups - 1) * g >= (long)N) continue;
+            const double cost = (double)((tiles * groups + resident - 1) / resident) * ((double)g * (double)row_steps * (double)segs + 3.0);
+            if (cost < best - 1e-9) { best = cost; ipw = (int)g; bands = 1; }
+        }
+    }
+    const int band_rows = (int)((row_steps + bands - 1) / bands) * SR;
+    bands = (int)((Ho + band_rows - 1) / band_rows);
+    const int n_groups = (int)((N + ipw - 1) / ipw);
+    if ((size_t)n_groups * (size_t)bands > 0x7fffffffull) return NZHIP_E_UNSUPPORTED;
+    const size_t regions = (size_t)chunks * otiles * n_groups * bands;
     float* partial = nullptr;
-    if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), regions * region_rows * DWG_OT * sizeof(float), s)) return rc;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), regions * DWG8_ROWS * DWG_OT * sizeof(float), s)) return rc;
     ConvDwGenArgs a;
     a.x = x; a.dy = dy; a.partial = partial;
     a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.Ho = (int)Ho; a.Wo = (int)Wo;
     a.Kh = (int)K_h; a.Kw = (int)K_w; a.stride = (int)stride; a.pad = (int)pad;
     a.cc = cc; a.pw = pw; a.shift = shift; a.sw_log = sw_log; a.span = span; a.bands = bands; a.band_rows = band_rows; a.n_images = (int)N;
+    a.ipw = ipw; a.n_groups = n_groups;
     const size_t x_pieces = ((size_t)cc * span * (pw / 4) + DWG8_THREADS - 1) / DWG8_THREADS;
-    auto kfn = !vec ? conv_dwg_kernel
-               : stride == 1 ? (x_pieces <= 4 ? conv_dwg8_kernel<4, true> : conv_dwg8_kernel<DWG8_XMAX, true>)
-                             : (x_pieces <= 4 ? conv_dwg8_kernel<4, false> : conv_dwg8_kernel<DWG8_XMAX, false>);
+    auto pick = [&](auto vec_tag) {
+        constexpr bool V = decltype(vec_tag)::value;
+        return stride == 1 ? (x_pieces <= 4 ? conv_dwg8_kernel<4, true, V> : conv_dwg8_kernel<DWG8_XMAX, true, V>)
+                           : (x_pieces <= 4 ? conv_dwg8_kernel<4, false, V> : conv_dwg8_kernel<DWG8_XMAX, false, V>);
+    };
+    auto kfn = vec ? pick(std::true_type{}) : pick(std::false_type{});
     int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_bytes, "hipFuncSetAttribute(conv_dwg)");
     if (rc == NZHIP_OK) {
-        hipLaunchKernelGGL(kfn, dim3((unsigned)(N * bands), (unsigned)chunks, (unsigned)otiles), dim3(vec ? DWG8_THREADS : 256), lds_bytes, s, a);
+        hipLaunchKernelGGL(kfn, dim3((unsigned)(n_groups * bands), (unsigned)chunks, (unsigned)otiles), dim3(DWG8_THREADS), lds_bytes, s, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg kernel launch");
     }
     if (rc == NZHIP_OK) {
-        const int S = shared ? (int)(N * bands) : bands, groups = shared ? 1 : (int)N;
-        const long per_group = (long)S * region_rows * DWG_OT;
-        // partial regions of one (chunk, o_tile) are contiguous: [image][band]; a weight copy's regions start at b * S
-        dim3 grid((unsigned)((region_rows * DWG_OT + 255) / 256), (unsigned)(chunks * otiles), (unsigned)groups);
+        const int S = shared ? n_groups * bands : bands, groups = shared ? 1 : (int)N;
+        const long per_group = (long)S * DWG8_ROWS * DWG_OT;
+        // partial regions of one (chunk, o_tile) are contiguous: [image group][band]; a weight copy's regions start at b * S
+        dim3 grid((unsigned)((DWG8_ROWS * DWG_OT + 255) / 256), (unsigned)(chunks * otiles), (unsigned)groups);
         hipLaunchKernelGGL(conv_dwg_reduce_kernel, grid, dim3(256), 0, s, dw, partial, S, (int)C, (int)O, (int)taps, cc, otiles,
-                           per_group, (long)(C * taps * O), region_rows);
+                           per_group, (long)(C * taps * O), DWG8_ROWS);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg_reduce kernel launch");
     }
@@ -3225,7 +3199,11 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
     if (stride == 0 || K_h == 0 || K_w == 0) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_weights: zero stride or kernel extent");
     if (H + 2 * pad < K_h || W + 2 * pad < K_w)
         return set_error(NZHIP_E_SHAPE, "nzhip_conv2d_backward_weights: kernel larger than the padded input");
-    if (K_h != 3 || K_w != 3 || stride != 1 || pad != 1) {
+    // 3x3, stride 1, pad 1 has a kernel of its own, built around 16-byte pieces of rows that are multiples of 8 wide; narrower
+    // or odd rows (28-, 14-wide images) are better off on the gather kernel (16 x 256 x 28 x 28 -> 256: 163 us there)
+    const bool own3x3 = K_h == 3 && K_w == 3 && stride == 1 && pad == 1 &&
+                        ((W % 8 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0) || (C <= 4 && O <= 2));
+    if (!own3x3) {
         // any other geometry: the gather kernel (up to 128 taps, stride up to 4, extents that fit its index arithmetic)
         const bool fits = K_h * K_w <= (size_t)DWG_ROWS && stride <= 4 && pad < 0x10000 && H < 0x3fffffff && W < 0x3fffffff &&
                           C < 0x3fffffff && O < 0x3fffffff && N <= 65535 && H * W < 0x3fffffffull;

@@ -380,7 +380,11 @@ CONV_GEN_BWD_W = [  # N, C, H, W, O, Kh, Kw, stride, pad, w_batch: every geometr
     (1, 130, 12, 12, 8, 1, 1, 2, 0, 1), (2, 6, 40, 50, 5, 3, 3, 1, 0, 1), (1, 4, 70, 64, 130, 5, 5, 1, 2, 1),   # segment widths 64 and (two rows of) 64
     # rows that allow 16-byte loads (the eight-wave kernel): stride 2 with seven pieces of input rows per thread and two chunks,
     # per-sample weights, stride 2 over three segments per row, stride 1 with seven pieces per thread
-    (2, 40, 32, 64, 100, 3, 3, 2, 1, 1), (2, 6, 16, 16, 5, 5, 5, 1, 2, 2), (1, 8, 12, 520, 12, 3, 3, 2, 1, 1), (1, 70, 10, 128, 8, 2, 1, 1, 0, 1)]
+    (2, 40, 32, 64, 100, 3, 3, 2, 1, 1), (2, 6, 16, 16, 5, 5, 5, 1, 2, 2), (1, 8, 12, 520, 12, 3, 3, 2, 1, 1), (1, 70, 10, 128, 8, 2, 1, 1, 0, 1),
+    # many small images: a workgroup walks several images and leaves one set of partial sums for them (rows that are whole
+    # 16-byte pieces, and rows that are not); 3x3 stride 1 pad 1 on 28- and 14-wide images, which the gather kernel takes
+    # from the kernel built for rows that are multiples of 8 wide
+    (40, 256, 8, 8, 16, 3, 3, 2, 1, 1), (40, 256, 8, 8, 16, 3, 3, 1, 0, 1), (3, 40, 28, 28, 24, 3, 3, 1, 1, 1), (20, 200, 14, 14, 20, 3, 3, 1, 1, 1)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", CONV_GEN_BWD_W)
