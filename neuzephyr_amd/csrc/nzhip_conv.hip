@@ -1889,6 +1889,21 @@ static bool conv_igemm_gen_applicable(const float* x, size_t C, size_t H, size_t
            N <= 65535 && H * W < 0x7fffffffull && C * H * W < 0x7fffffffull;
 }
 
+// Whether the any-geometry kernel's tile fits LDS and a thread's staging share (the same arithmetic as the launch below).
+static bool conv_igemm_gen_fits(size_t W_out, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad) {
+    const int taps = (int)(K_h * K_w);
+    int sw_log = 8;
+    while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
+    const int SW = 1 << sw_log, SR = CG_PX / SW;
+    const int shift = (int)(((4 - (long)(pad % 4)) % 4 + 4) % 4);
+    const int span = (int)((SR - 1) * stride + K_h);
+    int pw = (int)((SW - 1) * stride + K_w) + shift;
+    pw = (pw + 3) / 4 * 4;
+    const int BN = O > 64 ? 128 : 64;                              // the larger tile: the launch may still pick the smaller one
+    const size_t slab = (size_t)BN * (taps * 32 + 16);
+    return (slab + 1023) / 1024 * 1024 + (size_t)span * pw * 32 <= 160 * 1024 - 512 && (size_t)2 * span * (pw / 4) <= (size_t)CG_THREADS * CG_TP_MAX;
+}
+
 // Returns NZHIP_E_UNSUPPORTED (nothing enqueued, no error text) when the tile does not fit LDS or a thread's staging share.
 static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C, size_t H,
                                  size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t w_batch,
@@ -2461,6 +2476,55 @@ using namespace nzhip;
 
 // bias_stride_image != 0: the bias varies per image too (used to add into an existing tensor: bias = y with
 // strides (1, H_out*W_out, O*H_out*W_out)); only the implicit-GEMM kernels take it.
+// Which kernel family a forward convolution takes (a per-image bias, which only the data gradient uses, does not change
+// the choice; the two implicit-GEMM families support it, the others do not).
+enum ConvRoute { CONV_ROUTE_DIRECT, CONV_ROUTE_FIXED, CONV_ROUTE_ANY, CONV_ROUTE_WORKSPACE };
+
+static ConvRoute conv_forward_route(const float* x, size_t N, size_t C, size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride,
+                                    size_t pad, size_t w_batch, size_t H_out, size_t W_out, bool& wide, bool& bn128) {
+    static const char* route_env = getenv("NZHIP_CONV_ROUTE");      // "workspace": column matrix + GEMM; "gen": the any-geometry
+                                                                     // kernel wherever it applies (benchmarking only)
+    // NZHIP_CONV_TW=32|64 and NZHIP_CONV_BN=64|128 override the tile choice (benchmarking only)
+    static const char* tw_env = getenv("NZHIP_CONV_TW");
+    static const char* bn_env = getenv("NZHIP_CONV_BN");
+    wide = tw_env ? atoi(tw_env) == 64 : W_out >= 64;
+    bn128 = bn_env ? atoi(bn_env) == 128 : O > 64;
+    if (conv_direct_applicable(C, O, K_h, K_w, stride, pad)) return CONV_ROUTE_DIRECT;
+    const bool force_ws = route_env && route_env[0] == 'w', force_gen = route_env && route_env[0] == 'g';
+    if (force_ws) return CONV_ROUTE_WORKSPACE;
+    const bool fixed_ok = conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL;
+    // Small images with many channels: the weights do not fit LDS, so the implicit-GEMM kernel runs one
+    // patch per workgroup with the whole C x taps contraction inside, and there are too few patches to
+    // fill the CUs (8 x 512 x 16 x 16 -> 512: 64 workgroups, 190 us). The column matrix of such a layer is
+    // small; its batched GEMM splits the contraction over the idle CUs instead (83 us).
+    bool few_patches = false, sparse_patches = false;
+    {
+        const size_t tw = wide ? 64 : 32, th = 256 / tw, bn = bn128 ? 128 : 64;
+        const size_t units = N * ((W_out + tw - 1) / tw) * ((H_out + th - 1) / th) * ((O + bn - 1) / bn);
+        const size_t w_lds = ((C + IG_CC - 1) / IG_CC) * bn * K_h * K_w * 32;       // fp16 weight image of one channel tile
+        const bool resident = (w_batch == 1 || N * ((O + bn - 1) / bn) <= (size_t)device_cu_count()) && w_lds <= 148 * 1024;
+        few_patches = !resident && units * 4 <= (size_t)device_cu_count();
+        // Weights beyond LDS and fewer than 1.75 patches per compute unit (16 x 256 x 28 x 28 -> 256: 128): the any-geometry
+        // kernel splits the channels over workgroups and is faster there (58 against 87 us; 16 x 512 x 16 x 16 -> 512: 75
+        // against 193 us), as long as its 256-pixel segments are at least half full (4 x 512 x 8 x 8: 37 against 29 us).
+        sparse_patches = !resident && units * 4 < 7 * (size_t)device_cu_count();
+    }
+    // any other kernel extent or stride, when the segments (times the channel groups the contraction can be split into)
+    // occupy at least a quarter of the CUs
+    if ((!fixed_ok || force_gen || sparse_patches) && conv_igemm_gen_applicable(x, C, H, W, O, K_h, K_w, stride, pad, N) &&
+        (w_batch == 1 || w_batch * ((O + 63) / 64) * ((C + 15) / 16) <= 65535) && conv_igemm_gen_fits(W_out, O, K_h, K_w, stride, pad)) {
+        int sw_log = 8;
+        while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
+        const size_t sw = (size_t)1 << sw_log, sr = CG_PX / sw;
+        const size_t chunks = (C + IG_CC - 1) / IG_CC;
+        const size_t seg_rows = (H_out + sr - 1) / sr, segs_w = (W_out + sw - 1) / sw;
+        const size_t groups = N * seg_rows * segs_w * ((O + 127) / 128) * (chunks >= 4 ? chunks / 2 : 1);
+        const bool half_full = H_out * W_out * 2 >= seg_rows * sr * segs_w * sw;
+        if (force_gen || (groups * 4 >= (size_t)device_cu_count() && (!fixed_ok || half_full))) return CONV_ROUTE_ANY;
+    }
+    return fixed_ok && !few_patches ? CONV_ROUTE_FIXED : CONV_ROUTE_WORKSPACE;
+}
+
 static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
                                size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
                                size_t w_batch, int64_t bias_stride_pixel, int64_t bias_stride_channel,
@@ -2475,54 +2539,14 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
     const size_t H_out = (H + 2 * pad - K_h) / stride + 1, W_out = (W + 2 * pad - K_w) / stride + 1;   // Nodes.cu:605-617
     if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    const bool igemm_ok = !conv_direct_applicable(C, O, K_h, K_w, stride, pad) &&
-                          conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL;
-    if (bias_stride_image != 0 && !igemm_ok)
-        return set_error(NZHIP_E_UNSUPPORTED, "conv2d: a per-image bias needs the implicit-GEMM route");
-    if (conv_direct_applicable(C, O, K_h, K_w, stride, pad))
+    bool wide = false, bn128 = false;
+    const ConvRoute route = conv_forward_route(x, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, H_out, W_out, wide, bn128);
+    const bool fixed_geometry = route == CONV_ROUTE_FIXED, any_geometry = route == CONV_ROUTE_ANY;
+    if (bias_stride_image != 0 && !fixed_geometry && !any_geometry)
+        return set_error(NZHIP_E_UNSUPPORTED, "conv2d: a per-image bias needs an implicit-GEMM route");
+    if (route == CONV_ROUTE_DIRECT)
         return conv_direct(y, x, w_ref, bias, N, C, H, W, O, w_batch, bias_stride_pixel, bias_stride_channel,
                            activation, s);
-    static const char* route_env = getenv("NZHIP_CONV_ROUTE");      // "workspace": column matrix + GEMM (benchmarking only)
-    const bool force_ws = route_env && route_env[0] == 'w' && bias_stride_image == 0;
-    // NZHIP_CONV_TW=32|64 and NZHIP_CONV_BN=64|128 override the tile choice (benchmarking only)
-    static const char* tw_env = getenv("NZHIP_CONV_TW");
-    static const char* bn_env = getenv("NZHIP_CONV_BN");
-    const bool wide = tw_env ? atoi(tw_env) == 64 : W_out >= 64;
-    const bool bn128 = bn_env ? atoi(bn_env) == 128 : O > 64;
-    // Small images with many channels: the weights do not fit LDS, so the implicit-GEMM kernel runs one
-    // patch per workgroup with the whole C x taps contraction inside, and there are too few patches to
-    // fill the CUs (8 x 512 x 16 x 16 -> 512: 64 workgroups, 190 us). The column matrix of such a layer is
-    // small; its batched GEMM splits the contraction over the idle CUs instead (83 us).
-    bool few_patches = false, sparse_patches = false;
-    if (bias_stride_image == 0) {
-        const size_t tw = wide ? 64 : 32, th = 256 / tw, bn = bn128 ? 128 : 64;
-        const size_t units = N * ((W_out + tw - 1) / tw) * ((H_out + th - 1) / th) * ((O + bn - 1) / bn);
-        const size_t w_lds = ((C + IG_CC - 1) / IG_CC) * bn * K_h * K_w * 32;       // fp16 weight image of one channel tile
-        const bool resident = (w_batch == 1 || N * ((O + bn - 1) / bn) <= (size_t)device_cu_count()) && w_lds <= 148 * 1024;
-        few_patches = !resident && units * 4 <= (size_t)device_cu_count();
-        // Weights beyond LDS and fewer than 1.75 patches per compute unit (16 x 256 x 28 x 28 -> 256: 128): the any-geometry
-        // kernel splits the channels over workgroups and is faster there (58 against 87 us; 16 x 512 x 16 x 16 -> 512: 75
-        // against 193 us), as long as its 256-pixel segments are at least half full (4 x 512 x 8 x 8: 37 against 29 us).
-        sparse_patches = !resident && units * 4 < 7 * (size_t)device_cu_count();
-    }
-    const bool force_gen = route_env && route_env[0] == 'g';        // "gen": the any-geometry kernel wherever it applies (benchmarking only)
-    bool fixed_geometry = !force_ws && !few_patches && conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL;
-    // any other kernel extent or stride, when the rows allow 16-byte loads and the segments (times the channel groups the
-    // contraction can be split into) occupy at least a quarter of the CUs
-    bool any_geometry = false;
-    if ((!fixed_geometry || force_gen || sparse_patches) && !force_ws && bias_stride_image == 0 &&
-        (force_gen || sparse_patches || !conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N)) &&
-        conv_igemm_gen_applicable(x, C, H, W, O, K_h, K_w, stride, pad, N) && (w_batch == 1 || w_batch * ((O + 63) / 64) * ((C + 15) / 16) <= 65535)) {
-        int sw_log = 8;
-        while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
-        const size_t sw = (size_t)1 << sw_log, sr = CG_PX / sw;
-        const size_t chunks = (C + IG_CC - 1) / IG_CC;
-        const size_t groups = N * ((H_out + sr - 1) / sr) * ((W_out + sw - 1) / sw) * ((O + 127) / 128) * (chunks >= 4 ? chunks / 2 : 1);
-        const size_t seg_rows = (H_out + sr - 1) / sr, segs_w = (W_out + sw - 1) / sw;
-        const bool half_full = H_out * W_out * 2 >= seg_rows * sr * segs_w * sw;
-        any_geometry = force_gen || (groups * 4 >= (size_t)device_cu_count() && (!sparse_patches || half_full || !conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N)));
-        if (any_geometry) fixed_geometry = false;
-    }
     if (fixed_geometry || any_geometry) {
         // The reference's bias parameter is pixel-major ([1,1,H_out*W_out,O], src/Model.cu:252-256), while the kernels'
         // lanes are adjacent pixels: read as it lies, every bias load touches 64 lines 4 O bytes apart. One pass turns it
@@ -2547,6 +2571,7 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
                                                  bias_stride_image, activation, H_out, W_out, s);
             const int rc_free = finish(rc == NZHIP_E_UNSUPPORTED ? NZHIP_OK : rc);
             if (rc != NZHIP_E_UNSUPPORTED) return rc_free;
+            if (bias_stride_image != 0) return set_error(NZHIP_E_UNSUPPORTED, "conv2d: a per-image bias needs an implicit-GEMM route");
             return conv2d_via_workspace(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
                                         bias_stride_channel, activation, H_out, W_out, s);   // the tile does not fit: column matrix
         }
@@ -2627,6 +2652,21 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
                          "nzhip_conv2d_backward_data: only square kernels, pad <= K-1 and stride <= 8 (use the column-matrix chain)");
     if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (K_h == 1 && stride == 1 && pad == 0 && H * W < 0x3fffffff && C < 0x3fffffff && O < 0x3fffffff && N <= 65535) {
+        // 1x1: no window at all, dx[n] (C x pixels) (+)= W (C x O) * dy[n] (O x pixels), one batched product
+        // (16 x 256 x 14 x 14 <- 1024 channels: 38 us against 99 us through the convolution kernels)
+        nzhip_gemm_desc g = {};
+        g.A = w_ref; g.M = (int64_t)C; g.K = (int64_t)O; g.lda = (int64_t)O; g.a_layout = NZHIP_LAYOUT_ROW;
+        g.B = dy; g.N = (int64_t)(H * W); g.ldb = (int64_t)(H * W); g.b_layout = NZHIP_LAYOUT_ROW;
+        g.C = dx; g.ldc = (int64_t)(H * W);
+        g.batch_n = (int64_t)N; g.batch_c = 1;
+        g.a_stride_n = w_batch > 1 ? (int64_t)(C * O) : 0; g.b_stride_n = (int64_t)(O * H * W); g.c_stride_n = (int64_t)(C * H * W);
+        g.activation = NZHIP_ACT_NONE;
+        if (accumulate) {
+            g.bias = dx; g.bias_stride_n = g.c_stride_n; g.bias_stride_row = g.ldc; g.bias_stride_col = 1;
+        }
+        return nzhip_gemm(&g, s);
+    }
     if (stride > 1) {
         const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
         const size_t Hu = H + 2 * pad - K_h + 1, Wu = W + 2 * pad - K_w + 1, total = N * O * Hu * Wu;
@@ -2652,8 +2692,9 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     // "+=": the implicit-GEMM kernels read dx as their bias (same lane reads, then writes each element); the other
     // routes go through a temporary and one add pass
     const size_t pad_t = K_h - 1 - pad;
-    const bool in_place = accumulate && !conv_direct_applicable(O, C, K_h, K_w, 1, pad_t) &&
-                          conv_igemm_applicable(O, C, K_h, K_w, 1, pad_t, N) && (long)H_out * W_out < 0x7fffffffL;
+    bool wide_unused = false, bn_unused = false;
+    const ConvRoute route = conv_forward_route(dy, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t, w_batch, H, W, wide_unused, bn_unused);
+    const bool in_place = accumulate && (route == CONV_ROUTE_FIXED || route == CONV_ROUTE_ANY);
     if (accumulate && !in_place) rc = workspace_alloc(reinterpret_cast<void**>(&tmp), x_elems * sizeof(float), s);
     if (rc == NZHIP_OK) {
         hipLaunchKernelGGL(conv_weight_flip_kernel, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, s, wflip, w_ref,

@@ -217,7 +217,9 @@ def test_col2im_backward_bit_exact(nz, oracle, n, c, h, w):
 CONV_BWD_DATA = [  # N, C, H, W, O, K, pad, w_batch
     (2, 3, 5, 6, 4, 3, 1, 1), (1, 2, 4, 4, 3, 3, 0, 1), (2, 2, 6, 5, 2, 3, 2, 2), (1, 3, 5, 5, 2, 1, 0, 1),
     (2, 16, 20, 36, 24, 3, 1, 1), (1, 64, 32, 64, 128, 3, 1, 1), (3, 8, 17, 33, 70, 3, 1, 3), (2, 40, 9, 70, 12, 1, 0, 1),
-    (1, 3, 40, 40, 1, 3, 1, 1), (2, 1, 12, 16, 2, 3, 1, 1)]
+    (1, 3, 40, 40, 1, 3, 1, 1), (2, 1, 12, 16, 2, 3, 1, 1),
+    (3, 20, 9, 10, 33, 1, 0, 3), (4, 256, 14, 14, 300, 1, 0, 1),            # 1x1: one batched product (per-sample weights; many channels)
+    (4, 300, 14, 14, 64, 3, 1, 1), (16, 256, 7, 7, 40, 3, 1, 1), (2, 96, 28, 28, 160, 3, 1, 1)]   # deep layers on small images: accumulation in place on the any-geometry kernel, or through a temporary
 
 
 @pytest.mark.parametrize("N,C,H,W,O,K,pad,wb", CONV_BWD_DATA)
