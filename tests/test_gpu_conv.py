@@ -83,6 +83,9 @@ CONV_CASES = [
     (1, 3, 40, 64, 1, 3, 3, 1, 1, 1),
     (2, 8, 17, 19, 5, 5, 5, 2, 2, 1),
     (1, 70, 9, 9, 130, 1, 1, 1, 0, 1),
+    (2, 130, 9, 12, 70, 1, 1, 1, 0, 1),     # 1x1 with 128 or more input channels: one batched product
+    (2, 160, 8, 8, 40, 1, 1, 1, 0, 2),      # ... with per-sample weights
+    (2, 200, 5, 5, 16, 1, 1, 1, 0, 1),      # ... tiny images and fewer outputs than inputs: the convolution kernels again
     (2, 24, 40, 70, 9, 3, 3, 1, 0, 1),      # no padding, ragged width (scalar staging path)
     (1, 9, 33, 36, 140, 3, 3, 1, 2, 1),     # padding 2: both halo columns on the left
     (2, 20, 16, 64, 64, 3, 3, 1, 1, 2),     # per-sample weights
@@ -175,6 +178,7 @@ PER_SAMPLE = [  # N, C, H, W, O, k, pad, per-pixel bias: one weight copy per ima
     (5, 48, 10, 72, 100, 3, 1, False),    # three chunks: the single-buffer resident kernel
     (2, 64, 8, 64, 128, 3, 1, True),      # per-pixel bias with a 128-channel tile: the single-buffer resident kernel
     (6, 40, 9, 40, 70, 1, 0, False),      # 1x1, 32-wide patches, two channel tiles
+    (3, 128, 9, 12, 24, 1, 0, True),      # 1x1 as a batched product, per-pixel bias as its bias matrix
     (2, 160, 8, 64, 128, 3, 1, False),    # weights beyond LDS: the per-patch slab kernel
     (300, 16, 4, 32, 16, 3, 1, False),    # more images than workgroups: the per-patch slab kernel
 ]
