@@ -2983,10 +2983,11 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
 
     const int xn = (n4 + DWG8_THREADS - 1) / DWG8_THREADS;                             // pieces per thread that exist at all (uniform)
     floatx4 xr[XP], zr[8];
-    unsigned xin = 0, zin = 0;                            // four bits per piece: which of its columns lie inside the images
-    auto request = [&](int img, int ho, int wo0) {
-        const float* ximg = ximg0 + (long)img * x_image;
-        const float* zimg = zimg0 + (long)img * z_image;
+    constexpr int MB = VEC ? 1 : 4;                       // mask bits per piece: which of its columns lie inside the images
+    unsigned xin = 0, zin = 0;
+    const float* ximg = ximg0 + (long)img0 * x_image;     // the image being requested
+    const float* zimg = zimg0 + (long)img0 * z_image;
+    auto request = [&](int ho, int wo0) {
         const int hb = ho * p.stride - p.pad, wf = wo0 * p.stride - p.pad - p.shift;
         const int corner = hb * p.W + wf;
         xin = 0; zin = 0;
@@ -2998,13 +2999,13 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
                 if (VEC) {
                     const bool in = row_in && w >= 0 && w < p.W;
                     xr[k] = *reinterpret_cast<const floatx4*>(ximg + (in ? xoff[k] + corner : 0));
-                    xin |= (in ? 15u : 0u) << (4 * k);
+                    xin |= (in ? 1u : 0u) << k;
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const bool in = row_in && w + j >= 0 && w + j < p.W;
                         xr[k][j] = ximg[in ? xoff[k] + corner + j : 0];
-                        xin |= (in ? 1u : 0u) << (4 * k + j);
+                        xin |= (in ? 1u : 0u) << (MB * k + j);
                     }
                 }
             }
@@ -3018,13 +3019,13 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
             if (VEC) {
                 const bool in = o_in && wo0 + zkc < p.Wo;
                 zr[k] = *reinterpret_cast<const floatx4*>(zimg + (in ? (long)o * p.Ho * p.Wo + zpos : 0));
-                zin |= (in ? 15u : 0u) << (4 * k);
+                zin |= (in ? 1u : 0u) << k;
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const bool in = o_in && wo0 + zkc + j < p.Wo;
                     zr[k][j] = zimg[in ? (long)o * p.Ho * p.Wo + zpos + j : 0];
-                    zin |= (in ? 1u : 0u) << (4 * k + j);
+                    zin |= (in ? 1u : 0u) << (MB * k + j);
                 }
             }
         }
@@ -3035,7 +3036,7 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
             if (k < xn) {
                 half4_t hv;
 #pragma unroll
-                for (int j = 0; j < 4; j++) hv[j] = (xin >> (4 * k + (VEC ? 0 : j)) & 1) ? (_Float16)xr[k][j] : (_Float16)0.f;   // VEC: all four or none
+                for (int j = 0; j < 4; j++) hv[j] = (xin >> (MB * k + (VEC ? 0 : j)) & 1) ? (_Float16)xr[k][j] : (_Float16)0.f;   // VEC: all four or none
                 if (xrq[k] >= 0) *reinterpret_cast<half4_t*>(xs + 4 * (tid + DWG8_THREADS * k)) = hv;
             }
         }
@@ -3043,24 +3044,26 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
         for (int k = 0; k < 8; k++) {
             half4_t hv;
 #pragma unroll
-            for (int j = 0; j < 4; j++) hv[j] = (zin >> (4 * k + (VEC ? 0 : j)) & 1) ? (_Float16)zr[k][j] : (_Float16)0.f;
+            for (int j = 0; j < 4; j++) hv[j] = (zin >> (MB * k + (VEC ? 0 : j)) & 1) ? (_Float16)zr[k][j] : (_Float16)0.f;
             *reinterpret_cast<half4_t*>(zs + (zo + 16 * k) * DWG_ZPITCH + zk) = hv;
         }
     };
 
     const int n_steps = n_img > 0 ? n_img * ((h_end - h_begin + SR - 1) / SR * segs) : 0;
-    int img = img0, ho = h_begin, seg = 0;
-    if (n_steps > 0) request(img, ho, 0);
+    int ho = h_begin, seg = 0;
+    if (n_steps > 0) request(ho, 0);
     for (int step = 0; step < n_steps; step++) {
         deposit();
         __syncthreads();
         {   // the next segment (the last step asks for its own again: no branch around the requests)
-            int nseg = seg + 1, nho = ho, nimg = img;
+            int nseg = seg + 1, nho = ho;
+            bool next_image = false;
             if (nseg == segs) { nseg = 0; nho += SR; }
-            if (nho >= h_end) { nho = h_begin; nimg++; }
-            if (step + 1 == n_steps) { nseg = seg; nho = ho; nimg = img; }
-            request(nimg, nho, nseg * SW);
-            seg = nseg; ho = nho; img = nimg;
+            if (nho >= h_end) { nho = h_begin; next_image = true; }
+            if (step + 1 == n_steps) { nseg = seg; nho = ho; next_image = false; }
+            if (next_image) { ximg += x_image; zimg += z_image; }
+            request(nho, nseg * SW);
+            seg = nseg; ho = nho;
         }
         if (wave_live) {
             // two fragment sets: the reads of k step ks + 1 are issued before the MFMAs of step ks
