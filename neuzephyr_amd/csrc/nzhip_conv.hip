@@ -1768,6 +1768,50 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
 
     load_halo(chunk_lo);
     load_slab(chunk_lo);
+    // The sums start from the bias (a channel group's bare sums from zero), so the epilogue is stores only: bias loads
+    // between the blocks of stores would each wait until the stores before them are acknowledged. A per-channel bias
+    // goes through LDS, one load per channel and workgroup (every lane asking memory for its 16 NO values sends
+    // thousands of requests per workgroup to the same few lines); a per-pixel bias is read where the results will be
+    // stored, lanes on adjacent pixels.
+    if (p.bias && !p.partial) {
+        if (p.bias_sp == 0) {
+            float* lds_b = reinterpret_cast<float*>(lds_h);      // the halo area is free until the first store_halo
+            if (tid < BN) {
+                const int o = o_tile * BN + tid;
+                lds_b[tid] = o < p.O ? p.bias[(long)b * p.bias_sn + (long)o * p.bias_sc] : 0.f;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < NO; i++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const floatx4 v = *reinterpret_cast<const floatx4*>(lds_b + (wn * NO + i) * 32 + g * 8 + lh * 4);
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[i][j][g * 4 + e] = v[e];
+                }
+            __syncthreads();                                    // read before the first halo lands in the same bytes
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int px = (wm * 2 + j) * 32 + li;
+                const int ho = ho0 + (px >> p.sw_log), wo = wo0 + (px & (SW - 1));
+                const bool px_ok = ho < p.Ho && wo < p.Wo;
+                const float* bp = p.bias + (long)b * p.bias_sn + (px_ok ? ((long)ho * p.Wo + wo) * p.bias_sp : 0);
+#pragma unroll
+                for (int i = 0; i < NO; i++) {
+                    const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
+#pragma unroll
+                    for (int rr = 0; rr < 16; rr++) {
+                        const int o = o_base + (rr >> 2) * 8 + (rr & 3);
+                        const float v = bp[(long)(o < p.O ? o : 0) * p.bias_sc];
+                        acc[i][j][rr] = (px_ok && o < p.O) ? v : 0.f;
+                    }
+                }
+            }
+        }
+    }
     for (int chunk = chunk_lo; chunk < chunk_hi; chunk++) {
         store_halo(chunk);                                      // registers (chunk) -> LDS, fp16 channel-last
         __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): this wave's slab pieces landed
@@ -1815,7 +1859,7 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
     }
     __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);                // the halo requested once more after the last chunk
 
-    // ---- epilogue: bias + activation + NCHW store (lanes = adjacent pixels), or the bare sums of this channel group ----
+    // ---- epilogue: activation + NCHW store (lanes = adjacent pixels), or the bare sums of this channel group ----
     const long hw_out = (long)p.Ho * p.Wo;
     if (p.partial) {
         float* pb = p.partial + ((long)group * (gridDim.z / p.chunk_groups) + b) * p.O * hw_out;
@@ -1847,16 +1891,10 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
 #pragma unroll
         for (int i = 0; i < NO; i++) {
             const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
-            float bv[16];
 #pragma unroll
             for (int rr = 0; rr < 16; rr++) {
                 const int o = o_base + (rr >> 2) * 8 + (rr & 3);
-                bv[rr] = (p.bias && o < p.O) ? p.bias[(long)b * p.bias_sn + pix * p.bias_sp + (long)o * p.bias_sc] : 0.f;
-            }
-#pragma unroll
-            for (int rr = 0; rr < 16; rr++) {
-                const int o = o_base + (rr >> 2) * 8 + (rr & 3);
-                float v = acc[i][j][rr] + bv[rr];
+                float v = acc[i][j][rr];
                 if (p.relu) v = v > 0.f ? v : 0.f;
                 if (o < p.O) yb[(long)o * hw_out + pix] = v;
             }
