@@ -639,6 +639,49 @@ __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(con
 
     load_halo(0);
     load_slab(0);
+    // The sums start from the bias, so the epilogue is stores only (a load issued after stores is not counted as
+    // returned before those stores are acknowledged: bias loads between the blocks of stores made every block wait for
+    // the one before). Per channel: one load per channel and workgroup, handed out through LDS; per pixel: read where
+    // the results will go, lanes on adjacent pixels.
+    if (p.bias) {
+        const bool o_full = o_tile * BN + BN <= p.O;
+        if (p.bias_sp == 0) {
+            float* lds_b = reinterpret_cast<float*>(lds_h);      // the halo area is free until the first store_halo
+            if (tid < BN) {
+                const int o = o_tile * BN + tid;
+                lds_b[tid] = o < p.O ? p.bias[(long)b * p.bias_sn + (long)o * p.bias_sc] : 0.f;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const floatx4 v = *reinterpret_cast<const floatx4*>(lds_b + wn * 64 + i * 32 + g * 8 + lh * 4);
+#pragma unroll
+                    for (int j = 0; j < FP; j++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[i][j][g * 4 + e] = v[e];
+                }
+            __syncthreads();                                    // read before the first halo lands in the same bytes
+        } else {
+#pragma unroll
+            for (int j = 0; j < FP; j++) {
+                const int blk = wm * FP + j;
+                const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
+                const bool px_ok = ho < p.H_out && wo < p.W_out;
+                const float* bp = p.bias + (long)b * p.bias_sn + (px_ok ? ((long)ho * p.W_out + wo) * p.bias_sp : 0);
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int o = o_tile * BN + wn * 64 + lh * 4 + i * 32 + (r >> 2) * 8 + (r & 3);
+                        const bool ok = px_ok && (o_full || o < p.O);
+                        const float v = bp[(long)(ok ? o : 0) * p.bias_sc];
+                        acc[i][j][r] = ok ? v : 0.f;
+                    }
+            }
+        }
+    }
     for (int chunk = 0; chunk < p.n_chunks; chunk++) {
         store_halo();                                           // registers (chunk) -> LDS, fp16 channel-last
         __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): this wave's slab pieces landed
@@ -671,9 +714,7 @@ __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(con
         if (chunk + 1 < p.n_chunks) load_slab(chunk + 1);
     }
 
-    // ---- epilogue: bias + activation + NCHW store (lanes = adjacent pixels) -------------------
-    // The bias values of one pixel row are requested together, so the wave waits for memory
-    // once per row instead of once per element.
+    // ---- epilogue: activation + NCHW store (lanes = adjacent pixels) --------------------------
     float* yb = p.y + (long)b * p.O * p.H_out * p.W_out;
     const long hw_out = (long)p.H_out * p.W_out;
     const int o_base = o_tile * BN + wn * 64 + lh * 4;
@@ -684,21 +725,13 @@ __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(con
         const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
         if (ho >= p.H_out || wo >= p.W_out) continue;
         const long pix = (long)ho * p.W_out + wo;
-        float bv[2][16];
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int o = o_base + i * 32 + (r >> 2) * 8 + (r & 3);
-                bv[i][r] = (p.bias && (o_full || o < p.O)) ? p.bias[(long)b * p.bias_sn + pix * p.bias_sp + (long)o * p.bias_sc] : 0.f;
-            }
         float* dst = yb + pix;
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int o = o_base + i * 32 + (r >> 2) * 8 + (r & 3);
-                float v = acc[i][j][r] + bv[i][r];
+                float v = acc[i][j][r];
                 if (p.relu) v = v > 0.f ? v : 0.f;
                 if (o_full || o < p.O) dst[(long)o * hw_out] = v;
             }
@@ -987,7 +1020,23 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     // is a wave-uniform channel plane (scalar registers, stepped with scalar adds) plus one per-lane
     // byte offset shared by the 16 stores: pixel, and 4 planes up for the upper half-wave.
     // A patch that lies wholly inside the output takes the unpredicated path.
-    auto flush_unit = [&](const int j, const int i, const int patch) {
+    // The per-pixel bias of unit (j, i), requested one unit ahead of its use (the first unit's at the start of the
+    // patch): a request issued after a unit's stores would not be counted as returned before those stores are.
+    auto bias_request = [&](float (&bv)[16], const int j, const int i, const int patch) {
+        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
+        const int blk = wm * FP + j;
+        const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
+        const long pix = (ho < p.H_out && wo < p.W_out) ? (long)ho * p.W_out + wo : 0;
+        const int o_lane = o_wave + i * 32 + lh * 4;
+        const float* bp = p.bias + (long)b * p.bias_sn + pix * p.bias_sp;
+#pragma unroll
+        for (int rr = 0; rr < 16; rr++) {
+            const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
+            bv[rr] = bp[(long)((o_full || o < p.O) ? o : 0) * p.bias_sc];
+        }
+    };
+    auto flush_unit = [&](const int j, const int i, const int patch, const float (&bv)[16]) {
         const int b = patch / patches_per_image, r = patch % patches_per_image;
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
         const int blk = wm * FP + j;
@@ -998,14 +1047,6 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
         const unsigned lane_bytes = (unsigned)((pix + (long)lh * 4 * hw_out) * 4);
         char* pl = reinterpret_cast<char*>(p.y + ((long)b * p.O + o_wave + i * 32) * hw_out);
         const int o_lane = o_wave + i * 32 + lh * 4;
-        float bv[16];
-        if (PIX_BIAS) {                                          // one batch of requests per unit
-#pragma unroll
-            for (int rr = 0; rr < 16; rr++) {
-                const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
-                bv[rr] = p.bias[(long)b * p.bias_sn + pix * p.bias_sp + (long)((o_full || o < p.O) ? o : 0) * p.bias_sc];
-            }
-        }
         auto finished = [&](const int rr) {
             float v = acc[i][j][rr];
             if (PIX_BIAS) v += bv[rr];                           // a per-channel bias is already in the accumulator
@@ -1058,17 +1099,24 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     if (tid < BN) lds_bias[tid] = my_bias;
     __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);                 // vmcnt(0): resident weights landed
     lds_barrier();
+    float bvs[2][16];
     for (int pi = 0; pi < my_patches; pi++) {
         init_acc();
+        const int patch = first_patch + pi * patch_stride;
+        if (PIX_BIAS) bias_request(bvs[0], 0, 0, patch);         // lands under the patch's MFMAs
         for (int c = 0; c < n_items; c += 2) {
             item(raw[0], nv[0], c);
             item(raw[1], nv[1], c + 1);
         }
-        const int patch = first_patch + pi * patch_stride;
 #pragma unroll
         for (int j = 0; j < FP; j++)
 #pragma unroll
-            for (int i = 0; i < NI; i++) flush_unit(j, i, patch);
+            for (int i = 0; i < NI; i++) {
+                constexpr int UNITS = FP * NI;
+                const int u = j * NI + i;
+                if (PIX_BIAS && u + 1 < UNITS) bias_request(bvs[(u + 1) & 1], (u + 1) / NI, (u + 1) % NI, patch);
+                flush_unit(j, i, patch, bvs[u & 1]);
+            }
     }
 }
 
@@ -1318,7 +1366,23 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
     const int o_wave = o_tile * BN + wn * WCH;
     const bool o_full = o_tile * BN + BN <= p.O;
     const long hw_out = (long)p.H_out * p.W_out;
-    auto flush_unit = [&](const int j, const int i, const int patch) {
+    // The per-pixel bias of unit (j, i), requested one unit ahead of its use (the first unit's at the start of the
+    // patch): a request issued after a unit's stores would not be counted as returned before those stores are.
+    auto bias_request = [&](float (&bv)[16], const int j, const int i, const int patch) {
+        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
+        const int blk = wm * FP + j;
+        const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
+        const long pix = (ho < p.H_out && wo < p.W_out) ? (long)ho * p.W_out + wo : 0;
+        const int o_lane = o_wave + i * 32 + lh * 4;
+        const float* bp = p.bias + (long)b * p.bias_sn + pix * p.bias_sp;
+#pragma unroll
+        for (int rr = 0; rr < 16; rr++) {
+            const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
+            bv[rr] = bp[(long)((o_full || o < p.O) ? o : 0) * p.bias_sc];
+        }
+    };
+    auto flush_unit = [&](const int j, const int i, const int patch, const float (&bv)[16]) {
         const int b = patch / patches_per_image, r = patch % patches_per_image;
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
         const int blk = wm * FP + j;
@@ -1329,14 +1393,6 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
         const unsigned lane_bytes = (unsigned)((pix + (long)lh * 4 * hw_out) * 4);
         char* pl = reinterpret_cast<char*>(p.y + ((long)b * p.O + o_wave + i * 32) * hw_out);
         const int o_lane = o_wave + i * 32 + lh * 4;
-        float bv[16];
-        if (PIX_BIAS) {
-#pragma unroll
-            for (int rr = 0; rr < 16; rr++) {
-                const int o = o_lane + (rr >> 2) * 8 + (rr & 3);
-                bv[rr] = p.bias[(long)b * p.bias_sn + pix * p.bias_sp + (long)((o_full || o < p.O) ? o : 0) * p.bias_sc];
-            }
-        }
         auto finished = [&](const int rr) {
             float v = acc[i][j][rr];
             if (PIX_BIAS) v += bv[rr];
@@ -1400,18 +1456,25 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
     store_halo(raw[0], nv[0], lds_h0);
     load_item(raw[0], nv[0]);                                    // item 2
     lds_barrier();
+    float bvs[2][16];
     for (int pi = 0; pi < my_patches; pi++) {
         init_acc();
+        const int patch = first_patch + pi * patch_stride;
+        if (PIX_BIAS) bias_request(bvs[0], 0, 0, patch);         // lands under the patch's MFMAs
 #pragma unroll 1
         for (int c = 0; c < NCH; c += 2) {
             item(raw[1], nv[1], c, lds_h0, lds_h1, w8[0], w8[1]);
             item(raw[0], nv[0], c + 1, lds_h1, lds_h0, w8[1], w8[0]);
         }
-        const int patch = first_patch + pi * patch_stride;
 #pragma unroll
         for (int j = 0; j < FP; j++)
 #pragma unroll
-            for (int i = 0; i < NI; i++) flush_unit(j, i, patch);
+            for (int i = 0; i < NI; i++) {
+                constexpr int UNITS = FP * NI;
+                const int u = j * NI + i;
+                if (PIX_BIAS && u + 1 < UNITS) bias_request(bvs[(u + 1) & 1], (u + 1) / NI, (u + 1) % NI, patch);
+                flush_unit(j, i, patch, bvs[u & 1]);
+            }
     }
     // the requests issued for items past the end are still in flight
     __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);
@@ -1660,7 +1723,8 @@ __global__ __launch_bounds__(256) void conv_weight_image_gen_kernel(_Float16* __
 // NO: 32-channel blocks per wave (BN / 64); every wave also owns two 32-pixel blocks. TP: staging tasks per thread.
 // VEC: image rows are whole 16-byte pieces (W a multiple of 4, aligned x): a task's four columns are one load per
 // channel and lie inside or outside the image together; otherwise (14 x 14 images ...) four loads with their own bounds.
-template <int NO, int TP, bool VEC>
+// PIXB: the bias varies per pixel (the reference's Bias node after the matmul; the per-image bias of an in-place data gradient).
+template <int NO, int TP, bool VEC, bool PIXB>
 __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGenArgs p) {
     constexpr int BN = NO * 64;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -1768,55 +1832,50 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
 
     load_halo(chunk_lo);
     load_slab(chunk_lo);
-    // The sums start from the bias (a channel group's bare sums from zero), so the epilogue is stores only: bias loads
-    // between the blocks of stores would each wait until the stores before them are acknowledged. A per-channel bias
-    // goes through LDS, one load per channel and workgroup (every lane asking memory for its 16 NO values sends
-    // thousands of requests per workgroup to the same few lines); a per-pixel bias is read where the results will be
-    // stored, lanes on adjacent pixels.
-    if (p.bias && !p.partial) {
-        if (p.bias_sp == 0) {
-            float* lds_b = reinterpret_cast<float*>(lds_h);      // the halo area is free until the first store_halo
-            if (tid < BN) {
-                const int o = o_tile * BN + tid;
-                lds_b[tid] = o < p.O ? p.bias[(long)b * p.bias_sn + (long)o * p.bias_sc] : 0.f;
-            }
-            __syncthreads();
-#pragma unroll
-            for (int i = 0; i < NO; i++)
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const floatx4 v = *reinterpret_cast<const floatx4*>(lds_b + (wn * NO + i) * 32 + g * 8 + lh * 4);
-#pragma unroll
-                    for (int j = 0; j < 2; j++)
-#pragma unroll
-                        for (int e = 0; e < 4; e++) acc[i][j][g * 4 + e] = v[e];
-                }
-            __syncthreads();                                    // read before the first halo lands in the same bytes
-        } else {
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const int px = (wm * 2 + j) * 32 + li;
-                const int ho = ho0 + (px >> p.sw_log), wo = wo0 + (px & (SW - 1));
-                const bool px_ok = ho < p.Ho && wo < p.Wo;
-                const float* bp = p.bias + (long)b * p.bias_sn + (px_ok ? ((long)ho * p.Wo + wo) * p.bias_sp : 0);
-#pragma unroll
-                for (int i = 0; i < NO; i++) {
-                    const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
-#pragma unroll
-                    for (int rr = 0; rr < 16; rr++) {
-                        const int o = o_base + (rr >> 2) * 8 + (rr & 3);
-                        const float v = bp[(long)(o < p.O ? o : 0) * p.bias_sc];
-                        acc[i][j][rr] = (px_ok && o < p.O) ? v : 0.f;
-                    }
-                }
-            }
+    // Bias. Loads between the epilogue's blocks of stores would each wait until the stores before them are
+    // acknowledged (a load issued after stores is not counted as returned before they are), and every lane asking
+    // memory for its own per-channel values sends thousands of requests per workgroup to the same few lines. So a
+    // per-channel bias is the starting value of the sums -- one load per channel and workgroup, handed out through
+    // LDS -- and a per-pixel bias is requested one unit (32 pixels x 32 channels) ahead of the stores that need it,
+    // the first unit's before the last chunk's taps when the registers allow (one staging task per thread).
+    const bool pix_bias = PIXB && p.bias && !p.partial;
+    if (!PIXB && p.bias && !p.partial) {
+        float* lds_b = reinterpret_cast<float*>(lds_h);          // the halo area is free until the first store_halo
+        if (tid < BN) {
+            const int o = o_tile * BN + tid;
+            lds_b[tid] = o < p.O ? p.bias[(long)b * p.bias_sn + (long)o * p.bias_sc] : 0.f;
         }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NO; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const floatx4 v = *reinterpret_cast<const floatx4*>(lds_b + (wn * NO + i) * 32 + g * 8 + lh * 4);
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[i][j][g * 4 + e] = v[e];
+            }
+        __syncthreads();                                        // read before the first halo lands in the same bytes
     }
+    float bvs[2][16];
+    auto bias_request = [&](float (&bv)[16], const int j, const int i) {
+        const int px = (wm * 2 + j) * 32 + li;
+        const int ho = ho0 + (px >> p.sw_log), wo = wo0 + (px & (SW - 1));
+        const float* bp = p.bias + (long)b * p.bias_sn + ((ho < p.Ho && wo < p.Wo) ? ((long)ho * p.Wo + wo) * p.bias_sp : 0);
+        const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
+#pragma unroll
+        for (int rr = 0; rr < 16; rr++) {
+            const int o = o_base + (rr >> 2) * 8 + (rr & 3);
+            bv[rr] = bp[(long)(o < p.O ? o : 0) * p.bias_sc];
+        }
+    };
     for (int chunk = chunk_lo; chunk < chunk_hi; chunk++) {
         store_halo(chunk);                                      // registers (chunk) -> LDS, fp16 channel-last
         __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): this wave's slab pieces landed
         __syncthreads();
         load_halo(chunk + 1 < chunk_hi ? chunk + 1 : chunk);    // lands while the MFMAs below run (the last: once more, unused)
+        if (PIXB && TP == 1 && pix_bias && chunk + 1 == chunk_hi) bias_request(bvs[0], 0, 0);   // (more tasks per thread leave no registers for it)
         // two fragment sets: the reads of tap t + 1 are issued before the MFMAs of tap t
         half8_t wf_[2][NO], pf_[2][2];
         auto fragments = [&](const int tap, const int r, const int sx, const int set) {
@@ -1882,21 +1941,25 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
         return;
     }
     float* yb = p.y + (long)b * p.O * p.Ho * p.Wo;
+    if (PIXB && TP != 1 && pix_bias) bias_request(bvs[0], 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int px = (wm * 2 + j) * 32 + li;
         const int ho = ho0 + (px >> p.sw_log), wo = wo0 + (px & (SW - 1));
-        if (ho >= p.Ho || wo >= p.Wo) continue;
-        const long pix = (long)ho * p.Wo + wo;
+        const bool px_ok = ho < p.Ho && wo < p.Wo;
+        const long pix = px_ok ? (long)ho * p.Wo + wo : 0;
 #pragma unroll
         for (int i = 0; i < NO; i++) {
+            const int u = j * NO + i;
+            if (PIXB && pix_bias && u + 1 < 2 * NO) bias_request(bvs[(u + 1) & 1], (u + 1) / NO, (u + 1) % NO);
             const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
 #pragma unroll
             for (int rr = 0; rr < 16; rr++) {
                 const int o = o_base + (rr >> 2) * 8 + (rr & 3);
                 float v = acc[i][j][rr];
+                if (PIXB && pix_bias) v += bvs[u & 1][rr];
                 if (p.relu) v = v > 0.f ? v : 0.f;
-                if (o < p.O) yb[(long)o * hw_out + pix] = v;
+                if (px_ok && o < p.O) yb[(long)o * hw_out + pix] = v;
             }
         }
     }
@@ -2012,12 +2075,14 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     }
     const int tp = (int)((tasks + CG_THREADS - 1) / CG_THREADS);
     const bool vec = W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
-    auto pick = [&](auto vec_tag) {
-        constexpr bool V = decltype(vec_tag)::value;
-        return BN == 128 ? (tp <= 1 ? conv_igemm_gen_kernel<2, 1, V> : tp == 2 ? conv_igemm_gen_kernel<2, 2, V> : conv_igemm_gen_kernel<2, 3, V>)
-                         : (tp <= 1 ? conv_igemm_gen_kernel<1, 1, V> : tp == 2 ? conv_igemm_gen_kernel<1, 2, V> : conv_igemm_gen_kernel<1, 3, V>);
+    auto pick = [&](auto vec_tag, auto pix_tag) {
+        constexpr bool V = decltype(vec_tag)::value, P = decltype(pix_tag)::value;
+        return BN == 128 ? (tp <= 1 ? conv_igemm_gen_kernel<2, 1, V, P> : tp == 2 ? conv_igemm_gen_kernel<2, 2, V, P> : conv_igemm_gen_kernel<2, 3, V, P>)
+                         : (tp <= 1 ? conv_igemm_gen_kernel<1, 1, V, P> : tp == 2 ? conv_igemm_gen_kernel<1, 2, V, P> : conv_igemm_gen_kernel<1, 3, V, P>);
     };
-    auto kfn = vec ? pick(std::true_type{}) : pick(std::false_type{});
+    const bool pixb = bias && bias_sp != 0 && chunk_groups == 1;
+    auto kfn = vec ? (pixb ? pick(std::true_type{}, std::true_type{}) : pick(std::true_type{}, std::false_type{}))
+                   : (pixb ? pick(std::false_type{}, std::true_type{}) : pick(std::false_type{}, std::false_type{}));
     int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_need, "hipFuncSetAttribute(conv_igemm_gen)");
     if (rc == NZHIP_OK) {
         hipLaunchKernelGGL(kfn, dim3((unsigned)(seg_rows * segs_w), (unsigned)n_otiles, (unsigned)(N * chunk_groups)), dim3(CG_THREADS),
