@@ -341,27 +341,50 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16mfma_kernel(const GemmKer
     const bool bias_rowless = bias && p.bias_sm == 0;
 #pragma unroll
     for (int j = 0; j < FN; j++) bcol[j] = (bias_rowless && gn + j < p.N) ? bias[(long)(gn + j) * p.bias_sk] : 0.f;
+    // A bias that varies along rows (a bias matrix, C itself when a gradient is accumulated in place) is requested half
+    // a block (8 rows) ahead of the stores that need it: a load issued after stores is not counted as returned before
+    // those stores are acknowledged, so requesting a block after storing the one before made every block wait for
+    // its predecessor. 16- or 8-byte loads when the bias rows are contiguous and aligned like the rows of C.
+    const bool bias_rows = bias && !bias_rowless;
+    const bool bias_vec = bias_rows && (FN == 2 || FN == 4) && p.bias_sk == 1 && (p.bias_sm & (FN - 1)) == 0 &&
+                          (reinterpret_cast<uintptr_t>(bias) & (FN * 4 - 1)) == 0 && gn + FN <= p.N;
+    float bvs[2][8][FN];
+    auto bias_request = [&](float (&bv)[8][FN], const int i, const int h) {
+#pragma unroll
+        for (int r8 = 0; r8 < 8; r8++) {
+            const int r = h * 8 + r8;
+            const int gm = m0 + wm * TM + ((r >> 2) * 8 + lh * 4 + (r & 3)) * FM + i;
+            const float* bp = bias + (long)(gm < p.M ? gm : 0) * p.bias_sm;
+            if (bias_vec) {
+                if constexpr (FN == 4) {
+                    const floatx4 v = *reinterpret_cast<const floatx4*>(bp + gn);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) bv[r8][e] = v[e];
+                } else if constexpr (FN == 2) {
+                    const floatx2 v = *reinterpret_cast<const floatx2*>(bp + gn);
+                    bv[r8][0] = v[0];
+                    bv[r8][1] = v[1];
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < FN; j++) bv[r8][j] = bp[gn + j < p.N ? (long)(gn + j) * p.bias_sk : 0];
+            }
+        }
+    };
+    if (bias_rows) bias_request(bvs[0], 0, 0);
 #pragma unroll
     for (int i = 0; i < FM; i++) {
-        float bv[16][FN];
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const int gm = m0 + wm * TM + ((r >> 2) * 8 + lh * 4 + (r & 3)) * FM + i;
-#pragma unroll
-            for (int j = 0; j < FN; j++)
-                bv[r][j] = (bias && !bias_rowless && gm < p.M && gn + j < p.N)
-                               ? bias[(long)gm * p.bias_sm + (long)(gn + j) * p.bias_sk]
-                               : bcol[j];
-        }
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
+            if (bias_rows && (r & 7) == 0 && i * 2 + (r >> 3) + 1 < 2 * FM)
+                bias_request(bvs[(i * 2 + (r >> 3) + 1) & 1], (i * 2 + (r >> 3) + 1) >> 1, (i * 2 + (r >> 3) + 1) & 1);
             const int im = (r >> 2) * 8 + lh * 4 + (r & 3);
             const int gm = m0 + wm * TM + im * FM + i;
             if (!FULL && gm >= p.M) continue;
             float v[FN];
 #pragma unroll
             for (int j = 0; j < FN; j++) {
-                float x = acc[i][j][r] + bv[r][j];
+                float x = acc[i][j][r] + (bias_rows ? bvs[(i * 2 + (r >> 3)) & 1][r & 7][j] : bcol[j]);
                 if (p.relu) x = x > 0.f ? x : 0.f;
                 v[j] = x;
             }
