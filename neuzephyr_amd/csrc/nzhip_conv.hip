@@ -1734,11 +1734,14 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, lh = lane >> 5;
     const int wm = wave & 3, wn = wave >> 2;                    // pixel blocks 2 wm, 2 wm + 1; channel blocks NO wn ..
-    const int b = blockIdx.z / p.chunk_groups, group = blockIdx.z % p.chunk_groups, o_tile = blockIdx.y;
+    // neighbouring segments share input rows: the compute units of one XCD take a contiguous run of them
+    int seg_x, o_tile, bz;
+    xcd_contiguous_block(seg_x, o_tile, bz);
+    const int b = bz / p.chunk_groups, group = bz % p.chunk_groups;
     const int chunk_lo = group * p.chunks_per_group;
     const int chunk_hi = chunk_lo + p.chunks_per_group < p.n_chunks ? chunk_lo + p.chunks_per_group : p.n_chunks;
     const int SW = 1 << p.sw_log, SR = CG_PX >> p.sw_log;
-    const int ho0 = (blockIdx.x / p.segs_w) * SR, wo0 = (blockIdx.x % p.segs_w) * SW;
+    const int ho0 = (seg_x / p.segs_w) * SR, wo0 = (seg_x % p.segs_w) * SW;
     const int hb = ho0 * p.stride - p.pad, wf = wo0 * p.stride - p.pad - p.shift;   // image position of staged (0, 0)
     const int taps = p.Kh * p.Kw;
     const long plane = (long)p.H * p.W;
@@ -1986,7 +1989,7 @@ static bool conv_igemm_gen_applicable(const float* x, size_t C, size_t H, size_t
     (void)O;
     // (a strided 1x1 convolution has one tap per chunk to multiply between two barriers: its column matrix is the cheaper way)
     (void)x; (void)W;
-    return C >= 8 && stride <= 4 && K_h * K_w >= 2 && K_h * K_w <= 64 && pad < 0x10000 &&
+    return C >= 1 && stride <= 4 && K_h * K_w >= 2 && K_h * K_w <= 64 && pad < 0x10000 &&
            N <= 65535 && H * W < 0x7fffffffull && C * H * W < 0x7fffffffull;
 }
 
