@@ -1993,19 +1993,30 @@ static bool conv_igemm_gen_applicable(const float* x, size_t C, size_t H, size_t
            N <= 65535 && H * W < 0x7fffffffull && C * H * W < 0x7fffffffull;
 }
 
-// Whether the any-geometry kernel's tile fits LDS and a thread's staging share (the same arithmetic as the launch below).
-static bool conv_igemm_gen_fits(size_t W_out, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad) {
+// The segment width of the any-geometry kernel: the power of two >= 16 that covers the output width, or, when the slab
+// and the halo of that tile do not fit LDS or a thread's staging share, the widest narrower one that does (more rows of
+// fewer columns: 7x7 stride 2 on 112 output columns takes 4 x 64 instead of 2 x 128 pixels). Returns log2 of the
+// width, 0 when nothing fits. Sized for the larger channel tile; the launch may still pick the smaller one.
+static int conv_igemm_gen_sw_log(size_t W_out, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad) {
     const int taps = (int)(K_h * K_w);
     int sw_log = 8;
     while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
-    const int SW = 1 << sw_log, SR = CG_PX / SW;
     const int shift = (int)(((4 - (long)(pad % 4)) % 4 + 4) % 4);
-    const int span = (int)((SR - 1) * stride + K_h);
-    int pw = (int)((SW - 1) * stride + K_w) + shift;
-    pw = (pw + 3) / 4 * 4;
-    const int BN = O > 64 ? 128 : 64;                              // the larger tile: the launch may still pick the smaller one
+    const int BN = O > 64 ? 128 : 64;
     const size_t slab = (size_t)BN * (taps * 32 + 16);
-    return (slab + 1023) / 1024 * 1024 + (size_t)span * pw * 32 <= 160 * 1024 - 512 && (size_t)2 * span * (pw / 4) <= (size_t)CG_THREADS * CG_TP_MAX;
+    for (; sw_log >= 4; sw_log--) {
+        const int SW = 1 << sw_log, SR = CG_PX / SW;
+        const int span = (int)((SR - 1) * stride + K_h);
+        int pw = (int)((SW - 1) * stride + K_w) + shift;
+        pw = (pw + 3) / 4 * 4;
+        if ((slab + 1023) / 1024 * 1024 + (size_t)span * pw * 32 <= 160 * 1024 - 512 &&
+            (size_t)2 * span * (pw / 4) <= (size_t)CG_THREADS * CG_TP_MAX)
+            return sw_log;
+    }
+    return 0;
+}
+static bool conv_igemm_gen_fits(size_t W_out, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad) {
+    return conv_igemm_gen_sw_log(W_out, O, K_h, K_w, stride, pad) != 0;
 }
 
 // Returns NZHIP_E_UNSUPPORTED (nothing enqueued, no error text) when the tile does not fit LDS or a thread's staging share.
@@ -2014,8 +2025,8 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
                                  int64_t bias_sp, int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out,
                                  hipStream_t s) {
     const int taps = (int)(K_h * K_w);
-    int sw_log = 8;
-    while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
+    const int sw_log = conv_igemm_gen_sw_log(W_out, O, K_h, K_w, stride, pad);
+    if (sw_log == 0) return NZHIP_E_UNSUPPORTED;
     const int SW = 1 << sw_log, SR = CG_PX / SW;
     // 128 output channels per workgroup, unless that leaves compute units without one (16 x 128 x 56 x 56 -> 128 at
     // stride 2: 64 workgroups; with 64-channel tiles 128 of them, 40 against 49 us)
@@ -2619,8 +2630,7 @@ static ConvRoute conv_forward_route(const float* x, size_t N, size_t C, size_t H
     // occupy at least a quarter of the CUs
     if ((!fixed_ok || force_gen || sparse_patches) && conv_igemm_gen_applicable(x, C, H, W, O, K_h, K_w, stride, pad, N) &&
         (w_batch == 1 || w_batch * ((O + 63) / 64) * ((C + 15) / 16) <= 65535) && conv_igemm_gen_fits(W_out, O, K_h, K_w, stride, pad)) {
-        int sw_log = 8;
-        while (sw_log > 4 && (size_t)(1 << (sw_log - 1)) >= W_out) sw_log--;
+        const int sw_log = conv_igemm_gen_sw_log(W_out, O, K_h, K_w, stride, pad);     // (not 0: it fits)
         const size_t sw = (size_t)1 << sw_log, sr = CG_PX / sw;
         const size_t chunks = (C + IG_CC - 1) / IG_CC;
         const size_t seg_rows = (H_out + sr - 1) / sr, segs_w = (W_out + sw - 1) / sw;

@@ -152,6 +152,7 @@ CONV_ANY_GEOMETRY = [  # N, C, H, W, O, k_h, k_w, stride, pad, w_batch, per-pixe
     (8, 3, 64, 64, 64, 3, 3, 1, 1, 1, True),        # RGB, 3x3 stride 1, the reference's per-pixel bias
     (32, 1, 28, 28, 6, 5, 5, 1, 0, 1, False),       # one channel, 5x5 without padding, six output channels
     (8, 3, 96, 96, 20, 7, 7, 2, 3, 1, False),       # 7x7 stride 2: the slab of 49 taps beside a 13-row halo
+    (6, 3, 50, 224, 64, 7, 7, 2, 3, 1, False),      # ... on 112 output columns: 128-wide segments do not fit, 4 x 64 pixels do
     (16, 5, 30, 30, 9, 3, 3, 1, 1, 16, False),      # rows that are not whole 16-byte pieces, per-sample weights
     # the per-pixel bias on the 128-channel tile and with two and three staging tasks per thread
     (64, 8, 32, 32, 65, 5, 5, 1, 2, 1, True),
