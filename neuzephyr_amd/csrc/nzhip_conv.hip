@@ -2589,6 +2589,54 @@ __global__ __launch_bounds__(256) void accumulate_kernel(float* __restrict__ dst
 
 }  // namespace nzhip
 
+namespace nzhip {
+// A 1x1 convolution with a stride and no padding only ever looks at every stride-th pixel of every stride-th row:
+// dst[plane][ho][wo] = src[plane][ho * stride][wo * stride]. On that smaller image it is the 1x1 stride-1 convolution,
+// forward and both gradients (the reference lowers it like any other: column matrix, product, and for the data
+// gradient a scatter over the windows, src/Nodes.cu:605-640).
+__global__ __launch_bounds__(256) void subsample_kernel(float* __restrict__ dst, const float* __restrict__ src, long total, int H, int W,
+                                                        int Ho, int Wo, int stride) {
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int wo = (int)(t % Wo), ho = (int)((t / Wo) % Ho);
+    const long plane = t / ((long)Wo * Ho);
+    dst[t] = src[(plane * H + (long)ho * stride) * W + (long)wo * stride];
+}
+// The way back for the data gradient: dx[plane][h][w] (+)= sub[plane][h / stride][w / stride] where both divide and the
+// pixel was looked at; the other pixels get no gradient (zero when dx is overwritten).
+__global__ __launch_bounds__(256) void scatter_strided_kernel(float* __restrict__ dx, const float* __restrict__ sub, long total, int H, int W,
+                                                              int Ho, int Wo, int stride, int accumulate) {
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int w = (int)(t % W), h = (int)((t / W) % H);
+    const long plane = t / ((long)W * H);
+    const int ho = h / stride, wo = w / stride;
+    const bool hit = ho * stride == h && wo * stride == w && ho < Ho && wo < Wo;
+    if (accumulate) {
+        if (hit) dx[t] += sub[(plane * Ho + ho) * Wo + wo];
+    } else {
+        dx[t] = hit ? sub[(plane * Ho + ho) * Wo + wo] : 0.f;
+    }
+}
+static bool conv1x1_strided(size_t K_h, size_t K_w, size_t stride, size_t pad, size_t N, size_t C, size_t H, size_t W) {
+    return K_h == 1 && K_w == 1 && stride > 1 && pad == 0 && H > 0 && W > 0 && H < 0x3fffffff && W < 0x3fffffff &&
+           (N * C * H * W + 255) / 256 < 0x7fffffffull;
+}
+// x [N, C, H, W] -> a pooled workspace [N, C, Ho, Wo] with every stride-th pixel of every stride-th row
+static int conv_subsample(float** sub, const float* x, size_t planes, size_t H, size_t W, size_t Ho, size_t Wo, size_t stride, hipStream_t s) {
+    const size_t total = planes * Ho * Wo;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(sub), total * sizeof(float), s)) return rc;
+    hipLaunchKernelGGL(subsample_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, *sub, x, (long)total, (int)H, (int)W, (int)Ho,
+                       (int)Wo, (int)stride);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        workspace_free(*sub, s);
+        return set_hip_error(e, "subsample kernel launch");
+    }
+    return NZHIP_OK;
+}
+}  // namespace nzhip
+
 using namespace nzhip;
 
 // bias_stride_image != 0: the bias varies per image too (used to add into an existing tensor: bias = y with
@@ -2655,6 +2703,17 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
     const size_t H_out = (H + 2 * pad - K_h) / stride + 1, W_out = (W + 2 * pad - K_w) / stride + 1;   // Nodes.cu:605-617
     if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (conv1x1_strided(K_h, K_w, stride, pad, N, C, H, W) && H_out * W_out >= 64) {
+        // 1x1 with a stride: gather the pixels it looks at, then the 1x1 stride-1 convolution of the smaller image
+        // (16 x 512 x 28 x 28 -> 1024 at stride 2: 42 -> 32 us; not with fewer than 64 pixels left per image, where the
+        // column matrix and one product over all images is the better way: 16 x 1024 x 14 x 14 -> 2048: 39 against 72 us)
+        float* sub = nullptr;
+        if (int rc = conv_subsample(&sub, x, N * C, H, W, H_out, W_out, stride, s)) return rc;
+        const int rc = conv2d_forward_impl(y, sub, w_ref, bias, N, C, H_out, W_out, O, 1, 1, 1, 0, w_batch, bias_stride_pixel,
+                                           bias_stride_channel, bias_stride_image, activation, stream);
+        const int rc2 = workspace_free(sub, s);
+        return rc ? rc : rc2;
+    }
     // 1x1, stride 1, no padding: no window at all, y[n] (O x pixels) = W^T (O x C) * x[n] (C x pixels) is one batched product,
     // every bias form is a bias matrix with strides. With at least 128 input channels that beats the implicit-GEMM kernels
     // (16 x 512 x 28 x 28 -> 128: 16 against 31 us; 16 x 256 x 14 x 14 -> 1024: 20 against 55 us) unless the images are tiny
@@ -2787,6 +2846,23 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
                          "nzhip_conv2d_backward_data: only square kernels, pad <= K-1 and stride <= 8 (use the column-matrix chain)");
     if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (conv1x1_strided(K_h, K_w, stride, pad, N, C, H, W) && ((H - 1) / stride + 1) * ((W - 1) / stride + 1) >= 64) {
+        // 1x1 with a stride: the gradient of the pixels the convolution looked at, as a 1x1 stride-1 problem on the
+        // smaller image, then put back between pixels that get none (16 x 512 x 28 x 28 <- 1024 at stride 2: 62 -> 45 us;
+        // with fewer than 64 pixels left per image the per-image products are too small: 16 x 1024 x 14 x 14 <- 2048: 66 -> 86)
+        const size_t Ho = (H - 1) / stride + 1, Wo = (W - 1) / stride + 1, total = N * C * H * W;
+        float* sub = nullptr;
+        if (int rc = workspace_alloc(reinterpret_cast<void**>(&sub), N * C * Ho * Wo * sizeof(float), s)) return rc;
+        int rc = nzhip_conv2d_backward_data(sub, dy, w_ref, N, C, Ho, Wo, O, 1, 1, 1, 0, w_batch, 0, stream);
+        if (rc == NZHIP_OK) {
+            hipLaunchKernelGGL(scatter_strided_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, dx, sub, (long)total, (int)H, (int)W,
+                               (int)Ho, (int)Wo, (int)stride, accumulate ? 1 : 0);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) rc = set_hip_error(e, "scatter_strided kernel launch");
+        }
+        const int rc2 = workspace_free(sub, s);
+        return rc ? rc : rc2;
+    }
     if (K_h == 1 && stride == 1 && pad == 0 && H * W < 0x3fffffff && C < 0x3fffffff && O < 0x3fffffff && N <= 65535) {
         // 1x1: no window at all, dx[n] (C x pixels) (+)= W (C x O) * dy[n] (O x pixels), one batched product
         // (16 x 256 x 14 x 14 <- 1024 channels: 38 us against 99 us through the convolution kernels)
@@ -3378,6 +3454,18 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
     if (stride == 0 || K_h == 0 || K_w == 0) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_weights: zero stride or kernel extent");
     if (H + 2 * pad < K_h || W + 2 * pad < K_w)
         return set_error(NZHIP_E_SHAPE, "nzhip_conv2d_backward_weights: kernel larger than the padded input");
+    if (conv1x1_strided(K_h, K_w, stride, pad, N, C, H, W)) {
+        // 1x1 with a stride: the pixels the convolution looked at, gathered once, then the 1x1 stride-1 product
+        // (16 x 1024 x 14 x 14 -> 2048 at stride 2: 351 -> 35 us)
+        if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
+        hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+        const size_t Ho = (H - 1) / stride + 1, Wo = (W - 1) / stride + 1;
+        float* sub = nullptr;
+        if (int rc = conv_subsample(&sub, x, N * C, H, W, Ho, Wo, stride, s)) return rc;
+        const int rc = nzhip_conv2d_backward_weights(dw, sub, dy, N, C, Ho, Wo, O, 1, 1, 1, 0, w_batch, stream);
+        const int rc2 = workspace_free(sub, s);
+        return rc ? rc : rc2;
+    }
     // 3x3, stride 1, pad 1 has a kernel of its own, built around 16-byte pieces of rows that are multiples of 8 wide; narrower
     // or odd rows (28-, 14-wide images) are better off on the gather kernel (16 x 256 x 28 x 28 -> 256: 163 us there)
     const bool own3x3 = K_h == 3 && K_w == 3 && stride == 1 && pad == 1 &&

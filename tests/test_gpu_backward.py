@@ -268,7 +268,9 @@ def test_conv2d_backward_data_float_tolerance_and_adjoint(nz, oracle):
 CONV_BWD_DATA_STRIDED = [  # N, C, H, W, O, K, stride, pad, w_batch: rows and columns no window reaches, strides 2..4, per-sample weights
     (2, 3, 7, 8, 4, 3, 2, 1, 1), (1, 2, 9, 9, 3, 3, 2, 0, 1), (2, 2, 11, 10, 2, 5, 3, 2, 2), (1, 3, 8, 6, 2, 1, 2, 0, 1),
     (2, 16, 21, 36, 24, 3, 2, 1, 1), (1, 64, 32, 64, 128, 3, 2, 1, 1), (3, 8, 17, 33, 70, 5, 2, 2, 3), (2, 24, 30, 40, 16, 3, 4, 1, 1),
-    (8, 32, 28, 28, 64, 3, 2, 1, 1)]
+    (8, 32, 28, 28, 64, 3, 2, 1, 1),
+    # 1x1 with a stride: the gradient on the gathered pixels, put back between pixels that get none
+    (2, 20, 9, 11, 33, 1, 2, 0, 1), (3, 130, 7, 13, 24, 1, 3, 0, 3), (4, 256, 14, 14, 64, 1, 2, 0, 1)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,K,stride,pad,wb", CONV_BWD_DATA_STRIDED)
@@ -386,7 +388,9 @@ CONV_GEN_BWD_W = [  # N, C, H, W, O, Kh, Kw, stride, pad, w_batch: every geometr
     # many small images: a workgroup walks several images and leaves one set of partial sums for them (rows that are whole
     # 16-byte pieces, and rows that are not); 3x3 stride 1 pad 1 on 28- and 14-wide images, which the gather kernel takes
     # from the kernel built for rows that are multiples of 8 wide
-    (40, 256, 8, 8, 16, 3, 3, 2, 1, 1), (40, 256, 8, 8, 16, 3, 3, 1, 0, 1), (3, 40, 28, 28, 24, 3, 3, 1, 1, 1), (20, 200, 14, 14, 20, 3, 3, 1, 1, 1)]
+    (40, 256, 8, 8, 16, 3, 3, 2, 1, 1), (40, 256, 8, 8, 16, 3, 3, 1, 0, 1), (3, 40, 28, 28, 24, 3, 3, 1, 1, 1), (20, 200, 14, 14, 20, 3, 3, 1, 1, 1),
+    # 1x1 with a stride: the pixels it looks at gathered once, then the 1x1 stride-1 product (shared and per-sample weights)
+    (4, 70, 14, 14, 130, 1, 1, 2, 0, 1), (3, 20, 9, 11, 33, 1, 1, 3, 0, 3)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", CONV_GEN_BWD_W)

@@ -86,6 +86,8 @@ CONV_CASES = [
     (2, 130, 9, 12, 70, 1, 1, 1, 0, 1),     # 1x1 with 128 or more input channels: one batched product
     (2, 160, 8, 8, 40, 1, 1, 1, 0, 2),      # ... with per-sample weights
     (2, 200, 5, 5, 16, 1, 1, 1, 0, 1),      # ... tiny images and fewer outputs than inputs: the convolution kernels again
+    (2, 24, 9, 11, 40, 1, 1, 2, 0, 1),      # 1x1 with a stride: every second pixel gathered, then the 1x1 stride-1 kernels
+    (3, 130, 7, 13, 20, 1, 1, 3, 0, 3),     # ... stride 3, odd extents, per-sample weights, as a batched product
     (2, 24, 40, 70, 9, 3, 3, 1, 0, 1),      # no padding, ragged width (scalar staging path)
     (1, 9, 33, 36, 140, 3, 3, 1, 2, 1),     # padding 2: both halo columns on the left
     (2, 20, 16, 64, 64, 3, 3, 1, 1, 2),     # per-sample weights
