@@ -140,7 +140,8 @@ CONV_ANY_GEOMETRY = [  # N, C, H, W, O, k_h, k_w, stride, pad, w_batch, per-pixe
     (4, 8, 66, 260, 9, 3, 3, 2, 1, 1, False),       # 130 output columns: one row per segment, the second half of it empty
     (40, 40, 20, 24, 130, 2, 3, 2, 0, 40, False),   # 2x3 kernel, no padding, per-sample weights, two channel tiles
     (32, 32, 30, 40, 64, 5, 5, 2, 3, 1, True),      # padding 3, per-pixel bias (turned into channel planes first)
-    (64, 16, 14, 16, 32, 3, 3, 2, 1, 1, False),     # 7 x 8 outputs: a segment spans the whole image and more
+    (64, 16, 14, 16, 32, 3, 3, 2, 1, 1, False),     # 7 x 8 outputs: a 16 x 16 segment would be less than half full, column matrix
+    (32, 16, 24, 32, 32, 3, 3, 2, 1, 1, False),     # 12 x 16 outputs: a segment spans the whole image and more
     (4, 16, 40, 128, 16, 5, 5, 4, 2, 1, False),     # stride 4 with 128-wide... the tile does not fit a thread's staging share: column matrix
     # few segments and many channels: the contraction split over groups of channel chunks, the groups' sums added by a
     # second kernel (a 3x3 stride-1 layer whose weights are beyond LDS, and a 5x5 stride-2 one)
