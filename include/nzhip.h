@@ -306,6 +306,18 @@ int nzhip_sgd_step(float* data, const float* grad, float lr, size_t n, void* str
 int nzhip_adam_step(float* data, float* m, float* v, const float* grad, float lr, float beta1,
                     float beta2, float eps, int t, size_t n, void* stream);
 
+/* The same steps, and nzhip_fill, for `count` tensors in one launch per NZHIP_MANY_MAX tensors.  No counterpart
+ * in the reference, which launches one kernel per parameter (ComputeGraph::update, src/ComputeGraph.cu:541-547;
+ * Tensor::zeroGrad, src/Tensor.cu:306-314): the parameters of a small network are a dozen tensors of a few floats
+ * each, and a dozen launches cost more than the work.  Every element gets exactly the arithmetic of the one-tensor
+ * call (bit-identical results); t[k] is tensor k's step count (Adam counts per call, so the tensors of one update
+ * have consecutive counts).  Tensors must not overlap. */
+#define NZHIP_MANY_MAX 16
+int nzhip_fill_many(int count, float* const* data, const size_t* n, float value, void* stream);
+int nzhip_sgd_step_many(int count, float* const* data, const float* const* grad, const size_t* n, float lr, void* stream);
+int nzhip_adam_step_many(int count, float* const* data, float* const* m, float* const* v, const float* const* grad,
+                         const size_t* n, const int* t, float lr, float beta1, float beta2, float eps, void* stream);
+
 /* ---- softmax (third caller of the GEMM entry: its backward is Jacobian x gradient) --------- */
 /* nz::data::Softmax over `batch` contiguous vectors of `len` elements (TensorOperations.cuh:379-392;
  * SummationExpKernel + SoftmaxKernel, src/OperationKernels.cu:477-523): out = exp(in) / sum(exp(in)),

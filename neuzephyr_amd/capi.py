@@ -20,7 +20,7 @@ EXPORTS = [
     "nzhip_prepared_destroy", "nzhip_gemm_prepared_b", "nzhip_conv2d_forward_prepared", "nzhip_tensorcore_gemm",
     "nzhip_im2col", "nzhip_col2im", "nzhip_conv2d_forward", "nzhip_add_broadcast", "nzhip_relu", "nzhip_fill",
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
-    "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step",
+    "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step", "nzhip_fill_many", "nzhip_sgd_step_many", "nzhip_adam_step_many",
     "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
     "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_mse_loss", "nzhip_mse_backward", "nzhip_expand", "nzhip_compress",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_host_malloc", "nzhip_host_free", "nzhip_memset",
@@ -117,6 +117,9 @@ def load() -> C.CDLL:
     lib.nzhip_expand.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_compress.argtypes = [vp, vp, sz, sz, vp]
     lib.nzhip_adam_step.argtypes = [vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, sz, vp]
+    lib.nzhip_fill_many.argtypes = [C.c_int, vp, vp, C.c_float, vp]
+    lib.nzhip_sgd_step_many.argtypes = [C.c_int, vp, vp, vp, C.c_float, vp]
+    lib.nzhip_adam_step_many.argtypes = [C.c_int, vp, vp, vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, C.c_float, vp]
     lib.nzhip_default_stream.restype = vp
     lib.nzhip_malloc.argtypes = [C.POINTER(vp), sz]
     lib.nzhip_free_async.argtypes = [vp]
@@ -425,6 +428,36 @@ def adam_step(data, m, v, grad, lr, beta1, beta2, eps, t, stream=None):
     check(lib.nzhip_adam_step(_dev(data), _dev(m), _dev(v), _dev(grad), lr, beta1, beta2, eps, t, data.numel(),
                               _stream_handle(stream)))
     return data, m, v
+
+
+def _pointer_array(tensors):
+    return (C.c_void_p * len(tensors))(*[_dev(t) for t in tensors])
+
+
+def _count_array(tensors):
+    return (C.c_size_t * len(tensors))(*[t.numel() for t in tensors])
+
+
+def fill_many(tensors, value, stream=None):
+    """nzhip_fill for a list of tensors in one launch per NZHIP_MANY_MAX of them."""
+    lib = load()
+    check(lib.nzhip_fill_many(len(tensors), _pointer_array(tensors), _count_array(tensors), float(value), _stream_handle(stream)))
+    return tensors
+
+
+def sgd_step_many(datas, grads, lr, stream=None):
+    lib = load()
+    check(lib.nzhip_sgd_step_many(len(datas), _pointer_array(datas), _pointer_array(grads), _count_array(datas), lr,
+                                  _stream_handle(stream)))
+    return datas
+
+
+def adam_step_many(datas, ms, vs, grads, ts, lr, beta1, beta2, eps, stream=None):
+    """ts[k]: the step count of tensor k (>= 1)."""
+    lib = load()
+    check(lib.nzhip_adam_step_many(len(datas), _pointer_array(datas), _pointer_array(ms), _pointer_array(vs), _pointer_array(grads),
+                                   _count_array(datas), (C.c_int * len(ts))(*ts), lr, beta1, beta2, eps, _stream_handle(stream)))
+    return datas, ms, vs
 
 
 def softmax(x, stream=None):

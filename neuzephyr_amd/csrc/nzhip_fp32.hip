@@ -215,6 +215,81 @@ __global__ __launch_bounds__(256) void adam_kernel(float* __restrict__ data, flo
     }
 }
 
+// ---- the same steps for several tensors in one launch ------------------------------------------
+// A small network has a dozen parameter tensors of a few floats each: one launch per tensor is a dozen launch
+// latencies for microseconds of work. Workgroups [first[k], first[k + 1]) belong to tensor k and do exactly what
+// the one-tensor kernel does with them (same element arithmetic, same 16-byte / scalar choice per tensor).
+constexpr int MANY_MAX = NZHIP_MANY_MAX;
+struct ManyArgs {
+    float* data[MANY_MAX];
+    float* m[MANY_MAX];
+    float* v[MANY_MAX];
+    const float* grad[MANY_MAX];
+    long n[MANY_MAX];
+    unsigned first[MANY_MAX + 1];
+    float corr1[MANY_MAX], corr2[MANY_MAX];
+    unsigned vec_mask;
+    int count;
+    float lr, beta1, beta2, eps, value;
+};
+
+__device__ __forceinline__ int many_tensor_of(const ManyArgs& a, unsigned block) {
+    int k = 0;
+    while (k + 1 < a.count && block >= a.first[k + 1]) k++;     // (uniform)
+    return k;
+}
+
+// MODE 0: fill with a.value; 1: SGD; 2: Adam
+template <int MODE>
+__global__ __launch_bounds__(256) void many_kernel(const ManyArgs a) {
+    const int k = many_tensor_of(a, blockIdx.x);
+    const unsigned blk = blockIdx.x - a.first[k], n_blk = a.first[k + 1] - a.first[k];
+    float* data = a.data[k];
+    const float* grad = a.grad[k];
+    const long n = a.n[k];
+    const long i = (long)blk * 256 + threadIdx.x;
+    AdamArgs ad;
+    ad.lr = a.lr; ad.beta1 = a.beta1; ad.beta2 = a.beta2; ad.eps = a.eps; ad.corr1 = a.corr1[k]; ad.corr2 = a.corr2[k];
+    auto one = [&](const long e) {
+        if (MODE == 0) data[e] = a.value;
+        else if (MODE == 1) data[e] = sgd_one(data[e], grad[e], a.lr);
+        else adam_one(data[e], a.m[k][e], a.v[k][e], grad[e], ad);
+    };
+    if (a.vec_mask >> k & 1) {
+        const long n4 = n >> 2;
+        if (i < n4) {
+            if (MODE == 0) {
+                const floatx4 f = {a.value, a.value, a.value, a.value};
+                reinterpret_cast<floatx4*>(data)[i] = f;
+            } else if (MODE == 1) {
+                floatx4 d = reinterpret_cast<const floatx4*>(data)[i];
+                const floatx4 g = reinterpret_cast<const floatx4*>(grad)[i];
+#pragma unroll
+                for (int e = 0; e < 4; e++) d[e] = sgd_one(d[e], g[e], a.lr);
+                reinterpret_cast<floatx4*>(data)[i] = d;
+            } else {
+                floatx4 d = reinterpret_cast<const floatx4*>(data)[i];
+                floatx4 mm = reinterpret_cast<const floatx4*>(a.m[k])[i];
+                floatx4 vv = reinterpret_cast<const floatx4*>(a.v[k])[i];
+                const floatx4 g = reinterpret_cast<const floatx4*>(grad)[i];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float de = d[e], me = mm[e], ve = vv[e];
+                    adam_one(de, me, ve, g[e], ad);
+                    d[e] = de; mm[e] = me; vv[e] = ve;
+                }
+                reinterpret_cast<floatx4*>(data)[i] = d;
+                reinterpret_cast<floatx4*>(a.m[k])[i] = mm;
+                reinterpret_cast<floatx4*>(a.v[k])[i] = vv;
+            }
+        }
+        const long t = n4 * 4 + threadIdx.x;
+        if (blk == n_blk - 1 && t < n) one(t);
+    } else if (i < n) {
+        one(i);
+    }
+}
+
 // ---- softmax over one vector per (n, c) and its Jacobian ---------------------------------------
 // One workgroup per vector: exp(x) summed in a fixed tree order (lane stride, wave shuffle, four
 // waves), then every element divided by the sum. No maximum is subtracted, like the reference
@@ -307,6 +382,55 @@ __global__ __launch_bounds__(256) void softmax_backward_kernel(float* __restrict
 
 using namespace nzhip;
 
+// Launches many_kernel<MODE> over tensors [0, count) in groups of at most MANY_MAX
+template <int MODE>
+static int many_launch(const char* who, int count, float* const* data, float* const* m, float* const* v, const float* const* grad,
+                       const size_t* n, const int* t, float lr, float beta1, float beta2, float eps, float value, void* stream) {
+    if (count < 0) return set_error(NZHIP_E_INVALID, "%s: negative count", who);
+    if (count && (!data || !n || (MODE >= 1 && !grad) || (MODE == 2 && (!m || !v || !t))))
+        return set_error(NZHIP_E_INVALID, "%s: null pointer", who);
+    for (int k = 0; k < count; k++) {
+        if (n[k] && (!data[k] || (MODE >= 1 && !grad[k]) || (MODE == 2 && (!m[k] || !v[k]))))
+            return set_error(NZHIP_E_INVALID, "%s: null pointer (tensor %d)", who, k);
+        if (MODE == 2 && t[k] < 1) return set_error(NZHIP_E_INVALID, "%s: the step count starts at 1 (tensor %d)", who, k);
+    }
+    int k = 0;
+    while (k < count) {
+        ManyArgs a = {};
+        a.lr = lr; a.beta1 = beta1; a.beta2 = beta2; a.eps = eps; a.value = value;
+        unsigned long long blocks = 0;
+        for (; k < count && a.count < MANY_MAX; k++) {
+            if (n[k] == 0) continue;
+            const int j = a.count;
+            const bool vec = aligned16(data[k]) && (MODE < 1 || aligned16(grad[k])) && (MODE < 2 || (aligned16(m[k]) && aligned16(v[k]))) &&
+                             n[k] >= 4;
+            const unsigned long long nb = vec ? (n[k] / 4 + 255) / 256 : (n[k] + 255) / 256;
+            if (blocks + nb > 0x7fffffffull) {
+                if (a.count == 0) return set_error(NZHIP_E_UNSUPPORTED, "%s: more than 2^39 elements in one tensor", who);
+                break;                                            // this tensor starts the next launch
+            }
+            a.data[j] = data[k];
+            a.grad[j] = MODE >= 1 ? grad[k] : nullptr;
+            a.m[j] = MODE == 2 ? m[k] : nullptr;
+            a.v[j] = MODE == 2 ? v[k] : nullptr;
+            a.n[j] = (long)n[k];
+            if (MODE == 2) {
+                a.corr1[j] = 1.0f - powf(beta1, (float)t[k]);
+                a.corr2[j] = 1.0f - powf(beta2, (float)t[k]);
+            }
+            if (vec) a.vec_mask |= 1u << j;
+            a.first[j] = (unsigned)blocks;
+            blocks += nb;
+            a.first[j + 1] = (unsigned)blocks;
+            a.count++;
+        }
+        if (a.count == 0) continue;
+        hipLaunchKernelGGL(many_kernel<MODE>, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), a);
+        if (int rc = check_launch("many_kernel")) return rc;
+    }
+    return NZHIP_OK;
+}
+
 extern "C" {
 
 int nzhip_matmul_f32(const float* A, const float* B, float* C, const size_t sA[4], const size_t sB[4],
@@ -365,6 +489,19 @@ int nzhip_adam_step(float* data, float* m, float* v, const float* grad, float lr
         hipLaunchKernelGGL(adam_kernel<1>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), data, m, v,
                            grad, a, (long)n);
     return check_launch("adam_kernel");
+}
+
+int nzhip_fill_many(int count, float* const* data, const size_t* n, float value, void* stream) {
+    return many_launch<0>("nzhip_fill_many", count, data, nullptr, nullptr, nullptr, n, nullptr, 0.f, 0.f, 0.f, 0.f, value, stream);
+}
+
+int nzhip_sgd_step_many(int count, float* const* data, const float* const* grad, const size_t* n, float lr, void* stream) {
+    return many_launch<1>("nzhip_sgd_step_many", count, data, nullptr, nullptr, grad, n, nullptr, lr, 0.f, 0.f, 0.f, 0.f, stream);
+}
+
+int nzhip_adam_step_many(int count, float* const* data, float* const* m, float* const* v, const float* const* grad, const size_t* n,
+                         const int* t, float lr, float beta1, float beta2, float eps, void* stream) {
+    return many_launch<2>("nzhip_adam_step_many", count, data, m, v, grad, n, t, lr, beta1, beta2, eps, 0.f, stream);
 }
 
 int nzhip_softmax(float* out, const float* in, size_t len, size_t batch, void* stream) {

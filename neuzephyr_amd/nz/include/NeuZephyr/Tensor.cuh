@@ -71,6 +71,9 @@ namespace nz::data {
         void dataInject(const std::initializer_list<value_type>& data, bool grad = false) const;
 
         void zeroGrad() const;
+        // Runs the clears that zeroGrad() left pending on these tensors in one launch (a backward pass that will add
+        // into a dozen small parameter gradients would otherwise start a dozen clears, one per first touch).
+        static void clearPendingGrads(const std::vector<const Tensor*>& tensors);
         void clear() const;
         void fill(value_type value, bool isGrad = false) const;
         // Deterministic uniform (0,1] fill. The reference draws from cuRAND's XORWOW stream

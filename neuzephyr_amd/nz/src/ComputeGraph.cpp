@@ -357,6 +357,11 @@ namespace nz::graph {
             for (Node* node : fusedMembers) node->forward();
             intermediatesStale = false;
         }
+        // the leaves' gradients are added into: whatever zeroGrad() left to clear on them is cleared in one launch
+        std::vector<const Tensor*> leaves;
+        for (Node* node : nodes)
+            if (node->inputs.empty() && node->output && node->output->requiresGrad()) leaves.push_back(node->output.get());
+        Tensor::clearPendingGrads(leaves);
         for (auto& step : backPlan) step();
     }
 
@@ -367,11 +372,13 @@ namespace nz::graph {
         // skip(), which keeps an optimizer's per-call state in step with the reference: Adam's bias
         // corrections use the number of step() calls so far (src/Optimizer.cu:86-101), so a leaf must see
         // the same count as it would there.
+        optimizer->begin();                              // the steps of all leaves may go out as one launch
         for (Node* node : nodes) {
             if (!node->output || !node->output->requiresGrad()) continue;
             if (node->inputs.empty()) optimizer->step(node);
             else optimizer->skip(node);
         }
+        optimizer->end();
     }
 
     unsigned long long ComputeGraph::weightImageBuilds() const {

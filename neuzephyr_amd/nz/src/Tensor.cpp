@@ -170,6 +170,19 @@ namespace nz::data {
         if (_requires_grad && _size && _grad) _gradZeroPending = true;
     }
 
+    void Tensor::clearPendingGrads(const std::vector<const Tensor*>& tensors) {
+        std::vector<value_type*> ptrs;
+        std::vector<size_t> counts;
+        for (const Tensor* t : tensors) {
+            if (!t || !t->_requires_grad || !t->_grad || !t->_gradZeroPending || t->_size == 0) continue;
+            ptrs.push_back(t->_grad);
+            counts.push_back(t->_size);
+            t->_gradZeroPending = false;
+        }
+        if (!ptrs.empty())
+            NZ_CHECK(nzhip_fill_many(static_cast<int>(ptrs.size()), ptrs.data(), counts.data(), 0.f, nzhip_default_stream()));
+    }
+
     void Tensor::clear() const {
         if (_size) NZ_CHECK(nzhip_memset(data(), 0, _size * sizeof(value_type)));
     }

@@ -93,6 +93,47 @@ def test_adam_steps_match_oracle(nz, oracle):
         nz.adam_step(d, m, v, dev(grad), 0.01, 0.9, 0.999, 1e-6, 0)
 
 
+def test_many_tensor_steps_equal_the_one_tensor_calls(nz):
+    """One launch for up to 16 tensors: every element gets the arithmetic of the one-tensor call (bit-identical),
+    for sizes with and without 16-byte tails, an unaligned tensor, an empty one, and more tensors than one launch takes."""
+    import torch
+    rng = np.random.default_rng(59)
+    sizes = [1, 3, 4, 27, 72, 1024, 4097, 0, 260100, 16, 5, 300000, 7, 64, 129, 2, 33, 1000, 6]      # 19 tensors: two launches
+    def tensors(seed, offset_one=True):
+        r = np.random.default_rng(seed)
+        out = []
+        for i, n in enumerate(sizes):
+            base = dev(r.uniform(-10, 10, n + 1).astype(np.float32))
+            out.append(base[1:] if (offset_one and i == 5) else base[:n])       # tensor 5 is not 16-byte aligned
+        return out
+    # fill
+    a, b = tensors(1), tensors(1)
+    nz.fill_many(a, 0.25)
+    for t in b: nz.fill(t, 0.25)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    # SGD
+    a, b, g = tensors(2), tensors(2), tensors(3)
+    nz.sgd_step_many(a, g, 0.01)
+    for x, gg in zip(b, g):
+        if x.numel(): nz.sgd_step(x, gg, 0.01)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    # Adam, two updates with consecutive step counts per tensor as ComputeGraph::update produces them
+    a, b, g = tensors(4), tensors(4), tensors(5)
+    ma, mb = [torch.zeros_like(x) for x in a], [torch.zeros_like(x) for x in b]
+    va, vb = [torch.zeros_like(x) for x in a], [torch.zeros_like(x) for x in b]
+    count = 0
+    for update in range(2):
+        ts = list(range(count + 1, count + 1 + len(sizes)))
+        count += len(sizes)
+        nz.adam_step_many(a, ma, va, g, ts, 0.01, 0.9, 0.999, 1e-6)
+        for x, m, v, gg, t in zip(b, mb, vb, g, ts):
+            if x.numel(): nz.adam_step(x, m, v, gg, 0.01, 0.9, 0.999, 1e-6, t)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    assert all(torch.equal(x, y) for x, y in zip(ma, mb)) and all(torch.equal(x, y) for x, y in zip(va, vb))
+    with pytest.raises(nz.NzHipError):
+        nz.adam_step_many(a[:2], ma[:2], va[:2], g[:2], [1, 0], 0.01, 0.9, 0.999, 1e-6)
+
+
 def test_softmax_forward_jacobian_backward(nz, oracle):
     rng = np.random.default_rng(47)
     for shape in [(2, 3, 12, 1), (1, 2, 1, 300), (3, 1, 1000, 1), (1, 1, 1, 1)]:
