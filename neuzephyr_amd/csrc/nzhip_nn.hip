@@ -26,6 +26,9 @@ struct PoolArgs {
 
 // One thread per output element: the window is summed row by row, left to right (the reference's
 // loop order), and divided by the number of window cells inside the image.
+// POOL: the window extent at compile time (0: p.pool); a window inside the image is then pool^2 loads and adds
+// without a loop or a bounds test.
+template <int POOL>
 __global__ __launch_bounds__(256) void avgpool_kernel(float* __restrict__ out, const float* __restrict__ in,
                                                       const PoolArgs p) {
     // grid: x = (output row, 256-column block), y and z = plane; nothing here divides per thread
@@ -37,14 +40,26 @@ __global__ __launch_bounds__(256) void avgpool_kernel(float* __restrict__ out, c
     const float* src = in + plane * p.H_in * p.W_in;
     float sum = 0.f;
     int count = 0;
-    for (int i = 0; i < p.pool; i++) {
-        const int hi = h0 + i;
-        if (hi < 0 || hi >= p.H_in) continue;
-        for (int j = 0; j < p.pool; j++) {
-            const int wi = w0 + j;
-            if (wi >= 0 && wi < p.W_in) {
-                sum += src[(long)hi * p.W_in + wi];
-                count++;
+    if (POOL && h0 >= 0 && h0 + POOL <= p.H_in && w0 >= 0 && w0 + POOL <= p.W_in) {
+        const float* win = src + (long)h0 * p.W_in + w0;
+        float v[POOL ? POOL * POOL : 1];
+#pragma unroll
+        for (int i = 0; i < POOL; i++)
+#pragma unroll
+            for (int j = 0; j < POOL; j++) v[i * POOL + j] = win[(long)i * p.W_in + j];
+#pragma unroll
+        for (int k = 0; k < POOL * POOL; k++) sum += v[k];
+        count = POOL * POOL;
+    } else {
+        for (int i = 0; i < p.pool; i++) {
+            const int hi = h0 + i;
+            if (hi < 0 || hi >= p.H_in) continue;
+            for (int j = 0; j < p.pool; j++) {
+                const int wi = w0 + j;
+                if (wi >= 0 && wi < p.W_in) {
+                    sum += src[(long)hi * p.W_in + wi];
+                    count++;
+                }
             }
         }
     }
@@ -90,6 +105,77 @@ __global__ __launch_bounds__(256) void avgpool_backward_kernel(float* __restrict
     for (int oh = oh_lo; oh <= oh_hi; oh++)
         for (int ow = ow_lo; ow <= ow_hi; ow++) acc += g[(long)oh * p.W_out + ow];
     din[idx] = acc;
+}
+
+// The same sums for four adjacent input columns per thread (rows of whole 16-byte pieces): the gradient row moves as
+// 16-byte accesses, and a share that several of the four columns need is requested once. Every column still adds its
+// shares in ascending (row, column) order of the windows.
+// RMAX, CMAX: the most window rows that cover an input row ((pool - 1) / stride + 1) and the most window columns that
+// cover four adjacent input columns ((pool + 2) / stride + 1), at compile time: all RMAX * CMAX shares are then requested
+// at once (clamped addresses) before the first is added. 0: bounds known only at run time, one request per loop step.
+template <int RMAX, int CMAX>
+// This kernel reads dout and divides by the window's cell count itself (the same fp32 division as avgpool_share_kernel:
+// a dozen divisions per thread cost less than a pass that writes the shares and another that reads them).
+__global__ __launch_bounds__(256) void avgpool_backward_vec_kernel(float* __restrict__ din, const float* __restrict__ dout,
+                                                                   const PoolArgs p, const int wblocks4) {
+    typedef float floatx4 __attribute__((ext_vector_type(4)));
+    const int h = blockIdx.x / wblocks4, w = ((blockIdx.x % wblocks4) * 256 + threadIdx.x) * 4;
+    const long plane = blockIdx.y + (long)gridDim.y * blockIdx.z;
+    if (w >= p.W_in || plane >= p.planes) return;
+    const long idx = (plane * p.H_in + h) * p.W_in + w;
+    const int hp = h + p.pad;
+    const int oh_lo = hp - p.pool + 1 <= 0 ? 0 : (hp - p.pool + p.stride) / p.stride;
+    int oh_hi = hp / p.stride;
+    if (oh_hi > p.H_out - 1) oh_hi = p.H_out - 1;
+    const float fs = (float)p.stride;
+    int lo[4], hi[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int wp = w + e + p.pad;
+        lo[e] = wp - p.pool + 1 <= 0 ? 0 : (int)((float)(wp - p.pool + p.stride) / fs);
+        hi[e] = (int)((float)wp / fs);
+        if (hi[e] > p.W_out - 1) hi[e] = p.W_out - 1;
+    }
+    const float* g = dout + plane * p.H_out * p.W_out;
+    auto divisor = [&](const int oh, const int ow) {
+        if (p.pad == 0) return (float)(p.pool * p.pool);
+        const int h0 = oh * p.stride - p.pad, w0 = ow * p.stride - p.pad;
+        const int rows = min(h0 + p.pool, p.H_in) - max(h0, 0), cols = min(w0 + p.pool, p.W_in) - max(w0, 0);
+        return (float)(rows * cols);
+    };
+    floatx4 acc = *reinterpret_cast<const floatx4*>(din + idx);
+    if (RMAX) {
+        float sv[RMAX ? RMAX * CMAX : 1];
+#pragma unroll
+        for (int r = 0; r < RMAX; r++)
+#pragma unroll
+            for (int c = 0; c < CMAX; c++) {
+                const int oh = oh_lo + r, ow = lo[0] + c;
+                const bool ok = oh <= oh_hi && ow <= hi[3];
+                sv[r * CMAX + c] = g[ok ? (long)oh * p.W_out + ow : 0];
+            }
+#pragma unroll
+        for (int r = 0; r < RMAX; r++)
+#pragma unroll
+            for (int c = 0; c < CMAX; c++) {
+                const int oh = oh_lo + r, ow = lo[0] + c;
+                const float v = sv[r * CMAX + c] / divisor(oh, ow);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (oh <= oh_hi && ow >= lo[e] && ow <= hi[e]) acc[e] += v;
+            }
+    } else {
+        for (int oh = oh_lo; oh <= oh_hi; oh++) {
+            const float* grow = g + (long)oh * p.W_out;
+            for (int ow = lo[0]; ow <= hi[3]; ow++) {                   // (bounds are monotone in the column)
+                const float v = grow[ow] / divisor(oh, ow);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (ow >= lo[e] && ow <= hi[e]) acc[e] += v;
+            }
+        }
+    }
+    *reinterpret_cast<floatx4*>(din + idx) = acc;
 }
 
 // ---- binary cross-entropy ------------------------------------------------------------------------
@@ -208,7 +294,8 @@ int nzhip_avgpool2d(float* out, const float* in, size_t pool, size_t stride, siz
     if (int rc = pool_args(p, pool, stride, pad, batches, channels, H_in, W_in, H_out, W_out, "nzhip_avgpool2d")) return rc;
     const size_t total = batches * channels * H_out * W_out;
     if (total == 0) return NZHIP_OK;
-    hipLaunchKernelGGL(avgpool_kernel, pool_grid(p.wblocks, p.H_out, p.planes), dim3(256), 0, as_stream(stream), out, in, p);
+    auto kfn = p.pool == 2 ? avgpool_kernel<2> : p.pool == 3 ? avgpool_kernel<3> : p.pool == 5 ? avgpool_kernel<5> : avgpool_kernel<0>;
+    hipLaunchKernelGGL(kfn, pool_grid(p.wblocks, p.H_out, p.planes), dim3(256), 0, as_stream(stream), out, in, p);
     return check_launch("avgpool_kernel");
 }
 
@@ -222,6 +309,18 @@ int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t 
     const size_t outs = batches * channels * H_out * W_out;
     if (outs == 0) return NZHIP_OK;
     hipStream_t s = as_stream(stream);
+    if (p.W_in % 4 == 0 && (reinterpret_cast<uintptr_t>(din) & 15) == 0) {
+        const int wblocks4 = (p.W_in / 4 + 255) / 256;
+        const int rmax = (p.pool - 1) / p.stride + 1, cmax = (p.pool + 2) / p.stride + 1;
+        auto kfn = rmax == 3 && cmax == 4   ? avgpool_backward_vec_kernel<3, 4>      // 5 / 2
+                   : rmax == 2 && cmax == 3 ? avgpool_backward_vec_kernel<2, 3>      // 3 / 2
+                   : rmax == 1 && cmax == 3 ? avgpool_backward_vec_kernel<1, 3>      // 2 / 2
+                   : rmax == 3 && cmax == 6 ? avgpool_backward_vec_kernel<3, 6>      // 3 / 1
+                   : rmax == 2 && cmax == 5 ? avgpool_backward_vec_kernel<2, 5>      // 2 / 1
+                                            : avgpool_backward_vec_kernel<0, 0>;
+        hipLaunchKernelGGL(kfn, pool_grid(wblocks4, p.H_in, p.planes), dim3(256), 0, s, din, dout, p, wblocks4);
+        return check_launch("avgpool_backward_vec_kernel");
+    }
     float* share = nullptr;
     if (int rc = workspace_alloc(reinterpret_cast<void**>(&share), outs * sizeof(float), s)) return rc;
     hipLaunchKernelGGL(avgpool_share_kernel, pool_grid(p.wblocks, p.H_out, p.planes), dim3(256), 0, s, share, dout, p);

@@ -9,7 +9,11 @@ pytestmark = pytest.mark.gpu
 
 POOL_CASES = [((2, 3, 4, 5), 2, 2, 0), ((1, 2, 9, 7), 3, 1, 1), ((2, 1, 10, 10), 5, 2, 0), ((1, 1, 6, 8), 4, 3, 2),
               ((1, 3, 5, 5), 5, 1, 2), ((2, 2, 7, 3), 1, 1, 0), ((1, 1, 8, 8), 3, 2, 1), ((3, 5, 33, 47), 3, 2, 1),
-              ((1, 1, 70, 300), 5, 2, 0), ((2, 2, 16, 16), 2, 2, 0), ((1, 1, 9, 9), 4, 5, 3)]
+              ((1, 1, 70, 300), 5, 2, 0), ((2, 2, 16, 16), 2, 2, 0), ((1, 1, 9, 9), 4, 5, 3),
+              # several 256-column blocks and row tiles of the LDS-tile kernel, rows of whole 16-byte pieces for the
+              # four-column gradient kernel (with and without padding), a stride whose tile does not fit LDS
+              ((2, 1, 40, 1100), 5, 2, 0), ((1, 2, 30, 64), 3, 2, 1), ((1, 1, 24, 520), 2, 2, 0), ((1, 1, 20, 36), 7, 3, 2),
+              ((1, 1, 40, 2000), 3, 20, 0)]
 
 
 @pytest.fixture(scope="module")
