@@ -30,11 +30,13 @@ struct PoolArgs {
 // without a loop or a bounds test.
 template <int POOL>
 __global__ __launch_bounds__(256) void avgpool_kernel(float* __restrict__ out, const float* __restrict__ in,
-                                                      const PoolArgs p) {
-    // grid: x = (output row, 256-column block), y and z = plane; nothing here divides per thread
-    const int h = blockIdx.x / p.wblocks, w = (blockIdx.x % p.wblocks) * 256 + threadIdx.x;
+                                                      const PoolArgs p, const int cw_log, const int wblocks) {
+    // grid: x = (block of 256 >> cw_log output rows, block of 1 << cw_log columns), y and z = plane; nothing here divides
+    // per thread. Narrow images get several rows per workgroup instead of a row of mostly idle lanes.
+    const int h = (blockIdx.x / wblocks) * (256 >> cw_log) + (threadIdx.x >> cw_log);
+    const int w = ((blockIdx.x % wblocks) << cw_log) + (threadIdx.x & ((1 << cw_log) - 1));
     const long plane = blockIdx.y + (long)gridDim.y * blockIdx.z;
-    if (w >= p.W_out || plane >= p.planes) return;
+    if (w >= p.W_out || h >= p.H_out || plane >= p.planes) return;
     const long idx = (plane * p.H_out + h) * p.W_out + w;
     const int h0 = h * p.stride - p.pad, w0 = w * p.stride - p.pad;
     const float* src = in + plane * p.H_in * p.W_in;
@@ -117,11 +119,13 @@ template <int RMAX, int CMAX>
 // This kernel reads dout and divides by the window's cell count itself (the same fp32 division as avgpool_share_kernel:
 // a dozen divisions per thread cost less than a pass that writes the shares and another that reads them).
 __global__ __launch_bounds__(256) void avgpool_backward_vec_kernel(float* __restrict__ din, const float* __restrict__ dout,
-                                                                   const PoolArgs p, const int wblocks4) {
+                                                                   const PoolArgs p, const int cw_log, const int wblocks4) {
     typedef float floatx4 __attribute__((ext_vector_type(4)));
-    const int h = blockIdx.x / wblocks4, w = ((blockIdx.x % wblocks4) * 256 + threadIdx.x) * 4;
+    // (block of 256 >> cw_log input rows, block of 1 << cw_log column quads), as in the forward kernel
+    const int h = (blockIdx.x / wblocks4) * (256 >> cw_log) + (threadIdx.x >> cw_log);
+    const int w = (((blockIdx.x % wblocks4) << cw_log) + (threadIdx.x & ((1 << cw_log) - 1))) * 4;
     const long plane = blockIdx.y + (long)gridDim.y * blockIdx.z;
-    if (w >= p.W_in || plane >= p.planes) return;
+    if (w >= p.W_in || h >= p.H_in || plane >= p.planes) return;
     const long idx = (plane * p.H_in + h) * p.W_in + w;
     const int hp = h + p.pad;
     const int oh_lo = hp - p.pool + 1 <= 0 ? 0 : (hp - p.pool + p.stride) / p.stride;
@@ -275,6 +279,13 @@ static int pool_args(PoolArgs& p, size_t pool, size_t stride, size_t pad, size_t
     return NZHIP_OK;
 }
 
+// log2 of the column-block width for rows of `width` elements: the power of two from 16 to 256 that covers them
+static int pool_cw_log(long width) {
+    int cw_log = 8;
+    while (cw_log > 4 && (1l << (cw_log - 1)) >= width) cw_log--;
+    return cw_log;
+}
+
 // x = rows x column blocks, planes folded into y (up to 65535) and z
 static dim3 pool_grid(int wblocks, int rows, long planes) {
     const long gy = planes < 65535 ? planes : 65535;
@@ -295,7 +306,8 @@ int nzhip_avgpool2d(float* out, const float* in, size_t pool, size_t stride, siz
     const size_t total = batches * channels * H_out * W_out;
     if (total == 0) return NZHIP_OK;
     auto kfn = p.pool == 2 ? avgpool_kernel<2> : p.pool == 3 ? avgpool_kernel<3> : p.pool == 5 ? avgpool_kernel<5> : avgpool_kernel<0>;
-    hipLaunchKernelGGL(kfn, pool_grid(p.wblocks, p.H_out, p.planes), dim3(256), 0, as_stream(stream), out, in, p);
+    const int cw_log = pool_cw_log(p.W_out), wblocks = (p.W_out + (1 << cw_log) - 1) >> cw_log, rb = 256 >> cw_log;
+    hipLaunchKernelGGL(kfn, pool_grid(wblocks, (p.H_out + rb - 1) / rb, p.planes), dim3(256), 0, as_stream(stream), out, in, p, cw_log, wblocks);
     return check_launch("avgpool_kernel");
 }
 
@@ -310,7 +322,7 @@ int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t 
     if (outs == 0) return NZHIP_OK;
     hipStream_t s = as_stream(stream);
     if (p.W_in % 4 == 0 && (reinterpret_cast<uintptr_t>(din) & 15) == 0) {
-        const int wblocks4 = (p.W_in / 4 + 255) / 256;
+        const int cw_log = pool_cw_log(p.W_in / 4), wblocks4 = (p.W_in / 4 + (1 << cw_log) - 1) >> cw_log, rb = 256 >> cw_log;
         const int rmax = (p.pool - 1) / p.stride + 1, cmax = (p.pool + 2) / p.stride + 1;
         auto kfn = rmax == 3 && cmax == 4   ? avgpool_backward_vec_kernel<3, 4>      // 5 / 2
                    : rmax == 2 && cmax == 3 ? avgpool_backward_vec_kernel<2, 3>      // 3 / 2
@@ -318,7 +330,7 @@ int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t 
                    : rmax == 3 && cmax == 6 ? avgpool_backward_vec_kernel<3, 6>      // 3 / 1
                    : rmax == 2 && cmax == 5 ? avgpool_backward_vec_kernel<2, 5>      // 2 / 1
                                             : avgpool_backward_vec_kernel<0, 0>;
-        hipLaunchKernelGGL(kfn, pool_grid(wblocks4, p.H_in, p.planes), dim3(256), 0, s, din, dout, p, wblocks4);
+        hipLaunchKernelGGL(kfn, pool_grid(wblocks4, (p.H_in + rb - 1) / rb, p.planes), dim3(256), 0, s, din, dout, p, cw_log, wblocks4);
         return check_launch("avgpool_backward_vec_kernel");
     }
     float* share = nullptr;
