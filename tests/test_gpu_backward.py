@@ -187,7 +187,10 @@ def test_fill_writes_every_element(nz):
 
 IM2COL_CASES = [((2, 3, 4, 5), 3, 3, 1, 1), ((1, 1, 1, 1), 1, 1, 1, 0), ((2, 2, 7, 6), 3, 2, 2, 0),
                 ((1, 3, 8, 9), 2, 4, 2, 2), ((3, 1, 5, 5), 5, 5, 1, 2), ((2, 4, 6, 6), 1, 1, 3, 0),
-                ((2, 5, 33, 47), 3, 3, 1, 1), ((1, 2, 9, 9), 3, 3, 3, 1)]
+                ((2, 5, 33, 47), 3, 3, 1, 1), ((1, 2, 9, 9), 3, 3, 3, 1),
+                # wide rows and many channels, strides 2 and 4, padding beyond the reach of a tap, a window of most of the image
+                ((2, 19, 12, 70), 3, 3, 1, 1), ((1, 6, 10, 150), 5, 5, 1, 2), ((1, 3, 11, 300), 7, 7, 2, 3), ((2, 2, 9, 40), 11, 11, 4, 5),
+                ((1, 9, 20, 33), 3, 3, 2, 1), ((1, 1, 70, 70), 65, 65, 1, 0)]
 
 
 @pytest.mark.parametrize("shape,k_h,k_w,stride,pad", IM2COL_CASES)
