@@ -3469,9 +3469,14 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
         return rc ? rc : rc2;
     }
     // 3x3, stride 1, pad 1 has a kernel of its own, built around 16-byte pieces of rows that are multiples of 8 wide; narrower
-    // or odd rows (28-, 14-wide images) are better off on the gather kernel (16 x 256 x 28 x 28 -> 256: 163 us there)
+    // or odd rows (28-, 14-wide images) are better off on the gather kernel (16 x 256 x 28 x 28 -> 256: 163 us there), and so
+    // are images up to 64 wide with 128 or more input channels (16 x 512 x 32 x 32 -> 512: 450 against 150 us; 16 x 128 x
+    // 56 x 56 -> 256: 110 against 86), whose 32-channel workgroups re-read the output gradient once per 32 input channels
+    static const char* dw_env = getenv("NZHIP_CONV_DW");             // benchmarking only: "gather" / "own" force either where both apply
+    const bool prefer_gather = dw_env ? dw_env[0] == 'g' : (W <= 64 && C >= 128);
     const bool own3x3 = K_h == 3 && K_w == 3 && stride == 1 && pad == 1 &&
-                        ((W % 8 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0) || (C <= 4 && O <= 2));
+                        ((W % 8 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0 && !prefer_gather) ||
+                         (C <= 4 && O <= 2));
     if (!own3x3) {
         // any other geometry: the gather kernel (up to 128 taps, stride up to 4, extents that fit its index arithmetic)
         const bool fits = K_h * K_w <= (size_t)DWG_ROWS && stride <= 4 && pad < 0x10000 && H < 0x3fffffff && W < 0x3fffffff &&

@@ -306,7 +306,9 @@ CONV_BWD_W = [  # N, C, H, W, O, w_batch   (3x3, stride 1, pad 1; W a multiple o
     # C <= 4, O <= 2, W a multiple of 4: the streaming kernel (strips of 16 rows, 256 columns per wave; partial last
     # strip, several column blocks with a ragged last one, per-sample and shared weights)
     (2, 3, 20, 24, 1, 2), (3, 1, 33, 260, 1, 3), (1, 4, 5, 8, 2, 1), (2, 2, 70, 516, 2, 1), (2, 3, 64, 256, 1, 1),
-    (1, 1, 1, 4, 1, 1)]
+    (1, 1, 1, 4, 1, 1),
+    # 128 or more input channels on images up to 64 wide: the gather kernel although the rows are multiples of 8 wide
+    (2, 130, 9, 24, 40, 1), (2, 128, 6, 64, 33, 2)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,wb", CONV_BWD_W)
