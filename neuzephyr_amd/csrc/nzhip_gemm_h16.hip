@@ -1037,8 +1037,8 @@ static inline long round_up(long v, long q) { return (v + q - 1) / q * q; }
 bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
     // Worth it when each operand element is re-read by many tiles, i.e. when the GEMM does far
     // more work per operand byte than the extra rounding pass moves. Measured on MI355X
-    // (microseconds, fused / two-pass): 4096x1024x4096 66 / 60, 3072^3 136 / 102, 4096^3 197 / 163,
-    // but 2048^3 44 / 53, 4096x256x4096 30 / 36, 8192x512x8192 160 / 168 (short contractions leave
+    // (microseconds, fused / two-pass): 3072^3 136 / 102, 4096^3 197 / 163, 4096x4096x1024 60 / 52,
+    // but 2048^3 44 / 53, 4096x1024x4096 67 / 77, 4096x256x4096 30 / 36, 8192x512x8192 160 / 168 (short contractions leave
     // the rounding pass and the C stores nothing to hide behind). Shapes that are not whole
     // 256x256x32 tiles take the fused kernel's predicated instance, which is much slower, so the
     // threshold is lower for them: 2500^3 101 / 68, 5000x1000x5000 156 / 94, 2000^3 56 / 55.
@@ -1047,7 +1047,9 @@ bool gemm_h16_applicable(const nzhip_gemm_desc& d) {
     const double cvt_bytes = 6.0 * ((double)d.M * d.K + (double)d.N * d.K);
     const bool whole_tiles = d.M % 256 == 0 && d.N % 256 == 0 && d.K % 32 == 0 && d.lda % 4 == 0 && d.ldb % 4 == 0 &&
                              d.ldc % 4 == 0;
-    return flops / cvt_bytes >= (whole_tiles ? 512.0 : 300.0);
+    // (whole tiles, fused / two-pass: 2048^3 38 / 45 and 2048x2048x4096 67 / 74 at a ratio of 341, but 2304^3 62 / 50 at 384,
+    // 3072x2048x2048 55 / 47 at 410, 2560^3 71 / 55 at 427, 4096x2048x4096 118 / 92 and 2048x4096x3072 94 / 73 at 455)
+    return flops / cvt_bytes >= (whole_tiles ? 360.0 : 300.0);
 }
 
 // Host-side bookkeeping of the bounded waits: which stream the products enqueued since the last look went to,
