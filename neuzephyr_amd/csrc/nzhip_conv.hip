@@ -1700,6 +1700,7 @@ struct ConvGenArgs {
     int w_pitch, slab_bytes, halo_off;
     long bias_sp, bias_sc, bias_sn;
     int relu;
+    int img_chunks, halo_plane;           // chunks per channel tile in the weight image (n_chunks rounded up to CPB); bytes of one halo plane
     int chunk_groups, chunks_per_group;   // the contraction split over groups of channel chunks (blockIdx.z = image * groups + group)
     float* partial;                       // with more than one group: [group][image][O][Ho * Wo] sums without bias or activation
 };
@@ -1724,7 +1725,10 @@ __global__ __launch_bounds__(256) void conv_weight_image_gen_kernel(_Float16* __
 // VEC: image rows are whole 16-byte pieces (W a multiple of 4, aligned x): a task's four columns are one load per
 // channel and lie inside or outside the image together; otherwise (14 x 14 images ...) four loads with their own bounds.
 // PIXB: the bias varies per pixel (the reference's Bias node after the matmul; the per-image bias of an in-place data gradient).
-template <int NO, int TP, bool VEC, bool PIXB>
+// CPB: 16-channel chunks per loop step (p.n_chunks counts steps). With 2, a step stages two halo planes and two slabs and
+// multiplies 2 x taps times between its two barriers: the store / barrier / request phases, which cost as much as the 9
+// taps of a 3x3 chunk, are paid half as often (layers with many channels; 16 x 256 x 56 x 56 -> 256: 124 -> 95 us).
+template <int NO, int TP, bool VEC, bool PIXB, int CPB>
 __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGenArgs p) {
     constexpr int BN = NO * 64;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -1747,12 +1751,12 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
     const long plane = (long)p.H * p.W;
     const float* xb = p.x + (long)b * p.C * plane;
     const char* wsrc = reinterpret_cast<const char*>(p.wimg) +
-                       ((long)(p.w_batched ? b : 0) * p.n_otiles + o_tile) * p.n_chunks * p.slab_bytes + lane * 16;
+                       ((long)(p.w_batched ? b : 0) * p.n_otiles + o_tile) * p.img_chunks * p.slab_bytes + lane * 16;
 
-    // staging tasks: task e = tid + 512 k is (8-channel half, staged row, column quad)
-    const int pw4 = p.pw >> 2, n_tasks = 2 * p.span * pw4;
+    // staging tasks: task e = tid + 512 k is (8-channel group of the step's 16 CPB channels, staged row, column quad)
+    const int pw4 = p.pw >> 2, n_tasks = 2 * CPB * p.span * pw4;
     int t_off[TP], t_dst[TP];                                   // image offset of the quad's first column, LDS byte offset of its first pixel (or -1)
-    int t_h8[TP];                                               // bits 0..3: which of the four columns are inside the image; bit 4: the channel half
+    int t_h8[TP];                                               // bits 0..3: which of the four columns are inside the image; bits 4..: the 8-channel group
 #pragma unroll
     for (int k = 0; k < TP; k++) {
         const int e = tid + CG_THREADS * k;
@@ -1779,7 +1783,7 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
     auto load_halo = [&](const int chunk) {
 #pragma unroll
         for (int k = 0; k < TP; k++) {
-            const int c0 = chunk * IG_CC + (t_h8[k] >> 4) * 8;
+            const int c0 = chunk * (IG_CC * CPB) + (t_h8[k] >> 4) * 8;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 const bool c_ok = c0 + e < p.C;
@@ -1800,24 +1804,25 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
 #pragma unroll
         for (int k = 0; k < TP; k++) {
             if (t_dst[k] < 0) continue;
-            const int h8 = t_h8[k] >> 4;
-            const int c0 = chunk * IG_CC + h8 * 8;
+            const int g8 = t_h8[k] >> 4, h8 = g8 & 1;            // 8-channel group of the step; half of its 16-channel plane
+            const int c0 = chunk * (IG_CC * CPB) + g8 * 8;
             const int col0 = (t_dst[k] >> 5) % p.pw;            // staged column of the quad's first pixel (a multiple of 4)
+            char* plane_h = lds_h + (CPB > 1 ? (g8 >> 1) * p.halo_plane : 0);
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 half8_t h;
 #pragma unroll
                 for (int e = 0; e < 8; e++) h[e] = ((t_h8[k] >> q & 1) && c0 + e < p.C) ? (_Float16)raw[k][e][q] : (_Float16)0.f;
                 const int col = col0 + q;
-                *reinterpret_cast<half8_t*>(lds_h + t_dst[k] + q * 32 + ((h8 ^ ((col >> 3) & 1)) << 4)) = h;
+                *reinterpret_cast<half8_t*>(plane_h + t_dst[k] + q * 32 + ((h8 ^ ((col >> 3) & 1)) << 4)) = h;
             }
         }
     };
     auto load_slab = [&](const int chunk) {
-        const int pieces = p.slab_bytes >> 10;
+        const int pieces = (CPB * p.slab_bytes) >> 10;          // the step's slabs follow each other in the image
         for (int j = wave; j < pieces; j += CG_THREADS / 64)
             __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void*)(wsrc + (long)chunk * p.slab_bytes + j * 1024),
+                (const __attribute__((address_space(1))) void*)(wsrc + (long)chunk * (CPB * p.slab_bytes) + j * 1024),
                 (__attribute__((address_space(3))) void*)(lds_w + j * 1024), 16, 0, 0);
     };
 
@@ -1879,41 +1884,48 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
         __syncthreads();
         load_halo(chunk + 1 < chunk_hi ? chunk + 1 : chunk);    // lands while the MFMAs below run (the last: once more, unused)
         if (PIXB && TP == 1 && pix_bias && chunk + 1 == chunk_hi) bias_request(bvs[0], 0, 0);   // (more tasks per thread leave no registers for it)
-        // two fragment sets: the reads of tap t + 1 are issued before the MFMAs of tap t
+        // two fragment sets: the reads of tap t + 1 are issued before the MFMAs of tap t. A step's CPB planes and slabs
+        // follow each other as one run of CPB * taps positions (plane, kernel row, kernel column).
         half8_t wf_[2][NO], pf_[2][2];
-        auto fragments = [&](const int tap, const int r, const int sx, const int set) {
+        auto fragments = [&](const int pl, const int tap, const int r, const int sx, const int set) {
+            const int w_at = (CPB > 1 ? pl * p.slab_bytes : 0) + tap * 32;
+            const char* hp = lds_h + (CPB > 1 ? pl * p.halo_plane : 0);
 #pragma unroll
-            for (int i = 0; i < NO; i++) wf_[set][i] = *reinterpret_cast<const half8_t*>(wrow[i] + tap * 32);
+            for (int i = 0; i < NO; i++) wf_[set][i] = *reinterpret_cast<const half8_t*>(wrow[i] + w_at);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const int col = pcol[j] + sx;
-                pf_[set][j] = *reinterpret_cast<const half8_t*>(lds_h + ((prow[j] + r) * p.pw + col) * 32 + ((lh ^ ((col >> 3) & 1)) << 4));
+                pf_[set][j] = *reinterpret_cast<const half8_t*>(hp + ((prow[j] + r) * p.pw + col) * 32 + ((lh ^ ((col >> 3) & 1)) << 4));
             }
         };
-        int r = 0, sx = 0;
-        fragments(0, 0, 0, 0);
-        for (int tap = 0; tap < taps; tap += 2) {
-            {
-                int r1 = r, s1 = sx + 1;
-                if (s1 == p.Kw) { s1 = 0; r1++; }
-                if (tap + 1 < taps) fragments(tap + 1, r1, s1, 1);
-#pragma unroll
-                for (int i = 0; i < NO; i++)
-#pragma unroll
-                    for (int j = 0; j < 2; j++)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[0][i], pf_[0][j], acc[i][j], 0, 0, 0);
-                r = r1; sx = s1;
+        int pl = 0, tp_ = 0, r = 0, sx = 0;                      // the position whose fragments were requested last
+        auto next_position = [&]() {
+            tp_++;
+            if (++sx == p.Kw) { sx = 0; r++; }
+            if (tp_ == taps) { tp_ = 0; r = 0; sx = 0; pl++; }
+        };
+        const int positions = CPB * taps;
+        fragments(0, 0, 0, 0, 0);
+        for (int pos = 0; pos < positions; pos += 2) {
+            if (pos + 1 < positions) {
+                next_position();
+                fragments(pl, tp_, r, sx, 1);
             }
-            if (tap + 1 < taps) {
-                int r1 = r, s1 = sx + 1;
-                if (s1 == p.Kw) { s1 = 0; r1++; }
-                if (tap + 2 < taps) fragments(tap + 2, r1, s1, 0);
+#pragma unroll
+            for (int i = 0; i < NO; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[0][i], pf_[0][j], acc[i][j], 0, 0, 0);
+            if (pos + 1 < positions) {
+                if (pos + 2 < positions) {
+                    next_position();
+                    fragments(pl, tp_, r, sx, 0);
+                }
 #pragma unroll
                 for (int i = 0; i < NO; i++)
 #pragma unroll
                     for (int j = 0; j < 2; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(wf_[1][i], pf_[1][j], acc[i][j], 0, 0, 0);
-                r = r1; sx = s1;
             }
         }
         __syncthreads();                                        // everyone is done reading this chunk's LDS
@@ -2058,16 +2070,26 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
         }
         if (N * (size_t)chunk_groups > 65535) return NZHIP_E_UNSUPPORTED;
     }
-    const size_t image_bytes = (size_t)n_otiles * n_chunks * slab_bytes, bytes = image_bytes * w_batch;
+    // Two chunks per loop step (the store / barrier / request phases paid half as often) when the contraction is long and
+    // not split, the rows allow 16-byte loads and two slabs and two halo planes fit LDS and a thread's staging share;
+    // the weight image then holds an even number of slabs per channel tile, the last one zero when n_chunks is odd.
+    static const char* cpb_env = getenv("NZHIP_CONV_CPB");           // benchmarking only: 1 keeps one chunk per step
+    const bool vec = W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    const bool two = vec && chunk_groups == 1 && n_chunks >= 4 && !(cpb_env && atoi(cpb_env) == 1) &&
+                     ((size_t)2 * slab_bytes + 1023) / 1024 * 1024 + (size_t)2 * span * pw * 32 <= 160 * 1024 - 512 &&
+                     2 * tasks <= (size_t)CG_THREADS * CG_TP_MAX;
+    const int cpb = two ? 2 : 1;
+    const int img_chunks = (n_chunks + cpb - 1) / cpb * cpb;
+    const size_t image_bytes = (size_t)n_otiles * img_chunks * slab_bytes, bytes = image_bytes * w_batch;
     uint64_t key[PREPARED_KEY_WORDS];
-    conv_image_key(key, 3, (int)K_h, (int)K_w, BN, w_ref, C, O, n_chunks, n_otiles, w_batch);
+    conv_image_key(key, 3, (int)K_h, (int)K_w, BN, w_ref, C, O, img_chunks, n_otiles, w_batch);
     ImageLease lease;
     if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
     _Float16* wimg = static_cast<_Float16*>(lease.ptr);
     if (lease.fill) {
-        dim3 pg((unsigned)((BN * taps * IG_CC + 255) / 256), (unsigned)(w_batch * n_otiles * n_chunks));
+        dim3 pg((unsigned)((BN * taps * IG_CC + 255) / 256), (unsigned)(w_batch * n_otiles * img_chunks));
         hipLaunchKernelGGL(conv_weight_image_gen_kernel, pg, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O, taps, BN, w_pitch / 2,
-                           n_chunks, n_otiles);
+                           img_chunks, n_otiles);
     }
     ConvGenArgs a;
     a.y = y; a.x = x; a.wimg = wimg; a.bias = bias;
@@ -2078,6 +2100,13 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     a.w_pitch = w_pitch; a.slab_bytes = slab_bytes; a.halo_off = halo_off;
     a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
     a.chunk_groups = chunk_groups; a.chunks_per_group = chunks_per_group; a.partial = nullptr;
+    a.img_chunks = img_chunks; a.halo_plane = span * pw * 32;
+    size_t lds_use = lds_need;
+    if (two) {                                                       // the kernel counts steps of two chunks
+        a.n_chunks = img_chunks / 2; a.chunks_per_group = a.n_chunks;
+        a.halo_off = (2 * slab_bytes + 1023) / 1024 * 1024;
+        lds_use = (size_t)a.halo_off + (size_t)2 * a.halo_plane;
+    }
     const size_t per_group = N * O * H_out * W_out;
     float* partial = nullptr;
     if (chunk_groups > 1) {
@@ -2087,20 +2116,27 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
         }
         a.partial = partial;
     }
-    const int tp = (int)((tasks + CG_THREADS - 1) / CG_THREADS);
-    const bool vec = W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
-    auto pick = [&](auto vec_tag, auto pix_tag) {
+    const int tp = (int)((cpb * tasks + CG_THREADS - 1) / CG_THREADS);
+    auto pick = [&](auto vec_tag, auto pix_tag, auto cpb_tag) {
         constexpr bool V = decltype(vec_tag)::value, P = decltype(pix_tag)::value;
-        return BN == 128 ? (tp <= 1 ? conv_igemm_gen_kernel<2, 1, V, P> : tp == 2 ? conv_igemm_gen_kernel<2, 2, V, P> : conv_igemm_gen_kernel<2, 3, V, P>)
-                         : (tp <= 1 ? conv_igemm_gen_kernel<1, 1, V, P> : tp == 2 ? conv_igemm_gen_kernel<1, 2, V, P> : conv_igemm_gen_kernel<1, 3, V, P>);
+        constexpr int B = decltype(cpb_tag)::value;
+        return BN == 128 ? (tp <= 1   ? conv_igemm_gen_kernel<2, 1, V, P, B>
+                            : tp == 2 ? conv_igemm_gen_kernel<2, 2, V, P, B>
+                                      : conv_igemm_gen_kernel<2, 3, V, P, B>)
+                         : (tp <= 1   ? conv_igemm_gen_kernel<1, 1, V, P, B>
+                            : tp == 2 ? conv_igemm_gen_kernel<1, 2, V, P, B>
+                                      : conv_igemm_gen_kernel<1, 3, V, P, B>);
     };
+    using one_t = std::integral_constant<int, 1>;
+    using two_t = std::integral_constant<int, 2>;
     const bool pixb = bias && bias_sp != 0 && chunk_groups == 1;
-    auto kfn = vec ? (pixb ? pick(std::true_type{}, std::true_type{}) : pick(std::true_type{}, std::false_type{}))
-                   : (pixb ? pick(std::false_type{}, std::true_type{}) : pick(std::false_type{}, std::false_type{}));
-    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_need, "hipFuncSetAttribute(conv_igemm_gen)");
+    auto kfn = two   ? (pixb ? pick(std::true_type{}, std::true_type{}, two_t{}) : pick(std::true_type{}, std::false_type{}, two_t{}))
+               : vec ? (pixb ? pick(std::true_type{}, std::true_type{}, one_t{}) : pick(std::true_type{}, std::false_type{}, one_t{}))
+                     : (pixb ? pick(std::false_type{}, std::true_type{}, one_t{}) : pick(std::false_type{}, std::false_type{}, one_t{}));
+    int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(kfn), (int)lds_use, "hipFuncSetAttribute(conv_igemm_gen)");
     if (rc == NZHIP_OK) {
         hipLaunchKernelGGL(kfn, dim3((unsigned)(seg_rows * segs_w), (unsigned)n_otiles, (unsigned)(N * chunk_groups)), dim3(CG_THREADS),
-                           lds_need, s, a);
+                           lds_use, s, a);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_igemm_gen kernel launch");
     }
@@ -2662,7 +2698,7 @@ static ConvRoute conv_forward_route(const float* x, size_t N, size_t C, size_t H
     // patch per workgroup with the whole C x taps contraction inside, and there are too few patches to
     // fill the CUs (8 x 512 x 16 x 16 -> 512: 64 workgroups, 190 us). The column matrix of such a layer is
     // small; its batched GEMM splits the contraction over the idle CUs instead (83 us).
-    bool few_patches = false, sparse_patches = false;
+    bool few_patches = false, sparse_patches = false, long_contraction = false;
     {
         const size_t tw = wide ? 64 : 32, th = 256 / tw, bn = bn128 ? 128 : 64;
         const size_t units = N * ((W_out + tw - 1) / tw) * ((H_out + th - 1) / th) * ((O + bn - 1) / bn);
@@ -2673,10 +2709,14 @@ static ConvRoute conv_forward_route(const float* x, size_t N, size_t C, size_t H
         // kernel splits the channels over workgroups and is faster there (58 against 87 us; 16 x 512 x 16 x 16 -> 512: 75
         // against 193 us), as long as its 256-pixel segments are at least half full (4 x 512 x 8 x 8: 37 against 29 us).
         sparse_patches = !resident && units * 4 < 7 * (size_t)device_cu_count();
+        // Weights beyond LDS and 192 or more input channels: the any-geometry kernel takes two chunks per step there and is
+        // 3-8 % faster than one patch per workgroup (16 x 512 x 28 x 28 -> 512: 118 against 128 us; 16 x 192 x 64 x 64 -> 192:
+        // 82 against 87; with 128 channels the two are level or the other way round)
+        long_contraction = !resident && C >= 192 && K_h == 3 && K_w == 3 && W % 4 == 0;
     }
     // any other kernel extent or stride, when the segments (times the channel groups the contraction can be split into)
     // occupy at least a quarter of the CUs
-    if ((!fixed_ok || force_gen || sparse_patches) && conv_igemm_gen_applicable(x, C, H, W, O, K_h, K_w, stride, pad, N) &&
+    if ((!fixed_ok || force_gen || sparse_patches || long_contraction) && conv_igemm_gen_applicable(x, C, H, W, O, K_h, K_w, stride, pad, N) &&
         (w_batch == 1 || w_batch * ((O + 63) / 64) * ((C + 15) / 16) <= 65535) && conv_igemm_gen_fits(W_out, O, K_h, K_w, stride, pad)) {
         const int sw_log = conv_igemm_gen_sw_log(W_out, O, K_h, K_w, stride, pad);     // (not 0: it fits)
         const size_t sw = (size_t)1 << sw_log, sr = CG_PX / sw;

@@ -157,6 +157,13 @@ CONV_ANY_GEOMETRY = [  # N, C, H, W, O, k_h, k_w, stride, pad, w_batch, per-pixe
     (8, 3, 96, 96, 20, 7, 7, 2, 3, 1, False),       # 7x7 stride 2: the slab of 49 taps beside a 13-row halo
     (6, 3, 50, 224, 64, 7, 7, 2, 3, 1, False),      # ... on 112 output columns: 128-wide segments do not fit, 4 x 64 pixels do
     (16, 5, 30, 30, 9, 3, 3, 1, 1, 16, False),      # rows that are not whole 16-byte pieces, per-sample weights
+    # two chunks per loop step (at least four chunks, contraction not split, rows of whole 16-byte pieces): both channel
+    # tiles with one, two and three staging tasks per thread, with and without the per-pixel bias, an odd number of
+    # chunks (the step's second slab is zero) and a 3x3 stride-1 layer with 192 channels, which takes this kernel
+    (256, 64, 16, 16, 48, 5, 5, 1, 2, 1, False), (256, 80, 16, 16, 48, 5, 5, 1, 2, 1, True),
+    (16, 192, 32, 128, 40, 3, 3, 1, 1, 1, True), (128, 64, 32, 64, 24, 3, 3, 2, 1, 1, False),
+    (256, 192, 16, 16, 70, 3, 3, 1, 1, 1, False), (256, 200, 16, 16, 70, 3, 3, 1, 1, 1, True),
+    (16, 192, 32, 128, 130, 3, 3, 1, 1, 1, False), (128, 72, 32, 64, 70, 3, 3, 2, 1, 1, True),
     # the per-pixel bias on the 128-channel tile and with two and three staging tasks per thread
     (64, 8, 32, 32, 65, 5, 5, 1, 2, 1, True),
     (256, 8, 32, 32, 70, 3, 3, 2, 1, 1, True),
