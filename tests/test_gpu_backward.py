@@ -518,3 +518,56 @@ def test_conv2d_backward_weights_rejects_what_it_does_not_cover(nz):
     with pytest.raises(NzHipError) as e:      # a kernel larger than the padded input
         nz.conv2d_backward_weights(dev(np.zeros((1, 1, 50, 3))), dev(np.zeros((1, 2, 2, 2))), dev(np.zeros((1, 3, 1, 1))), 5, 5, 1, 0)
     assert e.value.status == -2
+
+
+def _random_conv_geometries(count, seed, many_images=False):
+    """Seeded geometries across every conv route: few and many channels, 1x1 to 7x7 kernels (also rectangular),
+    strides 1..4, paddings up to the kernel's reach and one beyond, shared and per-sample weights. many_images: enough
+    images that the implicit-GEMM kernels have a workgroup for every compute unit (instead of the few-patch routes)."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        N = int(rng.integers(24, 97)) if many_images else int(rng.integers(1, 7))
+        C = int(rng.choice([1, 2, 3, 5, 8, 16, 24, 40, 70, 130, 200]))
+        O = int(rng.choice([1, 2, 3, 5, 17, 64, 70, 130]))
+        Kh, Kw = int(rng.integers(1, 8)), int(rng.integers(1, 8))
+        if rng.random() < 0.6:
+            Kw = Kh
+        stride = int(rng.choice([1, 1, 1, 2, 2, 3, 4]))
+        pad = int(rng.integers(0, max(Kh, Kw) + 1))
+        H, W = int(rng.integers(Kh, 41)), int(rng.choice([8, 12, 16, 20, 28, 30, 33, 40, 64, 70]))
+        if W + 2 * pad < Kw or H + 2 * pad < Kh or C * Kh * Kw * O > 300000 or N * C * H * W > 6000000 or N * O * H * W > 12000000:
+            continue
+        wb = N if rng.random() < 0.25 else 1
+        cases.append((N, C, H, W, O, Kh, Kw, stride, pad, wb))
+    return cases
+
+
+@pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", _random_conv_geometries(48, 2024) + _random_conv_geometries(32, 7, many_images=True))
+def test_random_conv_geometries_forward_and_gradients_bit_exact(nz, oracle, N, C, H, W, O, Kh, Kw, stride, pad, wb):
+    """Forward, weight gradient and (where the entry point covers the geometry) data gradient of one seeded random layer
+    on integer-valued data against the oracle; whatever route the shape takes, the sums are exact."""
+    from neuzephyr_amd.capi import NzHipError
+    rng = np.random.default_rng(N + 3 * C + 5 * H + 7 * W + 11 * O + 13 * Kh + 17 * Kw + 19 * stride + 23 * pad)
+    Ho, Wo = (H + 2 * pad - Kh) // stride + 1, (W + 2 * pad - Kw) // stride + 1
+    x = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+    ws = [rng.integers(-2, 3, size=(O, C, Kh, Kw)).astype(np.float32) for _ in range(wb)]
+    w_ref = np.concatenate([oracle.weights_oihw_to_ref(w) for w in ws], axis=0)
+    bias = rng.integers(-2, 3, size=(O,)).astype(np.float32)
+    got = host(nz.conv2d_forward(dev(x), dev(w_ref), dev(bias), Kh, Kw, stride, pad, relu=True))
+    for n in range(N):
+        truth = np.maximum(oracle.conv2d_direct_f64(x[n:n + 1], ws[n if wb > 1 else 0], None, stride, pad) + bias.reshape(1, O, 1, 1), 0)
+        assert np.array_equal(got[n:n + 1].astype(np.float64), truth), ("forward", n)
+    dy = rng.integers(-3, 4, size=(N, O, Ho, Wo)).astype(np.float32)
+    dw0 = rng.integers(-4, 5, size=w_ref.shape).astype(np.float32)
+    want_dw = oracle.conv2d_backward_weights(dw0.copy(), x, dy, Kh, Kw, pad, stride)
+    assert np.array_equal(host(nz.conv2d_backward_weights(dev(dw0), dev(x), dev(dy), Kh, Kw, stride, pad)), want_dw), "weights"
+    dx0 = rng.integers(-3, 4, size=x.shape).astype(np.float32)
+    if Kh == Kw and pad <= Kh - 1:
+        for accumulate in (True, False):
+            want_dx = oracle.conv2d_backward_data(dx0.copy() if accumulate else np.zeros_like(dx0), dy, w_ref, Kh, Kw, pad, stride)
+            got_dx = host(nz.conv2d_backward_data(dev(dx0), dev(dy), dev(w_ref), Kh, Kw, stride, pad, accumulate=accumulate))
+            assert np.array_equal(got_dx, want_dx), ("data", accumulate)
+    else:
+        with pytest.raises(NzHipError):
+            nz.conv2d_backward_data(dev(dx0), dev(dy), dev(w_ref), Kh, Kw, stride, pad)
