@@ -48,6 +48,32 @@ def test_avgpool_forward_and_backward_bit_exact(nz, oracle, shape, pool, stride,
     assert np.array_equal(host(dx), oracle.avgpool2d_backward(base, dy, pool, stride, pad))
 
 
+def _random_pool_cases(count, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    while len(cases) < count:
+        pool, stride = int(rng.integers(1, 8)), int(rng.integers(1, 5))
+        pad = int(rng.integers(0, pool))
+        H, W = int(rng.integers(pool, 60)), int(rng.choice([8, 12, 16, 28, 31, 40, 64, 112, 300]))
+        if W + 2 * pad < pool or H + 2 * pad < pool:
+            continue
+        cases.append(((int(rng.integers(1, 4)), int(rng.integers(1, 5)), H, W), pool, stride, pad))
+    return cases
+
+
+@pytest.mark.parametrize("shape,pool,stride,pad", _random_pool_cases(40, 11))
+def test_avgpool_random_geometries_bit_exact(nz, oracle, shape, pool, stride, pad):
+    rng = np.random.default_rng(sum(shape) * 3 + pool * 5 + stride * 7 + pad)
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    want = oracle.avgpool2d(x, pool, stride, pad)
+    assert np.array_equal(host(nz.avgpool2d(dev(x), pool, stride, pad)), want)
+    dy = rng.uniform(-1, 1, want.shape).astype(np.float32)
+    base = rng.uniform(-1, 1, shape).astype(np.float32)
+    dx = dev(base)
+    nz.avgpool2d_backward(dx, dev(dy), pool, stride, pad)
+    assert np.array_equal(host(dx), oracle.avgpool2d_backward(base, dy, pool, stride, pad))
+
+
 def test_avgpool_rejects_bad_geometry(nz):
     x = dev(np.zeros((1, 1, 4, 4)))
     with pytest.raises(nz.NzHipError):
