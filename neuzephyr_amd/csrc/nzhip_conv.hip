@@ -2922,6 +2922,53 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     }
     if (stride > 1) {
         const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
+        // The convolution of the zero-filled gradient does stride^2 times the multiply-adds; the reference's own chain
+        // (src/Nodes.cu:660-665, 169-182, 632-640: column gradient = dy^T x W^T, then the gather into the image) does them
+        // once but writes and reads the column gradient. Many channels on small images favour the chain (16 x 512 x 14 x 14
+        // <- 512 at stride 2: 103 against 45 us), few channels on large images the convolution (16 x 64 x 128 x 128 <- 128:
+        // 101 against 269). The estimate: both sides at the rates measured for them (flops: resident / streamed weights,
+        // the product of the chain; bytes: the zero-filled gradient, three passes over the column gradient), the
+        // convolution favoured up to 1.5 x because its measured side came out better than estimated on every shape tried.
+        static const char* dx_env = getenv("NZHIP_CONV_DX");              // benchmarking only: "chain" | "conv"
+        const double flops = 2.0 * N * Ho * Wo * C * K_h * K_w * O;
+        const bool resident = ((O + 15) / 16) * (C > 64 ? 128 : 64) * K_h * K_w * 32 <= 148 * 1024;
+        const double hu = (double)(H + 2 * pad - K_h + 1), wu = (double)(W + 2 * pad - K_w + 1);
+        // (the convolution's output channels are the C input channels here, in tiles of 64: with 3 of them it multiplies
+        // mostly padding, 16 x 3 x 224 x 224 <- 64 at 7x7 stride 2: 630 against 208 us)
+        const double tile_fill = (double)((C + 63) / 64 * 64) / (double)C;
+        const double as_conv = stride * stride * flops * tile_fill / (resident ? 600e6 : 300e6) + N * O * hu * wu * 4.0 / 5e6;
+        const double as_chain = flops / 400e6 + 3.0 * N * Ho * Wo * C * K_h * K_w * 4.0 / 4e6;
+        const size_t P = Ho * Wo, CKK = C * K_h * K_w;
+        const bool chain_fits = N * P < 0x3fffffff && CKK < 0x3fffffff && O < 0x3fffffff && N <= 65535 && P * O < 0x7fffffffull;
+        if (chain_fits && (dx_env ? dx_env[1] == 'h' : as_conv >= 1.5 * as_chain)) {
+            float* dyt = nullptr;
+            float* dcol = nullptr;
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&dyt), N * P * O * sizeof(float), s)) return rc;
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&dcol), N * P * CKK * sizeof(float), s)) {
+                workspace_free(dyt, s);
+                return rc;
+            }
+            int rc = nzhip_col2im_backward(dyt, dy, Ho, Wo, O, N, stream);                 // [N][P][O]
+            if (rc == NZHIP_OK) {
+                nzhip_gemm_desc g = {};
+                g.A = dyt; g.K = (int64_t)O; g.lda = (int64_t)O; g.a_layout = NZHIP_LAYOUT_ROW;
+                g.B = w_ref; g.N = (int64_t)CKK; g.ldb = (int64_t)O; g.b_layout = NZHIP_LAYOUT_TRANS;       // w_ref holds CKK x O
+                g.C = dcol; g.ldc = (int64_t)CKK;
+                g.batch_c = 1;
+                if (w_batch > 1) {                                                           // one product per image
+                    g.M = (int64_t)P; g.batch_n = (int64_t)N;
+                    g.a_stride_n = (int64_t)(P * O); g.b_stride_n = (int64_t)(CKK * O); g.c_stride_n = (int64_t)(P * CKK);
+                } else {                                                                     // all images as rows of one product
+                    g.M = (int64_t)(N * P); g.batch_n = 1;
+                }
+                g.activation = NZHIP_ACT_NONE;
+                rc = nzhip_gemm(&g, s);
+            }
+            if (rc == NZHIP_OK && !accumulate) rc = nzhip_fill(dx, 0.f, N * C * H * W, stream);
+            if (rc == NZHIP_OK) rc = nzhip_im2col_backward(dx, dcol, Ho, Wo, C, K_h, K_w, stride, pad, H, W, N, stream);
+            const int rc2 = workspace_free(dcol, s), rc3 = workspace_free(dyt, s);
+            return rc ? rc : (rc2 ? rc2 : rc3);
+        }
         const size_t Hu = H + 2 * pad - K_h + 1, Wu = W + 2 * pad - K_w + 1, total = N * O * Hu * Wu;
         const size_t quads = N * O * Hu * ((Wu + 3) / 4);
         if (Hu > 0x3fffffff || Wu > 0x3fffffff || (quads + 255) / 256 > 0x7fffffffull)

@@ -71,23 +71,6 @@ namespace nz::graph {
         T* as(Node* n, const char* type) {
             return (n && n->type == type) ? dynamic_cast<T*>(n) : nullptr;
         }
-
-        // Data gradient of a strided convolution: as ONE convolution it runs on the output gradient spread out with zeros,
-        // stride^2 times the multiply-adds; the column-matrix chain does the real ones but writes and re-reads a column
-        // gradient of K^2 / stride^2 times the input. Estimates in microseconds from rates measured on the MI355X
-        // (resident-weight convolution 600 TFLOP/s, otherwise 300; chain product 400 TFLOP/s; 4-5 TB/s of traffic); the
-        // estimates are both about half the measured times, and the convolution is favoured up to 1.5x because its
-        // measured side came out better than estimated on every shape tried (16x64x128x128 -> 128, 3x3 stride 2: 101
-        // against 269 us; 16x256x28x28 -> 512: 205 against 93 us, which this rule leaves to the chain).
-        bool stridedDataGradientAsConvolution(size_t N, size_t C, size_t H, size_t W, size_t O, size_t K, size_t stride, size_t pad) {
-            const double Ho = static_cast<double>((H + 2 * pad - K) / stride + 1), Wo = static_cast<double>((W + 2 * pad - K) / stride + 1);
-            const double Hu = static_cast<double>(H + 2 * pad - K + 1), Wu = static_cast<double>(W + 2 * pad - K + 1);
-            const double flops = 2.0 * N * Ho * Wo * C * K * K * O;
-            const bool resident = ((O + 15) / 16) * (C > 64 ? 128 : 64) * K * K * 32 <= 148 * 1024;
-            const double asConvolution = stride * stride * flops / (resident ? 600e6 : 300e6) + N * O * Hu * Wu * 4.0 / 5e6;
-            const double asChain = flops / 400e6 + 3.0 * N * Ho * Wo * C * K * K * 4.0 / 4e6;
-            return asConvolution < 1.5 * asChain;
-        }
     }
 
     // Turns the sorted node list into the list of calls forward() makes. A chain is fused only if
@@ -162,9 +145,7 @@ namespace nz::graph {
                     // to 8; a chain whose input carries no gradient does not need it at all)
                     const bool dataGradientFused =
                         i2c->kernelHeight == i2c->kernelWidth && i2c->padding <= i2c->kernelHeight - 1 && i2c->stride >= 1 &&
-                        i2c->stride <= 8 &&
-                        (i2c->stride == 1 || stridedDataGradientAsConvolution(xs[0], xs[1], xs[2], xs[3], O, i2c->kernelHeight,
-                                                                              i2c->stride, i2c->padding));
+                        i2c->stride <= 8;       // (strided: the call itself chooses between one convolution and the column-gradient chain)
                     {
                         Node* pre = add ? static_cast<Node*>(add) : static_cast<Node*>(mm);   // holds [N,1,HW,O] gradients
                         back = [=] {
