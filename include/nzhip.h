@@ -234,8 +234,10 @@ int nzhip_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, s
  * Img2ColNode::forward wrote (:605-630) and dC the pixel-major gradient from Col2ImgNode::backward (:660-665):
  *   dw[wb][(c,r,s)][o] += sum over h, w (and n, for shared weights) of
  *                         f16(x[n][c][h+r-pad][w+s-pad]) * f16(dy[n][o][h][w])
- * Supported: 3x3, stride 1, pad 1, and 1x1, stride 1, pad 0 (whose column matrix is x itself: one batched product);
- * anything else returns NZHIP_E_UNSUPPORTED and the caller runs the chain. */
+ * Supported: any K_h x K_w of at most 128 taps with stride <= 4 (1x1 is a product on x itself or on its strided
+ * pixels); anything else returns NZHIP_E_UNSUPPORTED and the caller runs the chain. Shared weights on images of fewer
+ * than 64 output pixels run that chain inside the library as ONE product whose contraction is the pixels of all
+ * images (column matrix and transposed gradient in pooled workspaces); same sums either way. */
 int nzhip_conv2d_backward_weights(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H,
                                   size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
                                   size_t w_batch, void* stream);

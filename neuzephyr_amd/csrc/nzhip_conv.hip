@@ -3535,6 +3535,42 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
                                              size_t w_batch, void* stream) {
     if (!dw || !x || !dy) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_weights: null pointer");
     if (w_batch != 1 && w_batch != N) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
+    // Images of fewer than 64 output pixels (7 x 7 outputs of a network's last stage) with shared weights: a product per
+    // image has a contraction of 49, and a 128-pixel segment of the gather kernel is mostly padding. The column matrices
+    // of all images follow each other in memory as ONE [N pixels, C K_h K_w] matrix, so the reference's own chain
+    // (Img2ColNode::forward, then dB += A^T dC of MatMulNode::backward, src/Nodes.cu:605-630, 169-182) becomes one product
+    // with the contraction over all pixels of all images: dw += col^T x dy^T (16 x 512 x 14 x 14 -> 512 at stride 2:
+    // 91 -> 55 us; 16 x 1024 x 14 x 14 -> 2048 1x1 stride 2: 105 -> 56; 16 x 2048 x 7 x 7 -> 512 1x1: 57 -> 40).
+    static const char* dwf_env = getenv("NZHIP_CONV_DW_FOLD");          // benchmarking only: 0 never, 1 wherever it applies
+    if (stride != 0 && K_h != 0 && K_w != 0 && H + 2 * pad >= K_h && W + 2 * pad >= K_w && w_batch == 1 && N != 0 && C != 0 && O != 0) {
+        const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1, P = Ho * Wo, CKK = C * K_h * K_w;
+        const bool fits = N * P < 0x3fffffff && CKK < 0x3fffffff && O < 0x3fffffff && N <= 65535 && N * P * CKK <= ((size_t)1 << 27);
+        const bool wanted = dwf_env ? atoi(dwf_env) != 0 : (P < 64 && N * P >= 256 && CKK >= 256 && O >= 64 && CKK * O >= 65536);
+        if (fits && wanted) {
+            hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+            float* col = nullptr;
+            float* dyt = nullptr;
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&col), N * P * CKK * sizeof(float), s)) return rc;
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&dyt), N * P * O * sizeof(float), s)) {
+                workspace_free(col, s);
+                return rc;
+            }
+            int rc = nzhip_im2col(col, x, Ho, Wo, C, K_h, K_w, stride, pad, H, W, N, stream);
+            if (rc == NZHIP_OK) rc = nzhip_col2im_backward(dyt, dy, Ho, Wo, O, N, stream);          // [N][pixels][O]
+            if (rc == NZHIP_OK) {
+                nzhip_gemm_desc g = {};
+                g.A = col; g.M = (int64_t)CKK; g.K = (int64_t)(N * P); g.lda = (int64_t)CKK; g.a_layout = NZHIP_LAYOUT_TRANS;   // col holds K x M
+                g.B = dyt; g.N = (int64_t)O; g.ldb = (int64_t)O; g.b_layout = NZHIP_LAYOUT_ROW;
+                g.C = dw; g.ldc = (int64_t)O;
+                g.bias = dw; g.bias_stride_row = (int64_t)O; g.bias_stride_col = 1;                    // dw += ...
+                g.batch_n = 1; g.batch_c = 1;
+                g.activation = NZHIP_ACT_NONE;
+                rc = nzhip_gemm(&g, s);
+            }
+            const int rc2 = workspace_free(dyt, s), rc3 = workspace_free(col, s);
+            return rc ? rc : (rc2 ? rc2 : rc3);
+        }
+    }
     if (K_h == 1 && K_w == 1 && stride == 1 && pad == 0 && H > 0 && W > 0 && H * W < 0x3fffffff && C < 0x3fffffff &&
         O < 0x3fffffff && N <= 65535 && N * C * O < 0x7fffffffull) {
         if (N == 0 || C == 0 || O == 0) return NZHIP_OK;

@@ -395,7 +395,11 @@ CONV_GEN_BWD_W = [  # N, C, H, W, O, Kh, Kw, stride, pad, w_batch: every geometr
     # from the kernel built for rows that are multiples of 8 wide
     (40, 256, 8, 8, 16, 3, 3, 2, 1, 1), (40, 256, 8, 8, 16, 3, 3, 1, 0, 1), (3, 40, 28, 28, 24, 3, 3, 1, 1, 1), (20, 200, 14, 14, 20, 3, 3, 1, 1, 1),
     # 1x1 with a stride: the pixels it looks at gathered once, then the 1x1 stride-1 product (shared and per-sample weights)
-    (4, 70, 14, 14, 130, 1, 1, 2, 0, 1), (3, 20, 9, 11, 33, 1, 1, 3, 0, 3)]
+    (4, 70, 14, 14, 130, 1, 1, 2, 0, 1), (3, 20, 9, 11, 33, 1, 1, 3, 0, 3),
+    # shared weights and fewer than 64 output pixels per image: one product over the pixels of all images (3x3 stride 2,
+    # 1x1, 3x3 on 4x4 images, 1x1 stride 2); the last has too few pixels in all and stays with the gather kernel
+    (16, 128, 14, 14, 128, 3, 3, 2, 1, 1), (8, 300, 7, 7, 260, 1, 1, 1, 0, 1), (70, 64, 4, 4, 128, 3, 3, 1, 1, 1),
+    (6, 256, 13, 13, 256, 1, 1, 2, 0, 1), (4, 128, 7, 7, 128, 3, 3, 1, 1, 1)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", CONV_GEN_BWD_W)
