@@ -2630,29 +2630,91 @@ namespace nzhip {
 // dst[plane][ho][wo] = src[plane][ho * stride][wo * stride]. On that smaller image it is the 1x1 stride-1 convolution,
 // forward and both gradients (the reference lowers it like any other: column matrix, product, and for the data
 // gradient a scatter over the windows, src/Nodes.cu:605-640).
-__global__ __launch_bounds__(256) void subsample_kernel(float* __restrict__ dst, const float* __restrict__ src, long total, int H, int W,
-                                                        int Ho, int Wo, int stride) {
-    const long t = (long)blockIdx.x * 256 + threadIdx.x;
-    if (t >= total) return;
-    const int wo = (int)(t % Wo), ho = (int)((t / Wo) % Ho);
-    const long plane = t / ((long)Wo * Ho);
-    dst[t] = src[(plane * H + (long)ho * stride) * W + (long)wo * stride];
-}
-// The way back for the data gradient: dx[plane][h][w] (+)= sub[plane][h / stride][w / stride] where both divide and the
-// pixel was looked at; the other pixels get no gradient (zero when dx is overwritten).
-__global__ __launch_bounds__(256) void scatter_strided_kernel(float* __restrict__ dx, const float* __restrict__ sub, long total, int H, int W,
-                                                              int Ho, int Wo, int stride, int accumulate) {
-    const long t = (long)blockIdx.x * 256 + threadIdx.x;
-    if (t >= total) return;
-    const int w = (int)(t % W), h = (int)((t / W) % H);
-    const long plane = t / ((long)W * H);
-    const int ho = h / stride, wo = w / stride;
-    const bool hit = ho * stride == h && wo * stride == w && ho < Ho && wo < Wo;
-    if (accumulate) {
-        if (hit) dx[t] += sub[(plane * Ho + ho) * Wo + wo];
-    } else {
-        dx[t] = hit ? sub[(plane * Ho + ho) * Wo + wo] : 0.f;
+// A workgroup takes 256 >> wq_log rows of 1 << wq_log threads, a thread four adjacent columns of its row (one 16-byte
+// store when the rows allow it): one division per thread instead of three per element.
+template <bool VEC>
+__global__ __launch_bounds__(256) void subsample_kernel(float* __restrict__ dst, const float* __restrict__ src, long rows, int H, int W,
+                                                        int Ho, int Wo, int stride, int wq_log) {
+    const long row = (long)blockIdx.x * (256 >> wq_log) + (threadIdx.x >> wq_log);      // (plane, ho)
+    if (row >= rows) return;
+    const long plane = rows <= 0x7fffffffl ? (long)((unsigned)row / (unsigned)Ho) : row / Ho;
+    const int ho = (int)(row - plane * Ho);
+    const float* srow = src + (plane * H + (long)ho * stride) * W;
+    float* drow = dst + row * Wo;
+    for (int w0 = (threadIdx.x & ((1 << wq_log) - 1)) * 4; w0 < Wo; w0 += 4 << wq_log) {
+        floatx4 v;
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = srow[(long)min(w0 + j, Wo - 1) * stride];
+        if (VEC) {
+            *reinterpret_cast<floatx4*>(drow + w0) = v;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (w0 + j < Wo) drow[w0 + j] = v[j];
+        }
     }
+}
+// The way back: dst[plane][h][w] (+)= src[plane][h / stride][w / stride] where both divide and the source pixel exists;
+// the other pixels get nothing (zero when dst is overwritten). The data gradient of a strided 1x1 convolution put back
+// between the pixels it never looked at, and the output gradient of any strided convolution spread out to the positions
+// its windows started at. Same thread layout as above; rows that no source row reaches are one store per piece (or
+// nothing at all when accumulating).
+template <bool VEC>
+__global__ __launch_bounds__(256) void spread_strided_kernel(float* __restrict__ dst, const float* __restrict__ src, long rows, int H, int W,
+                                                             int Ho, int Wo, int stride, int accumulate, int wq_log) {
+    const long row = (long)blockIdx.x * (256 >> wq_log) + (threadIdx.x >> wq_log);      // (plane, h)
+    if (row >= rows) return;
+    const long plane = rows <= 0x7fffffffl ? (long)((unsigned)row / (unsigned)H) : row / H;
+    const int h = (int)(row - plane * H);
+    const int ho = h / stride;
+    const bool row_hit = ho * stride == h && ho < Ho;
+    if (accumulate && !row_hit) return;
+    const float* srow = src + (plane * Ho + (row_hit ? ho : 0)) * Wo;
+    float* drow = dst + row * W;
+    for (int w0 = (threadIdx.x & ((1 << wq_log) - 1)) * 4; w0 < W; w0 += 4 << wq_log) {
+        int wo = (w0 + stride - 1) / stride;          // the first source column at or right of w0
+        int w_next = wo * stride;
+        floatx4 v;
+        bool hits[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            hits[j] = row_hit && w0 + j == w_next && wo < Wo;
+            v[j] = hits[j] ? srow[wo] : 0.f;
+            if (w0 + j == w_next) { w_next += stride; wo++; }
+        }
+        if (VEC) {
+            if (accumulate) {                           // pixels without a source keep their bits
+                const floatx4 old = *reinterpret_cast<const floatx4*>(drow + w0);
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = hits[j] ? old[j] + v[j] : old[j];
+            }
+            *reinterpret_cast<floatx4*>(drow + w0) = v;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (w0 + j < W && (hits[j] || !accumulate)) drow[w0 + j] = accumulate ? drow[w0 + j] + v[j] : v[j];
+        }
+    }
+}
+// log2 of the threads per row: the power of two that covers a row's 4-column pieces, 256 at most
+static int strided_wq_log(size_t W) {
+    int l = 0;
+    while (l < 8 && ((size_t)4 << l) < W) l++;
+    return l;
+}
+static int spread_strided(float* dst, const float* src, size_t planes, size_t H, size_t W, size_t Ho, size_t Wo, size_t stride,
+                          int accumulate, hipStream_t s) {
+    const size_t rows = planes * H;
+    const int wq_log = strided_wq_log(W);
+    const size_t blocks = (rows + (256 >> wq_log) - 1) / (256 >> wq_log);
+    if (H > 0x3fffffff || W > 0x3fffffff || blocks > 0x7fffffffull)
+        return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_data: extents beyond the fused kernels (use the column-matrix chain)");
+    if (rows == 0 || W == 0) return NZHIP_OK;
+    const bool vec = W % 4 == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0;
+    hipLaunchKernelGGL(vec ? spread_strided_kernel<true> : spread_strided_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, dst, src,
+                       (long)rows, (int)H, (int)W, (int)Ho, (int)Wo, (int)stride, accumulate, wq_log);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "spread_strided kernel launch");
 }
 static bool conv1x1_strided(size_t K_h, size_t K_w, size_t stride, size_t pad, size_t N, size_t C, size_t H, size_t W) {
     return K_h == 1 && K_w == 1 && stride > 1 && pad == 0 && H > 0 && W > 0 && H < 0x3fffffff && W < 0x3fffffff &&
@@ -2662,8 +2724,11 @@ static bool conv1x1_strided(size_t K_h, size_t K_w, size_t stride, size_t pad, s
 static int conv_subsample(float** sub, const float* x, size_t planes, size_t H, size_t W, size_t Ho, size_t Wo, size_t stride, hipStream_t s) {
     const size_t total = planes * Ho * Wo;
     if (int rc = workspace_alloc(reinterpret_cast<void**>(sub), total * sizeof(float), s)) return rc;
-    hipLaunchKernelGGL(subsample_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, *sub, x, (long)total, (int)H, (int)W, (int)Ho,
-                       (int)Wo, (int)stride);
+    const size_t rows = planes * Ho;
+    const int wq_log = strided_wq_log(Wo);
+    const bool vec = Wo % 4 == 0;                       // pooled workspaces are 256-byte aligned
+    hipLaunchKernelGGL(vec ? subsample_kernel<true> : subsample_kernel<false>, dim3((unsigned)((rows + (256 >> wq_log) - 1) / (256 >> wq_log))),
+                       dim3(256), 0, s, *sub, x, (long)rows, (int)H, (int)W, (int)Ho, (int)Wo, (int)stride, wq_log);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         workspace_free(*sub, s);
@@ -2836,39 +2901,6 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
                                bias_stride_channel, 0, activation, stream);
 }
 
-namespace nzhip {
-// dst[plane][h][w] = src[plane][h / stride][w / stride] where both divide and the source pixel exists, else 0: the output
-// gradient of a strided convolution spread out to the positions its windows started at (H_up = H + 2 pad - K + 1 rows).
-// A thread writes four adjacent columns of one row (VEC: as one 16-byte store; Wu a multiple of 4, aligned dst).
-template <bool VEC>
-__global__ __launch_bounds__(256) void upsample_zero_kernel(float* __restrict__ dst, const float* __restrict__ src, long quads, int Ho,
-                                                            int Wo, int Hu, int Wu, int stride) {
-    const long t = (long)blockIdx.x * 256 + threadIdx.x;
-    if (t >= quads) return;
-    const int wq = (Wu + 3) >> 2;
-    const int w0 = (int)(t % wq) * 4, h = (int)((t / wq) % Hu);
-    const long plane = t / ((long)wq * Hu);
-    const int ho = h / stride;
-    const bool row_hit = ho * stride == h && ho < Ho;
-    const float* srow = src + (plane * Ho + (row_hit ? ho : 0)) * Wo;
-    floatx4 v;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int w = w0 + j, wo = w / stride;
-        const bool hit = row_hit && wo * stride == w && wo < Wo;
-        v[j] = hit ? srow[wo] : 0.f;
-    }
-    float* drow = dst + (plane * Hu + h) * Wu + w0;
-    if (VEC) {
-        *reinterpret_cast<floatx4*>(drow) = v;
-    } else {
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            if (w0 + j < Wu) drow[j] = v[j];
-    }
-}
-}  // namespace nzhip
-
 /* Gradient of nzhip_conv2d_forward with respect to x: one convolution of dy with the
  * mirrored weights instead of the reference's chain Col2ImgNode::backward -> MatMulNode::backward
  * (dA += dC * B^T) -> Img2ColNode::backward (src/Nodes.cu:660-665, 169-182, 632-640), which writes and
@@ -2892,16 +2924,11 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
         // 1x1 with a stride: the gradient of the pixels the convolution looked at, as a 1x1 stride-1 problem on the
         // smaller image, then put back between pixels that get none (16 x 512 x 28 x 28 <- 1024 at stride 2: 62 -> 45 us;
         // with fewer than 64 pixels left per image the per-image products are too small: 16 x 1024 x 14 x 14 <- 2048: 66 -> 86)
-        const size_t Ho = (H - 1) / stride + 1, Wo = (W - 1) / stride + 1, total = N * C * H * W;
+        const size_t Ho = (H - 1) / stride + 1, Wo = (W - 1) / stride + 1;
         float* sub = nullptr;
         if (int rc = workspace_alloc(reinterpret_cast<void**>(&sub), N * C * Ho * Wo * sizeof(float), s)) return rc;
         int rc = nzhip_conv2d_backward_data(sub, dy, w_ref, N, C, Ho, Wo, O, 1, 1, 1, 0, w_batch, 0, stream);
-        if (rc == NZHIP_OK) {
-            hipLaunchKernelGGL(scatter_strided_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, dx, sub, (long)total, (int)H, (int)W,
-                               (int)Ho, (int)Wo, (int)stride, accumulate ? 1 : 0);
-            hipError_t e = hipGetLastError();
-            if (e != hipSuccess) rc = set_hip_error(e, "scatter_strided kernel launch");
-        }
+        if (rc == NZHIP_OK) rc = spread_strided(dx, sub, N * C, H, W, Ho, Wo, stride, accumulate ? 1 : 0, s);
         const int rc2 = workspace_free(sub, s);
         return rc ? rc : rc2;
     }
@@ -2970,15 +2997,11 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
             return rc ? rc : (rc2 ? rc2 : rc3);
         }
         const size_t Hu = H + 2 * pad - K_h + 1, Wu = W + 2 * pad - K_w + 1, total = N * O * Hu * Wu;
-        const size_t quads = N * O * Hu * ((Wu + 3) / 4);
-        if (Hu > 0x3fffffff || Wu > 0x3fffffff || (quads + 255) / 256 > 0x7fffffffull)
+        if (Hu > 0x3fffffff || Wu > 0x3fffffff)
             return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_data: extents beyond the fused kernels (use the column-matrix chain)");
         float* up = nullptr;
         if (int rc = workspace_alloc(reinterpret_cast<void**>(&up), total * sizeof(float), s)) return rc;
-        hipLaunchKernelGGL(Wu % 4 == 0 ? upsample_zero_kernel<true> : upsample_zero_kernel<false>, dim3((unsigned)((quads + 255) / 256)),
-                           dim3(256), 0, s, up, dy, (long)quads, (int)Ho, (int)Wo, (int)Hu, (int)Wu, (int)stride);
-        hipError_t e = hipGetLastError();
-        int rc = e == hipSuccess ? NZHIP_OK : set_hip_error(e, "upsample_zero kernel launch");
+        int rc = spread_strided(up, dy, N * O, Hu, Wu, Ho, Wo, stride, 0, s);
         if (rc == NZHIP_OK) rc = nzhip_conv2d_backward_data(dx, up, w_ref, N, C, H, W, O, K_h, K_w, 1, pad, w_batch, accumulate, stream);
         const int rc2 = workspace_free(up, s);
         return rc ? rc : rc2;
