@@ -479,21 +479,45 @@ struct IgemmGeom {
     static constexpr int PASSES = (UNITS + 255) / 256;
 };
 
+// Where the weight of (input channel c, tap, output channel o) of the convolution a kernel runs lies in w_ref.
+// mirror == 0: w_ref is that convolution's own parameter, [(c, tap)][o]. mirror != 0: the kernel runs the data gradient
+// of a convolution whose parameter w_ref is ([(c_f, tap_f)][o_f] with C output and O input channels in the kernel's
+// terms): its weights are w'[(o_f, tap)][c_f] = w[(c_f, taps - 1 - tap)][o_f], read in place, so that no mirrored
+// copy has to be written first.
+__device__ __forceinline__ long weight_source_index(int c, int tap, int o, int C, int O, int taps, int mirror) {
+    return mirror ? ((long)o * taps + (taps - 1 - tap)) * C + c : ((long)c * taps + tap) * O + o;
+}
+// Element t of a [BN rows][taps][16 channels] slab, enumerated with the source's contiguous index fastest (o for a
+// convolution's own parameter, the channel within the chunk for a mirrored one). False past the slab's end.
+template <int BN>
+__device__ __forceinline__ bool weight_image_element(int t, int taps, int mirror, int& o_l, int& cc, int& tap) {
+    if (mirror) {
+        cc = t % IG_CC;
+        o_l = (t / IG_CC) % BN;
+        tap = t / (IG_CC * BN);
+        return tap < taps;
+    }
+    o_l = t % BN;
+    const int rest = t / BN;
+    cc = rest % IG_CC;
+    tap = rest / IG_CC;
+    return rest < taps * IG_CC;
+}
+
 // Pre-pass: w_ref [wb][C*TAPS][O] fp32  ->  fp16 slabs [wb][o_tile][chunk][BN][W_PITCH/2].
 template <int KH, int KW, int BN>
 __global__ __launch_bounds__(256) void conv_weight_image_kernel(_Float16* __restrict__ dst,
                                                                 const float* __restrict__ w_ref, int C, int O,
-                                                                int n_chunks, int n_otiles) {
+                                                                int n_chunks, int n_otiles, int mirror) {
     using G = IgemmGeom<KH, KW, 32, BN>;
     const int slab = blockIdx.y;                               // (wb * n_otiles + o_tile) * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = (slab / n_chunks) % n_otiles, wb = slab / (n_chunks * n_otiles);
-    const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, o fastest
-    const int o_l = t % BN, rest = t / BN;
-    if (rest >= G::TAPS * IG_CC) return;
-    const int cc = rest % IG_CC, tap = rest / IG_CC;
+    const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, the source's contiguous index fastest
+    int o_l, cc, tap;
+    if (!weight_image_element<BN>(t, G::TAPS, mirror, o_l, cc, tap)) return;
     const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
     float v = 0.f;
-    if (c < C && o < O) v = w_ref[((long)wb * C * G::TAPS + (long)c * G::TAPS + tap) * O + o];
+    if (c < C && o < O) v = w_ref[(long)wb * C * G::TAPS * O + weight_source_index(c, tap, o, C, O, G::TAPS, mirror)];
     dst[(long)slab * (G::W_BYTES / 2) + o_l * (G::W_PITCH / 2) + tap * IG_CC + cc] = (_Float16)v;
 }
 
@@ -748,7 +772,7 @@ __global__ __launch_bounds__(256, (BN == 64 ? 3 : 2)) void conv_igemm_kernel(con
 template <int KH, int KW, int BN>
 __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float16* __restrict__ dst,
                                                                          const float* __restrict__ w_ref, int C,
-                                                                         int O, int n_chunks, int n_otiles) {
+                                                                         int O, int n_chunks, int n_otiles, int mirror) {
     constexpr int TAPS = KH * KW;
     // blockIdx.z: weight copy (one per sample for the reference's Conv2d parameter); images follow each other
     w_ref += (long)blockIdx.z * C * TAPS * O;
@@ -756,12 +780,11 @@ __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float1
     const int slab = blockIdx.y;                               // o_tile * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = slab / n_chunks;
     const int t = blockIdx.x * 256 + threadIdx.x;
-    const int o_l = t % BN, rest = t / BN;
-    if (rest >= TAPS * IG_CC) return;
-    const int cc = rest % IG_CC, tap = rest / IG_CC;
+    int o_l, cc, tap;
+    if (!weight_image_element<BN>(t, TAPS, mirror, o_l, cc, tap)) return;
     const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
     float v = 0.f;
-    if (c < C && o < O) v = w_ref[((long)c * TAPS + tap) * O + o];
+    if (c < C && o < O) v = w_ref[weight_source_index(c, tap, o, C, O, TAPS, mirror)];
     const int half = (cc >> 3) ^ ((o_l >> 3) & 1);
     dst[(long)slab * (BN * TAPS * IG_CC) + o_l * (TAPS * IG_CC) + tap * IG_CC + half * 8 + (cc & 7)] = (_Float16)v;
 }
@@ -1131,9 +1154,10 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
 // Image of one channel tile: [chunk][BN rows][256 B] for taps 0..7, then [chunk][BN rows][32 B] for tap 8.
 template <int BN>
 __global__ __launch_bounds__(256) void conv_weight_image_db_kernel(_Float16* __restrict__ dst, const float* __restrict__ w_ref,
-                                                                   int C, int O, int n_chunks, int n_otiles) {
+                                                                   int C, int O, int n_chunks, int n_otiles, int mirror) {
     // One thread per (row, tap) of a slab: 16 reads that are contiguous across the threads of a wave (adjacent
-    // output channels) and two 16-byte stores, instead of one 2-byte store per element.
+    // output channels; with mirrored weights the 16 reads of a thread are the contiguous ones) and two 16-byte
+    // stores, instead of one 2-byte store per element.
     // blockIdx.z: weight copy (one per sample for the reference's Conv2d parameter); images follow each other
     w_ref += (long)blockIdx.z * C * 9 * O;
     dst += (long)blockIdx.z * n_otiles * n_chunks * BN * 144;
@@ -1148,7 +1172,7 @@ __global__ __launch_bounds__(256) void conv_weight_image_db_kernel(_Float16* __r
     for (int cc = 0; cc < IG_CC; cc++) {
         const int c = chunk * IG_CC + cc;
         const bool ok = c < C && o < O;
-        const float v = w_ref[ok ? ((long)c * 9 + tap) * O + o : 0];
+        const float v = w_ref[ok ? weight_source_index(c, tap, o, C, O, 9, mirror) : 0];
         h[cc >> 3][cc & 7] = ok ? (_Float16)v : (_Float16)0.f;
     }
     _Float16* tile = dst + (long)o_tile * n_chunks * BN * 144;   // 288 bytes per (chunk, row)
@@ -1496,9 +1520,9 @@ static int resident_grid_per_sample(size_t N, int n_otiles) {
 
 // Key of a weight image: everything the conversion kernel's output depends on (image kind, tile shape, source and extents).
 static void conv_image_key(uint64_t (&key)[PREPARED_KEY_WORDS], int kind, int kh, int kw, int bn, const float* w_ref, size_t C,
-                           size_t O, int n_chunks, int n_otiles, size_t w_batch) {
+                           size_t O, int n_chunks, int n_otiles, size_t w_batch, bool w_mirror) {
     for (auto& k : key) k = 0;
-    key[0] = (uint64_t)kind | ((uint64_t)kh << 8) | ((uint64_t)kw << 16) | ((uint64_t)bn << 24);
+    key[0] = (uint64_t)kind | ((uint64_t)kh << 8) | ((uint64_t)kw << 16) | ((uint64_t)bn << 24) | ((uint64_t)(w_mirror ? 1 : 0) << 40);
     key[1] = reinterpret_cast<uintptr_t>(w_ref);
     key[2] = C; key[3] = O; key[4] = (uint64_t)n_chunks; key[5] = (uint64_t)n_otiles; key[6] = w_batch;
 }
@@ -1506,7 +1530,7 @@ static void conv_image_key(uint64_t (&key)[PREPARED_KEY_WORDS], int kind, int kh
 template <int KH, int KW, int TW, int BN>
 static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
                              size_t H, size_t W, size_t O, size_t pad, size_t w_batch, int64_t bias_sp,
-                             int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out, hipStream_t s) {
+                             int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out, bool w_mirror, hipStream_t s) {
     using G = IgemmGeom<KH, KW, TW, BN>;
     const int n_chunks = (int)((C + IG_CC - 1) / IG_CC), n_otiles = (int)((O + BN - 1) / BN);
     if (n_otiles > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: too many output channels");
@@ -1527,13 +1551,13 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                 static_assert(lds_need <= 160 * 1024 - 512, "LDS budget");
                 const size_t image_bytes = (size_t)n_otiles * NCH * BN * 288, bytes = image_bytes * w_batch;
                 uint64_t key[PREPARED_KEY_WORDS];
-                conv_image_key(key, 1, 3, 3, BN, w_ref, C, O, NCH, n_otiles, w_batch);
+                conv_image_key(key, 1, 3, 3, BN, w_ref, C, O, NCH, n_otiles, w_batch, w_mirror);
                 ImageLease lease;
                 if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
                 _Float16* wres = static_cast<_Float16*>(lease.ptr);
                 dim3 pg((unsigned)((BN * 9 + 255) / 256), (unsigned)(n_otiles * NCH), (unsigned)w_batch);
                 if (lease.fill)
-                    hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles);
+                    hipLaunchKernelGGL((conv_weight_image_db_kernel<BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C, (int)O, NCH, n_otiles, w_mirror ? 1 : 0);
                 IgemmArgs a;
                 a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
                 a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.H_out = (int)H_out; a.W_out = (int)W_out;
@@ -1580,14 +1604,14 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         if (allow && (w_batch == 1 || grid_ps > 0) && lds_need <= 160 * 1024 - 512) {
             const size_t image_bytes = (size_t)n_otiles * n_chunks * W_CHUNK_R, bytes = image_bytes * w_batch;
             uint64_t key[PREPARED_KEY_WORDS];
-            conv_image_key(key, 2, KH, KW, BN, w_ref, C, O, n_chunks, n_otiles, w_batch);
+            conv_image_key(key, 2, KH, KW, BN, w_ref, C, O, n_chunks, n_otiles, w_batch, w_mirror);
             ImageLease lease;
             if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
             _Float16* wres = static_cast<_Float16*>(lease.ptr);
             dim3 pg((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)(n_otiles * n_chunks), (unsigned)w_batch);
             if (lease.fill)
                 hipLaunchKernelGGL((conv_weight_image_resident_kernel<KH, KW, BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C,
-                                   (int)O, n_chunks, n_otiles);
+                                   (int)O, n_chunks, n_otiles, w_mirror ? 1 : 0);
             IgemmArgs a;
             a.y = y; a.x = x; a.wimg = wres; a.bias = bias;
             a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.H_out = (int)H_out; a.W_out = (int)W_out;
@@ -1626,7 +1650,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     const size_t slabs = (size_t)w_batch * n_otiles * n_chunks;
     if (slabs > 65535) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_forward: weight set too large for the fused route");
     uint64_t key[PREPARED_KEY_WORDS];
-    conv_image_key(key, 3, KH, KW, BN, w_ref, C, O, n_chunks, n_otiles, w_batch);
+    conv_image_key(key, 3, KH, KW, BN, w_ref, C, O, n_chunks, n_otiles, w_batch, w_mirror);
     ImageLease lease;
     if (int rc = image_acquire(PREPARED_CONV_W, key, slabs * G::W_BYTES, s, &lease)) return rc;
     _Float16* wimg = static_cast<_Float16*>(lease.ptr);
@@ -1635,7 +1659,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
         // pad bytes of the slabs are never read as data; no need to clear them
         dim3 grid((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)slabs);
         hipLaunchKernelGGL((conv_weight_image_kernel<KH, KW, BN>), grid, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O,
-                           n_chunks, n_otiles);
+                           n_chunks, n_otiles, w_mirror ? 1 : 0);
     }
     if (rc == NZHIP_OK) {
         IgemmArgs a;
@@ -1708,16 +1732,15 @@ struct ConvGenArgs {
 // Pre-pass: w_ref [wb][C * taps][O] fp32 -> fp16 slabs [wb][o tile][chunk][BN][taps * 16 + 8]
 __global__ __launch_bounds__(256) void conv_weight_image_gen_kernel(_Float16* __restrict__ dst, const float* __restrict__ w_ref, int C,
                                                                     int O, int taps, int BN, int w_pitch_halfs, int n_chunks,
-                                                                    int n_otiles) {
+                                                                    int n_otiles, int mirror) {
     const int slab = blockIdx.y;                               // (wb * n_otiles + o_tile) * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = (slab / n_chunks) % n_otiles, wb = slab / (n_chunks * n_otiles);
-    const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, o fastest
-    const int o_l = t % BN, rest = t / BN;
-    if (rest >= taps * IG_CC) return;
-    const int cc = rest % IG_CC, tap = rest / IG_CC;
+    const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, the source's contiguous index fastest
+    int o_l, cc, tap;
+    if (BN == 128 ? !weight_image_element<128>(t, taps, mirror, o_l, cc, tap) : !weight_image_element<64>(t, taps, mirror, o_l, cc, tap)) return;
     const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
     float v = 0.f;
-    if (c < C && o < O) v = w_ref[((long)wb * C * taps + (long)c * taps + tap) * O + o];
+    if (c < C && o < O) v = w_ref[(long)wb * C * taps * O + weight_source_index(c, tap, o, C, O, taps, mirror)];
     dst[(long)slab * BN * w_pitch_halfs + (long)o_l * w_pitch_halfs + tap * IG_CC + cc] = (_Float16)v;
 }
 
@@ -2035,7 +2058,7 @@ static bool conv_igemm_gen_fits(size_t W_out, size_t O, size_t K_h, size_t K_w, 
 static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C, size_t H,
                                  size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t w_batch,
                                  int64_t bias_sp, int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out,
-                                 hipStream_t s) {
+                                 bool w_mirror, hipStream_t s) {
     const int taps = (int)(K_h * K_w);
     const int sw_log = conv_igemm_gen_sw_log(W_out, O, K_h, K_w, stride, pad);
     if (sw_log == 0) return NZHIP_E_UNSUPPORTED;
@@ -2082,14 +2105,14 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     const int img_chunks = (n_chunks + cpb - 1) / cpb * cpb;
     const size_t image_bytes = (size_t)n_otiles * img_chunks * slab_bytes, bytes = image_bytes * w_batch;
     uint64_t key[PREPARED_KEY_WORDS];
-    conv_image_key(key, 3, (int)K_h, (int)K_w, BN, w_ref, C, O, img_chunks, n_otiles, w_batch);
+    conv_image_key(key, 3, (int)K_h, (int)K_w, BN, w_ref, C, O, img_chunks, n_otiles, w_batch, w_mirror);
     ImageLease lease;
     if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
     _Float16* wimg = static_cast<_Float16*>(lease.ptr);
     if (lease.fill) {
         dim3 pg((unsigned)((BN * taps * IG_CC + 255) / 256), (unsigned)(w_batch * n_otiles * img_chunks));
         hipLaunchKernelGGL(conv_weight_image_gen_kernel, pg, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O, taps, BN, w_pitch / 2,
-                           img_chunks, n_otiles);
+                           img_chunks, n_otiles, w_mirror ? 1 : 0);
     }
     ConvGenArgs a;
     a.y = y; a.x = x; a.wimg = wimg; a.bias = bias;
@@ -2796,10 +2819,37 @@ static ConvRoute conv_forward_route(const float* x, size_t N, size_t C, size_t H
     return fixed_ok && !few_patches ? CONV_ROUTE_FIXED : CONV_ROUTE_WORKSPACE;
 }
 
+// w_mirror: w_ref is the parameter of the convolution whose DATA GRADIENT this call computes ([(c_f, tap)][o_f] with
+// c_f running over this call's O channels and o_f over its C), to be used with channels swapped and taps mirrored.
+// The implicit-GEMM routes read it that way while they build their fp16 weight image; the routes that take the
+// weights as they lie (column matrix, direct kernels) get a mirrored copy first.
 static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
                                size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
                                size_t w_batch, int64_t bias_stride_pixel, int64_t bias_stride_channel,
-                               int64_t bias_stride_image, int activation, void* stream) {
+                               int64_t bias_stride_image, int activation, void* stream, bool w_mirror = false);
+static int conv2d_forward_mirrored_copy(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
+                                        size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                                        size_t w_batch, int64_t bias_stride_pixel, int64_t bias_stride_channel,
+                                        int64_t bias_stride_image, int activation, void* stream) {
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const size_t w_elems = w_batch * C * K_h * K_w * O;
+    float* wflip = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&wflip), w_elems * sizeof(float), s)) return rc;
+    // the copy is this call's own parameter: [(c, tap)][o] with c over this call's C input channels
+    hipLaunchKernelGGL(conv_weight_flip_kernel, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, s, wflip, w_ref, (int)O, (int)C,
+                       (int)K_h, (int)K_w, (long)w_elems);
+    hipError_t e = hipGetLastError();
+    int rc = e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv_weight_flip kernel launch");
+    if (rc == NZHIP_OK)
+        rc = conv2d_forward_impl(y, x, wflip, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
+                                 bias_stride_channel, bias_stride_image, activation, stream, false);
+    const int rc2 = workspace_free(wflip, s);
+    return rc ? rc : rc2;
+}
+static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C,
+                               size_t H, size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
+                               size_t w_batch, int64_t bias_stride_pixel, int64_t bias_stride_channel,
+                               int64_t bias_stride_image, int activation, void* stream, bool w_mirror) {
     if (!y || !x || !w_ref) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_forward: null pointer");
     if (stride == 0 || K_h == 0 || K_w == 0) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_forward: zero stride or kernel extent");
     if (w_batch != 1 && w_batch != N) return set_error(NZHIP_E_SHAPE, "Shapes are not broadcast compatible.");
@@ -2810,6 +2860,9 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
     const size_t H_out = (H + 2 * pad - K_h) / stride + 1, W_out = (W + 2 * pad - K_w) / stride + 1;   // Nodes.cu:605-617
     if (N == 0 || O == 0 || C == 0) return NZHIP_OK;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (w_mirror && (K_h != K_w || (K_h == 1 && K_w == 1)))     // mirrored taps as one reversed index need a square kernel; 1x1 routes take the weights as they lie
+        return conv2d_forward_mirrored_copy(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
+                                            bias_stride_channel, bias_stride_image, activation, stream);
     if (conv1x1_strided(K_h, K_w, stride, pad, N, C, H, W) && H_out * W_out >= 64) {
         // 1x1 with a stride: gather the pixels it looks at, then the 1x1 stride-1 convolution of the smaller image
         // (16 x 512 x 28 x 28 -> 1024 at stride 2: 42 -> 32 us; not with fewer than 64 pixels left per image, where the
@@ -2845,6 +2898,9 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
     const bool fixed_geometry = route == CONV_ROUTE_FIXED, any_geometry = route == CONV_ROUTE_ANY;
     if (bias_stride_image != 0 && !fixed_geometry && !any_geometry)
         return set_error(NZHIP_E_UNSUPPORTED, "conv2d: a per-image bias needs an implicit-GEMM route");
+    if (w_mirror && !fixed_geometry && !any_geometry)
+        return conv2d_forward_mirrored_copy(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
+                                            bias_stride_channel, bias_stride_image, activation, stream);
     if (route == CONV_ROUTE_DIRECT)
         return conv_direct(y, x, w_ref, bias, N, C, H, W, O, w_batch, bias_stride_pixel, bias_stride_channel,
                            activation, s);
@@ -2869,16 +2925,30 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
         };
         if (any_geometry) {
             const int rc = conv_igemm_gen_launch(y, x, w_ref, bias_use, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bsp, bsc,
-                                                 bias_stride_image, activation, H_out, W_out, s);
+                                                 bias_stride_image, activation, H_out, W_out, w_mirror, s);
             const int rc_free = finish(rc == NZHIP_E_UNSUPPORTED ? NZHIP_OK : rc);
             if (rc != NZHIP_E_UNSUPPORTED) return rc_free;
             if (bias_stride_image != 0) return set_error(NZHIP_E_UNSUPPORTED, "conv2d: a per-image bias needs an implicit-GEMM route");
+            if (w_mirror) {                                                                   // the column-matrix route needs the weights as they lie
+                float* wflip = nullptr;
+                const size_t w_elems = w_batch * C * K_h * K_w * O;
+                if (int rc_a = workspace_alloc(reinterpret_cast<void**>(&wflip), w_elems * sizeof(float), s)) return rc_a;
+                hipLaunchKernelGGL(conv_weight_flip_kernel, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, s, wflip, w_ref, (int)O,
+                                   (int)C, (int)K_h, (int)K_w, (long)w_elems);
+                hipError_t e = hipGetLastError();
+                int rc_w = e == hipSuccess ? NZHIP_OK : set_hip_error(e, "conv_weight_flip kernel launch");
+                if (rc_w == NZHIP_OK)
+                    rc_w = conv2d_via_workspace(y, x, wflip, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
+                                                bias_stride_channel, activation, H_out, W_out, s);
+                const int rc_f = workspace_free(wflip, s);
+                return rc_w ? rc_w : rc_f;
+            }
             return conv2d_via_workspace(y, x, w_ref, bias, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, bias_stride_pixel,
                                         bias_stride_channel, activation, H_out, W_out, s);   // the tile does not fit: column matrix
         }
 #define NZHIP_IG(KH_, TW_, BN_)                                                                                      \
     return finish(conv_igemm_launch<KH_, KH_, TW_, BN_>(y, x, w_ref, bias_use, N, C, H, W, O, pad, w_batch, bsp, bsc, \
-                                                        bias_stride_image, activation, H_out, W_out, s))
+                                                        bias_stride_image, activation, H_out, W_out, w_mirror, s))
         if (K_h == 3) {
             if (wide && bn128) NZHIP_IG(3, 64, 128);
             if (wide) NZHIP_IG(3, 64, 64);
@@ -3007,10 +3077,8 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
         return rc ? rc : rc2;
     }
     const size_t H_out = H + 2 * pad - K_h + 1, W_out = W + 2 * pad - K_w + 1;
-    const size_t w_elems = w_batch * C * K_h * K_w * O, x_elems = N * C * H * W;
-    float* wflip = nullptr;
+    const size_t x_elems = N * C * H * W;
     float* tmp = nullptr;
-    if (int rc = workspace_alloc(reinterpret_cast<void**>(&wflip), w_elems * sizeof(float), s)) return rc;
     int rc = NZHIP_OK;
     // "+=": the implicit-GEMM kernels read dx as their bias (same lane reads, then writes each element); the other
     // routes go through a temporary and one add pass
@@ -3019,27 +3087,22 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     const ConvRoute route = conv_forward_route(dy, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t, w_batch, H, W, wide_unused, bn_unused);
     const bool in_place = accumulate && (route == CONV_ROUTE_FIXED || route == CONV_ROUTE_ANY);
     if (accumulate && !in_place) rc = workspace_alloc(reinterpret_cast<void**>(&tmp), x_elems * sizeof(float), s);
-    if (rc == NZHIP_OK) {
-        hipLaunchKernelGGL(conv_weight_flip_kernel, dim3((unsigned)((w_elems + 255) / 256)), dim3(256), 0, s, wflip, w_ref,
-                           (int)C, (int)O, (int)K_h, (int)K_w, (long)w_elems);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) rc = set_hip_error(e, "conv_weight_flip kernel launch");
-    }
+    // the weights go in as they are: the implicit-GEMM routes mirror them while they build their fp16 image, the others
+    // make a mirrored copy themselves
     if (rc == NZHIP_OK && in_place)
-        rc = conv2d_forward_impl(dx, dy, wflip, dx, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t, w_batch, 1, (int64_t)(H * W),
-                                 (int64_t)(C * H * W), NZHIP_ACT_NONE, stream);
+        rc = conv2d_forward_impl(dx, dy, w_ref, dx, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t, w_batch, 1, (int64_t)(H * W),
+                                 (int64_t)(C * H * W), NZHIP_ACT_NONE, stream, true);
     else if (rc == NZHIP_OK)
-        rc = conv2d_forward_impl(accumulate ? tmp : dx, dy, wflip, nullptr, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t,
-                                 w_batch, 0, 0, 0, NZHIP_ACT_NONE, stream);
+        rc = conv2d_forward_impl(accumulate ? tmp : dx, dy, w_ref, nullptr, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t,
+                                 w_batch, 0, 0, 0, NZHIP_ACT_NONE, stream, true);
     if (rc == NZHIP_OK && accumulate && !in_place) {
         hipLaunchKernelGGL(accumulate_kernel, dim3((unsigned)((x_elems / 4 + 256) / 256)), dim3(256), 0, s, dx, tmp,
                            (long)x_elems);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "accumulate kernel launch");
     }
-    int rc2 = tmp ? workspace_free(tmp, s) : NZHIP_OK;
-    int rc3 = workspace_free(wflip, s);
-    return rc ? rc : (rc2 ? rc2 : rc3);
+    const int rc2 = tmp ? workspace_free(tmp, s) : NZHIP_OK;
+    return rc ? rc : rc2;
 }
 
 namespace nzhip {
