@@ -487,21 +487,30 @@ struct IgemmGeom {
 __device__ __forceinline__ long weight_source_index(int c, int tap, int o, int C, int O, int taps, int mirror) {
     return mirror ? ((long)o * taps + (taps - 1 - tap)) * C + c : ((long)c * taps + tap) * O + o;
 }
-// Element t of a [BN rows][taps][16 channels] slab, enumerated with the source's contiguous index fastest (o for a
-// convolution's own parameter, the channel within the chunk for a mirrored one). False past the slab's end.
-template <int BN>
-__device__ __forceinline__ bool weight_image_element(int t, int taps, int mirror, int& o_l, int& cc, int& tap) {
-    if (mirror) {
-        cc = t % IG_CC;
-        o_l = (t / IG_CC) % BN;
-        tap = t / (IG_CC * BN);
-        return tap < taps;
+// The 16 input channels of chunk `chunk` at (tap, output channel o), rounded: h[0] holds channels 0..7, h[1] 8..15
+// (zeros past C or O). The pre-passes below give one thread one (row, tap) of a slab, adjacent threads adjacent output
+// channels: with a convolution's own parameter each of the 16 reads is contiguous across the wave; with a mirrored one
+// the 16 reads of a thread are 64 contiguous bytes (four 16-byte loads when the rows allow it). Either way the thread
+// writes its 32 bytes of the image as two 16-byte stores instead of sixteen 2-byte ones.
+__device__ __forceinline__ void weight_row_tap(half8_t (&h)[2], const float* __restrict__ w, int chunk, int tap, int o, int C, int O,
+                                               int taps, int mirror) {
+    const int c0 = chunk * IG_CC;
+    if (mirror && o < O && c0 + IG_CC <= C && (C & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+        const floatx4* q = reinterpret_cast<const floatx4*>(w + weight_source_index(c0, tap, o, C, O, taps, 1));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const floatx4 v = q[i];
+#pragma unroll
+            for (int j = 0; j < 4; j++) h[i >> 1][(i & 1) * 4 + j] = (_Float16)v[j];
+        }
+        return;
     }
-    o_l = t % BN;
-    const int rest = t / BN;
-    cc = rest % IG_CC;
-    tap = rest / IG_CC;
-    return rest < taps * IG_CC;
+#pragma unroll
+    for (int cc = 0; cc < IG_CC; cc++) {
+        const bool ok = c0 + cc < C && o < O;
+        const float v = w[ok ? weight_source_index(c0 + cc, tap, o, C, O, taps, mirror) : 0];
+        h[cc >> 3][cc & 7] = ok ? (_Float16)v : (_Float16)0.f;
+    }
 }
 
 // Pre-pass: w_ref [wb][C*TAPS][O] fp32  ->  fp16 slabs [wb][o_tile][chunk][BN][W_PITCH/2].
@@ -512,13 +521,14 @@ __global__ __launch_bounds__(256) void conv_weight_image_kernel(_Float16* __rest
     using G = IgemmGeom<KH, KW, 32, BN>;
     const int slab = blockIdx.y;                               // (wb * n_otiles + o_tile) * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = (slab / n_chunks) % n_otiles, wb = slab / (n_chunks * n_otiles);
-    const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, the source's contiguous index fastest
-    int o_l, cc, tap;
-    if (!weight_image_element<BN>(t, G::TAPS, mirror, o_l, cc, tap)) return;
-    const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
-    float v = 0.f;
-    if (c < C && o < O) v = w_ref[(long)wb * C * G::TAPS * O + weight_source_index(c, tap, o, C, O, G::TAPS, mirror)];
-    dst[(long)slab * (G::W_BYTES / 2) + o_l * (G::W_PITCH / 2) + tap * IG_CC + cc] = (_Float16)v;
+    const int t = blockIdx.x * 256 + threadIdx.x;             // (row, tap) within the slab, rows fastest
+    const int o_l = t % BN, tap = t / BN;
+    if (tap >= G::TAPS) return;
+    half8_t h[2];
+    weight_row_tap(h, w_ref + (long)wb * C * G::TAPS * O, chunk, tap, o_tile * BN + o_l, C, O, G::TAPS, mirror);
+    half8_t* q = reinterpret_cast<half8_t*>(dst + (long)slab * (G::W_BYTES / 2) + o_l * (G::W_PITCH / 2) + tap * IG_CC);
+    q[0] = h[0];
+    q[1] = h[1];
 }
 
 struct IgemmArgs {
@@ -779,14 +789,15 @@ __global__ __launch_bounds__(256) void conv_weight_image_resident_kernel(_Float1
     dst += (long)blockIdx.z * n_otiles * n_chunks * (BN * TAPS * IG_CC);
     const int slab = blockIdx.y;                               // o_tile * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = slab / n_chunks;
-    const int t = blockIdx.x * 256 + threadIdx.x;
-    int o_l, cc, tap;
-    if (!weight_image_element<BN>(t, TAPS, mirror, o_l, cc, tap)) return;
-    const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
-    float v = 0.f;
-    if (c < C && o < O) v = w_ref[weight_source_index(c, tap, o, C, O, TAPS, mirror)];
-    const int half = (cc >> 3) ^ ((o_l >> 3) & 1);
-    dst[(long)slab * (BN * TAPS * IG_CC) + o_l * (TAPS * IG_CC) + tap * IG_CC + half * 8 + (cc & 7)] = (_Float16)v;
+    const int t = blockIdx.x * 256 + threadIdx.x;             // (row, tap) within the slab, rows fastest
+    const int o_l = t % BN, tap = t / BN;
+    if (tap >= TAPS) return;
+    half8_t h[2];
+    weight_row_tap(h, w_ref, chunk, tap, o_tile * BN + o_l, C, O, TAPS, mirror);
+    half8_t* q = reinterpret_cast<half8_t*>(dst + (long)slab * (BN * TAPS * IG_CC) + o_l * (TAPS * IG_CC) + tap * IG_CC);
+    const int swap = (o_l >> 3) & 1;
+    q[swap] = h[0];
+    q[swap ^ 1] = h[1];
 }
 
 // PIX_BIAS: the bias varies per pixel (the reference's Bias node after the matmul); otherwise it is
@@ -1168,13 +1179,7 @@ __global__ __launch_bounds__(256) void conv_weight_image_db_kernel(_Float16* __r
     if (tap >= 9) return;
     const int o = o_tile * BN + o_l;
     half8_t h[2];
-#pragma unroll
-    for (int cc = 0; cc < IG_CC; cc++) {
-        const int c = chunk * IG_CC + cc;
-        const bool ok = c < C && o < O;
-        const float v = w_ref[ok ? weight_source_index(c, tap, o, C, O, 9, mirror) : 0];
-        h[cc >> 3][cc & 7] = ok ? (_Float16)v : (_Float16)0.f;
-    }
+    weight_row_tap(h, w_ref, chunk, tap, o, C, O, 9, mirror);
     _Float16* tile = dst + (long)o_tile * n_chunks * BN * 144;   // 288 bytes per (chunk, row)
 #pragma unroll
     for (int half = 0; half < 2; half++) {
@@ -1608,7 +1613,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
             ImageLease lease;
             if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
             _Float16* wres = static_cast<_Float16*>(lease.ptr);
-            dim3 pg((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)(n_otiles * n_chunks), (unsigned)w_batch);
+            dim3 pg((unsigned)((BN * G::TAPS + 255) / 256), (unsigned)(n_otiles * n_chunks), (unsigned)w_batch);
             if (lease.fill)
                 hipLaunchKernelGGL((conv_weight_image_resident_kernel<KH, KW, BN>), pg, dim3(256), 0, s, wres, w_ref, (int)C,
                                    (int)O, n_chunks, n_otiles, w_mirror ? 1 : 0);
@@ -1657,7 +1662,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
     int rc = NZHIP_OK;
     if (lease.fill) {
         // pad bytes of the slabs are never read as data; no need to clear them
-        dim3 grid((unsigned)((BN * G::TAPS * IG_CC + 255) / 256), (unsigned)slabs);
+        dim3 grid((unsigned)((BN * G::TAPS + 255) / 256), (unsigned)slabs);
         hipLaunchKernelGGL((conv_weight_image_kernel<KH, KW, BN>), grid, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O,
                            n_chunks, n_otiles, w_mirror ? 1 : 0);
     }
@@ -1735,13 +1740,14 @@ __global__ __launch_bounds__(256) void conv_weight_image_gen_kernel(_Float16* __
                                                                     int n_otiles, int mirror) {
     const int slab = blockIdx.y;                               // (wb * n_otiles + o_tile) * n_chunks + chunk
     const int chunk = slab % n_chunks, o_tile = (slab / n_chunks) % n_otiles, wb = slab / (n_chunks * n_otiles);
-    const int t = blockIdx.x * 256 + threadIdx.x;             // element within the slab, the source's contiguous index fastest
-    int o_l, cc, tap;
-    if (BN == 128 ? !weight_image_element<128>(t, taps, mirror, o_l, cc, tap) : !weight_image_element<64>(t, taps, mirror, o_l, cc, tap)) return;
-    const int c = chunk * IG_CC + cc, o = o_tile * BN + o_l;
-    float v = 0.f;
-    if (c < C && o < O) v = w_ref[(long)wb * C * taps * O + weight_source_index(c, tap, o, C, O, taps, mirror)];
-    dst[(long)slab * BN * w_pitch_halfs + (long)o_l * w_pitch_halfs + tap * IG_CC + cc] = (_Float16)v;
+    const int t = blockIdx.x * 256 + threadIdx.x;             // (row, tap) within the slab, rows fastest
+    const int o_l = t % BN, tap = t / BN;
+    if (tap >= taps) return;
+    half8_t h[2];
+    weight_row_tap(h, w_ref + (long)wb * C * taps * O, chunk, tap, o_tile * BN + o_l, C, O, taps, mirror);
+    half8_t* q = reinterpret_cast<half8_t*>(dst + (long)slab * BN * w_pitch_halfs + (long)o_l * w_pitch_halfs + tap * IG_CC);
+    q[0] = h[0];
+    q[1] = h[1];
 }
 
 // NO: 32-channel blocks per wave (BN / 64); every wave also owns two 32-pixel blocks. TP: staging tasks per thread.
@@ -2110,7 +2116,7 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
     _Float16* wimg = static_cast<_Float16*>(lease.ptr);
     if (lease.fill) {
-        dim3 pg((unsigned)((BN * taps * IG_CC + 255) / 256), (unsigned)(w_batch * n_otiles * img_chunks));
+        dim3 pg((unsigned)((BN * taps + 255) / 256), (unsigned)(w_batch * n_otiles * img_chunks));
         hipLaunchKernelGGL(conv_weight_image_gen_kernel, pg, dim3(256), 0, s, wimg, w_ref, (int)C, (int)O, taps, BN, w_pitch / 2,
                            img_chunks, n_otiles, w_mirror ? 1 : 0);
     }
