@@ -3518,7 +3518,9 @@ __global__ __launch_bounds__(256) void conv_dwg_reduce_kernel(float* __restrict_
 // Row bands per image for the weight-gradient kernels: with `units` (chunk, output tile, image) triples and `resident`
 // workgroups running at a time, the number of bands that minimises rounds x (segments of a band + the cost of a
 // workgroup's result stores, in segment times). More bands even the rounds out, fewer keep the partial sums small.
-static int dwg_pick_bands(long units, long resident, long row_steps, long segs, double store_cost) {
+// `region_cost`: what one more set of partial sums costs the reduction that follows, in segment times (0 leaves it out).
+static int dwg_pick_bands(long units, long resident, long row_steps, long segs, double store_cost, double region_cost = 0.0,
+                          double* cost_out = nullptr) {
     int best = 1;
     double best_cost = 1e300;
     const long max_bands = row_steps < 64 ? row_steps : 64;
@@ -3527,9 +3529,10 @@ static int dwg_pick_bands(long units, long resident, long row_steps, long segs, 
         const long bands = (row_steps + steps - 1) / steps;
         if (bands != b) continue;                                     // the same split as a smaller count
         const long rounds = (units * bands + resident - 1) / resident;
-        const double cost = (double)rounds * ((double)steps * (double)segs + store_cost);
+        const double cost = (double)rounds * ((double)steps * (double)segs + store_cost) + (double)(units * bands) * region_cost;
         if (cost < best_cost - 1e-9) { best_cost = cost; best = (int)b; }
     }
+    if (cost_out) *cost_out = best_cost;
     return best;
 }
 
@@ -3565,14 +3568,18 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     const long row_steps = ((long)Ho + SR - 1) / SR, segs = ((long)Wo + SW - 1) / SW;
     const long resident = (long)device_cu_count();
     const long tiles = (long)chunks * otiles;
-    int bands = dwg_pick_bands(tiles * (long)N, resident, row_steps, segs, 3.0), ipw = 1;
+    // A set of partial sums (256 rows x 128 channels of fp32, 128 KiB) is read back by the reduction at about 0.03 us,
+    // a hundredth of the 2.5-3 us a segment takes: that decides between splits of nearly equal rounds (16 x 256 x 56 x 56 -> 256: 4 bands of 7 row steps left
+    // 1280 sets, 168 MB, and 46 us of reduction behind a 154 us kernel).
+    const double region_cost = 0.011;
+    double best = 0.0;
+    int bands = dwg_pick_bands(tiles * (long)N, resident, row_steps, segs, 3.0, region_cost, &best), ipw = 1;
     if (shared && N > 1) {
-        const double steps1 = (double)((row_steps + bands - 1) / bands) * (double)segs;
-        double best = (double)((tiles * (long)N * bands + resident - 1) / resident) * (steps1 + 3.0);
         for (long g = 2; g <= (long)N && g <= 64; g++) {
             const long groups = ((long)N + g - 1) / g;
             if ((groups - 1) * g >= (long)N) continue;
-            const double cost = (double)((tiles * groups + resident - 1) / resident) * ((double)g * (double)row_steps * (double)segs + 3.0);
+            const double cost = (double)((tiles * groups + resident - 1) / resident) * ((double)g * (double)row_steps * (double)segs + 3.0) +
+                                (double)(tiles * groups) * region_cost;
             if (cost < best - 1e-9) { best = cost; ipw = (int)g; bands = 1; }
         }
     }
