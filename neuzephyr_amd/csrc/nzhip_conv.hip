@@ -2061,6 +2061,24 @@ static bool conv_igemm_gen_fits(size_t W_out, size_t O, size_t K_h, size_t K_w, 
 }
 
 // Returns NZHIP_E_UNSUPPORTED (nothing enqueued, no error text) when the tile does not fit LDS or a thread's staging share.
+// dst[row][0 .. Ww) = src[row][0 .. W) followed by zeros, Ww the next multiple of 4: image rows that are whole 16-byte
+// pieces. The zeros stand where the convolution's padding would: the kernel below then reads columns W .. Ww - 1 as
+// zeros from memory instead of as zeros from its bounds check, and the output extents stay what they were.
+// 256 >> wq_log rows per workgroup, a thread four columns of a row.
+__global__ __launch_bounds__(256) void widen_rows_kernel(float* __restrict__ dst, const float* __restrict__ src, long rows, int W, int Ww,
+                                                         int wq_log) {
+    const long row = (long)blockIdx.x * (256 >> wq_log) + (threadIdx.x >> wq_log);
+    if (row >= rows) return;
+    const float* srow = src + row * W;
+    float* drow = dst + row * Ww;
+    for (int w0 = (threadIdx.x & ((1 << wq_log) - 1)) * 4; w0 < Ww; w0 += 4 << wq_log) {
+        floatx4 v;
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = w0 + j < W ? srow[w0 + j] : 0.f;
+        *reinterpret_cast<floatx4*>(drow + w0) = v;
+    }
+}
+
 static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C, size_t H,
                                  size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t w_batch,
                                  int64_t bias_sp, int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out,
@@ -2103,6 +2121,30 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     // not split, the rows allow 16-byte loads and two slabs and two halo planes fit LDS and a thread's staging share;
     // the weight image then holds an even number of slabs per channel tile, the last one zero when n_chunks is odd.
     static const char* cpb_env = getenv("NZHIP_CONV_CPB");           // benchmarking only: 1 keeps one chunk per step
+    // Rows that are not whole 16-byte pieces (14-, 30-, 35-wide images) stage with four loads and four bounds per task
+    // and never two chunks per step. From about 8 GFLOP on, a zero-filled copy with rows of the next multiple of 4 pays
+    // for itself (16 x 192 x 35 x 35 -> 192: 120 -> 81 us; 16 x 512 x 14 x 14 -> 512: 85 -> 70; 16 x 256 x 14 x 14 -> 256
+    // would stay at 37).
+    const char* widen_env = getenv("NZHIP_CONV_WIDEN");              // benchmarks and tests: 0 never, 1 wherever rows are not whole pieces (read per call)
+    float* x_wide = nullptr;
+    const double flops = 2.0 * (double)N * (double)H_out * (double)W_out * (double)C * (double)taps * (double)O;
+    if (W % 4 != 0 && (widen_env ? atoi(widen_env) != 0 : flops >= 8e9)) {
+        const size_t Ww = (W + 3) / 4 * 4, rows = N * C * H;
+        int wq_log = 0;
+        while (wq_log < 8 && ((size_t)4 << wq_log) < Ww) wq_log++;
+        const size_t blocks = (rows + (256 >> wq_log) - 1) / (256 >> wq_log);
+        if (blocks <= 0x7fffffffull && Ww < 0x3fffffff && C * H * Ww < 0x7fffffffull) {      // the kernel's int offsets
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&x_wide), rows * Ww * sizeof(float), s)) return rc;
+            hipLaunchKernelGGL(widen_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x_wide, x, (long)rows, (int)W, (int)Ww, wq_log);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) {
+                workspace_free(x_wide, s);
+                return set_hip_error(e, "widen_rows kernel launch");
+            }
+            x = x_wide;
+            W = Ww;
+        }
+    }
     const bool vec = W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
     const bool two = vec && chunk_groups == 1 && n_chunks >= 4 && !(cpb_env && atoi(cpb_env) == 1) &&
                      ((size_t)2 * slab_bytes + 1023) / 1024 * 1024 + (size_t)2 * span * pw * 32 <= 160 * 1024 - 512 &&
@@ -2113,7 +2155,10 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     uint64_t key[PREPARED_KEY_WORDS];
     conv_image_key(key, 3, (int)K_h, (int)K_w, BN, w_ref, C, O, img_chunks, n_otiles, w_batch, w_mirror);
     ImageLease lease;
-    if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) return rc;
+    if (int rc = image_acquire(PREPARED_CONV_W, key, bytes, s, &lease)) {
+        if (x_wide) workspace_free(x_wide, s);
+        return rc;
+    }
     _Float16* wimg = static_cast<_Float16*>(lease.ptr);
     if (lease.fill) {
         dim3 pg((unsigned)((BN * taps + 255) / 256), (unsigned)(w_batch * n_otiles * img_chunks));
@@ -2141,6 +2186,7 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     if (chunk_groups > 1) {
         if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), (size_t)chunk_groups * per_group * sizeof(float), s)) {
             image_release(lease, s, true);
+            if (x_wide) workspace_free(x_wide, s);
             return rc;
         }
         a.partial = partial;
@@ -2178,7 +2224,8 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     }
     const int rc3 = partial ? workspace_free(partial, s) : NZHIP_OK;
     const int rc2 = image_release(lease, s, rc == NZHIP_OK);
-    return rc ? rc : (rc2 ? rc2 : rc3);
+    const int rc4 = x_wide ? workspace_free(x_wide, s) : NZHIP_OK;
+    return rc ? rc : (rc2 ? rc2 : (rc3 ? rc3 : rc4));
 }
 
 // General route: column matrix in a pooled workspace, then ONE batched GEMM that computes the

@@ -191,6 +191,44 @@ def test_conv2d_any_geometry_integers_bit_exact(nz, oracle, N, C, H, W, O, k_h, 
         assert np.array_equal(got[n:n + 1].astype(np.float64), truth), (n,)
 
 
+WIDENED = [  # N, C, H, W, O, k, stride, pad, w_batch, per-pixel bias: rows that are not whole 16-byte pieces on the any-geometry kernel
+    # (5x5; stride 2 with the per-pixel bias; a split contraction; per-sample weights; two chunks per loop step, which such
+    # rows only reach through the copy; 7x7 stride 2 on three channels)
+    (64, 16, 14, 14, 32, 5, 1, 2, 1, False), (64, 24, 21, 30, 70, 3, 2, 1, 1, True), (16, 256, 14, 14, 96, 3, 1, 1, 1, False),
+    (16, 5, 30, 30, 9, 3, 1, 1, 16, False), (256, 64, 14, 14, 48, 5, 1, 2, 1, False), (8, 3, 97, 97, 20, 7, 2, 3, 1, False)]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,k,stride,pad,w_batch,pix", WIDENED)
+def test_conv2d_on_rows_widened_to_16_byte_pieces_is_bit_exact(nz, oracle, monkeypatch, N, C, H, W, O, k, stride, pad, w_batch, pix):
+    # Large layers with such rows run on a zero-filled copy whose rows are the next multiple of 4 wide; the library reads
+    # NZHIP_CONV_WIDEN per call, so the copy can be forced for shapes an oracle finishes quickly. Forward, and the
+    # stride-1 data gradient (the same kernel on the output gradient, mirrored weights, accumulating in place).
+    monkeypatch.setenv("NZHIP_CONV_WIDEN", "1")
+    rng = np.random.default_rng(N * 3 + C * 5 + H * 7 + W * 11 + O * 13 + k + stride)
+    Ho, Wo = oracle.out_hw(H, W, k, k, stride, pad)
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    ws = [rng.integers(-3, 4, size=(O, C, k, k)).astype(np.float32) for _ in range(w_batch)]
+    w_ref = np.concatenate([oracle.weights_oihw_to_ref(w) for w in ws], axis=0)
+    if pix:
+        bias = rng.integers(-2, 3, size=(1, 1, Ho * Wo, O)).astype(np.float32)
+        strides, badd = (O, 1), bias.reshape(Ho, Wo, O).transpose(2, 0, 1)[None].astype(np.float64)
+    else:
+        bias = rng.integers(-2, 3, size=(O,)).astype(np.float32)
+        strides, badd = (0, 1), bias.reshape(1, O, 1, 1).astype(np.float64)
+    got = host(nz.conv2d_forward(dev(x), dev(w_ref), dev(bias), k, k, stride, pad, bias_strides=strides, relu=True))
+    for n in range(N):
+        w = ws[n if w_batch > 1 else 0]
+        truth = np.maximum(oracle.conv2d_direct_f64(x[n:n + 1], w, None, stride, pad) + badd, 0)
+        assert np.array_equal(got[n:n + 1].astype(np.float64), truth), ("forward", n)
+    if stride == 1:
+        dy = rng.integers(-4, 5, size=(N, O, Ho, Wo)).astype(np.float32)
+        dx0 = rng.integers(-3, 4, size=(N, C, H, W)).astype(np.float32)
+        for accumulate in (False, True):
+            expect = oracle.conv2d_backward_data(dx0.copy() if accumulate else np.zeros_like(dx0), dy, w_ref, k, k, pad)
+            got_dx = host(nz.conv2d_backward_data(dev(dx0), dev(dy), dev(w_ref), k, k, 1, pad, accumulate=accumulate))
+            assert np.array_equal(got_dx, expect), ("data gradient", accumulate)
+
+
 PER_SAMPLE = [  # N, C, H, W, O, k, pad, per-pixel bias: one weight copy per image, every copy different
     (4, 32, 12, 64, 128, 3, 1, False),    # two halo buffers, 128-channel tile, 64 workgroups per image
     (3, 64, 9, 64, 64, 3, 1, True),       # two halo buffers, 64-channel tile, per-pixel bias; 255 of 256 workgroups used
