@@ -2078,6 +2078,23 @@ __global__ __launch_bounds__(256) void widen_rows_kernel(float* __restrict__ dst
         *reinterpret_cast<floatx4*>(drow + w0) = v;
     }
 }
+// *out: a pooled workspace holding `rows` rows of src widened from W to the next multiple of 4 columns
+static int widen_rows(float** out, const float* src, size_t rows, size_t W, hipStream_t s) {
+    const size_t Ww = (W + 3) / 4 * 4;
+    int wq_log = 0;
+    while (wq_log < 8 && ((size_t)4 << wq_log) < Ww) wq_log++;
+    const size_t blocks = (rows + (256 >> wq_log) - 1) / (256 >> wq_log);
+    if (blocks > 0x7fffffffull || Ww >= 0x3fffffff) return set_error(NZHIP_E_UNSUPPORTED, "widen_rows: extents beyond the kernel's grid");
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(out), rows * Ww * sizeof(float), s)) return rc;
+    hipLaunchKernelGGL(widen_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, *out, src, (long)rows, (int)W, (int)Ww, wq_log);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        workspace_free(*out, s);
+        *out = nullptr;
+        return set_hip_error(e, "widen_rows kernel launch");
+    }
+    return NZHIP_OK;
+}
 
 static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C, size_t H,
                                  size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t w_batch,
@@ -2129,18 +2146,9 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     float* x_wide = nullptr;
     const double flops = 2.0 * (double)N * (double)H_out * (double)W_out * (double)C * (double)taps * (double)O;
     if (W % 4 != 0 && (widen_env ? atoi(widen_env) != 0 : flops >= 8e9)) {
-        const size_t Ww = (W + 3) / 4 * 4, rows = N * C * H;
-        int wq_log = 0;
-        while (wq_log < 8 && ((size_t)4 << wq_log) < Ww) wq_log++;
-        const size_t blocks = (rows + (256 >> wq_log) - 1) / (256 >> wq_log);
-        if (blocks <= 0x7fffffffull && Ww < 0x3fffffff && C * H * Ww < 0x7fffffffull) {      // the kernel's int offsets
-            if (int rc = workspace_alloc(reinterpret_cast<void**>(&x_wide), rows * Ww * sizeof(float), s)) return rc;
-            hipLaunchKernelGGL(widen_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, x_wide, x, (long)rows, (int)W, (int)Ww, wq_log);
-            hipError_t e = hipGetLastError();
-            if (e != hipSuccess) {
-                workspace_free(x_wide, s);
-                return set_hip_error(e, "widen_rows kernel launch");
-            }
+        const size_t Ww = (W + 3) / 4 * 4;
+        if (C * H * Ww < 0x7fffffffull && N * C * H < 0x7fffffffull) {      // the kernels' int offsets and grids
+            if (int rc = widen_rows(&x_wide, x, N * C * H, W, s)) return rc;
             x = x_wide;
             W = Ww;
         }
@@ -3583,10 +3591,11 @@ static int dwg_pick_bands(long units, long resident, long row_steps, long segs, 
     return best;
 }
 
-static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W, size_t O,
-                           size_t K_h, size_t K_w, size_t stride, size_t pad, bool shared, hipStream_t s) {
+// Ho, Wo: the extents of dy as it lies in memory. Wo may exceed what (W, K_w, stride, pad) give when dy is a copy with
+// zero-filled columns appended (below): those columns add nothing to any sum.
+static int conv_dw_generic_run(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W, size_t O,
+                               size_t K_h, size_t K_w, size_t stride, size_t pad, size_t Ho, size_t Wo, bool shared, hipStream_t s) {
     const size_t taps = K_h * K_w;
-    const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
     const bool vec = W % 4 == 0 && Wo % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(dy)) & 15) == 0;
     int cc = (int)(DWG8_ROWS / taps);
     if (cc > (int)C) cc = (int)C;
@@ -3668,6 +3677,33 @@ static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N,
     }
     const int rc2 = workspace_free(partial, s);
     return rc ? rc : rc2;
+}
+
+// Rows of x or dy that are not whole 16-byte pieces (14-wide images, 28-wide ones at stride 2) put the kernel on four
+// loads and four bounds per piece and one fragment set. From about 3 GFLOP on, zero-filled copies with rows of the next
+// multiple of 4 pay for themselves; appended zeros of dy add nothing, and the columns appended to x are the zeros its
+// bounds check would have produced (16 x 512 x 14 x 14 -> 512: 89 -> 56 us + two copies of 6 MB; 16 x 192 x 35 x 35 -> 192:
+// 123 -> 66; 16 x 256 x 28 x 28 -> 256 at stride 2: 55 -> 33). NZHIP_CONV_WIDEN (read per call): 0 never, 1 always.
+static int conv_dw_generic(float* dw, const float* x, const float* dy, size_t N, size_t C, size_t H, size_t W, size_t O,
+                           size_t K_h, size_t K_w, size_t stride, size_t pad, bool shared, hipStream_t s) {
+    const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
+    const char* widen_env = getenv("NZHIP_CONV_WIDEN");
+    const double flops = 2.0 * (double)N * (double)Ho * (double)Wo * (double)C * (double)(K_h * K_w) * (double)O;
+    const size_t Ww = (W + 3) / 4 * 4, Wow = (Wo + 3) / 4 * 4;
+    const bool widen = (W % 4 != 0 || Wo % 4 != 0) && (widen_env ? atoi(widen_env) != 0 : flops >= 3e9) && H * Ww < 0x3fffffffull &&
+                       N * C * H < 0x7fffffffull && N * O * Ho < 0x7fffffffull;
+    if (!widen) return conv_dw_generic_run(dw, x, dy, N, C, H, W, O, K_h, K_w, stride, pad, Ho, Wo, shared, s);
+    float* x_wide = nullptr;
+    float* dy_wide = nullptr;
+    int rc = NZHIP_OK;
+    if (W % 4 != 0) rc = widen_rows(&x_wide, x, N * C * H, W, s);
+    if (rc == NZHIP_OK && Wo % 4 != 0) rc = widen_rows(&dy_wide, dy, N * O * Ho, Wo, s);
+    if (rc == NZHIP_OK)
+        rc = conv_dw_generic_run(dw, x_wide ? x_wide : x, dy_wide ? dy_wide : dy, N, C, H, x_wide ? Ww : W, O, K_h, K_w, stride, pad, Ho,
+                                 dy_wide ? Wow : Wo, shared, s);
+    const int rc2 = dy_wide ? workspace_free(dy_wide, s) : NZHIP_OK;
+    const int rc3 = x_wide ? workspace_free(x_wide, s) : NZHIP_OK;
+    return rc ? rc : (rc2 ? rc2 : rc3);
 }
 
 }  // namespace nzhip

@@ -414,6 +414,14 @@ def test_conv_backward_weights_any_geometry_is_bit_exact_on_integers(nz, oracle,
     assert np.array_equal(got, expect)
 
 
+@pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", [c for c in CONV_GEN_BWD_W if c[3] % 4 != 0 or ((c[3] + 2 * c[8] - c[6]) // c[7] + 1) % 4 != 0])
+def test_conv_backward_weights_on_rows_widened_to_16_byte_pieces(nz, oracle, monkeypatch, N, C, H, W, O, Kh, Kw, stride, pad, wb):
+    # Large layers whose rows of x or dy are not whole 16-byte pieces run on zero-filled copies with rows of the next
+    # multiple of 4; the library reads NZHIP_CONV_WIDEN per call, so the copies can be forced for these small shapes.
+    monkeypatch.setenv("NZHIP_CONV_WIDEN", "1")
+    test_conv_backward_weights_any_geometry_is_bit_exact_on_integers(nz, oracle, N, C, H, W, O, Kh, Kw, stride, pad, wb)
+
+
 def test_conv_backward_weights_any_geometry_float_tolerance(nz, oracle):
     N, C, H, W, O, K, stride, pad = 2, 24, 40, 72, 48, 5, 2, 2
     Ho, Wo = (H + 2 * pad - K) // stride + 1, (W + 2 * pad - K) // stride + 1
