@@ -2096,6 +2096,18 @@ static int widen_rows(float** out, const float* src, size_t rows, size_t W, hipS
     return NZHIP_OK;
 }
 
+// 1x1 layers are products whose operands have an image's pixels as their contiguous rows: with a pixel count that is not
+// a multiple of 4 (7 x 7, 17 x 17, 35 x 35 images) the product loads them element by element. A zero-filled copy with
+// planes of the next multiple of 4 pays for itself when the copied operand is the small one of the product, i.e. when
+// every copied element takes part in many multiply-adds (`flops_per_element`: 2 x the channels on the other side):
+// 16 x 512 x 7 x 7 -> 2048 forward 40 -> 25 us, its data gradient 47 -> 29; 16 x 192 x 35 x 35 -> 64 forward would go from
+// 22 to 33 us (the copy of x costs what the whole product does) and stays as it is.
+static bool conv1x1_wants_wide_planes(size_t HW, double flops, double flops_per_element) {
+    const char* widen_env = getenv("NZHIP_CONV_WIDEN");              // benchmarks and tests: 0 never, 1 always (read per call)
+    if (HW % 4 == 0) return false;
+    return widen_env ? atoi(widen_env) != 0 : (flops >= 4e8 && flops_per_element >= 512.0);
+}
+
 static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, const float* bias, size_t N, size_t C, size_t H,
                                  size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad, size_t w_batch,
                                  int64_t bias_sp, int64_t bias_sc, int64_t bias_sn, int act, size_t H_out, size_t W_out,
@@ -2952,7 +2964,16 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
         g.a_stride_n = w_batch > 1 ? (int64_t)(C * O) : 0; g.b_stride_n = (int64_t)(C * H * W); g.c_stride_n = (int64_t)(O * H * W);
         g.bias = bias; g.bias_stride_row = bias_stride_channel; g.bias_stride_col = bias_stride_pixel; g.bias_stride_n = bias_stride_image;
         g.activation = activation;
-        return nzhip_gemm(&g, s);
+        float* x_wide = nullptr;
+        const double flops = 2.0 * (double)N * (double)(H * W) * (double)C * (double)O;
+        if (conv1x1_wants_wide_planes(H * W, flops, 2.0 * (double)O)) {
+            if (int rc = widen_rows(&x_wide, x, N * C, H * W, s)) return rc;
+            const size_t HWp = (H * W + 3) / 4 * 4;
+            g.B = x_wide; g.ldb = (int64_t)HWp; g.b_stride_n = (int64_t)(C * HWp);
+        }
+        const int rc = x_wide ? gemm_padded_rows(g, 2, s) : nzhip_gemm(&g, s);
+        const int rc2 = x_wide ? workspace_free(x_wide, s) : NZHIP_OK;
+        return rc ? rc : rc2;
     }
     bool wide = false, bn128 = false;
     const ConvRoute route = conv_forward_route(x, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, H_out, W_out, wide, bn128);
@@ -3076,7 +3097,16 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
         if (accumulate) {
             g.bias = dx; g.bias_stride_n = g.c_stride_n; g.bias_stride_row = g.ldc; g.bias_stride_col = 1;
         }
-        return nzhip_gemm(&g, s);
+        float* dy_wide = nullptr;
+        const double flops = 2.0 * (double)N * (double)(H * W) * (double)C * (double)O;
+        if (conv1x1_wants_wide_planes(H * W, flops, 2.0 * (double)C)) {
+            if (int rc = widen_rows(&dy_wide, dy, N * O, H * W, s)) return rc;
+            const size_t HWp = (H * W + 3) / 4 * 4;
+            g.B = dy_wide; g.ldb = (int64_t)HWp; g.b_stride_n = (int64_t)(O * HWp);
+        }
+        const int rc = dy_wide ? gemm_padded_rows(g, 2, s) : nzhip_gemm(&g, s);
+        const int rc2 = dy_wide ? workspace_free(dy_wide, s) : NZHIP_OK;
+        return rc ? rc : rc2;
     }
     if (stride > 1) {
         const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
@@ -3756,7 +3786,19 @@ extern "C" int nzhip_conv2d_backward_weights(float* dw, const float* x, const fl
     if (K_h == 1 && K_w == 1 && stride == 1 && pad == 0 && H > 0 && W > 0 && H * W < 0x3fffffff && C < 0x3fffffff &&
         O < 0x3fffffff && N <= 65535 && N * C * O < 0x7fffffffull) {
         if (N == 0 || C == 0 || O == 0) return NZHIP_OK;
-        return conv1x1_backward_weights(dw, x, dy, N, C, H * W, O, w_batch == 1, reinterpret_cast<hipStream_t>(stream));
+        hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+        if (conv1x1_wants_wide_planes(H * W, 2.0 * (double)N * (double)(H * W) * (double)C * (double)O,
+                                      2.0 * (double)C * (double)O / (double)(C + O))) {   // zero-filled planes of whole 16-byte pieces: the zeros add nothing
+            float* x_wide = nullptr;
+            float* dy_wide = nullptr;
+            int rc = widen_rows(&x_wide, x, N * C, H * W, s);
+            if (rc == NZHIP_OK) rc = widen_rows(&dy_wide, dy, N * O, H * W, s);
+            if (rc == NZHIP_OK) rc = conv1x1_backward_weights(dw, x_wide, dy_wide, N, C, (H * W + 3) / 4 * 4, O, w_batch == 1, s);
+            const int rc2 = dy_wide ? workspace_free(dy_wide, s) : NZHIP_OK;
+            const int rc3 = x_wide ? workspace_free(x_wide, s) : NZHIP_OK;
+            return rc ? rc : (rc2 ? rc2 : rc3);
+        }
+        return conv1x1_backward_weights(dw, x, dy, N, C, H * W, O, w_batch == 1, s);
     }
     if (stride == 0 || K_h == 0 || K_w == 0) return set_error(NZHIP_E_INVALID, "nzhip_conv2d_backward_weights: zero stride or kernel extent");
     if (H + 2 * pad < K_h || W + 2 * pad < K_w)

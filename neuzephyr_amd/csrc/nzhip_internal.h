@@ -29,6 +29,9 @@ bool gemm_vec_legal(const nzhip_gemm_desc& d);   // 16-byte global accesses are 
 bool gemm_operand_vec_legal(const float* X, int64_t ld, int64_t contig, int64_t stride_n, int64_t stride_c);
 bool gemm_operands_vec_legal(const nzhip_gemm_desc& d, int padded = 0);   // ... for A and B (decides the kernel instance)
 bool gemm_c_vec_legal(const nzhip_gemm_desc& d);          // ... for C (decides the epilogue's stores)
+// nzhip_gemm for operands the library itself made: padded bit 0 / bit 1 = the rows of A / B are readable up to the next
+// multiple of 4 elements and hold zeros there, so 16-byte loads are legal although the extents are not multiples of 4.
+int gemm_padded_rows(const nzhip_gemm_desc& d, int padded, hipStream_t stream);
 // waves: 0 = choose, else 2 / 4 / 8; mfma: 0 = choose, else 16 (16x16x32) / 32 (32x32x16)
 int gemm_h16_dispatch(const nzhip_gemm_desc& d, hipStream_t stream, int waves = 0, int mfma = 0);
 // Both passes in one kernel (rounding overlapped with the MFMA loop) for products of whole 4096 x 4096 x 1024 blocks.

@@ -493,6 +493,14 @@ int nzhip_gemm(const nzhip_gemm_desc* desc, void* stream) {
 
 }  // extern "C"
 
+namespace nzhip {
+int gemm_padded_rows(const nzhip_gemm_desc& d, int padded, hipStream_t stream) {
+    if (int rc = validate_gemm(d)) return rc;
+    if (d.M == 0 || d.N == 0) return NZHIP_OK;
+    return gemm_routed(d, stream, padded);
+}
+}  // namespace nzhip
+
 // The route choice behind nzhip_gemm, for a validated descriptor with M, N > 0.
 static int gemm_routed(const nzhip_gemm_desc& d, hipStream_t s, int padded) {
     if (d.K == 0) {

@@ -414,7 +414,8 @@ def test_conv_backward_weights_any_geometry_is_bit_exact_on_integers(nz, oracle,
     assert np.array_equal(got, expect)
 
 
-@pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", [c for c in CONV_GEN_BWD_W if c[3] % 4 != 0 or ((c[3] + 2 * c[8] - c[6]) // c[7] + 1) % 4 != 0])
+@pytest.mark.parametrize("N,C,H,W,O,Kh,Kw,stride,pad,wb", [c for c in CONV_GEN_BWD_W if c[3] % 4 != 0 or ((c[3] + 2 * c[8] - c[6]) // c[7] + 1) % 4 != 0] +
+                         [(3, 40, 7, 7, 24, 1, 1, 1, 0, 1), (2, 20, 5, 5, 33, 1, 1, 1, 0, 2), (2, 70, 35, 35, 9, 1, 1, 1, 0, 1)])   # and 1x1 products on planes of 49, 25, 1225 pixels
 def test_conv_backward_weights_on_rows_widened_to_16_byte_pieces(nz, oracle, monkeypatch, N, C, H, W, O, Kh, Kw, stride, pad, wb):
     # Large layers whose rows of x or dy are not whole 16-byte pieces run on zero-filled copies with rows of the next
     # multiple of 4; the library reads NZHIP_CONV_WIDEN per call, so the copies can be forced for these small shapes.

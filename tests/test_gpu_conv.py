@@ -195,7 +195,10 @@ WIDENED = [  # N, C, H, W, O, k, stride, pad, w_batch, per-pixel bias: rows that
     # (5x5; stride 2 with the per-pixel bias; a split contraction; per-sample weights; two chunks per loop step, which such
     # rows only reach through the copy; 7x7 stride 2 on three channels)
     (64, 16, 14, 14, 32, 5, 1, 2, 1, False), (64, 24, 21, 30, 70, 3, 2, 1, 1, True), (16, 256, 14, 14, 96, 3, 1, 1, 1, False),
-    (16, 5, 30, 30, 9, 3, 1, 1, 16, False), (256, 64, 14, 14, 48, 5, 1, 2, 1, False), (8, 3, 97, 97, 20, 7, 2, 3, 1, False)]
+    (16, 5, 30, 30, 9, 3, 1, 1, 16, False), (256, 64, 14, 14, 48, 5, 1, 2, 1, False), (8, 3, 97, 97, 20, 7, 2, 3, 1, False),
+    # 1x1 layers as products: planes of 49, 35 and 1225 pixels widened to 52, 36 and 1228 (shared and per-sample weights,
+    # per-channel and per-pixel bias)
+    (8, 130, 7, 7, 140, 1, 1, 0, 1, False), (6, 128, 5, 7, 130, 1, 1, 0, 6, True), (2, 136, 35, 35, 20, 1, 1, 0, 1, False)]
 
 
 @pytest.mark.parametrize("N,C,H,W,O,k,stride,pad,w_batch,pix", WIDENED)
