@@ -224,7 +224,8 @@ int nzhip_conv2d_forward_prepared(float* y, const float* x, const float* w_ref, 
  * accumulate != 0 adds into dx (what the chain does), 0 overwrites it. Supported: K_h == K_w, pad <= K_h - 1,
  * stride <= 8; anything else returns NZHIP_E_UNSUPPORTED and the caller runs the chain. With a stride above 1 the
  * call is either one convolution of the zero-filled output gradient or that chain inside the library (column
- * gradient in a pooled workspace), whichever an estimate from the shape finds cheaper; same sums either way. */
+ * gradient in a pooled workspace), whichever an estimate from the shape finds cheaper; stride-1 layers on images so
+ * small that the convolution would write a column matrix itself take the chain too. Same sums either way. */
 int nzhip_conv2d_backward_data(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H,
                                size_t W, size_t O, size_t K_h, size_t K_w, size_t stride, size_t pad,
                                size_t w_batch, int accumulate, void* stream);

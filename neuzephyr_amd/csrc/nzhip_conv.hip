@@ -3053,6 +3053,42 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
                                bias_stride_channel, 0, activation, stream);
 }
 
+// The reference's own chain for the data gradient (src/Nodes.cu:660-665, 169-182, 632-640) inside the library: the output
+// gradient pixel-major, the column gradient = dy^T x W^T as one product (all images as its rows when the weights are
+// shared), then the gather into the image. No mirrored weights, no column matrix of dy.
+static int conv_dx_chain(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H, size_t W, size_t O, size_t K_h,
+                         size_t K_w, size_t stride, size_t pad, size_t Ho, size_t Wo, size_t w_batch, int accumulate, void* stream) {
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const size_t P = Ho * Wo, CKK = C * K_h * K_w;
+    float* dyt = nullptr;
+    float* dcol = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&dyt), N * P * O * sizeof(float), s)) return rc;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&dcol), N * P * CKK * sizeof(float), s)) {
+        workspace_free(dyt, s);
+        return rc;
+    }
+    int rc = nzhip_col2im_backward(dyt, dy, Ho, Wo, O, N, stream);                 // [N][P][O]
+    if (rc == NZHIP_OK) {
+        nzhip_gemm_desc g = {};
+        g.A = dyt; g.K = (int64_t)O; g.lda = (int64_t)O; g.a_layout = NZHIP_LAYOUT_ROW;
+        g.B = w_ref; g.N = (int64_t)CKK; g.ldb = (int64_t)O; g.b_layout = NZHIP_LAYOUT_TRANS;       // w_ref holds CKK x O
+        g.C = dcol; g.ldc = (int64_t)CKK;
+        g.batch_c = 1;
+        if (w_batch > 1) {                                                           // one product per image
+            g.M = (int64_t)P; g.batch_n = (int64_t)N;
+            g.a_stride_n = (int64_t)(P * O); g.b_stride_n = (int64_t)(CKK * O); g.c_stride_n = (int64_t)(P * CKK);
+        } else {                                                                     // all images as rows of one product
+            g.M = (int64_t)(N * P); g.batch_n = 1;
+        }
+        g.activation = NZHIP_ACT_NONE;
+        rc = nzhip_gemm(&g, s);
+    }
+    if (rc == NZHIP_OK && !accumulate) rc = nzhip_fill(dx, 0.f, N * C * H * W, stream);
+    if (rc == NZHIP_OK) rc = nzhip_im2col_backward(dx, dcol, Ho, Wo, C, K_h, K_w, stride, pad, H, W, N, stream);
+    const int rc2 = workspace_free(dcol, s), rc3 = workspace_free(dyt, s);
+    return rc ? rc : (rc2 ? rc2 : rc3);
+}
+
 /* Gradient of nzhip_conv2d_forward with respect to x: one convolution of dy with the
  * mirrored weights instead of the reference's chain Col2ImgNode::backward -> MatMulNode::backward
  * (dA += dC * B^T) -> Img2ColNode::backward (src/Nodes.cu:660-665, 169-182, 632-640), which writes and
@@ -3128,35 +3164,8 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
         const double as_chain = flops / 400e6 + 3.0 * N * Ho * Wo * C * K_h * K_w * 4.0 / 4e6;
         const size_t P = Ho * Wo, CKK = C * K_h * K_w;
         const bool chain_fits = N * P < 0x3fffffff && CKK < 0x3fffffff && O < 0x3fffffff && N <= 65535 && P * O < 0x7fffffffull;
-        if (chain_fits && (dx_env ? dx_env[1] == 'h' : as_conv >= 1.5 * as_chain)) {
-            float* dyt = nullptr;
-            float* dcol = nullptr;
-            if (int rc = workspace_alloc(reinterpret_cast<void**>(&dyt), N * P * O * sizeof(float), s)) return rc;
-            if (int rc = workspace_alloc(reinterpret_cast<void**>(&dcol), N * P * CKK * sizeof(float), s)) {
-                workspace_free(dyt, s);
-                return rc;
-            }
-            int rc = nzhip_col2im_backward(dyt, dy, Ho, Wo, O, N, stream);                 // [N][P][O]
-            if (rc == NZHIP_OK) {
-                nzhip_gemm_desc g = {};
-                g.A = dyt; g.K = (int64_t)O; g.lda = (int64_t)O; g.a_layout = NZHIP_LAYOUT_ROW;
-                g.B = w_ref; g.N = (int64_t)CKK; g.ldb = (int64_t)O; g.b_layout = NZHIP_LAYOUT_TRANS;       // w_ref holds CKK x O
-                g.C = dcol; g.ldc = (int64_t)CKK;
-                g.batch_c = 1;
-                if (w_batch > 1) {                                                           // one product per image
-                    g.M = (int64_t)P; g.batch_n = (int64_t)N;
-                    g.a_stride_n = (int64_t)(P * O); g.b_stride_n = (int64_t)(CKK * O); g.c_stride_n = (int64_t)(P * CKK);
-                } else {                                                                     // all images as rows of one product
-                    g.M = (int64_t)(N * P); g.batch_n = 1;
-                }
-                g.activation = NZHIP_ACT_NONE;
-                rc = nzhip_gemm(&g, s);
-            }
-            if (rc == NZHIP_OK && !accumulate) rc = nzhip_fill(dx, 0.f, N * C * H * W, stream);
-            if (rc == NZHIP_OK) rc = nzhip_im2col_backward(dx, dcol, Ho, Wo, C, K_h, K_w, stride, pad, H, W, N, stream);
-            const int rc2 = workspace_free(dcol, s), rc3 = workspace_free(dyt, s);
-            return rc ? rc : (rc2 ? rc2 : rc3);
-        }
+        if (chain_fits && (dx_env ? dx_env[1] == 'h' : as_conv >= 1.5 * as_chain))
+            return conv_dx_chain(dx, dy, w_ref, N, C, H, W, O, K_h, K_w, stride, pad, Ho, Wo, w_batch, accumulate, stream);
         const size_t Hu = H + 2 * pad - K_h + 1, Wu = W + 2 * pad - K_w + 1, total = N * O * Hu * Wu;
         if (Hu > 0x3fffffff || Wu > 0x3fffffff)
             return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_data: extents beyond the fused kernels (use the column-matrix chain)");
@@ -3176,6 +3185,18 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     const size_t pad_t = K_h - 1 - pad;
     bool wide_unused = false, bn_unused = false;
     const ConvRoute route = conv_forward_route(dy, N, O, H_out, W_out, C, K_h, K_w, 1, pad_t, w_batch, H, W, wide_unused, bn_unused);
+    {
+        // Where the convolution itself would write dy's column matrix (tiny images: 7 x 7, 4 x 4), the chain is the shorter
+        // way: no mirrored copy of the weights, no column matrix of dy, no second pass for "+=" (16 x 512 x 7 x 7 <- 512, 3x3:
+        // 56 -> 33 us).
+        static const char* dx_env = getenv("NZHIP_CONV_DX");              // benchmarking only: "chain" | "conv"
+        const size_t P = H_out * W_out, CKK = C * K_h * K_w;
+        const bool chain_fits = N * P < 0x3fffffff && CKK < 0x3fffffff && O < 0x3fffffff && N <= 65535 && P * O < 0x7fffffffull &&
+                                N * P * CKK <= ((size_t)1 << 28);
+        const bool column_route = route != CONV_ROUTE_FIXED && route != CONV_ROUTE_ANY && route != CONV_ROUTE_DIRECT;
+        if (chain_fits && (dx_env ? dx_env[1] == 'h' : column_route))
+            return conv_dx_chain(dx, dy, w_ref, N, C, H, W, O, K_h, K_w, 1, pad, H_out, W_out, w_batch, accumulate, stream);
+    }
     const bool in_place = accumulate && (route == CONV_ROUTE_FIXED || route == CONV_ROUTE_ANY);
     if (accumulate && !in_place) rc = workspace_alloc(reinterpret_cast<void**>(&tmp), x_elems * sizeof(float), s);
     // the weights go in as they are: the implicit-GEMM routes mirror them while they build their fp16 image, the others
