@@ -3053,10 +3053,78 @@ extern "C" int nzhip_conv2d_forward(float* y, const float* x, const float* w_ref
                                bias_stride_channel, 0, activation, stream);
 }
 
-// The reference's own chain for the data gradient (src/Nodes.cu:660-665, 169-182, 632-640) inside the library: the output
-// gradient pixel-major, the column gradient = dy^T x W^T as one product (all images as its rows when the weights are
-// shared), then the gather into the image. No mirrored weights, no column matrix of dy.
-static int conv_dx_chain(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H, size_t W, size_t O, size_t K_h,
+namespace nzhip {
+// img2colBackwardKernel (src/OperationKernels.cu:1337-1355) as a gather from the TRANSPOSED column gradient
+// colT[image][(c, r, s)][pixel] (rows `pitch` floats apart): one thread owns one element of dx and adds the entries that
+// were copied from it in ascending pixel order, the order of the library's im2col_backward kernel and of the reference's
+// element index. With the pixels contiguous, the threads of a wave (adjacent w) read adjacent addresses; from the
+// reference's layout [pixel][(c, r, s)] every lane touches a line of its own.
+__global__ __launch_bounds__(256) void col_t_gather_kernel(float* __restrict__ dx, const float* __restrict__ colT, int H_out, int W_out,
+                                                           int C, int K_h, int K_w, int stride, int pad, int H_in, int W_in, long pitch,
+                                                           int accumulate) {
+    const long per_img = (long)C * H_in * W_in;
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= per_img) return;
+    const int b = blockIdx.y;
+    const int c = (int)(t / ((long)H_in * W_in));
+    const int h = (int)((t / W_in) % H_in), w = (int)(t % W_in);
+    const float* col = colT + ((long)b * C + c) * K_h * K_w * pitch;
+    float acc = accumulate ? dx[(long)b * per_img + t] : 0.f;
+    const int ho_lo = h + pad - K_h + 1 > 0 ? (h + pad - K_h + 1 + stride - 1) / stride : 0;
+    const int ho_hi = (h + pad) / stride < H_out - 1 ? (h + pad) / stride : H_out - 1;
+    const int wo_lo = w + pad - K_w + 1 > 0 ? (w + pad - K_w + 1 + stride - 1) / stride : 0;
+    const int wo_hi = (w + pad) / stride < W_out - 1 ? (w + pad) / stride : W_out - 1;
+    for (int ho = ho_lo; ho <= ho_hi; ho++) {
+        const int r = h + pad - ho * stride;
+        for (int wo = wo_lo; wo <= wo_hi; wo++) {
+            const int sx = w + pad - wo * stride;
+            acc += col[(long)(r * K_w + sx) * pitch + (long)ho * W_out + wo];
+        }
+    }
+    dx[(long)b * per_img + t] = acc;
+}
+}  // namespace nzhip
+
+// The reference's own chain for the data gradient (src/Nodes.cu:660-665, 169-182, 632-640) inside the library, with the
+// column gradient transposed: per image colT[(c, r, s)][pixel] = W [(c, r, s)][o] x dy[o][pixel] is a product on dy as
+// it lies (no pixel-major copy of dy, no mirrored weights), and the gather into the image reads it along the pixels.
+// Every entry is the same sum over o as in the reference's dC x B^T, and they are added into dx in the same order.
+static int conv_dx_chain_planes(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H, size_t W, size_t O, size_t K_h,
+                                size_t K_w, size_t stride, size_t pad, size_t Ho, size_t Wo, size_t w_batch, int accumulate, void* stream) {
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const size_t P = Ho * Wo, Pp = (P + 3) / 4 * 4, CKK = C * K_h * K_w;
+    if ((C * H * W + 255) / 256 > 0x7fffffffull) return set_error(NZHIP_E_UNSUPPORTED, "nzhip_conv2d_backward_data: image beyond the gather kernel's grid");
+    float* colT = nullptr;
+    float* dy_wide = nullptr;
+    if (int rc = workspace_alloc(reinterpret_cast<void**>(&colT), N * CKK * Pp * sizeof(float), s)) return rc;
+    int rc = NZHIP_OK;
+    if (P % 4 != 0) rc = widen_rows(&dy_wide, dy, N * O, P, s);       // planes of whole 16-byte pieces for the product's loads
+    if (rc == NZHIP_OK) {
+        nzhip_gemm_desc g = {};
+        g.A = w_ref; g.M = (int64_t)CKK; g.K = (int64_t)O; g.lda = (int64_t)O; g.a_layout = NZHIP_LAYOUT_ROW;   // w_ref holds CKK x O
+        g.B = dy_wide ? dy_wide : dy; g.N = (int64_t)P; g.ldb = (int64_t)(dy_wide ? Pp : P); g.b_layout = NZHIP_LAYOUT_ROW;
+        g.C = colT; g.ldc = (int64_t)Pp;
+        g.batch_n = (int64_t)N; g.batch_c = 1;
+        g.a_stride_n = w_batch > 1 ? (int64_t)(CKK * O) : 0; g.b_stride_n = (int64_t)(O * (dy_wide ? Pp : P)); g.c_stride_n = (int64_t)(CKK * Pp);
+        g.activation = NZHIP_ACT_NONE;
+        rc = dy_wide ? gemm_padded_rows(g, 2, s) : nzhip_gemm(&g, s);
+    }
+    if (rc == NZHIP_OK) {
+        hipLaunchKernelGGL(col_t_gather_kernel, dim3((unsigned)((C * H * W + 255) / 256), (unsigned)N), dim3(256), 0, s, dx, colT, (int)Ho,
+                           (int)Wo, (int)C, (int)K_h, (int)K_w, (int)stride, (int)pad, (int)H, (int)W, (long)Pp, accumulate ? 1 : 0);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = set_hip_error(e, "col_t_gather kernel launch");
+    }
+    const int rc2 = dy_wide ? workspace_free(dy_wide, s) : NZHIP_OK;
+    const int rc3 = workspace_free(colT, s);
+    return rc ? rc : (rc2 ? rc2 : rc3);
+}
+
+// The reference's own chain for the data gradient (src/Nodes.cu:660-665, 169-182, 632-640) inside the library, in the
+// reference's layouts: the output gradient pixel-major, the column gradient = dy^T x W^T as ONE product with all images
+// as its rows, then the gather into the image. For images of fewer than 64 output pixels with shared weights: a product
+// per image would read the weights once per image for a handful of columns (16 x 512 x 7 x 7 <- 512: 40 against 52 us).
+static int conv_dx_chain_rows(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H, size_t W, size_t O, size_t K_h,
                          size_t K_w, size_t stride, size_t pad, size_t Ho, size_t Wo, size_t w_batch, int accumulate, void* stream) {
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const size_t P = Ho * Wo, CKK = C * K_h * K_w;
@@ -3087,6 +3155,13 @@ static int conv_dx_chain(float* dx, const float* dy, const float* w_ref, size_t 
     if (rc == NZHIP_OK) rc = nzhip_im2col_backward(dx, dcol, Ho, Wo, C, K_h, K_w, stride, pad, H, W, N, stream);
     const int rc2 = workspace_free(dcol, s), rc3 = workspace_free(dyt, s);
     return rc ? rc : (rc2 ? rc2 : rc3);
+}
+
+static int conv_dx_chain(float* dx, const float* dy, const float* w_ref, size_t N, size_t C, size_t H, size_t W, size_t O, size_t K_h,
+                         size_t K_w, size_t stride, size_t pad, size_t Ho, size_t Wo, size_t w_batch, int accumulate, void* stream) {
+    if (w_batch == 1 && Ho * Wo < 64)
+        return conv_dx_chain_rows(dx, dy, w_ref, N, C, H, W, O, K_h, K_w, stride, pad, Ho, Wo, w_batch, accumulate, stream);
+    return conv_dx_chain_planes(dx, dy, w_ref, N, C, H, W, O, K_h, K_w, stride, pad, Ho, Wo, w_batch, accumulate, stream);
 }
 
 /* Gradient of nzhip_conv2d_forward with respect to x: one convolution of dy with the
@@ -3147,24 +3222,28 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
     if (stride > 1) {
         const size_t Ho = (H + 2 * pad - K_h) / stride + 1, Wo = (W + 2 * pad - K_w) / stride + 1;
         // The convolution of the zero-filled gradient does stride^2 times the multiply-adds; the reference's own chain
-        // (src/Nodes.cu:660-665, 169-182, 632-640: column gradient = dy^T x W^T, then the gather into the image) does them
+        // (src/Nodes.cu:660-665, 169-182, 632-640: column gradient = W x dy, then the gather into the image) does them
         // once but writes and reads the column gradient. Many channels on small images favour the chain (16 x 512 x 14 x 14
-        // <- 512 at stride 2: 103 against 45 us), few channels on large images the convolution (16 x 64 x 128 x 128 <- 128:
-        // 101 against 269). The estimate: both sides at the rates measured for them (flops: resident / streamed weights,
-        // the product of the chain; bytes: the zero-filled gradient, three passes over the column gradient), the
-        // convolution favoured up to 1.5 x because its measured side came out better than estimated on every shape tried.
+        // <- 512 at stride 2: 42 against 71 us; 16 x 192 x 17 x 17 <- 192: 19 against 51), few channels on large images the
+        // convolution (16 x 64 x 128 x 128 <- 128: 88 against 163). The estimate, in us, from the rates measured for both
+        // sides on thirteen layers: the convolution at 600 (resident weights) or 300 TFLOP/s, half again as slow when the
+        // zero-filled rows are not whole 16-byte pieces, plus the zero-filled gradient at 5 TB/s and 15-25 us for its four
+        // launches; the chain's product at 500 TFLOP/s plus the column gradient (written, then gathered) at 1.1 TB/s and
+        // 10 us for its launches.
         static const char* dx_env = getenv("NZHIP_CONV_DX");              // benchmarking only: "chain" | "conv"
         const double flops = 2.0 * N * Ho * Wo * C * K_h * K_w * O;
         const bool resident = ((O + 15) / 16) * (C > 64 ? 128 : 64) * K_h * K_w * 32 <= 148 * 1024;
         const double hu = (double)(H + 2 * pad - K_h + 1), wu = (double)(W + 2 * pad - K_w + 1);
+        const bool pieces = (W + 2 * pad - K_w + 1) % 4 == 0;
         // (the convolution's output channels are the C input channels here, in tiles of 64: with 3 of them it multiplies
-        // mostly padding, 16 x 3 x 224 x 224 <- 64 at 7x7 stride 2: 630 against 208 us)
+        // mostly padding, 16 x 3 x 224 x 224 <- 64 at 7x7 stride 2: 605 against 99 us)
         const double tile_fill = (double)((C + 63) / 64 * 64) / (double)C;
-        const double as_conv = stride * stride * flops * tile_fill / (resident ? 600e6 : 300e6) + N * O * hu * wu * 4.0 / 5e6;
-        const double as_chain = flops / 400e6 + 3.0 * N * Ho * Wo * C * K_h * K_w * 4.0 / 4e6;
+        const double as_conv = stride * stride * flops * tile_fill * (pieces ? 1.0 : 1.5) / (resident ? 600e6 : 300e6) +
+                               N * O * hu * wu * 4.0 / 5e6 + (pieces ? 15.0 : 25.0);
+        const double as_chain = 10.0 + flops / 500e6 + (double)N * Ho * Wo * C * K_h * K_w * 4.0 / 1.1e6;
         const size_t P = Ho * Wo, CKK = C * K_h * K_w;
         const bool chain_fits = N * P < 0x3fffffff && CKK < 0x3fffffff && O < 0x3fffffff && N <= 65535 && P * O < 0x7fffffffull;
-        if (chain_fits && (dx_env ? dx_env[1] == 'h' : as_conv >= 1.5 * as_chain))
+        if (chain_fits && (dx_env && dx_env[0] ? dx_env[1] == 'h' : as_conv >= as_chain))
             return conv_dx_chain(dx, dy, w_ref, N, C, H, W, O, K_h, K_w, stride, pad, Ho, Wo, w_batch, accumulate, stream);
         const size_t Hu = H + 2 * pad - K_h + 1, Wu = W + 2 * pad - K_w + 1, total = N * O * Hu * Wu;
         if (Hu > 0x3fffffff || Wu > 0x3fffffff)
@@ -3194,7 +3273,7 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
         const bool chain_fits = N * P < 0x3fffffff && CKK < 0x3fffffff && O < 0x3fffffff && N <= 65535 && P * O < 0x7fffffffull &&
                                 N * P * CKK <= ((size_t)1 << 28);
         const bool column_route = route != CONV_ROUTE_FIXED && route != CONV_ROUTE_ANY && route != CONV_ROUTE_DIRECT;
-        if (chain_fits && (dx_env ? dx_env[1] == 'h' : column_route))
+        if (chain_fits && (dx_env && dx_env[0] ? dx_env[1] == 'h' : column_route))
             return conv_dx_chain(dx, dy, w_ref, N, C, H, W, O, K_h, K_w, 1, pad, H_out, W_out, w_batch, accumulate, stream);
     }
     const bool in_place = accumulate && (route == CONV_ROUTE_FIXED || route == CONV_ROUTE_ANY);
