@@ -3474,6 +3474,8 @@ struct ConvDwGenArgs {
     int span;              // staged input rows per channel: (128 / SW - 1) * stride + Kh
     int bands, band_rows, n_images;
     int ipw, n_groups;     // images per workgroup and groups of that many images (partial sums: one region per group and band)
+    float* dw_direct;      // not null: one workgroup per (image, tile) and per-sample weights -- its sums are the whole
+    long dw_stride;        // gradient of that tile, added straight into dW[image] (dw_stride floats apart), no partial sums
 };
 
 // Eight waves: a workgroup owns up to 256 rows (channel, tap) x 128 output channels, and the requests for the NEXT
@@ -3671,6 +3673,30 @@ __global__ __launch_bounds__(DWG8_THREADS) void conv_dwg8_kernel(const ConvDwGen
         __syncthreads();
     }
     // accumulator (block j, register r): row 32 wave + (r >> 2) * 8 + lh * 4 + (r & 3), column 32 j + li
+    if (p.dw_direct) {
+        float* dst = p.dw_direct + (long)group * p.dw_stride + (long)c0 * taps * p.O + o0;
+        if (wave_live) {
+            // all of a column block's old values requested before the first is added and stored (a store might alias
+            // a later load as far as the compiler knows, which would put one memory round trip behind the other)
+#pragma unroll
+            for (int j = 0; j < DWG_NB; j++) {
+                const int col = j * 32 + li;
+                float old[16];
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = wave * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    const bool ok = row < nch * taps && o0 + col < p.O;
+                    old[r] = ok ? dst[(long)row * p.O + col] : 0.f;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = wave * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    if (row < nch * taps && o0 + col < p.O) dst[(long)row * p.O + col] = old[r] + acc[j][r];
+                }
+            }
+        }
+        return;
+    }
     float* out = p.partial + ((((long)blockIdx.y * gridDim.z + blockIdx.z) * p.n_groups + group) * p.bands + band) * (DWG8_ROWS * DWG_OT);
     if (wave_live) {
 #pragma unroll
@@ -3760,6 +3786,12 @@ static int conv_dw_generic_run(float* dw, const float* x, const float* dy, size_
     const double region_cost = 0.011;
     double best = 0.0;
     int bands = dwg_pick_bands(tiles * (long)N, resident, row_steps, segs, 3.0, region_cost, &best), ipw = 1;
+    if (!shared && bands > 1) {
+        // one band per image needs no partial sums and no reduction at all (below): its cost without those
+        const long units = tiles * (long)N;
+        const double one = (double)((units + resident - 1) / resident) * ((double)row_steps * (double)segs + 3.0) - 1.7;
+        if (one <= best) bands = 1;
+    }
     if (shared && N > 1) {
         for (long g = 2; g <= (long)N && g <= 64; g++) {
             const long groups = ((long)N + g - 1) / g;
@@ -3774,10 +3806,16 @@ static int conv_dw_generic_run(float* dw, const float* x, const float* dy, size_
     const int n_groups = (int)((N + ipw - 1) / ipw);
     if ((size_t)n_groups * (size_t)bands > 0x7fffffffull) return NZHIP_E_UNSUPPORTED;
     const size_t regions = (size_t)chunks * otiles * n_groups * bands;
+    // Per-sample weights and one workgroup per (image, tile): its sums are that tile's whole gradient and go straight
+    // into dW[image] -- no partial sums written and read back (16 x 512 x 7 x 7 -> 512 with a weight copy per image: 302 MB
+    // of dW traffic instead of 604 MB).
+    const bool direct = !shared && bands == 1 && ipw == 1;
     float* partial = nullptr;
-    if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), regions * DWG8_ROWS * DWG_OT * sizeof(float), s)) return rc;
+    if (!direct)
+        if (int rc = workspace_alloc(reinterpret_cast<void**>(&partial), regions * DWG8_ROWS * DWG_OT * sizeof(float), s)) return rc;
     ConvDwGenArgs a;
     a.x = x; a.dy = dy; a.partial = partial;
+    a.dw_direct = direct ? dw : nullptr; a.dw_stride = (long)(C * taps * O);
     a.C = (int)C; a.H = (int)H; a.W = (int)W; a.O = (int)O; a.Ho = (int)Ho; a.Wo = (int)Wo;
     a.Kh = (int)K_h; a.Kw = (int)K_w; a.stride = (int)stride; a.pad = (int)pad;
     a.cc = cc; a.pw = pw; a.shift = shift; a.sw_log = sw_log; a.span = span; a.bands = bands; a.band_rows = band_rows; a.n_images = (int)N;
@@ -3795,7 +3833,7 @@ static int conv_dw_generic_run(float* dw, const float* x, const float* dy, size_
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg kernel launch");
     }
-    if (rc == NZHIP_OK) {
+    if (rc == NZHIP_OK && !direct) {
         const int S = shared ? n_groups * bands : bands, groups = shared ? 1 : (int)N;
         const long per_group = (long)S * DWG8_ROWS * DWG_OT;
         // partial regions of one (chunk, o_tile) are contiguous: [image group][band]; a weight copy's regions start at b * S
@@ -3805,7 +3843,7 @@ static int conv_dw_generic_run(float* dw, const float* x, const float* dy, size_
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) rc = set_hip_error(e, "conv_dwg_reduce kernel launch");
     }
-    const int rc2 = workspace_free(partial, s);
+    const int rc2 = partial ? workspace_free(partial, s) : NZHIP_OK;
     return rc ? rc : rc2;
 }
 
