@@ -2854,6 +2854,13 @@ static ConvRoute conv_forward_route(const float* x, size_t N, size_t C, size_t H
     if (conv_direct_applicable(C, O, K_h, K_w, stride, pad)) return CONV_ROUTE_DIRECT;
     const bool force_ws = route_env && route_env[0] == 'w', force_gen = route_env && route_env[0] == 'g';
     if (force_ws) return CONV_ROUTE_WORKSPACE;
+    // One weight copy per image, each used for a single small image: the fp16 image the implicit-GEMM kernels want costs a
+    // pass over all copies (read fp32, write fp16, read fp16 again) for weights the column-matrix product reads once as they
+    // lie. Cheaper whenever the column matrix is smaller than the weights, output pixels x 2 <= output channels
+    // (16 x 512 x 14 x 14 -> 512, 151 MB of weights: 103 against 130 us; the data gradient 83 against 133), unless the caller
+    // keeps the image across calls.
+    if (w_batch > 1 && !force_gen && K_h * K_w > 1 && H_out * W_out * 2 <= O && !image_kept_by_caller(PREPARED_CONV_W))
+        return CONV_ROUTE_WORKSPACE;
     const bool fixed_ok = conv_igemm_applicable(C, O, K_h, K_w, stride, pad, N) && (long)H * W < 0x7fffffffL;
     // Small images with many channels: the weights do not fit LDS, so the implicit-GEMM kernel runs one
     // patch per workgroup with the whole C x taps contraction inside, and there are too few patches to

@@ -70,6 +70,8 @@ struct ImageLease {
     void* owner = nullptr;      // that handle
 };
 int image_acquire(int kind, const uint64_t key[PREPARED_KEY_WORDS], size_t bytes, hipStream_t s, ImageLease* out);
+// True while a *_prepared entry point of this kind is on the calling thread's stack with a handle: an image built now is kept.
+bool image_kept_by_caller(int kind);
 // `enqueued`: every launch between acquire and release went through. A handle whose image was to be rebuilt under this
 // lease is only then marked as holding it; otherwise the next call rebuilds.
 int image_release(const ImageLease& lease, hipStream_t s, bool enqueued);

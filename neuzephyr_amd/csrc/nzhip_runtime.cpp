@@ -157,6 +157,8 @@ struct PreparedScope {
 };
 static thread_local PreparedScope t_prepared;
 
+bool image_kept_by_caller(int kind) { return t_prepared.handle && t_prepared.kind == kind && !t_arena.active; }
+
 int image_acquire(int kind, const uint64_t key[PREPARED_KEY_WORDS], size_t bytes, hipStream_t s, ImageLease* out) {
     nzhip_prepared* h = (t_prepared.handle && t_prepared.kind == kind && !t_arena.active) ? t_prepared.handle : nullptr;
     if (!h) {
