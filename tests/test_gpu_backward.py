@@ -222,7 +222,9 @@ CONV_BWD_DATA = [  # N, C, H, W, O, K, pad, w_batch
     (2, 16, 20, 36, 24, 3, 1, 1), (1, 64, 32, 64, 128, 3, 1, 1), (3, 8, 17, 33, 70, 3, 1, 3), (2, 40, 9, 70, 12, 1, 0, 1),
     (1, 3, 40, 40, 1, 3, 1, 1), (2, 1, 12, 16, 2, 3, 1, 1),
     (3, 20, 9, 10, 33, 1, 0, 3), (4, 256, 14, 14, 300, 1, 0, 1),            # 1x1: one batched product (per-sample weights; many channels)
-    (4, 300, 14, 14, 64, 3, 1, 1), (16, 256, 7, 7, 40, 3, 1, 1), (2, 96, 28, 28, 160, 3, 1, 1)]   # deep layers on small images: accumulation in place on the any-geometry kernel, or through a temporary
+    (4, 300, 14, 14, 64, 3, 1, 1), (16, 256, 7, 7, 40, 3, 1, 1), (2, 96, 28, 28, 160, 3, 1, 1),   # deep layers on small images: accumulation in place on the any-geometry kernel, or through a temporary
+    (3, 80, 6, 6, 20, 3, 1, 3), (4, 130, 5, 7, 33, 5, 2, 4),            # per-sample weights larger than the column gradient: the chain on dy as it lies (planes of 36 and 35 pixels)
+    (16, 64, 7, 7, 64, 3, 1, 1), (5, 70, 4, 4, 90, 3, 1, 1)]             # tiny images, shared weights: the chain with all images as rows of one product
 
 
 @pytest.mark.parametrize("N,C,H,W,O,K,pad,wb", CONV_BWD_DATA)

@@ -85,13 +85,15 @@ CONV_CASES = [
     (1, 70, 9, 9, 130, 1, 1, 1, 0, 1),
     (2, 130, 9, 12, 70, 1, 1, 1, 0, 1),     # 1x1 with 128 or more input channels: one batched product
     (2, 160, 8, 8, 40, 1, 1, 1, 0, 2),      # ... with per-sample weights
-    (2, 200, 5, 5, 16, 1, 1, 1, 0, 1),      # ... tiny images and fewer outputs than inputs: the convolution kernels again
+    (2, 200, 5, 5, 16, 1, 1, 1, 0, 1),      # ... tiny images and fewer outputs than inputs: a product as well
     (2, 24, 9, 11, 40, 1, 1, 2, 0, 1),      # 1x1 with a stride: every second pixel gathered, then the 1x1 stride-1 kernels
     (3, 130, 7, 13, 20, 1, 1, 3, 0, 3),     # ... stride 3, odd extents, per-sample weights, as a batched product
     (2, 24, 40, 70, 9, 3, 3, 1, 0, 1),      # no padding, ragged width (scalar staging path)
     (1, 9, 33, 36, 140, 3, 3, 1, 2, 1),     # padding 2: both halo columns on the left
     (2, 20, 16, 64, 64, 3, 3, 1, 1, 2),     # per-sample weights
     (1, 16, 12, 40, 8, 3, 3, 1, 3, 1),      # padding larger than the kernel reach: workspace route
+    (3, 20, 6, 6, 80, 3, 3, 1, 1, 3),       # per-sample weights, output pixels x 2 <= output channels: the column matrix instead of a weight image per copy
+    (4, 33, 5, 7, 130, 5, 5, 1, 2, 4),      # ... 5x5, two channel tiles' worth of outputs
     # resident weights with two halo buffers (64 channels -> 128-channel tile, 128 -> 64-channel tile, 64-wide patches)
     (1, 64, 9, 64, 128, 3, 3, 1, 1, 1),     # rows not a multiple of the 4-row patch
     (2, 50, 12, 72, 100, 3, 3, 1, 1, 1),    # last chunk with 2 of 16 channels, part of a channel tile, ragged second patch
