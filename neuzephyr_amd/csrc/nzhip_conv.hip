@@ -3249,7 +3249,8 @@ extern "C" int nzhip_conv2d_backward_data(float* dx, const float* dy, const floa
                                N * O * hu * wu * 4.0 / 5e6 + (pieces ? 15.0 : 25.0);
         const double as_chain = 10.0 + flops / 500e6 + (double)N * Ho * Wo * C * K_h * K_w * 4.0 / 1.1e6;
         const size_t P = Ho * Wo, CKK = C * K_h * K_w;
-        const bool chain_fits = N * P < 0x3fffffff && CKK < 0x3fffffff && O < 0x3fffffff && N <= 65535 && P * O < 0x7fffffffull;
+        const bool chain_fits = N * P < 0x3fffffff && CKK < 0x3fffffff && O < 0x3fffffff && N <= 65535 && P * O < 0x7fffffffull &&
+                                N * P * CKK <= ((size_t)1 << 29);      // a column gradient of at most 2 GiB
         if (chain_fits && (dx_env && dx_env[0] ? dx_env[1] == 'h' : as_conv >= as_chain))
             return conv_dx_chain(dx, dy, w_ref, N, C, H, W, O, K_h, K_w, stride, pad, Ho, Wo, w_batch, accumulate, stream);
         const size_t Hu = H + 2 * pad - K_h + 1, Wu = W + 2 * pad - K_w + 1, total = N * O * Hu * Wu;
