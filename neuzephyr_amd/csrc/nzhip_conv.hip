@@ -542,10 +542,27 @@ struct IgemmArgs {
     long bias_sp, bias_sc, bias_sn;   // bias element of (image b, pixel, channel o): bias[b*bias_sn + pixel*bias_sp + o*bias_sc]
     int relu;
     int patch_map;                    // resident kernels: 0 strided by the grid, 1 XCD-contiguous, 2 XCD-contiguous runs,
-                                      // 3 image-major (per-sample weights: every workgroup stays inside one image)
+                                      // 3 image-major (per-sample weights: every workgroup stays inside one image);
+                                      // 4, 5: 1 and 3 with every XCD on the same eighth of ALL images (a per-pixel bias
+                                      // shared by the images is then read once per XCD instead of once per image)
     int n_images;                     // patch_map 3: images of the batch (the grid is a multiple of it wide)
     long w_image_bytes;               // patch_map 3: bytes from one image's weight image to the next
 };
+
+// Image b and place r (tile index inside the image) of a patch index. Under patch_map 4 the index runs over (eighth of
+// the image, image, place inside the eighth), so that the contiguous range of an XCD is one eighth of every image.
+__device__ __forceinline__ void patch_image_and_place(const IgemmArgs& p, int patch, int patches_per_image, int& b, int& r) {
+    if (p.patch_map == 4) {
+        const int s = patches_per_image >> 3;
+        const int blk = patch / s, q = patch - blk * s;
+        const int e = blk / p.n_images;
+        b = blk - e * p.n_images;
+        r = e * s + q;
+    } else {
+        b = patch / patches_per_image;
+        r = patch - b * patches_per_image;
+    }
+}
 
 // Patches of a workgroup of the resident kernels under patch_map 3, for the reference's Conv2d parameter with one
 // weight copy per sample (src/Model.cu:248-252): the grid's G workgroups are split evenly over the images (G / n_images
@@ -554,8 +571,20 @@ struct IgemmArgs {
 __device__ __forceinline__ void image_major_patches(const IgemmArgs& p, int patches_per_image, int& image, int& first_patch,
                                                     int& patch_stride, int& my_patches) {
     const int G = gridDim.x;
-    const int u = (G % 8 == 0) ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
     const int wpi = G / p.n_images;
+    if (p.patch_map == 5) {
+        // (the host checked: G, wpi and patches_per_image are multiples of 8) XCD e holds wpi / 8 workgroups of every
+        // image, and they walk the e-th eighth of that image's patches: the eighth of a per-pixel bias that those
+        // patches read is the same for all images and stays in the XCD's L2
+        const int e = blockIdx.x & 7, slot = blockIdx.x >> 3, wpx = wpi >> 3, s = patches_per_image >> 3;
+        image = slot / wpx;
+        const int k = slot - image * wpx;
+        first_patch = image * patches_per_image + e * s + k;
+        patch_stride = wpx;
+        my_patches = k < s ? (s - k + wpx - 1) / wpx : 0;
+        return;
+    }
+    const int u = (G % 8 == 0) ? (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
     image = u / wpi;
     const int j = u - image * wpi;
     first_patch = image * patches_per_image + j;
@@ -834,7 +863,7 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
 
     int w_image = 0, first_patch = blockIdx.x, patch_stride = gridDim.x;
     int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-    if (p.patch_map == 3) image_major_patches(p, patches_per_image, w_image, first_patch, patch_stride, my_patches);
+    if (p.patch_map == 3 || p.patch_map == 5) image_major_patches(p, patches_per_image, w_image, first_patch, patch_stride, my_patches);
 
     // resident weights: n_chunks * W_CHUNK bytes, 1 KiB per wave-wide request
     {
@@ -877,10 +906,10 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     // is a multiple of 8 wide) the workgroups of one XCD share a contiguous eighth of the patches: halo
     // rows and columns that neighbouring patches have in common are then found in that L2 instead of
     // being fetched again from memory.
-    if (p.patch_map != 0 && p.patch_map != 3 && gridDim.x % 8 == 0) {
+    if (p.patch_map != 0 && p.patch_map != 3 && p.patch_map != 5 && gridDim.x % 8 == 0) {
         const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3, nq = gridDim.x >> 3;
         const int lo = (int)((long)n_patches * xcd / 8), hi = (int)((long)n_patches * (xcd + 1) / 8);
-        if (p.patch_map == 1) {                                  // the XCD's workgroups sweep its range side by side
+        if (p.patch_map == 1 || p.patch_map == 4) {              // the XCD's workgroups sweep its range side by side
             first_patch = lo + q;
             patch_stride = nq;
             my_patches = q < hi - lo ? (hi - lo - q + nq - 1) / nq : 0;
@@ -919,7 +948,8 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
         if (ld_chunk == 0) {                                     // new patch: redo the geometry (uniform branch)
             const bool live = ld_it < total;
             const int patch = live ? ld_patch : 0;
-            const int b = patch / patches_per_image, r = patch % patches_per_image;
+            int b, r;
+            patch_image_and_place(p, patch, patches_per_image, b, r);
             const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
             ld_hin = th0 + t_hh - p.pad;
             ld_win = tw0 + t_ww - p.pad;
@@ -1057,7 +1087,8 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
     // The per-pixel bias of unit (j, i), requested one unit ahead of its use (the first unit's at the start of the
     // patch): a request issued after a unit's stores would not be counted as returned before those stores are.
     auto bias_request = [&](float (&bv)[16], const int j, const int i, const int patch) {
-        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        int b, r;
+            patch_image_and_place(p, patch, patches_per_image, b, r);
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
         const int blk = wm * FP + j;
         const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
@@ -1071,7 +1102,8 @@ __global__ __launch_bounds__(512) void conv_igemm_resident_kernel(const IgemmArg
         }
     };
     auto flush_unit = [&](const int j, const int i, const int patch, const float (&bv)[16]) {
-        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        int b, r;
+            patch_image_and_place(p, patch, patches_per_image, b, r);
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
         const int blk = wm * FP + j;
         const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
@@ -1222,7 +1254,7 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
 
     int w_image = 0, first_patch = blockIdx.x, patch_stride = gridDim.x;
     int my_patches = (n_patches - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x;
-    if (p.patch_map == 3) image_major_patches(p, patches_per_image, w_image, first_patch, patch_stride, my_patches);
+    if (p.patch_map == 3 || p.patch_map == 5) image_major_patches(p, patches_per_image, w_image, first_patch, patch_stride, my_patches);
 
     const char* wtile = reinterpret_cast<const char*>(p.wimg) + (long)w_image * p.w_image_bytes + (long)o_tile * NCH * BN * 288;
     {
@@ -1268,7 +1300,7 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
         return hb + (t_q4 >> 1) * H_PLANE + (hh * G::WW + ww) * 16 + (t_q4 & 1) * 8;
     };
 
-    if (p.patch_map != 0 && p.patch_map != 3 && gridDim.x % 8 == 0) {   // the workgroups of an XCD sweep a contiguous eighth
+    if (p.patch_map != 0 && p.patch_map != 3 && p.patch_map != 5 && gridDim.x % 8 == 0) {   // the workgroups of an XCD sweep a contiguous eighth
         const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3, nq = gridDim.x >> 3;
         const int lo = (int)((long)n_patches * xcd / 8), hi = (int)((long)n_patches * (xcd + 1) / 8);
         first_patch = lo + q;
@@ -1291,7 +1323,8 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
         if (ld_chunk == 0) {
             const bool live = ld_it < total;
             const int patch = live ? ld_patch : 0;
-            const int b = patch / patches_per_image, r = patch % patches_per_image;
+            int b, r;
+            patch_image_and_place(p, patch, patches_per_image, b, r);
             const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
             ld_hin = th0 + t_hh - p.pad;
             ld_win = tw0 + t_ww - p.pad;
@@ -1398,7 +1431,8 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
     // The per-pixel bias of unit (j, i), requested one unit ahead of its use (the first unit's at the start of the
     // patch): a request issued after a unit's stores would not be counted as returned before those stores are.
     auto bias_request = [&](float (&bv)[16], const int j, const int i, const int patch) {
-        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        int b, r;
+            patch_image_and_place(p, patch, patches_per_image, b, r);
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
         const int blk = wm * FP + j;
         const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
@@ -1412,7 +1446,8 @@ __global__ __launch_bounds__(512) void conv3x3_resident_db_kernel(const IgemmArg
         }
     };
     auto flush_unit = [&](const int j, const int i, const int patch, const float (&bv)[16]) {
-        const int b = patch / patches_per_image, r = patch % patches_per_image;
+        int b, r;
+            patch_image_and_place(p, patch, patches_per_image, b, r);
         const int th0 = (r / p.tiles_w) * G::TH, tw0 = (r % p.tiles_w) * TW;
         const int blk = wm * FP + j;
         const int ho = th0 + blk / CB, wo = tw0 + (blk % CB) * 32 + li;
@@ -1523,6 +1558,19 @@ static int resident_grid_per_sample(size_t N, int n_otiles) {
     return (int)(per_tile / (int)N * (int)N);
 }
 
+// A per-pixel bias that all images share (the reference's Bias node after the product, src/Model.cu:252-256) is read by
+// every patch of every image: 16 x 64 x 128 x 128 -> 128 reads its 8 MB sixteen times. With every XCD on the same eighth
+// of all images, that eighth stays in the XCD's L2 (patch maps 4 and 5 in place of 1 and 3; the grid, the workgroups
+// per image and the patches per image have to be multiples of 8).
+static int resident_patch_map(int map, const float* bias, int64_t bias_sp, int64_t bias_sn, int grid_x, size_t N, size_t patches_per_image) {
+    static const char* env = getenv("NZHIP_CONV_BIAS_MAP");          // benchmarking only: 0 keeps maps 1 and 3
+    if (env && atoi(env) == 0) return map;
+    if (!bias || bias_sp == 0 || bias_sn != 0 || N < 2 || grid_x % 8 != 0 || patches_per_image % 8 != 0) return map;
+    if (map == 1) return 4;
+    if (map == 3 && grid_x % (int)N == 0 && (grid_x / (int)N) % 8 == 0) return 5;
+    return map;
+}
+
 // Key of a weight image: everything the conversion kernel's output depends on (image kind, tile shape, source and extents).
 static void conv_image_key(uint64_t (&key)[PREPARED_KEY_WORDS], int kind, int kh, int kw, int bn, const float* w_ref, size_t C,
                            size_t O, int n_chunks, int n_otiles, size_t w_batch, bool w_mirror) {
@@ -1586,6 +1634,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                     int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
                     if ((long)per_tile > n_patches) per_tile = (int)n_patches;
                     if (w_batch > 1) per_tile = grid_ps;                          // a whole number of workgroups per image
+                    a.patch_map = resident_patch_map(a.patch_map, bias, bias_sp, bias_sn, per_tile, N, (size_t)a.tiles_w * a.tiles_h);
                     hipLaunchKernelGGL(kdb, dim3((unsigned)per_tile, (unsigned)n_otiles, 1), dim3(512), lds_need, s, a, (int)n_patches);
                     hipError_t e = hipGetLastError();
                     if (e != hipSuccess) rc = set_hip_error(e, "conv3x3_resident_db kernel launch");
@@ -1643,6 +1692,7 @@ static int conv_igemm_launch(float* y, const float* x, const float* w_ref, const
                 int per_tile = cus / n_otiles > 0 ? cus / n_otiles : 1;      // one workgroup per CU in total
                 if ((long)per_tile > n_patches) per_tile = (int)n_patches;
                 if (w_batch > 1) per_tile = grid_ps;                          // a whole number of workgroups per image
+                a.patch_map = resident_patch_map(a.patch_map, bias, bias_sp, bias_sn, per_tile, N, (size_t)a.tiles_w * a.tiles_h);
                 dim3 grid((unsigned)per_tile, (unsigned)n_otiles, 1);
                 hipLaunchKernelGGL(kres, grid, dim3(512), lds_need, s, a, (int)n_patches);
                 hipError_t e = hipGetLastError();
