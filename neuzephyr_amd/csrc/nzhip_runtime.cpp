@@ -315,6 +315,15 @@ int nzhip_host_free(void* ptr) {
 
 int nzhip_memset(void* ptr, int value, size_t bytes) {
     if (!ptr && bytes) return set_error(NZHIP_E_INVALID, "nzhip_memset: null pointer");
+    // whole fp32 words of one byte value (clearing gradients, the usual case) go through the library's own fill kernel:
+    // a kernel node like any other for a caller that records the stream, where a memset node is a kind of its own
+    if (bytes % 4 == 0 && (reinterpret_cast<uintptr_t>(ptr) & 3) == 0) {
+        const unsigned word = 0x01010101u * (unsigned)(value & 0xff);
+        float as_float;
+        memcpy(&as_float, &word, sizeof(as_float));
+        if (bytes == 0) return NZHIP_OK;
+        return nzhip_fill(static_cast<float*>(ptr), as_float, bytes / 4, Runtime::instance().stream());
+    }
     hipError_t e = hipMemsetAsync(ptr, value, bytes, Runtime::instance().stream());
     return e == hipSuccess ? NZHIP_OK : set_hip_error(e, "hipMemsetAsync");
 }

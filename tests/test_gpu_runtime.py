@@ -65,6 +65,25 @@ def test_product_on_a_second_stream_then_free_and_reissue_through_the_runtime(nz
     nz.check(lib.nzhip_stream_wait(None))
 
 
+def test_memset_writes_the_byte_value_for_word_and_odd_sizes(nz):
+    # whole fp32 words go through the library's fill kernel (the byte repeated four times as one bit pattern, NaN patterns
+    # included), anything else through the runtime's memset; either way every byte of the range, and none beyond it
+    import ctypes as C
+    lib = nz.load()
+    for value, nbytes, offset in ((0x00, 4096, 0), (0xFF, 4096, 0), (0xAB, 4 * 1031, 0), (0x7F, 1001, 0), (0x3C, 64, 2)):
+        p = C.c_void_p()
+        nz.check(lib.nzhip_malloc(C.byref(p), nbytes + 64))
+        guard = np.full(nbytes + 64, 0x55, np.uint8)
+        nz.check(lib.nzhip_memcpy_h2d(p, guard.ctypes.data_as(C.c_void_p), guard.nbytes))
+        nz.check(lib.nzhip_memset(C.c_void_p(p.value + 16 + offset), value, nbytes))
+        got = np.empty_like(guard)
+        nz.check(lib.nzhip_memcpy_d2h(got.ctypes.data_as(C.c_void_p), p, got.nbytes))
+        want = guard.copy()
+        want[16 + offset:16 + offset + nbytes] = value
+        assert np.array_equal(got, want), (value, nbytes, offset)
+        nz.check(lib.nzhip_free_async(p))
+
+
 def test_pinned_host_operands(nz):
     # page-locked host memory is mapped into the device at the same address: the kernels take it as any operand
     # (the storage of nz::data::MappedTensor); host-memory result == device-memory result, bit for bit
