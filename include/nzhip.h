@@ -369,6 +369,10 @@ int nzhip_avgpool2d(float* out, const float* in, size_t pool, size_t stride, siz
  * serial run of that scatter. */
 int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches,
                              size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out, void* stream);
+/* The same with din = instead of din +=: din's old contents are not read. No counterpart in the reference; for the first
+ * writer of a gradient that would otherwise be cleared first and then read back as zeros. */
+int nzhip_avgpool2d_backward_overwrite(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches,
+                                       size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out, void* stream);
 
 /* BinaryCrossEntropyNode::forward (src/Nodes.cu:822-840; BinaryCrossEntropyKernel, src/OperationKernels.cu:648-685):
  * *loss (device memory) = sum_i (-t_i log p_i - (1 - t_i) log(1 - p_i)) / n with the fast hardware logarithm

@@ -22,7 +22,7 @@ EXPORTS = [
     "nzhip_gemm_backward", "nzhip_matmul_backward", "nzhip_relu_backward", "nzhip_add_backward",
     "nzhip_im2col_backward", "nzhip_col2im_backward", "nzhip_conv2d_backward_data", "nzhip_conv2d_backward_weights", "nzhip_conv2d_backward_bias", "nzhip_conv2d_backward_relu_bias", "nzhip_matmul_f32", "nzhip_sgd_step", "nzhip_adam_step", "nzhip_fill_many", "nzhip_sgd_step_many", "nzhip_adam_step_many",
     "nzhip_softmax", "nzhip_softmax_jacobian", "nzhip_softmax_backward",
-    "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_mse_loss", "nzhip_mse_backward", "nzhip_expand", "nzhip_compress",
+    "nzhip_avgpool2d", "nzhip_avgpool2d_backward", "nzhip_avgpool2d_backward_overwrite", "nzhip_bce_loss", "nzhip_bce_backward", "nzhip_mse_loss", "nzhip_mse_backward", "nzhip_expand", "nzhip_compress",
     "nzhip_default_stream", "nzhip_malloc", "nzhip_free_async", "nzhip_free", "nzhip_host_malloc", "nzhip_host_free", "nzhip_memset",
     "nzhip_memcpy_h2d", "nzhip_memcpy_d2d", "nzhip_memcpy_d2h", "nzhip_sync_ptr", "nzhip_stream_wait", "nzhip_sync_all",
     "nzhip_allocator_stats", "nzhip_allocator_trim",
@@ -110,6 +110,7 @@ def load() -> C.CDLL:
     lib.nzhip_conv2d_backward_relu_bias.argtypes = [vp, vp, vp, vp, sz, sz, sz, vp]
     lib.nzhip_avgpool2d.argtypes = [vp, vp] + [sz] * 9 + [vp]
     lib.nzhip_avgpool2d_backward.argtypes = [vp, vp] + [sz] * 9 + [vp]
+    lib.nzhip_avgpool2d_backward_overwrite.argtypes = [vp, vp] + [sz] * 9 + [vp]
     lib.nzhip_bce_loss.argtypes = [vp, vp, vp, sz, vp]
     lib.nzhip_bce_backward.argtypes = [vp, vp, vp, sz, vp]
     lib.nzhip_mse_loss.argtypes = [vp, vp, vp, sz, vp]
@@ -522,12 +523,12 @@ def avgpool2d(x, pool, stride, pad, stream=None):
     return out
 
 
-def avgpool2d_backward(dx, dy, pool, stride, pad, stream=None):
-    """dx += gradient of avgpool2d; dx has the input's shape, dy the output's."""
+def avgpool2d_backward(dx, dy, pool, stride, pad, stream=None, overwrite=False):
+    """dx += gradient of avgpool2d (overwrite: dx = it, dx's old contents are not read); dx has the input's shape, dy the output's."""
     lib = load()
     N, Cc, H, W = dx.shape
-    check(lib.nzhip_avgpool2d_backward(_dev(dx), _dev(dy), pool, stride, pad, N, Cc, H, W, dy.shape[2], dy.shape[3],
-                                       _stream_handle(stream)))
+    fn = lib.nzhip_avgpool2d_backward_overwrite if overwrite else lib.nzhip_avgpool2d_backward
+    check(fn(_dev(dx), _dev(dy), pool, stride, pad, N, Cc, H, W, dy.shape[2], dy.shape[3], _stream_handle(stream)))
     return dx
 
 

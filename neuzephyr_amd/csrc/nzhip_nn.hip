@@ -22,6 +22,7 @@ struct PoolArgs {
     int H_in, W_in, H_out, W_out;
     int wblocks, wblocks_in;    // 256-column blocks per output row / per input row
     long planes;                // batches * channels
+    int overwrite;              // backward: din = the sums instead of din += them (din's old contents are not read)
 };
 
 // One thread per output element: the window is summed row by row, left to right (the reference's
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256) void avgpool_backward_kernel(float* __restrict
     if (oh_hi > p.H_out - 1) oh_hi = p.H_out - 1;
     if (ow_hi > p.W_out - 1) ow_hi = p.W_out - 1;
     const float* g = share + plane * p.H_out * p.W_out;
-    float acc = din[idx];
+    float acc = p.overwrite ? 0.f : din[idx];
     for (int oh = oh_lo; oh <= oh_hi; oh++)
         for (int ow = ow_lo; ow <= ow_hi; ow++) acc += g[(long)oh * p.W_out + ow];
     din[idx] = acc;
@@ -147,7 +148,8 @@ __global__ __launch_bounds__(256) void avgpool_backward_vec_kernel(float* __rest
         const int rows = min(h0 + p.pool, p.H_in) - max(h0, 0), cols = min(w0 + p.pool, p.W_in) - max(w0, 0);
         return (float)(rows * cols);
     };
-    floatx4 acc = *reinterpret_cast<const floatx4*>(din + idx);
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    if (!p.overwrite) acc = *reinterpret_cast<const floatx4*>(din + idx);
     if (RMAX) {
         float sv[RMAX ? RMAX * CMAX : 1];
 #pragma unroll
@@ -271,6 +273,7 @@ static int pool_args(PoolArgs& p, size_t pool, size_t stride, size_t pad, size_t
     p.pool = (int)pool; p.stride = (int)stride; p.pad = (int)pad;
     p.H_in = (int)H_in; p.W_in = (int)W_in; p.H_out = (int)H_out; p.W_out = (int)W_out;
     p.planes = (long)(batches * channels);
+    p.overwrite = 0;
     p.wblocks = (int)((W_out + 255) / 256);
     p.wblocks_in = (int)((W_in + 255) / 256);
     if (W_in + pad + stride >= (1u << 24) || (size_t)p.wblocks_in * H_in > 0x7fffffffull ||
@@ -311,15 +314,26 @@ int nzhip_avgpool2d(float* out, const float* in, size_t pool, size_t stride, siz
     return check_launch("avgpool_kernel");
 }
 
+static int avgpool2d_backward_impl(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches, size_t channels,
+                                   size_t H_in, size_t W_in, size_t H_out, size_t W_out, int overwrite, void* stream);
 int nzhip_avgpool2d_backward(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches,
                              size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out, void* stream) {
+    return avgpool2d_backward_impl(din, dout, pool, stride, pad, batches, channels, H_in, W_in, H_out, W_out, 0, stream);
+}
+int nzhip_avgpool2d_backward_overwrite(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches,
+                                       size_t channels, size_t H_in, size_t W_in, size_t H_out, size_t W_out, void* stream) {
+    return avgpool2d_backward_impl(din, dout, pool, stride, pad, batches, channels, H_in, W_in, H_out, W_out, 1, stream);
+}
+static int avgpool2d_backward_impl(float* din, const float* dout, size_t pool, size_t stride, size_t pad, size_t batches, size_t channels,
+                                   size_t H_in, size_t W_in, size_t H_out, size_t W_out, int overwrite, void* stream) {
     if (!din || !dout) return set_error(NZHIP_E_INVALID, "nzhip_avgpool2d_backward: null pointer");
     PoolArgs p;
     if (int rc = pool_args(p, pool, stride, pad, batches, channels, H_in, W_in, H_out, W_out, "nzhip_avgpool2d_backward")) return rc;
+    p.overwrite = overwrite;
     const size_t total = batches * channels * H_in * W_in;
     if (total == 0) return NZHIP_OK;
     const size_t outs = batches * channels * H_out * W_out;
-    if (outs == 0) return NZHIP_OK;
+    if (outs == 0) return overwrite ? nzhip_fill(din, 0.f, total, stream) : NZHIP_OK;      // no window at all: the gradient is zero
     hipStream_t s = as_stream(stream);
     if (p.W_in % 4 == 0 && (reinterpret_cast<uintptr_t>(din) & 15) == 0) {
         const int cw_log = pool_cw_log(p.W_in / 4), wblocks4 = (p.W_in / 4 + (1 << cw_log) - 1) >> cw_log, rb = 256 >> cw_log;

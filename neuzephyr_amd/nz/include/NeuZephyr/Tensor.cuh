@@ -54,6 +54,9 @@ namespace nz::data {
         [[nodiscard]] value_type* grad() const;                    // throws std::runtime_error without gradients
         // the same buffer for a caller that is about to write EVERY element of it (contents undefined on return)
         [[nodiscard]] value_type* gradOverwrite() const;
+        // True when the next grad() call would hand out zeros (a clear is pending or the buffer does not exist yet): a writer
+        // that can overwrite instead of add may then take gradOverwrite() and skip both the clear and its own read of the zeros.
+        [[nodiscard]] bool gradIsZero() const noexcept { return _requires_grad && _size != 0 && (_gradZeroPending || !_grad); }
         [[nodiscard]] std::vector<value_type> hostData() const;    // blocks
         [[nodiscard]] std::vector<value_type> hostGrad() const;    // blocks
 

@@ -194,10 +194,14 @@ namespace nz::graph {
                                                 i2c->output->shape(), rhs->output->shape(), mm->output->shape());
                             }
                             if (x->output->requiresGrad()) {
+                                // the first writer of a gradient that is still to be cleared overwrites it: no clear, and the
+                                // kernels neither read the zeros nor go through a temporary and an add pass
+                                const bool fresh = dataGradientFused && x->output->gradIsZero();
+                                float* dX = fresh ? x->output->gradOverwrite() : x->output->grad();
                                 const bool asConvolution =
-                                    dataGradientFused && iConv2dBackwardData(x->output->grad(), dZ, const_cast<float*>(rhs->output->constData()),
+                                    dataGradientFused && iConv2dBackwardData(dX, dZ, const_cast<float*>(rhs->output->constData()),
                                                                              xs[0], xs[1], xs[2], xs[3], O, i2c->kernelHeight, i2c->kernelWidth,
-                                                                             i2c->stride, i2c->padding, ws[0]);
+                                                                             i2c->stride, i2c->padding, ws[0], !fresh);
                                 if (!asConvolution) {
                                     // the reference's chain for this one gradient: dCol = dPre * W^T, then the gather into dx
                                     if (O != 1 && dPre == dZ) {

@@ -170,8 +170,10 @@ namespace nz::nodes {
         void AveragePoolingNode::backward() {                          // src/Nodes.cu:684-690
             if (!inputs[0]->output->requiresGrad()) return;
             const auto si = inputs[0]->output->shape(), so = output->shape();
-            iAveragePoolingBackward(inputs[0]->output->grad(), output->grad(), poolSize, stride, padding, si[0], si[1], si[2],
-                                    si[3], so[2], so[3]);
+            // the first writer of a gradient that is still to be cleared overwrites it: no clear, no read of the zeros
+            const bool fresh = inputs[0]->output->gradIsZero();
+            iAveragePoolingBackward(fresh ? inputs[0]->output->gradOverwrite() : inputs[0]->output->grad(), output->grad(), poolSize,
+                                    stride, padding, si[0], si[1], si[2], si[3], so[2], so[3], fresh);
         }
 
         ReshapeNode::ReshapeNode(Node* input, const Tensor::shape_type& newShape) : newShape(newShape) {

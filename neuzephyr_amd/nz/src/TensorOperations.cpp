@@ -142,9 +142,9 @@ namespace nz::data {
 
     void iAveragePoolingBackward(float* out, float* in, const size_t pool_size, const size_t stride, const size_t padding,
                                  const size_t batches, const size_t channels, const size_t H_in, const size_t W_in,
-                                 const size_t H_out, const size_t W_out) {
-        NZ_CHECK(nzhip_avgpool2d_backward(out, in, pool_size, stride, padding, batches, channels, H_in, W_in, H_out, W_out,
-                                          nzhip_default_stream()));
+                                 const size_t H_out, const size_t W_out, const bool overwrite) {
+        NZ_CHECK((overwrite ? nzhip_avgpool2d_backward_overwrite : nzhip_avgpool2d_backward)(
+            out, in, pool_size, stride, padding, batches, channels, H_in, W_in, H_out, W_out, nzhip_default_stream()));
     }
 
     static float meanLoss(float* predict, float* real, const size_t n, const bool bce) {
@@ -207,9 +207,9 @@ namespace nz::data {
 
     bool iConv2dBackwardData(float* dx, float* dy, float* w, const size_t N, const size_t C, const size_t H,
                              const size_t W, const size_t O, const size_t K_h, const size_t K_w, const size_t stride,
-                             const size_t pad, const size_t weightBatch) {
+                             const size_t pad, const size_t weightBatch, const bool accumulate) {
         if (stride < 1 || stride > 8 || K_h != K_w || pad > K_h - 1) return false;
-        NZ_CHECK(nzhip_conv2d_backward_data(dx, dy, w, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch, 1,
+        NZ_CHECK(nzhip_conv2d_backward_data(dx, dy, w, N, C, H, W, O, K_h, K_w, stride, pad, weightBatch, accumulate ? 1 : 0,
                                             nzhip_default_stream()));
         return true;
     }

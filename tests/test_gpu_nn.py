@@ -72,6 +72,10 @@ def test_avgpool_random_geometries_bit_exact(nz, oracle, shape, pool, stride, pa
     dx = dev(base)
     nz.avgpool2d_backward(dx, dev(dy), pool, stride, pad)
     assert np.array_equal(host(dx), oracle.avgpool2d_backward(base, dy, pool, stride, pad))
+    # overwrite: the same sums started from zero, whatever dx held (NaN here: an old value that is read shows up)
+    dx = dev(np.full(shape, np.nan, np.float32))
+    nz.avgpool2d_backward(dx, dev(dy), pool, stride, pad, overwrite=True)
+    assert np.array_equal(host(dx), oracle.avgpool2d_backward(np.zeros(shape, np.float32), dy, pool, stride, pad))
 
 
 def test_avgpool_rejects_bad_geometry(nz):
