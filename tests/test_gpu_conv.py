@@ -247,6 +247,27 @@ PER_SAMPLE = [  # N, C, H, W, O, k, pad, per-pixel bias: one weight copy per ima
 ]
 
 
+BIAS_SHARED_BY_IMAGES = [  # N, C, H, W, O, per-sample weights: a per-pixel bias on the resident kernels with a patch count per image
+    # that is a multiple of 8, where every XCD takes the same eighth of all images (both halo-buffer variants, both
+    # channel tiles, three images in a grid of 24, sixteen images with two workgroups per XCD each)
+    (2, 32, 32, 64, 64, False), (2, 32, 32, 64, 64, True), (4, 64, 16, 128, 128, False), (4, 64, 16, 128, 128, True),
+    (3, 64, 32, 64, 128, False), (16, 48, 32, 64, 100, True), (16, 64, 32, 128, 128, True), (5, 16, 64, 64, 40, False)]
+
+
+@pytest.mark.parametrize("N,C,H,W,O,per_sample", BIAS_SHARED_BY_IMAGES)
+def test_conv2d_per_pixel_bias_with_every_xcd_on_one_eighth_of_all_images(nz, oracle, N, C, H, W, O, per_sample):
+    rng = np.random.default_rng(N * 7 + C * 3 + H + W + O + per_sample)
+    x = rng.integers(-4, 5, size=(N, C, H, W)).astype(np.float32)
+    wb = N if per_sample else 1
+    w = rng.integers(-3, 4, size=(wb, O, C, 3, 3)).astype(np.float32)
+    bias = rng.integers(-2, 3, size=(1, 1, H * W, O)).astype(np.float32)
+    badd = bias.reshape(H, W, O).transpose(2, 0, 1)[None].astype(np.float64)
+    w_ref = np.concatenate([oracle.weights_oihw_to_ref(w[b]) for b in range(wb)], axis=0)
+    truth = np.concatenate([oracle.conv2d_direct_f64(x[b:b + 1], w[b if per_sample else 0], None, 1, 1) for b in range(N)], axis=0) + badd
+    got = host(nz.conv2d_forward(dev(x), dev(w_ref), dev(bias), 3, 3, 1, 1, bias_strides=(O, 1), relu=False))
+    assert np.array_equal(got.astype(np.float64), truth)
+
+
 @pytest.mark.parametrize("N,C,H,W,O,k,pad,pix", PER_SAMPLE)
 def test_conv2d_per_sample_weights_that_differ_between_images(nz, oracle, N, C, H, W, O, k, pad, pix):
     # the reference's Conv2d parameter holds one weight copy per sample (src/Model.cu:248-252); here every copy is
