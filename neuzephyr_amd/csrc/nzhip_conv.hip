@@ -50,6 +50,20 @@ __device__ __forceinline__ void xcd_contiguous_block(int& bx, int& by, int& bz) 
     bz = (int)(unit / (gx * gy));
 }
 
+// The same with z (the image) fastest inside an XCD's run: the XCD then works on one stretch of the (x, y) grid for ALL
+// images, so whatever the images share per tile -- a per-pixel bias -- is fetched into its L2 once instead of once per image.
+__device__ __forceinline__ void xcd_contiguous_block_z_fastest(int& bx, int& by, int& bz) {
+    const long gx = gridDim.x, gz = gridDim.z;
+    const long total = gx * gridDim.y * gz;
+    const long lin = blockIdx.x + gx * (blockIdx.y + (long)gridDim.y * blockIdx.z);
+    const long xcd = lin & 7, q = lin >> 3;
+    const long rem = total & 7;
+    const long unit = xcd * (total >> 3) + (xcd < rem ? xcd : rem) + q;
+    bz = (int)(unit % gz);
+    bx = (int)((unit / gz) % gx);
+    by = (int)(unit / (gz * gx));
+}
+
 // O_T: output channels per thread; C_T: compile-time input-channel count (0 = runtime loop);
 // VEC: W % 4 == 0 and 16-byte aligned tensors, so every lane's 4 pixels are inside the row and
 // move as one 16-byte access.
@@ -1780,6 +1794,7 @@ struct ConvGenArgs {
     long bias_sp, bias_sc, bias_sn;
     int relu;
     int img_chunks, halo_plane;           // chunks per channel tile in the weight image (n_chunks rounded up to CPB); bytes of one halo plane
+    int bias_map;                         // a per-pixel bias shared by the images: every XCD on one stretch of segments of ALL images
     int chunk_groups, chunks_per_group;   // the contraction split over groups of channel chunks (blockIdx.z = image * groups + group)
     float* partial;                       // with more than one group: [group][image][O][Ho * Wo] sums without bias or activation
 };
@@ -1819,7 +1834,8 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
     const int wm = wave & 3, wn = wave >> 2;                    // pixel blocks 2 wm, 2 wm + 1; channel blocks NO wn ..
     // neighbouring segments share input rows: the compute units of one XCD take a contiguous run of them
     int seg_x, o_tile, bz;
-    xcd_contiguous_block(seg_x, o_tile, bz);
+    if (PIXB && p.bias_sn == 0 && p.bias_map) xcd_contiguous_block_z_fastest(seg_x, o_tile, bz);   // a bias all images share
+    else xcd_contiguous_block(seg_x, o_tile, bz);
     const int b = bz / p.chunk_groups, group = bz % p.chunk_groups;
     const int chunk_lo = group * p.chunks_per_group;
     const int chunk_hi = chunk_lo + p.chunks_per_group < p.n_chunks ? chunk_lo + p.chunks_per_group : p.n_chunks;
@@ -1923,8 +1939,9 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
     // acknowledged (a load issued after stores is not counted as returned before they are), and every lane asking
     // memory for its own per-channel values sends thousands of requests per workgroup to the same few lines. So a
     // per-channel bias is the starting value of the sums -- one load per channel and workgroup, handed out through
-    // LDS -- and a per-pixel bias is requested one unit (32 pixels x 32 channels) ahead of the stores that need it,
-    // the first unit's before the last chunk's taps when the registers allow (one staging task per thread).
+    // LDS -- and a per-pixel bias is requested straight into the sums before the first chunk: the loads land while the first
+    // halo and slab do, and the epilogue is stores only. (Requested in the epilogue, one 32 x 32 unit ahead of its stores,
+    // a wave had 4 KB in flight per memory round trip: 16 x 3 x 224 x 224 -> 64 took 133 us against 56 us without the bias.)
     const bool pix_bias = PIXB && p.bias && !p.partial;
     if (!PIXB && p.bias && !p.partial) {
         float* lds_b = reinterpret_cast<float*>(lds_h);          // the halo area is free until the first store_halo
@@ -1945,24 +1962,28 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
             }
         __syncthreads();                                        // read before the first halo lands in the same bytes
     }
-    float bvs[2][16];
-    auto bias_request = [&](float (&bv)[16], const int j, const int i) {
-        const int px = (wm * 2 + j) * 32 + li;
-        const int ho = ho0 + (px >> p.sw_log), wo = wo0 + (px & (SW - 1));
-        const float* bp = p.bias + (long)b * p.bias_sn + ((ho < p.Ho && wo < p.Wo) ? ((long)ho * p.Wo + wo) * p.bias_sp : 0);
-        const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
+    if (pix_bias) {
 #pragma unroll
-        for (int rr = 0; rr < 16; rr++) {
-            const int o = o_base + (rr >> 2) * 8 + (rr & 3);
-            bv[rr] = bp[(long)(o < p.O ? o : 0) * p.bias_sc];
+        for (int j = 0; j < 2; j++) {
+            const int px = (wm * 2 + j) * 32 + li;
+            const int ho = ho0 + (px >> p.sw_log), wo = wo0 + (px & (SW - 1));
+            const float* bp = p.bias + (long)b * p.bias_sn + ((ho < p.Ho && wo < p.Wo) ? ((long)ho * p.Wo + wo) * p.bias_sp : 0);
+#pragma unroll
+            for (int i = 0; i < NO; i++) {
+                const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
+#pragma unroll
+                for (int rr = 0; rr < 16; rr++) {
+                    const int o = o_base + (rr >> 2) * 8 + (rr & 3);
+                    acc[i][j][rr] = bp[(long)(o < p.O ? o : 0) * p.bias_sc];      // clamped: positions outside are never stored
+                }
+            }
         }
-    };
+    }
     for (int chunk = chunk_lo; chunk < chunk_hi; chunk++) {
         store_halo(chunk);                                      // registers (chunk) -> LDS, fp16 channel-last
         __builtin_amdgcn_s_waitcnt(0x0070 | 0x0F00);            // vmcnt(0): this wave's slab pieces landed
         __syncthreads();
         load_halo(chunk + 1 < chunk_hi ? chunk + 1 : chunk);    // lands while the MFMAs below run (the last: once more, unused)
-        if (PIXB && TP == 1 && pix_bias && chunk + 1 == chunk_hi) bias_request(bvs[0], 0, 0);   // (more tasks per thread leave no registers for it)
         // two fragment sets: the reads of tap t + 1 are issued before the MFMAs of tap t. A step's CPB planes and slabs
         // follow each other as one run of CPB * taps positions (plane, kernel row, kernel column).
         half8_t wf_[2][NO], pf_[2][2];
@@ -2035,7 +2056,6 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
         return;
     }
     float* yb = p.y + (long)b * p.O * p.Ho * p.Wo;
-    if (PIXB && TP != 1 && pix_bias) bias_request(bvs[0], 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int px = (wm * 2 + j) * 32 + li;
@@ -2044,14 +2064,11 @@ __global__ __launch_bounds__(CG_THREADS) void conv_igemm_gen_kernel(const ConvGe
         const long pix = px_ok ? (long)ho * p.Wo + wo : 0;
 #pragma unroll
         for (int i = 0; i < NO; i++) {
-            const int u = j * NO + i;
-            if (PIXB && pix_bias && u + 1 < 2 * NO) bias_request(bvs[(u + 1) & 1], (u + 1) / NO, (u + 1) % NO);
             const int o_base = o_tile * BN + (wn * NO + i) * 32 + lh * 4;
 #pragma unroll
             for (int rr = 0; rr < 16; rr++) {
                 const int o = o_base + (rr >> 2) * 8 + (rr & 3);
                 float v = acc[i][j][rr];
-                if (PIXB && pix_bias) v += bvs[u & 1][rr];
                 if (p.relu) v = v > 0.f ? v : 0.f;
                 if (px_ok && o < p.O) yb[(long)o * hw_out + pix] = v;
             }
@@ -2245,6 +2262,8 @@ static int conv_igemm_gen_launch(float* y, const float* x, const float* w_ref, c
     a.bias_sp = bias_sp; a.bias_sc = bias_sc; a.bias_sn = bias_sn; a.relu = act == NZHIP_ACT_RELU;
     a.chunk_groups = chunk_groups; a.chunks_per_group = chunks_per_group; a.partial = nullptr;
     a.img_chunks = img_chunks; a.halo_plane = span * pw * 32;
+    static const char* bias_map_env = getenv("NZHIP_CONV_BIAS_MAP");   // benchmarking only: 0 keeps the image-major order
+    a.bias_map = !(bias_map_env && atoi(bias_map_env) == 0) && N >= 2;
     size_t lds_use = lds_need;
     if (two) {                                                       // the kernel counts steps of two chunks
         a.n_chunks = img_chunks / 2; a.chunks_per_group = a.n_chunks;
@@ -3047,16 +3066,32 @@ static int conv2d_forward_impl(float* y, const float* x, const float* w_ref, con
         g.a_stride_n = w_batch > 1 ? (int64_t)(C * O) : 0; g.b_stride_n = (int64_t)(C * H * W); g.c_stride_n = (int64_t)(O * H * W);
         g.bias = bias; g.bias_stride_row = bias_stride_channel; g.bias_stride_col = bias_stride_pixel; g.bias_stride_n = bias_stride_image;
         g.activation = activation;
+        // The reference's bias is pixel-major ([1, 1, pixels, O], src/Model.cu:252-256) while the product's lanes run along
+        // the pixels: read as it lies, every bias load touches 64 lines 4 O bytes apart. One pass turns it into channel
+        // planes, the layout of y (16 x 64 x 56 x 56 -> 256: 41 -> 33 us).
+        float* bias_planes = nullptr;
+        if (bias && bias_stride_image == 0 && bias_stride_channel == 1 && bias_stride_pixel == (int64_t)O && O >= 8 && O * H * W >= 262144) {      // from 1 MB of bias on: below, the pass costs what it saves
+            if (int rc = workspace_alloc(reinterpret_cast<void**>(&bias_planes), O * H * W * sizeof(float), s)) return rc;
+            if (int rc = nzhip_col2im(bias_planes, bias, H, W, O, 1, s)) {
+                workspace_free(bias_planes, s);
+                return rc;
+            }
+            g.bias = bias_planes; g.bias_stride_row = (int64_t)(H * W); g.bias_stride_col = 1;
+        }
         float* x_wide = nullptr;
         const double flops = 2.0 * (double)N * (double)(H * W) * (double)C * (double)O;
         if (conv1x1_wants_wide_planes(H * W, flops, 2.0 * (double)O)) {
-            if (int rc = widen_rows(&x_wide, x, N * C, H * W, s)) return rc;
+            if (int rc = widen_rows(&x_wide, x, N * C, H * W, s)) {
+                if (bias_planes) workspace_free(bias_planes, s);
+                return rc;
+            }
             const size_t HWp = (H * W + 3) / 4 * 4;
             g.B = x_wide; g.ldb = (int64_t)HWp; g.b_stride_n = (int64_t)(C * HWp);
         }
         const int rc = x_wide ? gemm_padded_rows(g, 2, s) : nzhip_gemm(&g, s);
         const int rc2 = x_wide ? workspace_free(x_wide, s) : NZHIP_OK;
-        return rc ? rc : rc2;
+        const int rc3 = bias_planes ? workspace_free(bias_planes, s) : NZHIP_OK;
+        return rc ? rc : (rc2 ? rc2 : rc3);
     }
     bool wide = false, bn128 = false;
     const ConvRoute route = conv_forward_route(x, N, C, H, W, O, K_h, K_w, stride, pad, w_batch, H_out, W_out, wide, bn128);
