@@ -53,7 +53,7 @@ def test_gemm_with_a_prepared_b_image(nz, M, K, N, b_trans):
 CONVS = [  # N, C, H, W, O, K, pad, w_batch: double-buffer resident kernel, single-buffer resident kernel, slab kernel, ...,
     # and the any-geometry kernel (5x5)
     (4, 64, 64, 64, 128, 3, 1, 1), (2, 48, 40, 72, 64, 3, 1, 1), (2, 24, 33, 47, 40, 3, 1, 1), (8, 160, 64, 64, 128, 3, 1, 1),
-    (3, 32, 20, 20, 48, 1, 0, 1), (8, 16, 64, 64, 32, 3, 1, 8), (16, 16, 32, 32, 16, 5, 2, 1)]
+    (3, 24, 20, 20, 48, 1, 0, 1), (8, 16, 64, 64, 32, 3, 1, 8), (16, 16, 32, 32, 16, 5, 2, 1)]   # (1x1 below 32 channels: from there on it is a plain product without an image)
 
 
 @pytest.mark.parametrize("N,C,H,W,O,K,pad,wb", CONVS)
