@@ -684,6 +684,27 @@ def test_config5_large_square_sampled_rows(nz, oracle):
     assert np.array_equal(host(nz.gemm(Ad, I)), oracle.round_f16(A))
 
 
+@pytest.mark.parametrize("M,K,N,b_trans", [(8192, 8192, 8192, False), (8192, 8192, 8192, True), (4096, 1024, 4096, True), (1000, 777, 513, False)])
+def test_whole_output_at_full_size_against_torch_fp32_product(nz, M, K, N, b_trans):
+    # every element of the headline product (and of the Linear and ragged configs) against an implementation that shares
+    # nothing with this one: torch's fp32 matmul on the operands rounded to fp16 first. Both accumulate in fp32, in
+    # different orders: 1e-5 relative in the Frobenius norm (3e-7 measured), and no element off by more than 1e-3 of the
+    # largest one.
+    import torch
+    torch.backends.cuda.matmul.allow_tf32 = False
+    g = torch.Generator(device="cuda").manual_seed(M + K + N)
+    A = torch.randn(M, K, device="cuda", generator=g) / np.sqrt(K)
+    B = torch.randn((N, K) if b_trans else (K, N), device="cuda", generator=g)
+    got = nz.gemm(A, B, b_trans=b_trans)
+    Br = B.half().float()
+    want = torch.matmul(A.half().float(), Br.t() if b_trans else Br)
+    diff = got - want
+    assert float(diff.norm() / want.norm()) < 1e-5
+    assert float(diff.abs().max()) < 1e-3 * float(want.abs().max())
+    del got, want, diff, Br
+    torch.cuda.empty_cache()
+
+
 def test_config5_batched_1024(nz, oracle):
     # [8,16,1024,1024] x [8,16,1024,1024] over (N,C); three seeded batch members checked in full
     import torch
